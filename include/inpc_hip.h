@@ -1,0 +1,267 @@
+/*
+ * inpc_hip.h — C ABI of libinpc_hip.so, the MI355X (gfx950) implementation of the
+ * INPCCudaBackend hot path: view-dependent octree point sampling and the tile-based
+ * differentiable bilinear point rasterizer (forward, backward, inference).
+ *
+ * Conventions
+ *   - every pointer marked "dev" is a device pointer on the current HIP device;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - every function returns 0 on success and a negative INPC_E_* code on failure,
+ *     never throws; inpc_last_error() returns a thread-local message for the last failure;
+ *   - the library never allocates or frees device memory: the caller provides the
+ *     workspace whose size inpc_*_workspace_bytes() reports (sized for the worst case,
+ *     so no count has to travel back to the host between kernels);
+ *   - all kernels are enqueued on `stream`; no call synchronises the host unless its
+ *     comment says so.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference repository, B/ = INPCCudaBackend/INPCCudaBackend/).
+ */
+#ifndef INPC_HIP_H
+#define INPC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes -------------------------------------------------------------------- */
+#define INPC_OK 0
+#define INPC_E_INVALID_ARGUMENT (-1) /* bad size, tile, channel count, null pointer, ...   */
+#define INPC_E_WORKSPACE (-2)        /* workspace too small or misaligned                   */
+#define INPC_E_UNSUPPORTED (-3)      /* e.g. more than 65536 tiles, unknown feature mode    */
+#define INPC_E_HIP (-4)              /* a HIP runtime call failed (message has the detail)  */
+#define INPC_E_DEVICE (-5)           /* a kernel raised its device-side error flag          */
+
+/* ---- pinhole camera: the scalars B/torch_bindings/sampling.py:20-33 and
+ *      B/torch_bindings/rasterization.py:116-128 unpack from a View ---------------------- */
+typedef struct inpc_camera {
+    int32_t width;
+    int32_t height;
+    float focal_x;
+    float focal_y;
+    float center_x;
+    float center_y;
+    float near_plane;
+    float far_plane;
+} inpc_camera;
+
+/* ---- how the per-point features are stored ------------------------------------------- */
+#define INPC_FEAT_SH36_F16 0   /* (N,36) fp16, 9 SH coefficients x 4 channels -> 4 channels
+                                  (B/rasterization/include/sh_utils.cuh:6-23)              */
+#define INPC_FEAT_DIRECT_F32 1 /* (N,C) fp32, C in {4,8,16}, used as they are              */
+#define INPC_FEAT_DIRECT_F16 2 /* (N,C) fp16 stored, fp32 accumulated                      */
+#define INPC_FEAT_RAW37_F16 3  /* (N,37) fp16: [0] raw opacity, [1..36] SH coefficients
+                                  (B/rasterization/src/bilinear/kernels.cu:106-184)        */
+
+/* ---- rasterizer flags ------------------------------------------------------------------ */
+#define INPC_RASTER_INFERENCE 1u /* write a depth image, no blending weights
+                                    (B/rasterization/src/bilinear/kernels.cu:422-495)      */
+
+const char* inpc_last_error(void);
+int inpc_abi_version(void);
+
+/* =========================================================================================
+ * PCG32 host helpers (B/sampling/include/pcg32.h:42-201). `rng` is {state, inc}.
+ * The sampler keeps its generator in device memory (two uint64) so that a call whose
+ * consumption is data dependent needs no host read-back; these helpers build and step the
+ * same generator on the host.
+ * ======================================================================================= */
+void inpc_pcg32_seed(uint64_t rng[2], uint64_t initstate, uint64_t initseq);
+uint32_t inpc_pcg32_next_uint(uint64_t rng[2]);
+float inpc_pcg32_next_float(uint64_t rng[2]);
+void inpc_pcg32_advance(uint64_t rng[2], int64_t delta);
+
+/* =========================================================================================
+ * Sampler
+ * ======================================================================================= */
+
+/* Per-leaf view-dependent weight.
+ * Replaces compute_viewpoint_weights_wrapper (B/sampling/src/sampling_api.cu:10-47) and
+ * kernel compute_viewpoint_weights_cu (B/sampling/src/sampling_kernels.cu:9-64).
+ * centers (L,3) f32, levels (L,) i32, weights (L,) f32, w2c (4,4) f32 row-major (rows 0..2
+ * are read), out (L,) f32; all dev. */
+int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* weights,
+                      const float* w2c, float* out, uint32_t n_leaves, const inpc_camera* cam,
+                      float initial_size, void* stream);
+
+/* Bytes of scratch the CDF / counting passes need for n_leaves leaves. */
+size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
+
+/* Normalise the leaf weights and turn them into an inclusive CDF, in place.
+ * Replaces compute_cdf (B/sampling/src/sampling.cu:150-186): cub::DeviceReduce::Sum, the
+ * reciprocal-multiply normalisation (B/sampling/src/sampling_kernels.cu:66-75) and
+ * cub::DeviceScan::InclusiveSum. The float association order is fixed: left-to-right inside
+ * chunks of 64, chunk totals combined the same way one level up, recursively.
+ * `sum_out` (dev, 1 float) receives the un-normalised total; when it is <= 0 the weights are
+ * left un-normalised and later sampling kernels take the failure path themselves.
+ * No host synchronisation. */
+int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t workspace_bytes,
+                   uint32_t n_leaves, void* stream);
+
+/* Multinomial leaf pick + uniform in-leaf jitter, no culling.
+ * Replaces create_samples (B/sampling/src/sampling.cu:188-209) and create_samples_cu
+ * (B/sampling/src/sampling_kernels.cu:128-150). Sample i uses the generator `rng_dev`
+ * advanced by 4*i draws; afterwards the device generator is advanced by 4*n_samples.
+ * positions_out (n,3) f32; leaf_ids_out (n,) i32 or NULL. If *sum_dev <= 0 nothing is
+ * written and the generator is left untouched. */
+int inpc_sample(const float* centers, const int32_t* levels, const float* cdf, const float* sum_dev,
+                float* positions_out, int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves,
+                float initial_size, uint64_t* rng_dev, void* stream);
+
+/* Bytes of scratch for inpc_sample_cull_compact over up to n_candidates per round. */
+size_t inpc_cull_workspace_bytes(uint32_t n_candidates);
+
+/* Zero the round state (accepted count, consumed count) kept at the head of a cull
+ * workspace. Call once before the first round of a draw. */
+int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream);
+
+/* One round of the training sampler: candidates k0 .. k0+n_candidates-1 of the counter-based
+ * stream (candidate k uses the generator advanced by 4*k draws) are generated as in
+ * inpc_sample, tested against the frustum, and the accepted ones appended, in ascending k,
+ * to positions_out / leaf_ids_out behind the `accepted` count held in the workspace, up to
+ * `capacity` entries.
+ * Replaces create_training_samples_cu (B/sampling/src/sampling_kernels.cu:77-126); its
+ * scheduling-dependent atomic slot order is replaced by ascending candidate order.
+ * The workspace records, once `capacity` entries exist, how many candidates were consumed
+ * (index of the last accepted candidate + 1). The generator is NOT advanced here; see
+ * inpc_cull_finish. */
+int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const float* cdf,
+                             const float* sum_dev, const float* w2c, float* positions_out,
+                             int32_t* leaf_ids_out, uint32_t capacity, uint32_t k0,
+                             uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam,
+                             float initial_size, const uint64_t* rng_dev, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/* Copy {accepted, consumed} of the current draw to host memory. Synchronises `stream`. */
+int inpc_cull_read_counts(const void* workspace, uint32_t* accepted_host, uint32_t* consumed_host,
+                          void* stream);
+
+/* End of a draw: advance the device generator by 4*consumed draws (4*total_candidates when
+ * fewer than `capacity` samples were accepted), mirroring the host-side rng.advance of
+ * B/sampling/src/sampling.cu:208. When *sum_dev <= 0 the outputs are filled with the
+ * failure pattern of B/sampling/src/sampling.cu:107-111 (positions 0, ids -1). */
+int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_ids_out,
+                     uint32_t capacity, uint32_t total_candidates, uint64_t* rng_dev,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Widen int32 leaf ids to the int64 the Python API returns
+ * (B/sampling/src/sampling_api.cu:71). */
+int inpc_widen_ids(const int32_t* ids, int64_t* out, uint32_t n, void* stream);
+
+/* Expected-count sampler, step 1: count[l] = w>0 ? max(1, rint(w*(1/sum)*n_samples)) : 0 and
+ * its inclusive integer prefix sum. Replaces compute_sample_distribution
+ * (B/sampling/src/sampling.cu:211-253), compute_sample_counts_cu
+ * (B/sampling/src/sampling_kernels.cu:152-169). `weights` are the un-normalised leaf
+ * weights; sum_out (dev) gets their total; offsets_out (L,) i32 dev gets the inclusive sums
+ * (last entry = number of samples created). No host synchronisation. */
+int inpc_expected_counts(const float* weights, float* sum_out, int32_t* offsets_out,
+                         uint32_t n_samples, void* workspace, size_t workspace_bytes,
+                         uint32_t n_leaves, void* stream);
+
+/* Expected-count sampler, step 2: sample j (of n_created*n_multi) lies in leaf
+ * ids[j mod n_created], where ids is the repeat-interleave of the counts, with three
+ * jitters from the generator advanced by 3*j draws; afterwards the device generator is
+ * advanced by 3*n_total. Replaces create_expected_samples (B/sampling/src/sampling.cu:255-287),
+ * repeat_interleave_indices_cu and create_expected_samples_cu
+ * (B/sampling/src/sampling_kernels.cu:171-205). leaf_ids_scratch (n_created,) i32 dev. */
+int inpc_expected_samples(const float* centers, const int32_t* levels, const int32_t* offsets,
+                          int32_t* leaf_ids_scratch, float* positions_out, uint32_t n_created,
+                          uint32_t n_multi, uint32_t n_leaves, float initial_size,
+                          uint64_t* rng_dev, void* stream);
+
+/* =========================================================================================
+ * Rasterizer
+ * ======================================================================================= */
+
+/* Geometry of a rasterizer call; fills the derived fields. */
+typedef struct inpc_raster_config {
+    uint32_t n_points;
+    int32_t tile;         /* 8 (reference, B/rasterization/include/bilinear/config.h:23-25) or 16 */
+    int32_t channels;     /* 4, 8 or 16 (4 for the SH modes)                                       */
+    int32_t feature_mode; /* INPC_FEAT_*                                                           */
+    uint32_t flags;       /* INPC_RASTER_*                                                         */
+    inpc_camera cam;
+} inpc_raster_config;
+
+/* Offsets (bytes from the workspace base) of the buffers a caller may want to inspect.
+ * The layout is private otherwise. Counts live in device memory. */
+typedef struct inpc_raster_layout {
+    size_t total_bytes;
+    size_t counters;        /* u32[16]: [0] n_visible, [1] n_instances, [2] error flag          */
+    size_t point_record;    /* (N) {float sx, sy, opacity; u32 tileinfo}                        */
+    size_t point_depth;     /* (N) f32 view-space depth                                         */
+    size_t features_view;   /* (N,4) f32, SH modes only, else 0                                 */
+    size_t depth_order;     /* (N) u32: point ids in (depth, id) order, first n_visible valid   */
+    size_t depth_keys;      /* (N) u32: matching depth keys (float bits), first n_visible valid */
+    size_t instance_keys;   /* (4N) u16: tile id per instance in final order                    */
+    size_t instance_points; /* (4N) u32: point id per instance in final order                   */
+    size_t tile_ranges;     /* (n_tiles) {u32 begin, end}                                       */
+    uint32_t grid_width;
+    uint32_t grid_height;
+    uint32_t n_tiles;
+    uint32_t end_bit;       /* bit length of n_tiles-1
+                               (B/rasterization/include/rasterization_utils.h:3-13)             */
+    uint32_t depth_key_bias; /* depth_keys hold (float bits of the depth) - depth_key_bias       */
+} inpc_raster_layout;
+
+/* Workspace size and layout for a configuration. Replaces the three growable blobs of
+ * B/rasterization/include/bilinear/buffer_utils.h:24-115 and the resize callbacks of
+ * B/rasterization/include/torch_utils.h:6-12 with one caller-owned worst-case buffer
+ * (visible points <= N, instances <= 4N). */
+int inpc_raster_layout_query(const inpc_raster_config* cfg, inpc_raster_layout* out);
+
+/* Forward pass: project, cull, sort by (tile, depth, id), per-tile ranges, front-to-back
+ * bilinear 2x2 splat blend.
+ * Replaces forward_wrapper / inference_wrapper / inference_preextracted_wrapper
+ * (B/rasterization/src/rasterization_api.cu:23-107,192-374) and bilinear::forward /
+ * inference / inference_preextracted (B/rasterization/src/bilinear/forward.cu:12-170,
+ * inference.cu:11-167, inference_preextracted.cu:11-168).
+ *   positions (N,3) f32; features per cfg->feature_mode; opacities (N,) f32 (unused for
+ *   INPC_FEAT_RAW37_F16); w2c (4,4) f32; cam_position (3,) f32 (SH modes only);
+ *   image (C,H,W) f32; alpha (1,H,W) f32;
+ *   blending_weights (N,) f32 (training) or NULL; depth_image (1,H,W) f32 (inference) or NULL.
+ * The workspace is the saved state the backward pass needs. No host synchronisation. */
+int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, const void* features,
+                        const float* opacities, const float* w2c, const float* cam_position,
+                        float* image, float* alpha, float* blending_weights, float* depth_image,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward pass: replays the blend front to back with the saved final image.
+ * Replaces backward_wrapper (B/rasterization/src/rasterization_api.cu:109-190),
+ * bilinear::backward (B/rasterization/src/bilinear/backward.cu:9-67), blend_backward_cu and
+ * preprocess_backward_cu (B/rasterization/src/bilinear/kernels.cu:86-104,315-420).
+ *   grad_image (C,H,W), grad_alpha (1,H,W), image, alpha: f32, as produced by forward;
+ *   grad_features: (N,36) fp16 for INPC_FEAT_SH36_F16, (N,C) f32 for INPC_FEAT_DIRECT_F32,
+ *                  (N,C) fp16 for INPC_FEAT_DIRECT_F16; fully written (zeros where a point
+ *                  was not drawn);
+ *   grad_opacities (N,) f32, fully written;
+ *   grad_view_scratch: (N,4) f32 scratch for the SH mode, else NULL. */
+int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
+                         const float* grad_alpha, const float* image, const float* alpha,
+                         const float* positions, const void* features, const float* opacities,
+                         const float* cam_position, void* grad_features, float* grad_opacities,
+                         float* grad_view_scratch, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+/* Copy the rasterizer counters {n_visible, n_instances, error flag} to the host.
+ * Synchronises `stream`. Returns INPC_E_DEVICE if the error flag is set. */
+int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* workspace,
+                              uint32_t counters_host[3], void* stream);
+
+/* Per-kernel timing hooks for benchmarks: when enabled, every launch made by the calling
+ * thread is bracketed by HIP events on its stream; inpc_timing_collect synchronises and
+ * returns the number of records written as {name, milliseconds}. */
+typedef struct inpc_timing_record {
+    const char* name;
+    float ms;
+} inpc_timing_record;
+void inpc_timing_enable(int on);
+int inpc_timing_collect(inpc_timing_record* out, int capacity);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INPC_HIP_H */

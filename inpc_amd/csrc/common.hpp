@@ -1,0 +1,177 @@
+// common.hpp — helpers shared by the gfx950 kernels and the C-ABI layer of libinpc_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/inpc_hip.h"
+
+namespace inpc {
+
+// ------------------------------------------------------------------------------------------------
+// host side: error reporting and launches
+// ------------------------------------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+
+// Optional per-launch timing (HIP events on the launch stream), see inpc_timing_enable().
+void timing_begin(const char* name, hipStream_t stream);
+void timing_end(hipStream_t stream);
+
+#define INPC_HIP_CHECK(expr)                                                                        \
+    do {                                                                                            \
+        hipError_t _e = (expr);                                                                     \
+        if (_e != hipSuccess)                                                                       \
+            return ::inpc::fail(INPC_E_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e),  \
+                                __FILE__, __LINE__);                                                \
+    } while (0)
+
+// Launch `kernel<<<grid, block, 0, stream>>>(args...)`, bracketed by timing events when enabled,
+// and turn a launch failure into an INPC_E_HIP return.
+#define INPC_LAUNCH(name, kernel, grid, block, stream, ...)                                         \
+    do {                                                                                            \
+        ::inpc::timing_begin(name, stream);                                                         \
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);                            \
+        ::inpc::timing_end(stream);                                                                 \
+        hipError_t _e = hipGetLastError();                                                          \
+        if (_e != hipSuccess)                                                                       \
+            return ::inpc::fail(INPC_E_HIP, "launch of %s failed: %s", name, hipGetErrorString(_e)); \
+    } while (0)
+
+inline uint32_t div_up(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline int bit_length(uint32_t n) {
+    int b = 0;
+    while (n) {
+        ++b;
+        n >>= 1;
+    }
+    return b;
+}
+
+// Fill `n` 32-bit words with `value` (a kernel, not hipMemsetAsync, so that callers may capture
+// the stream into a graph).
+int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream);
+
+// ------------------------------------------------------------------------------------------------
+// device side
+// ------------------------------------------------------------------------------------------------
+constexpr int kWave = 64;
+
+__device__ __forceinline__ uint32_t lane_id() { return __lane_id(); }
+
+// Number of set bits of `mask` below the calling lane.
+__device__ __forceinline__ uint32_t mask_rank(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+// One row of the affine world-to-camera transform, evaluated left to right without fused
+// multiply-add (this translation unit is compiled with -ffp-contract=off).
+__device__ __forceinline__ float affine_row(const float4 r, float x, float y, float z) {
+    return ((r.x * x + r.y * y) + r.z * z) + r.w;
+}
+
+struct Camera {
+    float width, height, fx, fy, cx, cy, near_plane, far_plane;
+};
+
+inline Camera to_device_camera(const inpc_camera& c) {
+    return Camera{(float)c.width, (float)c.height, c.focal_x, c.focal_y, c.center_x, c.center_y, c.near_plane,
+                  c.far_plane};
+}
+
+// ---- PCG32 (XSH-RR 64/32) -----------------------------------------------------------------------
+constexpr uint64_t kPcgMult = 0x5851f42d4c957f2dULL;
+
+struct Pcg32 {
+    uint64_t state, inc;
+};
+
+__host__ __device__ __forceinline__ uint32_t pcg_next(Pcg32& r) {
+    const uint64_t old = r.state;
+    r.state = old * kPcgMult + r.inc;
+    const uint32_t xs = (uint32_t)(((old >> 18u) ^ old) >> 27u);
+    const uint32_t rot = (uint32_t)(old >> 59u);
+    return (xs >> rot) | (xs << ((~rot + 1u) & 31u));
+}
+
+__device__ __forceinline__ float pcg_float(Pcg32& r) {
+    return __uint_as_float((pcg_next(r) >> 9) | 0x3f800000u) - 1.0f;
+}
+
+// The generator stepped `delta` times is state -> mult * state + plus (Brown's jump-ahead).
+struct PcgJump {
+    uint64_t mult, plus;
+};
+
+__host__ __device__ __forceinline__ PcgJump pcg_jump(uint64_t inc, uint64_t delta) {
+    uint64_t cur_mult = kPcgMult, cur_plus = inc, acc_mult = 1u, acc_plus = 0u;
+    while (delta > 0) {
+        if (delta & 1) {
+            acc_mult *= cur_mult;
+            acc_plus = acc_plus * cur_mult + cur_plus;
+        }
+        cur_plus = (cur_mult + 1) * cur_plus;
+        cur_mult *= cur_mult;
+        delta >>= 1;
+    }
+    return PcgJump{acc_mult, acc_plus};
+}
+
+__host__ __device__ __forceinline__ uint64_t pcg_apply(const PcgJump& j, uint64_t state) {
+    return j.mult * state + j.plus;
+}
+
+// ---- decoupled look-back --------------------------------------------------------------------------
+// A status word is {2 flag bits, 30 value bits}. Blocks take their index from an atomic ticket, so
+// a block only ever waits on blocks that are already running; the wait is bounded and raises the
+// error flag instead of spinning forever.
+constexpr uint32_t kFlagAggregate = 1u << 30;
+constexpr uint32_t kFlagInclusive = 2u << 30;
+constexpr uint32_t kValueMask = (1u << 30) - 1u;
+constexpr uint32_t kSpinLimit = 1u << 22;
+
+__device__ __forceinline__ void status_store(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint32_t status_load(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Exclusive prefix of `aggregate` over blocks 0..bid-1, publishing this block's words on the way.
+// `status` points at this stream's word of block 0; consecutive blocks are `stride` words apart.
+__device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_t stride, uint32_t bid,
+                                                       uint32_t aggregate, uint32_t* error_flag) {
+    uint32_t* mine = status + (size_t)bid * stride;
+    if (bid == 0) {
+        status_store(mine, kFlagInclusive | aggregate);
+        return 0u;
+    }
+    status_store(mine, kFlagAggregate | aggregate);
+    uint32_t exclusive = 0u;
+    for (int64_t p = (int64_t)bid - 1; p >= 0; --p) {
+        const uint32_t* theirs = status + (size_t)p * stride;
+        uint32_t word = status_load(theirs);
+        uint32_t spins = 0;
+        while ((word & ~kValueMask) == 0u) {
+            if (++spins > kSpinLimit) {
+                atomicOr(error_flag, 1u);
+                word = kFlagInclusive;  // give up: terminate the walk with a wrong but finite value
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+            word = status_load(theirs);
+        }
+        exclusive += word & kValueMask;
+        if (word & kFlagInclusive) break;
+    }
+    status_store(mine, kFlagInclusive | ((exclusive + aggregate) & kValueMask));
+    return exclusive;
+}
+
+}  // namespace inpc

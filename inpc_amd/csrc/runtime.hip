@@ -1,0 +1,146 @@
+// runtime.hip — error reporting, per-launch timing hooks, fill kernel, PCG32 host helpers.
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+
+namespace inpc {
+
+namespace {
+thread_local char g_error[512] = "";
+
+struct TimingEntry {
+    const char* name;
+    hipEvent_t start, stop;
+};
+thread_local bool g_timing_on = false;
+thread_local std::vector<TimingEntry> g_timing_entries;
+thread_local std::vector<hipEvent_t> g_event_pool;
+thread_local TimingEntry g_open{nullptr, nullptr, nullptr};
+
+hipEvent_t take_event() {
+    if (!g_event_pool.empty()) {
+        hipEvent_t e = g_event_pool.back();
+        g_event_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+}  // namespace
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void timing_begin(const char* name, hipStream_t stream) {
+    if (!g_timing_on) return;
+    g_open.name = name;
+    g_open.start = take_event();
+    g_open.stop = take_event();
+    if (g_open.start) (void)hipEventRecord(g_open.start, stream);
+}
+
+void timing_end(hipStream_t stream) {
+    if (!g_timing_on || !g_open.name) return;
+    if (g_open.stop) (void)hipEventRecord(g_open.stop, stream);
+    g_timing_entries.push_back(g_open);
+    g_open = TimingEntry{nullptr, nullptr, nullptr};
+}
+
+__global__ void __launch_bounds__(256) k_fill_u32(uint32_t* dst, uint32_t value, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = value;
+}
+
+int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream) {
+    if (n_words == 0) return INPC_OK;
+    const uint32_t blocks = (uint32_t)std::min<size_t>((n_words + 255) / 256, 8192);
+    INPC_LAUNCH("fill_u32", k_fill_u32, dim3(blocks), dim3(256), stream, (uint32_t*)dst, value, n_words);
+    return INPC_OK;
+}
+
+}  // namespace inpc
+
+extern "C" {
+
+const char* inpc_last_error(void) { return inpc::g_error; }
+
+int inpc_abi_version(void) { return 1; }
+
+void inpc_timing_enable(int on) {
+    inpc::g_timing_on = on != 0;
+    if (!on) {
+        for (auto& e : inpc::g_timing_entries) {
+            inpc::g_event_pool.push_back(e.start);
+            inpc::g_event_pool.push_back(e.stop);
+        }
+        inpc::g_timing_entries.clear();
+    }
+}
+
+int inpc_timing_collect(inpc_timing_record* out, int capacity) {
+    int n = 0;
+    for (auto& e : inpc::g_timing_entries) {
+        float ms = 0.0f;
+        if (e.start && e.stop && hipEventSynchronize(e.stop) == hipSuccess &&
+            hipEventElapsedTime(&ms, e.start, e.stop) == hipSuccess) {
+            if (n < capacity) {
+                out[n].name = e.name;
+                out[n].ms = ms;
+                ++n;
+            }
+        }
+        if (e.start) inpc::g_event_pool.push_back(e.start);
+        if (e.stop) inpc::g_event_pool.push_back(e.stop);
+    }
+    inpc::g_timing_entries.clear();
+    return n;
+}
+
+void inpc_pcg32_seed(uint64_t rng[2], uint64_t initstate, uint64_t initseq) {
+    inpc::Pcg32 r;
+    r.state = 0u;
+    r.inc = (initseq << 1u) | 1u;
+    inpc::pcg_next(r);
+    r.state += initstate;
+    inpc::pcg_next(r);
+    rng[0] = r.state;
+    rng[1] = r.inc;
+}
+
+uint32_t inpc_pcg32_next_uint(uint64_t rng[2]) {
+    inpc::Pcg32 r{rng[0], rng[1]};
+    const uint32_t v = inpc::pcg_next(r);
+    rng[0] = r.state;
+    return v;
+}
+
+float inpc_pcg32_next_float(uint64_t rng[2]) {
+    union {
+        uint32_t u;
+        float f;
+    } x;
+    x.u = (inpc_pcg32_next_uint(rng) >> 9) | 0x3f800000u;
+    return x.f - 1.0f;
+}
+
+void inpc_pcg32_advance(uint64_t rng[2], int64_t delta) {
+    const inpc::PcgJump j = inpc::pcg_jump(rng[1], (uint64_t)delta);
+    rng[0] = inpc::pcg_apply(j, rng[0]);
+}
+
+}  // extern "C"

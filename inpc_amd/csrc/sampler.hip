@@ -1,0 +1,672 @@
+// sampler.hip — view-dependent point sampling from the octree probability field (gfx950).
+//
+//   k_leaf_weights        per-leaf visibility + weight   (B/sampling/src/sampling_kernels.cu:9-64)
+//   k_chunk_pass / k_chunk_add_prefix
+//                         normalise + float CDF with a fixed association order (chunks of 64,
+//                         left to right, recursively)      (B/sampling/src/sampling.cu:150-186)
+//   k_sample              multinomial leaf pick + jitter  (B/sampling/src/sampling_kernels.cu:128-150)
+//   k_sample_cull         the same draw, frustum test, ordered stream compaction
+//                                                         (B/sampling/src/sampling_kernels.cu:77-126)
+//   k_expected_counts / k_repeat_interleave / k_expected_samples
+//                                                         (B/sampling/src/sampling_kernels.cu:152-205)
+//
+// Candidate k always uses the sampler's generator advanced by 4*k draws. A thread walks candidates
+// 256 apart, so it pays one O(log k) jump at the start and one constant affine step per candidate.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace inpc {
+
+namespace {
+
+constexpr float kFltEps = 1e-8f;
+constexpr int kBlock = 256;
+constexpr int kChunk = 64;
+constexpr int kChunksPerBlock = 64;                      // one wave scans 64 chunks
+constexpr int kChunkTile = kChunk * kChunksPerBlock;     // 4096 floats per block
+constexpr int kSampleItems = 8;                          // candidates per thread
+constexpr int kSampleTile = kBlock * kSampleItems;       // candidates per block
+
+struct Rows {
+    float4 r1, r2, r3;
+};
+
+__device__ __forceinline__ Rows load_rows(const float* w2c) {
+    Rows r;
+    r.r1 = make_float4(w2c[0], w2c[1], w2c[2], w2c[3]);
+    r.r2 = make_float4(w2c[4], w2c[5], w2c[6], w2c[7]);
+    r.r3 = make_float4(w2c[8], w2c[9], w2c[10], w2c[11]);
+    return r;
+}
+
+// Conjunction of "inside" comparisons (NaN is not visible), sampling_kernels.cu:31-36.
+__device__ __forceinline__ bool leaf_point_visible(const Rows& m, float x, float y, float z, const Camera& cam) {
+    const float vz = affine_row(m.r3, x, y, z);
+    const float inv_z = 1.0f / (vz + kFltEps);
+    const float sx = affine_row(m.r1, x, y, z) * inv_z * cam.fx + cam.cx;
+    const float sy = affine_row(m.r2, x, y, z) * inv_z * cam.fy + cam.cy;
+    return (vz >= cam.near_plane) & (vz <= cam.far_plane) & (sx >= 0.0f) & (sx < cam.width) & (sy >= 0.0f) &
+           (sy < cam.height);
+}
+
+// Sequence of "outside" rejections (NaN is not rejected), sampling_kernels.cu:110-119.
+__device__ __forceinline__ bool sample_accepted(const Rows& m, float x, float y, float z, const Camera& cam) {
+    const float vz = affine_row(m.r3, x, y, z);
+    if (vz < cam.near_plane || vz > cam.far_plane) return false;
+    const float inv_z = 1.0f / (vz + kFltEps);
+    const float sx = affine_row(m.r1, x, y, z) * inv_z * cam.fx + cam.cx;
+    if (sx < 0.0f || sx >= cam.width) return false;
+    const float sy = affine_row(m.r2, x, y, z) * inv_z * cam.fy + cam.cy;
+    if (sy < 0.0f || sy >= cam.height) return false;
+    return true;
+}
+
+__global__ void __launch_bounds__(kBlock) k_leaf_weights(const float* __restrict__ centers,
+                                                         const int32_t* __restrict__ levels,
+                                                         const float* __restrict__ weights,
+                                                         const float* __restrict__ w2c, float* __restrict__ out,
+                                                         uint32_t n_leaves, Camera cam, float initial_size) {
+    const uint32_t l = blockIdx.x * kBlock + threadIdx.x;
+    if (l >= n_leaves) return;
+    const Rows m = load_rows(w2c);
+    const float cx = centers[3 * (size_t)l], cy = centers[3 * (size_t)l + 1], cz = centers[3 * (size_t)l + 2];
+    const int level = levels[l];
+    const float z = affine_row(m.r3, cx, cy, cz);
+    bool valid = leaf_point_visible(m, cx, cy, cz, cam);
+    if (!valid) {
+        const float half = ldexpf(initial_size, -(level + 1));
+        for (int corner = 0; corner < 8; ++corner) {
+            const float ox = (corner & 4) ? half : -half;
+            const float oy = (corner & 2) ? half : -half;
+            const float oz = (corner & 1) ? half : -half;
+            valid = valid | leaf_point_visible(m, cx + ox, cy + oy, cz + oz, cam);
+        }
+    }
+    float wgt = 0.0f;
+    if (valid) {
+        const float depth_scale = fmaxf(fabsf(z - cam.near_plane) / cam.far_plane, kFltEps);
+        const float size_scale = ldexpf((level & 1) ? 1.41421356f : 1.0f, level >> 1);
+        wgt = 1.0f / (depth_scale * size_scale) * weights[l];
+    }
+    out[l] = wgt;
+}
+
+// One wave per block; the block stages 64 chunks of 64 floats through LDS (coalesced), lane c adds
+// up chunk c left to right. SCAN = false: totals only. SCAN = true: in-place inclusive scan inside
+// each chunk, optionally after multiplying by 1/(*norm_sum).
+template <bool SCAN>
+__global__ void __launch_bounds__(kWave) k_chunk_pass(float* data, uint32_t n, float* __restrict__ totals,
+                                                      const float* __restrict__ guard_sum,
+                                                      const float* __restrict__ norm_sum) {
+    __shared__ float tile[kChunksPerBlock * (kChunk + 1)];
+    if (guard_sum && !(*guard_sum > 0.0f)) return;
+    const uint32_t lane = threadIdx.x;
+    const size_t base = (size_t)blockIdx.x * kChunkTile;
+    float norm = 1.0f;
+    const bool normalise = SCAN && norm_sum != nullptr;
+    if (normalise) norm = 1.0f / *norm_sum;
+    for (int r = 0; r < kChunksPerBlock; ++r) {
+        const size_t i = base + (size_t)r * kChunk + lane;
+        float v = i < n ? data[i] : 0.0f;
+        if (normalise) v *= norm;
+        tile[r * (kChunk + 1) + lane] = v;
+    }
+    __syncthreads();
+    const size_t chunk_base = base + (size_t)lane * kChunk;
+    if (chunk_base < n) {
+        const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
+        float* row = tile + lane * (kChunk + 1);
+        float s = row[0];
+        for (int i = 1; i < len; ++i) {
+            s += row[i];
+            if (SCAN) row[i] = s;
+        }
+        totals[(size_t)blockIdx.x * kChunksPerBlock + lane] = s;
+    }
+    if (SCAN) {
+        __syncthreads();
+        for (int r = 0; r < kChunksPerBlock; ++r) {
+            const size_t i = base + (size_t)r * kChunk + lane;
+            if (i < n) data[i] = tile[r * (kChunk + 1) + lane];
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) k_chunk_add_prefix(float* data, uint32_t n,
+                                                             const float* __restrict__ inclusive_totals,
+                                                             const float* __restrict__ guard_sum) {
+    if (guard_sum && !(*guard_sum > 0.0f)) return;
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t c = i >> 6;
+    if (c == 0) return;
+    data[i] = inclusive_totals[c - 1] + data[i];
+}
+
+// std::lower_bound with the probe sequence of B/sampling/include/sampling_utils.h:49-69.
+__device__ __forceinline__ uint32_t cdf_search(const float* __restrict__ cdf, float sample, uint32_t n) {
+    uint32_t first = 0, count = n;
+    while (count > 0) {
+        const uint32_t step = count >> 1;
+        const uint32_t it = first + step;
+        if (cdf[it] < sample) {
+            first = it + 1;
+            count -= step + 1;
+        } else {
+            count = step;
+        }
+    }
+    return min(first, n - 1);
+}
+
+struct Candidate {
+    uint32_t leaf;
+    float x, y, z;
+};
+
+// `r` stands at draw 4*k; leaves it at 4*k + 4.
+__device__ __forceinline__ Candidate draw_candidate(Pcg32& r, const float* __restrict__ centers,
+                                                    const int32_t* __restrict__ levels,
+                                                    const float* __restrict__ cdf, uint32_t n_leaves,
+                                                    float initial_size) {
+    const float u = pcg_float(r);
+    const float ox = pcg_float(r), oy = pcg_float(r), oz = pcg_float(r);
+    Candidate c;
+    c.leaf = cdf_search(cdf, u, n_leaves);
+    const float scale = ldexpf(1.0f, -levels[c.leaf]) * initial_size;
+    c.x = centers[3 * (size_t)c.leaf] + (ox - 0.5f) * scale;
+    c.y = centers[3 * (size_t)c.leaf + 1] + (oy - 0.5f) * scale;
+    c.z = centers[3 * (size_t)c.leaf + 2] + (oz - 0.5f) * scale;
+    return c;
+}
+
+// Generator of the first candidate of this thread: tile start (uniform jump) then 4*tid draws.
+__device__ __forceinline__ Pcg32 thread_generator(const uint64_t* rng_dev, uint64_t first_candidate_of_block) {
+    Pcg32 r{rng_dev[0], rng_dev[1]};
+    r.state = pcg_apply(pcg_jump(r.inc, 4ull * first_candidate_of_block), r.state);
+    r.state = pcg_apply(pcg_jump(r.inc, 4ull * threadIdx.x), r.state);
+    return r;
+}
+
+__global__ void __launch_bounds__(kBlock) k_sample(const float* __restrict__ centers,
+                                                   const int32_t* __restrict__ levels,
+                                                   const float* __restrict__ cdf, const float* __restrict__ sum_dev,
+                                                   float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
+                                                   uint32_t n_samples, uint32_t n_leaves, float initial_size,
+                                                   const uint64_t* __restrict__ rng_dev) {
+    if (!(*sum_dev > 0.0f)) return;
+    const uint64_t tile_first = (uint64_t)blockIdx.x * kSampleTile;
+    Pcg32 r = thread_generator(rng_dev, tile_first);
+    const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);  // from draw 4k+4 to 4(k+256)
+    for (int j = 0; j < kSampleItems; ++j) {
+        const uint64_t k = tile_first + (uint64_t)j * kBlock + threadIdx.x;
+        if (k < n_samples) {
+            const Candidate c = draw_candidate(r, centers, levels, cdf, n_leaves, initial_size);
+            positions[3 * k] = c.x;
+            positions[3 * k + 1] = c.y;
+            positions[3 * k + 2] = c.z;
+            if (leaf_ids) leaf_ids[k] = (int32_t)c.leaf;
+            r.state = pcg_apply(step, r.state);
+        }
+    }
+}
+
+// Advance the device generator by `mult * (*count_ptr or count)` draws, guarded by sum > 0.
+__global__ void k_rng_advance(uint64_t* rng_dev, const float* sum_dev, uint64_t draws) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    if (sum_dev && !(*sum_dev > 0.0f)) return;
+    rng_dev[0] = pcg_apply(pcg_jump(rng_dev[1], draws), rng_dev[0]);
+}
+
+// ---- training sampler round ---------------------------------------------------------------------------
+struct CullState {
+    uint32_t accepted;   // samples accepted so far in this draw (a lower bound once `consumed` is set)
+    uint32_t consumed;   // candidates consumed when the capacity-th sample was accepted, else 0
+    uint32_t error;      // look-back gave up
+    uint32_t ticket;     // block ordering of the current round
+    uint32_t pad[12];
+};
+constexpr size_t kCullHeaderWords = sizeof(CullState) / 4;
+
+__global__ void __launch_bounds__(kBlock)
+    k_sample_cull(const float* __restrict__ centers, const int32_t* __restrict__ levels,
+                  const float* __restrict__ cdf, const float* __restrict__ sum_dev, const float* __restrict__ w2c,
+                  float* __restrict__ positions, int32_t* __restrict__ leaf_ids, uint32_t capacity, uint32_t k0,
+                  uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam, float initial_size,
+                  const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
+    __shared__ uint32_t s_bid, s_accepted0, s_exclusive, s_done;
+    __shared__ uint32_t s_count[kSampleItems * (kBlock / kWave)];
+    if (!(*sum_dev > 0.0f)) return;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    if (tid == 0) {
+        const uint32_t bid = atomicAdd(&st->ticket, 1u);
+        s_bid = bid;
+        s_accepted0 = __hip_atomic_load(&st->accepted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t done = __hip_atomic_load(&st->consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+        s_done = done;
+        if (done) {
+            // The draw is already complete: tell later blocks that everything is taken.
+            status_store(status + bid, kFlagInclusive | min(capacity, kValueMask));
+            if (bid == n_blocks - 1) st->accepted = max(s_accepted0, capacity);
+        }
+    }
+    __syncthreads();
+    if (s_done) return;
+    const uint32_t bid = s_bid;
+    const uint64_t tile_first = (uint64_t)bid * kSampleTile;  // relative to k0
+    const Rows m = load_rows(w2c);
+    Pcg32 r = thread_generator(rng_dev, (uint64_t)k0 + tile_first);
+    const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);
+
+    Candidate cand[kSampleItems];
+    uint32_t rank[kSampleItems];
+    bool keep[kSampleItems];
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) {
+        const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
+        keep[j] = false;
+        if (rel < n_candidates) {
+            cand[j] = draw_candidate(r, centers, levels, cdf, n_leaves, initial_size);
+            keep[j] = sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
+            r.state = pcg_apply(step, r.state);
+        }
+        const uint64_t ballot = __ballot(keep[j]);
+        rank[j] = mask_rank(ballot);
+        if (lane == 0) s_count[j * (kBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t run = 0;
+        for (int e = 0; e < kSampleItems * (kBlock / kWave); ++e) {
+            const uint32_t c = s_count[e];
+            s_count[e] = run;
+            run += c;
+        }
+        const uint32_t exclusive = lookback_exclusive(status, 1u, bid, run, &st->error);
+        s_exclusive = exclusive;
+        if (bid == n_blocks - 1) st->accepted = s_accepted0 + exclusive + run;
+    }
+    __syncthreads();
+    const uint64_t base = (uint64_t)s_accepted0 + s_exclusive;
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) {
+        if (!keep[j]) continue;
+        const uint64_t slot = base + s_count[j * (kBlock / kWave) + wave] + rank[j];
+        if (slot >= capacity) continue;
+        positions[3 * slot] = cand[j].x;
+        positions[3 * slot + 1] = cand[j].y;
+        positions[3 * slot + 2] = cand[j].z;
+        leaf_ids[slot] = (int32_t)cand[j].leaf;
+        if (slot + 1 == capacity) {
+            const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
+            __hip_atomic_store(&st->consumed, (uint32_t)(k0 + rel + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+__global__ void k_cull_round_reset(CullState* st, uint32_t* status, uint32_t n_blocks) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i == 0) st->ticket = 0u;
+    if (i < n_blocks) status[i] = 0u;
+}
+
+// Failure pattern of B/sampling/src/sampling.cu:107-111 when the weight sum is not positive.
+__global__ void __launch_bounds__(kBlock) k_cull_failure_fill(const float* __restrict__ sum_dev, float* positions,
+                                                              int32_t* leaf_ids, uint32_t capacity) {
+    if (*sum_dev > 0.0f) return;
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= capacity) return;
+    positions[3 * (size_t)i] = 0.0f;
+    positions[3 * (size_t)i + 1] = 0.0f;
+    positions[3 * (size_t)i + 2] = 0.0f;
+    leaf_ids[i] = -1;
+}
+
+__global__ void k_cull_finish(const float* sum_dev, uint64_t* rng_dev, const CullState* st, uint32_t capacity,
+                              uint32_t total_candidates) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    if (!(*sum_dev > 0.0f)) return;
+    const uint32_t consumed = st->consumed != 0u ? st->consumed : total_candidates;
+    (void)capacity;
+    rng_dev[0] = pcg_apply(pcg_jump(rng_dev[1], 4ull * consumed), rng_dev[0]);
+}
+
+__global__ void __launch_bounds__(kBlock) k_widen_ids(const int32_t* __restrict__ ids, int64_t* __restrict__ out,
+                                                      uint32_t n) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) out[i] = (int64_t)ids[i];
+}
+
+// ---- expected-count sampler -------------------------------------------------------------------------
+constexpr int kCountItems = 4;
+constexpr int kCountTile = kBlock * kCountItems;
+
+struct ScanState {
+    uint32_t ticket;
+    uint32_t error;
+    uint32_t pad[14];
+};
+constexpr size_t kScanHeaderWords = sizeof(ScanState) / 4;
+
+// Block-wide exclusive scan of one value per thread (256 threads); returns the block total in `total`.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s_wave /*4*/, uint32_t& total) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(incl, d, 64);
+        if (lane >= (uint32_t)d) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t wave_base = 0, t = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w) {
+        const uint32_t c = s_wave[w];
+        if ((uint32_t)w < wave) wave_base += c;
+        t += c;
+    }
+    total = t;
+    __syncthreads();
+    return wave_base + incl - v;
+}
+
+// counts + inclusive integer scan in one pass (thread owns 4 consecutive leaves).
+__global__ void __launch_bounds__(kBlock)
+    k_expected_counts(const float* __restrict__ weights, const float* __restrict__ sum_dev,
+                      int32_t* __restrict__ offsets, uint32_t n_samples, uint32_t n_leaves, ScanState* st,
+                      uint32_t* status) {
+    __shared__ uint32_t s_bid, s_exclusive;
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    const float sum = *sum_dev;
+    if (!(sum > 0.0f)) return;
+    if (threadIdx.x == 0) s_bid = atomicAdd(&st->ticket, 1u);
+    __syncthreads();
+    const uint32_t bid = s_bid;
+    const size_t first = (size_t)bid * kCountTile + (size_t)threadIdx.x * kCountItems;
+    const float norm = 1.0f / sum;
+    uint32_t count[kCountItems];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kCountItems; ++j) {
+        count[j] = 0;
+        const size_t l = first + j;
+        if (l < n_leaves) {
+            const float w = weights[l];
+            if (w > 0.0f) count[j] = (uint32_t)max(__float2int_rn(w * norm * (float)n_samples), 1);
+        }
+        mine += count[j];
+    }
+    uint32_t total;
+    const uint32_t local = block_exclusive_scan(mine, s_wave, total);
+    if (threadIdx.x == 0) s_exclusive = lookback_exclusive(status, 1u, bid, total, &st->error);
+    __syncthreads();
+    uint32_t run = s_exclusive + local;
+#pragma unroll
+    for (int j = 0; j < kCountItems; ++j) {
+        const size_t l = first + j;
+        run += count[j];
+        if (l < n_leaves) offsets[l] = (int32_t)run;
+    }
+}
+
+// ids[offsets[l-1] .. offsets[l]) = l; one wave per 64 leaves, lanes stride over each leaf's run.
+__global__ void __launch_bounds__(kBlock) k_repeat_interleave(const int32_t* __restrict__ offsets,
+                                                              int32_t* __restrict__ ids, uint32_t n_leaves) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave_global = (blockIdx.x * kBlock + threadIdx.x) >> 6;
+    const uint32_t l0 = wave_global * 64u;
+    for (uint32_t l = l0; l < min(l0 + 64u, n_leaves); ++l) {
+        const int32_t b = l == 0 ? 0 : offsets[l - 1], e = offsets[l];
+        for (int32_t i = b + (int32_t)lane; i < e; i += 64) ids[i] = (int32_t)l;
+    }
+}
+
+__global__ void __launch_bounds__(kBlock)
+    k_expected_samples(const float* __restrict__ centers, const int32_t* __restrict__ levels,
+                       const int32_t* __restrict__ ids, float* __restrict__ positions, uint32_t n_total,
+                       uint32_t n_created, float initial_size, const uint64_t* __restrict__ rng_dev) {
+    const uint64_t tile_first = (uint64_t)blockIdx.x * kSampleTile;
+    Pcg32 r{rng_dev[0], rng_dev[1]};
+    r.state = pcg_apply(pcg_jump(r.inc, 3ull * tile_first), r.state);
+    r.state = pcg_apply(pcg_jump(r.inc, 3ull * threadIdx.x), r.state);
+    const PcgJump step = pcg_jump(r.inc, 3ull * kBlock - 3ull);
+    for (int j = 0; j < kSampleItems; ++j) {
+        const uint64_t s = tile_first + (uint64_t)j * kBlock + threadIdx.x;
+        if (s < n_total) {
+            const int32_t leaf = ids[s % n_created];
+            const float ox = pcg_float(r), oy = pcg_float(r), oz = pcg_float(r);
+            const float scale = ldexpf(1.0f, -levels[leaf]) * initial_size;
+            positions[3 * s] = centers[3 * (size_t)leaf] + (ox - 0.5f) * scale;
+            positions[3 * s + 1] = centers[3 * (size_t)leaf + 1] + (oy - 0.5f) * scale;
+            positions[3 * s + 2] = centers[3 * (size_t)leaf + 2] + (oz - 0.5f) * scale;
+            r.state = pcg_apply(step, r.state);
+        }
+    }
+}
+
+// Chunk-total levels for n leaves: sizes n1 = ceil(n/64), n2 = ceil(n1/64), ... down to 1.
+struct LevelPlan {
+    int n_levels;
+    uint32_t size[8];
+    size_t offset[8];  // in floats, from the start of the totals area
+    size_t total_floats;
+};
+
+LevelPlan plan_levels(uint32_t n) {
+    LevelPlan p{};
+    uint32_t m = n;
+    size_t off = 0;
+    do {
+        m = div_up(m, kChunk);
+        p.size[p.n_levels] = m;
+        p.offset[p.n_levels] = off;
+        off += align_up(m, 64);
+        ++p.n_levels;
+    } while (m > 1 && p.n_levels < 8);
+    p.total_floats = off;
+    return p;
+}
+
+// Canonical total of `data` (n floats) into *sum_out; `totals` is scratch of plan.total_floats.
+int launch_blocked_total(const float* data, uint32_t n, float* totals, float* sum_out, const LevelPlan& plan,
+                         hipStream_t stream) {
+    const float* cur = data;
+    uint32_t m = n;
+    for (int lv = 0; lv < plan.n_levels; ++lv) {
+        float* dst = (lv == plan.n_levels - 1) ? sum_out : totals + plan.offset[lv];
+        INPC_LAUNCH("chunk_reduce", k_chunk_pass<false>, dim3(div_up(m, kChunkTile)), dim3(kWave), stream,
+                    const_cast<float*>(cur), m, dst, (const float*)nullptr, (const float*)nullptr);
+        cur = dst;
+        m = plan.size[lv];
+    }
+    return INPC_OK;
+}
+
+}  // namespace
+
+size_t sampler_workspace_bytes(uint32_t n_leaves) {
+    const LevelPlan plan = plan_levels(std::max(n_leaves, 1u));
+    const uint32_t scan_blocks = div_up(std::max(n_leaves, 1u), kCountTile);
+    return align_up(plan.total_floats * 4, 256) + align_up((kScanHeaderWords + scan_blocks) * 4, 256) + 256;
+}
+
+}  // namespace inpc
+
+using namespace inpc;
+
+extern "C" {
+
+int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* weights, const float* w2c,
+                      float* out, uint32_t n_leaves, const inpc_camera* cam, float initial_size, void* stream) {
+    if (!cam) return fail(INPC_E_INVALID_ARGUMENT, "inpc_leaf_weights: camera is null");
+    if (n_leaves == 0) return INPC_OK;
+    if (!centers || !levels || !weights || !w2c || !out)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_leaf_weights: null pointer");
+    INPC_LAUNCH("leaf_weights", k_leaf_weights, dim3(div_up(n_leaves, kBlock)), dim3(kBlock), (hipStream_t)stream,
+                centers, levels, weights, w2c, out, n_leaves, to_device_camera(*cam), initial_size);
+    return INPC_OK;
+}
+
+size_t inpc_sampler_workspace_bytes(uint32_t n_leaves) { return sampler_workspace_bytes(n_leaves); }
+
+int inpc_build_cdf(float* w, float* sum_out, void* workspace, size_t workspace_bytes, uint32_t n_leaves,
+                   void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n_leaves == 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: no leaves");
+    if (!w || !sum_out || !workspace) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: null pointer");
+    if (workspace_bytes < sampler_workspace_bytes(n_leaves))
+        return fail(INPC_E_WORKSPACE, "inpc_build_cdf: workspace has %zu bytes, needs %zu", workspace_bytes,
+                    sampler_workspace_bytes(n_leaves));
+    const LevelPlan plan = plan_levels(n_leaves);
+    float* totals = (float*)workspace;
+    int rc = launch_blocked_total(w, n_leaves, totals, sum_out, plan, stream);
+    if (rc != INPC_OK) return rc;
+    // down: local scans, level 0 normalises; stops once a level has a single chunk
+    float* cur = w;
+    uint32_t m = n_leaves;
+    int depth = 0;
+    for (;;) {
+        float* tot = totals + plan.offset[depth];
+        INPC_LAUNCH("chunk_scan", k_chunk_pass<true>, dim3(div_up(m, kChunkTile)), dim3(kWave), stream, cur, m, tot,
+                    (const float*)sum_out, depth == 0 ? (const float*)sum_out : (const float*)nullptr);
+        if (plan.size[depth] == 1) break;
+        cur = tot;
+        m = plan.size[depth];
+        ++depth;
+    }
+    // up: add the scanned chunk totals of level d+1 to level d
+    for (int d = depth - 1; d >= 0; --d) {
+        float* dst = d == 0 ? w : totals + plan.offset[d - 1];
+        const uint32_t dn = d == 0 ? n_leaves : plan.size[d - 1];
+        INPC_LAUNCH("chunk_add_prefix", k_chunk_add_prefix, dim3(div_up(dn, kBlock)), dim3(kBlock), stream, dst, dn,
+                    (const float*)(totals + plan.offset[d]), (const float*)sum_out);
+    }
+    return INPC_OK;
+}
+
+int inpc_sample(const float* centers, const int32_t* levels, const float* cdf, const float* sum_dev,
+                float* positions_out, int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves,
+                float initial_size, uint64_t* rng_dev, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n_samples == 0) return INPC_OK;
+    if (n_samples >= (1u << 30)) return fail(INPC_E_UNSUPPORTED, "inpc_sample: n_samples must be below 2^30");
+    if (n_leaves == 0 || !centers || !levels || !cdf || !sum_dev || !positions_out || !rng_dev)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: null pointer or no leaves");
+    INPC_LAUNCH("sample", k_sample, dim3(div_up(n_samples, kSampleTile)), dim3(kBlock), stream, centers, levels, cdf,
+                sum_dev, positions_out, leaf_ids_out, n_samples, n_leaves, initial_size, (const uint64_t*)rng_dev);
+    INPC_LAUNCH("rng_advance", k_rng_advance, dim3(1), dim3(64), stream, rng_dev, sum_dev, 4ull * n_samples);
+    return INPC_OK;
+}
+
+size_t inpc_cull_workspace_bytes(uint32_t n_candidates) {
+    return align_up((kCullHeaderWords + div_up(std::max(n_candidates, 1u), kSampleTile)) * 4, 256);
+}
+
+int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream) {
+    if (!workspace || workspace_bytes < sizeof(CullState))
+        return fail(INPC_E_WORKSPACE, "inpc_cull_begin: workspace too small");
+    return fill_u32(workspace, 0u, kCullHeaderWords, (hipStream_t)stream);
+}
+
+int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const float* cdf, const float* sum_dev,
+                             const float* w2c, float* positions_out, int32_t* leaf_ids_out, uint32_t capacity,
+                             uint32_t k0, uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam,
+                             float initial_size, const uint64_t* rng_dev, void* workspace, size_t workspace_bytes,
+                             void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n_candidates == 0) return INPC_OK;
+    if (!cam || n_leaves == 0 || !centers || !levels || !cdf || !sum_dev || !w2c || !positions_out || !leaf_ids_out ||
+        !rng_dev || !workspace)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample_cull_compact: null pointer or no leaves");
+    if ((uint64_t)k0 + n_candidates >= (1ull << 30))
+        return fail(INPC_E_UNSUPPORTED, "inpc_sample_cull_compact: candidate index must stay below 2^30");
+    if (workspace_bytes < inpc_cull_workspace_bytes(n_candidates))
+        return fail(INPC_E_WORKSPACE, "inpc_sample_cull_compact: workspace has %zu bytes, needs %zu", workspace_bytes,
+                    inpc_cull_workspace_bytes(n_candidates));
+    CullState* st = (CullState*)workspace;
+    uint32_t* status = (uint32_t*)workspace + kCullHeaderWords;
+    const uint32_t n_blocks = div_up(n_candidates, kSampleTile);
+    INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(n_blocks, kBlock)), dim3(kBlock), stream, st,
+                status, n_blocks);
+    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(n_blocks), dim3(kBlock), stream, centers, levels, cdf,
+                sum_dev, w2c, positions_out, leaf_ids_out, capacity, k0, n_candidates, n_blocks, n_leaves,
+                to_device_camera(*cam), initial_size, rng_dev, st, status);
+    return INPC_OK;
+}
+
+int inpc_cull_read_counts(const void* workspace, uint32_t* accepted_host, uint32_t* consumed_host, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    uint32_t host[3] = {0, 0, 0};
+    INPC_HIP_CHECK(hipMemcpyAsync(host, workspace, sizeof(host), hipMemcpyDeviceToHost, stream));
+    INPC_HIP_CHECK(hipStreamSynchronize(stream));
+    if (accepted_host) *accepted_host = host[0];
+    if (consumed_host) *consumed_host = host[1];
+    if (host[2]) return fail(INPC_E_DEVICE, "sampler look-back gave up waiting (device error flag set)");
+    return INPC_OK;
+}
+
+int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_ids_out, uint32_t capacity,
+                     uint32_t total_candidates, uint64_t* rng_dev, void* workspace, size_t workspace_bytes,
+                     void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!sum_dev || !rng_dev || !workspace || workspace_bytes < sizeof(CullState))
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_cull_finish: null pointer");
+    if (capacity > 0 && positions_out && leaf_ids_out)
+        INPC_LAUNCH("cull_failure_fill", k_cull_failure_fill, dim3(div_up(capacity, kBlock)), dim3(kBlock), stream,
+                    sum_dev, positions_out, leaf_ids_out, capacity);
+    INPC_LAUNCH("cull_finish", k_cull_finish, dim3(1), dim3(64), stream, sum_dev, rng_dev, (const CullState*)workspace,
+                capacity, total_candidates);
+    return INPC_OK;
+}
+
+int inpc_widen_ids(const int32_t* ids, int64_t* out, uint32_t n, void* stream) {
+    if (n == 0) return INPC_OK;
+    INPC_LAUNCH("widen_ids", k_widen_ids, dim3(div_up(n, kBlock)), dim3(kBlock), (hipStream_t)stream, ids, out, n);
+    return INPC_OK;
+}
+
+int inpc_expected_counts(const float* weights, float* sum_out, int32_t* offsets_out, uint32_t n_samples,
+                         void* workspace, size_t workspace_bytes, uint32_t n_leaves, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n_leaves == 0 || !weights || !sum_out || !offsets_out || !workspace)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_expected_counts: null pointer or no leaves");
+    if (workspace_bytes < sampler_workspace_bytes(n_leaves))
+        return fail(INPC_E_WORKSPACE, "inpc_expected_counts: workspace too small");
+    const LevelPlan plan = plan_levels(n_leaves);
+    float* totals = (float*)workspace;
+    int rc = launch_blocked_total(weights, n_leaves, totals, sum_out, plan, stream);
+    if (rc != INPC_OK) return rc;
+    uint32_t* scan = (uint32_t*)((char*)workspace + align_up(plan.total_floats * 4, 256));
+    const uint32_t n_blocks = div_up(n_leaves, kCountTile);
+    rc = fill_u32(scan, 0u, kScanHeaderWords + n_blocks, stream);
+    if (rc != INPC_OK) return rc;
+    rc = fill_u32(offsets_out, 0u, n_leaves, stream);  // sum <= 0 leaves all offsets at zero
+    if (rc != INPC_OK) return rc;
+    INPC_LAUNCH("expected_counts", k_expected_counts, dim3(n_blocks), dim3(kBlock), stream, weights,
+                (const float*)sum_out, offsets_out, n_samples, n_leaves, (ScanState*)scan, scan + kScanHeaderWords);
+    return INPC_OK;
+}
+
+int inpc_expected_samples(const float* centers, const int32_t* levels, const int32_t* offsets,
+                          int32_t* leaf_ids_scratch, float* positions_out, uint32_t n_created, uint32_t n_multi,
+                          uint32_t n_leaves, float initial_size, uint64_t* rng_dev, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    const uint64_t total64 = (uint64_t)n_created * n_multi;
+    if (total64 == 0) return INPC_OK;
+    if (total64 >= (1ull << 30)) return fail(INPC_E_UNSUPPORTED, "inpc_expected_samples: too many samples");
+    if (!centers || !levels || !offsets || !leaf_ids_scratch || !positions_out || !rng_dev)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_expected_samples: null pointer");
+    const uint32_t n_total = (uint32_t)total64;
+    INPC_LAUNCH("repeat_interleave", k_repeat_interleave, dim3(div_up(div_up(n_leaves, 64u) * 64u, kBlock)),
+                dim3(kBlock), stream, offsets, leaf_ids_scratch, n_leaves);
+    INPC_LAUNCH("expected_samples", k_expected_samples, dim3(div_up(n_total, kSampleTile)), dim3(kBlock), stream,
+                centers, levels, (const int32_t*)leaf_ids_scratch, positions_out, n_total, n_created, initial_size,
+                (const uint64_t*)rng_dev);
+    INPC_LAUNCH("rng_advance", k_rng_advance, dim3(1), dim3(64), stream, rng_dev, (const float*)nullptr,
+                3ull * n_total);
+    return INPC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,250 @@
+"""Rasterizer operator API: `INPCRasterizer`, `RasterizerSettings`, `RasterizerMode`.
+
+Same names, arguments and error behaviour as B/torch_bindings/rasterization.py:15-189; the native
+side is libinpc_hip.so instead of the pybind11 module `_C`. On top of the reference's fixed shape
+(8x8 tiles, (N,36) fp16 SH features -> 4 channels) the constructor accepts the tile size, and
+`rasterize_points` exposes the direct-feature variants (C in {4, 8, 16}, fp32 or fp16 storage).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import logging
+from enum import Enum
+from typing import Any, NamedTuple, Optional
+
+import torch
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+from .views import is_perspective
+
+_log = logging.getLogger("inpc_amd")
+
+
+class RasterizerMode(Enum):
+    BILINEAR = 0
+    GAUSSIAN = 1
+
+
+class RasterizerSettings(NamedTuple):
+    w2c: torch.Tensor
+    cam_position: torch.Tensor
+    mode: RasterizerMode
+    width: int
+    height: int
+    focal_x: float
+    focal_y: float
+    center_x: float
+    center_y: float
+    near_plane: float
+    far_plane: float
+
+    def as_tuple(self) -> tuple:
+        return (self.w2c, self.cam_position, self.mode.value, self.width, self.height, self.focal_x, self.focal_y,
+                self.center_x, self.center_y, self.near_plane, self.far_plane)
+
+    def camera(self) -> _lib.Camera:
+        return _lib.Camera(int(self.width), int(self.height), float(self.focal_x), float(self.focal_y),
+                           float(self.center_x), float(self.center_y), float(self.near_plane), float(self.far_plane))
+
+
+_FEATURE_MODES = {"sh36": _lib.FEAT_SH36_F16, "f32": _lib.FEAT_DIRECT_F32, "f16": _lib.FEAT_DIRECT_F16,
+                  "raw37": _lib.FEAT_RAW37_F16}
+
+
+def _require_bilinear(settings: RasterizerSettings) -> None:
+    if settings.mode != RasterizerMode.BILINEAR:
+        # the reference throws std::runtime_error("unsupported rasterizer mode") for modes its
+        # native side does not know (B/rasterization/src/rasterization_api.cu:102-103); the
+        # Gaussian footprint is not part of this library
+        raise RuntimeError("unsupported rasterizer mode")
+
+
+def _config(settings: RasterizerSettings, n_points: int, tile: int, channels: int, feature_mode: int,
+            inference: bool) -> _lib.RasterConfig:
+    return _lib.RasterConfig(int(n_points), int(tile), int(channels), int(feature_mode),
+                             _lib.RASTER_INFERENCE if inference else 0, settings.camera())
+
+
+def query_layout(cfg: _lib.RasterConfig) -> _lib.RasterLayout:
+    layout = _lib.RasterLayout()
+    _lib.check(_lib.lib().inpc_raster_layout_query(C.byref(cfg), C.byref(layout)), "inpc_raster_layout_query")
+    return layout
+
+
+def _checked_inputs(positions, features, opacities, feature_mode: int, channels: int):
+    positions = positions.contiguous()
+    features = features.contiguous()
+    if positions.dtype != torch.float32:
+        raise RuntimeError("expected scalar type Float")
+    want = torch.float32 if feature_mode == _lib.FEAT_DIRECT_F32 else torch.float16
+    if features.dtype != want:
+        raise RuntimeError("expected scalar type Float" if want == torch.float32 else "expected scalar type Half")
+    n = positions.shape[0]
+    width = {_lib.FEAT_SH36_F16: 36, _lib.FEAT_RAW37_F16: 37}.get(feature_mode, channels)
+    if features.numel() != n * width:
+        raise RuntimeError(f"features must hold {width} values per point")
+    if opacities is not None:
+        opacities = opacities.contiguous()
+        if opacities.dtype != torch.float32:
+            raise RuntimeError("expected scalar type Float")
+        if opacities.numel() != n:
+            raise RuntimeError("opacities must hold one value per point")
+    if not positions.is_cuda or not features.is_cuda:
+        raise RuntimeError("expected tensors on the GPU")
+    return positions, features, opacities
+
+
+def _forward_native(settings: RasterizerSettings, positions, features, opacities, tile: int, channels: int,
+                    feature_mode: int, inference: bool):
+    """Runs inpc_raster_forward. Returns (image, alpha, third, workspace, cfg) where `third` is the
+    blending weights (training) or the depth image (inference)."""
+    _require_bilinear(settings)
+    n = positions.shape[0]
+    device = positions.device
+    sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
+    out_channels = 4 if sh else channels
+    cfg = _config(settings, n, tile, out_channels, feature_mode, inference)
+    layout = query_layout(cfg)
+    workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+    H, W = settings.height, settings.width
+    image = torch.empty((out_channels, H, W), dtype=torch.float32, device=device)
+    alpha = torch.empty((1, H, W), dtype=torch.float32, device=device)
+    weights = None if inference else torch.empty(n, dtype=torch.float32, device=device)
+    depth = torch.empty((1, H, W), dtype=torch.float32, device=device) if inference else None
+    w2c = settings.w2c.contiguous()
+    cam_position = settings.cam_position.contiguous()
+    _lib.check(_lib.lib().inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features),
+                                              _lib.ptr(opacities), _lib.ptr(w2c), _lib.ptr(cam_position),
+                                              _lib.ptr(image), _lib.ptr(alpha), _lib.ptr(weights), _lib.ptr(depth),
+                                              _lib.ptr(workspace), layout.total_bytes, _lib.current_stream()),
+               "inpc_raster_forward")
+    return image, alpha, (depth if inference else weights), workspace, cfg
+
+
+class _Rasterize(torch.autograd.Function):
+    """Counterpart of B/torch_bindings/rasterization.py:49-101."""
+
+    @staticmethod
+    def forward(ctx: Any, positions: torch.Tensor, features: torch.Tensor, opacities: torch.Tensor,
+                rasterizer_settings: RasterizerSettings, tile: int = 8, feature_mode: int = _lib.FEAT_SH36_F16,
+                channels: int = 4):
+        positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)
+        image, alpha, blending_weights, workspace, cfg = _forward_native(
+            rasterizer_settings, positions, features, opacities, tile, channels, feature_mode, inference=False)
+        ctx.save_for_backward(image, alpha, positions, features, opacities, workspace)
+        ctx.rasterizer_settings = rasterizer_settings
+        ctx.cfg = cfg
+        ctx.mark_non_differentiable(blending_weights)
+        ctx.set_materialize_grads(False)
+        return image, alpha, blending_weights
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad_image: Optional[torch.Tensor], grad_alpha: Optional[torch.Tensor], _):
+        image, alpha, positions, features, opacities, workspace = ctx.saved_tensors
+        cfg = ctx.cfg
+        settings = ctx.rasterizer_settings
+        n = positions.shape[0]
+        device = positions.device
+        # set_materialize_grads(False): an output nobody used arrives as None; substitute zeros
+        grad_image = torch.zeros_like(image) if grad_image is None else grad_image.contiguous()
+        grad_alpha = torch.zeros_like(alpha) if grad_alpha is None else grad_alpha.contiguous()
+        if grad_image.dtype != torch.float32 or grad_alpha.dtype != torch.float32:
+            raise RuntimeError("expected scalar type Float")
+        mode = cfg.feature_mode
+        scratch = None
+        if mode == _lib.FEAT_SH36_F16:
+            grad_features = torch.empty((n, 36), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
+        elif mode == _lib.FEAT_DIRECT_F16:
+            grad_features = torch.empty((n, cfg.channels), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, cfg.channels), dtype=torch.float32, device=device)
+        else:
+            grad_features = torch.empty((n, cfg.channels), dtype=torch.float32, device=device)
+        grad_opacities = torch.empty((n, 1), dtype=torch.float32, device=device)
+        cam_position = settings.cam_position.contiguous()
+        _lib.check(_lib.lib().inpc_raster_backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha),
+                                                   _lib.ptr(image), _lib.ptr(alpha), _lib.ptr(positions),
+                                                   _lib.ptr(features), _lib.ptr(opacities), _lib.ptr(cam_position),
+                                                   _lib.ptr(grad_features), _lib.ptr(grad_opacities),
+                                                   _lib.ptr(scratch), _lib.ptr(workspace), workspace.numel(),
+                                                   _lib.current_stream()), "inpc_raster_backward")
+        grad_features = grad_features.view(features.shape)
+        grad_opacities = grad_opacities.view(opacities.shape)
+        return None, grad_features, grad_opacities, None, None, None, None
+
+
+class INPCRasterizer(torch.nn.Module):
+    """Counterpart of B/torch_bindings/rasterization.py:104-189. `tile` is 8 in the reference
+    (B/rasterization/include/bilinear/config.h:23-25); 16 is the other supported size."""
+
+    def __init__(self, tile: int = 8) -> None:
+        super().__init__()
+        if tile not in (8, 16):
+            raise ValueError("tile must be 8 or 16")
+        self.tile = tile
+
+    @staticmethod
+    def extract_settings(view, mode: int) -> RasterizerSettings:
+        if not is_perspective(view.camera):
+            raise NotImplementedError
+        if getattr(view.camera, "distortion", None) is not None:
+            _log.warning("rasterizer ignores all distortion parameters")
+        try:
+            rasterizer_mode = RasterizerMode(mode)
+        except ValueError:
+            _log.warning("invalid rasterizer mode %s, defaulting to BILINEAR", mode)
+            rasterizer_mode = RasterizerMode.BILINEAR
+        return RasterizerSettings(view.w2c, view.position, rasterizer_mode, view.camera.width, view.camera.height,
+                                  view.camera.focal_x, view.camera.focal_y, view.camera.center_x,
+                                  view.camera.center_y, view.camera.near_plane, view.camera.far_plane)
+
+    @staticmethod
+    def extract_base_sigma_world(camera) -> float:
+        if not is_perspective(camera):
+            raise NotImplementedError
+        return 0.05 / camera.focal_y
+
+    def forward(self, view, mode: int, positions: torch.Tensor, features: torch.Tensor,
+                opacities: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """(image (4,H,W), alpha (1,H,W), blending_weights (N,)); differentiable in features and
+        opacities, positions get no gradient."""
+        return _Rasterize.apply(positions, features, opacities, self.extract_settings(view, mode), self.tile,
+                                _lib.FEAT_SH36_F16, 4)
+
+    def render(self, view, mode: int, positions: torch.Tensor, features_raw: torch.Tensor,
+               sigma_world_scale: float, sigma_cutoff: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """(image, depth, alpha) from raw (N,37) fp16 appearance output; the sigma arguments only
+        concern the Gaussian footprint and are ignored by the bilinear one, as in the reference."""
+        settings = self.extract_settings(view, mode)
+        positions, features_raw, _ = _checked_inputs(positions, features_raw, None, _lib.FEAT_RAW37_F16, 4)
+        image, alpha, depth, _, _ = _forward_native(settings, positions, features_raw, None, self.tile, 4,
+                                                    _lib.FEAT_RAW37_F16, inference=True)
+        return image, depth, alpha
+
+    def render_preextracted(self, view, mode: int, positions: torch.Tensor, features: torch.Tensor,
+                            opacities: torch.Tensor, scales: Optional[torch.Tensor] = None,
+                            sigma_world_scale: float = 1.0,
+                            sigma_cutoff: float = 3.0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        settings = self.extract_settings(view, mode)
+        positions, features, opacities = _checked_inputs(positions, features, opacities, _lib.FEAT_SH36_F16, 4)
+        image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, self.tile, 4,
+                                                    _lib.FEAT_SH36_F16, inference=True)
+        return image, depth, alpha
+
+
+def rasterize_points(view, positions: torch.Tensor, features: torch.Tensor, opacities: torch.Tensor, tile: int = 16,
+                     inference: bool = False):
+    """Direct-feature rasterization: features (N,C), C in {4, 8, 16}, fp32 or fp16 storage, blended as
+    they are. Training: (image (C,H,W), alpha, blending_weights), differentiable in features and
+    opacities. Inference: (image, depth, alpha)."""
+    settings = INPCRasterizer.extract_settings(view, RasterizerMode.BILINEAR.value)
+    channels = features.shape[-1]
+    feature_mode = _lib.FEAT_DIRECT_F32 if features.dtype == torch.float32 else _lib.FEAT_DIRECT_F16
+    if inference:
+        positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)
+        image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, tile, channels,
+                                                    feature_mode, inference=True)
+        return image, depth, alpha
+    return _Rasterize.apply(positions, features, opacities, settings, tile, feature_mode, channels)

@@ -1,0 +1,345 @@
+"""ctypes binding of the CPU oracle (oracle/inpc_oracle.cpp).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py as the checker / the timed CPU baseline. The product package
+(inpc_amd) never imports this module.
+
+Every function takes and returns numpy arrays (host memory) and mirrors one exported function
+of the oracle; the reference lines each one follows are cited in inpc_oracle.cpp.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_DIR = Path(__file__).resolve().parent
+_LIB_PATH = _DIR / "liboracle.so"
+
+FEAT_SH36_F16 = 0
+FEAT_DIRECT_F32 = 1
+FEAT_DIRECT_F16 = 2
+FEAT_RAW37_F16 = 3
+RASTER_INFERENCE = 1
+
+
+def build(force: bool = False) -> Path:
+    """Compile liboracle.so with g++ (make decides whether anything is stale)."""
+    if force and _LIB_PATH.exists():
+        _LIB_PATH.unlink()
+    subprocess.run(["make", "-C", str(_DIR), "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+class Camera(C.Structure):
+    _fields_ = [
+        ("width", C.c_int32),
+        ("height", C.c_int32),
+        ("focal_x", C.c_float),
+        ("focal_y", C.c_float),
+        ("center_x", C.c_float),
+        ("center_y", C.c_float),
+        ("near_plane", C.c_float),
+        ("far_plane", C.c_float),
+    ]
+
+
+class RasterConfig(C.Structure):
+    _fields_ = [
+        ("n_points", C.c_uint32),
+        ("tile", C.c_int32),
+        ("channels", C.c_int32),
+        ("feature_mode", C.c_int32),
+        ("flags", C.c_uint32),
+        ("cam", Camera),
+    ]
+
+
+class _RasterDebug(C.Structure):
+    _fields_ = [
+        ("n_touched", C.c_void_p),
+        ("bounds", C.c_void_p),
+        ("screen_xy", C.c_void_p),
+        ("depth", C.c_void_p),
+        ("features_view", C.c_void_p),
+        ("opacity", C.c_void_p),
+        ("counts", C.c_void_p),
+        ("depth_keys", C.c_void_p),
+        ("depth_order", C.c_void_p),
+        ("instance_keys", C.c_void_p),
+        ("instance_points", C.c_void_p),
+        ("tile_ranges", C.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            build()
+        _lib = C.CDLL(str(_LIB_PATH))
+        _lib.oracle_pcg32_next_uint.restype = C.c_uint32
+        _lib.oracle_pcg32_next_float.restype = C.c_float
+        _lib.oracle_blocked_total.restype = C.c_float
+        _lib.oracle_cdf_search.restype = C.c_uint32
+        _lib.oracle_cdf_search.argtypes = [C.c_void_p, C.c_float, C.c_uint32]
+        _lib.oracle_training_samples.restype = C.c_uint32
+        _lib.oracle_expected_counts.restype = C.c_uint32
+        _lib.oracle_float_to_half.restype = C.c_uint16
+        _lib.oracle_float_to_half.argtypes = [C.c_float]
+        _lib.oracle_half_to_float.restype = C.c_float
+        _lib.oracle_half_to_float.argtypes = [C.c_uint16]
+        _lib.oracle_now.restype = C.c_double
+        _lib.oracle_num_threads.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def make_camera(width, height, fx, fy, cx=None, cy=None, near=0.01, far=100.0) -> Camera:
+    return Camera(int(width), int(height), float(fx), float(fy),
+                  float(width / 2 if cx is None else cx), float(height / 2 if cy is None else cy),
+                  float(near), float(far))
+
+
+def num_threads() -> int:
+    return int(lib().oracle_num_threads())
+
+
+def set_num_threads(n: int) -> None:
+    lib().oracle_set_num_threads(C.c_int(int(n)))
+
+
+def now() -> float:
+    return float(lib().oracle_now())
+
+
+# ----------------------------------------------------------------------------------------------
+# pcg32
+# ----------------------------------------------------------------------------------------------
+class Pcg32:
+    """Host generator; `state` is a uint64[2] numpy array {state, inc}."""
+
+    def __init__(self, initstate: int, initseq: int = 1):
+        self.state = np.zeros(2, dtype=np.uint64)
+        lib().oracle_pcg32_seed(_p(self.state), C.c_uint64(initstate & (2**64 - 1)), C.c_uint64(initseq))
+
+    def copy(self) -> "Pcg32":
+        other = Pcg32.__new__(Pcg32)
+        other.state = self.state.copy()
+        return other
+
+    def next_uint(self) -> int:
+        return int(lib().oracle_pcg32_next_uint(_p(self.state)))
+
+    def next_float(self) -> float:
+        return float(lib().oracle_pcg32_next_float(_p(self.state)))
+
+    def advance(self, delta: int) -> None:
+        lib().oracle_pcg32_advance(_p(self.state), C.c_int64(delta))
+
+
+def float_to_half(f: float) -> int:
+    return int(lib().oracle_float_to_half(C.c_float(f)))
+
+
+def half_to_float(h: int) -> float:
+    return float(lib().oracle_half_to_float(C.c_uint16(h)))
+
+
+# ----------------------------------------------------------------------------------------------
+# sampler
+# ----------------------------------------------------------------------------------------------
+def leaf_weights(centers, levels, weights, w2c, cam: Camera, initial_size: float) -> np.ndarray:
+    centers, levels, weights, w2c = _f32(centers), _i32(levels), _f32(weights), _f32(w2c)
+    out = np.empty(len(levels), dtype=np.float32)
+    lib().oracle_leaf_weights(_p(centers), _p(levels), _p(weights), _p(w2c), _p(out), C.c_uint32(len(levels)),
+                              C.byref(cam), C.c_float(initial_size))
+    return out
+
+
+def blocked_total(w) -> np.float32:
+    w = _f32(w)
+    return np.float32(lib().oracle_blocked_total(_p(w), C.c_uint32(len(w))))
+
+
+def blocked_inclusive_scan(w) -> np.ndarray:
+    out = _f32(w).copy()
+    lib().oracle_blocked_inclusive_scan(_p(out), C.c_uint32(len(out)))
+    return out
+
+
+def build_cdf(w):
+    """Returns (ok, cdf, sum)."""
+    out = _f32(w).copy()
+    s = C.c_float(0)
+    ok = lib().oracle_build_cdf(_p(out), C.c_uint32(len(out)), C.byref(s))
+    return bool(ok), out, np.float32(s.value)
+
+
+def cdf_search(cdf, sample: float) -> int:
+    cdf = _f32(cdf)
+    return int(lib().oracle_cdf_search(_p(cdf), C.c_float(sample), C.c_uint32(len(cdf))))
+
+
+def sample(centers, levels, cdf, n_samples: int, initial_size: float, rng: Pcg32):
+    """Returns (positions (n,3), leaf ids (n,)); advances rng by 4*n."""
+    centers, levels, cdf = _f32(centers), _i32(levels), _f32(cdf)
+    pos = np.empty((n_samples, 3), dtype=np.float32)
+    ids = np.empty(n_samples, dtype=np.int32)
+    lib().oracle_sample(_p(centers), _p(levels), _p(cdf), _p(pos), _p(ids), C.c_uint32(n_samples),
+                        C.c_uint32(len(levels)), C.c_float(initial_size), _p(rng.state))
+    return pos, ids
+
+
+def sample_cull_compact(centers, levels, cdf, w2c, cam: Camera, initial_size: float, rng: Pcg32, capacity: int,
+                        k0: int, n_candidates: int, positions=None, ids=None, accepted: int = 0):
+    """One round. Returns (positions, ids, accepted, consumed)."""
+    centers, levels, cdf, w2c = _f32(centers), _i32(levels), _f32(cdf), _f32(w2c)
+    if positions is None:
+        positions = np.zeros((capacity, 3), dtype=np.float32)
+        ids = np.full(capacity, -1, dtype=np.int32)
+    acc = C.c_uint32(accepted)
+    cons = C.c_uint32(0)
+    lib().oracle_sample_cull_compact(_p(centers), _p(levels), _p(cdf), _p(w2c), _p(positions), _p(ids),
+                                     C.c_uint32(capacity), C.c_uint32(k0), C.c_uint32(n_candidates),
+                                     C.c_uint32(len(levels)), C.byref(cam), C.c_float(initial_size), _p(rng.state),
+                                     C.byref(acc), C.byref(cons))
+    return positions, ids, int(acc.value), int(cons.value)
+
+
+def training_samples(centers, levels, weights, w2c, cam: Camera, initial_size: float, rng: Pcg32, n_samples: int):
+    """Whole draw. Returns (positions, ids int32, consumed); advances rng by 4*consumed."""
+    centers, levels, weights, w2c = _f32(centers), _i32(levels), _f32(weights), _f32(w2c)
+    pos = np.empty((n_samples, 3), dtype=np.float32)
+    ids = np.empty(n_samples, dtype=np.int32)
+    consumed = lib().oracle_training_samples(_p(centers), _p(levels), _p(weights), _p(w2c), _p(pos), _p(ids),
+                                             C.c_uint32(n_samples), C.c_uint32(len(levels)), C.byref(cam),
+                                             C.c_float(initial_size), _p(rng.state))
+    return pos, ids, int(consumed)
+
+
+def expected_counts(weights, n_samples: int):
+    """Returns (offsets int32 (L,), n_created, sum)."""
+    weights = _f32(weights)
+    offs = np.zeros(len(weights), dtype=np.int32)
+    s = C.c_float(0)
+    n = lib().oracle_expected_counts(_p(weights), _p(offs), C.c_uint32(n_samples), C.c_uint32(len(weights)),
+                                     C.byref(s))
+    return offs, int(n), np.float32(s.value)
+
+
+def expected_samples(centers, levels, offsets, n_created: int, n_multi: int, initial_size: float, rng: Pcg32):
+    centers, levels, offsets = _f32(centers), _i32(levels), _i32(offsets)
+    pos = np.empty((n_created * n_multi, 3), dtype=np.float32)
+    lib().oracle_expected_samples(_p(centers), _p(levels), _p(offsets), _p(pos), C.c_uint32(n_created),
+                                  C.c_uint32(n_multi), C.c_uint32(len(levels)), C.c_float(initial_size),
+                                  _p(rng.state))
+    return pos
+
+
+# ----------------------------------------------------------------------------------------------
+# rasterizer
+# ----------------------------------------------------------------------------------------------
+def make_config(n_points: int, cam: Camera, tile: int = 16, channels: int = 4, feature_mode: int = FEAT_DIRECT_F32,
+                flags: int = 0) -> RasterConfig:
+    return RasterConfig(int(n_points), int(tile), int(channels), int(feature_mode), int(flags), cam)
+
+
+def _features_array(features, feature_mode):
+    if feature_mode == FEAT_DIRECT_F32:
+        return _f32(features)
+    return np.ascontiguousarray(features, dtype=np.float16)
+
+
+def raster_forward(cfg: RasterConfig, positions, features, opacities, w2c, cam_position=None, debug: bool = False):
+    """Returns dict(image (C,H,W), alpha (1,H,W), blending_weights (N,) | depth_image (1,H,W), + debug buffers)."""
+    n = cfg.n_points
+    W, H = cfg.cam.width, cfg.cam.height
+    sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
+    Cn = 4 if sh else cfg.channels
+    positions, w2c = _f32(positions), _f32(w2c)
+    features = _features_array(features, cfg.feature_mode)
+    opacities = None if opacities is None else _f32(opacities).reshape(-1)
+    cam_position = _f32(np.zeros(3) if cam_position is None else cam_position)
+    inference = bool(cfg.flags & RASTER_INFERENCE)
+    image = np.zeros((Cn, H, W), dtype=np.float32)
+    alpha = np.zeros((1, H, W), dtype=np.float32)
+    bw = None if inference else np.zeros(n, dtype=np.float32)
+    depth_image = np.zeros((1, H, W), dtype=np.float32) if inference else None
+    out = {"image": image, "alpha": alpha, "blending_weights": bw, "depth_image": depth_image}
+    dbg_ptr = None
+    if debug:
+        T = cfg.tile
+        n_tiles = ((W + T - 1) // T) * ((H + T - 1) // T)
+        bufs = {
+            "n_touched": np.zeros(n, np.uint32),
+            "bounds": np.zeros((n, 4), np.uint16),
+            "screen_xy": np.zeros((n, 2), np.float32),
+            "depth": np.zeros(n, np.float32),
+            "features_view": np.zeros((n, Cn), np.float32),
+            "opacity": np.zeros(n, np.float32),
+            "counts": np.zeros(2, np.uint32),
+            "depth_keys": np.zeros(n, np.uint32),
+            "depth_order": np.zeros(n, np.uint32),
+            "instance_keys": np.zeros(4 * n, np.uint16),
+            "instance_points": np.zeros(4 * n, np.uint32),
+            "tile_ranges": np.zeros((n_tiles, 2), np.uint32),
+        }
+        dbg = _RasterDebug(*[_p(bufs[name]) for name, _ in _RasterDebug._fields_])
+        dbg_ptr = C.byref(dbg)
+        out.update(bufs)
+    rc = lib().oracle_raster_forward(C.byref(cfg), _p(positions), _p(features), _p(opacities), _p(w2c),
+                                     _p(cam_position), _p(image), _p(alpha), _p(bw), _p(depth_image), dbg_ptr)
+    if rc != 0:
+        raise RuntimeError(f"oracle_raster_forward failed with {rc}")
+    if debug:
+        v, i = int(out["counts"][0]), int(out["counts"][1])
+        out["n_visible"], out["n_instances"] = v, i
+        for name in ("depth_keys", "depth_order"):
+            out[name] = out[name][:v]
+        for name in ("instance_keys", "instance_points"):
+            out[name] = out[name][:i]
+    return out
+
+
+def raster_backward(cfg: RasterConfig, grad_image, grad_alpha, image, alpha, positions, features, opacities, w2c,
+                    cam_position=None):
+    """Returns (grad_features, grad_opacities (N,), grad_view (N,C))."""
+    n = cfg.n_points
+    sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
+    Cn = 4 if sh else cfg.channels
+    positions, w2c = _f32(positions), _f32(w2c)
+    features = _features_array(features, cfg.feature_mode)
+    opacities = _f32(opacities).reshape(-1)
+    cam_position = _f32(np.zeros(3) if cam_position is None else cam_position)
+    grad_image, grad_alpha, image, alpha = _f32(grad_image), _f32(grad_alpha), _f32(image), _f32(alpha)
+    if cfg.feature_mode == FEAT_SH36_F16:
+        gf = np.zeros((n, 36), dtype=np.float16)
+    elif cfg.feature_mode == FEAT_DIRECT_F16:
+        gf = np.zeros((n, Cn), dtype=np.float16)
+    else:
+        gf = np.zeros((n, Cn), dtype=np.float32)
+    go = np.zeros(n, dtype=np.float32)
+    gv = np.zeros((n, Cn), dtype=np.float32)
+    rc = lib().oracle_raster_backward(C.byref(cfg), _p(grad_image), _p(grad_alpha), _p(image), _p(alpha),
+                                      _p(positions), _p(features), _p(opacities), _p(w2c), _p(cam_position), _p(gf),
+                                      _p(go), _p(gv))
+    if rc != 0:
+        raise RuntimeError(f"oracle_raster_backward failed with {rc}")
+    return gf, go, gv

@@ -1,0 +1,231 @@
+"""Thin test-side wrappers that call libinpc_hip.so through its C ABI with torch device buffers and
+return numpy arrays shaped like the oracle's outputs."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+
+from inpc_amd import _lib
+
+
+def dev(a, device="cuda:0"):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def cam_struct(camera) -> _lib.Camera:
+    return _lib.make_camera(camera)
+
+
+def stream():
+    return _lib.current_stream()
+
+
+def make_rng(seed: int, device="cuda:0"):
+    host = (C.c_uint64 * 2)()
+    _lib.lib().inpc_pcg32_seed(host, C.c_uint64(seed), C.c_uint64(1))
+    signed = [int(v) - 2**64 if int(v) >= 2**63 else int(v) for v in host]
+    return torch.tensor(signed, dtype=torch.int64, device=device)
+
+
+def rng_values(rng_dev):
+    s, i = rng_dev.cpu().tolist()
+    return s % 2**64, i % 2**64
+
+
+def leaf_weights(oct, hv, device="cuda:0"):
+    lib = _lib.lib()
+    n = len(oct.levels)
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    cam = cam_struct(hv.camera)
+    _lib.check(lib.inpc_leaf_weights(_lib.ptr(dev(oct.centers)), _lib.ptr(dev(oct.levels)), _lib.ptr(dev(oct.weights)),
+                                     _lib.ptr(dev(hv.w2c)), _lib.ptr(out), n, C.byref(cam), oct.initial_size,
+                                     stream()), "inpc_leaf_weights")
+    return out
+
+
+def build_cdf(w_dev):
+    lib = _lib.lib()
+    n = w_dev.numel()
+    cdf = w_dev.clone()
+    ws_bytes = int(lib.inpc_sampler_workspace_bytes(n))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_dev.device)
+    total = torch.zeros(1, dtype=torch.float32, device=w_dev.device)
+    _lib.check(lib.inpc_build_cdf(_lib.ptr(cdf), _lib.ptr(total), _lib.ptr(ws), ws_bytes, n, stream()),
+               "inpc_build_cdf")
+    return cdf, total
+
+
+def sample(oct, cdf, total, n_samples, rng_dev):
+    lib = _lib.lib()
+    device = cdf.device
+    pos = torch.full((n_samples, 3), float("nan"), dtype=torch.float32, device=device)
+    ids = torch.full((n_samples,), -7, dtype=torch.int32, device=device)
+    _lib.check(lib.inpc_sample(_lib.ptr(dev(oct.centers)), _lib.ptr(dev(oct.levels)), _lib.ptr(cdf), _lib.ptr(total),
+                               _lib.ptr(pos), _lib.ptr(ids), n_samples, len(oct.levels), oct.initial_size,
+                               _lib.ptr(rng_dev), stream()), "inpc_sample")
+    return pos.cpu().numpy(), ids.cpu().numpy()
+
+
+class CullDraw:
+    """One training draw made of explicit rounds."""
+
+    def __init__(self, oct, hv, cdf, total, rng_dev, capacity, max_round):
+        self.lib = _lib.lib()
+        self.oct, self.hv, self.cdf, self.total, self.rng = oct, hv, cdf, total, rng_dev
+        self.capacity = capacity
+        device = cdf.device
+        self.centers, self.levels, self.w2c = dev(oct.centers), dev(oct.levels), dev(hv.w2c)
+        self.pos = torch.full((capacity, 3), float("nan"), dtype=torch.float32, device=device)
+        self.ids = torch.full((capacity,), -7, dtype=torch.int32, device=device)
+        self.ws_bytes = int(self.lib.inpc_cull_workspace_bytes(max_round))
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=device)
+        self.cam = cam_struct(hv.camera)
+        self.k0 = 0
+        _lib.check(self.lib.inpc_cull_begin(_lib.ptr(self.ws), self.ws_bytes, stream()), "inpc_cull_begin")
+
+    def round(self, n_candidates):
+        _lib.check(self.lib.inpc_sample_cull_compact(
+            _lib.ptr(self.centers), _lib.ptr(self.levels), _lib.ptr(self.cdf), _lib.ptr(self.total), _lib.ptr(self.w2c),
+            _lib.ptr(self.pos), _lib.ptr(self.ids), self.capacity, self.k0, n_candidates, len(self.oct.levels),
+            C.byref(self.cam), self.oct.initial_size, _lib.ptr(self.rng), _lib.ptr(self.ws), self.ws_bytes, stream()),
+            "inpc_sample_cull_compact")
+        self.k0 += n_candidates
+        return self.counts()
+
+    def counts(self):
+        a, c = C.c_uint32(0), C.c_uint32(0)
+        _lib.check(self.lib.inpc_cull_read_counts(_lib.ptr(self.ws), C.byref(a), C.byref(c), stream()),
+                   "inpc_cull_read_counts")
+        return int(a.value), int(c.value)
+
+    def finish(self):
+        _lib.check(self.lib.inpc_cull_finish(_lib.ptr(self.total), _lib.ptr(self.pos), _lib.ptr(self.ids),
+                                             self.capacity, self.k0, _lib.ptr(self.rng), _lib.ptr(self.ws),
+                                             self.ws_bytes, stream()), "inpc_cull_finish")
+
+
+FEATURE_DTYPES = {_lib.FEAT_SH36_F16: np.float16, _lib.FEAT_DIRECT_F32: np.float32, _lib.FEAT_DIRECT_F16: np.float16,
+                  _lib.FEAT_RAW37_F16: np.float16}
+
+
+class RasterRun:
+    """inpc_raster_forward (+ backward) through the C ABI on numpy inputs."""
+
+    def __init__(self, hv, positions, features, opacities, tile=16, channels=4, feature_mode=_lib.FEAT_DIRECT_F32,
+                 inference=False, device="cuda:0"):
+        self.lib = _lib.lib()
+        self.hv = hv
+        self.n = len(positions)
+        sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
+        self.C = 4 if sh else channels
+        self.cfg = _lib.RasterConfig(self.n, tile, self.C, feature_mode, _lib.RASTER_INFERENCE if inference else 0,
+                                     cam_struct(hv.camera))
+        self.layout = _lib.RasterLayout()
+        _lib.check(self.lib.inpc_raster_layout_query(C.byref(self.cfg), C.byref(self.layout)), "layout")
+        self.inference = inference
+        self.device = device
+        self.positions = dev(np.asarray(positions, np.float32).reshape(-1, 3), device)
+        self.features = dev(np.asarray(features, FEATURE_DTYPES[feature_mode]), device)
+        self.opacities = None if opacities is None else dev(np.asarray(opacities, np.float32).reshape(-1), device)
+        self.w2c = dev(hv.w2c, device)
+        self.cam_position = dev(hv.position, device)
+        H, W = hv.camera.height, hv.camera.width
+        self.image = torch.full((self.C, H, W), float("nan"), dtype=torch.float32, device=device)
+        self.alpha = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device)
+        self.bw = None if inference else torch.full((max(self.n, 1),), float("nan"), dtype=torch.float32, device=device)
+        self.depth_image = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device) if inference else None
+        self.ws = torch.empty(self.layout.total_bytes, dtype=torch.uint8, device=device)
+
+    def forward(self):
+        _lib.check(self.lib.inpc_raster_forward(
+            C.byref(self.cfg), _lib.ptr(self.positions), _lib.ptr(self.features), _lib.ptr(self.opacities),
+            _lib.ptr(self.w2c), _lib.ptr(self.cam_position), _lib.ptr(self.image), _lib.ptr(self.alpha),
+            _lib.ptr(self.bw), _lib.ptr(self.depth_image), _lib.ptr(self.ws), self.layout.total_bytes, stream()),
+            "inpc_raster_forward")
+        return self
+
+    def counters(self):
+        out = (C.c_uint32 * 3)()
+        _lib.check(self.lib.inpc_raster_read_counters(C.byref(self.cfg), _lib.ptr(self.ws), C.byref(out), stream()),
+                   "inpc_raster_read_counters")
+        return int(out[0]), int(out[1])
+
+    def _buf(self, offset, count, dtype):
+        nbytes = count * np.dtype(dtype).itemsize
+        return self.ws[offset:offset + nbytes].cpu().numpy().view(dtype)
+
+    def debug(self):
+        """Intermediate buffers decoded into the oracle's shapes."""
+        L, n = self.layout, self.n
+        v, i = self.counters()
+        rec = self._buf(L.point_record, 4 * n, np.float32).reshape(n, 4)
+        info = rec[:, 3].copy().view(np.uint32)
+        valid = (info >> 18) & 1
+        tile0 = info & 0xFFFF
+        nx = ((info >> 16) & 1) + 1
+        ny = ((info >> 17) & 1) + 1
+        x0, y0 = tile0 % L.grid_width, tile0 // L.grid_width
+        bounds = np.stack([x0, x0 + nx, y0, y0 + ny], axis=1).astype(np.uint16)
+        bounds[valid == 0] = 0
+        out = {
+            "n_visible": v, "n_instances": i,
+            "n_touched": np.where(valid == 1, nx * ny, 0).astype(np.uint32),
+            "bounds": bounds,
+            "screen_xy": np.where(valid[:, None] == 1, rec[:, :2], 0).astype(np.float32),
+            "opacity": np.where(valid == 1, rec[:, 2], 0).astype(np.float32),
+            "depth": self._buf(L.point_depth, n, np.float32),
+            "depth_keys": (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32),
+            "depth_order": self._buf(L.depth_order, n, np.uint32)[:v],
+            "instance_keys": self._buf(L.instance_keys, 4 * n, np.uint16)[:i],
+            "instance_points": self._buf(L.instance_points, 4 * n, np.uint32)[:i],
+            "tile_ranges": self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2),
+        }
+        if L.features_view:
+            out["features_view"] = self._buf(L.features_view, 4 * n, np.float32).reshape(n, 4)
+        return out
+
+    def outputs(self):
+        out = {"image": self.image.cpu().numpy(), "alpha": self.alpha.cpu().numpy()}
+        if self.inference:
+            out["depth_image"] = self.depth_image.cpu().numpy()
+        else:
+            out["blending_weights"] = self.bw.cpu().numpy()[:self.n]
+        return out
+
+    def backward(self, grad_image, grad_alpha):
+        mode = self.cfg.feature_mode
+        n, Cn = self.n, self.C
+        device = self.device
+        scratch = None
+        if mode == _lib.FEAT_SH36_F16:
+            gf = torch.full((n, 36), float("nan"), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
+        elif mode == _lib.FEAT_DIRECT_F16:
+            gf = torch.full((n, Cn), float("nan"), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, Cn), dtype=torch.float32, device=device)
+        else:
+            gf = torch.full((n, Cn), float("nan"), dtype=torch.float32, device=device)
+        go = torch.full((n,), float("nan"), dtype=torch.float32, device=device)
+        gi, ga = dev(np.asarray(grad_image, np.float32), device), dev(np.asarray(grad_alpha, np.float32), device)
+        _lib.check(self.lib.inpc_raster_backward(
+            C.byref(self.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(self.image), _lib.ptr(self.alpha),
+            _lib.ptr(self.positions), _lib.ptr(self.features), _lib.ptr(self.opacities), _lib.ptr(self.cam_position),
+            _lib.ptr(gf), _lib.ptr(go), _lib.ptr(scratch), _lib.ptr(self.ws), self.layout.total_bytes, stream()),
+            "inpc_raster_backward")
+        return gf.cpu().numpy(), go.cpu().numpy()
+
+
+def assert_close(actual, expected, rtol=1e-4, atol=1e-6, what=""):
+    """allclose with a report of the worst element."""
+    actual, expected = np.asarray(actual, np.float64), np.asarray(expected, np.float64)
+    assert actual.shape == expected.shape, f"{what}: shape {actual.shape} vs {expected.shape}"
+    err = np.abs(actual - expected)
+    tol = atol + rtol * np.abs(expected)
+    bad = err > tol
+    if bad.any() or not np.isfinite(actual).all():
+        idx = np.unravel_index(np.argmax(err - tol), err.shape)
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.size} elements differ; worst at {idx}: "
+                             f"{actual[idx]!r} vs {expected[idx]!r} (|err|={err[idx]:.3e}); "
+                             f"non-finite: {int((~np.isfinite(actual)).sum())}")

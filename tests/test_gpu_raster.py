@@ -1,0 +1,274 @@
+"""GPU parity of the rasterizer against the CPU oracle, through the C ABI.
+
+Bit-exact: tile bounds, screen coordinates, depth keys, depth order, instance order, tile ranges.
+Within 1e-4 relative (plus a small absolute floor for near-zero values): image, alpha, depth image,
+blending weights, feature and opacity gradients.
+"""
+import numpy as np
+import pytest
+import torch
+
+from inpc_amd import _lib, synthetic
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+
+
+def oracle_cfg(O, hv, n, tile, channels, mode, inference=False):
+    c = hv.camera
+    cam = O.make_camera(c.width, c.height, c.focal_x, c.focal_y, c.center_x, c.center_y, c.near_plane, c.far_plane)
+    return O.make_config(n, cam, tile, channels, mode, O.RASTER_INFERENCE if inference else 0)
+
+
+def scene(n, channels, seed=0, width=251, height=163, focal=230.0, side=1.6, distance=2.4, dtype=np.float32):
+    hv = synthetic.camera_on_z(width, height, focal, distance)
+    pos = synthetic.cube_points(n, side, seed)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", seed + 1, dtype)
+    return hv, pos, feats, opac
+
+
+def check_structure(dbg, ref):
+    assert dbg["n_visible"] == ref["n_visible"]
+    assert dbg["n_instances"] == ref["n_instances"]
+    np.testing.assert_array_equal(dbg["n_touched"], ref["n_touched"])
+    np.testing.assert_array_equal(dbg["bounds"], ref["bounds"])
+    np.testing.assert_array_equal(dbg["screen_xy"].view(np.uint32), ref["screen_xy"].view(np.uint32))
+    vis = ref["n_touched"] > 0
+    np.testing.assert_array_equal(dbg["depth"][vis].view(np.uint32), ref["depth"][vis].view(np.uint32))
+    np.testing.assert_array_equal(dbg["depth_keys"], ref["depth_keys"])
+    np.testing.assert_array_equal(dbg["depth_order"], ref["depth_order"])
+    np.testing.assert_array_equal(dbg["instance_keys"], ref["instance_keys"])
+    np.testing.assert_array_equal(dbg["instance_points"], ref["instance_points"])
+    np.testing.assert_array_equal(dbg["tile_ranges"], ref["tile_ranges"])
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+@pytest.mark.parametrize("channels", [4, 8, 16])
+def test_forward_direct_f32(gpu, oracle, tile, channels):
+    n = 60000
+    hv, pos, feats, opac = scene(n, channels, seed=tile + channels)
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32).forward()
+    ref = oracle.raster_forward(oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32), pos, feats, opac,
+                                hv.w2c, debug=True)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_forward_dense_opaque_scene_terminates_early(gpu, oracle, tile):
+    # many points per pixel with high opacity: exercises the transmittance early-out and multi-batch tiles
+    n = 200000
+    hv = synthetic.camera_on_z(97, 61, 90.0, 2.4)
+    pos = synthetic.cube_points(n, 1.2, 5)
+    feats, _ = synthetic.point_attributes(n, 4, "uniform", 6)
+    opac = np.random.default_rng(7).uniform(0.3, 0.999, n).astype(np.float32)
+    run = H.RasterRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_DIRECT_F32).forward()
+    ref = oracle.raster_forward(oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_DIRECT_F32), pos, feats, opac, hv.w2c,
+                                debug=True)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    assert (ref["alpha"] == 1.0).mean() > 0.5  # most pixels saturate
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_forward_sh36_and_backward(gpu, oracle, tile):
+    n = 50000
+    hv = synthetic.rotated_camera(233, 171, 210.0, 2.6, yaw=0.5, pitch=-0.3)
+    pos = synthetic.cube_points(n, 1.5, 11)
+    feats = synthetic.sh_features(n, 12)
+    _, opac = synthetic.point_attributes(n, 4, "normal", 13)
+    run = H.RasterRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_SH36_F16).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_SH36_F16)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, hv.position, debug=True)
+    dbg = run.debug()
+    check_structure(dbg, ref)
+    vis = ref["n_touched"] > 0
+    H.assert_close(dbg["features_view"][vis], ref["features_view"][vis], RTOL, 1e-5, "SH view features")
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
+
+    rng = np.random.default_rng(14)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                               hv.position)
+    assert (gf[~vis] == 0).all() and (go[~vis] == 0).all()
+    # fp16 outputs: one fp16 ulp of slack on top of the fp32 tolerance
+    H.assert_close(gf.astype(np.float32), gf_ref.astype(np.float32), 2e-3, 1e-7, "SH feature gradients")
+    H.assert_close(go, go_ref, RTOL, 1e-7, "opacity gradients")
+
+
+@pytest.mark.parametrize("tile,channels,mode", [(16, 8, "f32"), (8, 4, "f32"), (16, 16, "f32"), (8, 8, "f16"),
+                                                (16, 4, "f16")])
+def test_backward_direct(gpu, oracle, tile, channels, mode):
+    n = 40000
+    fmode = _lib.FEAT_DIRECT_F32 if mode == "f32" else _lib.FEAT_DIRECT_F16
+    hv, pos, feats, opac = scene(n, channels, seed=31 + channels, dtype=np.float32 if mode == "f32" else np.float16)
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, fmode).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, channels, fmode)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    rng = np.random.default_rng(32)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    # the backward replays against the forward's own outputs, as the autograd function does
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
+    if mode == "f32":
+        H.assert_close(gf, gf_ref, RTOL, 1e-7, "feature gradients")
+    else:
+        H.assert_close(gf.astype(np.float32), gf_ref.astype(np.float32), 2e-3, 1e-7, "feature gradients (fp16)")
+    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_inference_raw37_and_preextracted(gpu, oracle, tile):
+    n = 50000
+    hv = synthetic.rotated_camera(199, 140, 180.0, 2.5, yaw=-0.4, pitch=0.2)
+    pos = synthetic.cube_points(n, 1.5, 41)
+    rng = np.random.default_rng(42)
+    raw = np.concatenate([rng.normal(-1.0, 1.0, (n, 1)), synthetic.sh_features(n, 43).astype(np.float64)], axis=1)
+    raw = raw.astype(np.float16)
+    run = H.RasterRun(hv, pos, raw, None, tile, 4, _lib.FEAT_RAW37_F16, inference=True).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_RAW37_F16, inference=True)
+    ref = oracle.raster_forward(cfg, pos, raw, None, hv.w2c, hv.position, debug=True)
+    dbg = run.debug()
+    check_structure(dbg, ref)
+    vis = ref["n_touched"] > 0
+    H.assert_close(dbg["opacity"][vis], ref["opacity"][vis], RTOL, 1e-6, "activated opacity")
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], 2e-4, 1e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], 2e-4, 1e-6, "alpha")
+    H.assert_close(out["depth_image"], ref["depth_image"], 2e-4, 1e-5, "depth image")
+
+    feats = synthetic.sh_features(n, 44)
+    _, opac = synthetic.point_attributes(n, 4, "normal", 45)
+    run = H.RasterRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_SH36_F16, inference=True).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_SH36_F16, inference=True)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, hv.position)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(out["depth_image"], ref["depth_image"], RTOL, 1e-5, "depth image")
+
+
+def test_inference_direct_f16_16_channels(gpu, oracle):
+    n = 80000
+    hv, pos, feats, opac = scene(n, 16, seed=51, dtype=np.float16)
+    run = H.RasterRun(hv, pos, feats, opac, 16, 16, _lib.FEAT_DIRECT_F16, inference=True).forward()
+    cfg = oracle_cfg(oracle, hv, n, 16, 16, oracle.FEAT_DIRECT_F16, inference=True)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(out["depth_image"], ref["depth_image"], RTOL, 1e-5, "depth image")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_edge_cases(gpu, oracle, tile):
+    hv = synthetic.camera_on_z(64, 48, 50.0, 2.0)
+
+    def compare(pos, what):
+        pos = np.asarray(pos, np.float32).reshape(-1, 3)
+        n = len(pos)
+        feats, opac = synthetic.point_attributes(max(n, 1), 4, "uniform", 3)
+        feats, opac = feats[:n], opac[:n]
+        run = H.RasterRun(hv, pos, feats if n else np.zeros((0, 4), np.float32), opac if n else np.zeros(0, np.float32),
+                          tile, 4, _lib.FEAT_DIRECT_F32).forward()
+        ref = oracle.raster_forward(oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_DIRECT_F32), pos, feats, opac,
+                                    hv.w2c, debug=True)
+        if n:
+            check_structure(run.debug(), ref)
+        out = run.outputs()
+        H.assert_close(out["image"], ref["image"], RTOL, 1e-6, what + ": image")
+        H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, what + ": alpha")
+        if n:
+            H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, what + ": weights")
+        return ref
+
+    ref = compare(np.zeros((0, 3)), "empty")
+    assert (ref["image"] == 0).all()
+    ref = compare([[0, 0, -5.0], [0, 0, 200.0], [50.0, 0, 0]], "all culled")
+    assert ref["n_visible"] == 0
+    compare([[0.0, 0.0, 0.0]], "single point")
+    # a plane of points at one depth: every depth key ties, order must fall back to the point id
+    g = np.stack(np.meshgrid(np.linspace(-1.2, 1.2, 90), np.linspace(-0.9, 0.9, 70)), -1).reshape(-1, 2)
+    plane = np.concatenate([g, np.zeros((len(g), 1))], axis=1)
+    ref = compare(np.concatenate([plane, plane[::-1]]), "coplanar points")
+    assert ref["n_visible"] > 5000
+    # points that project exactly onto pixel centres, pixel corners and tile edges
+    px = np.array([0.5, 1.0, 7.5, 8.0, 8.5, 15.5, 16.0, 16.5, 31.5, 32.0, 63.5, 64.0, -0.4, -0.5, 64.4, 64.5])
+    xs, ys = np.meshgrid(px, px[:12] * 0.75)
+    z = 0.0
+    depth = 2.0
+    wx = (xs.ravel() - 32.0) / 50.0 * depth
+    wy = (ys.ravel() - 24.0) / 50.0 * depth
+    compare(np.stack([wx, wy, np.full_like(wx, z)], 1), "pixel / tile boundaries")
+
+
+def test_too_many_tiles_is_rejected(gpu):
+    hv = synthetic.camera_on_z(8 * 300, 8 * 300, 500.0, 3.0)
+    with pytest.raises(_lib.BackendError, match="16-bit tile key"):
+        H.RasterRun(hv, np.zeros((4, 3), np.float32), np.zeros((4, 4), np.float32), np.ones(4, np.float32), 8, 4,
+                    _lib.FEAT_DIRECT_F32)
+
+
+def test_autograd_api_sh_and_direct(gpu, oracle):
+    from inpc_amd import INPCRasterizer, rasterize_points
+
+    n = 30000
+    hv = synthetic.camera_on_z(160, 120, 140.0, 2.5)
+    view = hv.to_view(gpu)
+    pos = synthetic.cube_points(n, 1.5, 61)
+    feats = synthetic.sh_features(n, 62)
+    _, opac = synthetic.point_attributes(n, 4, "normal", 63)
+    positions = H.dev(pos)
+    features = H.dev(feats).requires_grad_(True)
+    opacities = H.dev(opac.reshape(-1, 1)).requires_grad_(True)
+    rasterizer = INPCRasterizer()
+    image, alpha, weights = rasterizer(view, 0, positions, features, opacities)
+    assert image.shape == (4, 120, 160) and alpha.shape == (1, 120, 160) and weights.shape == (n,)
+    assert not weights.requires_grad
+    cfg = oracle_cfg(oracle, hv, n, 8, 4, oracle.FEAT_SH36_F16)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, hv.position)
+    H.assert_close(image.detach().cpu().numpy(), ref["image"], RTOL, 1e-5, "image")
+    # only the image is used: grad_alpha arrives as None and must be treated as zero
+    gi = torch.randn_like(image) * 1e-2
+    (image * gi).sum().backward()
+    gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi.cpu().numpy(), np.zeros_like(ref["alpha"]),
+                                               image.detach().cpu().numpy(), alpha.detach().cpu().numpy(), pos, feats,
+                                               opac, hv.w2c, hv.position)
+    assert features.grad.shape == (n, 36) and features.grad.dtype == torch.float16
+    assert opacities.grad.shape == (n, 1)
+    H.assert_close(features.grad.float().cpu().numpy(), gf_ref.astype(np.float32), 2e-3, 1e-7, "SH gradients")
+    H.assert_close(opacities.grad.cpu().numpy().reshape(-1), go_ref, RTOL, 1e-7, "opacity gradients")
+
+    # render / render_preextracted return (image, depth, alpha)
+    img2, depth2, alpha2 = rasterizer.render_preextracted(view, 0, positions, features.detach(), opacities.detach())
+    H.assert_close(img2.cpu().numpy(), ref["image"], RTOL, 1e-5, "preextracted image")
+    assert depth2.shape == (1, 120, 160)
+    with pytest.raises(RuntimeError, match="unsupported rasterizer mode"):
+        rasterizer(view, 1, positions, features, opacities)
+
+    f8, o8 = synthetic.point_attributes(n, 8, "normal", 64)
+    f8d = H.dev(f8).requires_grad_(True)
+    o8d = H.dev(o8).requires_grad_(True)
+    image8, alpha8, w8 = rasterize_points(view, positions, f8d, o8d, tile=16)
+    (image8.sum() + alpha8.sum()).backward()
+    cfg8 = oracle_cfg(oracle, hv, n, 16, 8, oracle.FEAT_DIRECT_F32)
+    ref8 = oracle.raster_forward(cfg8, pos, f8, o8, hv.w2c)
+    ones_i, ones_a = np.ones_like(ref8["image"]), np.ones_like(ref8["alpha"])
+    gf8, go8, _ = oracle.raster_backward(cfg8, ones_i, ones_a, image8.detach().cpu().numpy(),
+                                         alpha8.detach().cpu().numpy(), pos, f8, o8, hv.w2c)
+    H.assert_close(f8d.grad.cpu().numpy(), gf8, RTOL, 1e-6, "direct feature gradients")
+    H.assert_close(o8d.grad.cpu().numpy(), go8, RTOL, 1e-5, "direct opacity gradients")

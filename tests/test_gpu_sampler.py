@@ -1,0 +1,204 @@
+"""GPU parity of the sampler against the CPU oracle, through the C ABI. Leaf weights, CDF, leaf ids,
+positions, cull decisions and the generator state must be bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from inpc_amd import _lib, synthetic
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def small_scene(n_leaves=6000, level=6, seed=3, mixed_levels=True, distance=3.5):
+    oct = synthetic.octree_leaves(n_leaves, level, initial_size=4.0, seed=seed)
+    if mixed_levels:  # leaves of several sizes (geometry need not tile space for the sampler)
+        rng = np.random.default_rng(seed + 100)
+        oct.levels = rng.integers(3, 9, size=n_leaves).astype(np.int32)
+    hv = synthetic.camera_on_z(311, 203, 260.0, distance)
+    return oct, hv
+
+
+def oracle_cam(O, hv):
+    c = hv.camera
+    return O.make_camera(c.width, c.height, c.focal_x, c.focal_y, c.center_x, c.center_y, c.near_plane, c.far_plane)
+
+
+@pytest.mark.parametrize("n_leaves,level", [(1, 0), (63, 4), (64, 4), (65, 4), (4097, 5), (6000, 6), (300000, 8)])
+def test_leaf_weights_and_cdf_bit_exact(gpu, oracle, n_leaves, level):
+    oct, hv = small_scene(n_leaves, level, mixed_levels=n_leaves > 100)
+    w_gpu = H.leaf_weights(oct, hv)
+    w_ref = oracle.leaf_weights(oct.centers, oct.levels, oct.weights, hv.w2c, oracle_cam(oracle, hv), oct.initial_size)
+    np.testing.assert_array_equal(w_gpu.cpu().numpy().view(np.uint32), w_ref.view(np.uint32))
+    cdf_gpu, total_gpu = H.build_cdf(w_gpu)
+    ok, cdf_ref, total_ref = oracle.build_cdf(w_ref)
+    assert ok
+    assert total_gpu.cpu().numpy().view(np.uint32)[0] == np.float32(total_ref).view(np.uint32)
+    np.testing.assert_array_equal(cdf_gpu.cpu().numpy().view(np.uint32), cdf_ref.view(np.uint32))
+
+
+def test_cdf_of_exact_integers_matches_cumsum(gpu):
+    # Integer-valued weights whose total is a power of two: the total, the reciprocal, the normalised
+    # weights and every partial sum are exact in fp32 whatever the association order, so the CDF must
+    # equal numpy's cumsum bit for bit. Pins chunk indexing (dropped / doubled elements) without the oracle.
+    rng = np.random.default_rng(0)
+    n = 70001
+    w = rng.integers(0, 8, size=n).astype(np.int64)
+    w[-1] += (1 << 18) - w.sum()
+    assert 0 <= w[-1] < (1 << 18)
+    cdf, tot = H.build_cdf(H.dev(w.astype(np.float32)))
+    assert float(tot.item()) == float(1 << 18)
+    expect = (np.cumsum(w).astype(np.float64) / (1 << 18)).astype(np.float32)
+    np.testing.assert_array_equal(cdf.cpu().numpy(), expect)
+
+
+def test_sum_not_positive_leaves_weights_untouched(gpu):
+    w = np.zeros(5000, dtype=np.float32)
+    cdf, total = H.build_cdf(H.dev(w))
+    assert float(total.item()) == 0.0
+    np.testing.assert_array_equal(cdf.cpu().numpy(), w)
+
+
+@pytest.mark.parametrize("n_samples", [1, 255, 2048, 2049, 100000])
+def test_sample_bit_exact_and_stream_continues(gpu, oracle, n_samples):
+    oct, hv = small_scene()
+    w = H.leaf_weights(oct, hv)
+    cdf, total = H.build_cdf(w)
+    rng_dev = H.make_rng(1234)
+    rng_ref = oracle.Pcg32(1234)
+    cdf_host = cdf.cpu().numpy()
+    for _ in range(2):  # the second call must continue the generator stream
+        pos, ids = H.sample(oct, cdf, total, n_samples, rng_dev)
+        pos_ref, ids_ref = oracle.sample(oct.centers, oct.levels, cdf_host, n_samples, oct.initial_size, rng_ref)
+        np.testing.assert_array_equal(ids, ids_ref)
+        np.testing.assert_array_equal(pos.view(np.uint32), pos_ref.view(np.uint32))
+        assert H.rng_values(rng_dev) == (int(rng_ref.state[0]), int(rng_ref.state[1]))
+
+
+def test_sample_failure_path_writes_nothing(gpu):
+    oct, hv = small_scene(500, 4)
+    w = torch.zeros(500, dtype=torch.float32, device=gpu)
+    cdf, total = H.build_cdf(w)
+    rng_dev = H.make_rng(5)
+    before = H.rng_values(rng_dev)
+    pos, ids = H.sample(oct, cdf, total, 1000, rng_dev)
+    assert np.isnan(pos).all() and (ids == -7).all()
+    assert H.rng_values(rng_dev) == before
+
+
+@pytest.mark.parametrize("rounds", [[50000], [2048, 2047, 1, 30000], [10000, 10000, 10000]])
+def test_cull_compact_rounds_bit_exact(gpu, oracle, rounds):
+    oct, hv = small_scene(distance=2.2)  # close camera: a good share of candidates is rejected
+    cam = oracle_cam(oracle, hv)
+    w = H.leaf_weights(oct, hv)
+    cdf, total = H.build_cdf(w)
+    cdf_host = cdf.cpu().numpy()
+    capacity = 20000
+    rng_dev = H.make_rng(77)
+    rng_ref = oracle.Pcg32(77)
+    draw = H.CullDraw(oct, hv, cdf, total, rng_dev, capacity, max(rounds))
+    pos_ref, ids_ref, acc_ref, cons_ref, k0 = None, None, 0, 0, 0
+    for m in rounds:
+        acc_gpu, cons_gpu = draw.round(m)
+        pos_ref, ids_ref, acc_ref, c = oracle.sample_cull_compact(oct.centers, oct.levels, cdf_host, hv.w2c, cam,
+                                                                  oct.initial_size, rng_ref, capacity, k0, m, pos_ref,
+                                                                  ids_ref, acc_ref)
+        cons_ref = c or cons_ref
+        k0 += m
+        assert cons_gpu == cons_ref
+        if cons_ref == 0:
+            assert acc_gpu == acc_ref
+        else:
+            assert acc_gpu >= capacity
+    filled = min(acc_ref, capacity)
+    assert 0 < filled
+    np.testing.assert_array_equal(draw.ids.cpu().numpy()[:filled], ids_ref[:filled])
+    np.testing.assert_array_equal(draw.pos.cpu().numpy()[:filled].view(np.uint32), pos_ref[:filled].view(np.uint32))
+    draw.finish()
+    rng_ref.advance(4 * (cons_ref if cons_ref else k0))
+    assert H.rng_values(rng_dev) == (int(rng_ref.state[0]), int(rng_ref.state[1]))
+
+
+def test_training_api_matches_oracle_draw(gpu, oracle):
+    from inpc_amd import ProbabilityFieldSampler
+
+    oct, hv = small_scene(distance=2.2)
+    view = hv.to_view(gpu)
+    sampler = ProbabilityFieldSampler(seed=9)
+    rng_ref = oracle.Pcg32(9)
+    centers, levels, weights = H.dev(oct.centers), H.dev(oct.levels), H.dev(oct.weights)
+    for n in (5000, 12345):  # two calls: the second continues the stream where the first stopped
+        pos, ids = sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)
+        pos_ref, ids_ref, consumed = oracle.training_samples(oct.centers, oct.levels, oct.weights, hv.w2c,
+                                                             oracle_cam(oracle, hv), oct.initial_size, rng_ref, n)
+        assert ids.dtype == torch.int64 and pos.shape == (n, 3)
+        np.testing.assert_array_equal(ids.cpu().numpy(), ids_ref.astype(np.int64))
+        np.testing.assert_array_equal(pos.cpu().numpy().view(np.uint32), pos_ref.view(np.uint32))
+        assert sampler.last_consumed == consumed
+        assert sampler.rng_state() == (int(rng_ref.state[0]), int(rng_ref.state[1]))
+
+
+def test_training_api_failure_pattern(gpu):
+    from inpc_amd import ProbabilityFieldSampler
+
+    oct, hv = small_scene(300, 4)
+    view = hv.to_view(gpu)
+    sampler = ProbabilityFieldSampler(seed=1)
+    before = sampler.rng_state()
+    zero = torch.zeros(300, dtype=torch.float32, device=gpu)
+    pos, ids = sampler.generate_training_samples(H.dev(oct.centers), H.dev(oct.levels), zero, view, 777,
+                                                 oct.initial_size)
+    assert (pos == 0).all() and (ids == -1).all()
+    assert sampler.rng_state() == before
+    empty = sampler.generate_samples(H.dev(oct.centers), H.dev(oct.levels), zero, view, 100, oct.initial_size)
+    assert empty.shape == (0, 3)
+    empty = sampler.generate_expected_samples(H.dev(oct.centers), H.dev(oct.levels), zero, view, 100, 2,
+                                              oct.initial_size)
+    assert empty.shape == (0, 3)
+
+
+def test_generate_samples_and_expected_samples_api(gpu, oracle):
+    from inpc_amd import ProbabilityFieldSampler, compute_viewpoint_weights
+
+    oct, hv = small_scene()
+    view = hv.to_view(gpu)
+    cam = oracle_cam(oracle, hv)
+    centers, levels, weights = H.dev(oct.centers), H.dev(oct.levels), H.dev(oct.weights)
+    w = compute_viewpoint_weights(centers, levels, weights, view, oct.initial_size)
+    w_ref = oracle.leaf_weights(oct.centers, oct.levels, oct.weights, hv.w2c, cam, oct.initial_size)
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), w_ref.view(np.uint32))
+
+    sampler = ProbabilityFieldSampler(seed=21)
+    rng_ref = oracle.Pcg32(21)
+    pos = sampler.generate_samples(centers, levels, weights, view, 33333, oct.initial_size)
+    ok, cdf_ref, _ = oracle.build_cdf(w_ref)
+    pos_ref, _ = oracle.sample(oct.centers, oct.levels, cdf_ref, 33333, oct.initial_size, rng_ref)
+    np.testing.assert_array_equal(pos.cpu().numpy().view(np.uint32), pos_ref.view(np.uint32))
+
+    out = sampler.generate_expected_samples(centers, levels, weights, view, 40000, 3, oct.initial_size)
+    offs_ref, n_created, _ = oracle.expected_counts(w_ref, 40000)
+    exp_ref = oracle.expected_samples(oct.centers, oct.levels, offs_ref, n_created, 3, oct.initial_size, rng_ref)
+    assert out.shape == (n_created * 3, 3)
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint32), exp_ref.view(np.uint32))
+    assert sampler.rng_state() == (int(rng_ref.state[0]), int(rng_ref.state[1]))
+
+
+def test_non_perspective_and_distorted_cameras_are_rejected(gpu):
+    from inpc_amd import ProbabilityFieldSampler, compute_viewpoint_weights
+    from inpc_amd.views import View
+
+    oct, hv = small_scene(100, 4)
+    view = hv.to_view(gpu)
+
+    class Fisheye:
+        width, height = 10, 10
+
+    bad = View(Fisheye(), view.w2c, view.position)
+    args = (H.dev(oct.centers), H.dev(oct.levels), H.dev(oct.weights))
+    with pytest.raises(NotImplementedError):
+        compute_viewpoint_weights(*args, bad, 4.0)
+    view.camera.distortion = object()
+    with pytest.raises(NotImplementedError):
+        ProbabilityFieldSampler(0).generate_samples(*args, view, 10, 4.0)
