@@ -39,9 +39,10 @@ def leaf_weights(oct, hv, device="cuda:0"):
     n = len(oct.levels)
     out = torch.empty(n, dtype=torch.float32, device=device)
     cam = cam_struct(hv.camera)
-    _lib.check(lib.inpc_leaf_weights(_lib.ptr(dev(oct.centers)), _lib.ptr(dev(oct.levels)), _lib.ptr(dev(oct.weights)),
-                                     _lib.ptr(dev(hv.w2c)), _lib.ptr(out), n, C.byref(cam), oct.initial_size,
-                                     stream()), "inpc_leaf_weights")
+    # keep the uploads alive until the launch is queued: a temporary's memory is recycled at once
+    centers, levels, weights, w2c = dev(oct.centers), dev(oct.levels), dev(oct.weights), dev(hv.w2c)
+    _lib.check(lib.inpc_leaf_weights(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(w2c),
+                                     _lib.ptr(out), n, C.byref(cam), oct.initial_size, stream()), "inpc_leaf_weights")
     return out
 
 
@@ -62,9 +63,10 @@ def sample(oct, cdf, total, n_samples, rng_dev):
     device = cdf.device
     pos = torch.full((n_samples, 3), float("nan"), dtype=torch.float32, device=device)
     ids = torch.full((n_samples,), -7, dtype=torch.int32, device=device)
-    _lib.check(lib.inpc_sample(_lib.ptr(dev(oct.centers)), _lib.ptr(dev(oct.levels)), _lib.ptr(cdf), _lib.ptr(total),
-                               _lib.ptr(pos), _lib.ptr(ids), n_samples, len(oct.levels), oct.initial_size,
-                               _lib.ptr(rng_dev), stream()), "inpc_sample")
+    centers, levels = dev(oct.centers), dev(oct.levels)
+    _lib.check(lib.inpc_sample(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(pos),
+                               _lib.ptr(ids), n_samples, len(oct.levels), oct.initial_size, _lib.ptr(rng_dev),
+                               stream()), "inpc_sample")
     return pos.cpu().numpy(), ids.cpu().numpy()
 
 
