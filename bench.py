@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+One step = one rasterizer forward + backward over 8,388,608 points at 1237x822 (8 fp32 channels,
+16x16 tiles), the configuration the headline metric is quoted on. The points are drawn on the GPU by the
+sampler (262,144 log-normal leaves of a depth-9 octree over [-2,2]^3, camera at (0,0,-6), f = 1000);
+features ~N(0,1), opacity = sigmoid(N(0,1)), image gradients ~N(0,1e-2). All inputs are resident in HBM
+before the timed region.
+
+Prints ONE JSON line. `value` is Mpoints/s of forward+backward; `roofline` describes the kernel with the
+largest share of the step (algorithmic bytes per launch / HIP-event duration on the launch stream);
+`cpu_baseline` is the CPU oracle running the same step on a bounded sample with all host threads.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (n_points, width, height, focal, channels, tile, n_leaves, level)
+    "config3": dict(n=8_388_608, width=1237, height=822, focal=1000.0, channels=8, tile=16, leaves=262_144, level=9,
+                    describe="rasterizer fwd+bwd, 8,388,608 pts @1237x822, C=8 fp32, 16x16 tiles"),
+    "config3_t8": dict(n=8_388_608, width=1237, height=822, focal=1000.0, channels=8, tile=8, leaves=262_144, level=9,
+                       describe="rasterizer fwd+bwd, 8,388,608 pts @1237x822, C=8 fp32, 8x8 tiles"),
+    "small": dict(n=262_144, width=640, height=400, focal=500.0, channels=8, tile=16, leaves=32_768, level=7,
+                  describe="rasterizer fwd+bwd, 262,144 pts @640x400, C=8 fp32, 16x16 tiles (quick check)"),
+}
+
+
+def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, depth_passes, tile_passes, end_bit):
+    """Algorithmic bytes one launch of `kernel` moves: each array of the pipeline touched the minimum
+    number of times its structure requires. F = feature bytes per point, R = blend record
+    (8 xy + 4 opacity + 4C features)."""
+    F = 4 * channels
+    R = 8 + 4 + 4 * channels
+    table = {
+        "raster_preprocess": n * (16 + F) + v * (R + 8),
+        "raster_depth_sort": v * 68 / max(depth_passes, 1),
+        "raster_expand": v * 36 + i * 6,
+        "raster_tile_sort": i * (2 + 12 * ((end_bit + 7) // 8)) / max(tile_passes, 1),
+        "raster_tile_ranges": i * 2,
+        "raster_blend_forward": i * (4 + R) + pixels * 4 * (channels + 1) + n * 4,
+        "raster_blend_backward": i * (4 + R) + pixels * 8 * (channels + 1) + n * (4 * channels + 4),
+        "fill_u32": n * (4 * channels + 4),
+    }
+    return float(table.get(kernel, 0.0))
+
+
+def step_algorithmic_bytes(n, v, i, pixels, channels, end_bit):
+    """Whole forward + backward step under the same model."""
+    R = 8 + 4 + 4 * channels
+    fwd = n * (16 + 4 * channels) + v * (R + 8 + 68 + 20 + 16) + n * 4 \
+        + i * (6 + 2 + 12 * ((end_bit + 7) // 8) + 2 + 4 + R) + pixels * 4 * (channels + 1)
+    bwd = i * (4 + R) + pixels * 8 * (channels + 1) + n * 2 * (4 * channels + 4)
+    return float(fwd), float(bwd)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target duration of the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
+              "(the path is single-GPU, see DESIGN.md for how it would shard)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from inpc_amd import ProbabilityFieldSampler, _lib, synthetic
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    lib = _lib.lib()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    wl = WORKLOADS[args.workload]
+    n, channels, tile = wl["n"], wl["channels"], wl["tile"]
+
+    # ---- inputs ---------------------------------------------------------------------------------------
+    hv = synthetic.camera_on_z(wl["width"], wl["height"], wl["focal"], 6.0)
+    view = hv.to_view(device)
+    oct = synthetic.octree_leaves(wl["leaves"], wl["level"], 4.0, seed=0)
+    centers = torch.from_numpy(oct.centers).to(device)
+    levels = torch.from_numpy(oct.levels).to(device)
+    weights = torch.from_numpy(oct.weights).to(device)
+    sampler = ProbabilityFieldSampler(seed=0)
+    positions, _ = sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)  # warm-up
+    sampler = ProbabilityFieldSampler(seed=0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    positions, leaf_ids = sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)
+    torch.cuda.synchronize()
+    sampler_ms = (time.perf_counter() - t0) * 1e3
+
+    gen = torch.Generator(device=device).manual_seed(1)
+    features = torch.randn((n, channels), generator=gen, device=device, dtype=torch.float32)
+    opacities = torch.sigmoid(torch.randn(n, generator=gen, device=device, dtype=torch.float32))
+    H, W = wl["height"], wl["width"]
+    grad_image = torch.randn((channels, H, W), generator=gen, device=device) * 1e-2
+    grad_alpha = torch.randn((1, H, W), generator=gen, device=device) * 1e-2
+
+    cfg = _lib.RasterConfig(n, tile, channels, _lib.FEAT_DIRECT_F32, 0, _lib.make_camera(hv.camera))
+    layout = _lib.RasterLayout()
+    _lib.check(lib.inpc_raster_layout_query(C.byref(cfg), C.byref(layout)), "layout")
+    workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+    image = torch.empty((channels, H, W), dtype=torch.float32, device=device)
+    alpha = torch.empty((1, H, W), dtype=torch.float32, device=device)
+    blending_weights = torch.empty(n, dtype=torch.float32, device=device)
+    grad_features = torch.empty((n, channels), dtype=torch.float32, device=device)
+    grad_opacities = torch.empty(n, dtype=torch.float32, device=device)
+    w2c, cam_position = view.w2c.contiguous(), view.position.contiguous()
+    stream = _lib.current_stream()
+
+    def forward():
+        _lib.check(lib.inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
+                                           _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image), _lib.ptr(alpha),
+                                           _lib.ptr(blending_weights), None, _lib.ptr(workspace), layout.total_bytes,
+                                           stream), "inpc_raster_forward")
+
+    def backward():
+        _lib.check(lib.inpc_raster_backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha), _lib.ptr(image),
+                                            _lib.ptr(alpha), _lib.ptr(positions), _lib.ptr(features),
+                                            _lib.ptr(opacities), _lib.ptr(cam_position), _lib.ptr(grad_features),
+                                            _lib.ptr(grad_opacities), None, _lib.ptr(workspace), layout.total_bytes,
+                                            stream), "inpc_raster_backward")
+
+    def step():
+        forward()
+        backward()
+
+    # ---- timed region ---------------------------------------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    counters = (C.c_uint32 * 3)()
+    _lib.check(lib.inpc_raster_read_counters(C.byref(cfg), _lib.ptr(workspace), C.byref(counters), stream), "counters")
+    n_visible, n_instances = int(counters[0]), int(counters[1])
+
+    # forward alone / backward alone
+    def time_calls(fn, reps):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e3 / reps
+
+    fwd_ms = time_calls(forward, args.steps)
+    bwd_ms = time_calls(backward, args.steps)
+
+    # ---- per-kernel durations: HIP events around every launch, on the launch stream, same steps ----------
+    with _lib.KernelTimer() as timer:
+        for _ in range(args.steps):
+            step()
+    per_kernel = {}
+    for name, ms in timer.records:
+        tot, cnt = per_kernel.get(name, (0.0, 0))
+        per_kernel[name] = (tot + ms, cnt + 1)
+    depth_passes = max(per_kernel.get("raster_depth_sort", (0, 0))[1] // args.steps, 1)
+    tile_passes = max(per_kernel.get("raster_tile_sort", (0, 0))[1] // args.steps, 1)
+    pixels = H * W
+    kernels = []
+    for name, (tot, cnt) in sorted(per_kernel.items(), key=lambda kv: -kv[1][0]):
+        avg_ms = tot / cnt
+        alg = algorithmic_bytes(name, n, n_visible, n_instances, pixels, channels, depth_passes, tile_passes,
+                                layout.end_bit)
+        kernels.append({"kernel": name, "launches_per_step": cnt / args.steps, "avg_ms": round(avg_ms, 5),
+                        "ms_per_step": round(tot / args.steps, 5),
+                        "algorithmic_GBps": round(alg / (avg_ms * 1e-3) / 1e9, 1) if avg_ms > 0 else None})
+    dominant = kernels[0]
+    dom_alg = algorithmic_bytes(dominant["kernel"], n, n_visible, n_instances, pixels, channels, depth_passes,
+                                tile_passes, layout.end_bit)
+    achieved = dom_alg / (dominant["avg_ms"] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dominant["kernel"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes_per_launch": dom_alg, "avg_launch_ms": dominant["avg_ms"]}
+    fwd_bytes, bwd_bytes = step_algorithmic_bytes(n, n_visible, n_instances, pixels, channels, layout.end_bit)
+    step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same workload --------------------------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import oracle as O
+
+        n_cpu = min(n, 1_048_576)
+        c = hv.camera
+        cam = O.make_camera(c.width, c.height, c.focal_x, c.focal_y, c.center_x, c.center_y, c.near_plane,
+                            c.far_plane)
+        ocfg = O.make_config(n_cpu, cam, tile, channels, O.FEAT_DIRECT_F32)
+        pos_h = positions[:n_cpu].cpu().numpy()
+        feat_h = features[:n_cpu].cpu().numpy()
+        opac_h = opacities[:n_cpu].cpu().numpy()
+        gi_h, ga_h = grad_image.cpu().numpy(), grad_alpha.cpu().numpy()
+        O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)  # warm-up
+        reps, spent = 0, 0.0
+        while spent < args.cpu_seconds and reps < 50:
+            t = O.now()
+            O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)
+            spent += O.now() - t
+            reps += 1
+        cpu = {"value": round(n_cpu * reps / spent / 1e6, 3), "unit": "Mpoints/s", "cores": O.num_threads(),
+               "kind": "port",
+               "sample": f"first {n_cpu} of the {n} points, same camera/image/channels/tiles, forward+backward, "
+                         f"{reps} repetitions, {spent:.1f} s"}
+
+    out = {
+        "metric": "Mpoints/s, rasterizer fwd+bwd, 8M pts @1237x822 (ms/frame in ms_per_step)",
+        "value": round(n / (ms_per_step * 1e-3) / 1e6, 2),
+        "unit": "Mpoints/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": wl["describe"], "n_points": n, "n_visible": n_visible, "n_instances": n_instances,
+                   "image": [W, H], "channels": channels, "tile": tile},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": {
+            "forward_ms": round(fwd_ms, 4), "backward_ms": round(bwd_ms, 4),
+            "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
+            "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
+            "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),
+            "kernels": kernels,
+        },
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -788,12 +788,8 @@ struct oracle_raster_debug {
 };
 
 // Forward / inference (B/rasterization/src/bilinear/forward.cu:12-170, kernels.cu:241-313,422-495).
-int oracle_raster_forward(const inpc_raster_config* cfg, const float* positions, const void* features,
-                          const float* opacities, const float* w2c, const float* cam_position, float* image,
-                          float* alpha, float* blending_weights, float* depth_image, oracle_raster_debug* dbg) {
-    RasterState st;
-    const int rc = raster_prepare(st, cfg, positions, features, opacities, w2c, cam_position);
-    if (rc != INPC_OK) return rc;
+static int raster_forward_with_state(const RasterState& st, const inpc_raster_config* cfg, float* image, float* alpha,
+                                     float* blending_weights, float* depth_image, oracle_raster_debug* dbg) {
     const int W = cfg->cam.width, H = cfg->cam.height, T = st.T, C = st.C;
     const bool inference = (cfg->flags & INPC_RASTER_INFERENCE) != 0;
     const size_t n_pixels = (size_t)W * H;
@@ -880,13 +876,10 @@ int oracle_raster_forward(const inpc_raster_config* cfg, const float* positions,
 // Backward (B/rasterization/src/bilinear/backward.cu:9-67, kernels.cu:86-104,315-420).
 // grad_features: (N,36) fp16 [SH36], (N,C) f32 [DIRECT_F32], (N,C) fp16 [DIRECT_F16];
 // grad_view_out (N,C) f32 optional copy of the per-point view-space feature gradient.
-int oracle_raster_backward(const inpc_raster_config* cfg, const float* grad_image, const float* grad_alpha,
-                           const float* image, const float* alpha, const float* positions, const void* features,
-                           const float* opacities, const float* w2c, const float* cam_position,
-                           void* grad_features, float* grad_opacities, float* grad_view_out) {
-    RasterState st;
-    const int rc = raster_prepare(st, cfg, positions, features, opacities, w2c, cam_position);
-    if (rc != INPC_OK) return rc;
+static int raster_backward_with_state(const RasterState& st, const inpc_raster_config* cfg, const float* grad_image,
+                                      const float* grad_alpha, const float* image, const float* alpha,
+                                      const float* positions, const float* cam_position, void* grad_features,
+                                      float* grad_opacities, float* grad_view_out) {
     const int W = cfg->cam.width, H = cfg->cam.height, T = st.T, C = st.C;
     const size_t n_pixels = (size_t)W * H;
     std::vector<float> gview((size_t)st.n * C, 0.0f);
@@ -976,6 +969,41 @@ int oracle_raster_backward(const inpc_raster_config* cfg, const float* grad_imag
         return INPC_E_UNSUPPORTED;
     }
     return INPC_OK;
+}
+
+int oracle_raster_forward(const inpc_raster_config* cfg, const float* positions, const void* features,
+                          const float* opacities, const float* w2c, const float* cam_position, float* image,
+                          float* alpha, float* blending_weights, float* depth_image, oracle_raster_debug* dbg) {
+    RasterState st;
+    const int rc = raster_prepare(st, cfg, positions, features, opacities, w2c, cam_position);
+    if (rc != INPC_OK) return rc;
+    return raster_forward_with_state(st, cfg, image, alpha, blending_weights, depth_image, dbg);
+}
+
+int oracle_raster_backward(const inpc_raster_config* cfg, const float* grad_image, const float* grad_alpha,
+                           const float* image, const float* alpha, const float* positions, const void* features,
+                           const float* opacities, const float* w2c, const float* cam_position,
+                           void* grad_features, float* grad_opacities, float* grad_view_out) {
+    RasterState st;
+    const int rc = raster_prepare(st, cfg, positions, features, opacities, w2c, cam_position);
+    if (rc != INPC_OK) return rc;
+    return raster_backward_with_state(st, cfg, grad_image, grad_alpha, image, alpha, positions, cam_position,
+                                      grad_features, grad_opacities, grad_view_out);
+}
+
+// Forward followed by backward on the same saved state, as one training step does (the sort and the
+// per-point records are computed once). Used as the timed CPU baseline.
+int oracle_raster_forward_backward(const inpc_raster_config* cfg, const float* positions, const void* features,
+                                   const float* opacities, const float* w2c, const float* cam_position,
+                                   const float* grad_image, const float* grad_alpha, float* image, float* alpha,
+                                   float* blending_weights, void* grad_features, float* grad_opacities) {
+    RasterState st;
+    int rc = raster_prepare(st, cfg, positions, features, opacities, w2c, cam_position);
+    if (rc != INPC_OK) return rc;
+    rc = raster_forward_with_state(st, cfg, image, alpha, blending_weights, nullptr, nullptr);
+    if (rc != INPC_OK) return rc;
+    return raster_backward_with_state(st, cfg, grad_image, grad_alpha, image, alpha, positions, cam_position,
+                                      grad_features, grad_opacities, nullptr);
 }
 
 // Wall-clock helper for benchmarks: seconds since an arbitrary origin.

@@ -343,3 +343,33 @@ def raster_backward(cfg: RasterConfig, grad_image, grad_alpha, image, alpha, pos
     if rc != 0:
         raise RuntimeError(f"oracle_raster_backward failed with {rc}")
     return gf, go, gv
+
+
+def raster_forward_backward(cfg: RasterConfig, positions, features, opacities, w2c, grad_image, grad_alpha,
+                            cam_position=None):
+    """One training step on shared state. Returns (image, alpha, blending_weights, grad_features, grad_opacities)."""
+    n = cfg.n_points
+    W, H = cfg.cam.width, cfg.cam.height
+    sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
+    Cn = 4 if sh else cfg.channels
+    positions, w2c = _f32(positions), _f32(w2c)
+    features = _features_array(features, cfg.feature_mode)
+    opacities = _f32(opacities).reshape(-1)
+    cam_position = _f32(np.zeros(3) if cam_position is None else cam_position)
+    grad_image, grad_alpha = _f32(grad_image), _f32(grad_alpha)
+    image = np.zeros((Cn, H, W), dtype=np.float32)
+    alpha = np.zeros((1, H, W), dtype=np.float32)
+    bw = np.zeros(n, dtype=np.float32)
+    if cfg.feature_mode == FEAT_SH36_F16:
+        gf = np.zeros((n, 36), dtype=np.float16)
+    elif cfg.feature_mode == FEAT_DIRECT_F16:
+        gf = np.zeros((n, Cn), dtype=np.float16)
+    else:
+        gf = np.zeros((n, Cn), dtype=np.float32)
+    go = np.zeros(n, dtype=np.float32)
+    rc = lib().oracle_raster_forward_backward(C.byref(cfg), _p(positions), _p(features), _p(opacities), _p(w2c),
+                                              _p(cam_position), _p(grad_image), _p(grad_alpha), _p(image), _p(alpha),
+                                              _p(bw), _p(gf), _p(go))
+    if rc != 0:
+        raise RuntimeError(f"oracle_raster_forward_backward failed with {rc}")
+    return image, alpha, bw, gf, go

@@ -72,7 +72,7 @@ def test_forward_dense_opaque_scene_terminates_early(gpu, oracle, tile):
                                 debug=True)
     check_structure(run.debug(), ref)
     out = run.outputs()
-    assert (ref["alpha"] == 1.0).mean() > 0.5  # most pixels saturate
+    assert (ref["alpha"] == 1.0).mean() > 0.3  # a large share of the pixels saturates
     H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
     H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
     H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
