@@ -135,12 +135,15 @@ constexpr uint32_t kFlagInclusive = 2u << 30;
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
 constexpr uint32_t kSpinLimit = 1u << 22;
 
+// Status words carry their payload themselves and no other memory is handed over between blocks of
+// one launch, so relaxed agent-scope accesses suffice. (Acquire / release at agent scope would make every
+// access write back or invalidate the whole L2 of its XCD.)
 __device__ __forceinline__ void status_store(uint32_t* p, uint32_t v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ uint32_t status_load(const uint32_t* p) {
-    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Exclusive prefix of `aggregate` over blocks 0..bid-1, publishing this block's words on the way.
