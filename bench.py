@@ -44,6 +44,7 @@ def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, depth_passes, tile
     F = 4 * channels
     R = 8 + 4 + 4 * channels
     table = {
+        "raster_bin_count": n * 12,
         "raster_preprocess": n * (16 + F) + v * (R + 8),
         "raster_depth_sort": v * 68 / max(depth_passes, 1),
         "raster_expand": v * 36 + i * 6,
@@ -136,10 +137,9 @@ def main() -> int:
 
     def backward():
         _lib.check(lib.inpc_raster_backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha), _lib.ptr(image),
-                                            _lib.ptr(alpha), _lib.ptr(positions), _lib.ptr(features),
-                                            _lib.ptr(opacities), _lib.ptr(cam_position), _lib.ptr(grad_features),
-                                            _lib.ptr(grad_opacities), None, _lib.ptr(workspace), layout.total_bytes,
-                                            stream), "inpc_raster_backward")
+                                            _lib.ptr(alpha), _lib.ptr(positions), _lib.ptr(cam_position),
+                                            _lib.ptr(grad_features), _lib.ptr(grad_opacities), None,
+                                            _lib.ptr(workspace), layout.total_bytes, stream), "inpc_raster_backward")
 
     def step():
         forward()

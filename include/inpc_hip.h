@@ -187,18 +187,26 @@ typedef struct inpc_raster_config {
 } inpc_raster_config;
 
 /* Offsets (bytes from the workspace base) of the buffers a caller may want to inspect.
- * The layout is private otherwise. Counts live in device memory. */
+ * The layout is private otherwise. Counts live in device memory.
+ *
+ * A drawn point owns one blend record of `record_stride` bytes; the records of the points whose first
+ * touched tile is t occupy slots bin_start[t] .. bin_start[t+1]-1, in no particular order. Sorted
+ * orders refer to record slots; the header of a record names its point:
+ *   float sx, sy, opacity; u32 point id; u32 tile info; float depth; 2 unused words; then the view
+ *   features (fp32, or fp16 for INPC_FEAT_DIRECT_F16).
+ *   tile info: bits 0-15 first tile id, bit 16 spans two tiles in x, bit 17 in y, bit 18 drawn. */
 typedef struct inpc_raster_layout {
     size_t total_bytes;
     size_t counters;        /* u32[16]: [0] n_visible, [1] n_instances, [2] error flag          */
-    size_t point_record;    /* (N) {float sx, sy, opacity; u32 tileinfo}                        */
-    size_t point_depth;     /* (N) f32 view-space depth                                         */
-    size_t features_view;   /* (N,4) f32, SH modes only, else 0                                 */
-    size_t depth_order;     /* (N) u32: point ids in (depth, id) order, first n_visible valid   */
-    size_t depth_keys;      /* (N) u32: matching depth keys (float bits), first n_visible valid */
+    size_t bin_start;       /* u32[n_tiles + 1]                                                 */
+    size_t point_record;    /* n_visible records of record_stride bytes, binned by first tile   */
+    size_t depth_order;     /* (N) u32: (record slot << 2 | span bits) in (depth, point id)
+                               order, first n_visible valid                                     */
+    size_t depth_keys;      /* (N) u32: matching depth keys, first n_visible valid              */
     size_t instance_keys;   /* (4N) u16: tile id per instance in final order                    */
-    size_t instance_points; /* (4N) u32: point id per instance in final order                   */
+    size_t instance_slots;  /* (4N) u32: record slot per instance in final order                */
     size_t tile_ranges;     /* (n_tiles) {u32 begin, end}                                       */
+    uint32_t record_stride;
     uint32_t grid_width;
     uint32_t grid_height;
     uint32_t n_tiles;
@@ -234,17 +242,18 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
  * bilinear::backward (B/rasterization/src/bilinear/backward.cu:9-67), blend_backward_cu and
  * preprocess_backward_cu (B/rasterization/src/bilinear/kernels.cu:86-104,315-420).
  *   grad_image (C,H,W), grad_alpha (1,H,W), image, alpha: f32, as produced by forward;
+ *   positions, cam_position: as in forward (read by the SH mode only, may be NULL otherwise);
  *   grad_features: (N,36) fp16 for INPC_FEAT_SH36_F16, (N,C) f32 for INPC_FEAT_DIRECT_F32,
  *                  (N,C) fp16 for INPC_FEAT_DIRECT_F16; fully written (zeros where a point
  *                  was not drawn);
  *   grad_opacities (N,) f32, fully written;
- *   grad_view_scratch: (N,4) f32 scratch for the SH mode, else NULL. */
+ *   grad_view_scratch: (N,C) f32 scratch for the SH and fp16 modes, else NULL.
+ * The features and opacities themselves are not needed: the workspace holds what the blend used. */
 int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
                          const float* grad_alpha, const float* image, const float* alpha,
-                         const float* positions, const void* features, const float* opacities,
-                         const float* cam_position, void* grad_features, float* grad_opacities,
-                         float* grad_view_scratch, void* workspace, size_t workspace_bytes,
-                         void* stream);
+                         const float* positions, const float* cam_position, void* grad_features,
+                         float* grad_opacities, float* grad_view_scratch, void* workspace,
+                         size_t workspace_bytes, void* stream);
 
 /* Copy the rasterizer counters {n_visible, n_instances, error flag} to the host.
  * Synchronises `stream`. Returns INPC_E_DEVICE if the error flag is set. */

@@ -47,14 +47,14 @@ class RasterLayout(C.Structure):
     _fields_ = [
         ("total_bytes", C.c_size_t),
         ("counters", C.c_size_t),
+        ("bin_start", C.c_size_t),
         ("point_record", C.c_size_t),
-        ("point_depth", C.c_size_t),
-        ("features_view", C.c_size_t),
         ("depth_order", C.c_size_t),
         ("depth_keys", C.c_size_t),
         ("instance_keys", C.c_size_t),
-        ("instance_points", C.c_size_t),
+        ("instance_slots", C.c_size_t),
         ("tile_ranges", C.c_size_t),
+        ("record_stride", C.c_uint32),
         ("grid_width", C.c_uint32),
         ("grid_height", C.c_uint32),
         ("n_tiles", C.c_uint32),
@@ -96,7 +96,7 @@ SIGNATURES = {
     "inpc_expected_samples": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _U32, _F, _P, _P]),
     "inpc_raster_layout_query": (C.c_int, [_CFG, C.POINTER(RasterLayout)]),
     "inpc_raster_forward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
-    "inpc_raster_backward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "inpc_raster_backward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "inpc_raster_read_counters": (C.c_int, [_CFG, _P, C.POINTER(_U32 * 3), _P]),
     "inpc_timing_enable": (None, [C.c_int]),
     "inpc_timing_collect": (C.c_int, [C.POINTER(TimingRecord), C.c_int]),

@@ -177,4 +177,38 @@ __device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_
     return exclusive;
 }
 
+// The same for a single value per block, walked by a whole wave: the 64 lanes look at 64 predecessors at
+// a time. Every lane of the calling wave must enter; all get the result.
+__device__ __forceinline__ uint32_t lookback_exclusive_wave(uint32_t* status, uint32_t bid, uint32_t aggregate,
+                                                            uint32_t* error_flag) {
+    const uint32_t lane = lane_id();
+    if (lane == 0) status_store(status + bid, (bid == 0 ? kFlagInclusive : kFlagAggregate) | aggregate);
+    if (bid == 0) return 0u;
+    uint32_t exclusive = 0u, spins = 0u;
+    int64_t window = (int64_t)bid - 1;  // lane l looks at block window - l
+    for (;;) {
+        const int64_t p = window - (int64_t)lane;
+        const uint32_t word = p >= 0 ? status_load(status + p) : kFlagInclusive;  // before block 0: nothing
+        const uint64_t ready = __ballot((word & ~kValueMask) != 0u);
+        const uint64_t inclusive = __ballot((word & kFlagInclusive) != 0u);
+        const uint32_t last = inclusive ? (uint32_t)__builtin_ctzll(inclusive) : 63u;  // walk ends at this lane
+        const uint64_t needed = last == 63u ? ~0ull : ((2ull << last) - 1ull);
+        if ((ready & needed) == needed) {
+            uint32_t v = lane <= last ? (word & kValueMask) : 0u;
+            for (int s = 32; s > 0; s >>= 1) v += __shfl_xor(v, s, 64);
+            exclusive += v;
+            if (inclusive) break;
+            window -= 64;
+        } else {
+            if (++spins > kSpinLimit) {
+                if (lane == 0) atomicOr(error_flag, 1u);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+    }
+    if (lane == 0) status_store(status + bid, kFlagInclusive | ((exclusive + aggregate) & kValueMask));
+    return exclusive;
+}
+
 }  // namespace inpc

@@ -92,8 +92,14 @@ __global__ void __launch_bounds__(kRadix) k_digit_bases(const uint32_t* __restri
     bases[blockIdx.x * kRadix + d] = base + incl - v;
 }
 
-// One digit pass. FIRST: the values are the element indices themselves, keys equal to kInvalidKey
-// are dropped (this compacts the visible points for free) and n comes from the host.
+// How the first pass of a sort treats its input.
+enum FirstPass : int {
+    kPlain = 0,        // n keys (n on the device), all valid
+    kSkipInvalid = 1,  // n_max keys (n on the host); keys equal to kInvalidKey are dropped, which compacts
+                       // the drawn points for free
+};
+
+// One digit pass. FIRST: n comes from the host and keys equal to kInvalidKey are dropped.
 template <typename KeyT, bool FIRST>
 __global__ void __launch_bounds__(kBlock)
     k_scatter(const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
@@ -129,12 +135,8 @@ __global__ void __launch_bounds__(kBlock)
         bool valid = idx < n;
         KeyT k = 0;
         if (valid) k = keys_in[idx];
-        if (FIRST) {
-            valid = valid && ((uint32_t)k != kInvalidKey);
-            val[r] = (uint32_t)idx;
-        } else {
-            val[r] = valid ? vals_in[idx] : 0u;
-        }
+        if (FIRST) valid = valid && ((uint32_t)k != kInvalidKey);
+        val[r] = valid ? vals_in[idx] : 0u;
         key[r] = k;
         const uint32_t d = ((uint32_t)k >> shift) & digit_mask;
         uint64_t peers = __ballot(valid);
@@ -214,12 +216,12 @@ __global__ void __launch_bounds__(kBlock)
 // Status words one pass needs for up to n_max keys.
 inline size_t status_words(uint32_t n_max) { return (size_t)div_up(n_max, kTile) * kRadix; }
 
-// Enqueue every pass of a sort. Buffers ping-pong: pass 0 reads keys_a (and, unless `first`, vals_a),
-// the result ends in the a-buffers when the pass count is even, else in the b-buffers.
+// Enqueue every pass of a sort. Buffers ping-pong: pass 0 reads keys_a / vals_a, the result ends in the
+// a-buffers when the pass count is even, else in the b-buffers.
 // hist: n_passes*256 filled histograms; bases: same size scratch; status: n_passes*status_words(n_max)
 // zeroed words; tickets: n_passes zeroed words.
 template <typename KeyT>
-int sort_pairs(const PassPlan& plan, bool first_identity, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b,
+int sort_pairs(const PassPlan& plan, FirstPass first, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b,
                uint32_t* vals_b, const uint32_t* n_dev, uint32_t n_max, const uint32_t* hist, uint32_t* bases,
                uint32_t* status, uint32_t* tickets, uint32_t* error_flag, hipStream_t stream, const char* name) {
     if (n_max == 0) return INPC_OK;
@@ -232,7 +234,7 @@ int sort_pairs(const PassPlan& plan, bool first_identity, KeyT* keys_a, uint32_t
     uint32_t* vout = vals_b;
     for (int p = 0; p < plan.n_passes; ++p) {
         const uint32_t mask = (1u << plan.bits[p]) - 1u;
-        if (p == 0 && first_identity) {
+        if (p == 0 && first == kSkipInvalid) {
             INPC_LAUNCH(name, (k_scatter<KeyT, true>), dim3(blocks), dim3(kBlock), stream, (const KeyT*)kin,
                         (const uint32_t*)vin, kout, vout, n_dev, n_max, plan.shift[p], mask, plan.bits[p],
                         (const uint32_t*)(bases + p * kRadix), status + p * words, tickets + p, error_flag);

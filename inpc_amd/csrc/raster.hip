@@ -1,12 +1,15 @@
 // raster.hip — tile-based differentiable bilinear point rasterizer for gfx950.
 //
 // Pipeline (all on the caller's stream, counts stay on the device):
-//   k_preprocess     project, cull, tile bounds, blend record, depth key, depth-digit histograms
-//                    (B/rasterization/src/bilinear/kernels.cu:11-84,106-184)
-//   radix sort       stable sort of the visible points by depth key; the first pass drops the
-//                    culled points, in ascending point id (forward.cu:91-98)
+//   k_bin_count      project every point and count the drawn ones per first touched tile
+//   k_bin_scan       exclusive scan of the counts: start of every tile's record bin
+//   k_preprocess     project, cull, tile bounds, depth key, depth-digit histograms; the blend record of a
+//                    drawn point (screen position, opacity, point id, view features) is written into the
+//                    bin of its first tile (B/rasterization/src/bilinear/kernels.cu:11-84,106-184)
+//   radix sort       stable sort of the drawn points by depth key; the first pass drops the culled
+//                    points, ties keep ascending point id (forward.cu:91-98)
 //   k_expand         per depth-sorted point: instance offsets (single-pass scan) and one
-//                    (tile, point) instance per touched tile, row-major; tile-digit histograms
+//                    (tile, record slot) instance per touched tile, row-major; tile-digit histograms
 //                    (kernels.cu:186-220, forward.cu:101-130)
 //   radix sort       stable sort of the instances by tile id (forward.cu:132-139)
 //   k_tile_ranges    [begin, end) of every tile (kernels.cu:222-239)
@@ -16,10 +19,11 @@
 //   k_sh_backward    view-space feature gradient -> 36 fp16 SH coefficient gradients
 //                    (kernels.cu:86-104, sh_utils.cuh:44-62)
 //
-// The blend kernels do not test every pixel against every instance. For a batch of instances staged
-// in LDS, each wave builds, with one ballot per tile column and per tile row, 64-bit masks of the
-// instances whose footprint covers that column / row (the exact float test of the reference). A pixel
-// ANDs its column and row mask and walks the set bits, i.e. exactly its own hits, in depth order.
+// Why the records are binned: the points arrive in no spatial order, and on this memory system a random
+// gather costs a whole 128-byte line whatever it uses of it, while a random aligned 64-byte store costs
+// 64 bytes. So the one pass that already reads every point scatters a 64-byte record per point into the
+// bin of its tile; the blend of a tile then gathers from a few contiguous kilobytes instead of from the
+// whole point cloud, and every fetched line is used completely.
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -48,13 +52,18 @@ enum Counter : int {
     kCntWords = 16
 };
 
-// tileinfo word of the blend record
+// tile info word: first tile id, spans, valid
 constexpr uint32_t kInfoValid = 1u << 18;
 __device__ __forceinline__ uint32_t info_tile0(uint32_t info) { return info & 0xFFFFu; }
 __device__ __forceinline__ uint32_t info_nx(uint32_t info) { return ((info >> 16) & 1u) + 1u; }
 __device__ __forceinline__ uint32_t info_ny(uint32_t info) { return ((info >> 17) & 1u) + 1u; }
-__device__ __forceinline__ uint32_t info_count(uint32_t info) {
-    return (info & kInfoValid) ? info_nx(info) * info_ny(info) : 0u;
+
+// Blend record of a drawn point: a 32-byte header followed by the view features, padded to a multiple
+// of 32 bytes (64 bytes for every configuration but 16 fp32 channels).
+//   header: float sx, sy, opacity; u32 point id; u32 tile info; float depth; 2 words unused
+constexpr uint32_t kRecordHeader = 32;
+inline uint32_t record_stride(int channels, bool half_features) {
+    return (uint32_t)align_up(kRecordHeader + (size_t)channels * (half_features ? 2 : 4), 32);
 }
 
 struct Geometry {
@@ -63,6 +72,7 @@ struct Geometry {
     uint32_t gw, gh, n_tiles;
     Camera cam;
     uint32_t key_bias;  // depth key = float bits - key_bias
+    uint32_t stride;    // record stride in bytes
 };
 
 // ---- SH degree 2 (sh_utils.cuh:6-23) ---------------------------------------------------------------------
@@ -100,66 +110,192 @@ __device__ __forceinline__ float4 sh_to_view(const ShBasis& s, const __half* __r
     return make_float4(acc[0], acc[1], acc[2], acc[3]);
 }
 
+// ---- projection (kernels.cu:40-64) ---------------------------------------------------------------------------
+struct Projected {
+    float sx, sy, depth;
+    uint32_t info;     // 0 when the point is not drawn
+    uint32_t touched;  // number of tiles
+};
+
+struct ViewRows {
+    float4 r1, r2, r3;
+};
+
+__device__ __forceinline__ ViewRows load_view_rows(const float* __restrict__ w2c) {
+    ViewRows m;
+    m.r1 = make_float4(w2c[0], w2c[1], w2c[2], w2c[3]);
+    m.r2 = make_float4(w2c[4], w2c[5], w2c[6], w2c[7]);
+    m.r3 = make_float4(w2c[8], w2c[9], w2c[10], w2c[11]);
+    return m;
+}
+
+template <int T>
+__device__ __forceinline__ Projected project_point(const ViewRows& m, const Geometry& g, float px, float py, float pz) {
+    Projected o;
+    o.sx = 0.0f;
+    o.sy = 0.0f;
+    o.info = 0u;
+    o.touched = 0u;
+    o.depth = affine_row(m.r3, px, py, pz);
+    if (o.depth < g.cam.near_plane || o.depth > g.cam.far_plane) return o;
+    const float fT = (float)T, fgw = (float)g.gw, fgh = (float)g.gh;
+    const float x = affine_row(m.r1, px, py, pz) / o.depth;
+    const float y = affine_row(m.r2, px, py, pz) / o.depth;
+    o.sx = x * g.cam.fx + g.cam.cx;
+    o.sy = y * g.cam.fy + g.cam.cy;
+    const uint32_t x0 = (uint32_t)fminf(fgw, fmaxf(0.0f, floorf((o.sx - 0.5f) / fT)));
+    const uint32_t x1 = (uint32_t)fminf(fgw, fmaxf(0.0f, ceilf((o.sx + 0.5f) / fT)));
+    const uint32_t y0 = (uint32_t)fminf(fgh, fmaxf(0.0f, floorf((o.sy - 0.5f) / fT)));
+    const uint32_t y1 = (uint32_t)fminf(fgh, fmaxf(0.0f, ceilf((o.sy + 0.5f) / fT)));
+    o.touched = (x1 - x0) * (y1 - y0);
+    if (o.touched != 0u) o.info = (y0 * g.gw + x0) | ((x1 - x0 - 1u) << 16) | ((y1 - y0 - 1u) << 17) | kInfoValid;
+    return o;
+}
+
+// ---- record bins ------------------------------------------------------------------------------------------------
+// The points are cut into kBinBlocks contiguous chunks, one per block, the same way in k_bin_count and in
+// k_preprocess. k_bin_count leaves, per (chunk, tile), the number of drawn points of the chunk whose first
+// tile it is; k_bin_offsets turns that table into the exclusive prefix over the chunks of every tile and
+// k_bin_scan into the start of every tile's bin. k_preprocess then hands out slots from LDS cursors
+// seeded with bin_start[tile] + prefix[chunk][tile]: no global atomic anywhere (they run at about
+// 10 G/s on this machine, far below what 8M points need).
+constexpr int kBinBlocks = 512;
+constexpr int kBinThreads = 512;
+constexpr uint32_t kMaxLdsTiles = 16384;  // tile counters a block keeps in LDS (64 KiB)
+
+__host__ __device__ inline uint32_t bin_chunk_size(uint32_t n) {
+    const uint32_t per = (n + kBinBlocks - 1) / kBinBlocks;
+    return (per + kBinThreads - 1) / kBinThreads * kBinThreads;
+}
+
+template <int T>
+__global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restrict__ positions,
+                                                           const float* __restrict__ w2c, uint32_t* __restrict__ table,
+                                                           Geometry g) {
+    extern __shared__ uint32_t s_count[];
+    for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_count[t] = 0u;
+    __syncthreads();
+    const ViewRows m = load_view_rows(w2c);
+    const uint32_t chunk = bin_chunk_size(g.n);
+    const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
+    for (uint32_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
+        const Projected p = project_point<T>(m, g, positions[3 * (size_t)i], positions[3 * (size_t)i + 1],
+                                             positions[3 * (size_t)i + 2]);
+        if (p.info) atomicAdd(&s_count[info_tile0(p.info)], 1u);
+    }
+    __syncthreads();
+    uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
+    for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) row[t] = s_count[t];
+}
+
+// table[c][t] <- sum of table[c'][t] over c' < c; total[t] <- sum over all chunks.
+__global__ void __launch_bounds__(kBlock) k_bin_offsets(uint32_t* __restrict__ table, uint32_t* __restrict__ total,
+                                                        uint32_t n_tiles) {
+    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= n_tiles) return;
+    uint32_t run = 0;
+    for (int c = 0; c < kBinBlocks; ++c) {
+        const uint32_t v = table[(size_t)c * n_tiles + t];
+        table[(size_t)c * n_tiles + t] = run;
+        run += v;
+    }
+    total[t] = run;
+}
+
+// bin_start[t] = number of records in bins before t (n_tiles + 1 entries).
+constexpr int kScanBlock = 1024;
+__global__ void __launch_bounds__(kScanBlock) k_bin_scan(const uint32_t* __restrict__ bin_count,
+                                                         uint32_t* __restrict__ bin_start, uint32_t n_tiles) {
+    __shared__ uint32_t s_wave[kScanBlock / kWave];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t per = (n_tiles + kScanBlock - 1) / kScanBlock;
+    const uint32_t begin = min(tid * per, n_tiles), end = min(begin + per, n_tiles);
+    uint32_t mine = 0;
+    for (uint32_t t = begin; t < end; ++t) mine += bin_count[t];
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s, 64);
+        if (lane >= (uint32_t)s) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - mine;
+    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
+    for (uint32_t t = begin; t < end; ++t) {
+        bin_start[t] = run;
+        run += bin_count[t];
+    }
+    if (end == n_tiles && begin < n_tiles) bin_start[n_tiles] = run;
+}
+
 // ---- preprocess -------------------------------------------------------------------------------------------
-template <int T, int FMODE>
-__global__ void __launch_bounds__(kBlock)
+template <int T, int FMODE, int C>
+__global__ void __launch_bounds__(kBinThreads)
     k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
                  const float* __restrict__ opacities, const float* __restrict__ w2c,
-                 const float* __restrict__ cam_position, float4* __restrict__ rec, float* __restrict__ depth_out,
-                 float4* __restrict__ features_view, uint32_t* __restrict__ keys, float* __restrict__ blending_weights,
+                 const float* __restrict__ cam_position, char* __restrict__ records,
+                 const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start,
+                 uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, float* __restrict__ blending_weights,
                  uint32_t* counters, uint32_t* g_hist, Geometry g, radix::DevicePlan plan) {
-    __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
+    extern __shared__ uint32_t s_dyn[];
+    uint32_t* s_cursor = s_dyn;                 // n_tiles
+    uint32_t* s_hist = s_dyn + g.n_tiles;       // kMaxPasses * kRadix
     __shared__ uint32_t s_visible, s_instances;
-    for (int i = threadIdx.x; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
+    {
+        const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
+        for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_cursor[t] = bin_start[t] + row[t];
+    }
+    for (int i = threadIdx.x; i < plan.n_passes * radix::kRadix; i += kBinThreads) s_hist[i] = 0u;
     if (threadIdx.x == 0) {
         s_visible = 0u;
         s_instances = 0u;
     }
     __syncthreads();
-    const float4 r1 = make_float4(w2c[0], w2c[1], w2c[2], w2c[3]);
-    const float4 r2 = make_float4(w2c[4], w2c[5], w2c[6], w2c[7]);
-    const float4 r3 = make_float4(w2c[8], w2c[9], w2c[10], w2c[11]);
-    const float fT = (float)T, fgw = (float)g.gw, fgh = (float)g.gh;
+    const ViewRows m = load_view_rows(w2c);
     uint32_t my_visible = 0, my_instances = 0;
-    const uint32_t stride = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < g.n; i += stride) {
+    const uint32_t chunk = bin_chunk_size(g.n);
+    const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
+    for (uint32_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
         const float px = positions[3 * (size_t)i], py = positions[3 * (size_t)i + 1], pz = positions[3 * (size_t)i + 2];
-        const float depth = affine_row(r3, px, py, pz);
-        uint32_t info = 0u, key = radix::kInvalidKey;
-        float sx = 0.0f, sy = 0.0f, opacity = 0.0f;
-        if (!(depth < g.cam.near_plane || depth > g.cam.far_plane)) {
-            const float x = affine_row(r1, px, py, pz) / depth;
-            const float y = affine_row(r2, px, py, pz) / depth;
-            sx = x * g.cam.fx + g.cam.cx;
-            sy = y * g.cam.fy + g.cam.cy;
-            const uint32_t x0 = (uint32_t)fminf(fgw, fmaxf(0.0f, floorf((sx - 0.5f) / fT)));
-            const uint32_t x1 = (uint32_t)fminf(fgw, fmaxf(0.0f, ceilf((sx + 0.5f) / fT)));
-            const uint32_t y0 = (uint32_t)fminf(fgh, fmaxf(0.0f, floorf((sy - 0.5f) / fT)));
-            const uint32_t y1 = (uint32_t)fminf(fgh, fmaxf(0.0f, ceilf((sy + 0.5f) / fT)));
-            const uint32_t touched = (x1 - x0) * (y1 - y0);
-            if (touched != 0u) {
-                info = (y0 * g.gw + x0) | ((x1 - x0 - 1u) << 16) | ((y1 - y0 - 1u) << 17) | kInfoValid;
-                key = __float_as_uint(depth) - g.key_bias;
-                my_visible += 1u;
-                my_instances += touched;
-                radix::hist_add(s_hist, plan, key);
+        const Projected p = project_point<T>(m, g, px, py, pz);
+        uint32_t key = radix::kInvalidKey, val = 0u;
+        if (p.info) {
+            key = __float_as_uint(p.depth) - g.key_bias;
+            my_visible += 1u;
+            my_instances += p.touched;
+            radix::hist_add(s_hist, plan, key);
+            const uint32_t slot = atomicAdd(&s_cursor[info_tile0(p.info)], 1u);
+            val = (slot << 2) | ((p.info >> 16) & 3u);
+            float4* rec = (float4*)(records + (size_t)slot * g.stride);
+            float opacity;
+            if (FMODE == INPC_FEAT_SH36_F16 || FMODE == INPC_FEAT_RAW37_F16) {
+                const ShBasis s = sh_basis(px, py, pz, cam_position);
                 if (FMODE == INPC_FEAT_SH36_F16) {
-                    const ShBasis s = sh_basis(px, py, pz, cam_position);
-                    features_view[i] = sh_to_view(s, (const __half*)features + 36 * (size_t)i);
+                    rec[2] = sh_to_view(s, (const __half*)features + 36 * (size_t)i);
                     opacity = opacities[i];
-                } else if (FMODE == INPC_FEAT_RAW37_F16) {
-                    const __half* raw = (const __half*)features + 37 * (size_t)i;
-                    const ShBasis s = sh_basis(px, py, pz, cam_position);
-                    features_view[i] = sh_to_view(s, raw + 1);
-                    opacity = 1.0f - expf(-expf(__half2float(raw[0])));
                 } else {
-                    opacity = opacities[i];
+                    const __half* raw = (const __half*)features + 37 * (size_t)i;
+                    rec[2] = sh_to_view(s, raw + 1);
+                    opacity = 1.0f - expf(-expf(__half2float(raw[0])));  // kernels.cu:142
                 }
+            } else if (FMODE == INPC_FEAT_DIRECT_F32) {
+                const float4* src = (const float4*)features + (size_t)i * (C / 4);
+#pragma unroll
+                for (int q = 0; q < C / 4; ++q) rec[2 + q] = src[q];
+                opacity = opacities[i];
+            } else {
+                const uint2* src = (const uint2*)features + (size_t)i * (C / 4);
+                uint2* dst = (uint2*)(rec + 2);
+#pragma unroll
+                for (int q = 0; q < C / 4; ++q) dst[q] = src[q];
+                opacity = opacities[i];
             }
+            rec[0] = make_float4(p.sx, p.sy, opacity, __uint_as_float(i));
+            rec[1] = make_float4(__uint_as_float(p.info), p.depth, 0.0f, 0.0f);
         }
-        rec[i] = make_float4(sx, sy, opacity, __uint_as_float(info));
-        depth_out[i] = depth;
         keys[i] = key;
+        vals[i] = val;
         if (blending_weights) blending_weights[i] = 0.0f;
     }
     // block totals -> one global atomic each
@@ -183,10 +319,22 @@ __global__ void __launch_bounds__(kBlock)
 constexpr int kExpandItems = 4;
 constexpr int kExpandTile = kBlock * kExpandItems;
 
+// Tile whose record bin holds `slot`: the last t with bin_start[t] <= slot.
+__device__ __forceinline__ uint32_t tile_of_slot(const uint32_t* __restrict__ bin_start, uint32_t n_tiles, uint32_t slot) {
+    uint32_t lo = 0, hi = n_tiles;  // invariant: bin_start[lo] <= slot < bin_start[hi]
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (bin_start[mid] <= slot) lo = mid;
+        else hi = mid;
+    }
+    return lo;
+}
+
 __global__ void __launch_bounds__(kBlock)
-    k_expand(const uint32_t* __restrict__ depth_order, const float4* __restrict__ rec, uint16_t* __restrict__ inst_keys,
-             uint32_t* __restrict__ inst_points, uint32_t* counters, uint32_t* status, uint32_t* g_hist, uint32_t gw,
-             radix::DevicePlan plan) {
+    k_expand(const uint32_t* __restrict__ depth_order, const uint32_t* __restrict__ bin_start_global,
+             uint16_t* __restrict__ inst_keys, uint32_t* __restrict__ inst_points, uint32_t* counters, uint32_t* status,
+             uint32_t* g_hist, uint32_t gw, uint32_t n_tiles, radix::DevicePlan plan) {
+    extern __shared__ uint32_t s_bin_start[];  // n_tiles + 1 entries
     __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
     __shared__ uint32_t s_wave[kBlock / kWave];
     __shared__ uint32_t s_bid, s_exclusive;
@@ -198,18 +346,17 @@ __global__ void __launch_bounds__(kBlock)
     const uint32_t n_visible = counters[kCntVisible];
     const uint64_t first = (uint64_t)bid * kExpandTile + (uint64_t)tid * kExpandItems;
     if ((uint64_t)bid * kExpandTile >= n_visible) return;
+    for (uint32_t t = tid; t <= n_tiles; t += kBlock) s_bin_start[t] = bin_start_global[t];
+    const uint32_t* bin_start = s_bin_start;  // visible after the barrier of the block scan below
 
-    uint32_t point[kExpandItems], info[kExpandItems];
+    uint32_t val[kExpandItems];
+    bool valid[kExpandItems];
     uint32_t mine = 0;
 #pragma unroll
     for (int j = 0; j < kExpandItems; ++j) {
-        point[j] = 0u;
-        info[j] = 0u;
-        if (first + j < n_visible) {
-            point[j] = depth_order[first + j];
-            info[j] = __float_as_uint(rec[point[j]].w);
-        }
-        mine += info_count(info[j]);
+        valid[j] = first + j < n_visible;
+        val[j] = valid[j] ? depth_order[first + j] : 0u;
+        if (valid[j]) mine += ((val[j] & 1u) + 1u) * (((val[j] >> 1) & 1u) + 1u);
     }
     // block exclusive scan of `mine`
     uint32_t incl = mine;
@@ -227,18 +374,22 @@ __global__ void __launch_bounds__(kBlock)
         if ((uint32_t)w < wave) wave_off += c;
         block_total += c;
     }
-    if (tid == 0) s_exclusive = lookback_exclusive(status, 1u, bid, block_total, &counters[kCntError]);
+    if (wave == 0) {
+        const uint32_t exclusive = lookback_exclusive_wave(status, bid, block_total, &counters[kCntError]);
+        if (lane == 0) s_exclusive = exclusive;
+    }
     __syncthreads();
     uint32_t offset = s_exclusive + wave_off + incl - mine;
 #pragma unroll
     for (int j = 0; j < kExpandItems; ++j) {
-        if (!(info[j] & kInfoValid)) continue;
-        const uint32_t tile0 = info_tile0(info[j]), nx = info_nx(info[j]), ny = info_ny(info[j]);
+        if (!valid[j]) continue;
+        const uint32_t slot = val[j] >> 2, nx = (val[j] & 1u) + 1u, ny = ((val[j] >> 1) & 1u) + 1u;
+        const uint32_t tile0 = tile_of_slot(bin_start, n_tiles, slot);
         for (uint32_t dy = 0; dy < ny; ++dy)
             for (uint32_t dx = 0; dx < nx; ++dx) {
                 const uint32_t tile = tile0 + dy * gw + dx;
                 inst_keys[offset] = (uint16_t)tile;
-                inst_points[offset] = point[j];
+                inst_points[offset] = slot;
                 radix::hist_add(s_hist, plan, tile);
                 ++offset;
             }
@@ -268,20 +419,31 @@ __global__ void __launch_bounds__(kBlock) k_tile_ranges(const uint16_t* __restri
 }
 
 // ---- blend -------------------------------------------------------------------------------------------------
-constexpr int kBatch = 256;            // instances staged per round
-constexpr int kWords = kBatch / kWave; // 64-bit mask words per column / row
+//
+// One block per tile, one thread per pixel (a wave always covers an 8x8 pixel quad). Only the
+// transmittance of a pixel has to be evaluated in depth order; everything else is done one thread per
+// instance, all lanes busy. A batch of kBatch instances goes through these phases (barriers between them):
+//   stage      thread j gathers the record of instance j, evaluates the reference's exact coverage test
+//              |s - centre| < 1 for the two tile columns and rows it can reach and ORs bit j into the
+//              column / row masks of the batch;
+//   count      a pixel's hits are the set bits of (column mask AND row mask): popcount, block scan ->
+//              start of every pixel's fragment list;
+//   place      thread j writes the alpha of each of its (at most four) fragments into the list of the
+//              pixel it covers, at the rank given by the popcount of that pixel's mask below bit j, so the
+//              list is in depth order;
+//   pixels     a pixel walks its contiguous list: blending weight = T * alpha, T *= 1 - alpha, early out;
+//              the weights replace the alphas in the list (this is the only sequential part);
+//   instances  thread j reads the weights of its fragments back and writes the point's result: a plain
+//              store when the point lies in one tile only, atomics when it straddles tiles.
+constexpr int kBatch = 256;             // instances staged per round
+constexpr int kWords = kBatch / kWave;  // 64-bit mask words per column / row
+constexpr int kFragments = kBatch * 4;  // an instance covers at most 2 x 2 pixels
 
-template <int FMODE, int C>
-__device__ __forceinline__ void load_features(float* dst, const void* __restrict__ features,
-                                              const float4* __restrict__ features_view, uint32_t point) {
-    if (FMODE == INPC_FEAT_SH36_F16 || FMODE == INPC_FEAT_RAW37_F16) {
-        const float4 f = features_view[point];
-        dst[0] = f.x;
-        dst[1] = f.y;
-        dst[2] = f.z;
-        dst[3] = f.w;
-    } else if (FMODE == INPC_FEAT_DIRECT_F32) {
-        const float4* src = (const float4*)features + (size_t)point * (C / 4);
+// View features of a record (they follow the 32-byte header), as C floats.
+template <int C, bool HALF>
+__device__ __forceinline__ void load_record_features(float* dst, const char* __restrict__ record) {
+    if (!HALF) {
+        const float4* src = (const float4*)(record + kRecordHeader);
 #pragma unroll
         for (int q = 0; q < C / 4; ++q) {
             const float4 f = src[q];
@@ -291,9 +453,16 @@ __device__ __forceinline__ void load_features(float* dst, const void* __restrict
             dst[4 * q + 3] = f.w;
         }
     } else {
-        const __half* src = (const __half*)features + (size_t)point * C;
+        const uint2* src = (const uint2*)(record + kRecordHeader);
 #pragma unroll
-        for (int c = 0; c < C; ++c) dst[c] = __half2float(src[c]);
+        for (int q = 0; q < C / 4; ++q) {
+            const uint2 v = src[q];
+            const __half2 lo = *reinterpret_cast<const __half2*>(&v.x), hi = *reinterpret_cast<const __half2*>(&v.y);
+            dst[4 * q] = __low2float(lo);
+            dst[4 * q + 1] = __high2float(lo);
+            dst[4 * q + 2] = __low2float(hi);
+            dst[4 * q + 3] = __high2float(hi);
+        }
     }
 }
 
@@ -309,82 +478,117 @@ __device__ __forceinline__ void pixel_of_thread(uint32_t tid, int& lx, int& ly) 
     }
 }
 
-// Stage one batch: records and features into LDS, then the column / row coverage masks.
-template <int T, int C, int FMODE, bool NEED_DEPTH>
-__device__ __forceinline__ void stage_batch(uint32_t begin, uint32_t count, const uint32_t* __restrict__ inst_points,
-                                            const float4* __restrict__ rec, const void* __restrict__ features,
-                                            const float4* __restrict__ features_view,
-                                            const float* __restrict__ depth, int tile_x0, int tile_y0,
-                                            uint32_t* s_point, float2* s_xy, float* s_opacity, uint32_t* s_multi,
-                                            float* s_feat, float* s_depth, uint64_t (*s_col)[kWords],
-                                            uint64_t (*s_row)[kWords]) {
-    constexpr int TT = T * T;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u;
-    for (uint32_t j = tid; j < (uint32_t)kBatch; j += TT) {
-        float sx = 0.0f, sy = 0.0f;
-        const bool valid = j < count;
-        if (valid) {
-            const uint32_t p = inst_points[begin + j];
-            const float4 r = rec[p];
-            sx = r.x;
-            sy = r.y;
-            s_point[j] = p;
-            s_xy[j] = make_float2(sx, sy);
-            s_opacity[j] = r.z;
-            const uint32_t info = __float_as_uint(r.w);
-            s_multi[j] = (info >> 16) & 3u;
-            float f[C];
-            load_features<FMODE, C>(f, features, features_view, p);
+// Tile-local index of the last pixel whose centre is not right of (not below) coordinate s, clamped so
+// that the conversion is safe for any float. Only this pixel and the next one can be closer than 1 to s.
+template <int T>
+__device__ __forceinline__ int left_pixel(float s, int tile_origin) {
+    return (int)fminf(fmaxf(floorf(s - 0.5f) - (float)tile_origin, -4.0f), (float)(T + 4));
+}
+
+// The two candidate pixels of one axis: which of them lie in the tile and pass the float test of
+// B/rasterization/src/bilinear/kernels.cu:284-285, and their interpolation weights (kernels.cu:286-287).
+struct AxisCover {
+    int first;      // tile-local index of candidate 0
+    bool hit[2];
+    float weight[2];
+};
+
+template <int T>
+__device__ __forceinline__ AxisCover cover_axis(float s, int tile_origin) {
+    AxisCover a;
+    a.first = left_pixel<T>(s, tile_origin);
 #pragma unroll
-            for (int c = 0; c < C; ++c) s_feat[j * C + c] = f[c];
-            if (NEED_DEPTH) s_depth[j] = depth[p];
-        }
-        // j / 64 is uniform over the wave: one mask word per ballot
-        const uint32_t word = j >> 6;
-        uint64_t mine = 0;
+    for (int k = 0; k < 2; ++k) {
+        const int c = a.first + k;
+        const float d = fabsf(s - ((float)(tile_origin + c) + 0.5f));
+        a.hit[k] = c >= 0 && c < T && !(d >= 1.0f);
+        a.weight[k] = __saturatef(1.0f - d);
+    }
+    return a;
+}
+
+template <int T>
+struct BatchMasks {
+    uint64_t col[T][kWords];
+    uint64_t row[T][kWords];
+};
+
+template <int T>
+__device__ __forceinline__ void clear_masks(BatchMasks<T>& m) {
+    for (uint32_t i = threadIdx.x; i < (uint32_t)(2 * T * kWords); i += T * T) (&m.col[0][0])[i] = 0ull;
+}
+
+template <int T>
+__device__ __forceinline__ void mark_coverage(BatchMasks<T>& m, uint32_t j, const AxisCover& ax, const AxisCover& ay) {
+    const uint32_t bit = 1u << (j & 31u), half = j >> 5;
 #pragma unroll
-        for (int x = 0; x < T; ++x) {
-            const float d = fabsf(sx - ((float)(tile_x0 + x) + 0.5f));
-            const uint64_t m = __ballot(valid && !(d >= 1.0f));
-            if (lane == (uint32_t)x) mine = m;
-        }
-#pragma unroll
-        for (int y = 0; y < T; ++y) {
-            const float d = fabsf(sy - ((float)(tile_y0 + y) + 0.5f));
-            const uint64_t m = __ballot(valid && !(d >= 1.0f));
-            if (lane == (uint32_t)(32 + y)) mine = m;
-        }
-        if (lane < (uint32_t)T) s_col[lane][word] = mine;
-        if (lane >= 32u && lane < (uint32_t)(32 + T)) s_row[lane - 32u][word] = mine;
+    for (int k = 0; k < 2; ++k) {
+        if (ax.hit[k]) atomicOr((uint32_t*)&m.col[ax.first + k][0] + half, bit);
+        if (ay.hit[k]) atomicOr((uint32_t*)&m.row[ay.first + k][0] + half, bit);
     }
 }
 
-template <int T, int C, int FMODE, bool INFERENCE>
-__global__ void __launch_bounds__(T* T)
-    k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_points,
-                    const float4* __restrict__ rec, const void* __restrict__ features,
-                    const float4* __restrict__ features_view, const float* __restrict__ depth,
-                    float* __restrict__ image, float* __restrict__ alpha_image, float* blending_weights,
-                    float* __restrict__ depth_image, int W, int H, uint32_t gw) {
-    constexpr int TT = T * T;
-    __shared__ uint32_t s_point[kBatch];
-    __shared__ float2 s_xy[kBatch];
-    __shared__ float s_opacity[kBatch];
-    __shared__ uint32_t s_multi[kBatch];
-    __shared__ float s_feat[kBatch * C];
-    __shared__ float s_depth[INFERENCE ? kBatch : 1];
-    __shared__ float s_acc[INFERENCE ? 1 : kBatch];
-    __shared__ uint64_t s_col[T][kWords];
-    __shared__ uint64_t s_row[T][kWords];
+// Number of hits of pixel (cx, cy) among the instances 0 .. j-1 of the batch. `word` = j / 64 must be
+// uniform over the wave and `lane` = j % 64.
+template <int T>
+__device__ __forceinline__ uint32_t hits_before(const BatchMasks<T>& m, int cx, int cy, uint32_t word) {
+    uint32_t rank = 0;
+    for (uint32_t w = 0; w < word; ++w) rank += (uint32_t)__popcll(m.col[cx][w] & m.row[cy][w]);
+    const uint64_t own = m.col[cx][word] & m.row[cy][word];
+    return rank + mask_rank(own);
+}
 
-    const uint32_t tid = threadIdx.x;
+template <int T>
+__device__ __forceinline__ uint32_t hits_total(const BatchMasks<T>& m, int cx, int cy, uint32_t n_words) {
+    uint32_t n = 0;
+    for (uint32_t w = 0; w < n_words; ++w) n += (uint32_t)__popcll(m.col[cx][w] & m.row[cy][w]);
+    return n;
+}
+
+// Exclusive scan of one value per thread over the block (threads in tid order).
+template <int TT>
+__device__ __forceinline__ uint32_t block_scan_exclusive(uint32_t v, uint32_t* s_wave_total) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(incl, d, 64);
+        if (lane >= (uint32_t)d) incl += up;
+    }
+    if (TT == 64) return incl - v;
+    if (lane == 63) s_wave_total[wave] = incl;
+    __syncthreads();
+    uint32_t base = 0;
+#pragma unroll
+    for (int w = 0; w < TT / 64; ++w)
+        if ((uint32_t)w < wave) base += s_wave_total[w];
+    return base + incl - v;
+}
+
+template <int T, int C, bool HALF, bool INFERENCE>
+__global__ void __launch_bounds__(T* T)
+    k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_slots,
+                    const char* __restrict__ records, uint32_t stride, float* __restrict__ image,
+                    float* __restrict__ alpha_image, float* blending_weights, float* __restrict__ depth_image, int W,
+                    int H, uint32_t gw) {
+    constexpr int TT = T * T;
+    constexpr int NI = kBatch / TT;  // instances per thread and batch
+    __shared__ BatchMasks<T> s_masks;
+    __shared__ uint16_t s_start[TT], s_count[TT];      // fragment list of every pixel
+    __shared__ float s_alpha[kFragments];              // alpha, then blending weight, per fragment in list order
+    __shared__ uint16_t s_instance[kFragments];        // batch index of the fragment's instance
+    __shared__ float4 s_feat[kBatch * (C / 4)];
+    __shared__ float s_depth[INFERENCE ? kBatch : 1];
+    __shared__ uint32_t s_wave_total[TT / 64];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t tile = blockIdx.x;
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     int lx, ly;
     pixel_of_thread<T>(tid, lx, ly);
+    const int lp = ly * T + lx;
     const int px = tile_x0 + lx, py = tile_y0 + ly;
     const bool inside = px < W && py < H;
-    const float pcx = (float)px + 0.5f, pcy = (float)py + 0.5f;
 
     float F[C];
 #pragma unroll
@@ -395,45 +599,115 @@ __global__ void __launch_bounds__(T* T)
     const uint2 range = ranges[tile];
     for (uint32_t begin = range.x; begin < range.y; begin += kBatch) {
         const uint32_t count = min((uint32_t)kBatch, range.y - begin);
-        if (!INFERENCE)
-            for (uint32_t j = tid; j < (uint32_t)kBatch; j += TT) s_acc[j] = 0.0f;
-        stage_batch<T, C, FMODE, INFERENCE>(begin, count, inst_points, rec, features, features_view, depth, tile_x0,
-                                            tile_y0, s_point, s_xy, s_opacity, s_multi, s_feat, s_depth, s_col, s_row);
+        const uint32_t n_words = (count + 63u) >> 6;
+        clear_masks<T>(s_masks);
         __syncthreads();
-        if (!done) {
-            const uint32_t n_words = (count + 63u) >> 6;
-            for (uint32_t w = 0; w < n_words && !done; ++w) {
-                uint64_t m = s_col[lx][w] & s_row[ly][w];
-                while (m) {
-                    const uint32_t j = (w << 6) + (uint32_t)__builtin_ctzll(m);
-                    m &= m - 1;
-                    const float2 xy = s_xy[j];
-                    const float dx = fabsf(xy.x - pcx), dy = fabsf(xy.y - pcy);
-                    const float wgt = __saturatef(1.0f - dx) * __saturatef(1.0f - dy);
-                    const float a = s_opacity[j] * wgt;
-                    const float bw = Tr * a;
-                    if (!INFERENCE) {
-                        if (bw > 0.0f) atomicAdd(&s_acc[j], bw * wgt);
-                    }
+        // ---- stage
+        float sx[NI], sy[NI], opacity[NI];
+        uint32_t point[NI];
+        bool multi[NI];
 #pragma unroll
-                    for (int c = 0; c < C; ++c) F[c] = fmaf(bw, s_feat[j * C + c], F[c]);
-                    if (INFERENCE) D = fmaf(bw, s_depth[j], D);
-                    Tr *= 1.0f - a;
-                    if (Tr < kTransmittanceThreshold) {
-                        done = true;
-                        break;
+        for (int k = 0; k < NI; ++k) {
+            const uint32_t j = tid + k * TT;
+            sx[k] = sy[k] = opacity[k] = 0.0f;
+            point[k] = 0u;
+            multi[k] = false;
+            if (j < count) {
+                const char* record = records + (size_t)inst_slots[begin + j] * stride;
+                const float4 h0 = ((const float4*)record)[0];
+                const float4 h1 = ((const float4*)record)[1];
+                sx[k] = h0.x;
+                sy[k] = h0.y;
+                opacity[k] = h0.z;
+                point[k] = __float_as_uint(h0.w);
+                multi[k] = ((__float_as_uint(h1.x) >> 16) & 3u) != 0u;
+                float f[C];
+                load_record_features<C, HALF>(f, record);
+#pragma unroll
+                for (int q = 0; q < C / 4; ++q) s_feat[j * (C / 4) + q] = make_float4(f[4 * q], f[4 * q + 1], f[4 * q + 2], f[4 * q + 3]);
+                if (INFERENCE) s_depth[j] = h1.y;
+                mark_coverage<T>(s_masks, j, cover_axis<T>(h0.x, tile_x0), cover_axis<T>(h0.y, tile_y0));
+            }
+        }
+        __syncthreads();
+        // ---- count: fragment list of every live pixel
+        const uint32_t my_count = done ? 0u : hits_total<T>(s_masks, lx, ly, n_words);
+        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total);
+        s_start[lp] = (uint16_t)my_start;
+        s_count[lp] = (uint16_t)my_count;
+        __syncthreads();
+        // ---- place: alpha of every fragment into its pixel's list, in depth order
+        uint32_t where[NI][4];
+        float weight[NI][4];
+#pragma unroll
+        for (int k = 0; k < NI; ++k) {
+            const uint32_t j = tid + k * TT;
+            const AxisCover ax = cover_axis<T>(sx[k], tile_x0), ay = cover_axis<T>(sy[k], tile_y0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                where[k][q] = 0xFFFFFFFFu;
+                weight[k][q] = ax.weight[q & 1] * ay.weight[q >> 1];
+                if (j < count && ax.hit[q & 1] && ay.hit[q >> 1]) {
+                    const int cx = ax.first + (q & 1), cy = ay.first + (q >> 1);
+                    const int pix = cy * T + cx;
+                    if (s_count[pix] != 0) {  // 0: the pixel is finished (it has this hit at least)
+                        const uint32_t pos = s_start[pix] + hits_before<T>(s_masks, cx, cy, j >> 6);
+                        where[k][q] = pos;
+                        s_alpha[pos] = opacity[k] * weight[k][q];
+                        s_instance[pos] = (uint16_t)j;
                     }
                 }
             }
         }
         __syncthreads();
-        if (!INFERENCE) {
-            for (uint32_t j = tid; j < count; j += TT) {
-                const float v = s_acc[j];
-                if (v != 0.0f) {
-                    if (s_multi[j]) atomicAdd(&blending_weights[s_point[j]], v);
-                    else blending_weights[s_point[j]] = v;
+        // ---- pixels: the sequential part
+        if (my_count != 0u) {
+            uint32_t f = my_start;
+            const uint32_t end = my_start + my_count;
+            for (; f < end; ++f) {
+                const float a = s_alpha[f];
+                const uint32_t j = s_instance[f];
+                const float bw = Tr * a;
+                s_alpha[f] = bw;
+#pragma unroll
+                for (int q4 = 0; q4 < C / 4; ++q4) {
+                    const float4 v = s_feat[j * (C / 4) + q4];
+                    F[4 * q4] = fmaf(bw, v.x, F[4 * q4]);
+                    F[4 * q4 + 1] = fmaf(bw, v.y, F[4 * q4 + 1]);
+                    F[4 * q4 + 2] = fmaf(bw, v.z, F[4 * q4 + 2]);
+                    F[4 * q4 + 3] = fmaf(bw, v.w, F[4 * q4 + 3]);
                 }
+                if (INFERENCE) D = fmaf(bw, s_depth[j], D);
+                Tr *= 1.0f - a;
+                if (Tr < kTransmittanceThreshold) {
+                    done = true;
+                    ++f;
+                    break;
+                }
+            }
+            for (; f < end; ++f) s_alpha[f] = 0.0f;  // fragments behind the early out contribute nothing
+        }
+        __syncthreads();
+        // ---- instances: blending weights of the points (B/rasterization/src/bilinear/kernels.cu:291-295)
+        if (!INFERENCE) {
+#pragma unroll
+            for (int k = 0; k < NI; ++k) {
+                const uint32_t j = tid + k * TT;
+                if (j >= count) continue;
+                float weight_sum = 0.0f;
+                bool any = false;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (where[k][q] == 0xFFFFFFFFu) continue;
+                    const float bw = s_alpha[where[k][q]];
+                    if (bw > 0.0f) {
+                        weight_sum = fmaf(bw, weight[k][q], weight_sum);
+                        any = true;
+                    }
+                }
+                if (!any) continue;
+                if (multi[k]) atomicAdd(&blending_weights[point[k]], weight_sum);
+                else blending_weights[point[k]] = weight_sum;
             }
         }
         if (__syncthreads_and(done)) break;
@@ -446,135 +720,201 @@ __global__ void __launch_bounds__(T* T)
         alpha_image[pix] = Tr < kTransmittanceThreshold ? 1.0f : alpha_px;
         if (INFERENCE) depth_image[pix] = alpha_px > 0.0f ? D / alpha_px : 0.0f;
     }
+    (void)lane;
 }
 
-template <int T, int C, int FMODE>
+// Backward. With s = features . grad of a fragment, R the running sum of weight x s of a pixel and S its
+// final value image . grad, the opacity gradient of the reference (kernels.cu:405-413),
+//   dot(T f + (F_running - F_final) / (1 - a), grad) + grad_alpha (1 - alpha_final) / (1 - a),
+// is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the pixel loop carries two scalars, not 2C.
+template <int T, int C, bool HALF>
 __global__ void __launch_bounds__(T* T)
-    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_points,
-                     const float4* __restrict__ rec, const void* __restrict__ features,
-                     const float4* __restrict__ features_view, const float* __restrict__ grad_image,
+    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_slots,
+                     const char* __restrict__ records, uint32_t stride, const float* __restrict__ grad_image,
                      const float* __restrict__ grad_alpha, const float* __restrict__ image,
                      const float* __restrict__ alpha_image, float* grad_view, float* grad_opacities, int W, int H,
                      uint32_t gw) {
     constexpr int TT = T * T;
-    __shared__ uint32_t s_point[kBatch];
-    __shared__ float2 s_xy[kBatch];
-    __shared__ float s_opacity[kBatch];
-    __shared__ uint32_t s_multi[kBatch];
-    __shared__ float s_feat[kBatch * C];
-    __shared__ float s_gfeat[kBatch * C];
-    __shared__ float s_gop[kBatch];
-    __shared__ uint64_t s_col[T][kWords];
-    __shared__ uint64_t s_row[T][kWords];
+    constexpr int NI = kBatch / TT;
+    __shared__ BatchMasks<T> s_masks;
+    __shared__ uint16_t s_start[TT], s_count[TT];
+    __shared__ float s_alpha[kFragments];   // alpha, then blending weight
+    __shared__ float s_dot[kFragments];     // features . grad, then d(loss)/d(alpha)
+    __shared__ float s_grad[C * TT];        // channel-major upstream gradient of the tile (0 outside the image)
+    __shared__ uint32_t s_wave_total[TT / 64];
 
     const uint32_t tid = threadIdx.x;
     const uint32_t tile = blockIdx.x;
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     int lx, ly;
     pixel_of_thread<T>(tid, lx, ly);
+    const int lp = ly * T + lx;
     const int px = tile_x0 + lx, py = tile_y0 + ly;
     const bool inside = px < W && py < H;
-    const float pcx = (float)px + 0.5f, pcy = (float)py + 0.5f;
 
-    float G[C], Ffin[C], Fnew[C];
-    float common = 0.0f;
-#pragma unroll
-    for (int c = 0; c < C; ++c) {
-        G[c] = 0.0f;
-        Ffin[c] = 0.0f;
-        Fnew[c] = 0.0f;
-    }
-    if (inside) {
+    float final_dot = 0.0f, common = 0.0f;
+    {
         const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            G[c] = grad_image[c * n_pixels + pix];
-            Ffin[c] = image[c * n_pixels + pix];
+            const float g = inside ? grad_image[c * n_pixels + pix] : 0.0f;
+            s_grad[c * TT + lp] = g;
+            if (inside) final_dot = fmaf(image[c * n_pixels + pix], g, final_dot);
         }
-        common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
+        if (inside) common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
     }
-    float Tr = 1.0f;
+    const float offset = common - final_dot;
+    float Tr = 1.0f, running = 0.0f;
     bool done = !inside;
 
     const uint2 range = ranges[tile];
     for (uint32_t begin = range.x; begin < range.y; begin += kBatch) {
         const uint32_t count = min((uint32_t)kBatch, range.y - begin);
-        for (uint32_t j = tid; j < (uint32_t)kBatch; j += TT) s_gop[j] = 0.0f;
-        for (uint32_t j = tid; j < (uint32_t)(kBatch * C); j += TT) s_gfeat[j] = 0.0f;
-        stage_batch<T, C, FMODE, false>(begin, count, inst_points, rec, features, features_view, nullptr, tile_x0,
-                                        tile_y0, s_point, s_xy, s_opacity, s_multi, s_feat, nullptr, s_col, s_row);
-        __syncthreads();
-        if (!done) {
-            const uint32_t n_words = (count + 63u) >> 6;
-            for (uint32_t w = 0; w < n_words && !done; ++w) {
-                uint64_t m = s_col[lx][w] & s_row[ly][w];
-                while (m) {
-                    const uint32_t j = (w << 6) + (uint32_t)__builtin_ctzll(m);
-                    m &= m - 1;
-                    const float2 xy = s_xy[j];
-                    const float dx = fabsf(xy.x - pcx), dy = fabsf(xy.y - pcy);
-                    const float wgt = __saturatef(1.0f - dx) * __saturatef(1.0f - dy);
-                    const float a = s_opacity[j] * wgt;
-                    const float bw = Tr * a;
-                    const float one_minus_a = 1.0f - a;
-                    const float rcp = 1.0f / fmaxf(one_minus_a, kOneMinusAlphaEps);
-                    float dot = 0.0f;
+        const uint32_t n_words = (count + 63u) >> 6;
+        clear_masks<T>(s_masks);
+        __syncthreads();  // also orders s_grad before its first use
+        // ---- stage
+        float sx[NI], sy[NI], opacity[NI];
+        float feat[NI][C];
+        uint32_t point[NI];
+        bool multi[NI];
 #pragma unroll
-                    for (int c = 0; c < C; ++c) {
-                        const float f = s_feat[j * C + c];
-                        if (bw > 0.0f) atomicAdd(&s_gfeat[j * C + c], bw * G[c]);
-                        Fnew[c] = fmaf(bw, f, Fnew[c]);
-                        dot = fmaf(fmaf(Tr, f, (Fnew[c] - Ffin[c]) * rcp), G[c], dot);
-                    }
-                    const float d_alpha = fmaf(common, rcp, dot);
-                    const float d_op = d_alpha * wgt;
-                    if (d_op != 0.0f) atomicAdd(&s_gop[j], d_op);
-                    Tr *= one_minus_a;
-                    if (Tr < kTransmittanceThreshold) {
-                        done = true;
-                        break;
+        for (int k = 0; k < NI; ++k) {
+            const uint32_t j = tid + k * TT;
+            sx[k] = sy[k] = opacity[k] = 0.0f;
+            point[k] = 0u;
+            multi[k] = false;
+            if (j < count) {
+                const char* record = records + (size_t)inst_slots[begin + j] * stride;
+                const float4 h0 = ((const float4*)record)[0];
+                const float4 h1 = ((const float4*)record)[1];
+                sx[k] = h0.x;
+                sy[k] = h0.y;
+                opacity[k] = h0.z;
+                point[k] = __float_as_uint(h0.w);
+                multi[k] = ((__float_as_uint(h1.x) >> 16) & 3u) != 0u;
+                load_record_features<C, HALF>(feat[k], record);
+                mark_coverage<T>(s_masks, j, cover_axis<T>(h0.x, tile_x0), cover_axis<T>(h0.y, tile_y0));
+            }
+        }
+        __syncthreads();
+        // ---- count
+        const uint32_t my_count = done ? 0u : hits_total<T>(s_masks, lx, ly, n_words);
+        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total);
+        s_start[lp] = (uint16_t)my_start;
+        s_count[lp] = (uint16_t)my_count;
+        __syncthreads();
+        // ---- place: alpha and features . grad of every fragment
+        uint32_t where[NI][4];
+        float weight[NI][4];
+#pragma unroll
+        for (int k = 0; k < NI; ++k) {
+            const uint32_t j = tid + k * TT;
+            const AxisCover ax = cover_axis<T>(sx[k], tile_x0), ay = cover_axis<T>(sy[k], tile_y0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                where[k][q] = 0xFFFFFFFFu;
+                weight[k][q] = ax.weight[q & 1] * ay.weight[q >> 1];
+                if (j < count && ax.hit[q & 1] && ay.hit[q >> 1]) {
+                    const int cx = ax.first + (q & 1), cy = ay.first + (q >> 1);
+                    const int pix = cy * T + cx;
+                    if (s_count[pix] != 0) {
+                        const uint32_t pos = s_start[pix] + hits_before<T>(s_masks, cx, cy, j >> 6);
+                        where[k][q] = pos;
+                        s_alpha[pos] = opacity[k] * weight[k][q];
+                        float d = 0.0f;
+#pragma unroll
+                        for (int c = 0; c < C; ++c) d = fmaf(feat[k][c], s_grad[c * TT + pix], d);
+                        s_dot[pos] = d;
                     }
                 }
             }
         }
         __syncthreads();
-        for (uint32_t e = tid; e < count * C; e += TT) {
-            const uint32_t j = e / C, c = e % C;
-            const float v = s_gfeat[e];
-            if (v != 0.0f) {
-                float* dst = grad_view + (size_t)s_point[j] * C + c;
-                if (s_multi[j]) atomicAdd(dst, v);
-                else *dst = v;
+        // ---- pixels: the sequential part
+        if (my_count != 0u) {
+            uint32_t f = my_start;
+            const uint32_t end = my_start + my_count;
+            for (; f < end; ++f) {
+                const float a = s_alpha[f], s = s_dot[f];
+                const float bw = Tr * a;
+                const float one_minus_a = 1.0f - a;
+                const float rcp = __frcp_rn(fmaxf(one_minus_a, kOneMinusAlphaEps));
+                running = fmaf(bw, s, running);
+                s_alpha[f] = bw;
+                s_dot[f] = fmaf(Tr, s, (running + offset) * rcp);
+                Tr *= one_minus_a;
+                if (Tr < kTransmittanceThreshold) {
+                    done = true;
+                    ++f;
+                    break;
+                }
+            }
+            for (; f < end; ++f) {
+                s_alpha[f] = 0.0f;
+                s_dot[f] = 0.0f;
             }
         }
-        for (uint32_t j = tid; j < count; j += TT) {
-            const float v = s_gop[j];
-            if (v != 0.0f) {
-                if (s_multi[j]) atomicAdd(&grad_opacities[s_point[j]], v);
-                else grad_opacities[s_point[j]] = v;
+        __syncthreads();
+        // ---- instances: gradient of the point
+#pragma unroll
+        for (int k = 0; k < NI; ++k) {
+            const uint32_t j = tid + k * TT;
+            if (j >= count) continue;
+            const AxisCover ax = cover_axis<T>(sx[k], tile_x0), ay = cover_axis<T>(sy[k], tile_y0);
+            float gf[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) gf[c] = 0.0f;
+            float gop = 0.0f;
+            bool any_weight = false;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (where[k][q] == 0xFFFFFFFFu) continue;
+                const float bw = s_alpha[where[k][q]];
+                gop = fmaf(s_dot[where[k][q]], weight[k][q], gop);
+                if (bw > 0.0f) {
+                    any_weight = true;
+                    const int pix = (ay.first + (q >> 1)) * T + ax.first + (q & 1);
+#pragma unroll
+                    for (int c = 0; c < C; ++c) gf[c] = fmaf(bw, s_grad[c * TT + pix], gf[c]);
+                }
+            }
+            if (!any_weight && gop == 0.0f) continue;
+            float* dst = grad_view + (size_t)point[k] * C;
+            if (multi[k]) {
+                if (any_weight) {
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                        if (gf[c] != 0.0f) atomicAdd(dst + c, gf[c]);
+                }
+                if (gop != 0.0f) atomicAdd(&grad_opacities[point[k]], gop);
+            } else {
+#pragma unroll
+                for (int q4 = 0; q4 < C / 4; ++q4)
+                    ((float4*)dst)[q4] = make_float4(gf[4 * q4], gf[4 * q4 + 1], gf[4 * q4 + 2], gf[4 * q4 + 3]);
+                grad_opacities[point[k]] = gop;
             }
         }
         if (__syncthreads_and(done)) break;
     }
 }
 
-// view-space feature gradient -> (N,36) fp16, zero where the point was not drawn
+// view-space feature gradient -> (N,36) fp16; a point that was not drawn has a zero view gradient and
+// gets zeros (kernels.cu:95)
 __global__ void __launch_bounds__(kBlock)
     k_sh_backward(const float* __restrict__ positions, const float* __restrict__ cam_position,
-                  const float4* __restrict__ rec, const float4* __restrict__ grad_view, __half* __restrict__ grad_features,
-                  uint32_t n) {
+                  const float4* __restrict__ grad_view, __half* __restrict__ grad_features, uint32_t n) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     __half* out = grad_features + 36 * (size_t)i;
-    const uint32_t info = __float_as_uint(rec[i].w);
-    if (!(info & kInfoValid)) {
+    const float4 g = grad_view[i];
+    if (g.x == 0.0f && g.y == 0.0f && g.z == 0.0f && g.w == 0.0f) {
 #pragma unroll
         for (int k = 0; k < 36; ++k) out[k] = __float2half_rn(0.0f);
         return;
     }
     const ShBasis s = sh_basis(positions[3 * (size_t)i], positions[3 * (size_t)i + 1], positions[3 * (size_t)i + 2],
                                cam_position);
-    const float4 g = grad_view[i];
 #pragma unroll
     for (int k = 0; k < 9; ++k) {
         out[4 * k + 0] = __float2half_rn(s.b[k] * g.x);
@@ -596,11 +936,12 @@ struct Layout {
     Geometry geo;
     radix::PassPlan depth_plan, tile_plan;
     int T, C, fmode;
-    bool inference, sh;
+    bool inference, sh, half_features;
     // private offsets
     size_t zero_begin, zero_words;  // region cleared at the start of every forward
     size_t hist_depth, hist_tile, bases_depth, bases_tile;
     size_t status_depth, status_tile, status_expand;
+    size_t bin_table, bin_total;
     size_t keys_a, keys_b, vals_a, vals_b;
     size_t inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
 };
@@ -619,8 +960,9 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     if (cfg->n_points >= (1u << 28)) return fail(INPC_E_UNSUPPORTED, "raster: n_points must be below 2^28");
     L.T = cfg->tile;
     L.fmode = cfg->feature_mode;
-    L.sh = L.fmode == INPC_FEAT_SH36_F16 || L.fmode == INPC_FEAT_RAW37_F16;
     if (L.fmode < 0 || L.fmode > 3) return fail(INPC_E_UNSUPPORTED, "raster: unknown feature mode %d", L.fmode);
+    L.sh = L.fmode == INPC_FEAT_SH36_F16 || L.fmode == INPC_FEAT_RAW37_F16;
+    L.half_features = L.fmode == INPC_FEAT_DIRECT_F16;
     L.C = L.sh ? 4 : cfg->channels;
     if (L.C != 4 && L.C != 8 && L.C != 16) return fail(INPC_E_INVALID_ARGUMENT, "raster: channels must be 4, 8 or 16");
     L.inference = (cfg->flags & INPC_RASTER_INFERENCE) != 0;
@@ -633,7 +975,11 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     g.n_tiles = g.gw * g.gh;
     if (g.n_tiles > 65536u)
         return fail(INPC_E_UNSUPPORTED, "raster: %u tiles exceed the 16-bit tile key (65536)", g.n_tiles);
+    if (g.n_tiles > kMaxLdsTiles)
+        return fail(INPC_E_UNSUPPORTED, "raster: %u tiles exceed the %u this build keeps counters for", g.n_tiles,
+                    kMaxLdsTiles);
     g.cam = to_device_camera(cam);
+    g.stride = record_stride(L.C, L.half_features);
     // depth keys of drawn points lie in [bits(near), bits(far)] when 0 < near <= far: sort on the offset
     int depth_bits = 32;
     g.key_bias = 0u;
@@ -654,7 +1000,7 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     };
     inpc_raster_layout& P = L.pub;
     memset(&P, 0, sizeof(P));
-    // zeroed region: counters, histograms, look-back status, tile ranges
+    // zeroed region: counters, histograms, look-back status, bin counts, tile ranges
     L.zero_begin = off;
     P.counters = take(kCntWords * 4);
     L.hist_depth = take(radix::kMaxPasses * radix::kRadix * 4);
@@ -664,11 +1010,12 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.status_expand = take((size_t)div_up(g.n, kExpandTile) * 4 + 4);
     P.tile_ranges = take((size_t)g.n_tiles * 8);
     L.zero_words = (off - L.zero_begin) / 4;
+    L.bin_table = take((size_t)kBinBlocks * g.n_tiles * 4);
+    L.bin_total = take((size_t)g.n_tiles * 4);
+    P.bin_start = take((size_t)(g.n_tiles + 1) * 4);
     L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
     L.bases_tile = take(radix::kMaxPasses * radix::kRadix * 4);
-    P.point_record = take(n * 16);
-    P.point_depth = take(n * 4);
-    P.features_view = L.sh ? take(n * 16) : 0;
+    P.point_record = take(n * g.stride);
     L.keys_a = take(n * 4);
     L.keys_b = take(n * 4);
     L.vals_a = take(n * 4);
@@ -682,8 +1029,9 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     P.depth_order = depth_in_a ? L.vals_a : L.vals_b;
     const bool tile_in_a = (L.tile_plan.n_passes % 2) == 0;
     P.instance_keys = tile_in_a ? L.inst_keys_a : L.inst_keys_b;
-    P.instance_points = tile_in_a ? L.inst_vals_a : L.inst_vals_b;
+    P.instance_slots = tile_in_a ? L.inst_vals_a : L.inst_vals_b;
     P.total_bytes = off;
+    P.record_stride = g.stride;
     P.grid_width = g.gw;
     P.grid_height = g.gh;
     P.n_tiles = g.n_tiles;
@@ -697,116 +1045,129 @@ Tp* at(void* ws, size_t off) {
     return (Tp*)((char*)ws + off);
 }
 
-template <int T, int FMODE>
+// Launch with `lds_bytes` of dynamic LDS; above 64 KiB the kernel has to be told once.
+#define INPC_LAUNCH_LDS(name, kernel, grid, block, lds_bytes, stream, ...)                                   \
+    do {                                                                                                     \
+        if ((lds_bytes) > 48 * 1024) {                                                                       \
+            hipError_t _a = hipFuncSetAttribute(reinterpret_cast<const void*>(&kernel),                      \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(lds_bytes)); \
+            if (_a != hipSuccess)                                                                            \
+                return fail(INPC_E_HIP, "%s: cannot reserve %zu bytes of LDS: %s", name, (size_t)(lds_bytes), \
+                            hipGetErrorString(_a));                                                          \
+        }                                                                                                    \
+        ::inpc::timing_begin(name, stream);                                                                  \
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, __VA_ARGS__);                             \
+        ::inpc::timing_end(stream);                                                                          \
+        hipError_t _e = hipGetLastError();                                                                   \
+        if (_e != hipSuccess) return fail(INPC_E_HIP, "launch of %s failed: %s", name, hipGetErrorString(_e)); \
+    } while (0)
+
+template <int T>
+int launch_bin_count(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
+    const size_t lds = (size_t)L.geo.n_tiles * 4;
+    INPC_LAUNCH_LDS("raster_bin_count", (k_bin_count<T>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream, positions,
+                    w2c, at<uint32_t>(ws, L.bin_table), L.geo);
+    return INPC_OK;
+}
+
+template <int T, int FMODE, int C>
 int launch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
                       const float* w2c, const float* cam_position, float* blending_weights, void* ws,
                       hipStream_t stream) {
-    const uint32_t blocks = std::min<uint32_t>(div_up(L.geo.n, kBlock), 2048u);
-    INPC_LAUNCH("raster_preprocess", (k_preprocess<T, FMODE>), dim3(blocks), dim3(kBlock), stream, positions, features,
-                opacities, w2c, cam_position, at<float4>(ws, L.pub.point_record), at<float>(ws, L.pub.point_depth),
-                L.sh ? at<float4>(ws, L.pub.features_view) : (float4*)nullptr, at<uint32_t>(ws, L.keys_a),
-                blending_weights, at<uint32_t>(ws, L.pub.counters), at<uint32_t>(ws, L.hist_depth), L.geo,
-                radix::to_device_plan(L.depth_plan));
+    const size_t lds = ((size_t)L.geo.n_tiles + radix::kMaxPasses * radix::kRadix) * 4;
+    INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream,
+                    positions, features, opacities, w2c, cam_position, at<char>(ws, L.pub.point_record),
+                    (const uint32_t*)at<uint32_t>(ws, L.bin_table), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
+                    at<uint32_t>(ws, L.keys_a), at<uint32_t>(ws, L.vals_a), blending_weights,
+                    at<uint32_t>(ws, L.pub.counters), at<uint32_t>(ws, L.hist_depth), L.geo,
+                    radix::to_device_plan(L.depth_plan));
     return INPC_OK;
 }
 
-template <int T, int C, int FMODE>
-int launch_blend_forward(const Layout& L, const void* features, float* image, float* alpha, float* blending_weights,
-                         float* depth_image, void* ws, hipStream_t stream) {
+template <int T, int C, bool HALF>
+int launch_blend_forward(const Layout& L, float* image, float* alpha, float* blending_weights, float* depth_image,
+                         void* ws, hipStream_t stream) {
     const uint2* ranges = at<uint2>(ws, L.pub.tile_ranges);
-    const uint32_t* inst = at<uint32_t>(ws, L.pub.instance_points);
-    const float4* rec = at<float4>(ws, L.pub.point_record);
-    const float4* fview = L.sh ? at<float4>(ws, L.pub.features_view) : (const float4*)nullptr;
-    const float* depth = at<float>(ws, L.pub.point_depth);
+    const uint32_t* inst = at<uint32_t>(ws, L.pub.instance_slots);
+    const char* records = at<char>(ws, L.pub.point_record);
     if (L.inference) {
-        INPC_LAUNCH("raster_blend_inference", (k_blend_forward<T, C, FMODE, true>), dim3(L.geo.n_tiles), dim3(T * T),
-                    stream, ranges, inst, rec, features, fview, depth, image, alpha, (float*)nullptr, depth_image,
-                    L.geo.W, L.geo.H, L.geo.gw);
+        INPC_LAUNCH("raster_blend_inference", (k_blend_forward<T, C, HALF, true>), dim3(L.geo.n_tiles), dim3(T * T),
+                    stream, ranges, inst, records, L.geo.stride, image, alpha, (float*)nullptr, depth_image, L.geo.W,
+                    L.geo.H, L.geo.gw);
     } else {
-        INPC_LAUNCH("raster_blend_forward", (k_blend_forward<T, C, FMODE, false>), dim3(L.geo.n_tiles), dim3(T * T),
-                    stream, ranges, inst, rec, features, fview, depth, image, alpha, blending_weights,
-                    (float*)nullptr, L.geo.W, L.geo.H, L.geo.gw);
+        INPC_LAUNCH("raster_blend_forward", (k_blend_forward<T, C, HALF, false>), dim3(L.geo.n_tiles), dim3(T * T),
+                    stream, ranges, inst, records, L.geo.stride, image, alpha, blending_weights, (float*)nullptr,
+                    L.geo.W, L.geo.H, L.geo.gw);
     }
     return INPC_OK;
 }
 
-template <int T, int C, int FMODE>
-int launch_blend_backward(const Layout& L, const void* features, const float* grad_image, const float* grad_alpha,
-                          const float* image, const float* alpha, float* grad_view, float* grad_opacities, void* ws,
-                          hipStream_t stream) {
-    INPC_LAUNCH("raster_blend_backward", (k_blend_backward<T, C, FMODE>), dim3(L.geo.n_tiles), dim3(T * T), stream,
-                at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.pub.instance_points),
-                at<float4>(ws, L.pub.point_record), features,
-                L.sh ? at<float4>(ws, L.pub.features_view) : (const float4*)nullptr, grad_image, grad_alpha, image,
-                alpha, grad_view, grad_opacities, L.geo.W, L.geo.H, L.geo.gw);
+template <int T, int C, bool HALF>
+int launch_blend_backward(const Layout& L, const float* grad_image, const float* grad_alpha, const float* image,
+                          const float* alpha, float* grad_view, float* grad_opacities, void* ws, hipStream_t stream) {
+    INPC_LAUNCH("raster_blend_backward", (k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
+                at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.pub.instance_slots),
+                at<char>(ws, L.pub.point_record), L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view,
+                grad_opacities, L.geo.W, L.geo.H, L.geo.gw);
     return INPC_OK;
 }
 
-// dispatch on (tile, channels, feature mode)
-#define INPC_DISPATCH_TC(FM, CALL)                                        \
-    do {                                                                  \
-        if (L.T == 8 && L.C == 4) return CALL(8, 4, FM);                  \
-        if (L.T == 8 && L.C == 8) return CALL(8, 8, FM);                  \
-        if (L.T == 8 && L.C == 16) return CALL(8, 16, FM);                \
-        if (L.T == 16 && L.C == 4) return CALL(16, 4, FM);                \
-        if (L.T == 16 && L.C == 8) return CALL(16, 8, FM);                \
-        if (L.T == 16 && L.C == 16) return CALL(16, 16, FM);              \
+// dispatch on (tile, channels, storage)
+#define INPC_DISPATCH_TCH(CALL)                                                   \
+    do {                                                                          \
+        const bool h = L.half_features;                                           \
+        if (L.T == 8 && L.C == 4) return h ? CALL(8, 4, true) : CALL(8, 4, false);       \
+        if (L.T == 8 && L.C == 8) return h ? CALL(8, 8, true) : CALL(8, 8, false);       \
+        if (L.T == 8 && L.C == 16) return h ? CALL(8, 16, true) : CALL(8, 16, false);    \
+        if (L.T == 16 && L.C == 4) return h ? CALL(16, 4, true) : CALL(16, 4, false);    \
+        if (L.T == 16 && L.C == 8) return h ? CALL(16, 8, true) : CALL(16, 8, false);    \
+        if (L.T == 16 && L.C == 16) return h ? CALL(16, 16, true) : CALL(16, 16, false); \
     } while (0)
 
-int dispatch_blend_forward(const Layout& L, const void* features, float* image, float* alpha, float* bw,
-                           float* depth_image, void* ws, hipStream_t stream) {
-#define CALL_FWD(T_, C_, FM_) launch_blend_forward<T_, C_, FM_>(L, features, image, alpha, bw, depth_image, ws, stream)
-    switch (L.fmode) {
-        case INPC_FEAT_SH36_F16:
-            if (L.T == 8) return CALL_FWD(8, 4, INPC_FEAT_SH36_F16);
-            return CALL_FWD(16, 4, INPC_FEAT_SH36_F16);
-        case INPC_FEAT_RAW37_F16:
-            if (L.T == 8) return CALL_FWD(8, 4, INPC_FEAT_RAW37_F16);
-            return CALL_FWD(16, 4, INPC_FEAT_RAW37_F16);
-        case INPC_FEAT_DIRECT_F32:
-            INPC_DISPATCH_TC(INPC_FEAT_DIRECT_F32, CALL_FWD);
-            break;
-        case INPC_FEAT_DIRECT_F16:
-            INPC_DISPATCH_TC(INPC_FEAT_DIRECT_F16, CALL_FWD);
-            break;
-    }
+int dispatch_blend_forward(const Layout& L, float* image, float* alpha, float* bw, float* depth_image, void* ws,
+                           hipStream_t stream) {
+#define CALL_FWD(T_, C_, H_) launch_blend_forward<T_, C_, H_>(L, image, alpha, bw, depth_image, ws, stream)
+    INPC_DISPATCH_TCH(CALL_FWD);
 #undef CALL_FWD
     return fail(INPC_E_UNSUPPORTED, "raster: unsupported blend configuration");
 }
 
-int dispatch_blend_backward(const Layout& L, const void* features, const float* grad_image, const float* grad_alpha,
-                            const float* image, const float* alpha, float* grad_view, float* grad_opacities, void* ws,
-                            hipStream_t stream) {
-#define CALL_BWD(T_, C_, FM_) \
-    launch_blend_backward<T_, C_, FM_>(L, features, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, ws, stream)
-    switch (L.fmode) {
-        case INPC_FEAT_SH36_F16:
-            if (L.T == 8) return CALL_BWD(8, 4, INPC_FEAT_SH36_F16);
-            return CALL_BWD(16, 4, INPC_FEAT_SH36_F16);
-        case INPC_FEAT_DIRECT_F32:
-            INPC_DISPATCH_TC(INPC_FEAT_DIRECT_F32, CALL_BWD);
-            break;
-        case INPC_FEAT_DIRECT_F16:
-            INPC_DISPATCH_TC(INPC_FEAT_DIRECT_F16, CALL_BWD);
-            break;
-    }
+int dispatch_blend_backward(const Layout& L, const float* grad_image, const float* grad_alpha, const float* image,
+                            const float* alpha, float* grad_view, float* grad_opacities, void* ws, hipStream_t stream) {
+#define CALL_BWD(T_, C_, H_) \
+    launch_blend_backward<T_, C_, H_>(L, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, ws, stream)
+    INPC_DISPATCH_TCH(CALL_BWD);
 #undef CALL_BWD
     return fail(INPC_E_UNSUPPORTED, "raster: unsupported backward configuration");
 }
 
 int dispatch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
                         const float* w2c, const float* cam_position, float* bw, void* ws, hipStream_t stream) {
-#define CALL_PRE(T_, FM_) launch_preprocess<T_, FM_>(L, positions, features, opacities, w2c, cam_position, bw, ws, stream)
+#define CALL_PRE(T_, FM_, C_) \
+    launch_preprocess<T_, FM_, C_>(L, positions, features, opacities, w2c, cam_position, bw, ws, stream)
+#define CALL_PRE_C(T_, FM_)                    \
+    do {                                       \
+        if (L.C == 4) return CALL_PRE(T_, FM_, 4);   \
+        if (L.C == 8) return CALL_PRE(T_, FM_, 8);   \
+        if (L.C == 16) return CALL_PRE(T_, FM_, 16); \
+    } while (0)
     switch (L.fmode) {
         case INPC_FEAT_SH36_F16:
-            return L.T == 8 ? CALL_PRE(8, INPC_FEAT_SH36_F16) : CALL_PRE(16, INPC_FEAT_SH36_F16);
+            return L.T == 8 ? CALL_PRE(8, INPC_FEAT_SH36_F16, 4) : CALL_PRE(16, INPC_FEAT_SH36_F16, 4);
         case INPC_FEAT_RAW37_F16:
-            return L.T == 8 ? CALL_PRE(8, INPC_FEAT_RAW37_F16) : CALL_PRE(16, INPC_FEAT_RAW37_F16);
-        default:
-            // the direct modes do not touch the features here
-            return L.T == 8 ? CALL_PRE(8, INPC_FEAT_DIRECT_F32) : CALL_PRE(16, INPC_FEAT_DIRECT_F32);
+            return L.T == 8 ? CALL_PRE(8, INPC_FEAT_RAW37_F16, 4) : CALL_PRE(16, INPC_FEAT_RAW37_F16, 4);
+        case INPC_FEAT_DIRECT_F32:
+            if (L.T == 8) CALL_PRE_C(8, INPC_FEAT_DIRECT_F32);
+            else CALL_PRE_C(16, INPC_FEAT_DIRECT_F32);
+            break;
+        case INPC_FEAT_DIRECT_F16:
+            if (L.T == 8) CALL_PRE_C(8, INPC_FEAT_DIRECT_F16);
+            else CALL_PRE_C(16, INPC_FEAT_DIRECT_F16);
+            break;
     }
+#undef CALL_PRE_C
 #undef CALL_PRE
+    return fail(INPC_E_UNSUPPORTED, "raster: unsupported preprocess configuration");
 }
 
 }  // namespace
@@ -846,27 +1207,36 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: blending weights are null");
     if (L.fmode == INPC_FEAT_DIRECT_F32 && ((uintptr_t)features & 15u) != 0)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: fp32 features must be 16-byte aligned");
+    if (L.fmode == INPC_FEAT_DIRECT_F16 && ((uintptr_t)features & 7u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: fp16 features must be 8-byte aligned");
 
     rc = fill_u32(at<uint32_t>(ws, L.zero_begin), 0u, L.zero_words, stream);
     if (rc != INPC_OK) return rc;
     uint32_t* counters = at<uint32_t>(ws, L.pub.counters);
     if (L.geo.n > 0) {
+        rc = L.T == 8 ? launch_bin_count<8>(L, positions, w2c, ws, stream) : launch_bin_count<16>(L, positions, w2c, ws, stream);
+        if (rc != INPC_OK) return rc;
+        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets, dim3(div_up(L.geo.n_tiles, kBlock)), dim3(kBlock), stream,
+                    at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
+        INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
+                    (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start), L.geo.n_tiles);
         rc = dispatch_preprocess(L, positions, features, opacities, w2c, cam_position,
                                  L.inference ? nullptr : blending_weights, ws, stream);
         if (rc != INPC_OK) return rc;
-        rc = radix::sort_pairs<uint32_t>(L.depth_plan, true, at<uint32_t>(ws, L.keys_a), at<uint32_t>(ws, L.vals_a),
-                                         at<uint32_t>(ws, L.keys_b), at<uint32_t>(ws, L.vals_b),
-                                         counters + kCntVisible, L.geo.n, at<uint32_t>(ws, L.hist_depth),
-                                         at<uint32_t>(ws, L.bases_depth), at<uint32_t>(ws, L.status_depth),
-                                         counters + kCntTicketDepth, counters + kCntError, stream, "raster_depth_sort");
+        rc = radix::sort_pairs<uint32_t>(L.depth_plan, radix::kSkipInvalid, at<uint32_t>(ws, L.keys_a),
+                                         at<uint32_t>(ws, L.vals_a), at<uint32_t>(ws, L.keys_b),
+                                         at<uint32_t>(ws, L.vals_b), counters + kCntVisible, L.geo.n,
+                                         at<uint32_t>(ws, L.hist_depth), at<uint32_t>(ws, L.bases_depth),
+                                         at<uint32_t>(ws, L.status_depth), counters + kCntTicketDepth,
+                                         counters + kCntError, stream, "raster_depth_sort");
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("raster_expand", k_expand, dim3(div_up(L.geo.n, kExpandTile)), dim3(kBlock), stream,
-                    (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order), (const float4*)at<float4>(ws, L.pub.point_record),
+        INPC_LAUNCH_LDS("raster_expand", k_expand, dim3(div_up(L.geo.n, kExpandTile)), dim3(kBlock),
+                    ((size_t)L.geo.n_tiles + 1) * 4, stream, (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
                     at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), counters,
-                    at<uint32_t>(ws, L.status_expand), at<uint32_t>(ws, L.hist_tile), L.geo.gw,
+                    at<uint32_t>(ws, L.status_expand), at<uint32_t>(ws, L.hist_tile), L.geo.gw, L.geo.n_tiles,
                     radix::to_device_plan(L.tile_plan));
         const uint32_t ni = 4u * L.geo.n;
-        rc = radix::sort_pairs<uint16_t>(L.tile_plan, false, at<uint16_t>(ws, L.inst_keys_a),
+        rc = radix::sort_pairs<uint16_t>(L.tile_plan, radix::kPlain, at<uint16_t>(ws, L.inst_keys_a),
                                          at<uint32_t>(ws, L.inst_vals_a), at<uint16_t>(ws, L.inst_keys_b),
                                          at<uint32_t>(ws, L.inst_vals_b), counters + kCntInstances, ni,
                                          at<uint32_t>(ws, L.hist_tile), at<uint32_t>(ws, L.bases_tile),
@@ -877,15 +1247,14 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                     dim3(kBlock), stream, (const uint16_t*)at<uint16_t>(ws, L.pub.instance_keys),
                     at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)counters, ni);
     }
-    return dispatch_blend_forward(L, features, image, alpha, blending_weights, depth_image, ws, stream);
+    return dispatch_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }
 
 int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image, const float* grad_alpha,
-                         const float* image, const float* alpha, const float* positions, const void* features,
-                         const float* opacities, const float* cam_position, void* grad_features,
-                         float* grad_opacities, float* grad_view_scratch, void* ws, size_t ws_bytes, void* stream_) {
+                         const float* image, const float* alpha, const float* positions, const float* cam_position,
+                         void* grad_features, float* grad_opacities, float* grad_view_scratch, void* ws,
+                         size_t ws_bytes, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
-    (void)opacities;
     Layout L;
     int rc = make_layout(cfg, L);
     if (rc != INPC_OK) return rc;
@@ -893,23 +1262,24 @@ int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
         return fail(INPC_E_UNSUPPORTED, "inpc_raster_backward: inference configurations have no backward pass");
     if (!ws || ws_bytes < L.pub.total_bytes) return fail(INPC_E_WORKSPACE, "inpc_raster_backward: workspace too small");
     if (L.geo.n == 0) return INPC_OK;
-    if (!grad_image || !grad_alpha || !image || !alpha || !positions || !grad_features || !grad_opacities)
+    if (!grad_image || !grad_alpha || !image || !alpha || !grad_features || !grad_opacities)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: null pointer");
-    if (!L.sh && !features) return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: features are null");
     const bool direct32 = L.fmode == INPC_FEAT_DIRECT_F32;
     float* grad_view = direct32 ? (float*)grad_features : grad_view_scratch;
     if (!grad_view) return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: this feature mode needs grad_view_scratch");
-    if (L.sh && !cam_position) return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: cam_position is null");
+    if (((uintptr_t)grad_view & 15u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: the fp32 gradient buffer must be 16-byte aligned");
+    if (L.sh && (!cam_position || !positions))
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: positions / cam_position are null");
     rc = fill_u32(grad_view, 0u, (size_t)L.geo.n * L.C, stream);
     if (rc != INPC_OK) return rc;
     rc = fill_u32(grad_opacities, 0u, L.geo.n, stream);
     if (rc != INPC_OK) return rc;
-    rc = dispatch_blend_backward(L, features, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, ws, stream);
+    rc = dispatch_blend_backward(L, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, ws, stream);
     if (rc != INPC_OK) return rc;
     if (L.fmode == INPC_FEAT_SH36_F16) {
         INPC_LAUNCH("raster_sh_backward", k_sh_backward, dim3(div_up(L.geo.n, kBlock)), dim3(kBlock), stream, positions,
-                    cam_position, (const float4*)at<float4>(ws, L.pub.point_record), (const float4*)grad_view,
-                    (__half*)grad_features, L.geo.n);
+                    cam_position, (const float4*)grad_view, (__half*)grad_features, L.geo.n);
     } else if (L.fmode == INPC_FEAT_DIRECT_F16) {
         const size_t total = (size_t)L.geo.n * L.C;
         INPC_LAUNCH("raster_grad_to_half", k_float_to_half, dim3((uint32_t)std::min<size_t>((total + 255) / 256, 8192)),

@@ -276,16 +276,22 @@ __global__ void __launch_bounds__(kBlock)
         if (lane == 0) s_count[j * (kBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
     }
     __syncthreads();
-    if (tid == 0) {
-        uint32_t run = 0;
-        for (int e = 0; e < kSampleItems * (kBlock / kWave); ++e) {
-            const uint32_t c = s_count[e];
-            s_count[e] = run;
-            run += c;
+    if (wave == 0) {
+        // exclusive scan of the 32 (round, wave) counts by the first lanes, then the block-level look-back
+        uint32_t c = lane < (uint32_t)(kSampleItems * (kBlock / kWave)) ? s_count[lane] : 0u;
+        uint32_t incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (lane >= (uint32_t)d) incl += up;
         }
-        const uint32_t exclusive = lookback_exclusive(status, 1u, bid, run, &st->error);
-        s_exclusive = exclusive;
-        if (bid == n_blocks - 1) st->accepted = s_accepted0 + exclusive + run;
+        if (lane < (uint32_t)(kSampleItems * (kBlock / kWave))) s_count[lane] = incl - c;
+        const uint32_t run = __shfl(incl, 63, 64);
+        const uint32_t exclusive = lookback_exclusive_wave(status, bid, run, &st->error);
+        if (lane == 0) {
+            s_exclusive = exclusive;
+            if (bid == n_blocks - 1) st->accepted = s_accepted0 + exclusive + run;
+        }
     }
     __syncthreads();
     const uint64_t base = (uint64_t)s_accepted0 + s_exclusive;
@@ -400,7 +406,10 @@ __global__ void __launch_bounds__(kBlock)
     }
     uint32_t total;
     const uint32_t local = block_exclusive_scan(mine, s_wave, total);
-    if (threadIdx.x == 0) s_exclusive = lookback_exclusive(status, 1u, bid, total, &st->error);
+    if (threadIdx.x < 64) {
+        const uint32_t exclusive = lookback_exclusive_wave(status, bid, total, &st->error);
+        if (threadIdx.x == 0) s_exclusive = exclusive;
+    }
     __syncthreads();
     uint32_t run = s_exclusive + local;
 #pragma unroll

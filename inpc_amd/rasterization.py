@@ -132,7 +132,8 @@ class _Rasterize(torch.autograd.Function):
         positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)
         image, alpha, blending_weights, workspace, cfg = _forward_native(
             rasterizer_settings, positions, features, opacities, tile, channels, feature_mode, inference=False)
-        ctx.save_for_backward(image, alpha, positions, features, opacities, workspace)
+        ctx.save_for_backward(image, alpha, positions, workspace)
+        ctx.features_shape, ctx.opacities_shape = features.shape, opacities.shape
         ctx.rasterizer_settings = rasterizer_settings
         ctx.cfg = cfg
         ctx.mark_non_differentiable(blending_weights)
@@ -142,7 +143,7 @@ class _Rasterize(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx: Any, grad_image: Optional[torch.Tensor], grad_alpha: Optional[torch.Tensor], _):
-        image, alpha, positions, features, opacities, workspace = ctx.saved_tensors
+        image, alpha, positions, workspace = ctx.saved_tensors
         cfg = ctx.cfg
         settings = ctx.rasterizer_settings
         n = positions.shape[0]
@@ -166,12 +167,12 @@ class _Rasterize(torch.autograd.Function):
         cam_position = settings.cam_position.contiguous()
         _lib.check(_lib.lib().inpc_raster_backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha),
                                                    _lib.ptr(image), _lib.ptr(alpha), _lib.ptr(positions),
-                                                   _lib.ptr(features), _lib.ptr(opacities), _lib.ptr(cam_position),
-                                                   _lib.ptr(grad_features), _lib.ptr(grad_opacities),
+                                                   _lib.ptr(cam_position), _lib.ptr(grad_features),
+                                                   _lib.ptr(grad_opacities),
                                                    _lib.ptr(scratch), _lib.ptr(workspace), workspace.numel(),
                                                    _lib.current_stream()), "inpc_raster_backward")
-        grad_features = grad_features.view(features.shape)
-        grad_opacities = grad_opacities.view(opacities.shape)
+        grad_features = grad_features.view(ctx.features_shape)
+        grad_opacities = grad_opacities.view(ctx.opacities_shape)
         return None, grad_features, grad_opacities, None, None, None, None
 
 

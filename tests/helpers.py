@@ -159,34 +159,52 @@ class RasterRun:
         return self.ws[offset:offset + nbytes].cpu().numpy().view(dtype)
 
     def debug(self):
-        """Intermediate buffers decoded into the oracle's shapes."""
+        """Intermediate buffers decoded into the oracle's shapes (record slots mapped back to point ids)."""
         L, n = self.layout, self.n
         v, i = self.counters()
-        rec = self._buf(L.point_record, 4 * n, np.float32).reshape(n, 4)
-        info = rec[:, 3].copy().view(np.uint32)
-        valid = (info >> 18) & 1
+        stride = L.record_stride
+        raw = self._buf(L.point_record, v * stride, np.uint8).reshape(v, stride)
+        head = raw[:, :32].copy().view(np.float32).reshape(v, 8)
+        head_u = head.view(np.uint32)
+        orig = head_u[:, 3].astype(np.int64)          # point id of every record slot
+        info = head_u[:, 4]
+        assert len(np.unique(orig)) == v, "two records name the same point"
+        assert ((info >> 18) & 1).all(), "a record of a point that is not drawn"
         tile0 = info & 0xFFFF
         nx = ((info >> 16) & 1) + 1
         ny = ((info >> 17) & 1) + 1
+        bin_start = self._buf(L.bin_start, L.n_tiles + 1, np.uint32)
+        assert bin_start[0] == 0 and bin_start[-1] == v and (np.diff(bin_start.astype(np.int64)) >= 0).all()
+        # every record lies in the bin of its first tile
+        slot_tile = np.searchsorted(bin_start, np.arange(v), side="right") - 1
+        assert (slot_tile == tile0).all(), "a record outside the bin of its first tile"
         x0, y0 = tile0 % L.grid_width, tile0 // L.grid_width
-        bounds = np.stack([x0, x0 + nx, y0, y0 + ny], axis=1).astype(np.uint16)
-        bounds[valid == 0] = 0
-        out = {
-            "n_visible": v, "n_instances": i,
-            "n_touched": np.where(valid == 1, nx * ny, 0).astype(np.uint32),
-            "bounds": bounds,
-            "screen_xy": np.where(valid[:, None] == 1, rec[:, :2], 0).astype(np.float32),
-            "opacity": np.where(valid == 1, rec[:, 2], 0).astype(np.float32),
-            "depth": self._buf(L.point_depth, n, np.float32),
+        n_touched = np.zeros(n, np.uint32)
+        bounds = np.zeros((n, 4), np.uint16)
+        xy = np.zeros((n, 2), np.float32)
+        opacity = np.zeros(n, np.float32)
+        depth = np.zeros(n, np.float32)
+        n_touched[orig] = nx * ny
+        bounds[orig] = np.stack([x0, x0 + nx, y0, y0 + ny], axis=1)
+        xy[orig] = head[:, :2]
+        opacity[orig] = head[:, 2]
+        depth[orig] = head[:, 5]
+        order_vals = self._buf(L.depth_order, n, np.uint32)[:v]
+        span = order_vals & 3
+        assert (span == ((info >> 16) & 3)[order_vals >> 2]).all(), "span bits of the sort value differ from the record"
+        feat_dtype = np.float16 if self.cfg.feature_mode == _lib.FEAT_DIRECT_F16 else np.float32
+        feats = raw[:, 32:32 + self.C * np.dtype(feat_dtype).itemsize].copy().view(feat_dtype).reshape(v, self.C)
+        features_view = np.zeros((n, self.C), np.float32)
+        features_view[orig] = feats.astype(np.float32)
+        return {
+            "n_visible": v, "n_instances": i, "n_touched": n_touched, "bounds": bounds, "screen_xy": xy,
+            "opacity": opacity, "depth": depth, "features_view": features_view,
             "depth_keys": (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32),
-            "depth_order": self._buf(L.depth_order, n, np.uint32)[:v],
+            "depth_order": orig[order_vals >> 2].astype(np.uint32),
             "instance_keys": self._buf(L.instance_keys, 4 * n, np.uint16)[:i],
-            "instance_points": self._buf(L.instance_points, 4 * n, np.uint32)[:i],
+            "instance_points": orig[self._buf(L.instance_slots, 4 * n, np.uint32)[:i]].astype(np.uint32),
             "tile_ranges": self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2),
         }
-        if L.features_view:
-            out["features_view"] = self._buf(L.features_view, 4 * n, np.float32).reshape(n, 4)
-        return out
 
     def outputs(self):
         out = {"image": self.image.cpu().numpy(), "alpha": self.alpha.cpu().numpy()}
@@ -213,8 +231,8 @@ class RasterRun:
         gi, ga = dev(np.asarray(grad_image, np.float32), device), dev(np.asarray(grad_alpha, np.float32), device)
         _lib.check(self.lib.inpc_raster_backward(
             C.byref(self.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(self.image), _lib.ptr(self.alpha),
-            _lib.ptr(self.positions), _lib.ptr(self.features), _lib.ptr(self.opacities), _lib.ptr(self.cam_position),
-            _lib.ptr(gf), _lib.ptr(go), _lib.ptr(scratch), _lib.ptr(self.ws), self.layout.total_bytes, stream()),
+            _lib.ptr(self.positions), _lib.ptr(self.cam_position), _lib.ptr(gf), _lib.ptr(go), _lib.ptr(scratch),
+            _lib.ptr(self.ws), self.layout.total_bytes, stream()),
             "inpc_raster_backward")
         return gf.cpu().numpy(), go.cpu().numpy()
 

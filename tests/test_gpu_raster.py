@@ -52,7 +52,9 @@ def test_forward_direct_f32(gpu, oracle, tile, channels):
     run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32).forward()
     ref = oracle.raster_forward(oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32), pos, feats, opac,
                                 hv.w2c, debug=True)
-    check_structure(run.debug(), ref)
+    dbg = run.debug()
+    check_structure(dbg, ref)
+    np.testing.assert_array_equal(dbg["features_view"], ref["features_view"])  # copied into the records as they are
     out = run.outputs()
     H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
     H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
