@@ -507,6 +507,10 @@ __device__ __forceinline__ AxisCover cover_axis(float s, int tile_origin) {
     return a;
 }
 
+__device__ __forceinline__ void lds_add(float* p, float v) {
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 template <int T>
 struct BatchMasks {
     uint64_t col[T][kWords];
@@ -545,9 +549,10 @@ __device__ __forceinline__ uint32_t hits_total(const BatchMasks<T>& m, int cx, i
     return n;
 }
 
-// Exclusive scan of one value per thread over the block (threads in tid order).
+// Exclusive scan of one value per thread over the block (threads in tid order); `total` gets the block sum.
+// Contains barriers: every thread of the block must call it.
 template <int TT>
-__device__ __forceinline__ uint32_t block_scan_exclusive(uint32_t v, uint32_t* s_wave_total) {
+__device__ __forceinline__ uint32_t block_scan_exclusive(uint32_t v, uint32_t* s_wave_total, uint32_t& total) {
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     uint32_t incl = v;
 #pragma unroll
@@ -555,15 +560,217 @@ __device__ __forceinline__ uint32_t block_scan_exclusive(uint32_t v, uint32_t* s
         const uint32_t up = __shfl_up(incl, d, 64);
         if (lane >= (uint32_t)d) incl += up;
     }
-    if (TT == 64) return incl - v;
+    if (TT == 64) {
+        total = __shfl(incl, 63, 64);
+        return incl - v;
+    }
+    __syncthreads();  // s_wave_total may still be read from the previous call
     if (lane == 63) s_wave_total[wave] = incl;
     __syncthreads();
-    uint32_t base = 0;
+    uint32_t base = 0, sum = 0;
 #pragma unroll
-    for (int w = 0; w < TT / 64; ++w)
-        if ((uint32_t)w < wave) base += s_wave_total[w];
+    for (int w = 0; w < TT / 64; ++w) {
+        const uint32_t c = s_wave_total[w];
+        if ((uint32_t)w < wave) base += c;
+        sum += c;
+    }
+    total = sum;
     return base + incl - v;
 }
+
+// ---- long fragment lists ---------------------------------------------------------------------------------------
+// A pixel-sized cluster of points puts a large share of a batch on a handful of pixels; walking such a list
+// on the one lane that owns the pixel would keep the whole block waiting. Lists longer than kLongList are
+// therefore evaluated over the flat, pixel-sorted fragment array by all threads: the running transmittance
+// (and, backward, the running weighted sum) is a segmented scan, the weighted feature sum a segmented
+// reduction. The scan multiplies in tree order, not front to back, so for these lists the transmittance can
+// differ from a sequential product in the last bits; short lists keep the sequential evaluation.
+constexpr uint32_t kLongList = 24;
+
+struct SegItem {
+    bool flag;   // a segment starts at or before the end of the span this item stands for
+    float value; // op-combination of the trailing run of the span
+};
+
+template <bool MUL>
+__device__ __forceinline__ float seg_identity() { return MUL ? 1.0f : 0.0f; }
+
+template <bool MUL>
+__device__ __forceinline__ float seg_apply(float a, float b) { return MUL ? a * b : a + b; }
+
+template <bool MUL>
+__device__ __forceinline__ SegItem seg_combine(const SegItem& left, const SegItem& right) {
+    SegItem r;
+    r.flag = left.flag || right.flag;
+    r.value = right.flag ? right.value : seg_apply<MUL>(left.value, right.value);
+    return r;
+}
+
+// Exclusive segmented scan of n elements, four consecutive elements per thread and round.
+//   get(f, flag, value): head flag and value of element f
+//   put(f, exclusive):   op-combination of the elements of f's segment before f (identity at a head)
+// Every thread of the block must call it; s_item has TT / 64 entries.
+template <int TT, bool MUL, typename Get, typename Put>
+__device__ __forceinline__ void segmented_scan(uint32_t n, SegItem* s_item, Get get, Put put) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    SegItem round_carry{false, seg_identity<MUL>()};
+    for (uint32_t round_base = 0; round_base < n; round_base += 4 * TT) {
+        const uint32_t base = round_base + 4 * threadIdx.x;
+        bool flag[4];
+        float value[4], before[4];
+        bool broken[4];
+        SegItem mine{false, seg_identity<MUL>()};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            flag[i] = true;
+            value[i] = seg_identity<MUL>();
+            if (base + i < n) get(base + i, flag[i], value[i]);
+            if (flag[i]) {
+                mine.flag = true;
+                mine.value = seg_identity<MUL>();
+            }
+            before[i] = mine.value;
+            broken[i] = mine.flag;
+            mine.value = seg_apply<MUL>(mine.value, value[i]);
+        }
+        // inclusive scan of the thread items over the wave
+        SegItem incl = mine;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            SegItem left;
+            left.flag = __shfl_up((int)incl.flag, d, 64) != 0;
+            left.value = __shfl_up(incl.value, d, 64);
+            if (lane >= (uint32_t)d) incl = seg_combine<MUL>(left, incl);
+        }
+        SegItem excl;
+        excl.flag = __shfl_up((int)incl.flag, 1, 64) != 0;
+        excl.value = __shfl_up(incl.value, 1, 64);
+        if (lane == 0) excl = SegItem{false, seg_identity<MUL>()};
+        if (TT > 64) {
+            __syncthreads();
+            if (lane == 63) s_item[wave] = incl;
+            __syncthreads();
+        }
+        SegItem incoming = round_carry;
+        if (TT > 64) {
+#pragma unroll
+            for (int w = 0; w < TT / 64; ++w)
+                if ((uint32_t)w < wave) incoming = seg_combine<MUL>(incoming, s_item[w]);
+        }
+        incoming = seg_combine<MUL>(incoming, excl);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (base + i < n) put(base + i, broken[i] ? before[i] : seg_apply<MUL>(incoming.value, before[i]));
+        // carry into the next round: everything up to the end of this round
+        if (TT > 64) {
+#pragma unroll
+            for (int w = 0; w < TT / 64; ++w) round_carry = seg_combine<MUL>(round_carry, s_item[w]);
+        } else {
+            SegItem last;
+            last.flag = __shfl((int)incl.flag, 63, 64) != 0;
+            last.value = __shfl(incl.value, 63, 64);
+            round_carry = seg_combine<MUL>(round_carry, last);
+        }
+    }
+}
+
+// Front-to-back walk over the fragment list [begin, end) of one pixel: alpha[f] is replaced by the blending
+// weight T * alpha, T is updated, and the walk stops behind the fragment that takes T below the threshold
+// (B/rasterization/src/bilinear/kernels.cu:289-299); fragments behind it get weight 0.
+// The alphas of eight fragments are fetched together so that the chain does not pay one LDS round trip each.
+__device__ __forceinline__ void transmittance_chain(float* alpha, uint32_t begin, uint32_t end, float& Tr, bool& done) {
+    constexpr int kAhead = 8;
+    for (uint32_t f = begin; f < end; f += kAhead) {
+        float a[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) a[i] = alpha[min(f + i, end - 1)];
+        // No branches in the chain: a fragment behind the end of the list or behind the early out gets
+        // alpha 0, which leaves T untouched and makes its blending weight 0.
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            const bool live = f + i < end && !done;
+            const float ai = live ? a[i] : 0.0f;
+            a[i] = Tr * ai;
+            Tr *= 1.0f - ai;
+            done = done || (live && Tr < kTransmittanceThreshold);
+        }
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i)
+            if (f + i < end) alpha[f + i] = a[i];
+    }
+}
+
+// A pixel-sized cluster of points puts a large share of a batch on a handful of pixels. Their weighted
+// feature sums are not left to the single lanes that own those pixels: every thread of the block takes four
+// consecutive fragments of the flat, pixel-sorted list, adds up the ones that belong to a long list, and
+// adds the partial sum to the pixel's accumulator in LDS (a few float atomics per thread).
+template <int TT, int C, bool WITH_DEPTH>
+__device__ __forceinline__ void sum_long_lists(const float* alpha, const uint16_t* instance, const uint8_t* pixel_of,
+                                               const uint16_t* count, const float4* feat, const float* depth,
+                                               uint32_t n_fragments, float* acc, float* dacc) {
+    for (uint32_t base = 4 * threadIdx.x; base < n_fragments; base += 4 * TT) {
+        float part[C];
+        float dpart = 0.0f;
+        int current = -1;
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            int pix = -1;
+            float bw = 0.0f;
+            uint32_t j = 0;
+            if (i < 4 && base + i < n_fragments) {
+                const int p = pixel_of[base + i];
+                bw = alpha[base + i];
+                j = instance[base + i];
+                if (count[p] > kLongList && bw != 0.0f) pix = p;
+            }
+            if (pix != current) {
+                if (current >= 0) {
+#pragma unroll
+                    for (int c = 0; c < C; ++c) lds_add(&acc[c * TT + current], part[c]);
+                    if (WITH_DEPTH) lds_add(&dacc[current], dpart);
+                }
+                current = pix;
+#pragma unroll
+                for (int c = 0; c < C; ++c) part[c] = 0.0f;
+                dpart = 0.0f;
+            }
+            if (pix >= 0) {
+#pragma unroll
+                for (int q4 = 0; q4 < C / 4; ++q4) {
+                    const float4 v = feat[j * (C / 4) + q4];
+                    part[4 * q4] = fmaf(bw, v.x, part[4 * q4]);
+                    part[4 * q4 + 1] = fmaf(bw, v.y, part[4 * q4 + 1]);
+                    part[4 * q4 + 2] = fmaf(bw, v.z, part[4 * q4 + 2]);
+                    part[4 * q4 + 3] = fmaf(bw, v.w, part[4 * q4 + 3]);
+                }
+                if (WITH_DEPTH) dpart = fmaf(bw, depth[j], dpart);
+            }
+        }
+    }
+}
+
+#ifdef INPC_BLEND_PROFILE
+// development aid: per-phase shader clocks of k_blend_forward, summed over blocks (thread 0 of each)
+__device__ unsigned long long g_blend_profile[8];
+#define INPC_PROF_DECL unsigned long long prof_t = clock64(), prof_acc[6] = {0, 0, 0, 0, 0, 0}, prof_batches = 0
+#define INPC_PROF_MARK(i)                          \
+    do {                                           \
+        const unsigned long long now_ = clock64(); \
+        prof_acc[i] += now_ - prof_t;              \
+        prof_t = now_;                             \
+    } while (0)
+#define INPC_PROF_FLUSH                                                         \
+    do {                                                                        \
+        if (threadIdx.x == 0) {                                                 \
+            for (int i_ = 0; i_ < 6; ++i_) atomicAdd(&g_blend_profile[i_], prof_acc[i_]); \
+            atomicAdd(&g_blend_profile[6], prof_batches);                       \
+        }                                                                       \
+    } while (0)
+#else
+#define INPC_PROF_DECL
+#define INPC_PROF_MARK(i)
+#define INPC_PROF_FLUSH
+#endif
 
 template <int T, int C, bool HALF, bool INFERENCE>
 __global__ void __launch_bounds__(T* T)
@@ -577,9 +784,14 @@ __global__ void __launch_bounds__(T* T)
     __shared__ uint16_t s_start[TT], s_count[TT];      // fragment list of every pixel
     __shared__ float s_alpha[kFragments];              // alpha, then blending weight, per fragment in list order
     __shared__ uint16_t s_instance[kFragments];        // batch index of the fragment's instance
+    __shared__ uint8_t s_pixel[kFragments];            // tile-local pixel of the fragment
     __shared__ float4 s_feat[kBatch * (C / 4)];
     __shared__ float s_depth[INFERENCE ? kBatch : 1];
-    __shared__ uint32_t s_wave_total[TT / 64];
+    __shared__ float s_acc[C * TT];                    // channel-major sums of the long lists
+    __shared__ float s_dacc[INFERENCE ? TT : 1];
+    __shared__ float s_t_in[TT], s_t_out[TT];          // transmittance of the pixels with long lists
+    __shared__ SegItem s_item[TT / 64];
+    __shared__ uint32_t s_wave_total[TT / 64 + 1];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t tile = blockIdx.x;
@@ -592,16 +804,22 @@ __global__ void __launch_bounds__(T* T)
 
     float F[C];
 #pragma unroll
-    for (int c = 0; c < C; ++c) F[c] = 0.0f;
+    for (int c = 0; c < C; ++c) {
+        F[c] = 0.0f;
+        s_acc[c * TT + lp] = 0.0f;
+    }
+    if (INFERENCE) s_dacc[lp] = 0.0f;
     float D = 0.0f, Tr = 1.0f;
     bool done = !inside;
 
     const uint2 range = ranges[tile];
+    INPC_PROF_DECL;
     for (uint32_t begin = range.x; begin < range.y; begin += kBatch) {
         const uint32_t count = min((uint32_t)kBatch, range.y - begin);
         const uint32_t n_words = (count + 63u) >> 6;
         clear_masks<T>(s_masks);
         __syncthreads();
+        INPC_PROF_MARK(0);
         // ---- stage
         float sx[NI], sy[NI], opacity[NI];
         uint32_t point[NI];
@@ -630,12 +848,31 @@ __global__ void __launch_bounds__(T* T)
             }
         }
         __syncthreads();
+        INPC_PROF_MARK(1);
         // ---- count: fragment list of every live pixel
         const uint32_t my_count = done ? 0u : hits_total<T>(s_masks, lx, ly, n_words);
-        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total);
+        uint32_t n_fragments;
+        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total, n_fragments);
+        if (n_fragments == 0u) {  // every instance of the batch falls on finished pixels only
+            if (__syncthreads_and(done)) break;
+            continue;
+        }
         s_start[lp] = (uint16_t)my_start;
         s_count[lp] = (uint16_t)my_count;
+        s_t_in[lp] = Tr;
+        const bool any_long = __syncthreads_or(my_count > kLongList) != 0;
+#ifdef INPC_BLEND_PROFILE
+        {
+            __shared__ uint32_t s_prof_max;
+            if (tid == 0) s_prof_max = 0u;
+            __syncthreads();
+            atomicMax(&s_prof_max, my_count);
+            __syncthreads();
+            if (tid == 0) atomicAdd(&g_blend_profile[7], (unsigned long long)n_fragments);
+        }
+#endif
         __syncthreads();
+        INPC_PROF_MARK(2);
         // ---- place: alpha of every fragment into its pixel's list, in depth order
         uint32_t where[NI][4];
         float weight[NI][4];
@@ -655,39 +892,84 @@ __global__ void __launch_bounds__(T* T)
                         where[k][q] = pos;
                         s_alpha[pos] = opacity[k] * weight[k][q];
                         s_instance[pos] = (uint16_t)j;
+                        s_pixel[pos] = (uint8_t)pix;
                     }
                 }
             }
         }
         __syncthreads();
-        // ---- pixels: the sequential part
-        if (my_count != 0u) {
-            uint32_t f = my_start;
-            const uint32_t end = my_start + my_count;
-            for (; f < end; ++f) {
-                const float a = s_alpha[f];
-                const uint32_t j = s_instance[f];
-                const float bw = Tr * a;
-                s_alpha[f] = bw;
+        INPC_PROF_MARK(3);
+        // ---- pixels: the sequential part touches the alphas only ...
+        const uint32_t end = my_start + my_count;
+        if (my_count != 0u && my_count <= kLongList) transmittance_chain(s_alpha, my_start, end, Tr, done);
+        if (any_long) {
+            // ... and for long lists it is a segmented product over the flat fragment array
+            segmented_scan<TT, true>(
+                n_fragments, s_item,
+                [&](uint32_t f, bool& flag, float& value) {
+                    const uint32_t p = s_pixel[f];
+                    const bool is_long = s_count[p] > kLongList;
+                    flag = !is_long || f == s_start[p];
+                    value = is_long ? 1.0f - s_alpha[f] : 1.0f;
+                },
+                [&](uint32_t f, float exclusive) {
+                    const uint32_t p = s_pixel[f];
+                    if (s_count[p] <= kLongList) return;
+                    const float a = s_alpha[f];
+                    const float t_before = s_t_in[p] * exclusive;
+                    const float t_after = t_before * (1.0f - a);
+                    const bool live = !(t_before < kTransmittanceThreshold);
+                    s_alpha[f] = live ? t_before * a : 0.0f;
+                    const bool last = f + 1 == (uint32_t)s_start[p] + s_count[p];
+                    // exactly one fragment hands the final transmittance back: the one that ends the walk
+                    if (live && (t_after < kTransmittanceThreshold || last)) s_t_out[p] = t_after;
+                });
+            __syncthreads();
+            if (my_count > kLongList) {
+                Tr = s_t_out[lp];
+                done = Tr < kTransmittanceThreshold;
+            }
+        }
+#ifdef INPC_BLEND_PROFILE
+        __syncthreads();
+        INPC_PROF_MARK(4);
+#endif
+        // ... the weighted feature sum has no dependence between its terms. A pixel with a short list sums
+        // it alone, four fragments per round with all loads of a round in flight together.
+        if (my_count <= kLongList) {
+            for (uint32_t f = my_start; f < end; f += 4) {
+                float bw[4];
+                uint32_t jj[4];
 #pragma unroll
-                for (int q4 = 0; q4 < C / 4; ++q4) {
-                    const float4 v = s_feat[j * (C / 4) + q4];
-                    F[4 * q4] = fmaf(bw, v.x, F[4 * q4]);
-                    F[4 * q4 + 1] = fmaf(bw, v.y, F[4 * q4 + 1]);
-                    F[4 * q4 + 2] = fmaf(bw, v.z, F[4 * q4 + 2]);
-                    F[4 * q4 + 3] = fmaf(bw, v.w, F[4 * q4 + 3]);
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t g = min(f + i, end - 1);
+                    bw[i] = f + i < end ? s_alpha[g] : 0.0f;
+                    jj[i] = s_instance[g];
                 }
-                if (INFERENCE) D = fmaf(bw, s_depth[j], D);
-                Tr *= 1.0f - a;
-                if (Tr < kTransmittanceThreshold) {
-                    done = true;
-                    ++f;
-                    break;
+                float4 v[4][C / 4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int q4 = 0; q4 < C / 4; ++q4) v[i][q4] = s_feat[jj[i] * (C / 4) + q4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                    for (int q4 = 0; q4 < C / 4; ++q4) {
+                        F[4 * q4] = fmaf(bw[i], v[i][q4].x, F[4 * q4]);
+                        F[4 * q4 + 1] = fmaf(bw[i], v[i][q4].y, F[4 * q4 + 1]);
+                        F[4 * q4 + 2] = fmaf(bw[i], v[i][q4].z, F[4 * q4 + 2]);
+                        F[4 * q4 + 3] = fmaf(bw[i], v[i][q4].w, F[4 * q4 + 3]);
+                    }
+                    if (INFERENCE) D = fmaf(bw[i], s_depth[jj[i]], D);
                 }
             }
-            for (; f < end; ++f) s_alpha[f] = 0.0f;  // fragments behind the early out contribute nothing
         }
+        __syncthreads();  // all blending weights are in place
+        if (any_long)
+            sum_long_lists<TT, C, INFERENCE>(s_alpha, s_instance, s_pixel, s_count, s_feat, s_depth, n_fragments,
+                                             s_acc, s_dacc);
         __syncthreads();
+        INPC_PROF_MARK(5);
         // ---- instances: blending weights of the points (B/rasterization/src/bilinear/kernels.cu:291-295)
         if (!INFERENCE) {
 #pragma unroll
@@ -710,15 +992,22 @@ __global__ void __launch_bounds__(T* T)
                 else blending_weights[point[k]] = weight_sum;
             }
         }
-        if (__syncthreads_and(done)) break;
+#ifdef INPC_BLEND_PROFILE
+        ++prof_batches;
+#endif
+        const bool all_done = __syncthreads_and(done);
+        INPC_PROF_MARK(0);
+        if (all_done) break;
     }
+    INPC_PROF_FLUSH;
+    __syncthreads();
     if (inside) {
         const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
 #pragma unroll
-        for (int c = 0; c < C; ++c) image[c * n_pixels + pix] = F[c];
+        for (int c = 0; c < C; ++c) image[c * n_pixels + pix] = F[c] + s_acc[c * TT + lp];
         const float alpha_px = 1.0f - Tr;
         alpha_image[pix] = Tr < kTransmittanceThreshold ? 1.0f : alpha_px;
-        if (INFERENCE) depth_image[pix] = alpha_px > 0.0f ? D / alpha_px : 0.0f;
+        if (INFERENCE) depth_image[pix] = alpha_px > 0.0f ? (D + s_dacc[lp]) / alpha_px : 0.0f;
     }
     (void)lane;
 }
@@ -741,7 +1030,11 @@ __global__ void __launch_bounds__(T* T)
     __shared__ float s_alpha[kFragments];   // alpha, then blending weight
     __shared__ float s_dot[kFragments];     // features . grad, then d(loss)/d(alpha)
     __shared__ float s_grad[C * TT];        // channel-major upstream gradient of the tile (0 outside the image)
-    __shared__ uint32_t s_wave_total[TT / 64];
+    __shared__ float s_tb[kFragments];      // long lists: transmittance in front of the fragment (0: not reached)
+    __shared__ uint8_t s_pixel[kFragments];
+    __shared__ float s_t_in[TT], s_t_out[TT], s_r_in[TT], s_r_out[TT], s_offset[TT];
+    __shared__ SegItem s_item[TT / 64];
+    __shared__ uint32_t s_wave_total[TT / 64 + 1];
 
     const uint32_t tid = threadIdx.x;
     const uint32_t tile = blockIdx.x;
@@ -800,10 +1093,18 @@ __global__ void __launch_bounds__(T* T)
         __syncthreads();
         // ---- count
         const uint32_t my_count = done ? 0u : hits_total<T>(s_masks, lx, ly, n_words);
-        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total);
+        uint32_t n_fragments;
+        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total, n_fragments);
+        if (n_fragments == 0u) {  // every instance of the batch falls on finished pixels only
+            if (__syncthreads_and(done)) break;
+            continue;
+        }
         s_start[lp] = (uint16_t)my_start;
         s_count[lp] = (uint16_t)my_count;
-        __syncthreads();
+        s_t_in[lp] = Tr;
+        s_r_in[lp] = running;
+        s_offset[lp] = offset;
+        const bool any_long = __syncthreads_or(my_count > kLongList) != 0;
         // ---- place: alpha and features . grad of every fragment
         uint32_t where[NI][4];
         float weight[NI][4];
@@ -822,6 +1123,7 @@ __global__ void __launch_bounds__(T* T)
                         const uint32_t pos = s_start[pix] + hits_before<T>(s_masks, cx, cy, j >> 6);
                         where[k][q] = pos;
                         s_alpha[pos] = opacity[k] * weight[k][q];
+                        s_pixel[pos] = (uint8_t)pix;
                         float d = 0.0f;
 #pragma unroll
                         for (int c = 0; c < C; ++c) d = fmaf(feat[k][c], s_grad[c * TT + pix], d);
@@ -831,28 +1133,86 @@ __global__ void __launch_bounds__(T* T)
             }
         }
         __syncthreads();
-        // ---- pixels: the sequential part
-        if (my_count != 0u) {
-            uint32_t f = my_start;
+        // ---- pixels: the sequential part, without branches (a fragment behind the end of the list or
+        // behind the early out gets alpha 0: T stays, its weight and gradient are 0)
+        if (my_count != 0u && my_count <= kLongList) {
+            constexpr int kAhead = 4;
             const uint32_t end = my_start + my_count;
-            for (; f < end; ++f) {
-                const float a = s_alpha[f], s = s_dot[f];
-                const float bw = Tr * a;
-                const float one_minus_a = 1.0f - a;
-                const float rcp = __frcp_rn(fmaxf(one_minus_a, kOneMinusAlphaEps));
-                running = fmaf(bw, s, running);
-                s_alpha[f] = bw;
-                s_dot[f] = fmaf(Tr, s, (running + offset) * rcp);
-                Tr *= one_minus_a;
-                if (Tr < kTransmittanceThreshold) {
-                    done = true;
-                    ++f;
-                    break;
+            for (uint32_t f = my_start; f < end; f += kAhead) {
+                float a[kAhead], sd[kAhead];
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i) {
+                    a[i] = s_alpha[min(f + i, end - 1)];
+                    sd[i] = s_dot[min(f + i, end - 1)];
+                }
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i) {
+                    const bool live = f + i < end && !done;
+                    const float ai = live ? a[i] : 0.0f;
+                    const float bw = Tr * ai;
+                    const float one_minus_a = 1.0f - ai;
+                    const float rcp = __frcp_rn(fmaxf(one_minus_a, kOneMinusAlphaEps));
+                    running = fmaf(bw, sd[i], running);
+                    a[i] = bw;
+                    sd[i] = live ? fmaf(Tr, sd[i], (running + offset) * rcp) : 0.0f;
+                    Tr *= one_minus_a;
+                    done = done || (live && Tr < kTransmittanceThreshold);
+                }
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i) {
+                    if (f + i < end) {
+                        s_alpha[f + i] = a[i];
+                        s_dot[f + i] = sd[i];
+                    }
                 }
             }
-            for (; f < end; ++f) {
-                s_alpha[f] = 0.0f;
-                s_dot[f] = 0.0f;
+        }
+        if (any_long) {
+            // long lists: transmittance as a segmented product over the flat fragment array ...
+            segmented_scan<TT, true>(
+                n_fragments, s_item,
+                [&](uint32_t f, bool& flag, float& value) {
+                    const uint32_t p = s_pixel[f];
+                    const bool is_long = s_count[p] > kLongList;
+                    flag = !is_long || f == s_start[p];
+                    value = is_long ? 1.0f - s_alpha[f] : 1.0f;
+                },
+                [&](uint32_t f, float exclusive) {
+                    const uint32_t p = s_pixel[f];
+                    if (s_count[p] <= kLongList) return;
+                    const float t_before = s_t_in[p] * exclusive;
+                    const float t_after = t_before * (1.0f - s_alpha[f]);
+                    const bool live = !(t_before < kTransmittanceThreshold);
+                    s_tb[f] = live ? t_before : 0.0f;
+                    const bool last = f + 1 == (uint32_t)s_start[p] + s_count[p];
+                    if (live && (t_after < kTransmittanceThreshold || last)) s_t_out[p] = t_after;
+                });
+            __syncthreads();
+            // ... then the running weighted sum as a segmented sum, and the gradient of every fragment
+            segmented_scan<TT, false>(
+                n_fragments, s_item,
+                [&](uint32_t f, bool& flag, float& value) {
+                    const uint32_t p = s_pixel[f];
+                    const bool is_long = s_count[p] > kLongList;
+                    flag = !is_long || f == s_start[p];
+                    value = is_long ? (s_tb[f] * s_alpha[f]) * s_dot[f] : 0.0f;
+                },
+                [&](uint32_t f, float exclusive) {
+                    const uint32_t p = s_pixel[f];
+                    if (s_count[p] <= kLongList) return;
+                    const float a = s_alpha[f], sd = s_dot[f], t_before = s_tb[f];
+                    const float bw = t_before * a;
+                    const float run = (s_r_in[p] + exclusive) + bw * sd;
+                    const float rcp = __frcp_rn(fmaxf(1.0f - a, kOneMinusAlphaEps));
+                    s_alpha[f] = bw;
+                    s_dot[f] = t_before != 0.0f ? fmaf(t_before, sd, (run + s_offset[p]) * rcp) : 0.0f;
+                    if (f + 1 == (uint32_t)s_start[p] + s_count[p]) s_r_out[p] = run;
+                });
+            __syncthreads();
+            if (my_count > kLongList) {
+                Tr = s_t_out[lp];
+                running = s_r_out[lp];
+                done = Tr < kTransmittanceThreshold;
             }
         }
         __syncthreads();
@@ -1287,6 +1647,18 @@ int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
     }
     return INPC_OK;
 }
+
+#ifdef INPC_BLEND_PROFILE
+// development aid: per-phase shader clocks of k_blend_forward, summed over blocks (thread 0 of each)
+int inpc_debug_blend_profile(unsigned long long out[8], int reset) {
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_blend_profile), 8 * sizeof(unsigned long long)) != hipSuccess) return -1;
+    if (reset) {
+        unsigned long long zero[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (hipMemcpyToSymbol(HIP_SYMBOL(g_blend_profile), zero, sizeof(zero)) != hipSuccess) return -1;
+    }
+    return 0;
+}
+#endif
 
 int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* ws, uint32_t counters_host[3], void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
