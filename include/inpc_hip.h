@@ -115,7 +115,8 @@ int inpc_sample(const float* centers, const int32_t* levels, const float* cdf, c
 size_t inpc_cull_workspace_bytes(uint32_t n_candidates);
 
 /* Zero the round state (accepted count, consumed count) kept at the head of a cull
- * workspace. Call once before the first round of a draw. */
+ * workspace. Call once before the first round of a draw. Replaces the zero-initialised
+ * sample_counter tensor of B/sampling/src/sampling_api.cu:72. */
 int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream);
 
 /* One round of the training sampler: candidates k0 .. k0+n_candidates-1 of the counter-based
@@ -135,7 +136,9 @@ int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const 
                              float initial_size, const uint64_t* rng_dev, void* workspace,
                              size_t workspace_bytes, void* stream);
 
-/* Copy {accepted, consumed} of the current draw to host memory. Synchronises `stream`. */
+/* Copy {accepted, consumed} of the current draw to host memory. Synchronises `stream`.
+ * The one host read-back of a training draw; it stands where the reference reads the weight
+ * sum back (B/sampling/src/sampling.cu:106-107) before launching its single sampling kernel. */
 int inpc_cull_read_counts(const void* workspace, uint32_t* accepted_host, uint32_t* consumed_host,
                           void* stream);
 

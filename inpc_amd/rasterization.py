@@ -129,6 +129,7 @@ class _Rasterize(torch.autograd.Function):
     def forward(ctx: Any, positions: torch.Tensor, features: torch.Tensor, opacities: torch.Tensor,
                 rasterizer_settings: RasterizerSettings, tile: int = 8, feature_mode: int = _lib.FEAT_SH36_F16,
                 channels: int = 4):
+        _require_bilinear(rasterizer_settings)
         positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)
         image, alpha, blending_weights, workspace, cfg = _forward_native(
             rasterizer_settings, positions, features, opacities, tile, channels, feature_mode, inference=False)
@@ -219,6 +220,7 @@ class INPCRasterizer(torch.nn.Module):
         """(image, depth, alpha) from raw (N,37) fp16 appearance output; the sigma arguments only
         concern the Gaussian footprint and are ignored by the bilinear one, as in the reference."""
         settings = self.extract_settings(view, mode)
+        _require_bilinear(settings)
         positions, features_raw, _ = _checked_inputs(positions, features_raw, None, _lib.FEAT_RAW37_F16, 4)
         image, alpha, depth, _, _ = _forward_native(settings, positions, features_raw, None, self.tile, 4,
                                                     _lib.FEAT_RAW37_F16, inference=True)
@@ -229,6 +231,7 @@ class INPCRasterizer(torch.nn.Module):
                             sigma_world_scale: float = 1.0,
                             sigma_cutoff: float = 3.0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         settings = self.extract_settings(view, mode)
+        _require_bilinear(settings)
         positions, features, opacities = _checked_inputs(positions, features, opacities, _lib.FEAT_SH36_F16, 4)
         image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, self.tile, 4,
                                                     _lib.FEAT_SH36_F16, inference=True)
@@ -242,6 +245,8 @@ def rasterize_points(view, positions: torch.Tensor, features: torch.Tensor, opac
     opacities. Inference: (image, depth, alpha)."""
     settings = INPCRasterizer.extract_settings(view, RasterizerMode.BILINEAR.value)
     channels = features.shape[-1]
+    if features.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError("expected scalar type Float or Half")
     feature_mode = _lib.FEAT_DIRECT_F32 if features.dtype == torch.float32 else _lib.FEAT_DIRECT_F16
     if inference:
         positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)

@@ -1,0 +1,148 @@
+"""The C-ABI library: every function include/inpc_hip.h declares is exported and bound, the ctypes mirror of each
+struct has the C layout, and the host-only entry points (layout query, generator helpers, argument checks) behave.
+No kernel is launched here."""
+import ctypes as C
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from inpc_amd import _lib
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "inpc_hip.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return re.findall(r"^[A-Za-z_][\w \*]*?\b(inpc_\w+)\s*\(", text, flags=re.M)
+
+
+def test_header_functions_are_exported_and_bound():
+    names = declared_functions()
+    assert len(names) >= 24 and len(set(names)) == len(names)
+    assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
+    handle = C.CDLL(str(_lib.LIB_PATH))
+    for name in names:
+        assert hasattr(handle, name), f"{name} is declared but not exported"
+
+
+def test_every_entry_point_cites_the_interface_it_replaces():
+    text = HEADER.read_text()
+    # the comment block in front of each declaration names a file of the reference with line numbers
+    for name in declared_functions():
+        if name in ("inpc_last_error", "inpc_abi_version", "inpc_timing_enable", "inpc_timing_collect",
+                    "inpc_raster_layout_query", "inpc_raster_read_counters", "inpc_sampler_workspace_bytes",
+                    "inpc_cull_workspace_bytes"):
+            continue  # library plumbing without a counterpart
+        at = text.index(name + "(")
+        before = text[:at]
+        comment = before[before.rindex("/*"):]
+        assert re.search(r"B/[\w/\.]+:\d+", comment), f"{name}: no reference file:line in its comment"
+
+
+def test_header_is_plain_c_and_structs_match_ctypes(tmp_path):
+    fields = {
+        "inpc_camera": (_lib.Camera, [f for f, _ in _lib.Camera._fields_]),
+        "inpc_raster_config": (_lib.RasterConfig, [f for f, _ in _lib.RasterConfig._fields_]),
+        "inpc_raster_layout": (_lib.RasterLayout, [f for f, _ in _lib.RasterLayout._fields_]),
+        "inpc_timing_record": (_lib.TimingRecord, [f for f, _ in _lib.TimingRecord._fields_]),
+    }
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {"]
+    for struct, (_, names) in fields.items():
+        lines.append(f'  printf("{struct} %zu\\n", sizeof({struct}));')
+        for f in names:
+            lines.append(f'  printf("{struct}.{f} %zu\\n", offsetof({struct}, {f}));')
+    lines += ['  printf("codes %d %d %d %d %d %d\\n", INPC_OK, INPC_E_INVALID_ARGUMENT, INPC_E_WORKSPACE, '
+              'INPC_E_UNSUPPORTED, INPC_E_HIP, INPC_E_DEVICE);',
+              '  printf("modes %d %d %d %d %u\\n", INPC_FEAT_SH36_F16, INPC_FEAT_DIRECT_F32, INPC_FEAT_DIRECT_F16, '
+              'INPC_FEAT_RAW37_F16, INPC_RASTER_INFERENCE);', "  return 0; }"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", str(src), "-o", str(exe)], check=True)
+    out = dict(line.split(" ", 1) for line in subprocess.run([str(exe)], check=True, capture_output=True,
+                                                             text=True).stdout.splitlines())
+    for struct, (cls, names) in fields.items():
+        assert int(out[struct]) == C.sizeof(cls)
+        for f in names:
+            assert int(out[f"{struct}.{f}"]) == getattr(cls, f).offset, (struct, f)
+    assert out["codes"] == "0 -1 -2 -3 -4 -5"
+    assert out["modes"] == f"{_lib.FEAT_SH36_F16} {_lib.FEAT_DIRECT_F32} {_lib.FEAT_DIRECT_F16} " \
+                           f"{_lib.FEAT_RAW37_F16} {_lib.RASTER_INFERENCE}"
+
+
+def make_cfg(n, w, h, tile=16, channels=8, mode=_lib.FEAT_DIRECT_F32, flags=0):
+    return _lib.RasterConfig(n, tile, channels, mode, flags, _lib.Camera(w, h, 1000.0, 1000.0, w / 2, h / 2, 0.01, 100.0))
+
+
+def test_layout_query_on_the_host():
+    lib = _lib.lib()
+    assert lib.inpc_abi_version() >= 1
+    layout = _lib.RasterLayout()
+    cfg = make_cfg(8_388_608, 1237, 822)
+    assert lib.inpc_raster_layout_query(C.byref(cfg), C.byref(layout)) == 0
+    assert (layout.grid_width, layout.grid_height, layout.n_tiles) == (78, 52, 78 * 52)
+    assert layout.record_stride == 64 and layout.total_bytes % 256 == 0
+    assert layout.depth_key_bias == int(np.float32(0.01).view(np.uint32))
+    offsets = [layout.counters, layout.bin_start, layout.point_record, layout.depth_order, layout.depth_keys,
+               layout.instance_keys, layout.instance_slots, layout.tile_ranges]
+    assert all(o % 256 == 0 and o < layout.total_bytes for o in offsets) and len(set(offsets)) == len(offsets)
+    # every point can touch four tiles: the workspace holds at least 4 N instances of 6 bytes and N records
+    assert layout.total_bytes >= 8_388_608 * (64 + 4 * 6)
+    # bits the tile sort has to look at
+    assert layout.end_bit == (layout.n_tiles - 1).bit_length() == 12
+    small = _lib.RasterLayout()
+    assert lib.inpc_raster_layout_query(C.byref(make_cfg(0, 64, 64, 8, 4)), C.byref(small)) == 0
+    assert small.total_bytes > 0 and small.n_tiles == 64
+
+
+@pytest.mark.parametrize("cfg,code", [
+    (make_cfg(10, 64, 64, tile=12), -1),
+    (make_cfg(10, 64, 64, channels=5), -1),
+    (make_cfg(10, 0, 64), -1),
+    (make_cfg(10, 64, 64, mode=9), -3),
+    (make_cfg(10, 8 * 300, 8 * 300, tile=8), -3),            # more than 65536 tiles
+])
+def test_layout_query_rejects_bad_configurations(cfg, code):
+    lib = _lib.lib()
+    layout = _lib.RasterLayout()
+    assert lib.inpc_raster_layout_query(C.byref(cfg), C.byref(layout)) == code
+    assert lib.inpc_last_error()  # a message names the problem
+    with pytest.raises(_lib.BackendError):
+        _lib.check(code, "inpc_raster_layout_query")
+
+
+def test_argument_checks_come_before_any_launch():
+    lib = _lib.lib()
+    cfg = make_cfg(10, 64, 64)
+    # null pointers and a short workspace are refused on the host, so no GPU is needed to see the codes
+    assert lib.inpc_raster_forward(C.byref(cfg), None, None, None, None, None, None, None, None, None, None, 0,
+                                   None) in (-1, -2)
+    assert lib.inpc_raster_layout_query(None, None) == -1
+    assert lib.inpc_build_cdf(None, None, None, 0, 10, None) in (-1, -2)
+    assert lib.inpc_cull_begin(None, 0, None) in (-1, -2)
+    assert lib.inpc_sampler_workspace_bytes(1) > 0
+    assert lib.inpc_sampler_workspace_bytes(1 << 27) >= lib.inpc_sampler_workspace_bytes(1 << 20)
+    assert lib.inpc_cull_workspace_bytes(1 << 20) >= 256  # status words only: accepted samples go straight to the output
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libinpc_hip.so")
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.lib()
+
+
+def test_product_does_not_import_the_oracle():
+    code = ("import sys, inpc_amd, inpc_amd.sampling, inpc_amd.rasterization, inpc_amd.synthetic\n"
+            "bad = [m for m in sys.modules if m == 'oracle' or m.startswith('oracle.')]\n"
+            "sys.exit(1 if bad else 0)")
+    assert subprocess.run([sys.executable, "-c", code], cwd=ROOT).returncode == 0
+    for path in (ROOT / "inpc_amd").rglob("*"):
+        if path.suffix in (".py", ".hip", ".hpp", ".h"):
+            text = path.read_text()
+            assert "oracle" not in text.lower() or path.name == "build.py", f"{path} mentions the oracle"

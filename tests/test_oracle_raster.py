@@ -1,0 +1,332 @@
+"""Pins the oracle's rasterizer against closed forms, numpy's sort / search routines, a float64 brute-force
+blend over all points in global depth order, and torch autograd through a dense float64 restatement (CPU only)."""
+import numpy as np
+import pytest
+import torch
+
+from inpc_amd import synthetic
+
+
+def cam_of(O, hv):
+    c = hv.camera
+    return O.make_camera(c.width, c.height, c.focal_x, c.focal_y, c.center_x, c.center_y, c.near_plane, c.far_plane)
+
+
+def cfg_of(O, hv, n, tile, channels, mode=None, inference=False):
+    mode = O.FEAT_DIRECT_F32 if mode is None else mode
+    return O.make_config(n, cam_of(O, hv), tile, channels, mode, O.RASTER_INFERENCE if inference else 0)
+
+
+def project64(hv, p):
+    m = hv.w2c.astype(np.float64)
+    q = p.astype(np.float64) @ m[:3, :3].T + m[:3, 3]
+    c = hv.camera
+    return q[:, 0] / q[:, 2] * c.focal_x + c.center_x, q[:, 1] / q[:, 2] * c.focal_y + c.center_y, q[:, 2]
+
+
+def brute_force(hv, pos, feats, opac, depth_order, want_depth=False):
+    """Per pixel, front to back over ALL drawn points in the given global order (tiles only accelerate)."""
+    c = hv.camera
+    sx, sy, z = project64(hv, pos)
+    C_ = feats.shape[1]
+    img = np.zeros((C_, c.height, c.width))
+    dep = np.zeros((c.height, c.width))
+    Tr = np.ones((c.height, c.width))
+    done = np.zeros((c.height, c.width), bool)
+    bw_out = np.zeros(len(pos))
+    f64 = feats.astype(np.float64)
+    for i in depth_order:
+        for py in range(int(np.floor(sy[i] - 1.5)), int(np.floor(sy[i] + 0.5)) + 2):
+            for px in range(int(np.floor(sx[i] - 1.5)), int(np.floor(sx[i] + 0.5)) + 2):
+                if not (0 <= px < c.width and 0 <= py < c.height) or done[py, px]:
+                    continue
+                dx, dy = abs(sx[i] - (px + 0.5)), abs(sy[i] - (py + 0.5))
+                if dx >= 1 or dy >= 1:
+                    continue
+                w = (1 - dx) * (1 - dy)
+                a = float(opac[i]) * w
+                b = Tr[py, px] * a
+                bw_out[i] += b * w
+                img[:, py, px] += b * f64[i]
+                dep[py, px] += b * z[i]
+                Tr[py, px] *= 1 - a
+                if Tr[py, px] < 1e-4:
+                    done[py, px] = True
+    alpha = np.where(Tr < 1e-4, 1.0, 1 - Tr)
+    depth_img = np.where(1 - Tr > 0, dep / np.maximum(1 - Tr, 1e-300), 0.0)
+    return img, alpha, bw_out, depth_img
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_tile_bounds_worked_cases(oracle, tile):
+    # a camera whose projection is exact: focal 1, principal point 0, points at depth 1 -> sx = x, sy = y
+    from inpc_amd.views import PerspectiveCamera
+
+    W, H = 1237, 40
+    cam = PerspectiveCamera(W, H, 1.0, 1.0, 0.0, 0.0, 0.01, 100.0)
+    hv = synthetic.HostView(cam, np.eye(4, dtype=np.float32), np.zeros(3, np.float32))
+    gw = (W + tile - 1) // tile
+    sx = np.array([7.5, 8.0, 8.6, -0.4, -0.5, 15.5, 16.0, W + 1.0, gw * tile + 0.6, 0.5], np.float32)
+    pos = np.stack([sx, np.full_like(sx, 3.25), np.ones_like(sx)], axis=1)
+    n = len(sx)
+    ref = oracle.raster_forward(cfg_of(oracle, hv, n, tile, 4), pos, np.ones((n, 4), np.float32),
+                                np.full(n, 0.5, np.float32), hv.w2c, debug=True)
+    x0 = np.minimum(gw, np.maximum(0, np.floor((sx.astype(np.float64) - 0.5) / tile))).astype(int)
+    x1 = np.minimum(gw, np.maximum(0, np.ceil((sx.astype(np.float64) + 0.5) / tile))).astype(int)
+    touched = (x1 - x0) * 1
+    np.testing.assert_array_equal(ref["n_touched"], touched)
+    vis = touched > 0
+    np.testing.assert_array_equal(ref["bounds"][vis, 0], x0[vis])
+    np.testing.assert_array_equal(ref["bounds"][vis, 1], x1[vis])
+    if tile == 8:
+        # sx = 7.5 -> tile 0 only; 8.0 -> tiles 0 and 1; 8.6 -> tile 1; -0.4 -> tile 0; -0.5 -> culled
+        assert list(touched[:5]) == [1, 2, 1, 1, 0]
+    # a point right of the image but inside the padded tile grid is kept although no pixel reads it
+    assert touched[7] == (1 if W + 1.5 <= gw * tile else touched[7]) and touched[8] == 0
+    assert ref["n_visible"] == vis.sum() and ref["n_instances"] == touched.sum()
+    # culling at the near / far planes
+    pos2 = np.array([[0.5, 0.5, 0.0099], [0.5, 0.5, 0.01], [0.5, 0.5, 100.0], [0.5, 0.5, 100.1]], np.float32)
+    pos2[:, :2] *= pos2[:, 2:3] * 8   # keep the projection inside the image at every depth
+    ref2 = oracle.raster_forward(cfg_of(oracle, hv, 4, tile, 4), pos2, np.ones((4, 4), np.float32),
+                                 np.full(4, 0.5, np.float32), hv.w2c, debug=True)
+    assert list(ref2["n_touched"] > 0) == [False, True, True, False]
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_structure_against_numpy_sorts(oracle, tile):
+    n = 30000
+    hv = synthetic.rotated_camera(150, 97, 120.0, 2.5, 0.3, 0.2)
+    pos = synthetic.cube_points(n, 1.8, 3)
+    pos[:2000] = pos[2000:4000]          # duplicate points: equal depth keys must fall back to the point id
+    pos[5000:5200, 2] = pos[5000, 2]
+    feats, opac = synthetic.point_attributes(n, 4, "uniform", 4)
+    ref = oracle.raster_forward(cfg_of(oracle, hv, n, tile, 4), pos, feats, opac, hv.w2c, debug=True)
+    sx, sy, z = project64(hv, pos)
+    np.testing.assert_allclose(ref["screen_xy"][ref["n_touched"] > 0],
+                               np.stack([sx, sy], 1)[ref["n_touched"] > 0], rtol=0, atol=2e-4)
+    gw, gh = (150 + tile - 1) // tile, (97 + tile - 1) // tile
+    vis = np.flatnonzero(ref["n_touched"])
+    keys = ref["depth"].view(np.uint32)[vis]
+    order = vis[np.lexsort((vis, keys))]
+    np.testing.assert_array_equal(ref["depth_order"], order)
+    np.testing.assert_array_equal(ref["depth_keys"], ref["depth"].view(np.uint32)[order])
+    # instances: every touched tile of every point; final order = (tile, depth key, point id)
+    b = ref["bounds"].astype(np.int64)
+    inst_tile, inst_point = [], []
+    for i in vis:
+        for ty in range(b[i, 2], b[i, 3]):
+            for tx in range(b[i, 0], b[i, 1]):
+                inst_tile.append(ty * gw + tx)
+                inst_point.append(i)
+    inst_tile, inst_point = np.array(inst_tile), np.array(inst_point)
+    final = np.lexsort((inst_point, ref["depth"].view(np.uint32)[inst_point], inst_tile))
+    np.testing.assert_array_equal(ref["instance_keys"], inst_tile[final])
+    np.testing.assert_array_equal(ref["instance_points"], inst_point[final])
+    sorted_tiles = inst_tile[final]
+    begin = np.searchsorted(sorted_tiles, np.arange(gw * gh), "left")
+    end = np.searchsorted(sorted_tiles, np.arange(gw * gh), "right")
+    expect = np.stack([begin, end], 1)
+    expect[begin == end] = 0  # untouched tiles keep (0, 0)
+    np.testing.assert_array_equal(ref["tile_ranges"], expect)
+    # coverage: every pixel a point can reach lies in a tile the point touches
+    for i in vis[:3000]:
+        for px in (int(np.floor(sx[i] - 0.5)), int(np.floor(sx[i] - 0.5)) + 1):
+            for py in (int(np.floor(sy[i] - 0.5)), int(np.floor(sy[i] - 0.5)) + 1):
+                if 0 <= px < 150 and 0 <= py < 97 and abs(sx[i] - px - 0.5) < 1 - 1e-4 and abs(sy[i] - py - 0.5) < 1 - 1e-4:
+                    assert b[i, 0] <= px // tile < b[i, 1] and b[i, 2] <= py // tile < b[i, 3]
+
+
+@pytest.mark.parametrize("tile,channels", [(8, 4), (16, 8)])
+def test_blend_against_float64_brute_force(oracle, tile, channels):
+    n = 40000
+    hv = synthetic.camera_on_z(70, 45, 60.0, 2.2)
+    pos = synthetic.cube_points(n, 1.5, 5)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", 6)
+    opac = np.clip(opac * 1.6, 0, 0.98).astype(np.float32)   # enough opacity for early termination
+    ref = oracle.raster_forward(cfg_of(oracle, hv, n, tile, channels), pos, feats, opac, hv.w2c, debug=True)
+    img, alpha, bw, _ = brute_force(hv, pos, feats, opac, ref["depth_order"])
+    assert (alpha == 1.0).sum() > 50
+    np.testing.assert_allclose(ref["image"], img, rtol=1e-4, atol=2e-5)
+    np.testing.assert_allclose(ref["alpha"][0], alpha, rtol=1e-4, atol=2e-6)
+    np.testing.assert_allclose(ref["blending_weights"], bw, rtol=1e-4, atol=2e-6)
+    # inference variant: depth image
+    inf = oracle.raster_forward(cfg_of(oracle, hv, n, tile, channels, inference=True), pos, feats, opac, hv.w2c)
+    _, _, _, depth_img = brute_force(hv, pos, feats, opac, ref["depth_order"])
+    np.testing.assert_allclose(inf["image"], img, rtol=1e-4, atol=2e-5)
+    np.testing.assert_allclose(inf["depth_image"][0], depth_img, rtol=1e-4, atol=2e-5)
+
+
+def test_tile_size_does_not_change_the_image(oracle):
+    n = 20000
+    hv = synthetic.camera_on_z(101, 67, 90.0, 2.4)
+    pos = synthetic.cube_points(n, 1.6, 7)
+    feats, opac = synthetic.point_attributes(n, 4, "uniform", 8)
+    a = oracle.raster_forward(cfg_of(oracle, hv, n, 8, 4), pos, feats, opac, hv.w2c)
+    b = oracle.raster_forward(cfg_of(oracle, hv, n, 16, 4), pos, feats, opac, hv.w2c)
+    np.testing.assert_array_equal(a["image"], b["image"])
+    np.testing.assert_array_equal(a["alpha"], b["alpha"])
+
+
+def test_closed_forms(oracle):
+    from inpc_amd.views import PerspectiveCamera
+
+    cam = PerspectiveCamera(32, 32, 1.0, 1.0, 0.0, 0.0, 0.01, 100.0)
+    hv = synthetic.HostView(cam, np.eye(4, dtype=np.float32), np.zeros(3, np.float32))
+    f = np.array([[0.25, -1.0, 2.0, 0.5]], np.float32)
+
+    def run(points, feats, opac, tile=8):
+        points = np.asarray(points, np.float32)
+        return oracle.raster_forward(cfg_of(oracle, hv, len(points), tile, 4), points, np.asarray(feats, np.float32),
+                                     np.asarray(opac, np.float32), hv.w2c)
+
+    # one point exactly on a pixel centre: that pixel gets opacity * f, alpha = opacity, no neighbour is touched
+    r = run([[10.5, 20.5, 1.0]], f, [0.6])
+    np.testing.assert_allclose(r["image"][:, 20, 10], 0.6 * f[0], rtol=1e-6)
+    assert r["alpha"][0, 20, 10] == pytest.approx(0.6, rel=1e-6) and np.count_nonzero(r["alpha"]) == 1
+    assert r["blending_weights"][0] == pytest.approx(0.6, rel=1e-6)
+    # a point on the corner shared by four pixels: weight 1/4 each
+    r = run([[11.0, 21.0, 1.0]], f, [0.8])
+    for py, px in [(20, 10), (20, 11), (21, 10), (21, 11)]:
+        assert r["alpha"][0, py, px] == pytest.approx(0.2, rel=1e-6)
+        np.testing.assert_allclose(r["image"][:, py, px], 0.2 * f[0], rtol=1e-6)
+    assert r["blending_weights"][0] == pytest.approx(4 * 0.2 * 0.25, rel=1e-6)
+    # two points on one pixel centre: the "over" operator, nearer point first whatever the input order
+    f2 = np.array([[1, 0, 0, 0], [0, 1, 0, 0]], np.float32)
+    for points, feats, opac in ([[[5.5, 5.5, 1.0], [5.5, 5.5, 2.0]], f2, [0.5, 0.4]],
+                                [[[5.5, 5.5, 2.0], [5.5, 5.5, 1.0]], f2[::-1], [0.4, 0.5]]):
+        # at depth 2 the point must be scaled to keep projecting to (5.5, 5.5)
+        pts = np.array(points, np.float32)
+        pts[:, :2] *= pts[:, 2:3]
+        r = run(pts, feats, opac)
+        np.testing.assert_allclose(r["image"][:2, 5, 5], [0.5, 0.5 * 0.4], rtol=1e-6)
+        assert r["alpha"][0, 5, 5] == pytest.approx(1 - 0.5 * 0.6, rel=1e-6)
+    # an opaque point hides everything behind it and the pixel reports alpha 1
+    pts = np.array([[7.5, 7.5, 1.0], [7.5, 7.5, 3.0]], np.float32)
+    pts[:, :2] *= pts[:, 2:3]
+    r = run(pts, f2, [1.0, 0.9])
+    np.testing.assert_allclose(r["image"][:2, 7, 7], [1.0, 0.0], atol=1e-7)
+    assert r["alpha"][0, 7, 7] == 1.0 and r["blending_weights"][1] == 0.0
+
+
+def sh_basis64(d):
+    x, y, z = d[:, 0], d[:, 1], d[:, 2]
+    return np.stack([0.28209479177387814 * np.ones_like(x), -0.48860251190291987 * y, 0.48860251190291987 * z,
+                     -0.48860251190291987 * x, 1.0925484305920792 * x * y, -1.0925484305920792 * y * z,
+                     0.94617469575755997 * z * z - 0.31539156525251999, -1.0925484305920792 * x * z,
+                     0.54627421529603959 * (x * x - y * y)], axis=1)
+
+
+def test_sh_conversion_activation_and_adjointness(oracle):
+    n = 4000
+    hv = synthetic.rotated_camera(90, 60, 80.0, 2.5, 0.6, -0.4)
+    pos = synthetic.cube_points(n, 1.5, 9)
+    sh = synthetic.sh_features(n, 10)
+    _, opac = synthetic.point_attributes(n, 4, "normal", 11)
+    cfg = cfg_of(oracle, hv, n, 8, 4, oracle.FEAT_SH36_F16)
+    ref = oracle.raster_forward(cfg, pos, sh, opac, hv.w2c, hv.position, debug=True)
+    vis = ref["n_touched"] > 0
+    d = pos.astype(np.float64) - hv.position.astype(np.float64)
+    d /= np.linalg.norm(d, axis=1, keepdims=True)
+    basis = sh_basis64(d)                                                    # standard real SH, degree 2
+    expect = np.einsum("nk,nkc->nc", basis, sh.astype(np.float64).reshape(n, 9, 4))
+    np.testing.assert_allclose(ref["features_view"][vis], expect[vis], rtol=2e-5, atol=2e-6)
+    # raw appearance output: opacity = 1 - exp(-exp(raw[0])), SH coefficients behind it
+    raw = np.concatenate([np.random.default_rng(12).normal(-1, 1, (n, 1)), sh.astype(np.float64)], 1).astype(np.float16)
+    cfg37 = cfg_of(oracle, hv, n, 8, 4, oracle.FEAT_RAW37_F16, inference=True)
+    ref37 = oracle.raster_forward(cfg37, pos, raw, None, hv.w2c, hv.position, debug=True)
+    np.testing.assert_allclose(ref37["opacity"][vis], (1 - np.exp(-np.exp(raw[:, 0].astype(np.float64))))[vis],
+                               rtol=1e-5)
+    np.testing.assert_allclose(ref37["features_view"][vis], expect[vis], rtol=2e-5, atol=2e-6)
+    # backward of the SH conversion is its transpose: <convert(f), g> = <f, convert_T(g)>
+    rng = np.random.default_rng(13)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go, gv = oracle.raster_backward(cfg, gi, ga, ref["image"], ref["alpha"], pos, sh, opac, hv.w2c, hv.position)
+    expect_gf = np.einsum("nk,nc->nkc", basis, gv.astype(np.float64)).reshape(n, 36)
+    np.testing.assert_allclose(gf.astype(np.float64)[vis], expect_gf[vis], rtol=2e-3, atol=1e-7)  # fp16 output
+    assert (gf[~vis] == 0).all() and (go[~vis] == 0).all()
+
+
+def dense_forward_torch(hv, pos, feats, opac, order):
+    """Differentiable float64 restatement of the blend (no early termination in the cases it is used for)."""
+    c = hv.camera
+    sx, sy, _ = project64(hv, pos)
+    C_ = feats.shape[1]
+    img = [[torch.zeros(C_, dtype=torch.float64) for _ in range(c.width)] for _ in range(c.height)]
+    Tr = [[torch.ones((), dtype=torch.float64) for _ in range(c.width)] for _ in range(c.height)]
+    for i in order:
+        for py in range(int(np.floor(sy[i] - 1.5)), int(np.floor(sy[i] + 0.5)) + 2):
+            for px in range(int(np.floor(sx[i] - 1.5)), int(np.floor(sx[i] + 0.5)) + 2):
+                if not (0 <= px < c.width and 0 <= py < c.height):
+                    continue
+                dx, dy = abs(sx[i] - (px + 0.5)), abs(sy[i] - (py + 0.5))
+                if dx >= 1 or dy >= 1:
+                    continue
+                a = opac[i] * ((1 - dx) * (1 - dy))
+                img[py][px] = img[py][px] + Tr[py][px] * a * feats[i]
+                Tr[py][px] = Tr[py][px] * (1 - a)
+    image = torch.stack([torch.stack(row) for row in img]).permute(2, 0, 1)
+    alpha = 1 - torch.stack([torch.stack(row) for row in Tr])
+    return image, alpha[None]
+
+
+@pytest.mark.parametrize("tile,channels", [(8, 4), (16, 8)])
+def test_backward_against_autograd_and_finite_differences(oracle, tile, channels):
+    n = 150
+    hv = synthetic.camera_on_z(18, 14, 14.0, 2.0)
+    pos = synthetic.cube_points(n, 1.2, 21)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", 22)
+    opac = (opac * 0.5).astype(np.float32)   # transmittance stays above the threshold everywhere
+    cfg = cfg_of(oracle, hv, n, tile, channels)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    assert (ref["alpha"] < 0.9999).all()
+    rng = np.random.default_rng(23)
+    gi = rng.normal(0, 1.0, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1.0, ref["alpha"].shape).astype(np.float32)
+    gf, go, _ = oracle.raster_backward(cfg, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c)
+    f_t = torch.tensor(feats.astype(np.float64), requires_grad=True)
+    o_t = torch.tensor(opac.astype(np.float64), requires_grad=True)
+    image, alpha = dense_forward_torch(hv, pos, f_t, o_t, ref["depth_order"])
+    np.testing.assert_allclose(image.detach().numpy(), ref["image"], rtol=1e-4, atol=1e-5)
+    loss = (image * torch.tensor(gi, dtype=torch.float64)).sum() + (alpha * torch.tensor(ga, dtype=torch.float64)).sum()
+    loss.backward()
+    np.testing.assert_allclose(gf, f_t.grad.numpy(), rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(go, o_t.grad.numpy(), rtol=2e-4, atol=2e-5)
+    # central finite differences on a few opacities, through the oracle's own forward
+    for i in np.flatnonzero(ref["n_touched"])[:5]:
+        eps = 1e-2
+        vals = []
+        for sgn in (+1, -1):
+            o2 = opac.copy()
+            o2[i] += sgn * eps
+            r2 = oracle.raster_forward(cfg, pos, feats, o2, hv.w2c)
+            vals.append(float((r2["image"].astype(np.float64) * gi).sum() + (r2["alpha"].astype(np.float64) * ga).sum()))
+        assert go[i] == pytest.approx((vals[0] - vals[1]) / (2 * eps), rel=2e-2, abs=2e-3)
+
+
+def test_combined_step_equals_separate_calls(oracle):
+    n = 20000
+    hv = synthetic.camera_on_z(120, 80, 100.0, 2.4)
+    pos = synthetic.cube_points(n, 1.6, 31)
+    feats, opac = synthetic.point_attributes(n, 8, "normal", 32)
+    cfg = cfg_of(oracle, hv, n, 16, 8)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c)
+    rng = np.random.default_rng(33)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go, _ = oracle.raster_backward(cfg, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c)
+    image, alpha, bw, gf2, go2 = oracle.raster_forward_backward(cfg, pos, feats, opac, hv.w2c, gi, ga)
+    np.testing.assert_array_equal(image, ref["image"])
+    np.testing.assert_allclose(gf2, gf, rtol=1e-5, atol=1e-9)   # threads add in a different order
+    np.testing.assert_allclose(go2, go, rtol=1e-5, atol=1e-9)
+
+
+def test_unsupported_configurations(oracle):
+    hv = synthetic.camera_on_z(8 * 300, 8 * 300, 500.0, 3.0)
+    with pytest.raises(RuntimeError):
+        oracle.raster_forward(cfg_of(oracle, hv, 1, 8, 4), np.zeros((1, 3), np.float32), np.zeros((1, 4), np.float32),
+                              np.ones(1, np.float32), hv.w2c)   # more than 65536 tiles
+    hv = synthetic.camera_on_z(64, 64, 50.0, 3.0)
+    with pytest.raises(RuntimeError):
+        oracle.raster_forward(cfg_of(oracle, hv, 1, 12, 4), np.zeros((1, 3), np.float32), np.zeros((1, 4), np.float32),
+                              np.ones(1, np.float32), hv.w2c)   # tile size
