@@ -57,6 +57,22 @@ def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, depth_passes, tile
     return float(table.get(kernel, 0.0))
 
 
+def measured_traffic(kernel: str, workload: str):
+    """HBM bytes per launch of `kernel` from the committed profiler-counter summary of this workload
+    (profiles/hbm_traffic_<workload>.txt, lines `<kernel> fetch_bytes=F write_bytes=W total_bytes=T`),
+    or None when no such measurement is on file."""
+    path = ROOT / "profiles" / f"hbm_traffic_{workload}.txt"
+    if not path.exists():
+        return None
+    for line in path.read_text().splitlines():
+        parts = line.split()
+        if parts and parts[0] == kernel:
+            for item in parts[1:]:
+                if item.startswith("total_bytes="):
+                    return float(item.split("=", 1)[1])
+    return None
+
+
 def step_algorithmic_bytes(n, v, i, pixels, channels, end_bit):
     """Whole forward + backward step under the same model."""
     R = 8 + 4 + 4 * channels
@@ -73,6 +89,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="config3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="also launch three 1 GiB plain copies (the yardstick for profiler byte counters)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target duration of the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -145,6 +163,14 @@ def main() -> int:
         forward()
         backward()
 
+    if args.pmc_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(lib.inpc_calibration_copy(_lib.ptr(src), _lib.ptr(dst), src.numel(), stream), "copy")
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- timed region ---------------------------------------------------------------------------------
     for _ in range(args.warmup):
         step()
@@ -195,7 +221,8 @@ def main() -> int:
                                 tile_passes, layout.end_bit)
     achieved = dom_alg / (dominant["avg_ms"] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant["kernel"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": measured_traffic(dominant["kernel"], args.workload),
                 "algorithmic_bytes_per_launch": dom_alg, "avg_launch_ms": dominant["avg_ms"]}
     fwd_bytes, bwd_bytes = step_algorithmic_bytes(n, n_visible, n_instances, pixels, channels, layout.end_bit)
     step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
@@ -216,7 +243,7 @@ def main() -> int:
         gi_h, ga_h = grad_image.cpu().numpy(), grad_alpha.cpu().numpy()
         O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)  # warm-up
         reps, spent = 0, 0.0
-        while spent < args.cpu_seconds and reps < 50:
+        while spent < args.cpu_seconds and reps < 1000:
             t = O.now()
             O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)
             spent += O.now() - t

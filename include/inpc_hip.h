@@ -273,6 +273,12 @@ typedef struct inpc_timing_record {
 void inpc_timing_enable(int on);
 int inpc_timing_collect(inpc_timing_record* out, int capacity);
 
+/* Plain device-to-device copy kernel (reads `bytes`, writes `bytes`; both dev, 16-byte
+ * aligned, bytes a multiple of 16). It exists so that a profiler's memory counters can be
+ * scaled by what they read for a kernel whose traffic is known; no counterpart in the
+ * reference. */
+int inpc_calibration_copy(const void* src, void* dst, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

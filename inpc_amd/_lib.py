@@ -100,6 +100,7 @@ SIGNATURES = {
     "inpc_raster_read_counters": (C.c_int, [_CFG, _P, C.POINTER(_U32 * 3), _P]),
     "inpc_timing_enable": (None, [C.c_int]),
     "inpc_timing_collect": (C.c_int, [C.POINTER(TimingRecord), C.c_int]),
+    "inpc_calibration_copy": (C.c_int, [_P, _P, _SZ, _P]),
 }
 
 _lib = None

@@ -73,9 +73,28 @@ int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream) {
     return INPC_OK;
 }
 
+// Plain streaming copy, 16 bytes per lane: the yardstick for profiler byte counters.
+__global__ void __launch_bounds__(256) k_copy_u128(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
 }  // namespace inpc
 
 extern "C" {
+
+int inpc_calibration_copy(const void* src, void* dst, size_t bytes, void* stream) {
+    using namespace inpc;
+    if (!src || !dst) return fail(INPC_E_INVALID_ARGUMENT, "calibration_copy: null pointer");
+    if (bytes % 16 != 0 || ((uintptr_t)src | (uintptr_t)dst) % 16 != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "calibration_copy: pointers and size must be multiples of 16 bytes");
+    if (bytes == 0) return INPC_OK;
+    const size_t n = bytes / 16;
+    const uint32_t blocks = (uint32_t)std::min<size_t>((n + 255) / 256, 16384);
+    INPC_LAUNCH("calibration_copy", k_copy_u128, dim3(blocks), dim3(256), (hipStream_t)stream, (const uint4*)src,
+                (uint4*)dst, n);
+    return INPC_OK;
+}
 
 const char* inpc_last_error(void) { return inpc::g_error; }
 
