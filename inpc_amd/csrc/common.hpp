@@ -156,22 +156,36 @@ __device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_
         return 0u;
     }
     status_store(mine, kFlagAggregate | aggregate);
-    uint32_t exclusive = 0u;
-    for (int64_t p = (int64_t)bid - 1; p >= 0; --p) {
-        const uint32_t* theirs = status + (size_t)p * stride;
-        uint32_t word = status_load(theirs);
-        uint32_t spins = 0;
-        while ((word & ~kValueMask) == 0u) {
+    // Several predecessors are fetched per round trip and consumed nearest first; the walk ends at the
+    // first one that carries an inclusive prefix and waits at the first one that has nothing yet.
+    constexpr int kAhead = 8;
+    uint32_t exclusive = 0u, spins = 0u;
+    int64_t p = (int64_t)bid - 1;
+    bool finished = false;
+    while (!finished && p >= 0) {
+        uint32_t word[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int64_t q = p - u;
+            word[u] = q >= 0 ? status_load(status + (size_t)q * stride) : kFlagInclusive;  // before block 0: nothing
+        }
+        int consumed = 0;
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            if (finished || consumed != u) continue;
+            if ((word[u] & ~kValueMask) == 0u) continue;  // not published yet: stop consuming here
+            exclusive += word[u] & kValueMask;
+            ++consumed;
+            finished = (word[u] & kFlagInclusive) != 0u;
+        }
+        p -= consumed;
+        if (consumed == 0) {
             if (++spins > kSpinLimit) {
-                atomicOr(error_flag, 1u);
-                word = kFlagInclusive;  // give up: terminate the walk with a wrong but finite value
+                atomicOr(error_flag, 1u);  // give up: the result is wrong but the kernel ends
                 break;
             }
             __builtin_amdgcn_s_sleep(2);
-            word = status_load(theirs);
         }
-        exclusive += word & kValueMask;
-        if (word & kFlagInclusive) break;
     }
     status_store(mine, kFlagInclusive | ((exclusive + aggregate) & kValueMask));
     return exclusive;

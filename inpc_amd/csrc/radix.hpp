@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(kBlock)
     }
     const uint32_t local_base = wave_off + incl - total;
     s_local_base[tid] = local_base;
-    {
+    if (tid <= digit_mask) {  // one look-back per digit in use
         const uint32_t exclusive = lookback_exclusive(status + tid, kRadix, bid, total, error_flag);
         s_global[tid] = digit_base[tid] + exclusive - local_base;
     }

@@ -316,12 +316,17 @@ __global__ void __launch_bounds__(kBinThreads)
 }
 
 // ---- instance expansion -----------------------------------------------------------------------------------
-constexpr int kExpandItems = 4;
+constexpr int kExpandItems = 16;
 constexpr int kExpandTile = kBlock * kExpandItems;
+constexpr int kExpandStage = 6144;  // instances staged in LDS per output round
+constexpr int kCoarseShift = 8;     // one coarse entry per 256 record slots
 
-// Tile whose record bin holds `slot`: the last t with bin_start[t] <= slot.
-__device__ __forceinline__ uint32_t tile_of_slot(const uint32_t* __restrict__ bin_start, uint32_t n_tiles, uint32_t slot) {
-    uint32_t lo = 0, hi = n_tiles;  // invariant: bin_start[lo] <= slot < bin_start[hi]
+inline uint32_t coarse_entries(uint32_t n) { return (n >> kCoarseShift) + 2u; }
+
+// Tile whose record bin holds `slot`: the last t in [lo, hi) with bin_start[t] <= slot.
+// Requires bin_start[lo] <= slot < bin_start[hi].
+__device__ __forceinline__ uint32_t tile_of_slot(const uint32_t* __restrict__ bin_start, uint32_t lo, uint32_t hi,
+                                                 uint32_t slot) {
     while (hi - lo > 1) {
         const uint32_t mid = (lo + hi) >> 1;
         if (bin_start[mid] <= slot) lo = mid;
@@ -330,33 +335,71 @@ __device__ __forceinline__ uint32_t tile_of_slot(const uint32_t* __restrict__ bi
     return lo;
 }
 
+// coarse[b] = tile of record slot b << kCoarseShift (the last tile for slots behind the last record), so
+// that the tile of any slot is found between two neighbouring entries.
+__global__ void __launch_bounds__(kBlock) k_bin_coarse(const uint32_t* __restrict__ bin_start, uint16_t* __restrict__ coarse,
+                                                       uint32_t n_tiles, uint32_t n_entries) {
+    const uint32_t b = blockIdx.x * kBlock + threadIdx.x;
+    if (b >= n_entries) return;
+    const uint64_t slot = (uint64_t)b << kCoarseShift;
+    uint32_t t = n_tiles - 1u;
+    if (slot < bin_start[n_tiles]) t = tile_of_slot(bin_start, 0u, n_tiles, (uint32_t)slot);
+    coarse[b] = (uint16_t)t;
+}
+
+// Depth-ordered points -> instances (tile key, record slot), consecutive per point, row-major over the
+// touched tiles (B/rasterization/src/bilinear/kernels.cu:186-220). The exclusive sum of the per-point tile
+// counts is a single-pass scan (decoupled look-back); a block stages its run of instances in LDS and writes
+// it out with consecutive lanes on consecutive addresses.
 __global__ void __launch_bounds__(kBlock)
-    k_expand(const uint32_t* __restrict__ depth_order, const uint32_t* __restrict__ bin_start_global,
-             uint16_t* __restrict__ inst_keys, uint32_t* __restrict__ inst_points, uint32_t* counters, uint32_t* status,
-             uint32_t* g_hist, uint32_t gw, uint32_t n_tiles, radix::DevicePlan plan) {
-    extern __shared__ uint32_t s_bin_start[];  // n_tiles + 1 entries
+    k_expand(const uint32_t* __restrict__ depth_order, const uint32_t* __restrict__ bin_start,
+             const uint16_t* __restrict__ coarse, uint16_t* __restrict__ inst_keys, uint32_t* __restrict__ inst_points,
+             uint32_t* counters, uint32_t* status, uint32_t* g_hist, uint32_t gw, uint32_t n_tiles,
+             radix::DevicePlan plan) {
     __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
     __shared__ uint32_t s_wave[kBlock / kWave];
     __shared__ uint32_t s_bid, s_exclusive;
+    __shared__ uint32_t s_slot[kExpandStage];
+    __shared__ uint16_t s_tile[kExpandStage];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     for (int i = tid; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
     if (tid == 0) s_bid = atomicAdd(&counters[kCntTicketExpand], 1u);
     __syncthreads();
     const uint32_t bid = s_bid;
     const uint32_t n_visible = counters[kCntVisible];
-    const uint64_t first = (uint64_t)bid * kExpandTile + (uint64_t)tid * kExpandItems;
-    if ((uint64_t)bid * kExpandTile >= n_visible) return;
-    for (uint32_t t = tid; t <= n_tiles; t += kBlock) s_bin_start[t] = bin_start_global[t];
-    const uint32_t* bin_start = s_bin_start;  // visible after the barrier of the block scan below
+    const uint64_t block_first = (uint64_t)bid * kExpandTile;
+    if (block_first >= n_visible) return;
+    const uint64_t first = block_first + (uint64_t)tid * kExpandItems;
 
     uint32_t val[kExpandItems];
-    bool valid[kExpandItems];
+    if (block_first + kExpandTile <= n_visible) {
+        const uint4* src = (const uint4*)(depth_order + first);
+#pragma unroll
+        for (int q = 0; q < kExpandItems / 4; ++q) {
+            const uint4 v = src[q];
+            val[4 * q] = v.x;
+            val[4 * q + 1] = v.y;
+            val[4 * q + 2] = v.z;
+            val[4 * q + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < kExpandItems; ++j) val[j] = first + j < n_visible ? depth_order[first + j] : 0xFFFFFFFFu;
+    }
+    // 0xFFFFFFFF marks a slot behind the end: record slots stay below 2^28
     uint32_t mine = 0;
 #pragma unroll
+    for (int j = 0; j < kExpandItems; ++j)
+        if (val[j] != 0xFFFFFFFFu) mine += ((val[j] & 1u) + 1u) * (((val[j] >> 1) & 1u) + 1u);
+    // the tile of every point's first instance: two neighbouring coarse entries bound a short search
+    uint16_t tile0[kExpandItems];
+#pragma unroll
     for (int j = 0; j < kExpandItems; ++j) {
-        valid[j] = first + j < n_visible;
-        val[j] = valid[j] ? depth_order[first + j] : 0u;
-        if (valid[j]) mine += ((val[j] & 1u) + 1u) * (((val[j] >> 1) & 1u) + 1u);
+        tile0[j] = 0;
+        if (val[j] != 0xFFFFFFFFu) {
+            const uint32_t slot = val[j] >> 2, b = slot >> kCoarseShift;
+            tile0[j] = (uint16_t)tile_of_slot(bin_start, coarse[b], (uint32_t)coarse[b + 1] + 1u, slot);
+        }
     }
     // block exclusive scan of `mine`
     uint32_t incl = mine;
@@ -378,23 +421,33 @@ __global__ void __launch_bounds__(kBlock)
         const uint32_t exclusive = lookback_exclusive_wave(status, bid, block_total, &counters[kCntError]);
         if (lane == 0) s_exclusive = exclusive;
     }
-    __syncthreads();
-    uint32_t offset = s_exclusive + wave_off + incl - mine;
+    const uint32_t local_first = wave_off + incl - mine;  // of this thread's first instance inside the block's run
+    for (uint32_t round = 0; round < block_total; round += kExpandStage) {
+        uint32_t local = local_first;
 #pragma unroll
-    for (int j = 0; j < kExpandItems; ++j) {
-        if (!valid[j]) continue;
-        const uint32_t slot = val[j] >> 2, nx = (val[j] & 1u) + 1u, ny = ((val[j] >> 1) & 1u) + 1u;
-        const uint32_t tile0 = tile_of_slot(bin_start, n_tiles, slot);
-        for (uint32_t dy = 0; dy < ny; ++dy)
-            for (uint32_t dx = 0; dx < nx; ++dx) {
-                const uint32_t tile = tile0 + dy * gw + dx;
-                inst_keys[offset] = (uint16_t)tile;
-                inst_points[offset] = slot;
-                radix::hist_add(s_hist, plan, tile);
-                ++offset;
-            }
+        for (int j = 0; j < kExpandItems; ++j) {
+            if (val[j] == 0xFFFFFFFFu) continue;
+            const uint32_t slot = val[j] >> 2, nx = (val[j] & 1u) + 1u, ny = ((val[j] >> 1) & 1u) + 1u;
+            for (uint32_t dy = 0; dy < ny; ++dy)
+                for (uint32_t dx = 0; dx < nx; ++dx) {
+                    const uint32_t at = local - round;  // wraps below the round: fails the test as well
+                    if (at < (uint32_t)kExpandStage) {
+                        s_tile[at] = (uint16_t)(tile0[j] + dy * gw + dx);
+                        s_slot[at] = slot;
+                    }
+                    ++local;
+                }
+        }
+        __syncthreads();  // staging complete (first round: s_exclusive too)
+        const uint32_t out = s_exclusive + round, n_out = min((uint32_t)kExpandStage, block_total - round);
+        for (uint32_t i = tid; i < n_out; i += kBlock) {
+            const uint32_t tile = s_tile[i];
+            inst_keys[out + i] = (uint16_t)tile;
+            inst_points[out + i] = s_slot[i];
+            radix::hist_add(s_hist, plan, tile);
+        }
+        __syncthreads();
     }
-    __syncthreads();
     radix::hist_flush(s_hist, plan, g_hist);
 }
 
@@ -1300,7 +1353,7 @@ struct Layout {
     // private offsets
     size_t zero_begin, zero_words;  // region cleared at the start of every forward
     size_t hist_depth, hist_tile, bases_depth, bases_tile;
-    size_t status_depth, status_tile, status_expand;
+    size_t status_depth, status_tile, status_expand, bin_coarse;
     size_t bin_table, bin_total;
     size_t keys_a, keys_b, vals_a, vals_b;
     size_t inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
@@ -1373,6 +1426,7 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.bin_table = take((size_t)kBinBlocks * g.n_tiles * 4);
     L.bin_total = take((size_t)g.n_tiles * 4);
     P.bin_start = take((size_t)(g.n_tiles + 1) * 4);
+    L.bin_coarse = take((size_t)coarse_entries(g.n) * 2);
     L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
     L.bases_tile = take(radix::kMaxPasses * radix::kRadix * 4);
     P.point_record = take(n * g.stride);
@@ -1580,6 +1634,9 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                     at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
         INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
                     (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start), L.geo.n_tiles);
+        INPC_LAUNCH("raster_bin_coarse", k_bin_coarse, dim3(div_up(coarse_entries(L.geo.n), kBlock)), dim3(kBlock),
+                    stream, (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start), at<uint16_t>(ws, L.bin_coarse),
+                    L.geo.n_tiles, coarse_entries(L.geo.n));
         rc = dispatch_preprocess(L, positions, features, opacities, w2c, cam_position,
                                  L.inference ? nullptr : blending_weights, ws, stream);
         if (rc != INPC_OK) return rc;
@@ -1590,9 +1647,10 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                                          at<uint32_t>(ws, L.status_depth), counters + kCntTicketDepth,
                                          counters + kCntError, stream, "raster_depth_sort");
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH_LDS("raster_expand", k_expand, dim3(div_up(L.geo.n, kExpandTile)), dim3(kBlock),
-                    ((size_t)L.geo.n_tiles + 1) * 4, stream, (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
-                    at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), counters,
+        INPC_LAUNCH("raster_expand", k_expand, dim3(div_up(L.geo.n, kExpandTile)), dim3(kBlock), stream,
+                    (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order),
+                    (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
+                    (const uint16_t*)at<uint16_t>(ws, L.bin_coarse), at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), counters,
                     at<uint32_t>(ws, L.status_expand), at<uint32_t>(ws, L.hist_tile), L.geo.gw, L.geo.n_tiles,
                     radix::to_device_plan(L.tile_plan));
         const uint32_t ni = 4u * L.geo.n;
