@@ -146,16 +146,18 @@ __device__ __forceinline__ uint32_t status_load(const uint32_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Exclusive prefix of `aggregate` over blocks 0..bid-1, publishing this block's words on the way.
+// Publish this block's aggregate (block 0: its inclusive prefix). Doing this as early as the aggregate is
+// known lets the blocks behind finish their walk without waiting for this block's remaining work.
+__device__ __forceinline__ void lookback_publish(uint32_t* status, uint32_t stride, uint32_t bid, uint32_t aggregate) {
+    status_store(status + (size_t)bid * stride, (bid == 0 ? kFlagInclusive : kFlagAggregate) | aggregate);
+}
+
+// Exclusive prefix of the aggregates of blocks 0..bid-1; publishes this block's inclusive prefix.
 // `status` points at this stream's word of block 0; consecutive blocks are `stride` words apart.
-__device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_t stride, uint32_t bid,
-                                                       uint32_t aggregate, uint32_t* error_flag) {
-    uint32_t* mine = status + (size_t)bid * stride;
-    if (bid == 0) {
-        status_store(mine, kFlagInclusive | aggregate);
-        return 0u;
-    }
-    status_store(mine, kFlagAggregate | aggregate);
+// lookback_publish must have been called for this block.
+__device__ __forceinline__ uint32_t lookback_walk(uint32_t* status, uint32_t stride, uint32_t bid, uint32_t aggregate,
+                                                  uint32_t* error_flag) {
+    if (bid == 0) return 0u;
     // Several predecessors are fetched per round trip and consumed nearest first; the walk ends at the
     // first one that carries an inclusive prefix and waits at the first one that has nothing yet.
     constexpr int kAhead = 8;
@@ -187,8 +189,14 @@ __device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_
             __builtin_amdgcn_s_sleep(2);
         }
     }
-    status_store(mine, kFlagInclusive | ((exclusive + aggregate) & kValueMask));
+    status_store(status + (size_t)bid * stride, kFlagInclusive | ((exclusive + aggregate) & kValueMask));
     return exclusive;
+}
+
+__device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_t stride, uint32_t bid,
+                                                       uint32_t aggregate, uint32_t* error_flag) {
+    lookback_publish(status, stride, bid, aggregate);
+    return lookback_walk(status, stride, bid, aggregate, error_flag);
 }
 
 // The same for a single value per block, walked by a whole wave: the 64 lanes look at 64 predecessors at

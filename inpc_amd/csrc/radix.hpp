@@ -99,7 +99,33 @@ enum FirstPass : int {
                        // the drawn points for free
 };
 
+#ifdef INPC_SORT_PROFILE
+// development aid: per-phase shader clocks of k_scatter, summed over blocks (thread 0 of each)
+__device__ unsigned long long g_sort_profile[8];
+#define INPC_SORT_PROF_DECL unsigned long long sp_t = clock64(), sp_acc[7] = {0, 0, 0, 0, 0, 0, 0}
+#define INPC_SORT_PROF_MARK(i)                    \
+    do {                                          \
+        const unsigned long long now_ = clock64(); \
+        sp_acc[i] += now_ - sp_t;                 \
+        sp_t = now_;                              \
+    } while (0)
+#define INPC_SORT_PROF_FLUSH                                                        \
+    do {                                                                            \
+        if (threadIdx.x == 0) {                                                     \
+            for (int i_ = 0; i_ < 7; ++i_) atomicAdd(&g_sort_profile[i_], sp_acc[i_]); \
+            atomicAdd(&g_sort_profile[7], 1ull);                                    \
+        }                                                                           \
+    } while (0)
+#else
+#define INPC_SORT_PROF_DECL
+#define INPC_SORT_PROF_MARK(i)
+#define INPC_SORT_PROF_FLUSH
+#endif
+
 // One digit pass. FIRST: n comes from the host and keys equal to kInvalidKey are dropped.
+// Order of work inside a block: load -> digit histogram (LDS atomics) -> publish the aggregates -> stable
+// ranking -> look-back walk -> LDS staging -> coalesced write. Publishing before the expensive ranking means
+// that, by the time a block walks back, its predecessors' aggregates are already there.
 template <typename KeyT, bool FIRST>
 __global__ void __launch_bounds__(kBlock)
     k_scatter(const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
@@ -107,6 +133,7 @@ __global__ void __launch_bounds__(kBlock)
               uint32_t digit_mask, int bits, const uint32_t* __restrict__ digit_base, uint32_t* status,
               uint32_t* ticket, uint32_t* error_flag) {
     __shared__ uint32_t s_cnt[kWaves][kRadix];
+    __shared__ uint32_t s_hist[kRadix];
     __shared__ uint32_t s_local_base[kRadix];
     __shared__ uint32_t s_global[kRadix];
     __shared__ KeyT s_keys[kTile];
@@ -115,9 +142,12 @@ __global__ void __launch_bounds__(kBlock)
     __shared__ uint32_t s_bid;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    INPC_SORT_PROF_DECL;
     if (tid == 0) s_bid = atomicAdd(ticket, 1u);
     for (int i = tid; i < kWaves * kRadix; i += kBlock) (&s_cnt[0][0])[i] = 0u;
+    s_hist[tid] = 0u;
     __syncthreads();
+    INPC_SORT_PROF_MARK(0);
     const uint32_t bid = s_bid;
     uint32_t n = n_host;
     if (!FIRST) n = min(n_host, *n_dev);
@@ -126,7 +156,6 @@ __global__ void __launch_bounds__(kBlock)
 
     KeyT key[kItems];
     uint32_t val[kItems];
-    uint32_t rank[kItems];
     uint32_t valid_bits = 0;
     const uint64_t wave_base = tile_base + (uint64_t)wave * (kItems * kWave);
 #pragma unroll
@@ -138,7 +167,30 @@ __global__ void __launch_bounds__(kBlock)
         if (FIRST) valid = valid && ((uint32_t)k != kInvalidKey);
         val[r] = valid ? vals_in[idx] : 0u;
         key[r] = k;
-        const uint32_t d = ((uint32_t)k >> shift) & digit_mask;
+        if (valid) valid_bits |= 1u << r;
+    }
+#pragma unroll
+    for (int r = 0; r < kItems; ++r)
+        if (valid_bits & (1u << r)) atomicAdd(&s_hist[((uint32_t)key[r] >> shift) & digit_mask], 1u);
+    __syncthreads();
+    // thread d owns digit d: block total, publish, position of the digit's run inside the block
+    const uint32_t total = s_hist[tid];
+    if (tid <= digit_mask) lookback_publish(status + tid, kRadix, bid, total);
+    uint32_t incl = total;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s, 64);
+        if (lane >= (uint32_t)s) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    INPC_SORT_PROF_MARK(1);
+
+    // stable rank of every key among the keys of its wave with the same digit
+    uint32_t rank[kItems];
+#pragma unroll
+    for (int r = 0; r < kItems; ++r) {
+        const bool valid = (valid_bits >> r) & 1u;
+        const uint32_t d = ((uint32_t)key[r] >> shift) & digit_mask;
         uint64_t peers = __ballot(valid);
         for (int b = 0; b < bits; ++b) {
             const bool bit = (d >> b) & 1u;
@@ -147,34 +199,25 @@ __global__ void __launch_bounds__(kBlock)
         }
         rank[r] = 0;
         if (valid) {
-            valid_bits |= 1u << r;
             const uint32_t before = s_cnt[wave][d];
             rank[r] = before + mask_rank(peers);
             if (lane == 63u - (uint32_t)__clzll((long long)peers)) s_cnt[wave][d] = before + (uint32_t)__popcll(peers);
         }
         __builtin_amdgcn_wave_barrier();
     }
+    INPC_SORT_PROF_MARK(2);
     __syncthreads();
 
-    // thread d owns digit d: per-wave offsets, block total, local base, global base
-    uint32_t total = 0;
+    // per-wave offsets inside the digit's run, block-level exclusive scan over the digits
     {
-        const uint32_t d = tid;
+        uint32_t run = 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            const uint32_t c = s_cnt[w][d];
-            s_cnt[w][d] = total;
-            total += c;
+            const uint32_t c = s_cnt[w][tid];
+            s_cnt[w][tid] = run;
+            run += c;
         }
     }
-    uint32_t incl = total;
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s, 64);
-        if (lane >= (uint32_t)s) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
     uint32_t wave_off = 0, block_total = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
@@ -184,11 +227,13 @@ __global__ void __launch_bounds__(kBlock)
     }
     const uint32_t local_base = wave_off + incl - total;
     s_local_base[tid] = local_base;
+    INPC_SORT_PROF_MARK(3);
     if (tid <= digit_mask) {  // one look-back per digit in use
-        const uint32_t exclusive = lookback_exclusive(status + tid, kRadix, bid, total, error_flag);
+        const uint32_t exclusive = lookback_walk(status + tid, kRadix, bid, total, error_flag);
         s_global[tid] = digit_base[tid] + exclusive - local_base;
     }
     __syncthreads();
+    INPC_SORT_PROF_MARK(4);
 
 #pragma unroll
     for (int r = 0; r < kItems; ++r) {
@@ -200,6 +245,7 @@ __global__ void __launch_bounds__(kBlock)
         }
     }
     __syncthreads();
+    INPC_SORT_PROF_MARK(5);
 #pragma unroll
     for (int j = 0; j < kItems; ++j) {
         const uint32_t idx = j * kBlock + tid;
@@ -211,6 +257,8 @@ __global__ void __launch_bounds__(kBlock)
             vals_out[out] = s_vals[idx];
         }
     }
+    INPC_SORT_PROF_MARK(6);
+    INPC_SORT_PROF_FLUSH;
 }
 
 // Status words one pass needs for up to n_max keys.

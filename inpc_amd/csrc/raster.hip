@@ -1718,6 +1718,17 @@ int inpc_debug_blend_profile(unsigned long long out[8], int reset) {
 }
 #endif
 
+#ifdef INPC_SORT_PROFILE
+int inpc_debug_sort_profile(unsigned long long out[8], int reset) {
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(inpc::radix::g_sort_profile), 8 * sizeof(unsigned long long)) != hipSuccess) return -1;
+    if (reset) {
+        unsigned long long zero[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (hipMemcpyToSymbol(HIP_SYMBOL(inpc::radix::g_sort_profile), zero, sizeof(zero)) != hipSuccess) return -1;
+    }
+    return 0;
+}
+#endif
+
 int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* ws, uint32_t counters_host[3], void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     Layout L;
