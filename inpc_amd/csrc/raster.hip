@@ -471,6 +471,49 @@ __global__ void __launch_bounds__(kBlock) k_tile_ranges(const uint16_t* __restri
     }
 }
 
+// ---- tile schedule -----------------------------------------------------------------------------------------------
+// Blocks of the blend kernels take their tiles from this list: longest instance list first, so that the
+// few very long tiles do not start last and run on alone. The order only affects scheduling, not results
+// (tiles are independent); ties inside a bucket of 64 instances are in no particular order.
+constexpr int kOrderBuckets = 4096;
+__global__ void __launch_bounds__(kScanBlock) k_tile_order(const uint2* __restrict__ ranges, uint32_t* __restrict__ order,
+                                                           uint32_t n_tiles) {
+    __shared__ uint32_t s_bucket[kOrderBuckets];
+    __shared__ uint32_t s_wave[kScanBlock / kWave];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    for (int i = tid; i < kOrderBuckets; i += kScanBlock) s_bucket[i] = 0u;
+    __syncthreads();
+    // bucket 0 holds the longest lists
+    auto bucket_of = [&](uint32_t t) {
+        const uint2 r = ranges[t];
+        return (uint32_t)(kOrderBuckets - 1) - min((r.y - r.x) >> 6, (uint32_t)(kOrderBuckets - 1));
+    };
+    for (uint32_t t = tid; t < n_tiles; t += kScanBlock) atomicAdd(&s_bucket[bucket_of(t)], 1u);
+    __syncthreads();
+    constexpr int kPer = kOrderBuckets / kScanBlock;
+    uint32_t mine = 0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) mine += s_bucket[tid * kPer + i];
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s, 64);
+        if (lane >= (uint32_t)s) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - mine;
+    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+        const uint32_t c = s_bucket[tid * kPer + i];
+        s_bucket[tid * kPer + i] = run;
+        run += c;
+    }
+    __syncthreads();
+    for (uint32_t t = tid; t < n_tiles; t += kScanBlock) order[atomicAdd(&s_bucket[bucket_of(t)], 1u)] = t;
+}
+
 // ---- blend -------------------------------------------------------------------------------------------------
 //
 // One block per tile, one thread per pixel (a wave always covers an 8x8 pixel quad). Only the
@@ -825,6 +868,8 @@ __device__ unsigned long long g_blend_profile[8];
 #define INPC_PROF_FLUSH
 #endif
 
+#include "blend.hpp"
+
 template <int T, int C, bool HALF, bool INFERENCE>
 __global__ void __launch_bounds__(T* T)
     k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_slots,
@@ -1071,8 +1116,9 @@ __global__ void __launch_bounds__(T* T)
 // is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the pixel loop carries two scalars, not 2C.
 template <int T, int C, bool HALF>
 __global__ void __launch_bounds__(T* T)
-    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_slots,
-                     const char* __restrict__ records, uint32_t stride, const float* __restrict__ grad_image,
+    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
+                     const uint32_t* __restrict__ inst_slots, const char* __restrict__ records, uint32_t stride,
+                     const float* __restrict__ grad_image,
                      const float* __restrict__ grad_alpha, const float* __restrict__ image,
                      const float* __restrict__ alpha_image, float* grad_view, float* grad_opacities, int W, int H,
                      uint32_t gw) {
@@ -1090,7 +1136,7 @@ __global__ void __launch_bounds__(T* T)
     __shared__ uint32_t s_wave_total[TT / 64 + 1];
 
     const uint32_t tid = threadIdx.x;
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = tile_order[blockIdx.x];
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     int lx, ly;
     pixel_of_thread<T>(tid, lx, ly);
@@ -1354,7 +1400,7 @@ struct Layout {
     size_t zero_begin, zero_words;  // region cleared at the start of every forward
     size_t hist_depth, hist_tile, bases_depth, bases_tile;
     size_t status_depth, status_tile, status_expand, bin_coarse;
-    size_t bin_table, bin_total;
+    size_t bin_table, bin_total, tile_order;
     size_t keys_a, keys_b, vals_a, vals_b;
     size_t inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
 };
@@ -1425,6 +1471,7 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.zero_words = (off - L.zero_begin) / 4;
     L.bin_table = take((size_t)kBinBlocks * g.n_tiles * 4);
     L.bin_total = take((size_t)g.n_tiles * 4);
+    L.tile_order = take((size_t)g.n_tiles * 4);
     P.bin_start = take((size_t)(g.n_tiles + 1) * 4);
     L.bin_coarse = take((size_t)coarse_entries(g.n) * 2);
     L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
@@ -1502,15 +1549,16 @@ template <int T, int C, bool HALF>
 int launch_blend_forward(const Layout& L, float* image, float* alpha, float* blending_weights, float* depth_image,
                          void* ws, hipStream_t stream) {
     const uint2* ranges = at<uint2>(ws, L.pub.tile_ranges);
+    const uint32_t* order = at<uint32_t>(ws, L.tile_order);
     const uint32_t* inst = at<uint32_t>(ws, L.pub.instance_slots);
     const char* records = at<char>(ws, L.pub.point_record);
     if (L.inference) {
-        INPC_LAUNCH("raster_blend_inference", (k_blend_forward<T, C, HALF, true>), dim3(L.geo.n_tiles), dim3(T * T),
-                    stream, ranges, inst, records, L.geo.stride, image, alpha, (float*)nullptr, depth_image, L.geo.W,
+        INPC_LAUNCH("raster_blend_inference", (blend::k_blend_forward<T, C, HALF, true>), dim3(L.geo.n_tiles), dim3(T * T),
+                    stream, ranges, order, inst, records, L.geo.stride, image, alpha, (float*)nullptr, depth_image, L.geo.W,
                     L.geo.H, L.geo.gw);
     } else {
-        INPC_LAUNCH("raster_blend_forward", (k_blend_forward<T, C, HALF, false>), dim3(L.geo.n_tiles), dim3(T * T),
-                    stream, ranges, inst, records, L.geo.stride, image, alpha, blending_weights, (float*)nullptr,
+        INPC_LAUNCH("raster_blend_forward", (blend::k_blend_forward<T, C, HALF, false>), dim3(L.geo.n_tiles), dim3(T * T),
+                    stream, ranges, order, inst, records, L.geo.stride, image, alpha, blending_weights, (float*)nullptr,
                     L.geo.W, L.geo.H, L.geo.gw);
     }
     return INPC_OK;
@@ -1520,8 +1568,9 @@ template <int T, int C, bool HALF>
 int launch_blend_backward(const Layout& L, const float* grad_image, const float* grad_alpha, const float* image,
                           const float* alpha, float* grad_view, float* grad_opacities, void* ws, hipStream_t stream) {
     INPC_LAUNCH("raster_blend_backward", (k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
-                at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.pub.instance_slots),
-                at<char>(ws, L.pub.point_record), L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view,
+                at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
+                at<uint32_t>(ws, L.pub.instance_slots), at<char>(ws, L.pub.point_record), L.geo.stride, grad_image,
+                grad_alpha, image, alpha, grad_view,
                 grad_opacities, L.geo.W, L.geo.H, L.geo.gw);
     return INPC_OK;
 }
@@ -1665,6 +1714,8 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                     dim3(kBlock), stream, (const uint16_t*)at<uint16_t>(ws, L.pub.instance_keys),
                     at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)counters, ni);
     }
+    INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
+                (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
     return dispatch_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }
 
