@@ -19,11 +19,10 @@
 namespace blend {
 
 constexpr int kQuad = 8;             // a wave's pixel quad is 8 x 8
-constexpr int kSubFragments = 256;   // 64 instances x at most 2 x 2 pixels
-constexpr uint32_t kLongList = 12;   // lists longer than this are evaluated by the whole wave
-
-// Flags kept per staged instance.
-constexpr uint32_t kFlagShared = 1u;  // more than one quad of this tile takes part: accumulate with LDS atomics
+#ifndef INPC_LONG_LIST
+#define INPC_LONG_LIST 12
+#endif
+constexpr uint32_t kLongList = INPC_LONG_LIST;  // lists longer than this are evaluated by the whole wave
 
 __device__ __forceinline__ uint64_t lanes_below() {
     const uint32_t lane = __lane_id();
@@ -46,15 +45,15 @@ __device__ __forceinline__ uint32_t dpp_take(uint32_t old, uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)v, CTRL, ROW_MASK, 0xf, false);
 }
 
-// Inclusive product over the lanes 0..lane.
-__device__ __forceinline__ float wave_inclusive_product(float v) {
-    v *= dpp_take<kDppRowShr1, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowShr2, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowShr4, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowShr8, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowBcast15, 0xa>(1.0f, v);
-    v *= dpp_take<kDppRowBcast31, 0xc>(1.0f, v);
-    return v;
+// T_i = (...((t_in * m_0) * m_1)...) * m_i for the lanes i < n, multiplied strictly left to right: the result is
+// bit-identical to a sequential walk, which the early-out test against the transmittance threshold needs
+// (a product taken in tree order may land on the other side of the threshold). Every step, every lane takes
+// its left neighbour's value (lane 0: t_in) times its own factor: after step s the lanes 0..s hold their final
+// value, and computing a final value again from a final neighbour reproduces it. One multiply per step, no LDS.
+__device__ __forceinline__ float wave_sequential_product(float m, float t_in, uint32_t n) {
+    float x = m;
+    for (uint32_t s = 0; s < n; ++s) x = dpp_take<kDppWaveShr1, 0xf>(t_in, x) * m;
+    return x;
 }
 
 __device__ __forceinline__ float wave_inclusive_sum(float v) {
@@ -108,17 +107,19 @@ struct Stage {
     float depth[WITH_DEPTH ? TT : 1];
     float weight[NQ][NF][TT];   // interpolation weight of the fragment
     uint8_t pixel[NQ][NF][TT];  // its pixel in the wave's grid (row * 8 + column), kNoPixel: no fragment
-    uint8_t flags[TT];
+    float2 result[NQ][NF][TT];  // what the blend made of the fragment (written by the quad's wave, else {0, 0})
     uint8_t list[NQ][NQ][64];   // [quad][source wave][rank]: staged instances with an open pixel in the quad
     uint8_t count[NQ][NQ];
     uint64_t done[NQ];          // per quad: pixels that are finished
 };
 constexpr uint32_t kNoPixel = 0xFFu;
 
-// Per-wave scratch of the consume phase.
+// Per-wave scratch of the consume phase. A fragment entry is {alpha, x} on the way in and {blending weight, y}
+// on the way out; forward: x = staged instance; backward: x = features . grad, y = d loss / d alpha.
+template <int NF>
 struct QuadScratch {
-    uint64_t hits[64];             // per pixel: lanes (instances of the sub-batch) that hit it
-    float2 fragment[kSubFragments];  // per fragment in list order: {alpha, then blending weight; staged instance}
+    uint64_t hits[64];          // per pixel: lanes (instances of the sub-batch) that hit it
+    float2 fragment[64 * NF];   // per fragment, pixel by pixel, in depth order
 };
 
 // The record header as the kernels use it.
@@ -184,11 +185,11 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
                     if (open) in_quad[0] = true;
                 }
             }
-        int reached = 0;
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) reached += in_quad[q] ? 1 : 0;
-        st.flags[t] = reached > 1 ? (uint8_t)kFlagShared : (uint8_t)0;
     }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+        for (int k = 0; k < Stage<T, C, WITH_DEPTH>::NF; ++k) st.result[q][k][t] = make_float2(0.0f, 0.0f);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
         const uint64_t members = __ballot(in_quad[q]);
@@ -221,12 +222,14 @@ struct LaneFragments {
     uint32_t where[NF];  // position in the fragment list (valid when pixel != kNoPixel)
 };
 
-// Per-pixel fragment lists of one sub-batch. In: every lane's fragments (pixel, weight) and the alpha factor
-// `opacity`. Out: every pixel lane's list [my_start, my_start + my_count) of {alpha, instance} in depth order in
-// qs.fragment, and `where` for every fragment. Every lane of the wave must call it.
-template <int NF>
-__device__ __forceinline__ void build_fragment_lists(QuadScratch& qs, uint32_t j, float opacity, LaneFragments<NF>& lf,
-                                                     uint32_t& my_start, uint32_t& my_count, uint32_t& n_fragments) {
+// Per-pixel fragment lists of one sub-batch. In: every lane's fragments (pixel, weight), the alpha factor
+// `opacity`, and payload(q), the second word of fragment q's entry. Out: every pixel lane's list
+// [my_start, my_start + my_count) of {alpha, payload} in depth order in qs.fragment, and `where` for every
+// fragment. Every lane of the wave must call it.
+template <int NF, typename Payload>
+__device__ __forceinline__ void build_fragment_lists(QuadScratch<NF>& qs, float opacity, LaneFragments<NF>& lf,
+                                                     uint32_t& my_start, uint32_t& my_count, uint32_t& n_fragments,
+                                                     Payload payload) {
     const uint32_t lane = __lane_id();
     qs.hits[lane] = 0ull;
     wave_sync();
@@ -247,7 +250,7 @@ __device__ __forceinline__ void build_fragment_lists(QuadScratch& qs, uint32_t j
         if (hit) {
             const uint32_t pos = start + (uint32_t)__popcll(qs.hits[pix] & below);
             lf.where[q] = pos;
-            qs.fragment[pos] = make_float2(opacity * lf.weight[q], __uint_as_float(j));
+            qs.fragment[pos] = make_float2(opacity * lf.weight[q], payload(q));
         }
     }
     wave_sync();
@@ -281,8 +284,7 @@ __global__ void __launch_bounds__(T* T)
     constexpr int NQ = TT / 64;
     constexpr int NF = Stage<T, C, INFERENCE>::NF;
     __shared__ Stage<T, C, INFERENCE> st;
-    __shared__ QuadScratch s_quad[NQ];
-    __shared__ float s_weight[INFERENCE ? 1 : TT];  // blending weight of every staged instance
+    __shared__ QuadScratch<NF> s_quad[NQ];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tile = tile_order[blockIdx.x];
@@ -290,7 +292,7 @@ __global__ void __launch_bounds__(T* T)
     const int px = tile_x0 + (T == 16 ? 2 * (int)(lane & 7u) + (int)(wave & 1u) : (int)(lane & 7u));
     const int py = tile_y0 + (T == 16 ? 2 * (int)(lane >> 3) + (int)(wave >> 1) : (int)(lane >> 3));
     const bool inside = px < W && py < H;
-    QuadScratch& qs = s_quad[wave];
+    QuadScratch<NF>& qs = s_quad[wave];
 
     float F[C];
 #pragma unroll
@@ -332,7 +334,6 @@ __global__ void __launch_bounds__(T* T)
         }
         if (begin + 2 * TT + tid < range.y) next_slot = inst_slots[begin + 2 * TT + tid];
         stage_instance<T, C, INFERENCE>(st, valid, h, f, tile_x0, tile_y0);
-        if (!INFERENCE) s_weight[tid] = 0.0f;
         INPC_PROF_MARK(0);
         __syncthreads();
         INPC_PROF_MARK(1);
@@ -347,7 +348,8 @@ __global__ void __launch_bounds__(T* T)
             LaneFragments<NF> lf;
             load_lane_fragments<T, C, INFERENCE>(st, wave, live, j, __ballot(done), lf);
             uint32_t my_start, my_count, n_fragments;
-            build_fragment_lists<NF>(qs, j, st.opacity[j], lf, my_start, my_count, n_fragments);
+            build_fragment_lists<NF>(qs, st.opacity[j], lf, my_start, my_count, n_fragments,
+                                     [&](int) { return __uint_as_float(j); });
             INPC_PROF_MARK(2);
             if (n_fragments == 0u) continue;
             // ---- pixels with short lists: the reference's sequential walk (kernels.cu:281-299)
@@ -390,9 +392,8 @@ __global__ void __launch_bounds__(T* T)
                     float2 e = make_float2(0.0f, 0.0f);
                     if (here) e = qs.fragment[pos];
                     const float a = e.x;
-                    const float incl = wave_inclusive_product(1.0f - a);
-                    const float excl = wave_previous(incl, 1.0f);
-                    const float t_before = p_T * excl;
+                    const float t_after = wave_sequential_product(1.0f - a, p_T, min(64u, p_count - base));
+                    const float t_before = wave_previous(t_after, p_T);
                     const bool reached = here && !(t_before < kTransmittanceThreshold);
                     const float bw = reached ? t_before * a : 0.0f;
                     if (here) qs.fragment[pos].x = bw;
@@ -411,7 +412,7 @@ __global__ void __launch_bounds__(T* T)
                     // transmittance behind the last fragment that was reached
                     const uint64_t reached_lanes = __ballot(reached);
                     const int last = 63 - __builtin_clzll(reached_lanes | 1ull);
-                    p_T = __shfl(p_T * incl, last, 64);
+                    p_T = __shfl(t_after, last, 64);
                     // a walk that ended inside this round leaves the rest of the list untouched: weights 0
                     if (p_T < kTransmittanceThreshold)
                         for (uint32_t rest = base + 64u + lane; rest < p_count; rest += 64u) qs.fragment[p_start + rest].x = 0.0f;
@@ -432,19 +433,11 @@ __global__ void __launch_bounds__(T* T)
             }
             wave_sync();
             INPC_PROF_MARK(4);
-            // ---- instances: blending weight of the point (kernels.cu:291-295)
+            // ---- instances: hand the blending weights of the fragments to the thread that owns the instance
             if (!INFERENCE) {
-                float weight_sum = 0.0f;
 #pragma unroll
-                for (int q = 0; q < NF; ++q) {
-                    if (lf.pixel[q] == kNoPixel) continue;
-                    const float bw = qs.fragment[lf.where[q]].x;
-                    if (bw > 0.0f) weight_sum = fmaf(bw, lf.weight[q], weight_sum);
-                }
-                if (weight_sum > 0.0f) {
-                    if (st.flags[j] & kFlagShared) lds_add(&s_weight[j], weight_sum);
-                    else s_weight[j] = weight_sum;
-                }
+                for (int q = 0; q < NF; ++q)
+                    if (lf.pixel[q] != kNoPixel) st.result[wave][q][j] = qs.fragment[lf.where[q]];
             }
         }
         {
@@ -457,9 +450,16 @@ __global__ void __launch_bounds__(T* T)
 #ifdef INPC_BLEND_PROFILE
         ++prof_batches;
 #endif
-        // ---- write: thread t owns staged instance t
+        // ---- write: thread t owns staged instance t (kernels.cu:291-295)
         if (!INFERENCE && valid) {
-            const float w = s_weight[tid];
+            float w = 0.0f;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+#pragma unroll
+                for (int k = 0; k < NF; ++k) {
+                    const float bw = st.result[q][k][tid].x;
+                    if (bw > 0.0f) w = fmaf(bw, st.weight[q][k][tid], w);
+                }
             if (w > 0.0f) {
                 if (h.multi) atomicAdd(&blending_weights[h.point], w);
                 else blending_weights[h.point] = w;
@@ -475,6 +475,209 @@ __global__ void __launch_bounds__(T* T)
         const float alpha_px = 1.0f - Tr;
         alpha_image[pix] = Tr < kTransmittanceThreshold ? 1.0f : alpha_px;
         if (INFERENCE) depth_image[pix] = alpha_px > 0.0f ? D / alpha_px : 0.0f;
+    }
+}
+
+// ---- backward -----------------------------------------------------------------------------------------------------
+// With s = features . grad of a fragment, R the running sum of weight x s of a pixel and S its final value
+// image . grad, the opacity gradient of the reference (kernels.cu:405-413),
+//   dot(T f + (F_running - F_final) / (1 - a), grad) + grad_alpha (1 - alpha_final) / (1 - a),
+// is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the pixel walk carries two scalars, not 2C.
+template <int T, int C, bool HALF>
+__global__ void __launch_bounds__(T* T)
+    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
+                     const uint32_t* __restrict__ inst_slots, const char* __restrict__ records, uint32_t stride,
+                     const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
+                     const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_view,
+                     float* grad_opacities, int W, int H, uint32_t gw) {
+    constexpr int TT = T * T;
+    constexpr int NQ = TT / 64;
+    constexpr int NF = Stage<T, C, false>::NF;
+    __shared__ Stage<T, C, false> st;
+    __shared__ QuadScratch<NF> s_quad[NQ];
+    __shared__ float s_grad[NQ][C][64];   // upstream gradient of every wave's pixels (0 outside the image)
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tile = tile_order[blockIdx.x];
+    const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
+    const int px = tile_x0 + (T == 16 ? 2 * (int)(lane & 7u) + (int)(wave & 1u) : (int)(lane & 7u));
+    const int py = tile_y0 + (T == 16 ? 2 * (int)(lane >> 3) + (int)(wave >> 1) : (int)(lane >> 3));
+    const bool inside = px < W && py < H;
+    QuadScratch<NF>& qs = s_quad[wave];
+
+    float final_dot = 0.0f, common = 0.0f;
+    {
+        const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const float g = inside ? grad_image[c * n_pixels + pix] : 0.0f;
+            s_grad[wave][c][lane] = g;
+            if (inside) final_dot = fmaf(image[c * n_pixels + pix], g, final_dot);
+        }
+        if (inside) common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
+    }
+    const float offset = common - final_dot;
+    float Tr = 1.0f, running = 0.0f;
+    bool done = !inside;
+    {
+        const uint64_t finished = __ballot(done);
+        if (lane == 0u) st.done[wave] = finished;
+    }
+    __syncthreads();
+
+    const uint2 range = ranges[tile];
+    uint32_t next_slot = 0u;
+    Header h_next{};
+    float f_next[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) f_next[c] = 0.0f;
+    if (range.x + tid < range.y) {
+        const char* record = records + (size_t)inst_slots[range.x + tid] * stride;
+        h_next = read_header(record);
+        load_record_features<C, HALF>(f_next, record);
+    }
+    if (range.x + TT + tid < range.y) next_slot = inst_slots[range.x + TT + tid];
+    for (uint32_t begin = range.x; begin < range.y; begin += TT) {
+        const uint32_t count = min((uint32_t)TT, range.y - begin);
+        const bool valid = tid < count;
+        const Header h = h_next;
+        float f[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) f[c] = f_next[c];
+        if (begin + TT + tid < range.y) {
+            const char* record = records + (size_t)next_slot * stride;
+            h_next = read_header(record);
+            load_record_features<C, HALF>(f_next, record);
+        }
+        if (begin + 2 * TT + tid < range.y) next_slot = inst_slots[begin + 2 * TT + tid];
+        stage_instance<T, C, false>(st, valid, h, f, tile_x0, tile_y0);
+        __syncthreads();
+
+        // ---- consume: this wave's list
+        uint32_t total = 0;
+#pragma unroll
+        for (int s = 0; s < NQ; ++s) total += st.count[wave][s];
+        for (uint32_t sub = 0; sub < total; sub += 64u) {
+            const bool live = sub + lane < total;
+            const uint32_t j = live ? list_entry<T, C, false>(st, wave, sub + lane) : 0u;
+            LaneFragments<NF> lf;
+            load_lane_fragments<T, C, false>(st, wave, live, j, __ballot(done), lf);
+            float feat[C];
+#pragma unroll
+            for (int q4 = 0; q4 < C / 4; ++q4) {
+                const float4 v = st.feat[j * (C / 4) + q4];
+                feat[4 * q4] = v.x;
+                feat[4 * q4 + 1] = v.y;
+                feat[4 * q4 + 2] = v.z;
+                feat[4 * q4 + 3] = v.w;
+            }
+            uint32_t my_start, my_count, n_fragments;
+            build_fragment_lists<NF>(qs, st.opacity[j], lf, my_start, my_count, n_fragments, [&](int q) {
+                float d = 0.0f;  // features . grad of the fragment's pixel
+#pragma unroll
+                for (int c = 0; c < C; ++c) d = fmaf(feat[c], s_grad[wave][c][lf.pixel[q]], d);
+                return d;
+            });
+            if (n_fragments == 0u) continue;
+            // ---- pixels with short lists: the sequential walk (kernels.cu:383-417)
+            if (my_count <= kLongList) {
+                for (uint32_t i = 0; i < my_count; ++i) {
+                    const uint32_t pos = my_start + i;
+                    const float2 e = qs.fragment[pos];
+                    const float a = done ? 0.0f : e.x, sd = e.y;
+                    const float bw = Tr * a;
+                    const float one_minus_a = 1.0f - a;
+                    const float rcp = __frcp_rn(fmaxf(one_minus_a, kOneMinusAlphaEps));
+                    running = fmaf(bw, sd, running);
+                    const float dalpha = done ? 0.0f : fmaf(Tr, sd, (running + offset) * rcp);
+                    qs.fragment[pos] = make_float2(bw, dalpha);
+                    Tr *= one_minus_a;
+                    done = done || Tr < kTransmittanceThreshold;
+                }
+            }
+            // ---- pixels with long lists, one after the other, 64 fragments at a time over the wave
+            uint64_t long_pixels = __ballot(my_count > kLongList);
+            while (long_pixels) {
+                const int p = __builtin_ctzll(long_pixels);
+                long_pixels &= long_pixels - 1ull;
+                const uint32_t p_start = __shfl(my_start, p, 64), p_count = __shfl(my_count, p, 64);
+                float p_T = __shfl(Tr, p, 64), p_R = __shfl(running, p, 64);
+                const float p_offset = __shfl(offset, p, 64);
+                for (uint32_t base = 0; base < p_count && !(p_T < kTransmittanceThreshold); base += 64u) {
+                    const bool here = base + lane < p_count;
+                    const uint32_t pos = p_start + base + lane;
+                    float2 e = make_float2(0.0f, 0.0f);
+                    if (here) e = qs.fragment[pos];
+                    const float a = e.x, sd = e.y;
+                    const float t_after = wave_sequential_product(1.0f - a, p_T, min(64u, p_count - base));
+                    const float t_before = wave_previous(t_after, p_T);
+                    const bool reached = here && !(t_before < kTransmittanceThreshold);
+                    const float bw = reached ? t_before * a : 0.0f;
+                    const float run = p_R + wave_inclusive_sum(bw * sd);
+                    const float rcp = __frcp_rn(fmaxf(1.0f - a, kOneMinusAlphaEps));
+                    const float dalpha = reached ? fmaf(t_before, sd, (run + p_offset) * rcp) : 0.0f;
+                    if (here) qs.fragment[pos] = make_float2(bw, dalpha);
+                    const uint64_t reached_lanes = __ballot(reached);
+                    const int last = 63 - __builtin_clzll(reached_lanes | 1ull);
+                    p_T = __shfl(t_after, last, 64);
+                    p_R = __shfl(run, last, 64);
+                    if (p_T < kTransmittanceThreshold)
+                        for (uint32_t rest = base + 64u + lane; rest < p_count; rest += 64u)
+                            qs.fragment[p_start + rest] = make_float2(0.0f, 0.0f);
+                }
+                if ((int)lane == p) {
+                    Tr = p_T;
+                    running = p_R;
+                    done = Tr < kTransmittanceThreshold;
+                }
+            }
+            wave_sync();
+            // ---- instances: hand {blending weight, d loss / d alpha} of the fragments to the instance's thread
+#pragma unroll
+            for (int q = 0; q < NF; ++q)
+                if (lf.pixel[q] != kNoPixel) st.result[wave][q][j] = qs.fragment[lf.where[q]];
+        }
+        {
+            const uint64_t finished = __ballot(done);
+            if (lane == 0u) st.done[wave] = finished;
+        }
+        const bool all_done = __syncthreads_and(done) != 0;
+        // ---- write: thread t owns staged instance t: gradient of the point from its fragments in all quads
+        if (valid) {
+            float gf[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) gf[c] = 0.0f;
+            float gop = 0.0f;
+            bool any_weight = false;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+#pragma unroll
+                for (int k = 0; k < NF; ++k) {
+                    const float2 e = st.result[q][k][tid];
+                    gop = fmaf(e.y, st.weight[q][k][tid], gop);
+                    if (e.x > 0.0f) {
+                        any_weight = true;
+                        const uint32_t pix = st.pixel[q][k][tid];
+#pragma unroll
+                        for (int c = 0; c < C; ++c) gf[c] = fmaf(e.x, s_grad[q][c][pix], gf[c]);
+                    }
+                }
+            if (any_weight || gop != 0.0f) {
+                float* dst = grad_view + (size_t)h.point * C;
+                if (h.multi) {
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                        if (gf[c] != 0.0f) atomicAdd(dst + c, gf[c]);
+                    if (gop != 0.0f) atomicAdd(&grad_opacities[h.point], gop);
+                } else {
+#pragma unroll
+                    for (int q4 = 0; q4 < C / 4; ++q4)
+                        ((float4*)dst)[q4] = make_float4(gf[4 * q4], gf[4 * q4 + 1], gf[4 * q4 + 2], gf[4 * q4 + 3]);
+                    grad_opacities[h.point] = gop;
+                }
+            }
+        }
+        if (all_done) break;
     }
 }
 

@@ -1567,7 +1567,7 @@ int launch_blend_forward(const Layout& L, float* image, float* alpha, float* ble
 template <int T, int C, bool HALF>
 int launch_blend_backward(const Layout& L, const float* grad_image, const float* grad_alpha, const float* image,
                           const float* alpha, float* grad_view, float* grad_opacities, void* ws, hipStream_t stream) {
-    INPC_LAUNCH("raster_blend_backward", (k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
+    INPC_LAUNCH("raster_blend_backward", (blend::k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 at<uint32_t>(ws, L.pub.instance_slots), at<char>(ws, L.pub.point_record), L.geo.stride, grad_image,
                 grad_alpha, image, alpha, grad_view,
