@@ -50,9 +50,13 @@ __device__ __forceinline__ uint32_t dpp_take(uint32_t old, uint32_t v) {
 // (a product taken in tree order may land on the other side of the threshold). Every step, every lane takes
 // its left neighbour's value (lane 0: t_in) times its own factor: after step s the lanes 0..s hold their final
 // value, and computing a final value again from a final neighbour reproduces it. One multiply per step, no LDS.
+// (Steps beyond n only recompute final values, so the loop runs in unrolled groups of eight.)
 __device__ __forceinline__ float wave_sequential_product(float m, float t_in, uint32_t n) {
     float x = m;
-    for (uint32_t s = 0; s < n; ++s) x = dpp_take<kDppWaveShr1, 0xf>(t_in, x) * m;
+    for (uint32_t s = 0; s < n; s += 8u) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x = dpp_take<kDppWaveShr1, 0xf>(t_in, x) * m;
+    }
     return x;
 }
 
@@ -306,7 +310,12 @@ __global__ void __launch_bounds__(T* T)
     __syncthreads();
 
     const uint2 range = ranges[tile];
+#ifdef INPC_PROFILE_BACKWARD
+#define FWD_MARK(i)
+#else
     INPC_PROF_DECL;
+#define FWD_MARK(i) INPC_PROF_MARK(i)
+#endif
     // the gather runs ahead of the blend: the record of batch b + 1 and the slot of batch b + 2 are in flight
     // while batch b is consumed
     uint32_t next_slot = 0u;
@@ -334,9 +343,9 @@ __global__ void __launch_bounds__(T* T)
         }
         if (begin + 2 * TT + tid < range.y) next_slot = inst_slots[begin + 2 * TT + tid];
         stage_instance<T, C, INFERENCE>(st, valid, h, f, tile_x0, tile_y0);
-        INPC_PROF_MARK(0);
+        FWD_MARK(0);
         __syncthreads();
-        INPC_PROF_MARK(1);
+        FWD_MARK(1);
 
         // ---- consume: this wave's list
         uint32_t total = 0;
@@ -350,7 +359,7 @@ __global__ void __launch_bounds__(T* T)
             uint32_t my_start, my_count, n_fragments;
             build_fragment_lists<NF>(qs, st.opacity[j], lf, my_start, my_count, n_fragments,
                                      [&](int) { return __uint_as_float(j); });
-            INPC_PROF_MARK(2);
+            FWD_MARK(2);
             if (n_fragments == 0u) continue;
             // ---- pixels with short lists: the reference's sequential walk (kernels.cu:281-299)
             if (my_count <= kLongList) {
@@ -374,7 +383,7 @@ __global__ void __launch_bounds__(T* T)
                     done = done || Tr < kTransmittanceThreshold;
                 }
             }
-            INPC_PROF_MARK(3);
+            FWD_MARK(3);
             // ---- pixels with long lists, one after the other, 64 fragments at a time over the wave
             uint64_t long_pixels = __ballot(my_count > kLongList);
             while (long_pixels) {
@@ -432,7 +441,7 @@ __global__ void __launch_bounds__(T* T)
                 }
             }
             wave_sync();
-            INPC_PROF_MARK(4);
+            FWD_MARK(4);
             // ---- instances: hand the blending weights of the fragments to the thread that owns the instance
             if (!INFERENCE) {
 #pragma unroll
@@ -444,10 +453,10 @@ __global__ void __launch_bounds__(T* T)
             const uint64_t finished = __ballot(done);
             if (lane == 0u) st.done[wave] = finished;
         }
-        INPC_PROF_MARK(2);
+        FWD_MARK(2);
         const bool all_done = __syncthreads_and(done) != 0;
-        INPC_PROF_MARK(5);
-#ifdef INPC_BLEND_PROFILE
+        FWD_MARK(5);
+#if defined(INPC_BLEND_PROFILE) && !defined(INPC_PROFILE_BACKWARD)
         ++prof_batches;
 #endif
         // ---- write: thread t owns staged instance t (kernels.cu:291-295)
@@ -467,7 +476,10 @@ __global__ void __launch_bounds__(T* T)
         }
         if (all_done) break;
     }
+#ifndef INPC_PROFILE_BACKWARD
     INPC_PROF_FLUSH;
+#endif
+#undef FWD_MARK
     if (inside) {
         const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
 #pragma unroll
@@ -526,6 +538,12 @@ __global__ void __launch_bounds__(T* T)
     __syncthreads();
 
     const uint2 range = ranges[tile];
+#ifdef INPC_PROFILE_BACKWARD
+    INPC_PROF_DECL;
+#define BWD_MARK(i) INPC_PROF_MARK(i)
+#else
+#define BWD_MARK(i)
+#endif
     uint32_t next_slot = 0u;
     Header h_next{};
     float f_next[C];
@@ -551,7 +569,9 @@ __global__ void __launch_bounds__(T* T)
         }
         if (begin + 2 * TT + tid < range.y) next_slot = inst_slots[begin + 2 * TT + tid];
         stage_instance<T, C, false>(st, valid, h, f, tile_x0, tile_y0);
+        BWD_MARK(0);
         __syncthreads();
+        BWD_MARK(1);
 
         // ---- consume: this wave's list
         uint32_t total = 0;
@@ -578,6 +598,7 @@ __global__ void __launch_bounds__(T* T)
                 for (int c = 0; c < C; ++c) d = fmaf(feat[c], s_grad[wave][c][lf.pixel[q]], d);
                 return d;
             });
+            BWD_MARK(2);
             if (n_fragments == 0u) continue;
             // ---- pixels with short lists: the sequential walk (kernels.cu:383-417)
             if (my_count <= kLongList) {
@@ -595,6 +616,7 @@ __global__ void __launch_bounds__(T* T)
                     done = done || Tr < kTransmittanceThreshold;
                 }
             }
+            BWD_MARK(3);
             // ---- pixels with long lists, one after the other, 64 fragments at a time over the wave
             uint64_t long_pixels = __ballot(my_count > kLongList);
             while (long_pixels) {
@@ -632,6 +654,7 @@ __global__ void __launch_bounds__(T* T)
                 }
             }
             wave_sync();
+            BWD_MARK(4);
             // ---- instances: hand {blending weight, d loss / d alpha} of the fragments to the instance's thread
 #pragma unroll
             for (int q = 0; q < NF; ++q)
@@ -641,7 +664,12 @@ __global__ void __launch_bounds__(T* T)
             const uint64_t finished = __ballot(done);
             if (lane == 0u) st.done[wave] = finished;
         }
+        BWD_MARK(2);
         const bool all_done = __syncthreads_and(done) != 0;
+        BWD_MARK(5);
+#if defined(INPC_PROFILE_BACKWARD) && defined(INPC_BLEND_PROFILE)
+        ++prof_batches;
+#endif
         // ---- write: thread t owns staged instance t: gradient of the point from its fragments in all quads
         if (valid) {
             float gf[C];
@@ -679,6 +707,10 @@ __global__ void __launch_bounds__(T* T)
         }
         if (all_done) break;
     }
+#ifdef INPC_PROFILE_BACKWARD
+    INPC_PROF_FLUSH;
+#endif
+#undef BWD_MARK
 }
 
 }  // namespace blend

@@ -17,7 +17,10 @@ namespace radix {
 
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / kWave;
-constexpr int kItems = 16;
+#ifndef INPC_RADIX_ITEMS
+#define INPC_RADIX_ITEMS 16
+#endif
+constexpr int kItems = INPC_RADIX_ITEMS;
 constexpr int kTile = kBlock * kItems;  // keys per block
 constexpr int kMaxBits = 8;
 constexpr int kRadix = 1 << kMaxBits;

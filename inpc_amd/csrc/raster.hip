@@ -2,7 +2,9 @@
 //
 // Pipeline (all on the caller's stream, counts stay on the device):
 //   k_bin_count      project every point and count the drawn ones per first touched tile
+//   k_bin_offsets    per tile: exclusive prefix of the counts over the chunks of points
 //   k_bin_scan       exclusive scan of the counts: start of every tile's record bin
+//   k_bin_coarse     tile of every 256th record slot (lets k_expand find a slot's tile with a short search)
 //   k_preprocess     project, cull, tile bounds, depth key, depth-digit histograms; the blend record of a
 //                    drawn point (screen position, opacity, point id, view features) is written into the
 //                    bin of its first tile (B/rasterization/src/bilinear/kernels.cu:11-84,106-184)
@@ -13,9 +15,10 @@
 //                    (kernels.cu:186-220, forward.cu:101-130)
 //   radix sort       stable sort of the instances by tile id (forward.cu:132-139)
 //   k_tile_ranges    [begin, end) of every tile (kernels.cu:222-239)
-//   k_blend_forward  front-to-back bilinear 2x2 splat blend, one block per tile
-//                    (kernels.cu:241-313,422-495)
-//   k_blend_backward replay of the blend with the saved final image (kernels.cu:315-420)
+//   k_tile_order     schedule of the blend blocks: tiles with the longest instance lists first
+//   blend.hpp        k_blend_forward: front-to-back bilinear 2x2 splat blend, one block per tile
+//                    (kernels.cu:241-313,422-495); k_blend_backward: replay of the blend with the saved
+//                    final image (kernels.cu:315-420)
 //   k_sh_backward    view-space feature gradient -> 36 fp16 SH coefficient gradients
 //                    (kernels.cu:86-104, sh_utils.cuh:44-62)
 //
@@ -189,17 +192,41 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
 }
 
 // table[c][t] <- sum of table[c'][t] over c' < c; total[t] <- sum over all chunks.
-__global__ void __launch_bounds__(kBlock) k_bin_offsets(uint32_t* __restrict__ table, uint32_t* __restrict__ total,
-                                                        uint32_t n_tiles) {
-    const uint32_t t = blockIdx.x * kBlock + threadIdx.x;
-    if (t >= n_tiles) return;
-    uint32_t run = 0;
-    for (int c = 0; c < kBinBlocks; ++c) {
-        const uint32_t v = table[(size_t)c * n_tiles + t];
-        table[(size_t)c * n_tiles + t] = run;
-        run += v;
+// A block owns 64 tiles (lane = tile); each of its 16 waves takes a run of consecutive chunks, keeps them in
+// registers, and gets the sum of the runs in front of it through LDS.
+constexpr int kOffsetWaves = 16;
+constexpr int kOffsetRun = kBinBlocks / kOffsetWaves;
+__global__ void __launch_bounds__(kOffsetWaves * kWave) k_bin_offsets(uint32_t* __restrict__ table,
+                                                                       uint32_t* __restrict__ total, uint32_t n_tiles) {
+    __shared__ uint32_t s_run[kOffsetWaves][kWave];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t t = blockIdx.x * kWave + lane;
+    const bool valid = t < n_tiles;
+    uint32_t v[kOffsetRun];
+    uint32_t sum = 0;
+    uint32_t* column = table + (size_t)wave * kOffsetRun * n_tiles + t;
+#pragma unroll
+    for (int c = 0; c < kOffsetRun; ++c) {
+        v[c] = valid ? column[(size_t)c * n_tiles] : 0u;
+        sum += v[c];
     }
-    total[t] = run;
+    s_run[wave][lane] = sum;
+    __syncthreads();
+    uint32_t run = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kOffsetWaves; ++w) {
+        const uint32_t r = s_run[w][lane];
+        if ((uint32_t)w < wave) run += r;
+        all += r;
+    }
+    if (valid) {
+#pragma unroll
+        for (int c = 0; c < kOffsetRun; ++c) {
+            column[(size_t)c * n_tiles] = run;
+            run += v[c];
+        }
+        if (wave == 0) total[t] = all;
+    }
 }
 
 // bin_start[t] = number of records in bins before t (n_tiles + 1 entries).
@@ -514,26 +541,7 @@ __global__ void __launch_bounds__(kScanBlock) k_tile_order(const uint2* __restri
     for (uint32_t t = tid; t < n_tiles; t += kScanBlock) order[atomicAdd(&s_bucket[bucket_of(t)], 1u)] = t;
 }
 
-// ---- blend -------------------------------------------------------------------------------------------------
-//
-// One block per tile, one thread per pixel (a wave always covers an 8x8 pixel quad). Only the
-// transmittance of a pixel has to be evaluated in depth order; everything else is done one thread per
-// instance, all lanes busy. A batch of kBatch instances goes through these phases (barriers between them):
-//   stage      thread j gathers the record of instance j, evaluates the reference's exact coverage test
-//              |s - centre| < 1 for the two tile columns and rows it can reach and ORs bit j into the
-//              column / row masks of the batch;
-//   count      a pixel's hits are the set bits of (column mask AND row mask): popcount, block scan ->
-//              start of every pixel's fragment list;
-//   place      thread j writes the alpha of each of its (at most four) fragments into the list of the
-//              pixel it covers, at the rank given by the popcount of that pixel's mask below bit j, so the
-//              list is in depth order;
-//   pixels     a pixel walks its contiguous list: blending weight = T * alpha, T *= 1 - alpha, early out;
-//              the weights replace the alphas in the list (this is the only sequential part);
-//   instances  thread j reads the weights of its fragments back and writes the point's result: a plain
-//              store when the point lies in one tile only, atomics when it straddles tiles.
-constexpr int kBatch = 256;             // instances staged per round
-constexpr int kWords = kBatch / kWave;  // 64-bit mask words per column / row
-constexpr int kFragments = kBatch * 4;  // an instance covers at most 2 x 2 pixels
+// ---- blend: helpers shared with blend.hpp ---------------------------------------------------------------------
 
 // View features of a record (they follow the 32-byte header), as C floats.
 template <int C, bool HALF>
@@ -559,18 +567,6 @@ __device__ __forceinline__ void load_record_features(float* dst, const char* __r
             dst[4 * q + 2] = __low2float(hi);
             dst[4 * q + 3] = __high2float(hi);
         }
-    }
-}
-
-// Pixel of thread `tid` inside a T x T tile: a wave always covers an 8x8 quad.
-template <int T>
-__device__ __forceinline__ void pixel_of_thread(uint32_t tid, int& lx, int& ly) {
-    const uint32_t lane = tid & 63u, wave = tid >> 6;
-    lx = (int)(lane & 7u);
-    ly = (int)(lane >> 3);
-    if (T == 16) {
-        lx += (int)(wave & 1u) * 8;
-        ly += (int)(wave >> 1) * 8;
     }
 }
 
@@ -603,248 +599,6 @@ __device__ __forceinline__ AxisCover cover_axis(float s, int tile_origin) {
     return a;
 }
 
-__device__ __forceinline__ void lds_add(float* p, float v) {
-    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-}
-
-template <int T>
-struct BatchMasks {
-    uint64_t col[T][kWords];
-    uint64_t row[T][kWords];
-};
-
-template <int T>
-__device__ __forceinline__ void clear_masks(BatchMasks<T>& m) {
-    for (uint32_t i = threadIdx.x; i < (uint32_t)(2 * T * kWords); i += T * T) (&m.col[0][0])[i] = 0ull;
-}
-
-template <int T>
-__device__ __forceinline__ void mark_coverage(BatchMasks<T>& m, uint32_t j, const AxisCover& ax, const AxisCover& ay) {
-    const uint32_t bit = 1u << (j & 31u), half = j >> 5;
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        if (ax.hit[k]) atomicOr((uint32_t*)&m.col[ax.first + k][0] + half, bit);
-        if (ay.hit[k]) atomicOr((uint32_t*)&m.row[ay.first + k][0] + half, bit);
-    }
-}
-
-// Number of hits of pixel (cx, cy) among the instances 0 .. j-1 of the batch. `word` = j / 64 must be
-// uniform over the wave and `lane` = j % 64.
-template <int T>
-__device__ __forceinline__ uint32_t hits_before(const BatchMasks<T>& m, int cx, int cy, uint32_t word) {
-    uint32_t rank = 0;
-    for (uint32_t w = 0; w < word; ++w) rank += (uint32_t)__popcll(m.col[cx][w] & m.row[cy][w]);
-    const uint64_t own = m.col[cx][word] & m.row[cy][word];
-    return rank + mask_rank(own);
-}
-
-template <int T>
-__device__ __forceinline__ uint32_t hits_total(const BatchMasks<T>& m, int cx, int cy, uint32_t n_words) {
-    uint32_t n = 0;
-    for (uint32_t w = 0; w < n_words; ++w) n += (uint32_t)__popcll(m.col[cx][w] & m.row[cy][w]);
-    return n;
-}
-
-// Exclusive scan of one value per thread over the block (threads in tid order); `total` gets the block sum.
-// Contains barriers: every thread of the block must call it.
-template <int TT>
-__device__ __forceinline__ uint32_t block_scan_exclusive(uint32_t v, uint32_t* s_wave_total, uint32_t& total) {
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    uint32_t incl = v;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t up = __shfl_up(incl, d, 64);
-        if (lane >= (uint32_t)d) incl += up;
-    }
-    if (TT == 64) {
-        total = __shfl(incl, 63, 64);
-        return incl - v;
-    }
-    __syncthreads();  // s_wave_total may still be read from the previous call
-    if (lane == 63) s_wave_total[wave] = incl;
-    __syncthreads();
-    uint32_t base = 0, sum = 0;
-#pragma unroll
-    for (int w = 0; w < TT / 64; ++w) {
-        const uint32_t c = s_wave_total[w];
-        if ((uint32_t)w < wave) base += c;
-        sum += c;
-    }
-    total = sum;
-    return base + incl - v;
-}
-
-// ---- long fragment lists ---------------------------------------------------------------------------------------
-// A pixel-sized cluster of points puts a large share of a batch on a handful of pixels; walking such a list
-// on the one lane that owns the pixel would keep the whole block waiting. Lists longer than kLongList are
-// therefore evaluated over the flat, pixel-sorted fragment array by all threads: the running transmittance
-// (and, backward, the running weighted sum) is a segmented scan, the weighted feature sum a segmented
-// reduction. The scan multiplies in tree order, not front to back, so for these lists the transmittance can
-// differ from a sequential product in the last bits; short lists keep the sequential evaluation.
-constexpr uint32_t kLongList = 24;
-
-struct SegItem {
-    bool flag;   // a segment starts at or before the end of the span this item stands for
-    float value; // op-combination of the trailing run of the span
-};
-
-template <bool MUL>
-__device__ __forceinline__ float seg_identity() { return MUL ? 1.0f : 0.0f; }
-
-template <bool MUL>
-__device__ __forceinline__ float seg_apply(float a, float b) { return MUL ? a * b : a + b; }
-
-template <bool MUL>
-__device__ __forceinline__ SegItem seg_combine(const SegItem& left, const SegItem& right) {
-    SegItem r;
-    r.flag = left.flag || right.flag;
-    r.value = right.flag ? right.value : seg_apply<MUL>(left.value, right.value);
-    return r;
-}
-
-// Exclusive segmented scan of n elements, four consecutive elements per thread and round.
-//   get(f, flag, value): head flag and value of element f
-//   put(f, exclusive):   op-combination of the elements of f's segment before f (identity at a head)
-// Every thread of the block must call it; s_item has TT / 64 entries.
-template <int TT, bool MUL, typename Get, typename Put>
-__device__ __forceinline__ void segmented_scan(uint32_t n, SegItem* s_item, Get get, Put put) {
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    SegItem round_carry{false, seg_identity<MUL>()};
-    for (uint32_t round_base = 0; round_base < n; round_base += 4 * TT) {
-        const uint32_t base = round_base + 4 * threadIdx.x;
-        bool flag[4];
-        float value[4], before[4];
-        bool broken[4];
-        SegItem mine{false, seg_identity<MUL>()};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            flag[i] = true;
-            value[i] = seg_identity<MUL>();
-            if (base + i < n) get(base + i, flag[i], value[i]);
-            if (flag[i]) {
-                mine.flag = true;
-                mine.value = seg_identity<MUL>();
-            }
-            before[i] = mine.value;
-            broken[i] = mine.flag;
-            mine.value = seg_apply<MUL>(mine.value, value[i]);
-        }
-        // inclusive scan of the thread items over the wave
-        SegItem incl = mine;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            SegItem left;
-            left.flag = __shfl_up((int)incl.flag, d, 64) != 0;
-            left.value = __shfl_up(incl.value, d, 64);
-            if (lane >= (uint32_t)d) incl = seg_combine<MUL>(left, incl);
-        }
-        SegItem excl;
-        excl.flag = __shfl_up((int)incl.flag, 1, 64) != 0;
-        excl.value = __shfl_up(incl.value, 1, 64);
-        if (lane == 0) excl = SegItem{false, seg_identity<MUL>()};
-        if (TT > 64) {
-            __syncthreads();
-            if (lane == 63) s_item[wave] = incl;
-            __syncthreads();
-        }
-        SegItem incoming = round_carry;
-        if (TT > 64) {
-#pragma unroll
-            for (int w = 0; w < TT / 64; ++w)
-                if ((uint32_t)w < wave) incoming = seg_combine<MUL>(incoming, s_item[w]);
-        }
-        incoming = seg_combine<MUL>(incoming, excl);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (base + i < n) put(base + i, broken[i] ? before[i] : seg_apply<MUL>(incoming.value, before[i]));
-        // carry into the next round: everything up to the end of this round
-        if (TT > 64) {
-#pragma unroll
-            for (int w = 0; w < TT / 64; ++w) round_carry = seg_combine<MUL>(round_carry, s_item[w]);
-        } else {
-            SegItem last;
-            last.flag = __shfl((int)incl.flag, 63, 64) != 0;
-            last.value = __shfl(incl.value, 63, 64);
-            round_carry = seg_combine<MUL>(round_carry, last);
-        }
-    }
-}
-
-// Front-to-back walk over the fragment list [begin, end) of one pixel: alpha[f] is replaced by the blending
-// weight T * alpha, T is updated, and the walk stops behind the fragment that takes T below the threshold
-// (B/rasterization/src/bilinear/kernels.cu:289-299); fragments behind it get weight 0.
-// The alphas of eight fragments are fetched together so that the chain does not pay one LDS round trip each.
-__device__ __forceinline__ void transmittance_chain(float* alpha, uint32_t begin, uint32_t end, float& Tr, bool& done) {
-    constexpr int kAhead = 8;
-    for (uint32_t f = begin; f < end; f += kAhead) {
-        float a[kAhead];
-#pragma unroll
-        for (int i = 0; i < kAhead; ++i) a[i] = alpha[min(f + i, end - 1)];
-        // No branches in the chain: a fragment behind the end of the list or behind the early out gets
-        // alpha 0, which leaves T untouched and makes its blending weight 0.
-#pragma unroll
-        for (int i = 0; i < kAhead; ++i) {
-            const bool live = f + i < end && !done;
-            const float ai = live ? a[i] : 0.0f;
-            a[i] = Tr * ai;
-            Tr *= 1.0f - ai;
-            done = done || (live && Tr < kTransmittanceThreshold);
-        }
-#pragma unroll
-        for (int i = 0; i < kAhead; ++i)
-            if (f + i < end) alpha[f + i] = a[i];
-    }
-}
-
-// A pixel-sized cluster of points puts a large share of a batch on a handful of pixels. Their weighted
-// feature sums are not left to the single lanes that own those pixels: every thread of the block takes four
-// consecutive fragments of the flat, pixel-sorted list, adds up the ones that belong to a long list, and
-// adds the partial sum to the pixel's accumulator in LDS (a few float atomics per thread).
-template <int TT, int C, bool WITH_DEPTH>
-__device__ __forceinline__ void sum_long_lists(const float* alpha, const uint16_t* instance, const uint8_t* pixel_of,
-                                               const uint16_t* count, const float4* feat, const float* depth,
-                                               uint32_t n_fragments, float* acc, float* dacc) {
-    for (uint32_t base = 4 * threadIdx.x; base < n_fragments; base += 4 * TT) {
-        float part[C];
-        float dpart = 0.0f;
-        int current = -1;
-#pragma unroll
-        for (int i = 0; i < 5; ++i) {
-            int pix = -1;
-            float bw = 0.0f;
-            uint32_t j = 0;
-            if (i < 4 && base + i < n_fragments) {
-                const int p = pixel_of[base + i];
-                bw = alpha[base + i];
-                j = instance[base + i];
-                if (count[p] > kLongList && bw != 0.0f) pix = p;
-            }
-            if (pix != current) {
-                if (current >= 0) {
-#pragma unroll
-                    for (int c = 0; c < C; ++c) lds_add(&acc[c * TT + current], part[c]);
-                    if (WITH_DEPTH) lds_add(&dacc[current], dpart);
-                }
-                current = pix;
-#pragma unroll
-                for (int c = 0; c < C; ++c) part[c] = 0.0f;
-                dpart = 0.0f;
-            }
-            if (pix >= 0) {
-#pragma unroll
-                for (int q4 = 0; q4 < C / 4; ++q4) {
-                    const float4 v = feat[j * (C / 4) + q4];
-                    part[4 * q4] = fmaf(bw, v.x, part[4 * q4]);
-                    part[4 * q4 + 1] = fmaf(bw, v.y, part[4 * q4 + 1]);
-                    part[4 * q4 + 2] = fmaf(bw, v.z, part[4 * q4 + 2]);
-                    part[4 * q4 + 3] = fmaf(bw, v.w, part[4 * q4 + 3]);
-                }
-                if (WITH_DEPTH) dpart = fmaf(bw, depth[j], dpart);
-            }
-        }
-    }
-}
-
 #ifdef INPC_BLEND_PROFILE
 // development aid: per-phase shader clocks of k_blend_forward, summed over blocks (thread 0 of each)
 __device__ unsigned long long g_blend_profile[8];
@@ -869,494 +623,6 @@ __device__ unsigned long long g_blend_profile[8];
 #endif
 
 #include "blend.hpp"
-
-template <int T, int C, bool HALF, bool INFERENCE>
-__global__ void __launch_bounds__(T* T)
-    k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ inst_slots,
-                    const char* __restrict__ records, uint32_t stride, float* __restrict__ image,
-                    float* __restrict__ alpha_image, float* blending_weights, float* __restrict__ depth_image, int W,
-                    int H, uint32_t gw) {
-    constexpr int TT = T * T;
-    constexpr int NI = kBatch / TT;  // instances per thread and batch
-    __shared__ BatchMasks<T> s_masks;
-    __shared__ uint16_t s_start[TT], s_count[TT];      // fragment list of every pixel
-    __shared__ float s_alpha[kFragments];              // alpha, then blending weight, per fragment in list order
-    __shared__ uint16_t s_instance[kFragments];        // batch index of the fragment's instance
-    __shared__ uint8_t s_pixel[kFragments];            // tile-local pixel of the fragment
-    __shared__ float4 s_feat[kBatch * (C / 4)];
-    __shared__ float s_depth[INFERENCE ? kBatch : 1];
-    __shared__ float s_acc[C * TT];                    // channel-major sums of the long lists
-    __shared__ float s_dacc[INFERENCE ? TT : 1];
-    __shared__ float s_t_in[TT], s_t_out[TT];          // transmittance of the pixels with long lists
-    __shared__ SegItem s_item[TT / 64];
-    __shared__ uint32_t s_wave_total[TT / 64 + 1];
-
-    const uint32_t tid = threadIdx.x, lane = tid & 63u;
-    const uint32_t tile = blockIdx.x;
-    const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
-    int lx, ly;
-    pixel_of_thread<T>(tid, lx, ly);
-    const int lp = ly * T + lx;
-    const int px = tile_x0 + lx, py = tile_y0 + ly;
-    const bool inside = px < W && py < H;
-
-    float F[C];
-#pragma unroll
-    for (int c = 0; c < C; ++c) {
-        F[c] = 0.0f;
-        s_acc[c * TT + lp] = 0.0f;
-    }
-    if (INFERENCE) s_dacc[lp] = 0.0f;
-    float D = 0.0f, Tr = 1.0f;
-    bool done = !inside;
-
-    const uint2 range = ranges[tile];
-    INPC_PROF_DECL;
-    for (uint32_t begin = range.x; begin < range.y; begin += kBatch) {
-        const uint32_t count = min((uint32_t)kBatch, range.y - begin);
-        const uint32_t n_words = (count + 63u) >> 6;
-        clear_masks<T>(s_masks);
-        __syncthreads();
-        INPC_PROF_MARK(0);
-        // ---- stage
-        float sx[NI], sy[NI], opacity[NI];
-        uint32_t point[NI];
-        bool multi[NI];
-#pragma unroll
-        for (int k = 0; k < NI; ++k) {
-            const uint32_t j = tid + k * TT;
-            sx[k] = sy[k] = opacity[k] = 0.0f;
-            point[k] = 0u;
-            multi[k] = false;
-            if (j < count) {
-                const char* record = records + (size_t)inst_slots[begin + j] * stride;
-                const float4 h0 = ((const float4*)record)[0];
-                const float4 h1 = ((const float4*)record)[1];
-                sx[k] = h0.x;
-                sy[k] = h0.y;
-                opacity[k] = h0.z;
-                point[k] = __float_as_uint(h0.w);
-                multi[k] = ((__float_as_uint(h1.x) >> 16) & 3u) != 0u;
-                float f[C];
-                load_record_features<C, HALF>(f, record);
-#pragma unroll
-                for (int q = 0; q < C / 4; ++q) s_feat[j * (C / 4) + q] = make_float4(f[4 * q], f[4 * q + 1], f[4 * q + 2], f[4 * q + 3]);
-                if (INFERENCE) s_depth[j] = h1.y;
-                mark_coverage<T>(s_masks, j, cover_axis<T>(h0.x, tile_x0), cover_axis<T>(h0.y, tile_y0));
-            }
-        }
-        __syncthreads();
-        INPC_PROF_MARK(1);
-        // ---- count: fragment list of every live pixel
-        const uint32_t my_count = done ? 0u : hits_total<T>(s_masks, lx, ly, n_words);
-        uint32_t n_fragments;
-        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total, n_fragments);
-        if (n_fragments == 0u) {  // every instance of the batch falls on finished pixels only
-            if (__syncthreads_and(done)) break;
-            continue;
-        }
-        s_start[lp] = (uint16_t)my_start;
-        s_count[lp] = (uint16_t)my_count;
-        s_t_in[lp] = Tr;
-        const bool any_long = __syncthreads_or(my_count > kLongList) != 0;
-#ifdef INPC_BLEND_PROFILE
-        {
-            __shared__ uint32_t s_prof_max;
-            if (tid == 0) s_prof_max = 0u;
-            __syncthreads();
-            atomicMax(&s_prof_max, my_count);
-            __syncthreads();
-            if (tid == 0) atomicAdd(&g_blend_profile[7], (unsigned long long)n_fragments);
-        }
-#endif
-        __syncthreads();
-        INPC_PROF_MARK(2);
-        // ---- place: alpha of every fragment into its pixel's list, in depth order
-        uint32_t where[NI][4];
-        float weight[NI][4];
-#pragma unroll
-        for (int k = 0; k < NI; ++k) {
-            const uint32_t j = tid + k * TT;
-            const AxisCover ax = cover_axis<T>(sx[k], tile_x0), ay = cover_axis<T>(sy[k], tile_y0);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                where[k][q] = 0xFFFFFFFFu;
-                weight[k][q] = ax.weight[q & 1] * ay.weight[q >> 1];
-                if (j < count && ax.hit[q & 1] && ay.hit[q >> 1]) {
-                    const int cx = ax.first + (q & 1), cy = ay.first + (q >> 1);
-                    const int pix = cy * T + cx;
-                    if (s_count[pix] != 0) {  // 0: the pixel is finished (it has this hit at least)
-                        const uint32_t pos = s_start[pix] + hits_before<T>(s_masks, cx, cy, j >> 6);
-                        where[k][q] = pos;
-                        s_alpha[pos] = opacity[k] * weight[k][q];
-                        s_instance[pos] = (uint16_t)j;
-                        s_pixel[pos] = (uint8_t)pix;
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        INPC_PROF_MARK(3);
-        // ---- pixels: the sequential part touches the alphas only ...
-        const uint32_t end = my_start + my_count;
-        if (my_count != 0u && my_count <= kLongList) transmittance_chain(s_alpha, my_start, end, Tr, done);
-        if (any_long) {
-            // ... and for long lists it is a segmented product over the flat fragment array
-            segmented_scan<TT, true>(
-                n_fragments, s_item,
-                [&](uint32_t f, bool& flag, float& value) {
-                    const uint32_t p = s_pixel[f];
-                    const bool is_long = s_count[p] > kLongList;
-                    flag = !is_long || f == s_start[p];
-                    value = is_long ? 1.0f - s_alpha[f] : 1.0f;
-                },
-                [&](uint32_t f, float exclusive) {
-                    const uint32_t p = s_pixel[f];
-                    if (s_count[p] <= kLongList) return;
-                    const float a = s_alpha[f];
-                    const float t_before = s_t_in[p] * exclusive;
-                    const float t_after = t_before * (1.0f - a);
-                    const bool live = !(t_before < kTransmittanceThreshold);
-                    s_alpha[f] = live ? t_before * a : 0.0f;
-                    const bool last = f + 1 == (uint32_t)s_start[p] + s_count[p];
-                    // exactly one fragment hands the final transmittance back: the one that ends the walk
-                    if (live && (t_after < kTransmittanceThreshold || last)) s_t_out[p] = t_after;
-                });
-            __syncthreads();
-            if (my_count > kLongList) {
-                Tr = s_t_out[lp];
-                done = Tr < kTransmittanceThreshold;
-            }
-        }
-#ifdef INPC_BLEND_PROFILE
-        __syncthreads();
-        INPC_PROF_MARK(4);
-#endif
-        // ... the weighted feature sum has no dependence between its terms. A pixel with a short list sums
-        // it alone, four fragments per round with all loads of a round in flight together.
-        if (my_count <= kLongList) {
-            for (uint32_t f = my_start; f < end; f += 4) {
-                float bw[4];
-                uint32_t jj[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t g = min(f + i, end - 1);
-                    bw[i] = f + i < end ? s_alpha[g] : 0.0f;
-                    jj[i] = s_instance[g];
-                }
-                float4 v[4][C / 4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int q4 = 0; q4 < C / 4; ++q4) v[i][q4] = s_feat[jj[i] * (C / 4) + q4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-#pragma unroll
-                    for (int q4 = 0; q4 < C / 4; ++q4) {
-                        F[4 * q4] = fmaf(bw[i], v[i][q4].x, F[4 * q4]);
-                        F[4 * q4 + 1] = fmaf(bw[i], v[i][q4].y, F[4 * q4 + 1]);
-                        F[4 * q4 + 2] = fmaf(bw[i], v[i][q4].z, F[4 * q4 + 2]);
-                        F[4 * q4 + 3] = fmaf(bw[i], v[i][q4].w, F[4 * q4 + 3]);
-                    }
-                    if (INFERENCE) D = fmaf(bw[i], s_depth[jj[i]], D);
-                }
-            }
-        }
-        __syncthreads();  // all blending weights are in place
-        if (any_long)
-            sum_long_lists<TT, C, INFERENCE>(s_alpha, s_instance, s_pixel, s_count, s_feat, s_depth, n_fragments,
-                                             s_acc, s_dacc);
-        __syncthreads();
-        INPC_PROF_MARK(5);
-        // ---- instances: blending weights of the points (B/rasterization/src/bilinear/kernels.cu:291-295)
-        if (!INFERENCE) {
-#pragma unroll
-            for (int k = 0; k < NI; ++k) {
-                const uint32_t j = tid + k * TT;
-                if (j >= count) continue;
-                float weight_sum = 0.0f;
-                bool any = false;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if (where[k][q] == 0xFFFFFFFFu) continue;
-                    const float bw = s_alpha[where[k][q]];
-                    if (bw > 0.0f) {
-                        weight_sum = fmaf(bw, weight[k][q], weight_sum);
-                        any = true;
-                    }
-                }
-                if (!any) continue;
-                if (multi[k]) atomicAdd(&blending_weights[point[k]], weight_sum);
-                else blending_weights[point[k]] = weight_sum;
-            }
-        }
-#ifdef INPC_BLEND_PROFILE
-        ++prof_batches;
-#endif
-        const bool all_done = __syncthreads_and(done);
-        INPC_PROF_MARK(0);
-        if (all_done) break;
-    }
-    INPC_PROF_FLUSH;
-    __syncthreads();
-    if (inside) {
-        const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
-#pragma unroll
-        for (int c = 0; c < C; ++c) image[c * n_pixels + pix] = F[c] + s_acc[c * TT + lp];
-        const float alpha_px = 1.0f - Tr;
-        alpha_image[pix] = Tr < kTransmittanceThreshold ? 1.0f : alpha_px;
-        if (INFERENCE) depth_image[pix] = alpha_px > 0.0f ? (D + s_dacc[lp]) / alpha_px : 0.0f;
-    }
-    (void)lane;
-}
-
-// Backward. With s = features . grad of a fragment, R the running sum of weight x s of a pixel and S its
-// final value image . grad, the opacity gradient of the reference (kernels.cu:405-413),
-//   dot(T f + (F_running - F_final) / (1 - a), grad) + grad_alpha (1 - alpha_final) / (1 - a),
-// is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the pixel loop carries two scalars, not 2C.
-template <int T, int C, bool HALF>
-__global__ void __launch_bounds__(T* T)
-    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
-                     const uint32_t* __restrict__ inst_slots, const char* __restrict__ records, uint32_t stride,
-                     const float* __restrict__ grad_image,
-                     const float* __restrict__ grad_alpha, const float* __restrict__ image,
-                     const float* __restrict__ alpha_image, float* grad_view, float* grad_opacities, int W, int H,
-                     uint32_t gw) {
-    constexpr int TT = T * T;
-    constexpr int NI = kBatch / TT;
-    __shared__ BatchMasks<T> s_masks;
-    __shared__ uint16_t s_start[TT], s_count[TT];
-    __shared__ float s_alpha[kFragments];   // alpha, then blending weight
-    __shared__ float s_dot[kFragments];     // features . grad, then d(loss)/d(alpha)
-    __shared__ float s_grad[C * TT];        // channel-major upstream gradient of the tile (0 outside the image)
-    __shared__ float s_tb[kFragments];      // long lists: transmittance in front of the fragment (0: not reached)
-    __shared__ uint8_t s_pixel[kFragments];
-    __shared__ float s_t_in[TT], s_t_out[TT], s_r_in[TT], s_r_out[TT], s_offset[TT];
-    __shared__ SegItem s_item[TT / 64];
-    __shared__ uint32_t s_wave_total[TT / 64 + 1];
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t tile = tile_order[blockIdx.x];
-    const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
-    int lx, ly;
-    pixel_of_thread<T>(tid, lx, ly);
-    const int lp = ly * T + lx;
-    const int px = tile_x0 + lx, py = tile_y0 + ly;
-    const bool inside = px < W && py < H;
-
-    float final_dot = 0.0f, common = 0.0f;
-    {
-        const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
-#pragma unroll
-        for (int c = 0; c < C; ++c) {
-            const float g = inside ? grad_image[c * n_pixels + pix] : 0.0f;
-            s_grad[c * TT + lp] = g;
-            if (inside) final_dot = fmaf(image[c * n_pixels + pix], g, final_dot);
-        }
-        if (inside) common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
-    }
-    const float offset = common - final_dot;
-    float Tr = 1.0f, running = 0.0f;
-    bool done = !inside;
-
-    const uint2 range = ranges[tile];
-    for (uint32_t begin = range.x; begin < range.y; begin += kBatch) {
-        const uint32_t count = min((uint32_t)kBatch, range.y - begin);
-        const uint32_t n_words = (count + 63u) >> 6;
-        clear_masks<T>(s_masks);
-        __syncthreads();  // also orders s_grad before its first use
-        // ---- stage
-        float sx[NI], sy[NI], opacity[NI];
-        float feat[NI][C];
-        uint32_t point[NI];
-        bool multi[NI];
-#pragma unroll
-        for (int k = 0; k < NI; ++k) {
-            const uint32_t j = tid + k * TT;
-            sx[k] = sy[k] = opacity[k] = 0.0f;
-            point[k] = 0u;
-            multi[k] = false;
-            if (j < count) {
-                const char* record = records + (size_t)inst_slots[begin + j] * stride;
-                const float4 h0 = ((const float4*)record)[0];
-                const float4 h1 = ((const float4*)record)[1];
-                sx[k] = h0.x;
-                sy[k] = h0.y;
-                opacity[k] = h0.z;
-                point[k] = __float_as_uint(h0.w);
-                multi[k] = ((__float_as_uint(h1.x) >> 16) & 3u) != 0u;
-                load_record_features<C, HALF>(feat[k], record);
-                mark_coverage<T>(s_masks, j, cover_axis<T>(h0.x, tile_x0), cover_axis<T>(h0.y, tile_y0));
-            }
-        }
-        __syncthreads();
-        // ---- count
-        const uint32_t my_count = done ? 0u : hits_total<T>(s_masks, lx, ly, n_words);
-        uint32_t n_fragments;
-        const uint32_t my_start = block_scan_exclusive<TT>(my_count, s_wave_total, n_fragments);
-        if (n_fragments == 0u) {  // every instance of the batch falls on finished pixels only
-            if (__syncthreads_and(done)) break;
-            continue;
-        }
-        s_start[lp] = (uint16_t)my_start;
-        s_count[lp] = (uint16_t)my_count;
-        s_t_in[lp] = Tr;
-        s_r_in[lp] = running;
-        s_offset[lp] = offset;
-        const bool any_long = __syncthreads_or(my_count > kLongList) != 0;
-        // ---- place: alpha and features . grad of every fragment
-        uint32_t where[NI][4];
-        float weight[NI][4];
-#pragma unroll
-        for (int k = 0; k < NI; ++k) {
-            const uint32_t j = tid + k * TT;
-            const AxisCover ax = cover_axis<T>(sx[k], tile_x0), ay = cover_axis<T>(sy[k], tile_y0);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                where[k][q] = 0xFFFFFFFFu;
-                weight[k][q] = ax.weight[q & 1] * ay.weight[q >> 1];
-                if (j < count && ax.hit[q & 1] && ay.hit[q >> 1]) {
-                    const int cx = ax.first + (q & 1), cy = ay.first + (q >> 1);
-                    const int pix = cy * T + cx;
-                    if (s_count[pix] != 0) {
-                        const uint32_t pos = s_start[pix] + hits_before<T>(s_masks, cx, cy, j >> 6);
-                        where[k][q] = pos;
-                        s_alpha[pos] = opacity[k] * weight[k][q];
-                        s_pixel[pos] = (uint8_t)pix;
-                        float d = 0.0f;
-#pragma unroll
-                        for (int c = 0; c < C; ++c) d = fmaf(feat[k][c], s_grad[c * TT + pix], d);
-                        s_dot[pos] = d;
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        // ---- pixels: the sequential part, without branches (a fragment behind the end of the list or
-        // behind the early out gets alpha 0: T stays, its weight and gradient are 0)
-        if (my_count != 0u && my_count <= kLongList) {
-            constexpr int kAhead = 4;
-            const uint32_t end = my_start + my_count;
-            for (uint32_t f = my_start; f < end; f += kAhead) {
-                float a[kAhead], sd[kAhead];
-#pragma unroll
-                for (int i = 0; i < kAhead; ++i) {
-                    a[i] = s_alpha[min(f + i, end - 1)];
-                    sd[i] = s_dot[min(f + i, end - 1)];
-                }
-#pragma unroll
-                for (int i = 0; i < kAhead; ++i) {
-                    const bool live = f + i < end && !done;
-                    const float ai = live ? a[i] : 0.0f;
-                    const float bw = Tr * ai;
-                    const float one_minus_a = 1.0f - ai;
-                    const float rcp = __frcp_rn(fmaxf(one_minus_a, kOneMinusAlphaEps));
-                    running = fmaf(bw, sd[i], running);
-                    a[i] = bw;
-                    sd[i] = live ? fmaf(Tr, sd[i], (running + offset) * rcp) : 0.0f;
-                    Tr *= one_minus_a;
-                    done = done || (live && Tr < kTransmittanceThreshold);
-                }
-#pragma unroll
-                for (int i = 0; i < kAhead; ++i) {
-                    if (f + i < end) {
-                        s_alpha[f + i] = a[i];
-                        s_dot[f + i] = sd[i];
-                    }
-                }
-            }
-        }
-        if (any_long) {
-            // long lists: transmittance as a segmented product over the flat fragment array ...
-            segmented_scan<TT, true>(
-                n_fragments, s_item,
-                [&](uint32_t f, bool& flag, float& value) {
-                    const uint32_t p = s_pixel[f];
-                    const bool is_long = s_count[p] > kLongList;
-                    flag = !is_long || f == s_start[p];
-                    value = is_long ? 1.0f - s_alpha[f] : 1.0f;
-                },
-                [&](uint32_t f, float exclusive) {
-                    const uint32_t p = s_pixel[f];
-                    if (s_count[p] <= kLongList) return;
-                    const float t_before = s_t_in[p] * exclusive;
-                    const float t_after = t_before * (1.0f - s_alpha[f]);
-                    const bool live = !(t_before < kTransmittanceThreshold);
-                    s_tb[f] = live ? t_before : 0.0f;
-                    const bool last = f + 1 == (uint32_t)s_start[p] + s_count[p];
-                    if (live && (t_after < kTransmittanceThreshold || last)) s_t_out[p] = t_after;
-                });
-            __syncthreads();
-            // ... then the running weighted sum as a segmented sum, and the gradient of every fragment
-            segmented_scan<TT, false>(
-                n_fragments, s_item,
-                [&](uint32_t f, bool& flag, float& value) {
-                    const uint32_t p = s_pixel[f];
-                    const bool is_long = s_count[p] > kLongList;
-                    flag = !is_long || f == s_start[p];
-                    value = is_long ? (s_tb[f] * s_alpha[f]) * s_dot[f] : 0.0f;
-                },
-                [&](uint32_t f, float exclusive) {
-                    const uint32_t p = s_pixel[f];
-                    if (s_count[p] <= kLongList) return;
-                    const float a = s_alpha[f], sd = s_dot[f], t_before = s_tb[f];
-                    const float bw = t_before * a;
-                    const float run = (s_r_in[p] + exclusive) + bw * sd;
-                    const float rcp = __frcp_rn(fmaxf(1.0f - a, kOneMinusAlphaEps));
-                    s_alpha[f] = bw;
-                    s_dot[f] = t_before != 0.0f ? fmaf(t_before, sd, (run + s_offset[p]) * rcp) : 0.0f;
-                    if (f + 1 == (uint32_t)s_start[p] + s_count[p]) s_r_out[p] = run;
-                });
-            __syncthreads();
-            if (my_count > kLongList) {
-                Tr = s_t_out[lp];
-                running = s_r_out[lp];
-                done = Tr < kTransmittanceThreshold;
-            }
-        }
-        __syncthreads();
-        // ---- instances: gradient of the point
-#pragma unroll
-        for (int k = 0; k < NI; ++k) {
-            const uint32_t j = tid + k * TT;
-            if (j >= count) continue;
-            const AxisCover ax = cover_axis<T>(sx[k], tile_x0), ay = cover_axis<T>(sy[k], tile_y0);
-            float gf[C];
-#pragma unroll
-            for (int c = 0; c < C; ++c) gf[c] = 0.0f;
-            float gop = 0.0f;
-            bool any_weight = false;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                if (where[k][q] == 0xFFFFFFFFu) continue;
-                const float bw = s_alpha[where[k][q]];
-                gop = fmaf(s_dot[where[k][q]], weight[k][q], gop);
-                if (bw > 0.0f) {
-                    any_weight = true;
-                    const int pix = (ay.first + (q >> 1)) * T + ax.first + (q & 1);
-#pragma unroll
-                    for (int c = 0; c < C; ++c) gf[c] = fmaf(bw, s_grad[c * TT + pix], gf[c]);
-                }
-            }
-            if (!any_weight && gop == 0.0f) continue;
-            float* dst = grad_view + (size_t)point[k] * C;
-            if (multi[k]) {
-                if (any_weight) {
-#pragma unroll
-                    for (int c = 0; c < C; ++c)
-                        if (gf[c] != 0.0f) atomicAdd(dst + c, gf[c]);
-                }
-                if (gop != 0.0f) atomicAdd(&grad_opacities[point[k]], gop);
-            } else {
-#pragma unroll
-                for (int q4 = 0; q4 < C / 4; ++q4)
-                    ((float4*)dst)[q4] = make_float4(gf[4 * q4], gf[4 * q4 + 1], gf[4 * q4 + 2], gf[4 * q4 + 3]);
-                grad_opacities[point[k]] = gop;
-            }
-        }
-        if (__syncthreads_and(done)) break;
-    }
-}
 
 // view-space feature gradient -> (N,36) fp16; a point that was not drawn has a zero view gradient and
 // gets zeros (kernels.cu:95)
@@ -1679,7 +945,7 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
     if (L.geo.n > 0) {
         rc = L.T == 8 ? launch_bin_count<8>(L, positions, w2c, ws, stream) : launch_bin_count<16>(L, positions, w2c, ws, stream);
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets, dim3(div_up(L.geo.n_tiles, kBlock)), dim3(kBlock), stream,
+        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets, dim3(div_up(L.geo.n_tiles, kWave)), dim3(kOffsetWaves * kWave), stream,
                     at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
         INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
                     (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start), L.geo.n_tiles);

@@ -138,7 +138,8 @@ class RasterRun:
         self.alpha = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device)
         self.bw = None if inference else torch.full((max(self.n, 1),), float("nan"), dtype=torch.float32, device=device)
         self.depth_image = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device) if inference else None
-        self.ws = torch.empty(self.layout.total_bytes, dtype=torch.uint8, device=device)
+        # poisoned: nothing may depend on what the workspace held before the call
+        self.ws = torch.randint(0, 256, (self.layout.total_bytes,), dtype=torch.uint8, device=device)
 
     def forward(self):
         _lib.check(self.lib.inpc_raster_forward(
