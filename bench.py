@@ -47,9 +47,10 @@ def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, depth_passes, tile
         "raster_bin_count": n * 12,
         "raster_preprocess": n * (16 + F) + v * (R + 8),
         "raster_depth_sort": v * 68 / max(depth_passes, 1),
-        "raster_expand": v * 36 + i * 6,
-        "raster_tile_sort": i * (2 + 12 * ((end_bit + 7) // 8)) / max(tile_passes, 1),
-        "raster_tile_ranges": i * 2,
+        # expansion reads + instance emission + tile sort + range scan of the reference structure, done here by
+        # raster_inst_count (reads the sort values once more) and raster_inst_emit
+        "raster_inst_count": v * 4,
+        "raster_inst_emit": v * 36 + i * (6 + 2 + 12 * ((end_bit + 7) // 8) + 2),
         "raster_blend_forward": i * (4 + R) + pixels * 4 * (channels + 1) + n * 4,
         "raster_blend_backward": i * (4 + R) + pixels * 8 * (channels + 1) + n * (4 * channels + 4),
         "fill_u32": n * (4 * channels + 4),

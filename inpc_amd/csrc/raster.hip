@@ -4,17 +4,16 @@
 //   k_bin_count      project every point and count the drawn ones per first touched tile
 //   k_bin_offsets    per tile: exclusive prefix of the counts over the chunks of points
 //   k_bin_scan       exclusive scan of the counts: start of every tile's record bin
-//   k_bin_coarse     tile of every 256th record slot (lets k_expand find a slot's tile with a short search)
+//   k_bin_coarse     tile of every 256th record slot (a slot's tile is then found with a short search)
 //   k_preprocess     project, cull, tile bounds, depth key, depth-digit histograms; the blend record of a
 //                    drawn point (screen position, opacity, point id, view features) is written into the
 //                    bin of its first tile (B/rasterization/src/bilinear/kernels.cu:11-84,106-184)
 //   radix sort       stable sort of the drawn points by depth key; the first pass drops the culled
 //                    points, ties keep ascending point id (forward.cu:91-98)
-//   k_expand         per depth-sorted point: instance offsets (single-pass scan) and one
-//                    (tile, record slot) instance per touched tile, row-major; tile-digit histograms
-//                    (kernels.cu:186-220, forward.cu:101-130)
-//   radix sort       stable sort of the instances by tile id (forward.cu:132-139)
-//   k_tile_ranges    [begin, end) of every tile (kernels.cu:222-239)
+//   instances.hpp    depth-ordered points -> every tile's instances in depth order and its [begin, end):
+//                    per-chunk instance counts per tile, prefix sums, then a block per chunk sorts a few
+//                    thousand instances by tile inside LDS and appends the runs at the tiles' cursors
+//                    (kernels.cu:186-239, forward.cu:101-143)
 //   k_tile_order     schedule of the blend blocks: tiles with the longest instance lists first
 //   blend.hpp        k_blend_forward: front-to-back bilinear 2x2 splat blend, one block per tile
 //                    (kernels.cu:241-313,422-495); k_blend_backward: replay of the blend with the saved
@@ -50,8 +49,6 @@ enum Counter : int {
     kCntInstances = 1,
     kCntError = 2,
     kCntTicketDepth = 4,   // 4 words
-    kCntTicketTile = 8,    // 4 words
-    kCntTicketExpand = 12,
     kCntWords = 16
 };
 
@@ -195,9 +192,10 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
 // A block owns 64 tiles (lane = tile); each of its 16 waves takes a run of consecutive chunks, keeps them in
 // registers, and gets the sum of the runs in front of it through LDS.
 constexpr int kOffsetWaves = 16;
-constexpr int kOffsetRun = kBinBlocks / kOffsetWaves;
+template <int ROWS>
 __global__ void __launch_bounds__(kOffsetWaves * kWave) k_bin_offsets(uint32_t* __restrict__ table,
                                                                        uint32_t* __restrict__ total, uint32_t n_tiles) {
+    constexpr int kOffsetRun = ROWS / kOffsetWaves;
     __shared__ uint32_t s_run[kOffsetWaves][kWave];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t t = blockIdx.x * kWave + lane;
@@ -342,10 +340,7 @@ __global__ void __launch_bounds__(kBinThreads)
     radix::hist_flush(s_hist, plan, g_hist);
 }
 
-// ---- instance expansion -----------------------------------------------------------------------------------
-constexpr int kExpandItems = 16;
-constexpr int kExpandTile = kBlock * kExpandItems;
-constexpr int kExpandStage = 6144;  // instances staged in LDS per output round
+// ---- record slot -> tile ------------------------------------------------------------------------------------------
 constexpr int kCoarseShift = 8;     // one coarse entry per 256 record slots
 
 inline uint32_t coarse_entries(uint32_t n) { return (n >> kCoarseShift) + 2u; }
@@ -374,129 +369,7 @@ __global__ void __launch_bounds__(kBlock) k_bin_coarse(const uint32_t* __restric
     coarse[b] = (uint16_t)t;
 }
 
-// Depth-ordered points -> instances (tile key, record slot), consecutive per point, row-major over the
-// touched tiles (B/rasterization/src/bilinear/kernels.cu:186-220). The exclusive sum of the per-point tile
-// counts is a single-pass scan (decoupled look-back); a block stages its run of instances in LDS and writes
-// it out with consecutive lanes on consecutive addresses.
-__global__ void __launch_bounds__(kBlock)
-    k_expand(const uint32_t* __restrict__ depth_order, const uint32_t* __restrict__ bin_start,
-             const uint16_t* __restrict__ coarse, uint16_t* __restrict__ inst_keys, uint32_t* __restrict__ inst_points,
-             uint32_t* counters, uint32_t* status, uint32_t* g_hist, uint32_t gw, uint32_t n_tiles,
-             radix::DevicePlan plan) {
-    __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
-    __shared__ uint32_t s_wave[kBlock / kWave];
-    __shared__ uint32_t s_bid, s_exclusive;
-    __shared__ uint32_t s_slot[kExpandStage];
-    __shared__ uint16_t s_tile[kExpandStage];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    for (int i = tid; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
-    if (tid == 0) s_bid = atomicAdd(&counters[kCntTicketExpand], 1u);
-    __syncthreads();
-    const uint32_t bid = s_bid;
-    const uint32_t n_visible = counters[kCntVisible];
-    const uint64_t block_first = (uint64_t)bid * kExpandTile;
-    if (block_first >= n_visible) return;
-    const uint64_t first = block_first + (uint64_t)tid * kExpandItems;
-
-    uint32_t val[kExpandItems];
-    if (block_first + kExpandTile <= n_visible) {
-        const uint4* src = (const uint4*)(depth_order + first);
-#pragma unroll
-        for (int q = 0; q < kExpandItems / 4; ++q) {
-            const uint4 v = src[q];
-            val[4 * q] = v.x;
-            val[4 * q + 1] = v.y;
-            val[4 * q + 2] = v.z;
-            val[4 * q + 3] = v.w;
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < kExpandItems; ++j) val[j] = first + j < n_visible ? depth_order[first + j] : 0xFFFFFFFFu;
-    }
-    // 0xFFFFFFFF marks a slot behind the end: record slots stay below 2^28
-    uint32_t mine = 0;
-#pragma unroll
-    for (int j = 0; j < kExpandItems; ++j)
-        if (val[j] != 0xFFFFFFFFu) mine += ((val[j] & 1u) + 1u) * (((val[j] >> 1) & 1u) + 1u);
-    // the tile of every point's first instance: two neighbouring coarse entries bound a short search
-    uint16_t tile0[kExpandItems];
-#pragma unroll
-    for (int j = 0; j < kExpandItems; ++j) {
-        tile0[j] = 0;
-        if (val[j] != 0xFFFFFFFFu) {
-            const uint32_t slot = val[j] >> 2, b = slot >> kCoarseShift;
-            tile0[j] = (uint16_t)tile_of_slot(bin_start, coarse[b], (uint32_t)coarse[b + 1] + 1u, slot);
-        }
-    }
-    // block exclusive scan of `mine`
-    uint32_t incl = mine;
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s, 64);
-        if (lane >= (uint32_t)s) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t wave_off = 0, block_total = 0;
-#pragma unroll
-    for (int w = 0; w < kBlock / kWave; ++w) {
-        const uint32_t c = s_wave[w];
-        if ((uint32_t)w < wave) wave_off += c;
-        block_total += c;
-    }
-    if (wave == 0) {
-        const uint32_t exclusive = lookback_exclusive_wave(status, bid, block_total, &counters[kCntError]);
-        if (lane == 0) s_exclusive = exclusive;
-    }
-    const uint32_t local_first = wave_off + incl - mine;  // of this thread's first instance inside the block's run
-    for (uint32_t round = 0; round < block_total; round += kExpandStage) {
-        uint32_t local = local_first;
-#pragma unroll
-        for (int j = 0; j < kExpandItems; ++j) {
-            if (val[j] == 0xFFFFFFFFu) continue;
-            const uint32_t slot = val[j] >> 2, nx = (val[j] & 1u) + 1u, ny = ((val[j] >> 1) & 1u) + 1u;
-            for (uint32_t dy = 0; dy < ny; ++dy)
-                for (uint32_t dx = 0; dx < nx; ++dx) {
-                    const uint32_t at = local - round;  // wraps below the round: fails the test as well
-                    if (at < (uint32_t)kExpandStage) {
-                        s_tile[at] = (uint16_t)(tile0[j] + dy * gw + dx);
-                        s_slot[at] = slot;
-                    }
-                    ++local;
-                }
-        }
-        __syncthreads();  // staging complete (first round: s_exclusive too)
-        const uint32_t out = s_exclusive + round, n_out = min((uint32_t)kExpandStage, block_total - round);
-        for (uint32_t i = tid; i < n_out; i += kBlock) {
-            const uint32_t tile = s_tile[i];
-            inst_keys[out + i] = (uint16_t)tile;
-            inst_points[out + i] = s_slot[i];
-            radix::hist_add(s_hist, plan, tile);
-        }
-        __syncthreads();
-    }
-    radix::hist_flush(s_hist, plan, g_hist);
-}
-
-// ---- tile ranges (kernels.cu:222-239) ------------------------------------------------------------------------
-__global__ void __launch_bounds__(kBlock) k_tile_ranges(const uint16_t* __restrict__ inst_keys, uint2* ranges,
-                                                        const uint32_t* __restrict__ counters, uint32_t n_max) {
-    const uint32_t n = min(counters[kCntInstances], n_max);
-    const uint32_t stride = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-        const uint32_t t = inst_keys[i];
-        if (i == 0) {
-            ranges[t].x = 0u;
-        } else {
-            const uint32_t prev = inst_keys[i - 1];
-            if (prev != t) {
-                ranges[prev].y = i;
-                ranges[t].x = i;
-            }
-        }
-        if (i == n - 1) ranges[t].y = n;
-    }
-}
+#include "instances.hpp"
 
 // ---- tile schedule -----------------------------------------------------------------------------------------------
 // Blocks of the blend kernels take their tiles from this list: longest instance list first, so that the
@@ -659,16 +532,16 @@ __global__ void __launch_bounds__(kBlock) k_float_to_half(const float* __restric
 struct Layout {
     inpc_raster_layout pub;
     Geometry geo;
-    radix::PassPlan depth_plan, tile_plan;
+    radix::PassPlan depth_plan;
     int T, C, fmode;
     bool inference, sh, half_features;
     // private offsets
     size_t zero_begin, zero_words;  // region cleared at the start of every forward
-    size_t hist_depth, hist_tile, bases_depth, bases_tile;
-    size_t status_depth, status_tile, status_expand, bin_coarse;
-    size_t bin_table, bin_total, tile_order;
+    size_t hist_depth, bases_depth;
+    size_t status_depth, bin_coarse;
+    size_t bin_table, bin_total, tile_order, inst_start;
     size_t keys_a, keys_b, vals_a, vals_b;
-    size_t inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
+    size_t inst_keys_a, inst_vals_a;
 };
 
 uint32_t float_bits(float f) {
@@ -714,7 +587,6 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     }
     L.depth_plan = radix::make_plan(depth_bits);
     const int end_bit = bit_length(g.n_tiles - 1);
-    L.tile_plan = radix::make_plan(std::max(end_bit, 1));
 
     const size_t n = std::max<size_t>(g.n, 1), ni = 4 * n;
     size_t off = 0;
@@ -729,34 +601,28 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.zero_begin = off;
     P.counters = take(kCntWords * 4);
     L.hist_depth = take(radix::kMaxPasses * radix::kRadix * 4);
-    L.hist_tile = take(radix::kMaxPasses * radix::kRadix * 4);
     L.status_depth = take(L.depth_plan.n_passes * radix::status_words(g.n) * 4);
-    L.status_tile = take(L.tile_plan.n_passes * radix::status_words((uint32_t)std::min<size_t>(ni, 0xFFFFFFFFu)) * 4);
-    L.status_expand = take((size_t)div_up(g.n, kExpandTile) * 4 + 4);
     P.tile_ranges = take((size_t)g.n_tiles * 8);
     L.zero_words = (off - L.zero_begin) / 4;
-    L.bin_table = take((size_t)kBinBlocks * g.n_tiles * 4);
+    L.bin_table = take((size_t)std::max<int>(kBinBlocks, instances::kChunks) * g.n_tiles * 4);
     L.bin_total = take((size_t)g.n_tiles * 4);
     L.tile_order = take((size_t)g.n_tiles * 4);
+    L.inst_start = take((size_t)(g.n_tiles + 1) * 4);
     P.bin_start = take((size_t)(g.n_tiles + 1) * 4);
     L.bin_coarse = take((size_t)coarse_entries(g.n) * 2);
     L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
-    L.bases_tile = take(radix::kMaxPasses * radix::kRadix * 4);
     P.point_record = take(n * g.stride);
     L.keys_a = take(n * 4);
     L.keys_b = take(n * 4);
     L.vals_a = take(n * 4);
     L.vals_b = take(n * 4);
     L.inst_keys_a = take(ni * 2);
-    L.inst_keys_b = take(ni * 2);
     L.inst_vals_a = take(ni * 4);
-    L.inst_vals_b = take(ni * 4);
     const bool depth_in_a = (L.depth_plan.n_passes % 2) == 0;
     P.depth_keys = depth_in_a ? L.keys_a : L.keys_b;
     P.depth_order = depth_in_a ? L.vals_a : L.vals_b;
-    const bool tile_in_a = (L.tile_plan.n_passes % 2) == 0;
-    P.instance_keys = tile_in_a ? L.inst_keys_a : L.inst_keys_b;
-    P.instance_slots = tile_in_a ? L.inst_vals_a : L.inst_vals_b;
+    P.instance_keys = L.inst_keys_a;
+    P.instance_slots = L.inst_vals_a;
     P.total_bytes = off;
     P.record_stride = g.stride;
     P.grid_width = g.gw;
@@ -945,7 +811,7 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
     if (L.geo.n > 0) {
         rc = L.T == 8 ? launch_bin_count<8>(L, positions, w2c, ws, stream) : launch_bin_count<16>(L, positions, w2c, ws, stream);
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets, dim3(div_up(L.geo.n_tiles, kWave)), dim3(kOffsetWaves * kWave), stream,
+        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<kBinBlocks>, dim3(div_up(L.geo.n_tiles, kWave)), dim3(kOffsetWaves * kWave), stream,
                     at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
         INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
                     (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start), L.geo.n_tiles);
@@ -962,23 +828,28 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                                          at<uint32_t>(ws, L.status_depth), counters + kCntTicketDepth,
                                          counters + kCntError, stream, "raster_depth_sort");
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("raster_expand", k_expand, dim3(div_up(L.geo.n, kExpandTile)), dim3(kBlock), stream,
-                    (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order),
-                    (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
-                    (const uint16_t*)at<uint16_t>(ws, L.bin_coarse), at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), counters,
-                    at<uint32_t>(ws, L.status_expand), at<uint32_t>(ws, L.hist_tile), L.geo.gw, L.geo.n_tiles,
-                    radix::to_device_plan(L.tile_plan));
-        const uint32_t ni = 4u * L.geo.n;
-        rc = radix::sort_pairs<uint16_t>(L.tile_plan, radix::kPlain, at<uint16_t>(ws, L.inst_keys_a),
-                                         at<uint32_t>(ws, L.inst_vals_a), at<uint16_t>(ws, L.inst_keys_b),
-                                         at<uint32_t>(ws, L.inst_vals_b), counters + kCntInstances, ni,
-                                         at<uint32_t>(ws, L.hist_tile), at<uint32_t>(ws, L.bases_tile),
-                                         at<uint32_t>(ws, L.status_tile), counters + kCntTicketTile,
-                                         counters + kCntError, stream, "raster_tile_sort");
-        if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("raster_tile_ranges", k_tile_ranges, dim3(std::min<uint32_t>(div_up(ni, kBlock), 4096u)),
-                    dim3(kBlock), stream, (const uint16_t*)at<uint16_t>(ws, L.pub.instance_keys),
-                    at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)counters, ni);
+        {
+            // depth-ordered points -> per-tile instance lists (instances.hpp); the bin table is free again
+            const uint32_t* order = at<uint32_t>(ws, L.pub.depth_order);
+            const uint32_t* bin_start = at<uint32_t>(ws, L.pub.bin_start);
+            const uint16_t* coarse = at<uint16_t>(ws, L.bin_coarse);
+            INPC_LAUNCH_LDS("raster_inst_count", instances::k_inst_count, dim3(instances::kChunks), dim3(kBinThreads),
+                            (size_t)L.geo.n_tiles * 4, stream, order, bin_start, coarse, (const uint32_t*)counters,
+                            at<uint32_t>(ws, L.bin_table), L.geo.n, L.geo.gw, L.geo.n_tiles);
+            INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<instances::kChunks>, dim3(div_up(L.geo.n_tiles, kWave)),
+                        dim3(kOffsetWaves * kWave), stream, at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total),
+                        L.geo.n_tiles);
+            INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
+                        (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.inst_start), L.geo.n_tiles);
+            INPC_LAUNCH("raster_tile_ranges", instances::k_ranges_from_starts, dim3(div_up(L.geo.n_tiles, kBlock)),
+                        dim3(kBlock), stream, (const uint32_t*)at<uint32_t>(ws, L.inst_start),
+                        at<uint2>(ws, L.pub.tile_ranges), L.geo.n_tiles);
+            INPC_LAUNCH_LDS("raster_inst_emit", instances::k_inst_emit, dim3(instances::kChunks), dim3(instances::kEmitThreads),
+                            (size_t)L.geo.n_tiles * 4, stream, order, bin_start, coarse, (const uint32_t*)counters,
+                            (const uint32_t*)at<uint32_t>(ws, L.bin_table),
+                            (const uint32_t*)at<uint32_t>(ws, L.inst_start), at<uint16_t>(ws, L.inst_keys_a),
+                            at<uint32_t>(ws, L.inst_vals_a), L.geo.n, L.geo.gw, L.geo.n_tiles, (int)L.pub.end_bit);
+        }
     }
     INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
                 (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
