@@ -160,6 +160,54 @@ __device__ __forceinline__ uint32_t cdf_search(const float* __restrict__ cdf, fl
     return min(first, n - 1);
 }
 
+// The same search with the top of its decision tree in LDS. Which element the k-th probe reads depends only on
+// the outcomes of the probes before it, so the first kTreeDepth probes can only touch 2^kTreeDepth - 1 fixed
+// elements; a block keeps those in LDS in heap order (node 1 = first probe, node 2n / 2n + 1 = the probe after
+// going left / right) and reads the CDF itself only below that depth. The comparisons are exactly those of
+// cdf_search, so the result is the same even where rounding leaves the CDF not perfectly monotone; for 262,144
+// leaves 11 of the 18 dependent cache round trips of a sample become LDS reads.
+constexpr int kTreeDepth = 11;
+constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNodes - 1
+
+// Every thread of the block must call it; ends with a barrier.
+__device__ __forceinline__ void load_search_tree(float* s_tree, const float* __restrict__ cdf, uint32_t n) {
+    for (uint32_t node = threadIdx.x + 1u; node < kTreeNodes; node += blockDim.x) {
+        // replay the decisions that lead to this node
+        const int depth = 31 - __clz(node);
+        uint32_t first = 0, count = n;
+        for (int l = depth - 1; l >= 0 && count > 0; --l) {
+            const uint32_t step = count >> 1;
+            if ((node >> l) & 1u) {
+                first += step + 1;
+                count -= step + 1;
+            } else {
+                count = step;
+            }
+        }
+        s_tree[node] = count > 0 ? cdf[first + (count >> 1)] : 0.0f;
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ uint32_t cdf_search(const float* s_tree, const float* __restrict__ cdf, float sample,
+                                               uint32_t n) {
+    uint32_t first = 0, count = n, node = 1;
+    while (count > 0) {
+        const uint32_t step = count >> 1;
+        const uint32_t it = first + step;
+        const float v = node < kTreeNodes ? s_tree[node] : cdf[it];
+        if (v < sample) {
+            first = it + 1;
+            count -= step + 1;
+            node = 2u * node + 1u;
+        } else {
+            count = step;
+            node = 2u * node;
+        }
+    }
+    return min(first, n - 1);
+}
+
 struct Candidate {
     uint32_t leaf;
     float x, y, z;
@@ -168,12 +216,12 @@ struct Candidate {
 // `r` stands at draw 4*k; leaves it at 4*k + 4.
 __device__ __forceinline__ Candidate draw_candidate(Pcg32& r, const float* __restrict__ centers,
                                                     const int32_t* __restrict__ levels,
-                                                    const float* __restrict__ cdf, uint32_t n_leaves,
-                                                    float initial_size) {
+                                                    const float* __restrict__ cdf, const float* s_tree,
+                                                    uint32_t n_leaves, float initial_size) {
     const float u = pcg_float(r);
     const float ox = pcg_float(r), oy = pcg_float(r), oz = pcg_float(r);
     Candidate c;
-    c.leaf = cdf_search(cdf, u, n_leaves);
+    c.leaf = cdf_search(s_tree, cdf, u, n_leaves);
     const float scale = ldexpf(1.0f, -levels[c.leaf]) * initial_size;
     c.x = centers[3 * (size_t)c.leaf] + (ox - 0.5f) * scale;
     c.y = centers[3 * (size_t)c.leaf + 1] + (oy - 0.5f) * scale;
@@ -195,14 +243,16 @@ __global__ void __launch_bounds__(kBlock) k_sample(const float* __restrict__ cen
                                                    float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
                                                    uint32_t n_samples, uint32_t n_leaves, float initial_size,
                                                    const uint64_t* __restrict__ rng_dev) {
+    __shared__ float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
+    load_search_tree(s_tree, cdf, n_leaves);
     const uint64_t tile_first = (uint64_t)blockIdx.x * kSampleTile;
     Pcg32 r = thread_generator(rng_dev, tile_first);
     const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);  // from draw 4k+4 to 4(k+256)
     for (int j = 0; j < kSampleItems; ++j) {
         const uint64_t k = tile_first + (uint64_t)j * kBlock + threadIdx.x;
         if (k < n_samples) {
-            const Candidate c = draw_candidate(r, centers, levels, cdf, n_leaves, initial_size);
+            const Candidate c = draw_candidate(r, centers, levels, cdf, s_tree, n_leaves, initial_size);
             positions[3 * k] = c.x;
             positions[3 * k + 1] = c.y;
             positions[3 * k + 2] = c.z;
@@ -237,6 +287,7 @@ __global__ void __launch_bounds__(kBlock)
                   const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
     __shared__ uint32_t s_bid, s_accepted0, s_exclusive, s_done;
     __shared__ uint32_t s_count[kSampleItems * (kBlock / kWave)];
+    __shared__ float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     if (tid == 0) {
@@ -253,6 +304,7 @@ __global__ void __launch_bounds__(kBlock)
     }
     __syncthreads();
     if (s_done) return;
+    load_search_tree(s_tree, cdf, n_leaves);
     const uint32_t bid = s_bid;
     const uint64_t tile_first = (uint64_t)bid * kSampleTile;  // relative to k0
     const Rows m = load_rows(w2c);
@@ -267,7 +319,7 @@ __global__ void __launch_bounds__(kBlock)
         const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
         keep[j] = false;
         if (rel < n_candidates) {
-            cand[j] = draw_candidate(r, centers, levels, cdf, n_leaves, initial_size);
+            cand[j] = draw_candidate(r, centers, levels, cdf, s_tree, n_leaves, initial_size);
             keep[j] = sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
             r.state = pcg_apply(step, r.state);
         }
