@@ -198,6 +198,14 @@ def main() -> int:
     fwd_ms = time_calls(forward, args.steps)
     bwd_ms = time_calls(backward, args.steps)
 
+    # the step that closes the loop: leaf statistics from this frame's leaf indices and blending weights
+    from inpc_amd import update_probability_field
+
+    field_weights = weights.clone()
+    field_scores = torch.zeros_like(weights)
+    field_ms = time_calls(lambda: update_probability_field(field_weights, field_scores, leaf_ids, blending_weights),
+                          args.steps)
+
     # ---- per-kernel durations: HIP events around every launch, on the launch stream, same steps ----------
     with _lib.KernelTimer() as timer:
         for _ in range(args.steps):
@@ -274,6 +282,7 @@ def main() -> int:
         "extra": {
             "forward_ms": round(fwd_ms, 4), "backward_ms": round(bwd_ms, 4),
             "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
+            "field_update_ms": round(field_ms, 4),
             "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
             "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),
             "kernels": kernels,

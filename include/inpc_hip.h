@@ -263,6 +263,31 @@ int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
 int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* workspace,
                               uint32_t counters_host[3], void* stream);
 
+/* =========================================================================================
+ * Probability-field statistics (the consumer of the sampler's leaf indices and the
+ * rasterizer's blending weights, once per training iteration)
+ * ======================================================================================= */
+
+/* Bytes of scratch for inpc_field_update over n_leaves leaves. */
+size_t inpc_field_update_workspace_bytes(uint32_t n_leaves);
+
+/* leaf_weights *= decay; leaf_scores *= decay; then, with max_s / min_s the per-leaf maximum /
+ * minimum of `weights` over the samples whose index names the leaf (0 for a leaf without
+ * samples), leaf_weights = max(leaf_weights, max_s) and
+ * leaf_scores = max(leaf_scores, clamp(max_s - min_s, 0, 1)), all in place.
+ * Replaces ProbabilityField.update (Modules/ProbabilityField.py:146-157): two mul_, two
+ * scatter_reduce_ (amax / amin, include_self=False) and two torch.maximum.
+ * indices (n,) i64 dev (the leaf indices generate_training_samples returned), weights (n,) f32
+ * dev (blending weights), leaf_weights / leaf_scores (L,) f32 dev. An index outside [0, L) is
+ * skipped and recorded; inpc_field_update_check reports it. No host synchronisation. */
+int inpc_field_update(const int64_t* indices, const float* weights, uint32_t n_samples,
+                      float* leaf_weights, float* leaf_scores, uint32_t n_leaves, float decay,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* INPC_E_INVALID_ARGUMENT if the last inpc_field_update on this workspace met an index outside
+ * [0, n_leaves) (the reference's scatter_reduce_ raises for those). Synchronises `stream`. */
+int inpc_field_update_check(const void* workspace, void* stream);
+
 /* Per-kernel timing hooks for benchmarks: when enabled, every launch made by the calling
  * thread is bracketed by HIP events on its stream; inpc_timing_collect synchronises and
  * returns the number of records written as {name, milliseconds}. */

@@ -373,3 +373,30 @@ def raster_forward_backward(cfg: RasterConfig, positions, features, opacities, w
     if rc != 0:
         raise RuntimeError(f"oracle_raster_forward_backward failed with {rc}")
     return image, alpha, bw, gf, go
+
+
+# ----------------------------------------------------------------------------------------------
+# probability-field statistics (Modules/ProbabilityField.py:146-157 of the reference), plain numpy
+# ----------------------------------------------------------------------------------------------
+def field_update(leaf_weights, leaf_scores, indices, weights, decay=0.9968):
+    """Returns the updated (leaf_weights, leaf_scores) as new float32 arrays. Follows the reference line by line:
+    decay (float32 multiply), per-leaf maximum / minimum of the sampled weights with 0 for leaves without samples
+    (scatter_reduce_ amax / amin, include_self=False), maximum with the decayed values, clamped spread."""
+    lw = np.asarray(leaf_weights, np.float32) * np.float32(decay)
+    ls = np.asarray(leaf_scores, np.float32) * np.float32(decay)
+    idx = np.asarray(indices, np.int64)
+    w = np.asarray(weights, np.float32).reshape(-1)
+    n = lw.shape[0]
+    if idx.size and (idx.min() < 0 or idx.max() >= n):
+        raise IndexError("sample index outside the leaf range")
+    max_sampled = np.full(n, -np.inf, np.float32)
+    min_sampled = np.full(n, np.inf, np.float32)
+    np.maximum.at(max_sampled, idx, w)
+    np.minimum.at(min_sampled, idx, w)
+    hit = np.zeros(n, bool)
+    hit[idx] = True
+    max_sampled[~hit] = 0.0
+    min_sampled[~hit] = 0.0
+    lw = np.maximum(lw, max_sampled)
+    ls = np.maximum(ls, np.clip(max_sampled - min_sampled, np.float32(0.0), np.float32(1.0)))
+    return lw.astype(np.float32), ls.astype(np.float32)

@@ -36,12 +36,13 @@ def test_every_entry_point_cites_the_interface_it_replaces():
     for name in declared_functions():
         if name in ("inpc_last_error", "inpc_abi_version", "inpc_timing_enable", "inpc_timing_collect",
                     "inpc_raster_layout_query", "inpc_raster_read_counters", "inpc_sampler_workspace_bytes",
-                    "inpc_cull_workspace_bytes", "inpc_calibration_copy"):
+                    "inpc_cull_workspace_bytes", "inpc_calibration_copy", "inpc_field_update_workspace_bytes",
+                    "inpc_field_update_check"):
             continue  # library plumbing without a counterpart
         at = text.index(name + "(")
         before = text[:at]
         comment = before[before.rindex("/*"):]
-        assert re.search(r"B/[\w/\.]+:\d+", comment), f"{name}: no reference file:line in its comment"
+        assert re.search(r"[\w/\.]+\.(py|cu|cuh|h|cpp):\d+", comment), f"{name}: no reference file:line in its comment"
 
 
 def test_header_is_plain_c_and_structs_match_ctypes(tmp_path):

@@ -1,0 +1,67 @@
+"""GPU parity of the probability-field update against the oracle, through the C ABI and the Python operator.
+Maximum and minimum are order independent: every output is bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from inpc_amd import _lib, update_probability_field
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n_leaves,n_samples", [(1, 7), (63, 0), (1000, 257), (262144, 1 << 20)])
+def test_update_bit_exact(gpu, oracle, n_leaves, n_samples):
+    rng = np.random.default_rng(n_leaves)
+    lw = rng.random(n_leaves).astype(np.float32)
+    ls = rng.random(n_leaves).astype(np.float32)
+    idx = rng.integers(0, n_leaves, n_samples).astype(np.int64)
+    w = (rng.random(n_samples) ** 3 * 1.5).astype(np.float32)
+    w[::97] = -0.25 * w[::97]                      # signs are handled too
+    d_lw, d_ls, d_idx, d_w = H.dev(lw), H.dev(ls), H.dev(idx), H.dev(w.reshape(-1, 1))
+    update_probability_field(d_lw, d_ls, d_idx, d_w, check=True)
+    a, b = oracle.field_update(lw, ls, idx, w)
+    np.testing.assert_array_equal(d_lw.cpu().numpy().view(np.uint32), a.view(np.uint32))
+    np.testing.assert_array_equal(d_ls.cpu().numpy().view(np.uint32), b.view(np.uint32))
+
+
+def test_two_updates_in_a_row_and_bad_index(gpu, oracle):
+    rng = np.random.default_rng(5)
+    lw = rng.random(500).astype(np.float32)
+    ls = np.zeros(500, np.float32)
+    d_lw, d_ls = H.dev(lw), H.dev(ls)
+    for step in range(2):
+        idx = rng.integers(0, 500, 3000).astype(np.int64)
+        w = rng.random(3000).astype(np.float32)
+        update_probability_field(d_lw, d_ls, H.dev(idx), H.dev(w))
+        lw, ls = oracle.field_update(lw, ls, idx, w)
+    np.testing.assert_array_equal(d_lw.cpu().numpy(), lw)
+    np.testing.assert_array_equal(d_ls.cpu().numpy(), ls)
+    bad = np.array([0, 500, 3], np.int64)
+    with pytest.raises(_lib.BackendError, match="outside"):
+        update_probability_field(d_lw, d_ls, H.dev(bad), H.dev(np.ones(3, np.float32)), check=True)
+
+
+def test_closes_the_loop_with_sampler_and_rasterizer(gpu, oracle):
+    """indices from generate_training_samples + blending weights from the rasterizer -> field update."""
+    from inpc_amd import ProbabilityFieldSampler, synthetic
+    from inpc_amd.rasterization import rasterize_points
+
+    oct = synthetic.octree_leaves(4096, 5, 4.0, seed=3)
+    hv = synthetic.camera_on_z(160, 120, 140.0, 6.0)
+    view = hv.to_view(gpu)
+    sampler = ProbabilityFieldSampler(seed=1)
+    pos, ids = sampler.generate_training_samples(H.dev(oct.centers), H.dev(oct.levels), H.dev(oct.weights), view, 50000,
+                                                 oct.initial_size)
+    gen = torch.Generator(device=gpu).manual_seed(2)
+    feats = torch.randn((50000, 4), generator=gen, device=gpu)
+    opac = torch.sigmoid(torch.randn(50000, generator=gen, device=gpu))
+    _, _, bw = rasterize_points(view, pos, feats, opac, tile=16)
+    lw = np.full(4096, 0.01, np.float32)
+    ls = np.zeros(4096, np.float32)
+    d_lw, d_ls = H.dev(lw), H.dev(ls)
+    update_probability_field(d_lw, d_ls, ids, bw, check=True)
+    a, b = oracle.field_update(lw, ls, ids.cpu().numpy(), bw.cpu().numpy())
+    np.testing.assert_array_equal(d_lw.cpu().numpy(), a)
+    np.testing.assert_array_equal(d_ls.cpu().numpy(), b)
+    assert (a > np.float32(0.01) * np.float32(0.9968)).sum() > 100   # sampled leaves took their maxima
