@@ -288,6 +288,26 @@ int inpc_field_update(const int64_t* indices, const float* weights, uint32_t n_s
  * [0, n_leaves) (the reference's scatter_reduce_ raises for those). Synchronises `stream`. */
 int inpc_field_update_check(const void* workspace, void* stream);
 
+/* =========================================================================================
+ * Element-wise steps between the sampler and the rasterizer
+ * ======================================================================================= */
+
+/* contracted = saturate(scale * p + 0.5), scale = (2 sqrt(L) - 1) / L / 4, L = max(|p|^2, 1):
+ * the unit ball maps linearly into [0.25, 0.75]^3, everything outside into the rest of the unit
+ * cube. Replaces spherical_contraction_cu (B/misc/src/misc_kernels.cu:49-66) behind
+ * spherical_contraction (B/torch_bindings/misc.py:17-18). positions, contracted (n,3) f32 dev. */
+int inpc_spherical_contraction(const float* positions, float* contracted, uint32_t n_points,
+                               void* stream);
+
+/* opacity = -expm1(-exp(raw)), element-wise: feature_to_opacity (utils.py:31-33) with the
+ * forward of TruncExp (utils.py:13-22). raw, opacity (n,) f32 dev. */
+int inpc_opacity_forward(const float* raw, float* opacity, size_t n, void* stream);
+
+/* grad_raw = grad_opacity * exp(-exp(raw)) * exp(clamp(raw, -15, 15)): the backward of the same
+ * expression, the truncated exponential's gradient as in TruncExp.backward (utils.py:24-28). */
+int inpc_opacity_backward(const float* grad_opacity, const float* raw, float* grad_raw, size_t n,
+                          void* stream);
+
 /* Per-kernel timing hooks for benchmarks: when enabled, every launch made by the calling
  * thread is bracketed by HIP events on its stream; inpc_timing_collect synchronises and
  * returns the number of records written as {name, milliseconds}. */

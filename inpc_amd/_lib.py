@@ -101,6 +101,9 @@ SIGNATURES = {
     "inpc_field_update_workspace_bytes": (_SZ, [_U32]),
     "inpc_field_update": (C.c_int, [_P, _P, _U32, _P, _P, _U32, _F, _P, _SZ, _P]),
     "inpc_field_update_check": (C.c_int, [_P, _P]),
+    "inpc_spherical_contraction": (C.c_int, [_P, _P, _U32, _P]),
+    "inpc_opacity_forward": (C.c_int, [_P, _P, _SZ, _P]),
+    "inpc_opacity_backward": (C.c_int, [_P, _P, _P, _SZ, _P]),
     "inpc_timing_enable": (None, [C.c_int]),
     "inpc_timing_collect": (C.c_int, [C.POINTER(TimingRecord), C.c_int]),
     "inpc_calibration_copy": (C.c_int, [_P, _P, _SZ, _P]),

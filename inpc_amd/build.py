@@ -11,7 +11,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libinpc_hip.so"
-SOURCES = ["runtime.hip", "sampler.hip", "raster.hip", "field.hip"]
+SOURCES = ["runtime.hip", "sampler.hip", "raster.hip", "field.hip", "misc.hip"]
 HEADERS = ["common.hpp", "radix.hpp", "blend.hpp", "instances.hpp"]
 
 # -ffp-contract=off: tile bounds, depth keys, leaf picks and cull decisions must be bit-identical to

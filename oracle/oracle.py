@@ -400,3 +400,29 @@ def field_update(leaf_weights, leaf_scores, indices, weights, decay=0.9968):
     lw = np.maximum(lw, max_sampled)
     ls = np.maximum(ls, np.clip(max_sampled - min_sampled, np.float32(0.0), np.float32(1.0)))
     return lw.astype(np.float32), ls.astype(np.float32)
+
+
+# ----------------------------------------------------------------------------------------------
+# element-wise steps between sampler and rasterizer, plain numpy in float32
+# ----------------------------------------------------------------------------------------------
+def spherical_contraction(positions):
+    """B/misc/src/misc_kernels.cu:49-66, every operation rounded to float32 in the written order."""
+    p = np.asarray(positions, np.float32).reshape(-1, 3)
+    f = np.float32
+    x, y, z = p[:, 0], p[:, 1], p[:, 2]
+    length_sq = np.maximum((x * x + y * y) + z * z, f(1.0))
+    scale = (np.sqrt(length_sq) * f(2.0) - f(1.0)) / length_sq * f(0.25)
+    return np.clip(scale[:, None] * p + f(0.5), f(0.0), f(1.0)).astype(np.float32)
+
+
+def feature_to_opacity(raw):
+    """utils.py:31-33: -expm1(-exp(x))."""
+    x = np.asarray(raw, np.float32)
+    return (-np.expm1(-np.exp(x))).astype(np.float32)
+
+
+def feature_to_opacity_backward(grad, raw):
+    """Gradient of the same expression with TruncExp's backward (utils.py:24-28)."""
+    x = np.asarray(raw, np.float32)
+    g = np.asarray(grad, np.float32)
+    return ((g * np.exp(-np.exp(x))) * np.exp(np.clip(x, np.float32(-15.0), np.float32(15.0)))).astype(np.float32)
