@@ -308,6 +308,24 @@ int inpc_opacity_forward(const float* raw, float* opacity, size_t n, void* strea
 int inpc_opacity_backward(const float* grad_opacity, const float* raw, float* grad_raw, size_t n,
                           void* stream);
 
+/* grads (= or +=, `add` != 0) factor(i) * weights[i], factor = 0.1 * 2 / (entries of the hash-grid
+ * level that holds flat index i), 0 in front of index 6144. Replaces
+ * compute_normalized_weight_decay_grads_cu<add> (B/misc/src/misc_kernels.cu:6-47) behind
+ * compute_normalized_weight_decay_grads / add_normalized_weight_decay_grads
+ * (B/torch_bindings/misc.py:9-14). weights, grads (n,) f32 dev. */
+int inpc_weight_decay_grads(const float* weights, float* grads, uint32_t n_weights, int add,
+                            void* stream);
+
+/* elementwise_loss[i] = log1p(12.5 (input[i] - target[i])^2) / n. Replaces cauchy_loss_cu
+ * (B/misc/src/misc_kernels.cu:68-79); the caller sums (B/misc/src/misc_api.cu:51-65). */
+int inpc_cauchy_loss(const float* input, const float* target, float* elementwise_loss, uint32_t n,
+                     void* stream);
+
+/* grad_input[i] = 25 d / max(n (12.5 d^2 + 1), 1e-12) * grad[0], d = input[i] - target[i].
+ * Replaces cauchy_loss_backward_cu (B/misc/src/misc_kernels.cu:81-94). grad: 1 f32 dev. */
+int inpc_cauchy_loss_backward(const float* grad, const float* input, const float* target,
+                              float* grad_input, uint32_t n, void* stream);
+
 /* Per-kernel timing hooks for benchmarks: when enabled, every launch made by the calling
  * thread is bracketed by HIP events on its stream; inpc_timing_collect synchronises and
  * returns the number of records written as {name, milliseconds}. */

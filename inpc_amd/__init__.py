@@ -5,7 +5,8 @@ Re-exports the operator API of the reference's INPCCudaBackend package
 the bilinear point rasterizer. Native code lives in libinpc_hip.so (build: python -m inpc_amd.build).
 """
 from .field import update_probability_field
-from .misc import feature_to_opacity, spherical_contraction
+from .misc import (add_normalized_weight_decay_grads, compute_normalized_weight_decay_grads, feature_to_opacity,
+                   fused_cauchy_loss, spherical_contraction)
 from .rasterization import INPCRasterizer, RasterizerMode, RasterizerSettings, rasterize_points
 from .sampling import ProbabilityFieldSampler, compute_viewpoint_weights
 from .views import PerspectiveCamera, View
@@ -13,6 +14,7 @@ from .views import PerspectiveCamera, View
 __all__ = [
     "INPCRasterizer", "RasterizerSettings", "RasterizerMode", "rasterize_points",
     "ProbabilityFieldSampler", "compute_viewpoint_weights", "update_probability_field",
-    "spherical_contraction", "feature_to_opacity",
+    "spherical_contraction", "feature_to_opacity", "compute_normalized_weight_decay_grads",
+    "add_normalized_weight_decay_grads", "fused_cauchy_loss",
     "PerspectiveCamera", "View",
 ]

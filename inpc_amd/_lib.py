@@ -104,6 +104,9 @@ SIGNATURES = {
     "inpc_spherical_contraction": (C.c_int, [_P, _P, _U32, _P]),
     "inpc_opacity_forward": (C.c_int, [_P, _P, _SZ, _P]),
     "inpc_opacity_backward": (C.c_int, [_P, _P, _P, _SZ, _P]),
+    "inpc_weight_decay_grads": (C.c_int, [_P, _P, _U32, C.c_int, _P]),
+    "inpc_cauchy_loss": (C.c_int, [_P, _P, _P, _U32, _P]),
+    "inpc_cauchy_loss_backward": (C.c_int, [_P, _P, _P, _P, _U32, _P]),
     "inpc_timing_enable": (None, [C.c_int]),
     "inpc_timing_collect": (C.c_int, [C.POINTER(TimingRecord), C.c_int]),
     "inpc_calibration_copy": (C.c_int, [_P, _P, _SZ, _P]),

@@ -1,6 +1,7 @@
-"""Element-wise operators between the sampler and the rasterizer.
+"""Element-wise operators around the appearance field and the loss.
 
-`spherical_contraction` has the signature of the reference's (B/torch_bindings/misc.py:17-18);
+`spherical_contraction`, `compute_normalized_weight_decay_grads`, `add_normalized_weight_decay_grads` and
+`fused_cauchy_loss` have the signatures of the reference's (B/torch_bindings/misc.py:9-44);
 `feature_to_opacity` that of utils.py:31-33, including its gradient (TruncExp, utils.py:13-28).
 """
 from __future__ import annotations
@@ -56,3 +57,56 @@ class _FeatureToOpacity(torch.autograd.Function):
 def feature_to_opacity(features: torch.Tensor) -> torch.Tensor:
     """Log-space volume density -> opacity in [0, 1]; differentiable."""
     return _FeatureToOpacity.apply(features)
+
+
+def compute_normalized_weight_decay_grads(weights: torch.Tensor) -> torch.Tensor:
+    """Per-level normalised weight-decay gradient of the flat hash-grid parameter vector."""
+    weights = _require_gpu_float(weights)
+    grads = torch.empty(weights.shape[0], dtype=torch.float32, device=weights.device)
+    _lib.check(_lib.lib().inpc_weight_decay_grads(_lib.ptr(weights), _lib.ptr(grads), weights.shape[0], 0,
+                                                  _lib.current_stream()), "inpc_weight_decay_grads")
+    return grads
+
+
+def add_normalized_weight_decay_grads(param: torch.nn.Parameter) -> None:
+    """param.grad += the same gradient, in place."""
+    if param.grad is None:
+        raise RuntimeError("the parameter has no gradient to add to")
+    if param.data.dtype != torch.float32 or param.grad.dtype != torch.float32:
+        raise RuntimeError("expected scalar type Float")
+    if not (param.data.is_cuda and param.grad.is_cuda and param.data.is_contiguous() and param.grad.is_contiguous()):
+        raise RuntimeError("expected contiguous tensors on the GPU")
+    _lib.check(_lib.lib().inpc_weight_decay_grads(_lib.ptr(param.data), _lib.ptr(param.grad), param.data.shape[0], 1,
+                                                  _lib.current_stream()), "inpc_weight_decay_grads")
+
+
+class _CauchyLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
+        input, target = _require_gpu_float(input), _require_gpu_float(target)
+        elementwise = torch.empty_like(input)
+        _lib.check(_lib.lib().inpc_cauchy_loss(_lib.ptr(input), _lib.ptr(target), _lib.ptr(elementwise), input.numel(),
+                                               _lib.current_stream()), "inpc_cauchy_loss")
+        ctx.save_for_backward(input, target)
+        ctx.set_materialize_grads(False)
+        return elementwise.sum()
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx: Any, grad: torch.Tensor):
+        input, target = ctx.saved_tensors
+        if grad is None:
+            return None, None
+        grad = _require_gpu_float(grad.reshape(1))
+        grad_input = torch.empty_like(input)
+        _lib.check(_lib.lib().inpc_cauchy_loss_backward(_lib.ptr(grad), _lib.ptr(input), _lib.ptr(target),
+                                                        _lib.ptr(grad_input), input.numel(), _lib.current_stream()),
+                   "inpc_cauchy_loss_backward")
+        return grad_input, None
+
+
+def fused_cauchy_loss(input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
+    """Cauchy loss between input and target with mean reduction."""
+    if input.shape != target.shape:
+        raise ValueError(f"input and target shapes must match ({input.shape} vs. {target.shape})")
+    return _CauchyLoss.apply(input, target)

@@ -426,3 +426,31 @@ def feature_to_opacity_backward(grad, raw):
     x = np.asarray(raw, np.float32)
     g = np.asarray(grad, np.float32)
     return ((g * np.exp(-np.exp(x))) * np.exp(np.clip(x, np.float32(-15.0), np.float32(15.0)))).astype(np.float32)
+
+
+_DECAY_LEVELS = [177362944, 143808512, 110254080, 76699648, 43145216, 9590784, 1202176, 153600, 22528, 6144]
+_DECAY_ENDS = [210917376] + _DECAY_LEVELS[:-1]
+
+
+def weight_decay_grads(weights, offset=0):
+    """B/misc/src/misc_kernels.cu:6-47 for the flat indices offset .. offset + len(weights) - 1."""
+    w = np.asarray(weights, np.float32)
+    idx = np.arange(w.shape[0], dtype=np.int64) + offset
+    factor = np.zeros(w.shape[0], np.float32)
+    for begin, end in zip(reversed(_DECAY_LEVELS), reversed(_DECAY_ENDS)):   # ascending thresholds: later ones win
+        f = np.float32(np.float32(0.1) * np.float32(2.0)) / np.float32(end - begin)
+        factor[idx >= begin] = f
+    return (factor * w).astype(np.float32)
+
+
+def cauchy_loss(input, target):
+    d = np.asarray(input, np.float32) - np.asarray(target, np.float32)
+    n = np.float32(d.size)
+    return (np.log1p(d * d * np.float32(12.5)) / n).astype(np.float32)
+
+
+def cauchy_loss_backward(grad, input, target):
+    d = np.asarray(input, np.float32) - np.asarray(target, np.float32)
+    n = np.float32(d.size)
+    den = n * (np.float32(12.5) * d * d + np.float32(1.0))
+    return (np.float32(25.0) * d / np.maximum(den, np.float32(1e-12)) * np.float32(grad)).astype(np.float32)

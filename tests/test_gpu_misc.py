@@ -31,3 +31,32 @@ def test_feature_to_opacity_forward_and_backward(gpu, oracle):
     small = x <= 1.0
     np.testing.assert_allclose(xt.grad.cpu().numpy()[small], oracle.feature_to_opacity_backward(g, x)[small], rtol=2e-6,
                                atol=1e-30)
+
+
+def test_weight_decay_grads(gpu, oracle):
+    from inpc_amd import add_normalized_weight_decay_grads, compute_normalized_weight_decay_grads
+
+    rng = np.random.default_rng(4)
+    w = rng.normal(size=1_300_000).astype(np.float32)      # spans the levels that start at 6144 .. 1202176
+    g = compute_normalized_weight_decay_grads(H.dev(w)).cpu().numpy()
+    ref = oracle.weight_decay_grads(w)
+    np.testing.assert_array_equal(g.view(np.uint32), ref.view(np.uint32))
+    param = torch.nn.Parameter(H.dev(w))
+    g0 = rng.normal(size=w.shape).astype(np.float32)
+    param.grad = H.dev(g0)
+    add_normalized_weight_decay_grads(param)
+    np.testing.assert_array_equal(param.grad.cpu().numpy(), g0 + ref)
+
+
+def test_fused_cauchy_loss(gpu, oracle):
+    from inpc_amd import fused_cauchy_loss
+
+    rng = np.random.default_rng(5)
+    a, b = rng.random((3, 64, 80)).astype(np.float32), rng.random((3, 64, 80)).astype(np.float32)
+    at = H.dev(a).requires_grad_(True)
+    loss = fused_cauchy_loss(at, H.dev(b))
+    assert loss.item() == pytest.approx(float(oracle.cauchy_loss(a, b).astype(np.float64).sum()), rel=1e-5)
+    (loss * 3.0).backward()
+    np.testing.assert_allclose(at.grad.cpu().numpy(), oracle.cauchy_loss_backward(3.0, a, b), rtol=2e-6, atol=1e-12)
+    with pytest.raises(ValueError):
+        fused_cauchy_loss(at, H.dev(b[:2]))

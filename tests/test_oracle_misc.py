@@ -39,3 +39,24 @@ def test_opacity_against_float64_and_autograd(oracle):
     big = np.array([-18.0, -16.0], np.float32)
     expect = np.exp(-np.exp(big.astype(np.float64))) * np.exp(-15.0)
     np.testing.assert_allclose(oracle.feature_to_opacity_backward(np.ones(2, np.float32), big), expect, rtol=5e-6)
+
+
+def test_weight_decay_factors(oracle):
+    # level boundaries and sizes as in the reference's table: factor = 0.2 / entries of the level, 0 below 6144
+    w = np.ones(30000, np.float32)
+    g = oracle.weight_decay_grads(w)
+    assert (g[:6144] == 0).all()
+    np.testing.assert_allclose(g[6144:22528], 0.2 / (22528 - 6144), rtol=1e-6)
+    np.testing.assert_allclose(g[22528:], 0.2 / (153600 - 22528), rtol=1e-6)
+    top = oracle.weight_decay_grads(np.full(4, 2.0, np.float32), offset=177362944 - 2)
+    np.testing.assert_allclose(top, [2 * 0.2 / (177362944 - 143808512)] * 2 + [2 * 0.2 / (210917376 - 177362944)] * 2, rtol=1e-6)
+
+
+def test_cauchy_loss_against_torch(oracle):
+    rng = np.random.default_rng(3)
+    a, b = rng.normal(size=5000).astype(np.float32), rng.normal(size=5000).astype(np.float32)
+    at = torch.tensor(a.astype(np.float64), requires_grad=True)
+    loss = torch.log1p(12.5 * (at - torch.tensor(b.astype(np.float64))) ** 2).mean()
+    np.testing.assert_allclose(oracle.cauchy_loss(a, b).astype(np.float64).sum(), loss.item(), rtol=1e-5)
+    loss.backward()
+    np.testing.assert_allclose(oracle.cauchy_loss_backward(1.0, a, b), at.grad.numpy(), rtol=1e-5, atol=1e-10)
