@@ -13,7 +13,7 @@
 //            product scan (long lists) -> per-instance results into LDS;
 //   write    thread t writes the result of instance t: a plain store when the point lies in one tile only,
 //            atomics when it straddles tiles.
-// Two block barriers per batch; the record gather of the next batch is in flight during consume.
+// Two block barriers per batch; the record gather runs two batches ahead of the blend.
 #pragma once
 
 namespace blend {
@@ -90,13 +90,6 @@ __device__ __forceinline__ uint32_t wave_exclusive_sum(uint32_t v, uint32_t& tot
     return incl - v;
 }
 
-// Orders the LDS traffic of one wave: everything issued before is visible to every lane after.
-__device__ __forceinline__ void wave_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 // Per-block staging area of one batch.
 //   NQ  waves ("quads") per tile
 //   NF  fragments one instance can have inside one wave's pixel grid: 4 (8x8 tiles: the whole 2 x 2 footprint),
@@ -130,9 +123,17 @@ struct QuadScratch {
 struct Header {
     float sx, sy, opacity;
     uint32_t point;
-    bool multi;  // the point touches more than one tile
+    uint32_t tiles;  // raw word; see multi()
     float depth;
+    // the point touches more than one tile (kept as the raw word until the write phase: a flag derived
+    // at the load would make the gather wait for its own first reply)
+    __device__ __forceinline__ bool multi() const { return ((tiles >> 16) & 3u) != 0u; }
 };
+
+// Makes the value available here: the wait for an outstanding load that produces it lands at this point and not
+// at a later first use.
+__device__ __forceinline__ void arrive(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void arrive(uint32_t& v) { asm volatile("" : "+v"(v)); }
 
 __device__ __forceinline__ Header read_header(const char* __restrict__ record) {
     const float4 h0 = ((const float4*)record)[0];
@@ -142,7 +143,7 @@ __device__ __forceinline__ Header read_header(const char* __restrict__ record) {
     h.sy = h0.y;
     h.opacity = h0.z;
     h.point = __float_as_uint(h0.w);
-    h.multi = ((__float_as_uint(h1.x) >> 16) & 3u) != 0u;
+    h.tiles = __float_as_uint(h1.x);
     h.depth = h1.y;
     return h;
 }
@@ -202,20 +203,39 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
     }
 }
 
-// The idx-th staged instance of quad q's list (the per-source-wave pieces concatenated in wave order).
+// A quad's list is the concatenation, in wave order, of the pieces the NQ source waves wrote. ListIndex holds
+// the piece boundaries of one batch (the same in every lane).
+template <int NQ>
+struct ListIndex {
+    uint32_t end[NQ];  // end[s]: entries in the pieces 0..s; end[NQ - 1] is the length of the list
+};
+
 template <int T, int C, bool WITH_DEPTH>
-__device__ __forceinline__ uint32_t list_entry(const Stage<T, C, WITH_DEPTH>& st, uint32_t q, uint32_t idx) {
+__device__ __forceinline__ ListIndex<T * T / 64> list_index(const Stage<T, C, WITH_DEPTH>& st, uint32_t q) {
     constexpr int NQ = T * T / 64;
-    uint32_t w = 0;
+    ListIndex<NQ> li;
+    uint32_t run = 0;
 #pragma unroll
-    for (int s = 0; s < NQ - 1; ++s) {
-        const uint32_t c = st.count[q][s];
-        if (w == (uint32_t)s && idx >= c) {
-            idx -= c;
-            w = s + 1;
-        }
+    for (int s = 0; s < NQ; ++s) {
+        run += st.count[q][s];
+        li.end[s] = (uint32_t)__builtin_amdgcn_readfirstlane((int)run);
     }
-    return st.list[q][w][idx];
+    return li;
+}
+
+// The idx-th staged instance of quad q's list, idx < li.end[NQ - 1].
+template <int T, int C, bool WITH_DEPTH>
+__device__ __forceinline__ uint32_t list_entry(const Stage<T, C, WITH_DEPTH>& st, const ListIndex<T * T / 64>& li,
+                                               uint32_t q, uint32_t idx) {
+    constexpr int NQ = T * T / 64;
+    uint32_t w = 0, first = 0;
+#pragma unroll
+    for (int s = 0; s < NQ - 1; ++s)
+        if (idx >= li.end[s]) {
+            w = s + 1;
+            first = li.end[s];
+        }
+    return st.list[q][w][idx - first];
 }
 
 // Fragments of one sub-batch lane: the (at most NF) pixels staged instance j covers in this wave's grid.
@@ -276,6 +296,73 @@ __device__ __forceinline__ void load_lane_fragments(const Stage<T, C, WITH_DEPTH
     }
 }
 
+// ---- the record gather, two batches ahead -------------------------------------------------------------------------
+// Per thread: the record of the batch being staged, the record of the batch after it (requested one batch
+// earlier, still in flight or arrived) and the slot of the batch after that.
+template <int C>
+struct Gather {
+    Header h;
+    float f[C];
+    Header h_next;
+    float f_next[C];
+    uint32_t next_slot;
+};
+
+template <int T, int C, bool HALF>
+__device__ __forceinline__ void start_gather(Gather<C>& g, const uint32_t* __restrict__ inst_slots,
+                                             const char* __restrict__ records, uint32_t stride, uint2 range) {
+    constexpr uint32_t TT = T * T;
+    const uint32_t at = range.x + threadIdx.x;
+    g.h = Header{};
+    g.h_next = Header{};
+#pragma unroll
+    for (int c = 0; c < C; ++c) g.f[c] = g.f_next[c] = 0.0f;
+    g.next_slot = 0u;
+    uint32_t slot0 = 0u, slot1 = 0u;
+    if (at < range.y) slot0 = inst_slots[at];
+    if (at + TT < range.y) slot1 = inst_slots[at + TT];
+    if (at + 2u * TT < range.y) g.next_slot = inst_slots[at + 2u * TT];
+    if (at < range.y) {
+        const char* record = records + (size_t)slot0 * stride;
+        g.h = read_header(record);
+        load_record_features<C, HALF>(g.f, record);
+    }
+    if (at + TT < range.y) {
+        const char* record = records + (size_t)slot1 * stride;
+        g.h_next = read_header(record);
+        load_record_features<C, HALF>(g.f_next, record);
+    }
+}
+
+// Called at the end of the batch that starts at `begin`, in front of the stores of its write phase, so that
+// waiting for the gather never waits for those stores: takes the record of the next batch (requested a whole
+// batch ago) and requests the record of the batch after it and the slot of the one after that.
+template <int T, int C, bool HALF>
+__device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __restrict__ inst_slots,
+                                               const char* __restrict__ records, uint32_t stride, uint32_t begin,
+                                               uint32_t end) {
+    constexpr uint32_t TT = T * T;
+    const uint32_t at = begin + threadIdx.x;
+    arrive(g.h_next.sx);
+    arrive(g.h_next.sy);
+    arrive(g.h_next.opacity);
+    arrive(g.h_next.point);
+    arrive(g.h_next.tiles);
+    arrive(g.h_next.depth);
+#pragma unroll
+    for (int c = 0; c < C; ++c) arrive(g.f_next[c]);
+    arrive(g.next_slot);
+    g.h = g.h_next;
+#pragma unroll
+    for (int c = 0; c < C; ++c) g.f[c] = g.f_next[c];
+    if (at + 2u * TT < end) {
+        const char* record = records + (size_t)g.next_slot * stride;
+        g.h_next = read_header(record);
+        load_record_features<C, HALF>(g.f_next, record);
+    }
+    if (at + 3u * TT < end) g.next_slot = inst_slots[at + 3u * TT];
+}
+
 // ---- forward ------------------------------------------------------------------------------------------------------
 template <int T, int C, bool HALF, bool INFERENCE>
 __global__ void __launch_bounds__(T* T)
@@ -316,44 +403,22 @@ __global__ void __launch_bounds__(T* T)
     INPC_PROF_DECL;
 #define FWD_MARK(i) INPC_PROF_MARK(i)
 #endif
-    // the gather runs ahead of the blend: the record of batch b + 1 and the slot of batch b + 2 are in flight
-    // while batch b is consumed
-    uint32_t next_slot = 0u;
-    Header h_next{};
-    float f_next[C];
-#pragma unroll
-    for (int c = 0; c < C; ++c) f_next[c] = 0.0f;
-    if (range.x + tid < range.y) {
-        const char* record = records + (size_t)inst_slots[range.x + tid] * stride;
-        h_next = read_header(record);
-        load_record_features<C, HALF>(f_next, record);
-    }
-    if (range.x + TT + tid < range.y) next_slot = inst_slots[range.x + TT + tid];
+    Gather<C> g;
+    start_gather<T, C, HALF>(g, inst_slots, records, stride, range);
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        const Header h = h_next;
-        float f[C];
-#pragma unroll
-        for (int c = 0; c < C; ++c) f[c] = f_next[c];
-        if (begin + TT + tid < range.y) {
-            const char* record = records + (size_t)next_slot * stride;
-            h_next = read_header(record);
-            load_record_features<C, HALF>(f_next, record);
-        }
-        if (begin + 2 * TT + tid < range.y) next_slot = inst_slots[begin + 2 * TT + tid];
-        stage_instance<T, C, INFERENCE>(st, valid, h, f, tile_x0, tile_y0);
+        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f, tile_x0, tile_y0);
         FWD_MARK(0);
         __syncthreads();
         FWD_MARK(1);
 
         // ---- consume: this wave's list
-        uint32_t total = 0;
-#pragma unroll
-        for (int s = 0; s < NQ; ++s) total += st.count[wave][s];
+        const ListIndex<NQ> li = list_index<T, C, INFERENCE>(st, wave);
+        const uint32_t total = li.end[NQ - 1];
         for (uint32_t sub = 0; sub < total; sub += 64u) {
             const bool live = sub + lane < total;
-            const uint32_t j = live ? list_entry<T, C, INFERENCE>(st, wave, sub + lane) : 0u;
+            const uint32_t j = live ? list_entry<T, C, INFERENCE>(st, li, wave, sub + lane) : 0u;
             LaneFragments<NF> lf;
             load_lane_fragments<T, C, INFERENCE>(st, wave, live, j, __ballot(done), lf);
             uint32_t my_start, my_count, n_fragments;
@@ -459,6 +524,10 @@ __global__ void __launch_bounds__(T* T)
 #if defined(INPC_BLEND_PROFILE) && !defined(INPC_PROFILE_BACKWARD)
         ++prof_batches;
 #endif
+        // ---- the gather moves on in front of the stores of the write phase
+        const uint32_t point = g.h.point;
+        const bool multi = g.h.multi();
+        advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
         // ---- write: thread t owns staged instance t (kernels.cu:291-295)
         if (!INFERENCE && valid) {
             float w = 0.0f;
@@ -470,8 +539,8 @@ __global__ void __launch_bounds__(T* T)
                     if (bw > 0.0f) w = fmaf(bw, st.weight[q][k][tid], w);
                 }
             if (w > 0.0f) {
-                if (h.multi) atomicAdd(&blending_weights[h.point], w);
-                else blending_weights[h.point] = w;
+                if (multi) atomicAdd(&blending_weights[point], w);
+                else blending_weights[point] = w;
             }
         }
         if (all_done) break;
@@ -507,7 +576,7 @@ __global__ void __launch_bounds__(T* T)
     constexpr int NF = Stage<T, C, false>::NF;
     __shared__ Stage<T, C, false> st;
     __shared__ QuadScratch<NF> s_quad[NQ];
-    __shared__ float s_grad[NQ][C][64];   // upstream gradient of every wave's pixels (0 outside the image)
+    __shared__ float4 s_grad[NQ][64][C / 4];   // upstream gradient of every wave's pixels (0 outside the image)
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tile = tile_order[blockIdx.x];
@@ -519,14 +588,23 @@ __global__ void __launch_bounds__(T* T)
 
     float final_dot = 0.0f, common = 0.0f;
     {
-        const size_t n_pixels = (size_t)W * H, pix = (size_t)py * W + px;
+        // all loads of the pixel in one go (a pixel outside the image reads pixel 0 and drops it)
+        const size_t n_pixels = (size_t)W * H, pix = inside ? (size_t)py * W + px : 0;
+        float g[C], v[C];
 #pragma unroll
         for (int c = 0; c < C; ++c) {
-            const float g = inside ? grad_image[c * n_pixels + pix] : 0.0f;
-            s_grad[wave][c][lane] = g;
-            if (inside) final_dot = fmaf(image[c * n_pixels + pix], g, final_dot);
+            g[c] = grad_image[c * n_pixels + pix];
+            v[c] = image[c * n_pixels + pix];
         }
-        if (inside) common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
+        const float ga = grad_alpha[pix], av = alpha_image[pix];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (!inside) g[c] = 0.0f;
+            if (inside) final_dot = fmaf(v[c], g[c], final_dot);
+        }
+#pragma unroll
+        for (int q4 = 0; q4 < C / 4; ++q4) s_grad[wave][lane][q4] = make_float4(g[4 * q4], g[4 * q4 + 1], g[4 * q4 + 2], g[4 * q4 + 3]);
+        if (inside) common = ga * (1.0f - av);
     }
     const float offset = common - final_dot;
     float Tr = 1.0f, running = 0.0f;
@@ -544,42 +622,22 @@ __global__ void __launch_bounds__(T* T)
 #else
 #define BWD_MARK(i)
 #endif
-    uint32_t next_slot = 0u;
-    Header h_next{};
-    float f_next[C];
-#pragma unroll
-    for (int c = 0; c < C; ++c) f_next[c] = 0.0f;
-    if (range.x + tid < range.y) {
-        const char* record = records + (size_t)inst_slots[range.x + tid] * stride;
-        h_next = read_header(record);
-        load_record_features<C, HALF>(f_next, record);
-    }
-    if (range.x + TT + tid < range.y) next_slot = inst_slots[range.x + TT + tid];
+    Gather<C> g;
+    start_gather<T, C, HALF>(g, inst_slots, records, stride, range);
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        const Header h = h_next;
-        float f[C];
-#pragma unroll
-        for (int c = 0; c < C; ++c) f[c] = f_next[c];
-        if (begin + TT + tid < range.y) {
-            const char* record = records + (size_t)next_slot * stride;
-            h_next = read_header(record);
-            load_record_features<C, HALF>(f_next, record);
-        }
-        if (begin + 2 * TT + tid < range.y) next_slot = inst_slots[begin + 2 * TT + tid];
-        stage_instance<T, C, false>(st, valid, h, f, tile_x0, tile_y0);
+        stage_instance<T, C, false>(st, valid, g.h, g.f, tile_x0, tile_y0);
         BWD_MARK(0);
         __syncthreads();
         BWD_MARK(1);
 
         // ---- consume: this wave's list
-        uint32_t total = 0;
-#pragma unroll
-        for (int s = 0; s < NQ; ++s) total += st.count[wave][s];
+        const ListIndex<NQ> li = list_index<T, C, false>(st, wave);
+        const uint32_t total = li.end[NQ - 1];
         for (uint32_t sub = 0; sub < total; sub += 64u) {
             const bool live = sub + lane < total;
-            const uint32_t j = live ? list_entry<T, C, false>(st, wave, sub + lane) : 0u;
+            const uint32_t j = live ? list_entry<T, C, false>(st, li, wave, sub + lane) : 0u;
             LaneFragments<NF> lf;
             load_lane_fragments<T, C, false>(st, wave, live, j, __ballot(done), lf);
             float feat[C];
@@ -595,7 +653,13 @@ __global__ void __launch_bounds__(T* T)
             build_fragment_lists<NF>(qs, st.opacity[j], lf, my_start, my_count, n_fragments, [&](int q) {
                 float d = 0.0f;  // features . grad of the fragment's pixel
 #pragma unroll
-                for (int c = 0; c < C; ++c) d = fmaf(feat[c], s_grad[wave][c][lf.pixel[q]], d);
+                for (int q4 = 0; q4 < C / 4; ++q4) {
+                    const float4 gr = s_grad[wave][lf.pixel[q]][q4];
+                    d = fmaf(feat[4 * q4], gr.x, d);
+                    d = fmaf(feat[4 * q4 + 1], gr.y, d);
+                    d = fmaf(feat[4 * q4 + 2], gr.z, d);
+                    d = fmaf(feat[4 * q4 + 3], gr.w, d);
+                }
                 return d;
             });
             BWD_MARK(2);
@@ -670,6 +734,10 @@ __global__ void __launch_bounds__(T* T)
 #if defined(INPC_PROFILE_BACKWARD) && defined(INPC_BLEND_PROFILE)
         ++prof_batches;
 #endif
+        // ---- the gather moves on before the stores of the write phase (see the forward kernel)
+        const uint32_t point = g.h.point;
+        const bool multi = g.h.multi();
+        advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
         // ---- write: thread t owns staged instance t: gradient of the point from its fragments in all quads
         if (valid) {
             float gf[C];
@@ -687,21 +755,27 @@ __global__ void __launch_bounds__(T* T)
                         any_weight = true;
                         const uint32_t pix = st.pixel[q][k][tid];
 #pragma unroll
-                        for (int c = 0; c < C; ++c) gf[c] = fmaf(e.x, s_grad[q][c][pix], gf[c]);
+                        for (int q4 = 0; q4 < C / 4; ++q4) {
+                            const float4 gr = s_grad[q][pix][q4];
+                            gf[4 * q4] = fmaf(e.x, gr.x, gf[4 * q4]);
+                            gf[4 * q4 + 1] = fmaf(e.x, gr.y, gf[4 * q4 + 1]);
+                            gf[4 * q4 + 2] = fmaf(e.x, gr.z, gf[4 * q4 + 2]);
+                            gf[4 * q4 + 3] = fmaf(e.x, gr.w, gf[4 * q4 + 3]);
+                        }
                     }
                 }
             if (any_weight || gop != 0.0f) {
-                float* dst = grad_view + (size_t)h.point * C;
-                if (h.multi) {
+                float* dst = grad_view + (size_t)point * C;
+                if (multi) {
 #pragma unroll
                     for (int c = 0; c < C; ++c)
                         if (gf[c] != 0.0f) atomicAdd(dst + c, gf[c]);
-                    if (gop != 0.0f) atomicAdd(&grad_opacities[h.point], gop);
+                    if (gop != 0.0f) atomicAdd(&grad_opacities[point], gop);
                 } else {
 #pragma unroll
                     for (int q4 = 0; q4 < C / 4; ++q4)
                         ((float4*)dst)[q4] = make_float4(gf[4 * q4], gf[4 * q4 + 1], gf[4 * q4 + 2], gf[4 * q4 + 3]);
-                    grad_opacities[h.point] = gop;
+                    grad_opacities[point] = gop;
                 }
             }
         }

@@ -62,6 +62,13 @@ int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream);
 // ------------------------------------------------------------------------------------------------
 constexpr int kWave = 64;
 
+// Orders the LDS traffic of one wave: everything issued before is visible to every lane after.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 __device__ __forceinline__ uint32_t lane_id() { return __lane_id(); }
 
 // Number of set bits of `mask` below the calling lane.

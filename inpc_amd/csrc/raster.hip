@@ -29,6 +29,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <type_traits>
 
 #include "common.hpp"
 #include "radix.hpp"
@@ -255,6 +256,16 @@ __global__ void __launch_bounds__(kScanBlock) k_bin_scan(const uint32_t* __restr
 }
 
 // ---- preprocess -------------------------------------------------------------------------------------------
+// Size of a record in 16-byte words, per feature mode and channel count (record_stride() / 16).
+template <int FMODE, int C>
+struct PreprocessShape {
+    static constexpr bool kHalf = FMODE == INPC_FEAT_DIRECT_F16;
+    static constexpr bool kDirect = FMODE == INPC_FEAT_DIRECT_F32 || kHalf;
+    static constexpr uint32_t kBytes = kRecordHeader + (kDirect ? C * (kHalf ? 2 : 4) : 16);
+    static constexpr uint32_t kStrideWords = (kBytes + 31u) / 32u * 2u;
+    static constexpr size_t kStageBytes = (size_t)kBinThreads * (kStrideWords + 1) * 16;   // padded rows, per block
+};
+
 template <int T, int FMODE, int C>
 __global__ void __launch_bounds__(kBinThreads)
     k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
@@ -263,9 +274,10 @@ __global__ void __launch_bounds__(kBinThreads)
                  const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start,
                  uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, float* __restrict__ blending_weights,
                  uint32_t* counters, uint32_t* g_hist, Geometry g, radix::DevicePlan plan) {
-    extern __shared__ uint32_t s_dyn[];
-    uint32_t* s_cursor = s_dyn;                 // n_tiles
-    uint32_t* s_hist = s_dyn + g.n_tiles;       // kMaxPasses * kRadix
+    extern __shared__ __align__(16) uint32_t s_dyn[];
+    float4* s_stage = (float4*)s_dyn;                                           // record staging, 64 rows per wave
+    uint32_t* s_cursor = s_dyn + PreprocessShape<FMODE, C>::kStageBytes / 4;     // n_tiles
+    uint32_t* s_hist = s_cursor + g.n_tiles;                                    // kMaxPasses * kRadix
     __shared__ uint32_t s_visible, s_instances;
     {
         const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
@@ -281,47 +293,84 @@ __global__ void __launch_bounds__(kBinThreads)
     uint32_t my_visible = 0, my_instances = 0;
     const uint32_t chunk = bin_chunk_size(g.n);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
-    for (uint32_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
-        const float px = positions[3 * (size_t)i], py = positions[3 * (size_t)i + 1], pz = positions[3 * (size_t)i + 2];
-        const Projected p = project_point<T>(m, g, px, py, pz);
-        uint32_t key = radix::kInvalidKey, val = 0u;
-        if (p.info) {
-            key = __float_as_uint(p.depth) - g.key_bias;
-            my_visible += 1u;
-            my_instances += p.touched;
-            radix::hist_add(s_hist, plan, key);
-            const uint32_t slot = atomicAdd(&s_cursor[info_tile0(p.info)], 1u);
-            val = (slot << 2) | ((p.info >> 16) & 3u);
-            float4* rec = (float4*)(records + (size_t)slot * g.stride);
-            float opacity;
-            if (FMODE == INPC_FEAT_SH36_F16 || FMODE == INPC_FEAT_RAW37_F16) {
-                const ShBasis s = sh_basis(px, py, pz, cam_position);
-                if (FMODE == INPC_FEAT_SH36_F16) {
-                    rec[2] = sh_to_view(s, (const __half*)features + 36 * (size_t)i);
-                    opacity = opacities[i];
-                } else {
-                    const __half* raw = (const __half*)features + 37 * (size_t)i;
-                    rec[2] = sh_to_view(s, raw + 1);
-                    opacity = 1.0f - expf(-expf(__half2float(raw[0])));  // kernels.cu:142
-                }
-            } else if (FMODE == INPC_FEAT_DIRECT_F32) {
-                const float4* src = (const float4*)features + (size_t)i * (C / 4);
+    // kUnroll points per thread and round, their loads issued together. A record leaves the block through LDS:
+    // every lane assembles its record in the wave's staging rows, then neighbouring lanes write the 16-byte
+    // words of one record, so that a store instruction covers whole records (contiguous 64 bytes and more)
+    // instead of one word of 64 different records.
+    constexpr bool kDirect = FMODE == INPC_FEAT_DIRECT_F32 || FMODE == INPC_FEAT_DIRECT_F16;
+    constexpr int kUnroll = kDirect ? 4 : 2;
+    using Word = std::conditional_t<FMODE == INPC_FEAT_DIRECT_F16, uint2, float4>;  // four channels
+    constexpr int kWords = kDirect ? C / 4 : 1;
+    constexpr uint32_t kStrideWords = PreprocessShape<FMODE, C>::kStrideWords, kRow = kStrideWords + 1;  // padded row
+    constexpr uint32_t kNoSlot = 0xFFFFFFFFu;
+    const uint32_t lane = threadIdx.x & 63u;
+    float4* stage = s_stage + (threadIdx.x >> 6) * (64u * kRow);
+    for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
+        float px[kUnroll], py[kUnroll], pz[kUnroll], op[kUnroll];
+        Word fw[kUnroll][kWords];
 #pragma unroll
-                for (int q = 0; q < C / 4; ++q) rec[2 + q] = src[q];
-                opacity = opacities[i];
-            } else {
-                const uint2* src = (const uint2*)features + (size_t)i * (C / 4);
-                uint2* dst = (uint2*)(rec + 2);
+        for (int u = 0; u < kUnroll; ++u) {
+            // a thread behind the end reads the chunk's first point and drops it
+            const uint32_t at = base + u * kBinThreads + threadIdx.x;
+            const size_t i = at < end ? at : begin;
+            px[u] = positions[3 * i];
+            py[u] = positions[3 * i + 1];
+            pz[u] = positions[3 * i + 2];
+            op[u] = FMODE == INPC_FEAT_RAW37_F16 ? 0.0f : opacities[i];
+            if (kDirect) {
+                const Word* src = (const Word*)features + i * kWords;
 #pragma unroll
-                for (int q = 0; q < C / 4; ++q) dst[q] = src[q];
-                opacity = opacities[i];
+                for (int q = 0; q < kWords; ++q) fw[u][q] = src[q];
             }
-            rec[0] = make_float4(p.sx, p.sy, opacity, __uint_as_float(i));
-            rec[1] = make_float4(__uint_as_float(p.info), p.depth, 0.0f, 0.0f);
         }
-        keys[i] = key;
-        vals[i] = val;
-        if (blending_weights) blending_weights[i] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t i = base + u * kBinThreads + threadIdx.x;
+            uint32_t slot = kNoSlot;
+            if (i < end) {
+                const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
+                uint32_t key = radix::kInvalidKey, val = 0u;
+                if (p.info) {
+                    key = __float_as_uint(p.depth) - g.key_bias;
+                    my_visible += 1u;
+                    my_instances += p.touched;
+                    radix::hist_add(s_hist, plan, key);
+                    slot = atomicAdd(&s_cursor[info_tile0(p.info)], 1u);
+                    val = (slot << 2) | ((p.info >> 16) & 3u);
+                    float4* rec = stage + lane * kRow;
+                    float opacity = op[u];
+#pragma unroll
+                    for (uint32_t w = 2; w < kStrideWords; ++w) rec[w] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    if (kDirect) {
+                        Word* dst = (Word*)(rec + 2);
+#pragma unroll
+                        for (int q = 0; q < kWords; ++q) dst[q] = fw[u][q];
+                    } else {
+                        const ShBasis sb = sh_basis(px[u], py[u], pz[u], cam_position);
+                        if (FMODE == INPC_FEAT_SH36_F16) {
+                            rec[2] = sh_to_view(sb, (const __half*)features + 36 * (size_t)i);
+                        } else {
+                            const __half* raw = (const __half*)features + 37 * (size_t)i;
+                            rec[2] = sh_to_view(sb, raw + 1);
+                            opacity = 1.0f - expf(-expf(__half2float(raw[0])));  // kernels.cu:142
+                        }
+                    }
+                    rec[0] = make_float4(p.sx, p.sy, opacity, __uint_as_float(i));
+                    rec[1] = make_float4(__uint_as_float(p.info), p.depth, 0.0f, 0.0f);
+                }
+                keys[i] = key;
+                vals[i] = val;
+                if (blending_weights) blending_weights[i] = 0.0f;
+            }
+            wave_sync();
+#pragma unroll
+            for (uint32_t k = 0; k < kStrideWords; ++k) {
+                const uint32_t flat = k * 64u + lane, r = flat / kStrideWords, w = flat % kStrideWords;
+                const uint32_t to = __shfl(slot, r, 64);
+                if (to != kNoSlot) ((float4*)(records + (size_t)to * g.stride))[w] = stage[r * kRow + w];
+            }
+            wave_sync();
+        }
     }
     // block totals -> one global atomic each
     for (int s = 32; s > 0; s >>= 1) {
@@ -667,7 +716,9 @@ template <int T, int FMODE, int C>
 int launch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
                       const float* w2c, const float* cam_position, float* blending_weights, void* ws,
                       hipStream_t stream) {
-    const size_t lds = ((size_t)L.geo.n_tiles + radix::kMaxPasses * radix::kRadix) * 4;
+    const size_t lds = PreprocessShape<FMODE, C>::kStageBytes + ((size_t)L.geo.n_tiles + radix::kMaxPasses * radix::kRadix) * 4;
+    if (L.pub.record_stride != PreprocessShape<FMODE, C>::kStrideWords * 16u)
+        return fail(INPC_E_UNSUPPORTED, "record stride %u does not match the preprocess kernel", L.pub.record_stride);
     INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream,
                     positions, features, opacities, w2c, cam_position, at<char>(ws, L.pub.point_record),
                     (const uint32_t*)at<uint32_t>(ws, L.bin_table), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
