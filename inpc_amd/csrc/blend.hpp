@@ -7,12 +7,12 @@
 // four waves evenly. Per batch of T*T instances:
 //   stage    thread t gathers the record of instance t into LDS, finds the waves ("quads") in which it covers a
 //            pixel that is still open, and appends t, in depth order, to the list of each such quad;
-//   consume  every wave walks its own list, 64 instances at a time, with wave-level
-//            synchronisation only: coverage bit masks per pixel column / row -> per-pixel fragment lists
-//            in depth order -> the sequential transmittance chain per pixel (short lists) or a wave-wide
-//            product scan (long lists) -> per-instance results into LDS;
-//   write    thread t writes the result of instance t: a plain store when the point lies in one tile only,
-//            atomics when it straddles tiles.
+//   consume  every wave takes its whole list at once (up to four entries per lane), with wave-level
+//            synchronisation only: hit masks per pixel -> per-pixel fragment lists in depth order -> the
+//            sequential transmittance chain per pixel (short lists) or a wave-wide product scan (long
+//            lists); the results stay in the fragment list;
+//   write    thread t collects the results of instance t's fragments: a plain store when the point lies in
+//            one tile only, atomics when it straddles tiles.
 // Two block barriers per batch; the record gather runs two batches ahead of the blend.
 #pragma once
 
@@ -20,9 +20,15 @@ namespace blend {
 
 constexpr int kQuad = 8;             // a wave's pixel quad is 8 x 8
 #ifndef INPC_LONG_LIST
-#define INPC_LONG_LIST 12
+#define INPC_LONG_LIST 32
 #endif
-constexpr uint32_t kLongList = INPC_LONG_LIST;  // lists longer than this are evaluated by the whole wave
+constexpr uint32_t kLongList = INPC_LONG_LIST;
+#ifndef INPC_FWD_WAVES
+#define INPC_FWD_WAVES 1
+#endif
+#ifndef INPC_BWD_WAVES
+#define INPC_BWD_WAVES 1
+#endif  // lists longer than this are evaluated by the whole wave
 
 __device__ __forceinline__ uint64_t lanes_below() {
     const uint32_t lane = __lane_id();
@@ -90,33 +96,47 @@ __device__ __forceinline__ uint32_t wave_exclusive_sum(uint32_t v, uint32_t& tot
     return incl - v;
 }
 
-// Per-block staging area of one batch.
+// Shape of the work per tile size.
 //   NQ  waves ("quads") per tile
 //   NF  fragments one instance can have inside one wave's pixel grid: 4 (8x8 tiles: the whole 2 x 2 footprint),
 //       1 (16x16 tiles: one pixel per parity class)
+//   K   list entries a lane takes per batch: a quad's list has up to T*T = 64 K entries
+// Either way an instance has four fragment slots in the tile (slot = quad for 16x16 tiles, = candidate pixel
+// ky * 2 + kx for 8x8 tiles) and a wave handles up to 256 fragments per batch.
+template <int T>
+struct Shape {
+    static constexpr int TT = T * T;
+    static constexpr int NQ = TT / 64;
+    static constexpr int NF = T == 16 ? 1 : 4;
+    static constexpr int K = T == 16 ? 4 : 1;
+};
+
+// Fragment field of a staged instance (16 bits per slot): bits 0-5 the pixel in the owning wave's grid
+// (row * 8 + column), bit 6: the instance has no fragment in this slot, bit 7: the wave has placed the
+// fragment in its list, bits 8-15: where.
+constexpr uint32_t kPixelMask = 63u, kNoFragment = 0x40u, kPlaced = 0x80u;
+constexpr uint32_t kNoPixel = 0xFFu;
+
+// Per-block staging area of one batch.
 template <int T, int C, bool WITH_DEPTH>
 struct Stage {
     static constexpr int TT = T * T;
     static constexpr int NQ = TT / 64;
-    static constexpr int NF = T == 16 ? 1 : 4;
-    float opacity[TT];
     float4 feat[TT * (C / 4)];
     float depth[WITH_DEPTH ? TT : 1];
-    float weight[NQ][NF][TT];   // interpolation weight of the fragment
-    uint8_t pixel[NQ][NF][TT];  // its pixel in the wave's grid (row * 8 + column), kNoPixel: no fragment
-    float2 result[NQ][NF][TT];  // what the blend made of the fragment (written by the quad's wave, else {0, 0})
-    uint8_t list[NQ][NQ][64];   // [quad][source wave][rank]: staged instances with an open pixel in the quad
+    alignas(16) float alpha[TT][4];     // per slot: opacity x interpolation weight
+    alignas(8) uint16_t frag[TT][4];    // per slot: the fragment field
+    uint8_t list[NQ][NQ][64];           // [quad][source wave][rank]: staged instances with an open pixel in the quad
     uint8_t count[NQ][NQ];
-    uint64_t done[NQ];          // per quad: pixels that are finished
+    uint64_t done[NQ];                  // per quad: pixels that are finished
 };
-constexpr uint32_t kNoPixel = 0xFFu;
 
 // Per-wave scratch of the consume phase. A fragment entry is {alpha, x} on the way in and {blending weight, y}
 // on the way out; forward: x = staged instance; backward: x = features . grad, y = d loss / d alpha.
-template <int NF>
+template <int T>
 struct QuadScratch {
-    uint64_t hits[64];          // per pixel: lanes (instances of the sub-batch) that hit it
-    float2 fragment[64 * NF];   // per fragment, pixel by pixel, in depth order
+    uint64_t hits[64][Shape<T>::K];  // per pixel and entry round: lanes whose entry hits the pixel
+    float2 fragment[256];            // per fragment, pixel by pixel, in depth order
 };
 
 // The record header as the kernels use it.
@@ -125,6 +145,7 @@ struct Header {
     uint32_t point;
     uint32_t tiles;  // raw word; see multi()
     float depth;
+    uint32_t split;  // index among the points that touch several tiles
     // the point touches more than one tile (kept as the raw word until the write phase: a flag derived
     // at the load would make the gather wait for its own first reply)
     __device__ __forceinline__ bool multi() const { return ((tiles >> 16) & 3u) != 0u; }
@@ -145,56 +166,72 @@ __device__ __forceinline__ Header read_header(const char* __restrict__ record) {
     h.point = __float_as_uint(h0.w);
     h.tiles = __float_as_uint(h1.x);
     h.depth = h1.y;
+    h.split = __float_as_uint(h1.z);
     return h;
 }
 
-// Stage instance `t` (thread t): features and opacity, the fragment it has in every quad (pixel + weight), and
-// its entry, in depth order, in the list of each quad where it covers an open pixel. `valid` is false for the
-// threads behind the end of the batch. Must be followed by a block barrier.
+// Stage instance `t` (thread t): features, the alpha and pixel of its fragment in every slot, and its entry, in
+// depth order, in the list of each quad where it covers an open pixel. `valid` is false for the threads behind
+// the end of the batch. Leaves the interpolation weights of the four slots in `weight`. Must be followed by a
+// block barrier.
 template <int T, int C, bool WITH_DEPTH>
 __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool valid, const Header& h,
-                                               const float (&f)[C], int tile_x0, int tile_y0) {
+                                               const float (&f)[C], int tile_x0, int tile_y0, float (&weight)[4]) {
     constexpr int NQ = T * T / 64;
     const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
     bool in_quad[NQ];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) in_quad[q] = false;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) weight[c] = 0.0f;
     if (valid) {
-        st.opacity[t] = h.opacity;
 #pragma unroll
         for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
         if (WITH_DEPTH) st.depth[t] = h.depth;
         // the float test of B/rasterization/src/bilinear/kernels.cu:284-287 for the 2 x 2 candidate pixels
         const AxisCover ax = cover_axis<T>(h.sx, tile_x0), ay = cover_axis<T>(h.sy, tile_y0);
+        uint32_t field[4];
+        if (T == 16) {
+            // slot = parity class (y parity, x parity) of the pixel; per axis, the candidate with parity b
+            const bool odd_x = (ax.first & 1) != 0, odd_y = (ay.first & 1) != 0;
+            bool hx[2], hy[2];
+            float wx[2], wy[2];
+            int gx[2], gy[2];
 #pragma unroll
-        for (int ky = 0; ky < 2; ++ky)
-#pragma unroll
-            for (int kx = 0; kx < 2; ++kx) {
-                const bool hit = ax.hit[kx] && ay.hit[ky];
-                const int cx = ax.first + kx, cy = ay.first + ky;
-                if (T == 16) {
-                    // quad = parity class of the pixel; every class has exactly one of the four candidates
-                    const int q = (cy & 1) * 2 + (cx & 1);
-                    const int pix = hit ? (cy >> 1) * 8 + (cx >> 1) : 0;
-                    const bool open = hit && ((st.done[q] >> pix) & 1ull) == 0ull;
-                    st.pixel[q][0][t] = hit ? (uint8_t)pix : (uint8_t)kNoPixel;
-                    st.weight[q][0][t] = ax.weight[kx] * ay.weight[ky];
-#pragma unroll
-                    for (int qq = 0; qq < NQ; ++qq)
-                        if (qq == q && open) in_quad[qq] = true;
-                } else {
-                    const int pix = hit ? cy * 8 + cx : 0;
-                    const bool open = hit && ((st.done[0] >> pix) & 1ull) == 0ull;
-                    st.pixel[0][ky * 2 + kx][t] = hit ? (uint8_t)pix : (uint8_t)kNoPixel;
-                    st.weight[0][ky * 2 + kx][t] = ax.weight[kx] * ay.weight[ky];
-                    if (open) in_quad[0] = true;
-                }
+            for (int b = 0; b < 2; ++b) {
+                const bool second_x = odd_x != (b != 0), second_y = odd_y != (b != 0);   // candidate 1 has parity b
+                hx[b] = second_x ? ax.hit[1] : ax.hit[0];
+                wx[b] = second_x ? ax.weight[1] : ax.weight[0];
+                gx[b] = (ax.first + (second_x ? 1 : 0)) >> 1;
+                hy[b] = second_y ? ay.hit[1] : ay.hit[0];
+                wy[b] = second_y ? ay.weight[1] : ay.weight[0];
+                gy[b] = (ay.first + (second_y ? 1 : 0)) >> 1;
             }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int by = c >> 1, bx = c & 1;
+                const bool hit = hx[bx] && hy[by];
+                const int pix = hit ? gy[by] * 8 + gx[bx] : 0;
+                weight[c] = wx[bx] * wy[by];
+                field[c] = hit ? (uint32_t)pix : kNoFragment;
+                in_quad[c] = hit && ((st.done[c] >> pix) & 1ull) == 0ull;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int ky = c >> 1, kx = c & 1;
+                const bool hit = ax.hit[kx] && ay.hit[ky];
+                const int pix = hit ? (ay.first + ky) * 8 + (ax.first + kx) : 0;
+                weight[c] = ax.weight[kx] * ay.weight[ky];
+                field[c] = hit ? (uint32_t)pix : kNoFragment;
+                if (hit && ((st.done[0] >> pix) & 1ull) == 0ull) in_quad[0] = true;
+            }
+        }
+        const float4 alpha = make_float4(h.opacity * weight[0], h.opacity * weight[1], h.opacity * weight[2], h.opacity * weight[3]);
+        __builtin_memcpy(st.alpha[t], &alpha, 16);
+        const uint2 fields = make_uint2(field[0] | (field[1] << 16), field[2] | (field[3] << 16));
+        __builtin_memcpy(st.frag[t], &fields, 8);
     }
-#pragma unroll
-    for (int q = 0; q < NQ; ++q)
-#pragma unroll
-        for (int k = 0; k < Stage<T, C, WITH_DEPTH>::NF; ++k) st.result[q][k][t] = make_float2(0.0f, 0.0f);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
         const uint64_t members = __ballot(in_quad[q]);
@@ -238,62 +275,107 @@ __device__ __forceinline__ uint32_t list_entry(const Stage<T, C, WITH_DEPTH>& st
     return st.list[q][w][idx - first];
 }
 
-// Fragments of one sub-batch lane: the (at most NF) pixels staged instance j covers in this wave's grid.
-template <int NF>
-struct LaneFragments {
-    uint32_t pixel[NF];  // kNoPixel: none, or the pixel is finished
-    float weight[NF];
-    uint32_t where[NF];  // position in the fragment list (valid when pixel != kNoPixel)
+// The list entries of one lane: entry k is number k * 64 + lane of the quad's list; its (at most NF) fragments
+// in this wave's grid. Depth order is the order of (k, lane).
+template <int T>
+struct Entries {
+    static constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
+    uint32_t j[K];           // staged instance (0 for an entry behind the end of the list)
+    uint32_t pixel[K][NF];   // kNoPixel: no fragment, or the pixel is finished
+    float alpha[K][NF];
 };
 
-// Per-pixel fragment lists of one sub-batch. In: every lane's fragments (pixel, weight), the alpha factor
-// `opacity`, and payload(q), the second word of fragment q's entry. Out: every pixel lane's list
-// [my_start, my_start + my_count) of {alpha, payload} in depth order in qs.fragment, and `where` for every
-// fragment. Every lane of the wave must call it.
-template <int NF, typename Payload>
-__device__ __forceinline__ void build_fragment_lists(QuadScratch<NF>& qs, float opacity, LaneFragments<NF>& lf,
-                                                     uint32_t& my_start, uint32_t& my_count, uint32_t& n_fragments,
-                                                     Payload payload) {
+template <int T, int C, bool WITH_DEPTH>
+__device__ __forceinline__ void load_entries(const Stage<T, C, WITH_DEPTH>& st, const ListIndex<T * T / 64>& li,
+                                             uint32_t quad, uint64_t finished, Entries<T>& e) {
+    constexpr int K = Shape<T>::K, NF = Shape<T>::NF, NQ = T * T / 64;
     const uint32_t lane = __lane_id();
-    qs.hits[lane] = 0ull;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t idx = k * 64u + lane;
+        const bool live = idx < li.end[NQ - 1];
+        const uint32_t j = live ? list_entry<T, C, WITH_DEPTH>(st, li, quad, idx) : 0u;
+        e.j[k] = j;
+        uint32_t field[NF];
+        if (T == 16) {
+            field[0] = st.frag[j][quad];
+            e.alpha[k][0] = st.alpha[j][quad];
+        } else {
+            uint2 fields;
+            float4 alpha;
+            __builtin_memcpy(&fields, st.frag[j], 8);
+            __builtin_memcpy(&alpha, st.alpha[j], 16);
+            field[0] = fields.x & 0xFFFFu;
+            field[NF > 1 ? 1 : 0] = fields.x >> 16;
+            field[NF > 2 ? 2 : 0] = fields.y & 0xFFFFu;
+            field[NF > 3 ? 3 : 0] = fields.y >> 16;
+            e.alpha[k][0] = alpha.x;
+            e.alpha[k][NF > 1 ? 1 : 0] = alpha.y;
+            e.alpha[k][NF > 2 ? 2 : 0] = alpha.z;
+            e.alpha[k][NF > 3 ? 3 : 0] = alpha.w;
+        }
+#pragma unroll
+        for (int q = 0; q < NF; ++q) {
+            uint32_t pix = (live && !(field[q] & kNoFragment)) ? (field[q] & kPixelMask) : kNoPixel;
+            if (pix != kNoPixel && ((finished >> pix) & 1ull)) pix = kNoPixel;
+            e.pixel[k][q] = pix;
+        }
+    }
+}
+
+// Per-pixel fragment lists of one batch. In: the lane's entries and payload(k, q), the second word of a
+// fragment's entry. Out: every pixel lane's list [my_start, my_start + my_count) of {alpha, payload} in depth
+// order in qs.fragment, and in the stage, for every fragment placed, where it is. Every lane of the wave
+// must call it.
+template <int T, int C, bool WITH_DEPTH, typename Payload>
+__device__ __forceinline__ void build_fragment_lists(QuadScratch<T>& qs, Stage<T, C, WITH_DEPTH>& st, uint32_t quad,
+                                                     const Entries<T>& e, uint32_t& my_start, uint32_t& my_count,
+                                                     uint32_t& n_fragments, Payload payload) {
+    constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
+    const uint32_t lane = __lane_id();
+#pragma unroll
+    for (int k = 0; k < K; ++k) qs.hits[lane][k] = 0ull;
     wave_sync();
     const unsigned long long bit = 1ull << lane;
 #pragma unroll
-    for (int q = 0; q < NF; ++q)
-        if (lf.pixel[q] != kNoPixel) atomicOr((unsigned long long*)&qs.hits[lf.pixel[q]], bit);
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+        for (int q = 0; q < NF; ++q)
+            if (e.pixel[k][q] != kNoPixel) atomicOr((unsigned long long*)&qs.hits[e.pixel[k][q]][k], bit);
     wave_sync();
-    my_count = (uint32_t)__popcll(qs.hits[lane]);
+    my_count = 0u;
+#pragma unroll
+    for (int k = 0; k < K; ++k) my_count += (uint32_t)__popcll(qs.hits[lane][k]);
     my_start = wave_exclusive_sum(my_count, n_fragments);
     if (n_fragments == 0u) return;
     const uint64_t below = lanes_below();
 #pragma unroll
-    for (int q = 0; q < NF; ++q) {
-        const bool hit = lf.pixel[q] != kNoPixel;
-        const uint32_t pix = hit ? lf.pixel[q] : 0u;
-        const uint32_t start = __shfl(my_start, pix, 64);  // every lane takes part in the exchange
-        if (hit) {
-            const uint32_t pos = start + (uint32_t)__popcll(qs.hits[pix] & below);
-            lf.where[q] = pos;
-            qs.fragment[pos] = make_float2(opacity * lf.weight[q], payload(q));
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+        for (int q = 0; q < NF; ++q) {
+            const bool hit = e.pixel[k][q] != kNoPixel;
+            const uint32_t pix = hit ? e.pixel[k][q] : 0u;
+            const uint32_t start = __shfl(my_start, pix, 64);  // every lane takes part in the exchange
+            if (hit) {
+                uint32_t pos = start + (uint32_t)__popcll(qs.hits[pix][k] & below);
+#pragma unroll
+                for (int kk = 0; kk < k; ++kk) pos += (uint32_t)__popcll(qs.hits[pix][kk]);
+                qs.fragment[pos] = make_float2(e.alpha[k][q], payload(k, q));
+                st.frag[e.j[k]][T == 16 ? quad : q] = (uint16_t)((pos << 8) | pix | kPlaced);
+            }
         }
-    }
     wave_sync();
 }
 
-// Lane l of a sub-batch: its staged instance and fragments (pixels that finished since staging are dropped).
+// Fragment fields of staged instance t, one per slot.
 template <int T, int C, bool WITH_DEPTH>
-__device__ __forceinline__ void load_lane_fragments(const Stage<T, C, WITH_DEPTH>& st, uint32_t quad, bool live,
-                                                    uint32_t j, uint64_t finished,
-                                                    LaneFragments<Stage<T, C, WITH_DEPTH>::NF>& lf) {
-    constexpr int NF = Stage<T, C, WITH_DEPTH>::NF;
-#pragma unroll
-    for (int q = 0; q < NF; ++q) {
-        uint32_t pix = live ? (uint32_t)st.pixel[quad][q][j] : kNoPixel;
-        if (pix != kNoPixel && ((finished >> pix) & 1ull)) pix = kNoPixel;
-        lf.pixel[q] = pix;
-        lf.weight[q] = st.weight[quad][q][j];
-        lf.where[q] = 0u;
-    }
+__device__ __forceinline__ void load_fields(const Stage<T, C, WITH_DEPTH>& st, uint32_t t, uint32_t (&field)[4]) {
+    uint2 fields;
+    __builtin_memcpy(&fields, st.frag[t], 8);
+    field[0] = fields.x & 0xFFFFu;
+    field[1] = fields.x >> 16;
+    field[2] = fields.y & 0xFFFFu;
+    field[3] = fields.y >> 16;
 }
 
 // ---- the record gather, two batches ahead -------------------------------------------------------------------------
@@ -349,6 +431,7 @@ __device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __r
     arrive(g.h_next.point);
     arrive(g.h_next.tiles);
     arrive(g.h_next.depth);
+    arrive(g.h_next.split);
 #pragma unroll
     for (int c = 0; c < C; ++c) arrive(g.f_next[c]);
     arrive(g.next_slot);
@@ -365,7 +448,7 @@ __device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __r
 
 // ---- forward ------------------------------------------------------------------------------------------------------
 template <int T, int C, bool HALF, bool INFERENCE>
-__global__ void __launch_bounds__(T* T)
+__global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1)
     k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
                     const uint32_t* __restrict__ inst_slots,
                     const char* __restrict__ records, uint32_t stride, float* __restrict__ image,
@@ -373,9 +456,8 @@ __global__ void __launch_bounds__(T* T)
                     int H, uint32_t gw) {
     constexpr int TT = T * T;
     constexpr int NQ = TT / 64;
-    constexpr int NF = Stage<T, C, INFERENCE>::NF;
     __shared__ Stage<T, C, INFERENCE> st;
-    __shared__ QuadScratch<NF> s_quad[NQ];
+    __shared__ QuadScratch<T> s_quad[NQ];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tile = tile_order[blockIdx.x];
@@ -383,7 +465,7 @@ __global__ void __launch_bounds__(T* T)
     const int px = tile_x0 + (T == 16 ? 2 * (int)(lane & 7u) + (int)(wave & 1u) : (int)(lane & 7u));
     const int py = tile_y0 + (T == 16 ? 2 * (int)(lane >> 3) + (int)(wave >> 1) : (int)(lane >> 3));
     const bool inside = px < W && py < H;
-    QuadScratch<NF>& qs = s_quad[wave];
+    QuadScratch<T>& qs = s_quad[wave];
 
     float F[C];
 #pragma unroll
@@ -408,24 +490,23 @@ __global__ void __launch_bounds__(T* T)
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f, tile_x0, tile_y0);
+        float weight[4];
+        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f, tile_x0, tile_y0, weight);
         FWD_MARK(0);
         __syncthreads();
         FWD_MARK(1);
 
         // ---- consume: this wave's list
         const ListIndex<NQ> li = list_index<T, C, INFERENCE>(st, wave);
-        const uint32_t total = li.end[NQ - 1];
-        for (uint32_t sub = 0; sub < total; sub += 64u) {
-            const bool live = sub + lane < total;
-            const uint32_t j = live ? list_entry<T, C, INFERENCE>(st, li, wave, sub + lane) : 0u;
-            LaneFragments<NF> lf;
-            load_lane_fragments<T, C, INFERENCE>(st, wave, live, j, __ballot(done), lf);
-            uint32_t my_start, my_count, n_fragments;
-            build_fragment_lists<NF>(qs, st.opacity[j], lf, my_start, my_count, n_fragments,
-                                     [&](int) { return __uint_as_float(j); });
-            FWD_MARK(2);
-            if (n_fragments == 0u) continue;
+        uint32_t my_start = 0, my_count = 0, n_fragments = 0;
+        if (li.end[NQ - 1] != 0u) {
+            Entries<T> e;
+            load_entries<T, C, INFERENCE>(st, li, wave, __ballot(done), e);
+            build_fragment_lists<T, C, INFERENCE>(qs, st, wave, e, my_start, my_count, n_fragments,
+                                                  [&](int k, int) { return __uint_as_float(e.j[k]); });
+        }
+        FWD_MARK(2);
+        if (n_fragments != 0u) {
             // ---- pixels with short lists: the reference's sequential walk (kernels.cu:281-299)
             if (my_count <= kLongList) {
                 for (uint32_t i = 0; i < my_count; ++i) {
@@ -505,14 +586,7 @@ __global__ void __launch_bounds__(T* T)
                     done = Tr < kTransmittanceThreshold;
                 }
             }
-            wave_sync();
             FWD_MARK(4);
-            // ---- instances: hand the blending weights of the fragments to the thread that owns the instance
-            if (!INFERENCE) {
-#pragma unroll
-                for (int q = 0; q < NF; ++q)
-                    if (lf.pixel[q] != kNoPixel) st.result[wave][q][j] = qs.fragment[lf.where[q]];
-            }
         }
         {
             const uint64_t finished = __ballot(done);
@@ -528,15 +602,17 @@ __global__ void __launch_bounds__(T* T)
         const uint32_t point = g.h.point;
         const bool multi = g.h.multi();
         advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
-        // ---- write: thread t owns staged instance t (kernels.cu:291-295)
+        // ---- write: thread t owns staged instance t (kernels.cu:291-295): its blending weight is the sum over
+        // the fragments the waves placed
         if (!INFERENCE && valid) {
+            uint32_t field[4];
+            load_fields<T, C, INFERENCE>(st, tid, field);
             float w = 0.0f;
 #pragma unroll
-            for (int q = 0; q < NQ; ++q)
-#pragma unroll
-                for (int k = 0; k < NF; ++k) {
-                    const float bw = st.result[q][k][tid].x;
-                    if (bw > 0.0f) w = fmaf(bw, st.weight[q][k][tid], w);
+            for (int c = 0; c < 4; ++c)
+                if (field[c] & kPlaced) {
+                    const float bw = s_quad[T == 16 ? c : 0].fragment[field[c] >> 8].x;
+                    if (bw > 0.0f) w = fmaf(bw, weight[c], w);
                 }
             if (w > 0.0f) {
                 if (multi) atomicAdd(&blending_weights[point], w);
@@ -559,23 +635,76 @@ __global__ void __launch_bounds__(T* T)
     }
 }
 
+// ---- gradients of points that straddle tiles --------------------------------------------------------------------
+// A point that touches several tiles has an index s among such points (record header) and four rows, one per
+// tile: features[4 s + part][C], opacities[4 s + part], and a flag byte per row in flags[s]: the row has been
+// written. The flags are zero after the forward pass and after k_grad_reduce.
+struct SplitRows {
+    float* features;
+    float* opacities;
+    uint32_t* flags;
+    const uint32_t* points;   // points[s]: the point
+    const uint32_t* count;    // number of such points
+};
+
+// Which of the (at most 2 x 2) tiles of a point `tile` is: 0 the first (top left), 1 its right neighbour,
+// 2 the one below, 3 the one below right. `info` is the tile word of the record.
+__device__ __forceinline__ uint32_t tile_part(uint32_t tile, uint32_t info, uint32_t gw) {
+    const uint32_t delta = tile - (info & 0xFFFFu);
+    return delta >= gw ? 2u + (delta - gw) : delta;
+}
+
+// gradient of the point = sum of its rows, in row order (the gradient buffers are zero before)
+template <int C>
+__global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __restrict__ grad_view,
+                                                     float* __restrict__ grad_opacities) {
+    const uint32_t n = *rows.count;
+    for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < n; s += gridDim.x * 256u) {
+        const uint32_t flags = rows.flags[s];
+        if (flags == 0u) continue;
+        rows.flags[s] = 0u;
+        const uint32_t i = rows.points[s];
+        float4 acc[C / 4];
+#pragma unroll
+        for (int q4 = 0; q4 < C / 4; ++q4) acc[q4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float opacity = 0.0f;
+#pragma unroll
+        for (uint32_t part = 0; part < 4u; ++part)
+            if ((flags >> (8u * part)) & 0xFFu) {
+                const float4* row = (const float4*)(rows.features + ((size_t)s * 4u + part) * C);
+#pragma unroll
+                for (int q4 = 0; q4 < C / 4; ++q4) {
+                    const float4 r = row[q4];
+                    acc[q4].x += r.x;
+                    acc[q4].y += r.y;
+                    acc[q4].z += r.z;
+                    acc[q4].w += r.w;
+                }
+                opacity += rows.opacities[(size_t)s * 4u + part];
+            }
+#pragma unroll
+        for (int q4 = 0; q4 < C / 4; ++q4) ((float4*)(grad_view + (size_t)i * C))[q4] = acc[q4];
+        grad_opacities[i] = opacity;
+    }
+}
+
 // ---- backward -----------------------------------------------------------------------------------------------------
 // With s = features . grad of a fragment, R the running sum of weight x s of a pixel and S its final value
 // image . grad, the opacity gradient of the reference (kernels.cu:405-413),
 //   dot(T f + (F_running - F_final) / (1 - a), grad) + grad_alpha (1 - alpha_final) / (1 - a),
 // is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the pixel walk carries two scalars, not 2C.
 template <int T, int C, bool HALF>
-__global__ void __launch_bounds__(T* T)
+__global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1)   // 16x16 tiles: registers for four blocks per CU
     k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
                      const uint32_t* __restrict__ inst_slots, const char* __restrict__ records, uint32_t stride,
                      const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
                      const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_view,
-                     float* grad_opacities, int W, int H, uint32_t gw) {
+                     float* grad_opacities, SplitRows rows, int W, int H, uint32_t gw) {
     constexpr int TT = T * T;
     constexpr int NQ = TT / 64;
-    constexpr int NF = Stage<T, C, false>::NF;
+    constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
     __shared__ Stage<T, C, false> st;
-    __shared__ QuadScratch<NF> s_quad[NQ];
+    __shared__ QuadScratch<T> s_quad[NQ];
     __shared__ float4 s_grad[NQ][64][C / 4];   // upstream gradient of every wave's pixels (0 outside the image)
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -584,7 +713,7 @@ __global__ void __launch_bounds__(T* T)
     const int px = tile_x0 + (T == 16 ? 2 * (int)(lane & 7u) + (int)(wave & 1u) : (int)(lane & 7u));
     const int py = tile_y0 + (T == 16 ? 2 * (int)(lane >> 3) + (int)(wave >> 1) : (int)(lane >> 3));
     const bool inside = px < W && py < H;
-    QuadScratch<NF>& qs = s_quad[wave];
+    QuadScratch<T>& qs = s_quad[wave];
 
     float final_dot = 0.0f, common = 0.0f;
     {
@@ -627,43 +756,45 @@ __global__ void __launch_bounds__(T* T)
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        stage_instance<T, C, false>(st, valid, g.h, g.f, tile_x0, tile_y0);
+        float weight[4];
+        stage_instance<T, C, false>(st, valid, g.h, g.f, tile_x0, tile_y0, weight);
         BWD_MARK(0);
         __syncthreads();
         BWD_MARK(1);
 
         // ---- consume: this wave's list
         const ListIndex<NQ> li = list_index<T, C, false>(st, wave);
-        const uint32_t total = li.end[NQ - 1];
-        for (uint32_t sub = 0; sub < total; sub += 64u) {
-            const bool live = sub + lane < total;
-            const uint32_t j = live ? list_entry<T, C, false>(st, li, wave, sub + lane) : 0u;
-            LaneFragments<NF> lf;
-            load_lane_fragments<T, C, false>(st, wave, live, j, __ballot(done), lf);
-            float feat[C];
+        uint32_t my_start = 0, my_count = 0, n_fragments = 0;
+        if (li.end[NQ - 1] != 0u) {
+            Entries<T> e;
+            load_entries<T, C, false>(st, li, wave, __ballot(done), e);
+            float dots[K][NF];   // features . grad of the fragment's pixel
 #pragma unroll
-            for (int q4 = 0; q4 < C / 4; ++q4) {
-                const float4 v = st.feat[j * (C / 4) + q4];
-                feat[4 * q4] = v.x;
-                feat[4 * q4 + 1] = v.y;
-                feat[4 * q4 + 2] = v.z;
-                feat[4 * q4 + 3] = v.w;
-            }
-            uint32_t my_start, my_count, n_fragments;
-            build_fragment_lists<NF>(qs, st.opacity[j], lf, my_start, my_count, n_fragments, [&](int q) {
-                float d = 0.0f;  // features . grad of the fragment's pixel
+            for (int k = 0; k < K; ++k) {
+                float4 feat[C / 4];
 #pragma unroll
-                for (int q4 = 0; q4 < C / 4; ++q4) {
-                    const float4 gr = s_grad[wave][lf.pixel[q]][q4];
-                    d = fmaf(feat[4 * q4], gr.x, d);
-                    d = fmaf(feat[4 * q4 + 1], gr.y, d);
-                    d = fmaf(feat[4 * q4 + 2], gr.z, d);
-                    d = fmaf(feat[4 * q4 + 3], gr.w, d);
+                for (int q4 = 0; q4 < C / 4; ++q4) feat[q4] = st.feat[e.j[k] * (C / 4) + q4];
+#pragma unroll
+                for (int q = 0; q < NF; ++q) {
+                    const uint32_t pix = e.pixel[k][q] != kNoPixel ? e.pixel[k][q] : 0u;
+                    float d = 0.0f;
+#pragma unroll
+                    for (int q4 = 0; q4 < C / 4; ++q4) {
+                        const float4 gr = s_grad[wave][pix][q4];
+                        d = fmaf(feat[q4].x, gr.x, d);
+                        d = fmaf(feat[q4].y, gr.y, d);
+                        d = fmaf(feat[q4].z, gr.z, d);
+                        d = fmaf(feat[q4].w, gr.w, d);
+                    }
+                    arrive(d);   // computed here, not where it is used: the loaded values are not kept alive
+                    dots[k][q] = d;
                 }
-                return d;
-            });
-            BWD_MARK(2);
-            if (n_fragments == 0u) continue;
+            }
+            build_fragment_lists<T, C, false>(qs, st, wave, e, my_start, my_count, n_fragments,
+                                              [&](int k, int q) { return dots[k][q]; });
+        }
+        BWD_MARK(2);
+        if (n_fragments != 0u) {
             // ---- pixels with short lists: the sequential walk (kernels.cu:383-417)
             if (my_count <= kLongList) {
                 for (uint32_t i = 0; i < my_count; ++i) {
@@ -717,12 +848,7 @@ __global__ void __launch_bounds__(T* T)
                     done = Tr < kTransmittanceThreshold;
                 }
             }
-            wave_sync();
             BWD_MARK(4);
-            // ---- instances: hand {blending weight, d loss / d alpha} of the fragments to the instance's thread
-#pragma unroll
-            for (int q = 0; q < NF; ++q)
-                if (lf.pixel[q] != kNoPixel) st.result[wave][q][j] = qs.fragment[lf.where[q]];
         }
         {
             const uint64_t finished = __ballot(done);
@@ -734,26 +860,28 @@ __global__ void __launch_bounds__(T* T)
 #if defined(INPC_PROFILE_BACKWARD) && defined(INPC_BLEND_PROFILE)
         ++prof_batches;
 #endif
-        // ---- the gather moves on before the stores of the write phase (see the forward kernel)
-        const uint32_t point = g.h.point;
+        // ---- the gather moves on in front of the stores of the write phase (see the forward kernel)
+        const uint32_t point = g.h.point, tiles = g.h.tiles, split = g.h.split;
         const bool multi = g.h.multi();
         advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
-        // ---- write: thread t owns staged instance t: gradient of the point from its fragments in all quads
+        // ---- write: thread t owns staged instance t: gradient of the point from the fragments the waves placed
         if (valid) {
+            uint32_t field[4];
+            load_fields<T, C, false>(st, tid, field);
             float gf[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) gf[c] = 0.0f;
             float gop = 0.0f;
             bool any_weight = false;
 #pragma unroll
-            for (int q = 0; q < NQ; ++q)
-#pragma unroll
-                for (int k = 0; k < NF; ++k) {
-                    const float2 e = st.result[q][k][tid];
-                    gop = fmaf(e.y, st.weight[q][k][tid], gop);
+            for (int c = 0; c < 4; ++c)
+                if (field[c] & kPlaced) {
+                    const int q = T == 16 ? c : 0;
+                    const float2 e = s_quad[q].fragment[field[c] >> 8];   // {blending weight, d loss / d alpha}
+                    gop = fmaf(e.y, weight[c], gop);
                     if (e.x > 0.0f) {
                         any_weight = true;
-                        const uint32_t pix = st.pixel[q][k][tid];
+                        const uint32_t pix = field[c] & kPixelMask;
 #pragma unroll
                         for (int q4 = 0; q4 < C / 4; ++q4) {
                             const float4 gr = s_grad[q][pix][q4];
@@ -765,18 +893,21 @@ __global__ void __launch_bounds__(T* T)
                     }
                 }
             if (any_weight || gop != 0.0f) {
+                // a point that straddles tiles gets its gradient from up to four blocks: each writes a row of
+                // its own (summed up by k_grad_reduce); no atomics, and the sum has a fixed order
                 float* dst = grad_view + (size_t)point * C;
+                float* dst_opacity = grad_opacities + point;
                 if (multi) {
-#pragma unroll
-                    for (int c = 0; c < C; ++c)
-                        if (gf[c] != 0.0f) atomicAdd(dst + c, gf[c]);
-                    if (gop != 0.0f) atomicAdd(&grad_opacities[point], gop);
-                } else {
-#pragma unroll
-                    for (int q4 = 0; q4 < C / 4; ++q4)
-                        ((float4*)dst)[q4] = make_float4(gf[4 * q4], gf[4 * q4 + 1], gf[4 * q4 + 2], gf[4 * q4 + 3]);
-                    grad_opacities[point] = gop;
+                    const uint32_t part = tile_part(tile, tiles, gw);
+                    const size_t row = (size_t)split * 4u + part;
+                    dst = rows.features + row * C;
+                    dst_opacity = rows.opacities + row;
+                    ((uint8_t*)(rows.flags + split))[part] = 1;
                 }
+#pragma unroll
+                for (int q4 = 0; q4 < C / 4; ++q4)
+                    ((float4*)dst)[q4] = make_float4(gf[4 * q4], gf[4 * q4 + 1], gf[4 * q4 + 2], gf[4 * q4 + 3]);
+                *dst_opacity = gop;
             }
         }
         if (all_done) break;

@@ -49,6 +49,7 @@ enum Counter : int {
     kCntVisible = 0,
     kCntInstances = 1,
     kCntError = 2,
+    kCntSplit = 3,         // drawn points that touch more than one tile
     kCntTicketDepth = 4,   // 4 words
     kCntWords = 16
 };
@@ -61,7 +62,8 @@ __device__ __forceinline__ uint32_t info_ny(uint32_t info) { return ((info >> 17
 
 // Blend record of a drawn point: a 32-byte header followed by the view features, padded to a multiple
 // of 32 bytes (64 bytes for every configuration but 16 fp32 channels).
-//   header: float sx, sy, opacity; u32 point id; u32 tile info; float depth; 2 words unused
+//   header: float sx, sy, opacity; u32 point id; u32 tile info; float depth; u32 index among the points that
+//           touch several tiles (0 for the others); 1 word unused
 constexpr uint32_t kRecordHeader = 32;
 inline uint32_t record_stride(int channels, bool half_features) {
     return (uint32_t)align_up(kRecordHeader + (size_t)channels * (half_features ? 2 : 4), 32);
@@ -172,10 +174,13 @@ __host__ __device__ inline uint32_t bin_chunk_size(uint32_t n) {
 template <int T>
 __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restrict__ positions,
                                                            const float* __restrict__ w2c, uint32_t* __restrict__ table,
-                                                           Geometry g) {
+                                                           uint32_t* __restrict__ split_count, Geometry g) {
     extern __shared__ uint32_t s_count[];
+    __shared__ uint32_t s_split;   // drawn points of the chunk that touch more than one tile
     for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_count[t] = 0u;
+    if (threadIdx.x == 0) s_split = 0u;
     __syncthreads();
+    uint32_t my_split = 0;
     const ViewRows m = load_view_rows(w2c);
     const uint32_t chunk = bin_chunk_size(g.n);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
@@ -183,10 +188,14 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
         const Projected p = project_point<T>(m, g, positions[3 * (size_t)i], positions[3 * (size_t)i + 1],
                                              positions[3 * (size_t)i + 2]);
         if (p.info) atomicAdd(&s_count[info_tile0(p.info)], 1u);
+        if (p.touched > 1u) my_split += 1u;
     }
+    for (int sh = 32; sh > 0; sh >>= 1) my_split += __shfl_down(my_split, sh, 64);
+    if ((threadIdx.x & 63u) == 0u && my_split) atomicAdd(&s_split, my_split);
     __syncthreads();
     uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
     for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) row[t] = s_count[t];
+    if (threadIdx.x == 0) split_count[blockIdx.x] = s_split;
 }
 
 // table[c][t] <- sum of table[c'][t] over c' < c; total[t] <- sum over all chunks.
@@ -273,12 +282,15 @@ __global__ void __launch_bounds__(kBinThreads)
                  const float* __restrict__ cam_position, char* __restrict__ records,
                  const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start,
                  uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, float* __restrict__ blending_weights,
-                 uint32_t* counters, uint32_t* g_hist, Geometry g, radix::DevicePlan plan) {
+                 const uint32_t* __restrict__ split_count, uint32_t* __restrict__ split_points,
+                 uint32_t* __restrict__ split_flags, uint32_t* counters, uint32_t* g_hist, Geometry g,
+                 radix::DevicePlan plan) {
     extern __shared__ __align__(16) uint32_t s_dyn[];
     float4* s_stage = (float4*)s_dyn;                                           // record staging, 64 rows per wave
     uint32_t* s_cursor = s_dyn + PreprocessShape<FMODE, C>::kStageBytes / 4;     // n_tiles
     uint32_t* s_hist = s_cursor + g.n_tiles;                                    // kMaxPasses * kRadix
     __shared__ uint32_t s_visible, s_instances;
+    __shared__ uint32_t s_split;   // next index for a point of this chunk that touches more than one tile
     {
         const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
         for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_cursor[t] = bin_start[t] + row[t];
@@ -287,8 +299,21 @@ __global__ void __launch_bounds__(kBinThreads)
     if (threadIdx.x == 0) {
         s_visible = 0u;
         s_instances = 0u;
+        s_split = 0u;
     }
     __syncthreads();
+    {
+        // the points that touch several tiles are numbered chunk by chunk (inside a chunk in no particular
+        // order): the index only names the rows their gradient is collected in
+        uint32_t before = 0;
+        for (uint32_t b = threadIdx.x; b < blockIdx.x; b += kBinThreads) before += split_count[b];
+        for (int sh = 32; sh > 0; sh >>= 1) before += __shfl_down(before, sh, 64);
+        if ((threadIdx.x & 63u) == 0u && before) atomicAdd(&s_split, before);
+        __syncthreads();
+        const uint32_t first = s_split;
+        __syncthreads();
+        if (threadIdx.x == 0 && blockIdx.x == gridDim.x - 1u) counters[kCntSplit] = first + split_count[blockIdx.x];
+    }
     const ViewRows m = load_view_rows(w2c);
     uint32_t my_visible = 0, my_instances = 0;
     const uint32_t chunk = bin_chunk_size(g.n);
@@ -355,8 +380,14 @@ __global__ void __launch_bounds__(kBinThreads)
                             opacity = 1.0f - expf(-expf(__half2float(raw[0])));  // kernels.cu:142
                         }
                     }
+                    uint32_t split = 0u;
+                    if (p.touched > 1u) {
+                        split = atomicAdd(&s_split, 1u);
+                        split_points[split] = i;
+                        split_flags[split] = 0u;
+                    }
                     rec[0] = make_float4(p.sx, p.sy, opacity, __uint_as_float(i));
-                    rec[1] = make_float4(__uint_as_float(p.info), p.depth, 0.0f, 0.0f);
+                    rec[1] = make_float4(__uint_as_float(p.info), p.depth, __uint_as_float(split), 0.0f);
                 }
                 keys[i] = key;
                 vals[i] = val;
@@ -591,6 +622,7 @@ struct Layout {
     size_t bin_table, bin_total, tile_order, inst_start;
     size_t keys_a, keys_b, vals_a, vals_b;
     size_t inst_keys_a, inst_vals_a;
+    size_t split_count, split_points, split_features, split_opacities, split_flags;  // points that straddle tiles
 };
 
 uint32_t float_bits(float f) {
@@ -667,6 +699,16 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.vals_b = take(n * 4);
     L.inst_keys_a = take(ni * 2);
     L.inst_vals_a = take(ni * 4);
+    // gradient rows of the points that touch several tiles, four per point; sized for the worst case
+    // (every point), touched only as far as such points exist
+    L.split_count = take(kBinBlocks * 4);
+    L.split_points = take(n * 4);
+    L.split_flags = take(n * 4);
+    L.split_features = L.split_opacities = 0;
+    if (!L.inference && L.fmode != INPC_FEAT_RAW37_F16) {   // configurations with a backward pass
+        L.split_features = take(4 * n * L.C * 4);
+        L.split_opacities = take(4 * n * 4);
+    }
     const bool depth_in_a = (L.depth_plan.n_passes % 2) == 0;
     P.depth_keys = depth_in_a ? L.keys_a : L.keys_b;
     P.depth_order = depth_in_a ? L.vals_a : L.vals_b;
@@ -708,7 +750,7 @@ template <int T>
 int launch_bin_count(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
     const size_t lds = (size_t)L.geo.n_tiles * 4;
     INPC_LAUNCH_LDS("raster_bin_count", (k_bin_count<T>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream, positions,
-                    w2c, at<uint32_t>(ws, L.bin_table), L.geo);
+                    w2c, at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.split_count), L.geo);
     return INPC_OK;
 }
 
@@ -723,7 +765,8 @@ int launch_preprocess(const Layout& L, const float* positions, const void* featu
                     positions, features, opacities, w2c, cam_position, at<char>(ws, L.pub.point_record),
                     (const uint32_t*)at<uint32_t>(ws, L.bin_table), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
                     at<uint32_t>(ws, L.keys_a), at<uint32_t>(ws, L.vals_a), blending_weights,
-                    at<uint32_t>(ws, L.pub.counters), at<uint32_t>(ws, L.hist_depth), L.geo,
+                    (const uint32_t*)at<uint32_t>(ws, L.split_count), at<uint32_t>(ws, L.split_points),
+                    at<uint32_t>(ws, L.split_flags), at<uint32_t>(ws, L.pub.counters), at<uint32_t>(ws, L.hist_depth), L.geo,
                     radix::to_device_plan(L.depth_plan));
     return INPC_OK;
 }
@@ -750,11 +793,16 @@ int launch_blend_forward(const Layout& L, float* image, float* alpha, float* ble
 template <int T, int C, bool HALF>
 int launch_blend_backward(const Layout& L, const float* grad_image, const float* grad_alpha, const float* image,
                           const float* alpha, float* grad_view, float* grad_opacities, void* ws, hipStream_t stream) {
+    const blend::SplitRows rows{at<float>(ws, L.split_features), at<float>(ws, L.split_opacities),
+                                at<uint32_t>(ws, L.split_flags), (const uint32_t*)at<uint32_t>(ws, L.split_points),
+                                (const uint32_t*)at<uint32_t>(ws, L.pub.counters) + kCntSplit};
     INPC_LAUNCH("raster_blend_backward", (blend::k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 at<uint32_t>(ws, L.pub.instance_slots), at<char>(ws, L.pub.point_record), L.geo.stride, grad_image,
                 grad_alpha, image, alpha, grad_view,
-                grad_opacities, L.geo.W, L.geo.H, L.geo.gw);
+                grad_opacities, rows, L.geo.W, L.geo.H, L.geo.gw);
+    INPC_LAUNCH("raster_grad_reduce", blend::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, 256u), 4096u)), dim3(256),
+                stream, rows, grad_view, grad_opacities);
     return INPC_OK;
 }
 
