@@ -324,15 +324,16 @@ __global__ void __launch_bounds__(kBinThreads)
     // instead of one word of 64 different records.
     constexpr bool kDirect = FMODE == INPC_FEAT_DIRECT_F32 || FMODE == INPC_FEAT_DIRECT_F16;
     constexpr int kUnroll = kDirect ? 4 : 2;
-    using Word = std::conditional_t<FMODE == INPC_FEAT_DIRECT_F16, uint2, float4>;  // four channels
+    using Word = std::conditional_t<FMODE == INPC_FEAT_DIRECT_F16, uint2, uint4>;  // four channels
     constexpr int kWords = kDirect ? C / 4 : 1;
+    constexpr int kPer = sizeof(Word) / 4;   // 32-bit registers per word
     constexpr uint32_t kStrideWords = PreprocessShape<FMODE, C>::kStrideWords, kRow = kStrideWords + 1;  // padded row
     constexpr uint32_t kNoSlot = 0xFFFFFFFFu;
     const uint32_t lane = threadIdx.x & 63u;
     float4* stage = s_stage + (threadIdx.x >> 6) * (64u * kRow);
     for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
         float px[kUnroll], py[kUnroll], pz[kUnroll], op[kUnroll];
-        Word fw[kUnroll][kWords];
+        uint32_t fw[kUnroll][kWords * kPer];   // plain registers (an array of vector types ends up in scratch memory)
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             // a thread behind the end reads the chunk's first point and drops it
@@ -345,7 +346,15 @@ __global__ void __launch_bounds__(kBinThreads)
             if (kDirect) {
                 const Word* src = (const Word*)features + i * kWords;
 #pragma unroll
-                for (int q = 0; q < kWords; ++q) fw[u][q] = src[q];
+                for (int q = 0; q < kWords; ++q) {
+                    const Word v = src[q];
+                    fw[u][q * kPer] = v.x;
+                    fw[u][q * kPer + 1] = v.y;
+                    if constexpr (kPer == 4) {
+                        fw[u][q * kPer + 2] = v.z;
+                        fw[u][q * kPer + 3] = v.w;
+                    }
+                }
             }
         }
 #pragma unroll
@@ -369,7 +378,16 @@ __global__ void __launch_bounds__(kBinThreads)
                     if (kDirect) {
                         Word* dst = (Word*)(rec + 2);
 #pragma unroll
-                        for (int q = 0; q < kWords; ++q) dst[q] = fw[u][q];
+                        for (int q = 0; q < kWords; ++q) {
+                            Word v;
+                            v.x = fw[u][q * kPer];
+                            v.y = fw[u][q * kPer + 1];
+                            if constexpr (kPer == 4) {
+                                v.z = fw[u][q * kPer + 2];
+                                v.w = fw[u][q * kPer + 3];
+                            }
+                            dst[q] = v;
+                        }
                     } else {
                         const ShBasis sb = sh_basis(px[u], py[u], pz[u], cam_position);
                         if (FMODE == INPC_FEAT_SH36_F16) {
