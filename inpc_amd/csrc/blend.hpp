@@ -654,33 +654,40 @@ __device__ __forceinline__ uint32_t tile_part(uint32_t tile, uint32_t info, uint
     return delta >= gw ? 2u + (delta - gw) : delta;
 }
 
-// gradient of the point = sum of its rows, in row order (the gradient buffers are zero before)
+// gradient of the point = sum of its rows, in row order (the gradient buffers are zero before). All four rows are
+// read whether written or not (stale rows are dropped by their flag): the reads are dense and independent.
 template <int C>
 __global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __restrict__ grad_view,
                                                      float* __restrict__ grad_opacities) {
     const uint32_t n = *rows.count;
     for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < n; s += gridDim.x * 256u) {
         const uint32_t flags = rows.flags[s];
+        const uint32_t i = rows.points[s];
+        const float4* row = (const float4*)(rows.features + (size_t)s * 4u * C);
+        float4 part[4][C / 4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+            for (int q4 = 0; q4 < C / 4; ++q4) part[p][q4] = row[p * (C / 4) + q4];
+        const float4 op = ((const float4*)rows.opacities)[s];
         if (flags == 0u) continue;
         rows.flags[s] = 0u;
-        const uint32_t i = rows.points[s];
+        const float part_opacity[4] = {op.x, op.y, op.z, op.w};
         float4 acc[C / 4];
 #pragma unroll
         for (int q4 = 0; q4 < C / 4; ++q4) acc[q4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         float opacity = 0.0f;
 #pragma unroll
-        for (uint32_t part = 0; part < 4u; ++part)
-            if ((flags >> (8u * part)) & 0xFFu) {
-                const float4* row = (const float4*)(rows.features + ((size_t)s * 4u + part) * C);
+        for (int p = 0; p < 4; ++p)
+            if ((flags >> (8 * p)) & 0xFFu) {
 #pragma unroll
                 for (int q4 = 0; q4 < C / 4; ++q4) {
-                    const float4 r = row[q4];
-                    acc[q4].x += r.x;
-                    acc[q4].y += r.y;
-                    acc[q4].z += r.z;
-                    acc[q4].w += r.w;
+                    acc[q4].x += part[p][q4].x;
+                    acc[q4].y += part[p][q4].y;
+                    acc[q4].z += part[p][q4].z;
+                    acc[q4].w += part[p][q4].w;
                 }
-                opacity += rows.opacities[(size_t)s * 4u + part];
+                opacity += part_opacity[p];
             }
 #pragma unroll
         for (int q4 = 0; q4 < C / 4; ++q4) ((float4*)(grad_view + (size_t)i * C))[q4] = acc[q4];

@@ -54,12 +54,30 @@ __global__ void __launch_bounds__(kBinThreads)
     const uint32_t n_visible = min(counters[kCntVisible], n_points);
     const uint32_t chunk = chunk_size(n_points);
     const uint32_t begin = min(blockIdx.x * chunk, n_visible), end = min(begin + chunk, n_visible);
-    for (uint32_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
-        const uint32_t val = depth_order[i];
-        const uint32_t tile0 = first_tile(val, bin_start, coarse);
-        const uint32_t nx = (val & 1u) + 1u, ny = ((val >> 1) & 1u) + 1u;
-        for (uint32_t dy = 0; dy < ny; ++dy)
-            for (uint32_t dx = 0; dx < nx; ++dx) atomicAdd(&s_count[tile0 + dy * gw + dx], 1u);
+    constexpr int kUnroll = 4;   // points per thread and round: the dependent loads of the tile search overlap
+    for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
+        uint32_t val[kUnroll], lo[kUnroll], hi[kUnroll];
+        bool live[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t i = base + u * kBinThreads + threadIdx.x;
+            live[u] = i < end;
+            val[u] = depth_order[live[u] ? i : begin];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t b = (val[u] >> 2) >> kCoarseShift;
+            lo[u] = coarse[b];
+            hi[u] = (uint32_t)coarse[b + 1] + 1u;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (!live[u]) continue;
+            const uint32_t tile0 = tile_of_slot(bin_start, lo[u], hi[u], val[u] >> 2);
+            const uint32_t nx = (val[u] & 1u) + 1u, ny = ((val[u] >> 1) & 1u) + 1u;
+            for (uint32_t dy = 0; dy < ny; ++dy)
+                for (uint32_t dx = 0; dx < nx; ++dx) atomicAdd(&s_count[tile0 + dy * gw + dx], 1u);
+        }
     }
     __syncthreads();
     uint32_t* row = table + (size_t)blockIdx.x * n_tiles;

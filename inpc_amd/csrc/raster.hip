@@ -184,11 +184,24 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
     const ViewRows m = load_view_rows(w2c);
     const uint32_t chunk = bin_chunk_size(g.n);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
-    for (uint32_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
-        const Projected p = project_point<T>(m, g, positions[3 * (size_t)i], positions[3 * (size_t)i + 1],
-                                             positions[3 * (size_t)i + 2]);
-        if (p.info) atomicAdd(&s_count[info_tile0(p.info)], 1u);
-        if (p.touched > 1u) my_split += 1u;
+    constexpr int kUnroll = 4;   // points per thread and round, their loads issued together
+    for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
+        float px[kUnroll], py[kUnroll], pz[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t at = base + u * kBinThreads + threadIdx.x;
+            const size_t i = at < end ? at : begin;
+            px[u] = positions[3 * i];
+            py[u] = positions[3 * i + 1];
+            pz[u] = positions[3 * i + 2];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            if (base + u * kBinThreads + threadIdx.x >= end) continue;
+            const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
+            if (p.info) atomicAdd(&s_count[info_tile0(p.info)], 1u);
+            if (p.touched > 1u) my_split += 1u;
+        }
     }
     for (int sh = 32; sh > 0; sh >>= 1) my_split += __shfl_down(my_split, sh, 64);
     if ((threadIdx.x & 63u) == 0u && my_split) atomicAdd(&s_split, my_split);
