@@ -57,6 +57,9 @@ inline int bit_length(uint32_t n) {
 // the stream into a graph).
 int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream);
 
+// Number of blocks of `threads` threads of `kernel` (static LDS only) that the current device holds at once.
+int resident_blocks(const void* kernel, int threads, uint32_t& blocks);
+
 // ------------------------------------------------------------------------------------------------
 // device side
 // ------------------------------------------------------------------------------------------------
@@ -134,9 +137,11 @@ __host__ __device__ __forceinline__ uint64_t pcg_apply(const PcgJump& j, uint64_
 }
 
 // ---- decoupled look-back --------------------------------------------------------------------------
-// A status word is {2 flag bits, 30 value bits}. Blocks take their index from an atomic ticket, so
-// a block only ever waits on blocks that are already running; the wait is bounded and raises the
-// error flag instead of spinning forever.
+// A status word is {2 flag bits, 30 value bits}. A block must only ever wait on blocks that are running. The
+// large kernels get that by running as one resident grid whose blocks take the tiles in order (block index,
+// + grid size, ...); the small ones by taking their tile index from an atomic ticket (thousands of blocks
+// taking tickets from one address at the start of a kernel cost more than the look-back itself). The wait is
+// bounded and raises the error flag instead of spinning forever.
 constexpr uint32_t kFlagAggregate = 1u << 30;
 constexpr uint32_t kFlagInclusive = 2u << 30;
 constexpr uint32_t kValueMask = (1u << 30) - 1u;

@@ -7,7 +7,7 @@
 //   - a block ranks its 4096 keys stably (per-wave ballot matching, 64-wide), stages them through
 //     LDS so that every digit leaves the block as one contiguous run, and finds its global offsets
 //     with a decoupled look-back over per-(block, digit) status words.
-// Blocks take their tile index from an atomic ticket, so look-back only waits on running blocks.
+// The grid is resident as a whole and walks over the tiles in order, so look-back only waits on running blocks.
 #pragma once
 
 #include "common.hpp"
@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(kBlock)
     k_scatter(const KeyT* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, KeyT* __restrict__ keys_out,
               uint32_t* __restrict__ vals_out, const uint32_t* __restrict__ n_dev, uint32_t n_host, int shift,
               uint32_t digit_mask, int bits, const uint32_t* __restrict__ digit_base, uint32_t* status,
-              uint32_t* ticket, uint32_t* error_flag) {
+              uint32_t* error_flag) {
     __shared__ uint32_t s_cnt[kWaves][kRadix];
     __shared__ uint32_t s_hist[kRadix];
     __shared__ uint32_t s_local_base[kRadix];
@@ -142,20 +142,21 @@ __global__ void __launch_bounds__(kBlock)
     __shared__ KeyT s_keys[kTile];
     __shared__ uint32_t s_vals[kTile];
     __shared__ uint32_t s_wave[kWaves];
-    __shared__ uint32_t s_bid;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     INPC_SORT_PROF_DECL;
-    if (tid == 0) s_bid = atomicAdd(ticket, 1u);
+    uint32_t n = n_host;
+    if (!FIRST) n = min(n_host, *n_dev);
+    // Tiles in order, bid = blockIdx.x, + gridDim.x, ...: a tile waits (look-back) only for tiles in front of it,
+    // and those belong to blocks that are running or to an earlier round of this grid, which the host sizes
+    // so that all of it is resident at once: no block has to end for another one to start.
+    for (uint32_t bid = blockIdx.x;; bid += gridDim.x) {
+    const uint64_t tile_base = (uint64_t)bid * kTile;
+    if (tile_base >= n) break;
     for (int i = tid; i < kWaves * kRadix; i += kBlock) (&s_cnt[0][0])[i] = 0u;
     s_hist[tid] = 0u;
     __syncthreads();
     INPC_SORT_PROF_MARK(0);
-    const uint32_t bid = s_bid;
-    uint32_t n = n_host;
-    if (!FIRST) n = min(n_host, *n_dev);
-    const uint64_t tile_base = (uint64_t)bid * kTile;
-    if (tile_base >= n) return;
 
     KeyT key[kItems];
     uint32_t val[kItems];
@@ -261,6 +262,8 @@ __global__ void __launch_bounds__(kBlock)
         }
     }
     INPC_SORT_PROF_MARK(6);
+    __syncthreads();   // the LDS arrays are reused by the next tile
+    }
     INPC_SORT_PROF_FLUSH;
 }
 
@@ -270,14 +273,19 @@ inline size_t status_words(uint32_t n_max) { return (size_t)div_up(n_max, kTile)
 // Enqueue every pass of a sort. Buffers ping-pong: pass 0 reads keys_a / vals_a, the result ends in the
 // a-buffers when the pass count is even, else in the b-buffers.
 // hist: n_passes*256 filled histograms; bases: same size scratch; status: n_passes*status_words(n_max)
-// zeroed words; tickets: n_passes zeroed words.
+// zeroed words.
 template <typename KeyT>
 int sort_pairs(const PassPlan& plan, FirstPass first, KeyT* keys_a, uint32_t* vals_a, KeyT* keys_b,
                uint32_t* vals_b, const uint32_t* n_dev, uint32_t n_max, const uint32_t* hist, uint32_t* bases,
-               uint32_t* status, uint32_t* tickets, uint32_t* error_flag, hipStream_t stream, const char* name) {
+               uint32_t* status, uint32_t* error_flag, hipStream_t stream, const char* name) {
     if (n_max == 0) return INPC_OK;
     INPC_LAUNCH("radix_digit_bases", k_digit_bases, dim3(plan.n_passes), dim3(kRadix), stream, hist, bases);
-    const uint32_t blocks = div_up(n_max, kTile);
+    uint32_t resident_first = 0, resident_rest = 0;
+    int rc = resident_blocks((const void*)k_scatter<KeyT, true>, kBlock, resident_first);
+    if (rc != INPC_OK) return rc;
+    rc = resident_blocks((const void*)k_scatter<KeyT, false>, kBlock, resident_rest);
+    if (rc != INPC_OK) return rc;
+    const uint32_t tiles = div_up(n_max, kTile);
     const size_t words = status_words(n_max);
     KeyT* kin = keys_a;
     uint32_t* vin = vals_a;
@@ -286,13 +294,13 @@ int sort_pairs(const PassPlan& plan, FirstPass first, KeyT* keys_a, uint32_t* va
     for (int p = 0; p < plan.n_passes; ++p) {
         const uint32_t mask = (1u << plan.bits[p]) - 1u;
         if (p == 0 && first == kSkipInvalid) {
-            INPC_LAUNCH(name, (k_scatter<KeyT, true>), dim3(blocks), dim3(kBlock), stream, (const KeyT*)kin,
+            INPC_LAUNCH(name, (k_scatter<KeyT, true>), dim3(std::min(tiles, resident_first)), dim3(kBlock), stream, (const KeyT*)kin,
                         (const uint32_t*)vin, kout, vout, n_dev, n_max, plan.shift[p], mask, plan.bits[p],
-                        (const uint32_t*)(bases + p * kRadix), status + p * words, tickets + p, error_flag);
+                        (const uint32_t*)(bases + p * kRadix), status + p * words, error_flag);
         } else {
-            INPC_LAUNCH(name, (k_scatter<KeyT, false>), dim3(blocks), dim3(kBlock), stream, (const KeyT*)kin,
+            INPC_LAUNCH(name, (k_scatter<KeyT, false>), dim3(std::min(tiles, resident_rest)), dim3(kBlock), stream, (const KeyT*)kin,
                         (const uint32_t*)vin, kout, vout, n_dev, n_max, plan.shift[p], mask, plan.bits[p],
-                        (const uint32_t*)(bases + p * kRadix), status + p * words, tickets + p, error_flag);
+                        (const uint32_t*)(bases + p * kRadix), status + p * words, error_flag);
         }
         std::swap(kin, kout);
         std::swap(vin, vout);

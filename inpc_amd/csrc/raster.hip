@@ -50,7 +50,6 @@ enum Counter : int {
     kCntInstances = 1,
     kCntError = 2,
     kCntSplit = 3,         // drawn points that touch more than one tile
-    kCntTicketDepth = 4,   // 4 words
     kCntWords = 16
 };
 
@@ -955,7 +954,7 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                                          at<uint32_t>(ws, L.vals_a), at<uint32_t>(ws, L.keys_b),
                                          at<uint32_t>(ws, L.vals_b), counters + kCntVisible, L.geo.n,
                                          at<uint32_t>(ws, L.hist_depth), at<uint32_t>(ws, L.bases_depth),
-                                         at<uint32_t>(ws, L.status_depth), counters + kCntTicketDepth,
+                                         at<uint32_t>(ws, L.status_depth),
                                          counters + kCntError, stream, "raster_depth_sort");
         if (rc != INPC_OK) return rc;
         {

@@ -73,6 +73,16 @@ int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream) {
     return INPC_OK;
 }
 
+int resident_blocks(const void* kernel, int threads, uint32_t& blocks) {
+    int device = 0, per_cu = 0, cus = 0;
+    INPC_HIP_CHECK(hipGetDevice(&device));
+    INPC_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    INPC_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0));
+    if (per_cu < 1 || cus < 1) return fail(INPC_E_HIP, "occupancy query returned %d blocks on %d compute units", per_cu, cus);
+    blocks = (uint32_t)per_cu * (uint32_t)cus;
+    return INPC_OK;
+}
+
 // Plain streaming copy, 16 bytes per lane: the yardstick for profiler byte counters.
 __global__ void __launch_bounds__(256) k_copy_u128(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;

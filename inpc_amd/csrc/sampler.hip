@@ -162,30 +162,40 @@ __device__ __forceinline__ uint32_t cdf_search(const float* __restrict__ cdf, fl
 
 // The same search with the top of its decision tree in LDS. Which element the k-th probe reads depends only on
 // the outcomes of the probes before it, so the first kTreeDepth probes can only touch 2^kTreeDepth - 1 fixed
-// elements; a block keeps those in LDS in heap order (node 1 = first probe, node 2n / 2n + 1 = the probe after
-// going left / right) and reads the CDF itself only below that depth. The comparisons are exactly those of
-// cdf_search, so the result is the same even where rounding leaves the CDF not perfectly monotone; for 262,144
-// leaves 11 of the 18 dependent cache round trips of a sample become LDS reads.
-constexpr int kTreeDepth = 11;
-constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNodes - 1
+// elements. inpc_build_cdf leaves those, in heap order (node 1 = first probe, node 2n / 2n + 1 = the probe after
+// going left / right), behind the total in the CDF head; a block copies them into LDS and reads the CDF itself
+// only below that depth. The comparisons are exactly those of cdf_search, so the result is the same even
+// where rounding leaves the CDF not perfectly monotone; for 262,144 leaves 13 of the 18 dependent cache round
+// trips of a sample become LDS reads and the other five fall into one 128-byte line.
+constexpr int kTreeDepth = 13;
+constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNodes - 1; index 0 of the head: the total
+static_assert(kTreeNodes == INPC_CDF_HEAD_FLOATS, "the CDF head holds the total and the search tree");
 
-// Every thread of the block must call it; ends with a barrier.
-__device__ __forceinline__ void load_search_tree(float* s_tree, const float* __restrict__ cdf, uint32_t n) {
-    for (uint32_t node = threadIdx.x + 1u; node < kTreeNodes; node += blockDim.x) {
-        // replay the decisions that lead to this node
-        const int depth = 31 - __clz(node);
-        uint32_t first = 0, count = n;
-        for (int l = depth - 1; l >= 0 && count > 0; --l) {
-            const uint32_t step = count >> 1;
-            if ((node >> l) & 1u) {
-                first += step + 1;
-                count -= step + 1;
-            } else {
-                count = step;
-            }
+// head[node] for every node of the tree (one thread per node).
+__global__ void __launch_bounds__(kBlock) k_build_search_tree(const float* __restrict__ cdf, float* __restrict__ head,
+                                                              uint32_t n) {
+    const uint32_t node = blockIdx.x * kBlock + threadIdx.x;
+    if (node == 0u || node >= kTreeNodes) return;
+    // replay the decisions that lead to this node
+    const int depth = 31 - __clz(node);
+    uint32_t first = 0, count = n;
+    for (int l = depth - 1; l >= 0 && count > 0; --l) {
+        const uint32_t step = count >> 1;
+        if ((node >> l) & 1u) {
+            first += step + 1;
+            count -= step + 1;
+        } else {
+            count = step;
         }
-        s_tree[node] = count > 0 ? cdf[first + (count >> 1)] : 0.0f;
     }
+    head[node] = count > 0 ? cdf[first + (count >> 1)] : 0.0f;
+}
+
+// Every thread of the block must call it; ends with a barrier. s_tree[0] (the total) is not used.
+__device__ __forceinline__ void load_search_tree(float* s_tree, const float* __restrict__ head) {
+    const float4* src = (const float4*)head;
+    float4* dst = (float4*)s_tree;
+    for (uint32_t i = threadIdx.x; i < kTreeNodes / 4; i += blockDim.x) dst[i] = src[i];
     __syncthreads();
 }
 
@@ -243,9 +253,9 @@ __global__ void __launch_bounds__(kBlock) k_sample(const float* __restrict__ cen
                                                    float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
                                                    uint32_t n_samples, uint32_t n_leaves, float initial_size,
                                                    const uint64_t* __restrict__ rng_dev) {
-    __shared__ float s_tree[kTreeNodes];
+    __shared__ __align__(16) float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
-    load_search_tree(s_tree, cdf, n_leaves);
+    load_search_tree(s_tree, sum_dev);
     const uint64_t tile_first = (uint64_t)blockIdx.x * kSampleTile;
     Pcg32 r = thread_generator(rng_dev, tile_first);
     const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);  // from draw 4k+4 to 4(k+256)
@@ -274,7 +284,7 @@ struct CullState {
     uint32_t accepted;   // samples accepted so far in this draw (a lower bound once `consumed` is set)
     uint32_t consumed;   // candidates consumed when the capacity-th sample was accepted, else 0
     uint32_t error;      // look-back gave up
-    uint32_t ticket;     // block ordering of the current round
+    uint32_t unused;
     uint32_t pad[12];
 };
 constexpr size_t kCullHeaderWords = sizeof(CullState) / 4;
@@ -285,87 +295,94 @@ __global__ void __launch_bounds__(kBlock)
                   float* __restrict__ positions, int32_t* __restrict__ leaf_ids, uint32_t capacity, uint32_t k0,
                   uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam, float initial_size,
                   const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
-    __shared__ uint32_t s_bid, s_accepted0, s_exclusive, s_done;
+    __shared__ uint32_t s_accepted0, s_exclusive, s_done;
     __shared__ uint32_t s_count[kSampleItems * (kBlock / kWave)];
-    __shared__ float s_tree[kTreeNodes];
+    __shared__ __align__(16) float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    if (tid == 0) {
-        const uint32_t bid = atomicAdd(&st->ticket, 1u);
-        s_bid = bid;
-        s_accepted0 = __hip_atomic_load(&st->accepted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t done = __hip_atomic_load(&st->consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-        s_done = done;
-        if (done) {
-            // The draw is already complete: tell later blocks that everything is taken.
-            status_store(status + bid, kFlagInclusive | min(capacity, kValueMask));
-            if (bid == n_blocks - 1) st->accepted = max(s_accepted0, capacity);
-        }
-    }
-    __syncthreads();
-    if (s_done) return;
-    load_search_tree(s_tree, cdf, n_leaves);
-    const uint32_t bid = s_bid;
-    const uint64_t tile_first = (uint64_t)bid * kSampleTile;  // relative to k0
+    // `accepted` keeps its value from the rounds before until the last tile of this round has its total, and
+    // that needs the count of every tile in front of it
+    if (tid == 0) s_accepted0 = __hip_atomic_load(&st->accepted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    load_search_tree(s_tree, sum_dev);
     const Rows m = load_rows(w2c);
-    Pcg32 r = thread_generator(rng_dev, (uint64_t)k0 + tile_first);
-    const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);
+    // Tiles in order: a tile waits (look-back) only for tiles in front of it, and those belong to blocks that are
+    // running or to an earlier round of this grid, which stays resident as a whole (the host sizes it so):
+    // no block has to end for another one to start.
+    for (uint32_t bid = blockIdx.x; bid < n_blocks; bid += gridDim.x) {
+        if (tid == 0) {
+            const uint32_t done = __hip_atomic_load(&st->consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+            s_done = done;
+            if (done) {
+                // The draw is already complete: tell later tiles that everything is taken.
+                status_store(status + bid, kFlagInclusive | min(capacity, kValueMask));
+                if (bid == n_blocks - 1) st->accepted = max(s_accepted0, capacity);
+            }
+        }
+        __syncthreads();
+        if (s_done) {   // uniform
+            __syncthreads();   // s_done is rewritten by the next tile
+            continue;
+        }
+        const uint64_t tile_first = (uint64_t)bid * kSampleTile;  // relative to k0
+        Pcg32 r = thread_generator(rng_dev, (uint64_t)k0 + tile_first);
+        const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);
 
-    Candidate cand[kSampleItems];
-    uint32_t rank[kSampleItems];
-    bool keep[kSampleItems];
+        Candidate cand[kSampleItems];
+        uint32_t rank[kSampleItems];
+        bool keep[kSampleItems];
 #pragma unroll
-    for (int j = 0; j < kSampleItems; ++j) {
-        const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
-        keep[j] = false;
-        if (rel < n_candidates) {
-            cand[j] = draw_candidate(r, centers, levels, cdf, s_tree, n_leaves, initial_size);
-            keep[j] = sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
-            r.state = pcg_apply(step, r.state);
-        }
-        const uint64_t ballot = __ballot(keep[j]);
-        rank[j] = mask_rank(ballot);
-        if (lane == 0) s_count[j * (kBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
-    }
-    __syncthreads();
-    if (wave == 0) {
-        // exclusive scan of the 32 (round, wave) counts by the first lanes, then the block-level look-back
-        uint32_t c = lane < (uint32_t)(kSampleItems * (kBlock / kWave)) ? s_count[lane] : 0u;
-        uint32_t incl = c;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t up = __shfl_up(incl, d, 64);
-            if (lane >= (uint32_t)d) incl += up;
-        }
-        if (lane < (uint32_t)(kSampleItems * (kBlock / kWave))) s_count[lane] = incl - c;
-        const uint32_t run = __shfl(incl, 63, 64);
-        const uint32_t exclusive = lookback_exclusive_wave(status, bid, run, &st->error);
-        if (lane == 0) {
-            s_exclusive = exclusive;
-            if (bid == n_blocks - 1) st->accepted = s_accepted0 + exclusive + run;
-        }
-    }
-    __syncthreads();
-    const uint64_t base = (uint64_t)s_accepted0 + s_exclusive;
-#pragma unroll
-    for (int j = 0; j < kSampleItems; ++j) {
-        if (!keep[j]) continue;
-        const uint64_t slot = base + s_count[j * (kBlock / kWave) + wave] + rank[j];
-        if (slot >= capacity) continue;
-        positions[3 * slot] = cand[j].x;
-        positions[3 * slot + 1] = cand[j].y;
-        positions[3 * slot + 2] = cand[j].z;
-        leaf_ids[slot] = (int32_t)cand[j].leaf;
-        if (slot + 1 == capacity) {
+        for (int j = 0; j < kSampleItems; ++j) {
             const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
-            __hip_atomic_store(&st->consumed, (uint32_t)(k0 + rel + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            keep[j] = false;
+            if (rel < n_candidates) {
+                cand[j] = draw_candidate(r, centers, levels, cdf, s_tree, n_leaves, initial_size);
+                keep[j] = sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
+                r.state = pcg_apply(step, r.state);
+            }
+            const uint64_t ballot = __ballot(keep[j]);
+            rank[j] = mask_rank(ballot);
+            if (lane == 0) s_count[j * (kBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
         }
+        __syncthreads();
+        if (wave == 0) {
+            // exclusive scan of the 32 (round, wave) counts by the first lanes, then the block-level look-back
+            uint32_t c = lane < (uint32_t)(kSampleItems * (kBlock / kWave)) ? s_count[lane] : 0u;
+            uint32_t incl = c;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t up = __shfl_up(incl, d, 64);
+                if (lane >= (uint32_t)d) incl += up;
+            }
+            if (lane < (uint32_t)(kSampleItems * (kBlock / kWave))) s_count[lane] = incl - c;
+            const uint32_t run = __shfl(incl, 63, 64);
+            const uint32_t exclusive = lookback_exclusive_wave(status, bid, run, &st->error);
+            if (lane == 0) {
+                s_exclusive = exclusive;
+                if (bid == n_blocks - 1) st->accepted = s_accepted0 + exclusive + run;
+            }
+        }
+        __syncthreads();
+        const uint64_t base = (uint64_t)s_accepted0 + s_exclusive;
+#pragma unroll
+        for (int j = 0; j < kSampleItems; ++j) {
+            if (!keep[j]) continue;
+            const uint64_t slot = base + s_count[j * (kBlock / kWave) + wave] + rank[j];
+            if (slot >= capacity) continue;
+            positions[3 * slot] = cand[j].x;
+            positions[3 * slot + 1] = cand[j].y;
+            positions[3 * slot + 2] = cand[j].z;
+            leaf_ids[slot] = (int32_t)cand[j].leaf;
+            if (slot + 1 == capacity) {
+                const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
+                __hip_atomic_store(&st->consumed, (uint32_t)(k0 + rel + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __syncthreads();   // s_count, s_exclusive and s_done are reused by the next tile
     }
 }
 
-__global__ void k_cull_round_reset(CullState* st, uint32_t* status, uint32_t n_blocks) {
+__global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i == 0) st->ticket = 0u;
     if (i < n_blocks) status[i] = 0u;
 }
 
@@ -604,6 +621,8 @@ int inpc_build_cdf(float* w, float* sum_out, void* workspace, size_t workspace_b
         INPC_LAUNCH("chunk_add_prefix", k_chunk_add_prefix, dim3(div_up(dn, kBlock)), dim3(kBlock), stream, dst, dn,
                     (const float*)(totals + plan.offset[d]), (const float*)sum_out);
     }
+    INPC_LAUNCH("search_tree", k_build_search_tree, dim3(kTreeNodes / kBlock), dim3(kBlock), stream, (const float*)w,
+                sum_out, n_leaves);
     return INPC_OK;
 }
 
@@ -649,9 +668,13 @@ int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const 
     CullState* st = (CullState*)workspace;
     uint32_t* status = (uint32_t*)workspace + kCullHeaderWords;
     const uint32_t n_blocks = div_up(n_candidates, kSampleTile);
-    INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(n_blocks, kBlock)), dim3(kBlock), stream, st,
-                status, n_blocks);
-    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(n_blocks), dim3(kBlock), stream, centers, levels, cdf,
+    INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(n_blocks, kBlock)), dim3(kBlock), stream, status,
+                n_blocks);
+    // the whole grid must be resident at once: its blocks wait for each other's tiles
+    uint32_t resident = 0;
+    const int rc = resident_blocks((const void*)k_sample_cull, kBlock, resident);
+    if (rc != INPC_OK) return rc;
+    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(std::min(n_blocks, resident)), dim3(kBlock), stream, centers, levels, cdf,
                 sum_dev, w2c, positions_out, leaf_ids_out, capacity, k0, n_candidates, n_blocks, n_leaves,
                 to_device_camera(*cam), initial_size, rng_dev, st, status);
     return INPC_OK;

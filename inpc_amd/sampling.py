@@ -101,7 +101,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
                    "inpc_leaf_weights")
         ws_bytes = int(lib.inpc_sampler_workspace_bytes(max(n, 1)))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=centers.device)
-        total = torch.zeros(1, dtype=torch.float32, device=centers.device)
+        total = torch.zeros(_lib.CDF_HEAD_FLOATS, dtype=torch.float32, device=centers.device)  # CDF head; [0] = total
         return vw, ws, ws_bytes, total, cam, stream
 
     def _cdf(self, centers, levels, weights, w2c, view, initial_size):
@@ -164,7 +164,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
         self.last_consumed = int(consumed.value) if consumed.value else k0
         _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0,
                                         _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream), "inpc_cull_finish")
-        if consumed.value == 0 and accepted.value < n_samples and float(total.item()) > 0.0:
+        if consumed.value == 0 and accepted.value < n_samples and float(total[0].item()) > 0.0:
             _log.warning("sampler accepted only %d of %d samples; the rest is uninitialised", accepted.value,
                          n_samples)
         _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
@@ -180,7 +180,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
         if n_leaves == 0:
             return torch.empty((0, 3), dtype=torch.float32, device=device)
         cdf, total, cam, stream = self._cdf(centers, levels, weights, w2c, view, initial_size)
-        if not float(total.item()) > 0.0:  # the reference reads the sum back here as well
+        if not float(total[0].item()) > 0.0:  # the reference reads the sum back here as well
             return torch.empty((0, 3), dtype=torch.float32, device=device)
         n_samples = int(n_samples)
         positions = torch.empty((n_samples, 3), dtype=torch.float32, device=device)

@@ -49,7 +49,7 @@ def test_cdf_of_exact_integers_matches_cumsum(gpu):
     w[-1] += (1 << 18) - w.sum()
     assert 0 <= w[-1] < (1 << 18)
     cdf, tot = H.build_cdf(H.dev(w.astype(np.float32)))
-    assert float(tot.item()) == float(1 << 18)
+    assert float(tot[0].item()) == float(1 << 18)
     expect = (np.cumsum(w).astype(np.float64) / (1 << 18)).astype(np.float32)
     np.testing.assert_array_equal(cdf.cpu().numpy(), expect)
 
@@ -57,7 +57,7 @@ def test_cdf_of_exact_integers_matches_cumsum(gpu):
 def test_sum_not_positive_leaves_weights_untouched(gpu):
     w = np.zeros(5000, dtype=np.float32)
     cdf, total = H.build_cdf(H.dev(w))
-    assert float(total.item()) == 0.0
+    assert float(total[0].item()) == 0.0
     np.testing.assert_array_equal(cdf.cpu().numpy(), w)
 
 
