@@ -1,5 +1,6 @@
 // runtime.hip — error reporting, per-launch timing hooks, fill kernel, PCG32 host helpers.
 #include <algorithm>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -74,12 +75,32 @@ int fill_u32(void* dst, uint32_t value, size_t n_words, hipStream_t stream) {
 }
 
 int resident_blocks(const void* kernel, int threads, uint32_t& blocks) {
-    int device = 0, per_cu = 0, cus = 0;
+    // asked on every launch of a resident grid: remembered per (device, kernel, block size)
+    struct Entry {
+        int device;
+        const void* kernel;
+        int threads;
+        uint32_t blocks;
+    };
+    static std::mutex lock;
+    static std::vector<Entry> known;
+    int device = 0;
     INPC_HIP_CHECK(hipGetDevice(&device));
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        for (const Entry& e : known)
+            if (e.device == device && e.kernel == kernel && e.threads == threads) {
+                blocks = e.blocks;
+                return INPC_OK;
+            }
+    }
+    int per_cu = 0, cus = 0;
     INPC_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
     INPC_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0));
     if (per_cu < 1 || cus < 1) return fail(INPC_E_HIP, "occupancy query returned %d blocks on %d compute units", per_cu, cus);
     blocks = (uint32_t)per_cu * (uint32_t)cus;
+    std::lock_guard<std::mutex> guard(lock);
+    known.push_back(Entry{device, kernel, threads, blocks});
     return INPC_OK;
 }
 

@@ -274,3 +274,29 @@ def test_autograd_api_sh_and_direct(gpu, oracle):
                                          alpha8.detach().cpu().numpy(), pos, f8, o8, hv.w2c)
     H.assert_close(f8d.grad.cpu().numpy(), gf8, RTOL, 1e-6, "direct feature gradients")
     H.assert_close(o8d.grad.cpu().numpy(), go8, RTOL, 1e-5, "direct opacity gradients")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_backward_twice_after_one_forward(gpu, oracle, tile):
+    # The gradient rows of points that straddle tiles carry flags from one backward call to the next: a second
+    # call with gradients that vanish on half of the image (so that fewer rows are written) must not see the
+    # first call's rows. Dense and opaque, so that tiles also end early.
+    n, channels = 120000, 8
+    hv = synthetic.camera_on_z(131, 93, 120.0, 2.4)
+    pos = synthetic.cube_points(n, 1.3, 41)
+    feats, _ = synthetic.point_attributes(n, channels, "normal", 42)
+    opac = np.random.default_rng(43).uniform(0.05, 0.9, n).astype(np.float32)
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32)
+    out = run.outputs()
+    rng = np.random.default_rng(44)
+    for half in (False, True):
+        gi = rng.normal(0, 1e-2, out["image"].shape).astype(np.float32)
+        ga = rng.normal(0, 1e-2, out["alpha"].shape).astype(np.float32)
+        if half:
+            gi[:, :, : gi.shape[2] // 2] = 0.0
+            ga[:, :, : ga.shape[2] // 2] = 0.0
+        gf, go = run.backward(gi, ga)
+        gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
+        H.assert_close(gf, gf_ref, RTOL, 1e-7, f"feature gradients (half={half})")
+        H.assert_close(go, go_ref, RTOL, 2e-7, f"opacity gradients (half={half})")
