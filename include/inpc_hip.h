@@ -314,6 +314,40 @@ int inpc_opacity_forward(const float* raw, float* opacity, size_t n, void* strea
 int inpc_opacity_backward(const float* grad_opacity, const float* raw, float* grad_raw, size_t n,
                           void* stream);
 
+/* Ordered selections over the leaves of the probability field. A leaf is selected when
+ * values[i] > threshold and (levels == NULL or levels[i] < max_level).
+ * inpc_field_select_workspace_bytes: scratch for n_leaves leaves.
+ * inpc_field_select_count: count_out (1 u32 dev) = number of selected leaves; replaces the mask sums
+ * `valid_mask.sum()` (Modules/ProbabilityField.py:222) and the shape of `self.leaf_weights[mask]`
+ * (:161): the caller reads it to size the outputs of the two calls below. */
+size_t inpc_field_select_workspace_bytes(uint32_t n_leaves);
+int inpc_field_select_count(const float* values, const int32_t* levels, uint32_t n_leaves,
+                            float threshold, int max_level, uint32_t* count_out, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
+/* Keeps the leaves with weights[i] > threshold, in order. Replaces ProbabilityField.prune
+ * (Modules/ProbabilityField.py:159-165). Outputs hold at least the selected count (n_leaves
+ * always suffices); count_out (1 u32 dev) receives it. centers (n,3) f32, levels (n,) i32. */
+int inpc_field_prune(const float* centers, const int32_t* levels, const float* weights,
+                     const float* scores, uint32_t n_leaves, float threshold, float* centers_out,
+                     int32_t* levels_out, float* weights_out, float* scores_out,
+                     uint32_t* count_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Splits the leaves with scores[i] > threshold and levels[i] < max_level into eight children
+ * each. Replaces the array part of ProbabilityField.subdivide
+ * (Modules/ProbabilityField.py:217-257): outputs = the other leaves in order, then the children,
+ * parents in order, child j
+ * at centre -/+ initial_size / 2^(level + 2) per axis (+ in x for odd j, in y for j % 4 >= 2, in
+ * z for j >= 4), level + 1, the parent's weight, score 0. count_out (1 u32 dev) receives the
+ * number s of split leaves; outputs must hold n_leaves + 7 s leaves (s from
+ * inpc_field_select_count with the same arguments). The reference's size limit (:223-224) is
+ * the caller's decision between the two calls. initial_size: 3 floats on the host. */
+int inpc_field_subdivide(const float* centers, const int32_t* levels, const float* weights,
+                         const float* scores, uint32_t n_leaves, float threshold, int max_level,
+                         const float initial_size[3], float* centers_out, int32_t* levels_out,
+                         float* weights_out, float* scores_out, uint32_t* count_out,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* grads (= or +=, `add` != 0) factor(i) * weights[i], factor = 0.1 * 2 / (entries of the hash-grid
  * level that holds flat index i), 0 in front of index 6144. Replaces
  * compute_normalized_weight_decay_grads_cu<add> (B/misc/src/misc_kernels.cu:6-47) behind

@@ -105,6 +105,11 @@ SIGNATURES = {
     "inpc_spherical_contraction": (C.c_int, [_P, _P, _U32, _P]),
     "inpc_opacity_forward": (C.c_int, [_P, _P, _SZ, _P]),
     "inpc_opacity_backward": (C.c_int, [_P, _P, _P, _SZ, _P]),
+    "inpc_field_select_workspace_bytes": (C.c_size_t, [_U32]),
+    "inpc_field_select_count": (C.c_int, [_P, _P, _U32, C.c_float, C.c_int, _P, _P, C.c_size_t, _P]),
+    "inpc_field_prune": (C.c_int, [_P, _P, _P, _P, _U32, C.c_float, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "inpc_field_subdivide": (C.c_int, [_P, _P, _P, _P, _U32, C.c_float, C.c_int, C.POINTER(C.c_float), _P, _P, _P, _P,
+                                       _P, _P, C.c_size_t, _P]),
     "inpc_weight_decay_grads": (C.c_int, [_P, _P, _U32, C.c_int, _P]),
     "inpc_cauchy_loss": (C.c_int, [_P, _P, _P, _U32, _P]),
     "inpc_cauchy_loss_backward": (C.c_int, [_P, _P, _P, _P, _U32, _P]),

@@ -69,6 +69,182 @@ __global__ void __launch_bounds__(kBlock) k_field_finish(const uint32_t* __restr
     }
 }
 
+
+// ---- prune / subdivide (Modules/ProbabilityField.py:159-165, 217-257) -----------------------------------------------
+// Both are ordered selections over the leaves: prune keeps the leaves whose weight exceeds a threshold, in
+// order; subdivide keeps the leaves that are not split, in order, and appends eight children per split leaf,
+// parents in order, children in the order x, y, z of the sign of their offset. A leaf is selected when
+// value > threshold and (levels == nullptr or level < max_level).
+//   k_select_count   per block of kSelectTile leaves: number of selected leaves
+//   k_select_scan    one block: exclusive scan of the block counts, total to counts[0]
+//   k_prune_apply / k_subdivide_apply   recompute the flags, rank inside the block by ballots, write
+constexpr int kSelectItems = 4;
+constexpr int kSelectTile = kBlock * kSelectItems;
+
+__device__ __forceinline__ bool leaf_selected(const float* __restrict__ values, const int32_t* __restrict__ levels,
+                                              uint32_t i, float threshold, int max_level) {
+    return values[i] > threshold && (levels == nullptr || levels[i] < max_level);
+}
+
+// Exclusive rank of this thread's flag among the flags of the block in thread order; `total` = their number.
+__device__ __forceinline__ uint32_t block_rank(bool flag, uint32_t* s_wave /* kBlock / kWave */, uint32_t& total) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint64_t ballot = __ballot(flag);
+    if (lane == 0) s_wave[wave] = (uint32_t)__popcll(ballot);
+    __syncthreads();
+    uint32_t before = 0;
+    total = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w) {
+        const uint32_t c = s_wave[w];
+        if ((uint32_t)w < wave) before += c;
+        total += c;
+    }
+    __syncthreads();
+    return before + mask_rank(ballot);
+}
+
+__global__ void __launch_bounds__(kBlock) k_select_count(const float* __restrict__ values, const int32_t* __restrict__ levels,
+                                                         uint32_t n, float threshold, int max_level,
+                                                         uint32_t* __restrict__ block_counts) {
+    __shared__ uint32_t s_count;
+    if (threadIdx.x == 0) s_count = 0u;
+    __syncthreads();
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kSelectItems; ++j) {
+        const uint32_t i = blockIdx.x * kSelectTile + j * kBlock + threadIdx.x;
+        if (i < n && leaf_selected(values, levels, i, threshold, max_level)) ++mine;
+    }
+    for (int sh = 32; sh > 0; sh >>= 1) mine += __shfl_down(mine, sh, 64);
+    if ((threadIdx.x & 63u) == 0u && mine) atomicAdd(&s_count, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) block_counts[blockIdx.x] = s_count;
+}
+
+__global__ void __launch_bounds__(kBlock) k_select_scan(uint32_t* block_counts, uint32_t n_blocks, uint32_t* counts) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    __shared__ uint32_t s_carry;
+    if (threadIdx.x == 0) s_carry = 0u;
+    __syncthreads();
+    for (uint32_t base = 0; base < n_blocks; base += kBlock) {
+        const uint32_t i = base + threadIdx.x, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+        const uint32_t v = i < n_blocks ? block_counts[i] : 0u;
+        uint32_t incl = v;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (lane >= (uint32_t)d) incl += up;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        uint32_t before = s_carry, all = 0;
+#pragma unroll
+        for (int w = 0; w < kBlock / kWave; ++w) {
+            const uint32_t c = s_wave[w];
+            if ((uint32_t)w < wave) before += c;
+            all += c;
+        }
+        if (i < n_blocks) block_counts[i] = before + incl - v;
+        __syncthreads();
+        if (threadIdx.x == 0) s_carry += all;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) counts[0] = s_carry;
+}
+
+struct LeafArrays {
+    const float* centers;
+    const int32_t* levels;
+    const float* weights;
+    const float* scores;
+};
+
+struct LeafOutputs {
+    float* centers;
+    int32_t* levels;
+    float* weights;
+    float* scores;
+};
+
+__global__ void __launch_bounds__(kBlock) k_prune_apply(LeafArrays in, LeafOutputs out, uint32_t n, float threshold,
+                                                        const uint32_t* __restrict__ block_offsets) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    uint32_t base = block_offsets[blockIdx.x];
+#pragma unroll
+    for (int j = 0; j < kSelectItems; ++j) {
+        const uint32_t i = blockIdx.x * kSelectTile + j * kBlock + threadIdx.x;
+        const bool keep = i < n && leaf_selected(in.weights, nullptr, i, threshold, 0);
+        uint32_t total;
+        const uint32_t slot = base + block_rank(keep, s_wave, total);
+        base += total;
+        if (keep) {
+            out.centers[3 * (size_t)slot] = in.centers[3 * (size_t)i];
+            out.centers[3 * (size_t)slot + 1] = in.centers[3 * (size_t)i + 1];
+            out.centers[3 * (size_t)slot + 2] = in.centers[3 * (size_t)i + 2];
+            out.levels[slot] = in.levels[i];
+            out.weights[slot] = in.weights[i];
+            out.scores[slot] = in.scores[i];
+        }
+    }
+}
+
+// Split leaf number r (in order) becomes the children n_kept + 8 r .. + 7; child j sits at
+// centre -/+ initial_size / 2^(level + 2) per axis, + in x for odd j, in y for j % 4 >= 2, in z for j >= 4
+// (ProbabilityField.py:233-250); its level is level + 1, its weight the parent's, its score 0.
+__global__ void __launch_bounds__(kBlock) k_subdivide_apply(LeafArrays in, LeafOutputs out, uint32_t n, float threshold,
+                                                            int max_level, float size_x, float size_y, float size_z,
+                                                            const uint32_t* __restrict__ block_offsets,
+                                                            const uint32_t* __restrict__ counts) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    const uint32_t n_split = counts[0], n_kept = n - n_split;
+    uint32_t split_base = block_offsets[blockIdx.x];
+#pragma unroll
+    for (int j = 0; j < kSelectItems; ++j) {
+        const uint32_t i = blockIdx.x * kSelectTile + j * kBlock + threadIdx.x;
+        const bool live = i < n;
+        const bool split = live && leaf_selected(in.scores, in.levels, i, threshold, max_level);
+        uint32_t total;
+        const uint32_t rank = block_rank(split, s_wave, total);
+        if (live) {
+            const float cx = in.centers[3 * (size_t)i], cy = in.centers[3 * (size_t)i + 1], cz = in.centers[3 * (size_t)i + 2];
+            const int32_t level = in.levels[i];
+            const float weight = in.weights[i];
+            if (!split) {
+                const uint32_t slot = i - (split_base + rank);   // kept leaves in front of this one
+                out.centers[3 * (size_t)slot] = cx;
+                out.centers[3 * (size_t)slot + 1] = cy;
+                out.centers[3 * (size_t)slot + 2] = cz;
+                out.levels[slot] = level;
+                out.weights[slot] = weight;
+                out.scores[slot] = in.scores[i];
+            } else {
+                const size_t first = (size_t)n_kept + 8u * (size_t)(split_base + rank);
+                const float ox = ldexpf(size_x, -(level + 2)), oy = ldexpf(size_y, -(level + 2)), oz = ldexpf(size_z, -(level + 2));
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    out.centers[3 * (first + c)] = (c & 1) ? cx + ox : cx - ox;
+                    out.centers[3 * (first + c) + 1] = (c & 2) ? cy + oy : cy - oy;
+                    out.centers[3 * (first + c) + 2] = (c & 4) ? cz + oz : cz - oz;
+                    out.levels[first + c] = level + 1;
+                    out.weights[first + c] = weight;
+                    out.scores[first + c] = 0.0f;
+                }
+            }
+        }
+        split_base += total;
+    }
+}
+
+int select_offsets(const float* values, const int32_t* levels, uint32_t n, float threshold, int max_level,
+                   uint32_t* block_offsets, uint32_t* counts, hipStream_t stream) {
+    const uint32_t blocks = div_up(n, kSelectTile);
+    INPC_LAUNCH("field_select_count", k_select_count, dim3(blocks), dim3(kBlock), stream, values, levels, n, threshold,
+                max_level, block_offsets);
+    INPC_LAUNCH("field_select_scan", k_select_scan, dim3(1), dim3(kBlock), stream, block_offsets, blocks, counts);
+    return INPC_OK;
+}
+
 }  // namespace
 }  // namespace inpc
 
@@ -110,6 +286,65 @@ int inpc_field_update_check(const void* workspace, void* stream_) {
     INPC_HIP_CHECK(hipMemcpyAsync(&flag, workspace, 4, hipMemcpyDeviceToHost, stream));
     INPC_HIP_CHECK(hipStreamSynchronize(stream));
     if (flag) return fail(INPC_E_INVALID_ARGUMENT, "field_update: a sample index lies outside [0, n_leaves)");
+    return INPC_OK;
+}
+
+
+size_t inpc_field_select_workspace_bytes(uint32_t n_leaves) {
+    return (size_t)inpc::div_up(std::max(n_leaves, 1u), (uint32_t)inpc::kSelectTile) * 4 + 256;
+}
+
+int inpc_field_select_count(const float* values, const int32_t* levels, uint32_t n_leaves, float threshold, int max_level,
+                            uint32_t* count_out, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace inpc;
+    if (!count_out) return fail(INPC_E_INVALID_ARGUMENT, "field_select_count: null count");
+    if (n_leaves == 0) return fill_u32(count_out, 0u, 1, (hipStream_t)stream);
+    if (!values) return fail(INPC_E_INVALID_ARGUMENT, "field_select_count: null values");
+    if (!workspace || workspace_bytes < inpc_field_select_workspace_bytes(n_leaves))
+        return fail(INPC_E_WORKSPACE, "field_select_count: workspace too small");
+    return select_offsets(values, levels, n_leaves, threshold, max_level, (uint32_t*)workspace, count_out, (hipStream_t)stream);
+}
+
+int inpc_field_prune(const float* centers, const int32_t* levels, const float* weights, const float* scores,
+                     uint32_t n_leaves, float threshold, float* centers_out, int32_t* levels_out, float* weights_out,
+                     float* scores_out, uint32_t* count_out, void* workspace, size_t workspace_bytes, void* stream_) {
+    using namespace inpc;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!count_out) return fail(INPC_E_INVALID_ARGUMENT, "field_prune: null count");
+    if (n_leaves == 0) return fill_u32(count_out, 0u, 1, stream);
+    if (!centers || !levels || !weights || !scores || !centers_out || !levels_out || !weights_out || !scores_out)
+        return fail(INPC_E_INVALID_ARGUMENT, "field_prune: null pointer");
+    if (!workspace || workspace_bytes < inpc_field_select_workspace_bytes(n_leaves))
+        return fail(INPC_E_WORKSPACE, "field_prune: workspace too small");
+    uint32_t* offsets = (uint32_t*)workspace;
+    const int rc = select_offsets(weights, nullptr, n_leaves, threshold, 0, offsets, count_out, stream);
+    if (rc != INPC_OK) return rc;
+    INPC_LAUNCH("field_prune", k_prune_apply, dim3(div_up(n_leaves, kSelectTile)), dim3(kBlock), stream,
+                (LeafArrays{centers, levels, weights, scores}), (LeafOutputs{centers_out, levels_out, weights_out, scores_out}),
+                n_leaves, threshold, (const uint32_t*)offsets);
+    return INPC_OK;
+}
+
+int inpc_field_subdivide(const float* centers, const int32_t* levels, const float* weights, const float* scores,
+                         uint32_t n_leaves, float threshold, int max_level, const float initial_size[3],
+                         float* centers_out, int32_t* levels_out, float* weights_out, float* scores_out,
+                         uint32_t* count_out, void* workspace, size_t workspace_bytes, void* stream_) {
+    using namespace inpc;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!count_out) return fail(INPC_E_INVALID_ARGUMENT, "field_subdivide: null count");
+    if (n_leaves == 0) return fill_u32(count_out, 0u, 1, stream);
+    if (!centers || !levels || !weights || !scores || !centers_out || !levels_out || !weights_out || !scores_out ||
+        !initial_size)
+        return fail(INPC_E_INVALID_ARGUMENT, "field_subdivide: null pointer");
+    if (!workspace || workspace_bytes < inpc_field_select_workspace_bytes(n_leaves))
+        return fail(INPC_E_WORKSPACE, "field_subdivide: workspace too small");
+    uint32_t* offsets = (uint32_t*)workspace;
+    const int rc = select_offsets(scores, levels, n_leaves, threshold, max_level, offsets, count_out, stream);
+    if (rc != INPC_OK) return rc;
+    INPC_LAUNCH("field_subdivide", k_subdivide_apply, dim3(div_up(n_leaves, kSelectTile)), dim3(kBlock), stream,
+                (LeafArrays{centers, levels, weights, scores}), (LeafOutputs{centers_out, levels_out, weights_out, scores_out}),
+                n_leaves, threshold, max_level, initial_size[0], initial_size[1], initial_size[2], (const uint32_t*)offsets,
+                (const uint32_t*)count_out);
     return INPC_OK;
 }
 

@@ -1,8 +1,11 @@
-"""Probability-field statistics update: the per-iteration step that feeds the sampler's leaf indices and the
-rasterizer's blending weights back into the octree (Modules/ProbabilityField.py:146-157 of the reference).
+"""Probability-field bookkeeping: the per-iteration statistics update that feeds the sampler's leaf indices and
+the rasterizer's blending weights back into the octree, and the two restructuring steps that follow from it
+(Modules/ProbabilityField.py:146-165, 217-257 of the reference).
 
 `update_probability_field(leaf_weights, leaf_subdivision_scores, indices, weights)` does in place what
-`ProbabilityField.update(indices, weights)` does to its two leaf tensors.
+`ProbabilityField.update(indices, weights)` does to its two leaf tensors; `prune_probability_field` and
+`subdivide_probability_field` return the four leaf tensors that `prune(threshold)` / `subdivide(threshold)` assign
+to the module's buffers.
 """
 from __future__ import annotations
 
@@ -44,3 +47,75 @@ def update_probability_field(leaf_weights: torch.Tensor, leaf_subdivision_scores
                                      stream), "inpc_field_update")
     if check:
         _lib.check(lib.inpc_field_update_check(_lib.ptr(ws), stream), "inpc_field_update")
+
+
+def _leaf_tensors(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores):
+    n = leaf_weights.numel()
+    if leaf_centers.dtype != torch.float32 or leaf_weights.dtype != torch.float32 or \
+            leaf_subdivision_scores.dtype != torch.float32:
+        raise RuntimeError("expected scalar type Float")
+    if leaf_levels.dtype != torch.int32:
+        raise RuntimeError("expected scalar type Int")
+    if leaf_centers.shape != (n, 3) or leaf_levels.shape != (n,) or leaf_subdivision_scores.shape != (n,) or \
+            leaf_weights.dim() != 1:
+        raise RuntimeError("leaf tensors of one octree expected: centers (n, 3), levels, weights, scores (n,)")
+    tensors = [t.contiguous() for t in (leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores)]
+    if not all(t.is_cuda for t in tensors):
+        raise RuntimeError("expected tensors on the GPU")
+    return tensors, n
+
+
+def _select_workspace(n, device):
+    ws_bytes = int(_lib.lib().inpc_field_select_workspace_bytes(n))
+    return torch.empty(ws_bytes, dtype=torch.uint8, device=device), ws_bytes
+
+
+@torch.no_grad()
+def prune_probability_field(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores, threshold: float):
+    """The leaves with weight > threshold, in order: (centers, levels, weights, scores), as
+    ProbabilityField.prune assigns them (Modules/ProbabilityField.py:159-165). Reads the count back, like the
+    reference's boolean indexing."""
+    (centers, levels, weights, scores), n = _leaf_tensors(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores)
+    device = weights.device
+    out = (torch.empty((n, 3), dtype=torch.float32, device=device), torch.empty(n, dtype=torch.int32, device=device),
+           torch.empty(n, dtype=torch.float32, device=device), torch.empty(n, dtype=torch.float32, device=device))
+    count = torch.zeros(1, dtype=torch.int32, device=device)
+    ws, ws_bytes = _select_workspace(n, device)
+    _lib.check(_lib.lib().inpc_field_prune(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(scores), n,
+                                           float(threshold), *(_lib.ptr(t) for t in out), _lib.ptr(count), _lib.ptr(ws),
+                                           ws_bytes, _lib.current_stream()), "inpc_field_prune")
+    kept = int(count.item())
+    return tuple(t[:kept].contiguous() for t in out)
+
+
+@torch.no_grad()
+def subdivide_probability_field(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores, initial_cell_size,
+                                threshold: float, max_level: int = 6, max_leaves: int = 16_777_216):
+    """The leaf tensors after splitting every leaf with score > threshold and level < max_level into eight, as
+    ProbabilityField.subdivide assigns them (Modules/ProbabilityField.py:217-257): (centers, levels, weights,
+    scores), or None when the octree would exceed max_leaves (the reference returns without a change, :223-224)."""
+    (centers, levels, weights, scores), n = _leaf_tensors(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores)
+    device = weights.device
+    lib = _lib.lib()
+    size = torch.as_tensor(initial_cell_size, dtype=torch.float32).flatten().cpu()
+    if size.numel() == 1:
+        size = size.repeat(3)
+    if size.numel() != 3:
+        raise RuntimeError("initial_cell_size: one value or one per axis expected")
+    import ctypes as C
+    size_host = (C.c_float * 3)(*[float(v) for v in size])
+    count = torch.zeros(1, dtype=torch.int32, device=device)
+    ws, ws_bytes = _select_workspace(n, device)
+    stream = _lib.current_stream()
+    _lib.check(lib.inpc_field_select_count(_lib.ptr(scores), _lib.ptr(levels), n, float(threshold), int(max_level),
+                                           _lib.ptr(count), _lib.ptr(ws), ws_bytes, stream), "inpc_field_select_count")
+    n_split = int(count.item())
+    if n_split * 8 + (n - n_split) > max_leaves:
+        return None
+    total = n + 7 * n_split
+    out = (torch.empty((total, 3), dtype=torch.float32, device=device), torch.empty(total, dtype=torch.int32, device=device),
+           torch.empty(total, dtype=torch.float32, device=device), torch.empty(total, dtype=torch.float32, device=device))
+    _lib.check(lib.inpc_field_subdivide(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(scores), n,
+                                        float(threshold), int(max_level), size_host, *(_lib.ptr(t) for t in out),
+                                        _lib.ptr(count), _lib.ptr(ws), ws_bytes, stream), "inpc_field_subdivide")
+    return out

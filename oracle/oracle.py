@@ -405,6 +405,46 @@ def field_update(leaf_weights, leaf_scores, indices, weights, decay=0.9968):
 # ----------------------------------------------------------------------------------------------
 # element-wise steps between sampler and rasterizer, plain numpy in float32
 # ----------------------------------------------------------------------------------------------
+def field_prune(centers, levels, weights, scores, threshold):
+    """Modules/ProbabilityField.py:159-165: the leaves with weight > threshold, in order."""
+    w = np.asarray(weights, np.float32)
+    keep = w > np.float32(threshold)
+    return (np.asarray(centers, np.float32)[keep], np.asarray(levels, np.int32)[keep], w[keep],
+            np.asarray(scores, np.float32)[keep])
+
+
+def field_subdivide(centers, levels, weights, scores, initial_size, threshold, max_level=6, max_leaves=16_777_216):
+    """Modules/ProbabilityField.py:217-257, leaf by leaf: the leaves that stay, in order, then eight children per
+    split leaf. None when the octree would exceed max_leaves."""
+    centers, levels = np.asarray(centers, np.float32), np.asarray(levels, np.int32)
+    weights, scores = np.asarray(weights, np.float32), np.asarray(scores, np.float32)
+    size = np.broadcast_to(np.asarray(initial_size, np.float32).reshape(-1), (3,))
+    split = (scores > np.float32(threshold)) & (levels < max_level)
+    n_split, n = int(split.sum()), len(levels)
+    if n_split * 8 + (n - n_split) > max_leaves:
+        return None
+    out_c = [centers[~split]]
+    out_l = [levels[~split]]
+    out_w = [weights[~split]]
+    out_s = [scores[~split]]
+    kids_c = np.empty((n_split, 8, 3), np.float32)
+    kids_l = np.empty((n_split, 8), np.int32)
+    kids_w = np.empty((n_split, 8), np.float32)
+    for r, i in enumerate(np.flatnonzero(split)):
+        level = int(levels[i]) + 1
+        offset = (size / np.float32(2.0 ** (level + 1))).astype(np.float32)
+        for c in range(8):
+            sign = np.array([1 if c & 1 else -1, 1 if c & 2 else -1, 1 if c & 4 else -1], np.float32)
+            kids_c[r, c] = centers[i] + sign * offset
+        kids_l[r] = level
+        kids_w[r] = weights[i]
+    out_c.append(kids_c.reshape(-1, 3))
+    out_l.append(kids_l.reshape(-1))
+    out_w.append(kids_w.reshape(-1))
+    out_s.append(np.zeros(n_split * 8, np.float32))
+    return np.concatenate(out_c), np.concatenate(out_l), np.concatenate(out_w), np.concatenate(out_s)
+
+
 def spherical_contraction(positions):
     """B/misc/src/misc_kernels.cu:49-66, every operation rounded to float32 in the written order."""
     p = np.asarray(positions, np.float32).reshape(-1, 3)

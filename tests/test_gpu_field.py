@@ -65,3 +65,48 @@ def test_closes_the_loop_with_sampler_and_rasterizer(gpu, oracle):
     np.testing.assert_array_equal(d_lw.cpu().numpy(), a)
     np.testing.assert_array_equal(d_ls.cpu().numpy(), b)
     assert (a > np.float32(0.01) * np.float32(0.9968)).sum() > 100   # sampled leaves took their maxima
+
+
+def _octree(rng, n):
+    centers = rng.uniform(-2, 2, (n, 3)).astype(np.float32)
+    levels = rng.integers(0, 8, n).astype(np.int32)
+    return centers, levels, rng.random(n).astype(np.float32), rng.random(n).astype(np.float32)
+
+
+@pytest.mark.parametrize("n", [1, 1023, 1024, 70001])
+def test_prune_bit_exact(gpu, oracle, n):
+    from inpc_amd import prune_probability_field
+
+    rng = np.random.default_rng(n)
+    arrays = _octree(rng, n)
+    got = prune_probability_field(*(H.dev(a) for a in arrays), 0.4)
+    want = oracle.field_prune(*arrays, 0.4)
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(g.cpu().numpy(), w)
+
+
+def test_prune_everything_and_nothing(gpu, oracle):
+    from inpc_amd import prune_probability_field
+
+    arrays = _octree(np.random.default_rng(5), 3000)
+    assert all(t.shape[0] == 0 for t in prune_probability_field(*(H.dev(a) for a in arrays), 2.0))
+    kept = prune_probability_field(*(H.dev(a) for a in arrays), -1.0)
+    for g, a in zip(kept, arrays):
+        np.testing.assert_array_equal(g.cpu().numpy(), a)
+
+
+@pytest.mark.parametrize("n", [1, 1024, 33333])
+def test_subdivide_bit_exact(gpu, oracle, n):
+    from inpc_amd import subdivide_probability_field
+
+    rng = np.random.default_rng(100 + n)
+    arrays = _octree(rng, n)
+    size = np.array([0.37, 0.37, 0.37], np.float32)
+    got = subdivide_probability_field(*(H.dev(a) for a in arrays), torch.from_numpy(size), 0.55)
+    want = oracle.field_subdivide(*arrays, size, 0.55)
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(g.cpu().numpy(), w)
+    # the size limit: nothing is returned, as the reference leaves the octree alone
+    n_split = (len(want[1]) - n) // 7
+    if n_split:
+        assert subdivide_probability_field(*(H.dev(a) for a in arrays), size, 0.55, max_leaves=len(want[1]) - 1) is None

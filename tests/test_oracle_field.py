@@ -55,3 +55,57 @@ def test_order_of_the_samples_does_not_matter(oracle):
     a2, b2 = oracle.field_update(lw, ls, idx[p], w[p])
     np.testing.assert_array_equal(a, a2)
     np.testing.assert_array_equal(b, b2)
+
+
+def _random_octree(rng, n):
+    centers = rng.uniform(-2, 2, (n, 3)).astype(np.float32)
+    levels = rng.integers(0, 8, n).astype(np.int32)
+    weights = rng.random(n).astype(np.float32)
+    scores = rng.random(n).astype(np.float32)
+    return centers, levels, weights, scores
+
+
+def test_prune_matches_the_references_torch_statements(oracle):
+    # Modules/ProbabilityField.py:159-165 run by torch on the CPU
+    rng = np.random.default_rng(21)
+    centers, levels, weights, scores = _random_octree(rng, 5000)
+    weights[::7] = 0.25  # values on the threshold are dropped (strict comparison)
+    mask = torch.from_numpy(weights) > 0.25
+    want = [torch.from_numpy(a)[mask].contiguous().numpy() for a in (centers, levels, weights, scores)]
+    got = oracle.field_prune(centers, levels, weights, scores, 0.25)
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(g, w)
+    assert len(got[0]) < 5000 and (got[2] > 0.25).all()
+
+
+def test_subdivide_matches_the_references_torch_statements(oracle):
+    # Modules/ProbabilityField.py:217-257 run by torch on the CPU, statement by statement
+    rng = np.random.default_rng(22)
+    centers, levels, weights, scores = _random_octree(rng, 3000)
+    initial = torch.tensor([0.37, 0.37, 0.37], dtype=torch.float32)
+    threshold = 0.6
+    c, l, w, s = (torch.from_numpy(a) for a in (centers, levels, weights, scores))
+    valid_mask = (s > threshold) & (l < 6)
+    valid_centers, valid_levels, valid_weights = c[valid_mask], l[valid_mask], w[valid_mask]
+    new_centers = torch.repeat_interleave(valid_centers, 8, dim=0)
+    new_levels = torch.repeat_interleave(valid_levels + 1, 8, dim=0)
+    new_weights = torch.repeat_interleave(valid_weights, 8, dim=0)
+    new_scores = torch.zeros_like(new_weights)
+    offset = initial / (2 ** (new_levels + 1))[:, None]
+    new_centers[0::2, 0] -= offset[0::2, 0]
+    new_centers[1::2, 0] += offset[1::2, 0]
+    new_centers[0::4, 1] -= offset[0::4, 1]
+    new_centers[1::4, 1] -= offset[1::4, 1]
+    new_centers[2::4, 1] += offset[2::4, 1]
+    new_centers[3::4, 1] += offset[3::4, 1]
+    for k in range(4):
+        new_centers[k::8, 2] -= offset[k::8, 2]
+        new_centers[4 + k::8, 2] += offset[4 + k::8, 2]
+    want = (torch.cat([c[~valid_mask], new_centers]), torch.cat([l[~valid_mask], new_levels]),
+            torch.cat([w[~valid_mask], new_weights]), torch.cat([s[~valid_mask], new_scores]))
+    got = oracle.field_subdivide(centers, levels, weights, scores, initial.numpy(), threshold)
+    assert int(valid_mask.sum()) > 100 and (levels[valid_mask.numpy()] < 6).all()
+    for g, t in zip(got, want):
+        np.testing.assert_array_equal(g, t.numpy())
+    # the size limit of :223-224
+    assert oracle.field_subdivide(centers, levels, weights, scores, initial.numpy(), threshold, max_leaves=3500) is None
