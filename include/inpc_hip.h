@@ -348,6 +348,24 @@ int inpc_field_subdivide(const float* centers, const int32_t* levels, const floa
                          float* weights_out, float* scores_out, uint32_t* count_out,
                          void* workspace, size_t workspace_bytes, void* stream);
 
+/* Quasi-random positions from per-leaf sample counts: the deterministic part of
+ * ProbabilityField.extract_global (Modules/ProbabilityField.py:131-140) with compute_halton_coords /
+ * generate_halton_sequence / halton_base (utils.py:36-64). Sample s lies in the leaf whose run of
+ * the exclusive sum of `counts` holds it; with h its 0-based number in that run, its position is
+ * centre - size / 2 + halton(h + 1; 2, 3, 5) * size, size = initial_size / 2^level, or the centre
+ * when the leaf has one sample. The radical inverses are accumulated in double precision as in
+ * the reference's Python loop and rounded to float once, so the positions are bit-identical.
+ * counts (L,) i64 dev as torch.bincount returns them; positions_out (n_samples, 3) f32 dev;
+ * initial_size: 3 floats on the host. The multinomial draw in front (:130) and the optional Morton
+ * order behind (:141-143, CudaUtils.MortonEncoding, not part of the reference tree) stay with the
+ * caller. inpc_extract_global_check synchronises and fails unless the counts are in range and add
+ * up to n_samples. */
+size_t inpc_extract_global_workspace_bytes(uint32_t n_leaves);
+int inpc_extract_global(const float* centers, const int32_t* levels, const int64_t* counts,
+                        uint32_t n_leaves, const float initial_size[3], float* positions_out,
+                        uint32_t n_samples, void* workspace, size_t workspace_bytes, void* stream);
+int inpc_extract_global_check(const void* workspace, uint32_t n_samples, void* stream);
+
 /* grads (= or +=, `add` != 0) factor(i) * weights[i], factor = 0.1 * 2 / (entries of the hash-grid
  * level that holds flat index i), 0 in front of index 6144. Replaces
  * compute_normalized_weight_decay_grads_cu<add> (B/misc/src/misc_kernels.cu:6-47) behind

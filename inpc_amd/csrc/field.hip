@@ -236,6 +236,106 @@ __global__ void __launch_bounds__(kBlock) k_subdivide_apply(LeafArrays in, LeafO
     }
 }
 
+
+// ---- quasi-random positions from per-leaf sample counts (Modules/ProbabilityField.py:131-140, utils.py:36-64) -------
+// Sample s belongs to the leaf whose run [first[leaf], first[leaf + 1]) of the exclusive sum of the counts
+// holds s (arange.repeat_interleave(counts)); with h = s - first[leaf] its position is
+//   centre - size / 2 + halton(h + 1) * size,  size = initial_size / 2^level,
+// or the centre itself when the leaf has a single sample. halton(i) = radical inverse of i in the bases 2, 3, 5,
+// accumulated in double precision exactly as the reference's Python loop does and rounded to float once.
+__global__ void __launch_bounds__(kBlock) k_count_block_sums(const int64_t* __restrict__ counts, uint32_t n,
+                                                             uint32_t* __restrict__ block_sums, uint32_t* error_flag) {
+    __shared__ uint32_t s_sum;
+    if (threadIdx.x == 0) s_sum = 0u;
+    __syncthreads();
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kSelectItems; ++j) {
+        const uint32_t i = blockIdx.x * kSelectTile + j * kBlock + threadIdx.x;
+        if (i < n) {
+            const int64_t c = counts[i];
+            if (c < 0 || c > 0x7FFFFFFF) atomicOr(error_flag, 1u);
+            else mine += (uint32_t)c;
+        }
+    }
+    for (int sh = 32; sh > 0; sh >>= 1) mine += __shfl_down(mine, sh, 64);
+    if ((threadIdx.x & 63u) == 0u && mine) atomicAdd(&s_sum, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = s_sum;
+}
+
+// first[i] = sum of counts[0 .. i), i = 0 .. n (block_first: the scanned block sums)
+__global__ void __launch_bounds__(kBlock) k_count_offsets(const int64_t* __restrict__ counts, uint32_t n,
+                                                          const uint32_t* __restrict__ block_first,
+                                                          uint32_t* __restrict__ first) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t run = block_first[blockIdx.x];
+#pragma unroll
+    for (int j = 0; j < kSelectItems; ++j) {
+        const uint32_t i = blockIdx.x * kSelectTile + j * kBlock + threadIdx.x;
+        const uint32_t v = i < n ? (uint32_t)counts[i] : 0u;
+        uint32_t incl = v;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (lane >= (uint32_t)d) incl += up;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        uint32_t before = run, all = 0;
+#pragma unroll
+        for (int w = 0; w < kBlock / kWave; ++w) {
+            const uint32_t c = s_wave[w];
+            if ((uint32_t)w < wave) before += c;
+            all += c;
+        }
+        if (i < n) {
+            first[i] = before + incl - v;
+            if (i == n - 1) first[n] = before + incl;
+        }
+        run += all;
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ float halton(uint32_t index, uint32_t base) {   // utils.py:36-45
+    double result = 0.0, f = 1.0 / (double)base;
+    for (uint32_t i = index; i > 0; i /= base) {
+        result += f * (double)(i % base);
+        f /= (double)base;
+    }
+    return (float)result;
+}
+
+__global__ void __launch_bounds__(kBlock) k_extract_global(const float* __restrict__ centers, const int32_t* __restrict__ levels,
+                                                           const uint32_t* __restrict__ first, uint32_t n_leaves,
+                                                           float size_x, float size_y, float size_z,
+                                                           float* __restrict__ positions, uint32_t n_samples) {
+    const uint32_t s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= n_samples) return;
+    // last leaf with first[leaf] <= s (leaves without samples have empty runs and are never that leaf)
+    uint32_t lo = 0, hi = n_leaves;
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (first[mid] <= s) lo = mid;
+        else hi = mid;
+    }
+    const uint32_t leaf = lo, begin = first[leaf], count = first[leaf + 1] - begin;
+    float x = centers[3 * (size_t)leaf], y = centers[3 * (size_t)leaf + 1], z = centers[3 * (size_t)leaf + 2];
+    if (count != 1u) {
+        const uint32_t h = s - begin + 1u;
+        const int level = levels[leaf];
+        const float sx = ldexpf(size_x, -level), sy = ldexpf(size_y, -level), sz = ldexpf(size_z, -level);
+        x = (x - sx / 2.0f) + halton(h, 2u) * sx;
+        y = (y - sy / 2.0f) + halton(h, 3u) * sy;
+        z = (z - sz / 2.0f) + halton(h, 5u) * sz;
+    }
+    positions[3 * (size_t)s] = x;
+    positions[3 * (size_t)s + 1] = y;
+    positions[3 * (size_t)s + 2] = z;
+}
+
 int select_offsets(const float* values, const int32_t* levels, uint32_t n, float threshold, int max_level,
                    uint32_t* block_offsets, uint32_t* counts, hipStream_t stream) {
     const uint32_t blocks = div_up(n, kSelectTile);
@@ -345,6 +445,52 @@ int inpc_field_subdivide(const float* centers, const int32_t* levels, const floa
                 (LeafArrays{centers, levels, weights, scores}), (LeafOutputs{centers_out, levels_out, weights_out, scores_out}),
                 n_leaves, threshold, max_level, initial_size[0], initial_size[1], initial_size[2], (const uint32_t*)offsets,
                 (const uint32_t*)count_out);
+    return INPC_OK;
+}
+
+
+size_t inpc_extract_global_workspace_bytes(uint32_t n_leaves) {
+    const size_t blocks = inpc::div_up(std::max(n_leaves, 1u), (uint32_t)inpc::kSelectTile);
+    return 256 + inpc::align_up(blocks * 4, 256) + ((size_t)n_leaves + 1) * 4;
+}
+
+int inpc_extract_global(const float* centers, const int32_t* levels, const int64_t* counts, uint32_t n_leaves,
+                        const float initial_size[3], float* positions_out, uint32_t n_samples, void* workspace,
+                        size_t workspace_bytes, void* stream_) {
+    using namespace inpc;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!workspace || workspace_bytes < inpc_extract_global_workspace_bytes(n_leaves))
+        return fail(INPC_E_WORKSPACE, "extract_global: workspace too small");
+    uint32_t* head = (uint32_t*)workspace;   // [0] total of the counts, [1] error flag
+    int rc = fill_u32(head, 0u, 2, stream);
+    if (rc != INPC_OK) return rc;
+    if (n_leaves == 0 || n_samples == 0) return INPC_OK;
+    if (!centers || !levels || !counts || !initial_size || !positions_out)
+        return fail(INPC_E_INVALID_ARGUMENT, "extract_global: null pointer");
+    const uint32_t blocks = div_up(n_leaves, kSelectTile);
+    uint32_t* block_sums = head + 64;
+    uint32_t* first = (uint32_t*)((char*)workspace + 256 + align_up((size_t)blocks * 4, 256));
+    INPC_LAUNCH("global_count_sums", k_count_block_sums, dim3(blocks), dim3(kBlock), stream, counts, n_leaves, block_sums,
+                head + 1);
+    INPC_LAUNCH("field_select_scan", k_select_scan, dim3(1), dim3(kBlock), stream, block_sums, blocks, head);
+    INPC_LAUNCH("global_count_offsets", k_count_offsets, dim3(blocks), dim3(kBlock), stream, counts, n_leaves,
+                (const uint32_t*)block_sums, first);
+    INPC_LAUNCH("extract_global", k_extract_global, dim3(div_up(n_samples, kBlock)), dim3(kBlock), stream, centers, levels,
+                (const uint32_t*)first, n_leaves, initial_size[0], initial_size[1], initial_size[2], positions_out,
+                n_samples);
+    return INPC_OK;
+}
+
+int inpc_extract_global_check(const void* workspace, uint32_t n_samples, void* stream_) {
+    using namespace inpc;
+    hipStream_t stream = (hipStream_t)stream_;
+    uint32_t head[2] = {0, 0};
+    INPC_HIP_CHECK(hipMemcpyAsync(head, workspace, 8, hipMemcpyDeviceToHost, stream));
+    INPC_HIP_CHECK(hipStreamSynchronize(stream));
+    if (head[1]) return fail(INPC_E_INVALID_ARGUMENT, "extract_global: a count is negative or above 2^31 - 1");
+    if (head[0] != n_samples)
+        return fail(INPC_E_INVALID_ARGUMENT, "extract_global: the counts add up to %u, not to the %u samples asked for",
+                    head[0], n_samples);
     return INPC_OK;
 }
 

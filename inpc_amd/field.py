@@ -9,6 +9,8 @@ to the module's buffers.
 """
 from __future__ import annotations
 
+import ctypes as C
+
 import torch
 
 from . import _lib
@@ -65,6 +67,15 @@ def _leaf_tensors(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scor
     return tensors, n
 
 
+def _host_size(initial_cell_size):
+    size = torch.as_tensor(initial_cell_size, dtype=torch.float32).flatten().cpu()
+    if size.numel() == 1:
+        size = size.repeat(3)
+    if size.numel() != 3:
+        raise RuntimeError("initial_cell_size: one value or one per axis expected")
+    return (C.c_float * 3)(*[float(v) for v in size])
+
+
 def _select_workspace(n, device):
     ws_bytes = int(_lib.lib().inpc_field_select_workspace_bytes(n))
     return torch.empty(ws_bytes, dtype=torch.uint8, device=device), ws_bytes
@@ -97,13 +108,7 @@ def subdivide_probability_field(leaf_centers, leaf_levels, leaf_weights, leaf_su
     (centers, levels, weights, scores), n = _leaf_tensors(leaf_centers, leaf_levels, leaf_weights, leaf_subdivision_scores)
     device = weights.device
     lib = _lib.lib()
-    size = torch.as_tensor(initial_cell_size, dtype=torch.float32).flatten().cpu()
-    if size.numel() == 1:
-        size = size.repeat(3)
-    if size.numel() != 3:
-        raise RuntimeError("initial_cell_size: one value or one per axis expected")
-    import ctypes as C
-    size_host = (C.c_float * 3)(*[float(v) for v in size])
+    size_host = _host_size(initial_cell_size)
     count = torch.zeros(1, dtype=torch.int32, device=device)
     ws, ws_bytes = _select_workspace(n, device)
     stream = _lib.current_stream()
@@ -119,3 +124,36 @@ def subdivide_probability_field(leaf_centers, leaf_levels, leaf_weights, leaf_su
                                         float(threshold), int(max_level), size_host, *(_lib.ptr(t) for t in out),
                                         _lib.ptr(count), _lib.ptr(ws), ws_bytes, stream), "inpc_field_subdivide")
     return out
+
+
+@torch.no_grad()
+def extract_global_samples(leaf_centers: torch.Tensor, leaf_levels: torch.Tensor, initial_cell_size,
+                           counts: torch.Tensor) -> torch.Tensor:
+    """Quasi-random positions, counts[l] of them in leaf l, leaves in order: what ProbabilityField.extract_global
+    computes between its multinomial draw and its optional Morton ordering (Modules/ProbabilityField.py:131-140;
+    Halton points in the cell, the centre for a leaf with a single sample). `counts` is the result of
+    `torch.bincount(indices, minlength=n_leaves)`."""
+    if leaf_centers.dtype != torch.float32:
+        raise RuntimeError("expected scalar type Float")
+    if leaf_levels.dtype != torch.int32:
+        raise RuntimeError("expected scalar type Int")
+    if counts.dtype != torch.int64:
+        raise RuntimeError("expected scalar type Long")
+    n = leaf_levels.numel()
+    if leaf_centers.shape != (n, 3) or counts.shape != (n,):
+        raise RuntimeError("centers (n, 3), levels (n,) and counts (n,) of one octree expected")
+    centers, levels, counts = leaf_centers.contiguous(), leaf_levels.contiguous(), counts.contiguous()
+    if not (centers.is_cuda and levels.is_cuda and counts.is_cuda):
+        raise RuntimeError("expected tensors on the GPU")
+    n_samples = int(counts.sum().item())   # the reference reads it as well (utils.py:58)
+    device = centers.device
+    positions = torch.empty((n_samples, 3), dtype=torch.float32, device=device)
+    lib = _lib.lib()
+    ws_bytes = int(lib.inpc_extract_global_workspace_bytes(n))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
+    stream = _lib.current_stream()
+    _lib.check(lib.inpc_extract_global(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(counts), n,
+                                       _host_size(initial_cell_size), _lib.ptr(positions), n_samples, _lib.ptr(ws),
+                                       ws_bytes, stream), "inpc_extract_global")
+    _lib.check(lib.inpc_extract_global_check(_lib.ptr(ws), n_samples, stream), "inpc_extract_global")
+    return positions

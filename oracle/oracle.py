@@ -445,6 +445,37 @@ def field_subdivide(centers, levels, weights, scores, initial_size, threshold, m
     return np.concatenate(out_c), np.concatenate(out_l), np.concatenate(out_w), np.concatenate(out_s)
 
 
+def halton_base(index: int, base: int) -> float:
+    """utils.py:36-45."""
+    result, f, i = 0.0, 1.0 / base, index
+    while i > 0:
+        result += f * (i % base)
+        i //= base
+        f /= base
+    return result
+
+
+def extract_global_samples(centers, levels, initial_size, counts):
+    """Modules/ProbabilityField.py:131-140 with utils.py:36-64, sample by sample."""
+    centers, levels = np.asarray(centers, np.float32), np.asarray(levels, np.int32)
+    counts = np.asarray(counts, np.int64)
+    size0 = np.broadcast_to(np.asarray(initial_size, np.float32).reshape(-1), (3,))
+    out = np.empty((int(counts.sum()), 3), np.float32)
+    s = 0
+    for leaf in np.flatnonzero(counts):
+        c = int(counts[leaf])
+        if c == 1:
+            out[s] = centers[leaf]
+        else:
+            size = (size0 / np.float32(2 ** int(levels[leaf]))).astype(np.float32)
+            corner = (centers[leaf] - size / np.float32(2.0)).astype(np.float32)
+            for h in range(c):
+                coords = np.array([halton_base(h + 1, 2), halton_base(h + 1, 3), halton_base(h + 1, 5)]).astype(np.float32)
+                out[s + h] = corner + (coords * size).astype(np.float32)
+        s += c
+    return out
+
+
 def spherical_contraction(positions):
     """B/misc/src/misc_kernels.cu:49-66, every operation rounded to float32 in the written order."""
     p = np.asarray(positions, np.float32).reshape(-1, 3)

@@ -110,3 +110,29 @@ def test_subdivide_bit_exact(gpu, oracle, n):
     n_split = (len(want[1]) - n) // 7
     if n_split:
         assert subdivide_probability_field(*(H.dev(a) for a in arrays), size, 0.55, max_leaves=len(want[1]) - 1) is None
+
+
+def test_extract_global_bit_exact(gpu, oracle):
+    from inpc_amd import extract_global_samples
+
+    rng = np.random.default_rng(9)
+    n_leaves = 5000
+    centers = rng.uniform(-2, 2, (n_leaves, 3)).astype(np.float32)
+    levels = rng.integers(0, 7, n_leaves).astype(np.int32)
+    size = np.array([0.37, 0.37, 0.37], np.float32)
+    indices = rng.integers(0, n_leaves, 40000)
+    indices[:3000] = 11         # one crowded leaf
+    indices = indices[indices % 5 != 0]   # a fifth of the leaves stays empty
+    counts = np.bincount(indices, minlength=n_leaves).astype(np.int64)
+    got = extract_global_samples(H.dev(centers), H.dev(levels), size, H.dev(counts)).cpu().numpy()
+    want = oracle.extract_global_samples(centers, levels, size, counts)
+    assert (counts == 1).sum() > 10 and (counts == 0).sum() > 100
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    # inside the cell
+    cell = np.repeat(np.arange(n_leaves), counts)
+    half = (size[None, :] / (2.0 ** levels[cell])[:, None]) / 2
+    assert (np.abs(got - centers[cell]) <= half * (1 + 1e-6)).all()
+    with pytest.raises(RuntimeError):
+        bad = counts.copy()
+        bad[0] = -1
+        extract_global_samples(H.dev(centers), H.dev(levels), size, H.dev(bad))

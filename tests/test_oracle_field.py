@@ -1,6 +1,7 @@
 """Pins the oracle's probability-field update against the reference's own formulation (the torch calls of
 Modules/ProbabilityField.py:146-157, evaluated by torch on the CPU) and against hand-checked cases."""
 import numpy as np
+import pytest
 import torch
 
 
@@ -109,3 +110,46 @@ def test_subdivide_matches_the_references_torch_statements(oracle):
         np.testing.assert_array_equal(g, t.numpy())
     # the size limit of :223-224
     assert oracle.field_subdivide(centers, levels, weights, scores, initial.numpy(), threshold, max_leaves=3500) is None
+
+
+def _reference_halton_base(index, base):
+    # utils.py:36-45
+    result = 0
+    f = 1 / base
+    i = index
+    while i > 0:
+        result += f * (i % base)
+        i = i // base
+        f /= base
+    return result
+
+
+def test_extract_global_matches_the_references_torch_statements(oracle):
+    # Modules/ProbabilityField.py:131-140 and utils.py:48-64 run by torch on the CPU, statement by statement
+    rng = np.random.default_rng(23)
+    n_leaves = 400
+    centers = torch.from_numpy(rng.uniform(-2, 2, (n_leaves, 3)).astype(np.float32))
+    levels = torch.from_numpy(rng.integers(0, 7, n_leaves).astype(np.int32))
+    initial = torch.tensor([0.37, 0.37, 0.37], dtype=torch.float32)
+    indices = torch.from_numpy(rng.integers(0, n_leaves, 900))
+    indices[:40] = 7           # one crowded leaf, many leaves with a single sample or none
+    counts = torch.bincount(indices, minlength=n_leaves)
+    cell = torch.arange(n_leaves, dtype=torch.int32).repeat_interleave(counts)
+    offsets = torch.cumsum(counts, dim=0) - counts
+    halton_indices = torch.arange(counts.sum().item(), dtype=torch.int32) - offsets[cell]
+    table = torch.zeros((halton_indices.max().item() + 1, 3))
+    for i in range(table.shape[0]):
+        for j, prime in enumerate([2, 3, 5]):
+            table[i][j] = _reference_halton_base(i + 1, prime)
+    halton_coords = table[halton_indices]
+    cell_size = initial / 2 ** levels[cell, None]
+    initial_samples = centers[cell]
+    samples = initial_samples - (cell_size / 2) + halton_coords * cell_size
+    single = (counts == 1).repeat_interleave(counts)
+    samples[single] = initial_samples[single]
+    got = oracle.extract_global_samples(centers.numpy(), levels.numpy(), initial.numpy(), counts.numpy())
+    assert (counts == 1).sum() > 5 and (counts == 0).sum() > 0 and counts.max() >= 40
+    np.testing.assert_array_equal(got.view(np.uint32), samples.numpy().view(np.uint32))
+    # the first Halton points, as published: 1/2, 1/3, 1/5; 1/4, 2/3, 2/5; 3/4, 1/9, 3/5
+    assert [oracle.halton_base(1, b) for b in (2, 3, 5)] == pytest.approx([1 / 2, 1 / 3, 1 / 5])
+    assert [oracle.halton_base(3, b) for b in (2, 3, 5)] == pytest.approx([3 / 4, 1 / 9, 3 / 5])
