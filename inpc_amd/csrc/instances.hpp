@@ -21,15 +21,23 @@ namespace instances {
 #define INPC_INST_CHUNKS 1024
 #endif
 constexpr int kChunks = INPC_INST_CHUNKS;  // contiguous chunks of the depth-ordered points, one block each
-constexpr int kEmitThreads = 256;
+#ifndef INPC_EMIT_THREADS
+#define INPC_EMIT_THREADS 512
+#endif
+constexpr int kEmitThreads = INPC_EMIT_THREADS;
 #ifndef INPC_EMIT_ITEMS
-#define INPC_EMIT_ITEMS 8
+#define INPC_EMIT_ITEMS 4
 #endif
 constexpr int kEmitItems = INPC_EMIT_ITEMS;                          // points per thread and sub-chunk
 constexpr int kEmitPoints = kEmitThreads * kEmitItems;  // points per sub-chunk
-constexpr int kStage = 3072;                            // instances sorted in LDS at a time
+#ifndef INPC_EMIT_STAGE
+#define INPC_EMIT_STAGE 3072
+#endif
+constexpr int kStage = INPC_EMIT_STAGE;                 // instances sorted in LDS at a time
 constexpr int kStageItems = kStage / kEmitThreads;      // per thread
 constexpr int kSortWaves = kEmitThreads / kWave;
+static_assert(kEmitThreads >= radix::kRadix, "thread d owns digit d in the LDS digit passes");
+static_assert(kStage % kEmitThreads == 0 && kEmitItems % 4 == 0, "whole rows per thread, 16-byte loads of the sort values");
 constexpr uint32_t kNoPoint = 0xFFFFFFFFu;
 
 __host__ __device__ inline uint32_t chunk_size(uint32_t n) {
@@ -156,7 +164,7 @@ __device__ __forceinline__ void lds_digit_pass(uint16_t* s_key, uint32_t* s_val,
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w)
         if ((uint32_t)w < wave) wave_off += s_wave_total[w];
-    s_base[tid] = wave_off + incl - total;
+    if (tid < (uint32_t)radix::kRadix) s_base[tid] = wave_off + incl - total;   // one entry per digit, not per thread
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kStageItems; ++r) {
