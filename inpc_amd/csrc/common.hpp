@@ -172,7 +172,10 @@ __device__ __forceinline__ uint32_t lookback_walk(uint32_t* status, uint32_t str
     if (bid == 0) return 0u;
     // Several predecessors are fetched per round trip and consumed nearest first; the walk ends at the
     // first one that carries an inclusive prefix and waits at the first one that has nothing yet.
-    constexpr int kAhead = 8;
+#ifndef INPC_LOOKBACK_AHEAD
+#define INPC_LOOKBACK_AHEAD 8
+#endif
+    constexpr int kAhead = INPC_LOOKBACK_AHEAD;
     uint32_t exclusive = 0u, spins = 0u;
     int64_t p = (int64_t)bid - 1;
     bool finished = false;

@@ -36,7 +36,8 @@ constexpr int kEmitPoints = kEmitThreads * kEmitItems;  // points per sub-chunk
 constexpr int kStage = INPC_EMIT_STAGE;                 // instances sorted in LDS at a time
 constexpr int kStageItems = kStage / kEmitThreads;      // per thread
 constexpr int kSortWaves = kEmitThreads / kWave;
-static_assert(kEmitThreads >= radix::kRadix, "thread d owns digit d in the LDS digit passes");
+constexpr int kDigits = 256;                            // the LDS digit passes take at most 8 bits (16-bit tile keys)
+static_assert(kEmitThreads >= kDigits, "thread d owns digit d in the LDS digit passes");
 static_assert(kStage % kEmitThreads == 0 && kEmitItems % 4 == 0, "whole rows per thread, 16-byte loads of the sort values");
 constexpr uint32_t kNoPoint = 0xFFFFFFFFu;
 
@@ -104,10 +105,10 @@ __global__ void __launch_bounds__(kBlock) k_ranges_from_starts(const uint32_t* _
 // One stable digit pass over s_key / s_val [0, n) in LDS. Element (wave w, row r, lane l) = w * kStageItems * 64 +
 // r * 64 + l, so a wave's elements are consecutive and the per-wave ranking by ballots is stable.
 __device__ __forceinline__ void lds_digit_pass(uint16_t* s_key, uint32_t* s_val, uint32_t n, int shift, int bits,
-                                               uint32_t (*s_cnt)[radix::kRadix], uint32_t* s_base) {
+                                               uint32_t (*s_cnt)[kDigits], uint32_t* s_base) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t digit_mask = (1u << bits) - 1u;
-    for (uint32_t i = tid; i < kSortWaves * radix::kRadix; i += kEmitThreads) (&s_cnt[0][0])[i] = 0u;
+    for (uint32_t i = tid; i < kSortWaves * kDigits; i += kEmitThreads) (&s_cnt[0][0])[i] = 0u;
     uint32_t key[kStageItems], val[kStageItems], rank[kStageItems];
     uint32_t valid_bits = 0;
 #pragma unroll
@@ -164,7 +165,7 @@ __device__ __forceinline__ void lds_digit_pass(uint16_t* s_key, uint32_t* s_val,
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w)
         if ((uint32_t)w < wave) wave_off += s_wave_total[w];
-    if (tid < (uint32_t)radix::kRadix) s_base[tid] = wave_off + incl - total;   // one entry per digit, not per thread
+    if (tid < (uint32_t)kDigits) s_base[tid] = wave_off + incl - total;   // one entry per digit, not per thread
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kStageItems; ++r) {
@@ -188,8 +189,8 @@ __global__ void __launch_bounds__(kEmitThreads)
     __shared__ uint16_t s_key[kStage];
     __shared__ uint32_t s_val[kStage];
     __shared__ uint16_t s_first[kStage];    // index of the first element of the element's tile run
-    __shared__ uint32_t s_cnt[kSortWaves][radix::kRadix];
-    __shared__ uint32_t s_base[radix::kRadix];
+    __shared__ uint32_t s_cnt[kSortWaves][kDigits];
+    __shared__ uint32_t s_base[kDigits];
     __shared__ uint32_t s_scan[kSortWaves];
     __shared__ int s_carry[kSortWaves];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;

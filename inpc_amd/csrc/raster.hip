@@ -161,7 +161,10 @@ __device__ __forceinline__ Projected project_point(const ViewRows& m, const Geom
 // k_bin_scan into the start of every tile's bin. k_preprocess then hands out slots from LDS cursors
 // seeded with bin_start[tile] + prefix[chunk][tile]: no global atomic anywhere (they run at about
 // 10 G/s on this machine, far below what 8M points need).
-constexpr int kBinBlocks = 512;
+#ifndef INPC_BIN_BLOCKS
+#define INPC_BIN_BLOCKS 512
+#endif
+constexpr int kBinBlocks = INPC_BIN_BLOCKS;
 constexpr int kBinThreads = 512;
 constexpr uint32_t kMaxLdsTiles = 16384;  // tile counters a block keeps in LDS (64 KiB)
 
