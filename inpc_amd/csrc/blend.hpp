@@ -184,6 +184,9 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
     for (int q = 0; q < NQ; ++q) in_quad[q] = false;
 #pragma unroll
     for (int c = 0; c < 4; ++c) weight[c] = 0.0f;
+    uint64_t finished[NQ];   // read up front, all at once: the tests below would each wait for their own read
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) finished[q] = st.done[q];
     if (valid) {
 #pragma unroll
         for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
@@ -214,7 +217,7 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
                 const int pix = hit ? gy[by] * 8 + gx[bx] : 0;
                 weight[c] = wx[bx] * wy[by];
                 field[c] = hit ? (uint32_t)pix : kNoFragment;
-                in_quad[c] = hit && ((st.done[c] >> pix) & 1ull) == 0ull;
+                in_quad[c] = hit && ((finished[c] >> pix) & 1ull) == 0ull;
             }
         } else {
 #pragma unroll
@@ -224,7 +227,7 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
                 const int pix = hit ? (ay.first + ky) * 8 + (ax.first + kx) : 0;
                 weight[c] = ax.weight[kx] * ay.weight[ky];
                 field[c] = hit ? (uint32_t)pix : kNoFragment;
-                if (hit && ((st.done[0] >> pix) & 1ull) == 0ull) in_quad[0] = true;
+                if (hit && ((finished[0] >> pix) & 1ull) == 0ull) in_quad[0] = true;
             }
         }
         const float4 alpha = make_float4(h.opacity * weight[0], h.opacity * weight[1], h.opacity * weight[2], h.opacity * weight[3]);
