@@ -96,7 +96,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
-              "(the path is single-GPU, see DESIGN.md for how it would shard)", file=sys.stderr)
+              "(the path runs on a single GPU)", file=sys.stderr)
         return 2
 
     import numpy as np
