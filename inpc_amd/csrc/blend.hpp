@@ -5,14 +5,14 @@
 // tiles; for 16x16 tiles the pixels of one parity class (x odd / even, y odd / even), so that the 2 x 2
 // footprint of a point gives every wave exactly one fragment and a cluster of points on one spot loads the
 // four waves evenly. Per batch of T*T instances:
-//   stage    thread t gathers the record of instance t into LDS, finds the waves ("quads") in which it covers a
-//            pixel that is still open, and appends t, in depth order, to the list of each such quad;
-//   consume  every wave takes its whole list at once (up to four entries per lane), with wave-level
-//            synchronisation only: hit masks per pixel -> per-pixel fragment lists in depth order -> the
+//   stage    thread t puts the record of instance t into LDS: screen position, opacity, features;
+//   consume  every wave goes over the whole batch (up to four instances per lane) and derives, for each
+//            instance, the one fragment that falls into its parity class (8x8 tiles: all four fragments), with
+//            wave-level synchronisation only: hit masks per pixel -> per-pixel fragment lists in depth order -> the
 //            sequential transmittance chain per pixel (short lists) or a wave-wide product scan (long
 //            lists); the results stay in the fragment list;
 //   write    thread t collects the results of instance t's fragments: a plain store when the point lies in
-//            one tile only, atomics when it straddles tiles.
+//            one tile only, rows of its own when it straddles tiles (forward: atomics).
 // Two block barriers per batch; the record gather runs two batches ahead of the blend.
 #pragma once
 
@@ -111,10 +111,9 @@ struct Shape {
     static constexpr int K = T == 16 ? 4 : 1;
 };
 
-// Fragment field of a staged instance (16 bits per slot): bits 0-5 the pixel in the owning wave's grid
-// (row * 8 + column), bit 6: the instance has no fragment in this slot, bit 7: the wave has placed the
-// fragment in its list, bits 8-15: where.
-constexpr uint32_t kPixelMask = 63u, kNoFragment = 0x40u, kPlaced = 0x80u;
+// Fragment field of a staged instance (16 bits per slot), 0 until the slot's wave places the fragment in its
+// list: bits 0-5 the pixel in the owning wave's grid (row * 8 + column), bit 7: placed, bits 8-15: where.
+constexpr uint32_t kPixelMask = 63u, kPlaced = 0x80u;
 constexpr uint32_t kNoPixel = 0xFFu;
 
 // Per-block staging area of one batch.
@@ -124,11 +123,8 @@ struct Stage {
     static constexpr int NQ = TT / 64;
     float4 feat[TT * (C / 4)];
     float depth[WITH_DEPTH ? TT : 1];
-    alignas(16) float alpha[TT][4];     // per slot: opacity x interpolation weight
-    alignas(8) uint16_t frag[TT][4];    // per slot: the fragment field
-    uint8_t list[NQ][NQ][64];           // [quad][source wave][rank]: staged instances with an open pixel in the quad
-    uint8_t count[NQ][NQ];
-    uint64_t done[NQ];                  // per quad: pixels that are finished
+    float4 point[TT];                   // sx, sy, opacity of the staged instance
+    alignas(8) uint16_t frag[TT][4];    // per slot: the fragment field, written by the wave that placed the fragment
 };
 
 // Per-wave scratch of the consume phase. A fragment entry is {alpha, x} on the way in and {blending weight, y}
@@ -170,158 +166,107 @@ __device__ __forceinline__ Header read_header(const char* __restrict__ record) {
     return h;
 }
 
-// Stage instance `t` (thread t): features, the alpha and pixel of its fragment in every slot, and its entry, in
-// depth order, in the list of each quad where it covers an open pixel. `valid` is false for the threads behind
-// the end of the batch. Leaves the interpolation weights of the four slots in `weight`. Must be followed by a
-// block barrier.
-template <int T, int C, bool WITH_DEPTH>
-__device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool valid, const Header& h,
-                                               const float (&f)[C], int tile_x0, int tile_y0, float (&weight)[4]) {
-    constexpr int NQ = T * T / 64;
-    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-    bool in_quad[NQ];
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) in_quad[q] = false;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) weight[c] = 0.0f;
-    uint64_t finished[NQ];   // read up front, all at once: the tests below would each wait for their own read
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) finished[q] = st.done[q];
-    if (valid) {
-#pragma unroll
-        for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
-        if (WITH_DEPTH) st.depth[t] = h.depth;
-        // the float test of B/rasterization/src/bilinear/kernels.cu:284-287 for the 2 x 2 candidate pixels
-        const AxisCover ax = cover_axis<T>(h.sx, tile_x0), ay = cover_axis<T>(h.sy, tile_y0);
-        uint32_t field[4];
-        if (T == 16) {
-            // slot = parity class (y parity, x parity) of the pixel; per axis, the candidate with parity b
-            const bool odd_x = (ax.first & 1) != 0, odd_y = (ay.first & 1) != 0;
-            bool hx[2], hy[2];
-            float wx[2], wy[2];
-            int gx[2], gy[2];
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const bool second_x = odd_x != (b != 0), second_y = odd_y != (b != 0);   // candidate 1 has parity b
-                hx[b] = second_x ? ax.hit[1] : ax.hit[0];
-                wx[b] = second_x ? ax.weight[1] : ax.weight[0];
-                gx[b] = (ax.first + (second_x ? 1 : 0)) >> 1;
-                hy[b] = second_y ? ay.hit[1] : ay.hit[0];
-                wy[b] = second_y ? ay.weight[1] : ay.weight[0];
-                gy[b] = (ay.first + (second_y ? 1 : 0)) >> 1;
-            }
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int by = c >> 1, bx = c & 1;
-                const bool hit = hx[bx] && hy[by];
-                const int pix = hit ? gy[by] * 8 + gx[bx] : 0;
-                weight[c] = wx[bx] * wy[by];
-                field[c] = hit ? (uint32_t)pix : kNoFragment;
-                in_quad[c] = hit && ((finished[c] >> pix) & 1ull) == 0ull;
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int ky = c >> 1, kx = c & 1;
-                const bool hit = ax.hit[kx] && ay.hit[ky];
-                const int pix = hit ? (ay.first + ky) * 8 + (ax.first + kx) : 0;
-                weight[c] = ax.weight[kx] * ay.weight[ky];
-                field[c] = hit ? (uint32_t)pix : kNoFragment;
-                if (hit && ((finished[0] >> pix) & 1ull) == 0ull) in_quad[0] = true;
-            }
-        }
-        const float4 alpha = make_float4(h.opacity * weight[0], h.opacity * weight[1], h.opacity * weight[2], h.opacity * weight[3]);
-        __builtin_memcpy(st.alpha[t], &alpha, 16);
-        const uint2 fields = make_uint2(field[0] | (field[1] << 16), field[2] | (field[3] << 16));
-        __builtin_memcpy(st.frag[t], &fields, 8);
-    }
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-        const uint64_t members = __ballot(in_quad[q]);
-        if (in_quad[q]) st.list[q][wave][mask_rank(members)] = (uint8_t)t;
-        if (lane == 0u) st.count[q][wave] = (uint8_t)__popcll(members);
-    }
-}
-
-// A quad's list is the concatenation, in wave order, of the pieces the NQ source waves wrote. ListIndex holds
-// the piece boundaries of one batch (the same in every lane).
-template <int NQ>
-struct ListIndex {
-    uint32_t end[NQ];  // end[s]: entries in the pieces 0..s; end[NQ - 1] is the length of the list
+// One candidate pixel of one axis: the one of the two candidates (left_pixel, left_pixel + 1) whose tile-local
+// index has parity `odd`; the float test of B/rasterization/src/bilinear/kernels.cu:284-285 and the
+// interpolation weight of :286-287, the same arithmetic as cover_axis.
+struct AxisCandidate {
+    int index;     // tile-local
+    bool hit;
+    float weight;
 };
 
-template <int T, int C, bool WITH_DEPTH>
-__device__ __forceinline__ ListIndex<T * T / 64> list_index(const Stage<T, C, WITH_DEPTH>& st, uint32_t q) {
-    constexpr int NQ = T * T / 64;
-    ListIndex<NQ> li;
-    uint32_t run = 0;
-#pragma unroll
-    for (int s = 0; s < NQ; ++s) {
-        run += st.count[q][s];
-        li.end[s] = (uint32_t)__builtin_amdgcn_readfirstlane((int)run);
-    }
-    return li;
+template <int T>
+__device__ __forceinline__ AxisCandidate candidate_of_parity(float s, int tile_origin, bool odd) {
+    AxisCandidate a;
+    const int first = left_pixel<T>(s, tile_origin);
+    a.index = first + ((((first & 1) != 0) != odd) ? 1 : 0);
+    const float d = fabsf(s - ((float)(tile_origin + a.index) + 0.5f));
+    a.hit = a.index >= 0 && a.index < T && !(d >= 1.0f);
+    a.weight = __saturatef(1.0f - d);
+    return a;
 }
 
-// The idx-th staged instance of quad q's list, idx < li.end[NQ - 1].
-template <int T, int C, bool WITH_DEPTH>
-__device__ __forceinline__ uint32_t list_entry(const Stage<T, C, WITH_DEPTH>& st, const ListIndex<T * T / 64>& li,
-                                               uint32_t q, uint32_t idx) {
-    constexpr int NQ = T * T / 64;
-    uint32_t w = 0, first = 0;
+// Interpolation weights of the four fragment slots of a point (whether the fragment exists or not).
+template <int T>
+__device__ __forceinline__ void slot_weights(float sx, float sy, int tile_x0, int tile_y0, float (&weight)[4]) {
+    if (T == 16) {
+        float wx[2], wy[2];
 #pragma unroll
-    for (int s = 0; s < NQ - 1; ++s)
-        if (idx >= li.end[s]) {
-            w = s + 1;
-            first = li.end[s];
+        for (int b = 0; b < 2; ++b) {
+            wx[b] = candidate_of_parity<T>(sx, tile_x0, b != 0).weight;
+            wy[b] = candidate_of_parity<T>(sy, tile_y0, b != 0).weight;
         }
-    return st.list[q][w][idx - first];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) weight[c] = wx[c & 1] * wy[c >> 1];
+    } else {
+        const AxisCover ax = cover_axis<T>(sx, tile_x0), ay = cover_axis<T>(sy, tile_y0);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) weight[c] = ax.weight[c & 1] * ay.weight[c >> 1];
+    }
 }
 
-// The list entries of one lane: entry k is number k * 64 + lane of the quad's list; its (at most NF) fragments
-// in this wave's grid. Depth order is the order of (k, lane).
+// Stage instance `t` (thread t). `valid` is false for the threads behind the end of the batch. Must be followed
+// by a block barrier.
+template <int T, int C, bool WITH_DEPTH>
+__device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool valid, const Header& h,
+                                               const float (&f)[C]) {
+    const uint32_t t = threadIdx.x;
+    if (!valid) return;
+#pragma unroll
+    for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
+    if (WITH_DEPTH) st.depth[t] = h.depth;
+    st.point[t] = make_float4(h.sx, h.sy, h.opacity, 0.0f);
+    const uint2 nothing_placed = make_uint2(0u, 0u);
+    __builtin_memcpy(st.frag[t], &nothing_placed, 8);
+}
+
+// The instances of one lane: entry k is staged instance k * 64 + lane; its (at most NF) fragments in this
+// wave's grid. Depth order is the order of (k, lane).
 template <int T>
 struct Entries {
     static constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
-    uint32_t j[K];           // staged instance (0 for an entry behind the end of the list)
-    uint32_t pixel[K][NF];   // kNoPixel: no fragment, or the pixel is finished
+    uint32_t j[K];           // staged instance
+    uint32_t pixel[K][NF];   // kNoPixel: no fragment in this wave's grid, or the pixel is finished
     float alpha[K][NF];
 };
 
+// `count`: staged instances of the batch; `finished`: this wave's pixels that are done.
 template <int T, int C, bool WITH_DEPTH>
-__device__ __forceinline__ void load_entries(const Stage<T, C, WITH_DEPTH>& st, const ListIndex<T * T / 64>& li,
-                                             uint32_t quad, uint64_t finished, Entries<T>& e) {
-    constexpr int K = Shape<T>::K, NF = Shape<T>::NF, NQ = T * T / 64;
+__device__ __forceinline__ void load_entries(const Stage<T, C, WITH_DEPTH>& st, uint32_t count, uint32_t quad,
+                                             int tile_x0, int tile_y0, uint64_t finished, Entries<T>& e) {
+    constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
     const uint32_t lane = __lane_id();
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const uint32_t idx = k * 64u + lane;
-        const bool live = idx < li.end[NQ - 1];
-        const uint32_t j = live ? list_entry<T, C, WITH_DEPTH>(st, li, quad, idx) : 0u;
+        const uint32_t j = k * 64u + lane;
+        const bool live = j < count;
         e.j[k] = j;
-        uint32_t field[NF];
+        const float4 p = st.point[live ? j : 0u];
+        bool hit[NF];
+        uint32_t pix[NF];
+        float weight[NF];
         if (T == 16) {
-            field[0] = st.frag[j][quad];
-            e.alpha[k][0] = st.alpha[j][quad];
+            // the fragment of this wave's parity class (x parity = quad & 1, y parity = quad >> 1)
+            const AxisCandidate cx = candidate_of_parity<T>(p.x, tile_x0, (quad & 1u) != 0u);
+            const AxisCandidate cy = candidate_of_parity<T>(p.y, tile_y0, (quad >> 1) != 0u);
+            hit[0] = cx.hit && cy.hit;
+            pix[0] = (uint32_t)((cy.index >> 1) * 8 + (cx.index >> 1));
+            weight[0] = cx.weight * cy.weight;
         } else {
-            uint2 fields;
-            float4 alpha;
-            __builtin_memcpy(&fields, st.frag[j], 8);
-            __builtin_memcpy(&alpha, st.alpha[j], 16);
-            field[0] = fields.x & 0xFFFFu;
-            field[NF > 1 ? 1 : 0] = fields.x >> 16;
-            field[NF > 2 ? 2 : 0] = fields.y & 0xFFFFu;
-            field[NF > 3 ? 3 : 0] = fields.y >> 16;
-            e.alpha[k][0] = alpha.x;
-            e.alpha[k][NF > 1 ? 1 : 0] = alpha.y;
-            e.alpha[k][NF > 2 ? 2 : 0] = alpha.z;
-            e.alpha[k][NF > 3 ? 3 : 0] = alpha.w;
+            const AxisCover ax = cover_axis<T>(p.x, tile_x0), ay = cover_axis<T>(p.y, tile_y0);
+#pragma unroll
+            for (int q = 0; q < NF; ++q) {
+                const int ky = q >> 1, kx = q & 1;
+                hit[q] = ax.hit[kx] && ay.hit[ky];
+                pix[q] = (uint32_t)((ay.first + ky) * 8 + (ax.first + kx));
+                weight[q] = ax.weight[kx] * ay.weight[ky];
+            }
         }
 #pragma unroll
         for (int q = 0; q < NF; ++q) {
-            uint32_t pix = (live && !(field[q] & kNoFragment)) ? (field[q] & kPixelMask) : kNoPixel;
-            if (pix != kNoPixel && ((finished >> pix) & 1ull)) pix = kNoPixel;
-            e.pixel[k][q] = pix;
+            const bool open = live && hit[q] && ((finished >> (pix[q] & kPixelMask)) & 1ull) == 0ull;
+            e.pixel[k][q] = open ? pix[q] : kNoPixel;
+            e.alpha[k][q] = p.z * weight[q];
         }
     }
 }
@@ -475,11 +420,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
     for (int c = 0; c < C; ++c) F[c] = 0.0f;
     float D = 0.0f, Tr = 1.0f;
     bool done = !inside;
-    {
-        const uint64_t finished = __ballot(done);
-        if (lane == 0u) st.done[wave] = finished;
-    }
-    __syncthreads();
 
     const uint2 range = ranges[tile];
 #ifdef INPC_PROFILE_BACKWARD
@@ -493,18 +433,16 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        float weight[4];
-        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f, tile_x0, tile_y0, weight);
+        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f);
         FWD_MARK(0);
         __syncthreads();
         FWD_MARK(1);
 
         // ---- consume: this wave's list
-        const ListIndex<NQ> li = list_index<T, C, INFERENCE>(st, wave);
         uint32_t my_start = 0, my_count = 0, n_fragments = 0;
-        if (li.end[NQ - 1] != 0u) {
+        {
             Entries<T> e;
-            load_entries<T, C, INFERENCE>(st, li, wave, __ballot(done), e);
+            load_entries<T, C, INFERENCE>(st, count, wave, tile_x0, tile_y0, __ballot(done), e);
             build_fragment_lists<T, C, INFERENCE>(qs, st, wave, e, my_start, my_count, n_fragments,
                                                   [&](int k, int) { return __uint_as_float(e.j[k]); });
         }
@@ -591,10 +529,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
             }
             FWD_MARK(4);
         }
-        {
-            const uint64_t finished = __ballot(done);
-            if (lane == 0u) st.done[wave] = finished;
-        }
         FWD_MARK(2);
         const bool all_done = __syncthreads_and(done) != 0;
         FWD_MARK(5);
@@ -604,12 +538,15 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
         // ---- the gather moves on in front of the stores of the write phase
         const uint32_t point = g.h.point;
         const bool multi = g.h.multi();
+        const float sx = g.h.sx, sy = g.h.sy;
         advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
         // ---- write: thread t owns staged instance t (kernels.cu:291-295): its blending weight is the sum over
         // the fragments the waves placed
         if (!INFERENCE && valid) {
             uint32_t field[4];
             load_fields<T, C, INFERENCE>(st, tid, field);
+            float weight[4];
+            slot_weights<T>(sx, sy, tile_x0, tile_y0, weight);
             float w = 0.0f;
 #pragma unroll
             for (int c = 0; c < 4; ++c)
@@ -748,11 +685,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
     const float offset = common - final_dot;
     float Tr = 1.0f, running = 0.0f;
     bool done = !inside;
-    {
-        const uint64_t finished = __ballot(done);
-        if (lane == 0u) st.done[wave] = finished;
-    }
-    __syncthreads();
 
     const uint2 range = ranges[tile];
 #ifdef INPC_PROFILE_BACKWARD
@@ -766,18 +698,16 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        float weight[4];
-        stage_instance<T, C, false>(st, valid, g.h, g.f, tile_x0, tile_y0, weight);
+        stage_instance<T, C, false>(st, valid, g.h, g.f);
         BWD_MARK(0);
         __syncthreads();
         BWD_MARK(1);
 
         // ---- consume: this wave's list
-        const ListIndex<NQ> li = list_index<T, C, false>(st, wave);
         uint32_t my_start = 0, my_count = 0, n_fragments = 0;
-        if (li.end[NQ - 1] != 0u) {
+        {
             Entries<T> e;
-            load_entries<T, C, false>(st, li, wave, __ballot(done), e);
+            load_entries<T, C, false>(st, count, wave, tile_x0, tile_y0, __ballot(done), e);
             float dots[K][NF];   // features . grad of the fragment's pixel
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -860,10 +790,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
             }
             BWD_MARK(4);
         }
-        {
-            const uint64_t finished = __ballot(done);
-            if (lane == 0u) st.done[wave] = finished;
-        }
         BWD_MARK(2);
         const bool all_done = __syncthreads_and(done) != 0;
         BWD_MARK(5);
@@ -873,11 +799,14 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
         // ---- the gather moves on in front of the stores of the write phase (see the forward kernel)
         const uint32_t point = g.h.point, tiles = g.h.tiles, split = g.h.split;
         const bool multi = g.h.multi();
+        const float sx = g.h.sx, sy = g.h.sy;
         advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
         // ---- write: thread t owns staged instance t: gradient of the point from the fragments the waves placed
         if (valid) {
             uint32_t field[4];
             load_fields<T, C, false>(st, tid, field);
+            float weight[4];
+            slot_weights<T>(sx, sy, tile_x0, tile_y0, weight);
             float gf[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) gf[c] = 0.0f;
