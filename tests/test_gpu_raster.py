@@ -300,3 +300,47 @@ def test_backward_twice_after_one_forward(gpu, oracle, tile):
         gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
         H.assert_close(gf, gf_ref, RTOL, 1e-7, f"feature gradients (half={half})")
         H.assert_close(go, go_ref, RTOL, 2e-7, f"opacity gradients (half={half})")
+
+
+RANDOM_CASES = [
+    # seed, n, width, height, focal, tile, channels, opacity range, cluster share
+    (101, 9000, 37, 29, 40.0, 8, 4, (0.0, 1.0), 0.0),
+    (102, 30000, 130, 71, 110.0, 16, 8, (0.0, 0.2), 0.3),
+    (103, 20000, 65, 65, 70.0, 16, 4, (0.9, 1.0), 0.5),
+    (104, 25000, 129, 33, 95.0, 8, 8, (0.3, 0.7), 0.8),
+    (105, 12000, 16, 16, 30.0, 16, 16, (0.0, 0.6), 0.2),
+    (106, 40000, 200, 120, 150.0, 8, 16, (0.01, 0.05), 0.6),
+]
+
+
+@pytest.mark.parametrize("case", RANDOM_CASES, ids=[f"seed{c[0]}" for c in RANDOM_CASES])
+def test_random_scenes_forward_backward(gpu, oracle, case):
+    # Odd image sizes, clusters of hundreds of points on single pixels (long per-pixel lists across several batches,
+    # early termination), opacities at exactly 0 and 1, points on tile borders: forward and backward against the oracle.
+    seed, n, width, height, focal, tile, channels, (lo, hi), cluster = case
+    rng = np.random.default_rng(seed)
+    hv = synthetic.camera_on_z(width, height, focal, 2.4)
+    pos = synthetic.cube_points(n, 1.4, seed)
+    n_cluster = int(n * cluster)
+    if n_cluster:
+        spots = rng.uniform(-0.5, 0.5, (7, 3)).astype(np.float32)
+        pos[:n_cluster] = spots[rng.integers(0, 7, n_cluster)] + rng.normal(0, 2e-3, (n_cluster, 3)).astype(np.float32)
+    feats, _ = synthetic.point_attributes(n, channels, "normal", seed + 1)
+    opac = rng.uniform(lo, hi, n).astype(np.float32)
+    opac[::97] = 0.0
+    if hi >= 1.0:
+        opac[5::89] = 1.0
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 2e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
+    H.assert_close(gf, gf_ref, RTOL, 2e-7, "feature gradients")
+    H.assert_close(go, go_ref, RTOL, 2e-6, "opacity gradients")
