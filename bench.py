@@ -198,6 +198,27 @@ def main() -> int:
     fwd_ms = time_calls(forward, args.steps)
     bwd_ms = time_calls(backward, args.steps)
 
+    # the same step replayed from a graph (the library only enqueues kernels, so a caller may capture it):
+    # what is left of the step when the host's launch work is taken away
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            s = _lib.current_stream()
+            _lib.check(lib.inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
+                                               _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image), _lib.ptr(alpha),
+                                               _lib.ptr(blending_weights), None, _lib.ptr(workspace), layout.total_bytes,
+                                               s), "inpc_raster_forward")
+            _lib.check(lib.inpc_raster_backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha), _lib.ptr(image),
+                                                _lib.ptr(alpha), _lib.ptr(positions), _lib.ptr(cam_position),
+                                                _lib.ptr(grad_features), _lib.ptr(grad_opacities), None,
+                                                _lib.ptr(workspace), layout.total_bytes, s), "inpc_raster_backward")
+        graph.replay()
+        graph_ms = time_calls(graph.replay, args.steps)
+    except Exception as exc:  # the figure is optional
+        print(f"bench.py: graph replay not measured: {exc}", file=sys.stderr)
+
     # the step that closes the loop: leaf statistics from this frame's leaf indices and blending weights
     from inpc_amd import update_probability_field
 
@@ -281,7 +302,7 @@ def main() -> int:
         "cpu_baseline": cpu,
         "extra": {
             "forward_ms": round(fwd_ms, 4), "backward_ms": round(bwd_ms, 4),
-            "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
+            "graph_replay_ms": None if graph_ms is None else round(graph_ms, 4), "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
             "field_update_ms": round(field_ms, 4),
             "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
             "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),

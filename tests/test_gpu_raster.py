@@ -4,6 +4,8 @@ Bit-exact: tile bounds, screen coordinates, depth keys, depth order, instance or
 Within 1e-4 relative (plus a small absolute floor for near-zero values): image, alpha, depth image,
 blending weights, feature and opacity gradients.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -344,3 +346,60 @@ def test_random_scenes_forward_backward(gpu, oracle, case):
     gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
     H.assert_close(gf, gf_ref, RTOL, 2e-7, "feature gradients")
     H.assert_close(go, go_ref, RTOL, 2e-6, "opacity gradients")
+
+
+def test_forward_backward_replays_from_a_graph(gpu, oracle):
+    # The library enqueues kernels only (no allocation, no memset nodes, no host read-back in forward / backward),
+    # so a caller may capture a step into a graph. Replays with new inputs written in place must give what eager
+    # calls give; the replays are interleaved with eager work and synchronisations.
+    n, channels, tile = 30000, 8, 16
+    hv, pos, feats, opac = scene(n, channels, seed=77)
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32)
+    lib = _lib.lib()
+    gf = torch.empty((n, channels), dtype=torch.float32, device="cuda:0")
+    go = torch.empty((n,), dtype=torch.float32, device="cuda:0")
+    Hh, Ww = hv.camera.height, hv.camera.width
+    gi = torch.zeros((channels, Hh, Ww), dtype=torch.float32, device="cuda:0")
+    ga = torch.zeros((1, Hh, Ww), dtype=torch.float32, device="cuda:0")
+
+    def step():
+        s = _lib.current_stream()
+        _lib.check(lib.inpc_raster_forward(
+            C.byref(run.cfg), _lib.ptr(run.positions), _lib.ptr(run.features), _lib.ptr(run.opacities), _lib.ptr(run.w2c),
+            _lib.ptr(run.cam_position), _lib.ptr(run.image), _lib.ptr(run.alpha), _lib.ptr(run.bw), None,
+            _lib.ptr(run.ws), run.layout.total_bytes, s), "forward")
+        _lib.check(lib.inpc_raster_backward(
+            C.byref(run.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(run.image), _lib.ptr(run.alpha), _lib.ptr(run.positions),
+            _lib.ptr(run.cam_position), _lib.ptr(gf), _lib.ptr(go), None, _lib.ptr(run.ws), run.layout.total_bytes, s),
+            "backward")
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        step()   # warm-up outside the capture (function attributes, occupancy queries)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step()
+    rng = np.random.default_rng(78)
+    cfg = oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32)
+    for replay in range(3):
+        new_pos = synthetic.cube_points(n, 1.6, 200 + replay)
+        new_feats, new_opac = synthetic.point_attributes(n, channels, "normal", 300 + replay, np.float32)
+        new_gi = rng.normal(0, 1e-2, (channels, Hh, Ww)).astype(np.float32)
+        new_ga = rng.normal(0, 1e-2, (1, Hh, Ww)).astype(np.float32)
+        run.positions.copy_(H.dev(new_pos))
+        run.features.copy_(H.dev(new_feats))
+        run.opacities.copy_(H.dev(new_opac))
+        gi.copy_(H.dev(new_gi))
+        ga.copy_(H.dev(new_ga))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = oracle.raster_forward(cfg, new_pos, new_feats, new_opac, hv.w2c)
+        out = run.outputs()
+        H.assert_close(out["image"], ref["image"], RTOL, 1e-5, f"image, replay {replay}")
+        H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, f"blending weights, replay {replay}")
+        gf_ref, go_ref, _ = oracle.raster_backward(cfg, new_gi, new_ga, out["image"], out["alpha"], new_pos, new_feats,
+                                                   new_opac, hv.w2c)
+        H.assert_close(gf.cpu().numpy(), gf_ref, RTOL, 1e-7, f"feature gradients, replay {replay}")
+        H.assert_close(go.cpu().numpy(), go_ref, RTOL, 2e-7, f"opacity gradients, replay {replay}")
