@@ -82,10 +82,12 @@ void inpc_pcg32_advance(uint64_t rng[2], int64_t delta);
  * Replaces compute_viewpoint_weights_wrapper (B/sampling/src/sampling_api.cu:10-47) and
  * kernel compute_viewpoint_weights_cu (B/sampling/src/sampling_kernels.cu:9-64).
  * centers (L,3) f32, levels (L,) i32, weights (L,) f32, w2c (4,4) f32 row-major (rows 0..2
- * are read), out (L,) f32; all dev. */
+ * are read), out (L,) f32; all dev. boxes_out (L,4) f32 dev, 16-byte aligned, or NULL: receives
+ * {centre, initial_size / 2^level} per leaf, the form in which the sampling calls below take the
+ * octree (one 16-byte gather per sample instead of four). */
 int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* weights,
-                      const float* w2c, float* out, uint32_t n_leaves, const inpc_camera* cam,
-                      float initial_size, void* stream);
+                      const float* w2c, float* out, float* boxes_out, uint32_t n_leaves,
+                      const inpc_camera* cam, float initial_size, void* stream);
 
 /* Bytes of scratch the CDF / counting passes need for n_leaves leaves. */
 size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
@@ -111,11 +113,11 @@ int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t
  * Replaces create_samples (B/sampling/src/sampling.cu:188-209) and create_samples_cu
  * (B/sampling/src/sampling_kernels.cu:128-150). Sample i uses the generator `rng_dev`
  * advanced by 4*i draws; afterwards the device generator is advanced by 4*n_samples.
- * positions_out (n,3) f32; leaf_ids_out (n,) i32 or NULL. If *sum_dev <= 0 nothing is
- * written and the generator is left untouched. */
-int inpc_sample(const float* centers, const int32_t* levels, const float* cdf, const float* sum_dev,
-                float* positions_out, int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves,
-                float initial_size, uint64_t* rng_dev, void* stream);
+ * boxes (L,4) f32 as written by inpc_leaf_weights; positions_out (n,3) f32; leaf_ids_out (n,) i32
+ * or NULL. If *sum_dev <= 0 nothing is written and the generator is left untouched. */
+int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, float* positions_out,
+                int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves, uint64_t* rng_dev,
+                void* stream);
 
 /* Bytes of scratch for inpc_sample_cull_compact over up to n_candidates per round. */
 size_t inpc_cull_workspace_bytes(uint32_t n_candidates);
@@ -135,12 +137,11 @@ int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream);
  * The workspace records, once `capacity` entries exist, how many candidates were consumed
  * (index of the last accepted candidate + 1). The generator is NOT advanced here; see
  * inpc_cull_finish. */
-int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const float* cdf,
-                             const float* sum_dev, const float* w2c, float* positions_out,
-                             int32_t* leaf_ids_out, uint32_t capacity, uint32_t k0,
-                             uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam,
-                             float initial_size, const uint64_t* rng_dev, void* workspace,
-                             size_t workspace_bytes, void* stream);
+int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* sum_dev,
+                             const float* w2c, float* positions_out, int32_t* leaf_ids_out,
+                             uint32_t capacity, uint32_t k0, uint32_t n_candidates,
+                             uint32_t n_leaves, const inpc_camera* cam, const uint64_t* rng_dev,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /* Copy {accepted, consumed} of the current draw to host memory. Synchronises `stream`.
  * The one host read-back of a training draw; it stands where the reference reads the weight

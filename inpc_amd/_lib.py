@@ -82,14 +82,13 @@ SIGNATURES = {
     "inpc_pcg32_next_uint": (_U32, [_P]),
     "inpc_pcg32_next_float": (_F, [_P]),
     "inpc_pcg32_advance": (None, [_P, C.c_int64]),
-    "inpc_leaf_weights": (C.c_int, [_P, _P, _P, _P, _P, _U32, _CAM, _F, _P]),
+    "inpc_leaf_weights": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _CAM, _F, _P]),
     "inpc_sampler_workspace_bytes": (_SZ, [_U32]),
     "inpc_build_cdf": (C.c_int, [_P, _P, _P, _SZ, _U32, _P]),
-    "inpc_sample": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _U32, _F, _P, _P]),
+    "inpc_sample": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _P, _P]),
     "inpc_cull_workspace_bytes": (_SZ, [_U32]),
     "inpc_cull_begin": (C.c_int, [_P, _SZ, _P]),
-    "inpc_sample_cull_compact": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _CAM, _F, _P, _P,
-                                           _SZ, _P]),
+    "inpc_sample_cull_compact": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _CAM, _P, _P, _SZ, _P]),
     "inpc_cull_read_counts": (C.c_int, [_P, C.POINTER(_U32), C.POINTER(_U32), _P]),
     "inpc_cull_finish": (C.c_int, [_P, _P, _P, _U32, _U32, _P, _P, _SZ, _P]),
     "inpc_widen_ids": (C.c_int, [_P, _P, _U32, _P]),

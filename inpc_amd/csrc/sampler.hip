@@ -66,12 +66,15 @@ __global__ void __launch_bounds__(kBlock) k_leaf_weights(const float* __restrict
                                                          const int32_t* __restrict__ levels,
                                                          const float* __restrict__ weights,
                                                          const float* __restrict__ w2c, float* __restrict__ out,
-                                                         uint32_t n_leaves, Camera cam, float initial_size) {
+                                                         float4* __restrict__ boxes, uint32_t n_leaves, Camera cam,
+                                                         float initial_size) {
     const uint32_t l = blockIdx.x * kBlock + threadIdx.x;
     if (l >= n_leaves) return;
     const Rows m = load_rows(w2c);
     const float cx = centers[3 * (size_t)l], cy = centers[3 * (size_t)l + 1], cz = centers[3 * (size_t)l + 2];
     const int level = levels[l];
+    // centre and edge length in one 16-byte word: the sampling kernels fetch it with one gather instead of four
+    if (boxes) boxes[l] = make_float4(cx, cy, cz, ldexpf(1.0f, -level) * initial_size);
     const float z = affine_row(m.r3, cx, cy, cz);
     bool valid = leaf_point_visible(m, cx, cy, cz, cam);
     if (!valid) {
@@ -223,19 +226,19 @@ struct Candidate {
     float x, y, z;
 };
 
-// `r` stands at draw 4*k; leaves it at 4*k + 4.
-__device__ __forceinline__ Candidate draw_candidate(Pcg32& r, const float* __restrict__ centers,
-                                                    const int32_t* __restrict__ levels,
+// `r` stands at draw 4*k; leaves it at 4*k + 4. boxes[leaf] = {centre, edge length} (B/sampling/src/
+// sampling_kernels.cu:141-147: centre + (u - 0.5) * initial_size / 2^level).
+__device__ __forceinline__ Candidate draw_candidate(Pcg32& r, const float4* __restrict__ boxes,
                                                     const float* __restrict__ cdf, const float* s_tree,
-                                                    uint32_t n_leaves, float initial_size) {
+                                                    uint32_t n_leaves) {
     const float u = pcg_float(r);
     const float ox = pcg_float(r), oy = pcg_float(r), oz = pcg_float(r);
     Candidate c;
     c.leaf = cdf_search(s_tree, cdf, u, n_leaves);
-    const float scale = ldexpf(1.0f, -levels[c.leaf]) * initial_size;
-    c.x = centers[3 * (size_t)c.leaf] + (ox - 0.5f) * scale;
-    c.y = centers[3 * (size_t)c.leaf + 1] + (oy - 0.5f) * scale;
-    c.z = centers[3 * (size_t)c.leaf + 2] + (oz - 0.5f) * scale;
+    const float4 box = boxes[c.leaf];
+    c.x = box.x + (ox - 0.5f) * box.w;
+    c.y = box.y + (oy - 0.5f) * box.w;
+    c.z = box.z + (oz - 0.5f) * box.w;
     return c;
 }
 
@@ -247,11 +250,9 @@ __device__ __forceinline__ Pcg32 thread_generator(const uint64_t* rng_dev, uint6
     return r;
 }
 
-__global__ void __launch_bounds__(kBlock) k_sample(const float* __restrict__ centers,
-                                                   const int32_t* __restrict__ levels,
-                                                   const float* __restrict__ cdf, const float* __restrict__ sum_dev,
-                                                   float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
-                                                   uint32_t n_samples, uint32_t n_leaves, float initial_size,
+__global__ void __launch_bounds__(kBlock) k_sample(const float4* __restrict__ boxes, const float* __restrict__ cdf,
+                                                   const float* __restrict__ sum_dev, float* __restrict__ positions,
+                                                   int32_t* __restrict__ leaf_ids, uint32_t n_samples, uint32_t n_leaves,
                                                    const uint64_t* __restrict__ rng_dev) {
     __shared__ __align__(16) float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
@@ -262,7 +263,7 @@ __global__ void __launch_bounds__(kBlock) k_sample(const float* __restrict__ cen
     for (int j = 0; j < kSampleItems; ++j) {
         const uint64_t k = tile_first + (uint64_t)j * kBlock + threadIdx.x;
         if (k < n_samples) {
-            const Candidate c = draw_candidate(r, centers, levels, cdf, s_tree, n_leaves, initial_size);
+            const Candidate c = draw_candidate(r, boxes, cdf, s_tree, n_leaves);
             positions[3 * k] = c.x;
             positions[3 * k + 1] = c.y;
             positions[3 * k + 2] = c.z;
@@ -290,10 +291,9 @@ struct CullState {
 constexpr size_t kCullHeaderWords = sizeof(CullState) / 4;
 
 __global__ void __launch_bounds__(kBlock)
-    k_sample_cull(const float* __restrict__ centers, const int32_t* __restrict__ levels,
-                  const float* __restrict__ cdf, const float* __restrict__ sum_dev, const float* __restrict__ w2c,
-                  float* __restrict__ positions, int32_t* __restrict__ leaf_ids, uint32_t capacity, uint32_t k0,
-                  uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam, float initial_size,
+    k_sample_cull(const float4* __restrict__ boxes, const float* __restrict__ cdf, const float* __restrict__ sum_dev,
+                  const float* __restrict__ w2c, float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
+                  uint32_t capacity, uint32_t k0, uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam,
                   const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
     __shared__ uint32_t s_accepted0, s_exclusive, s_done;
     __shared__ uint32_t s_count[kSampleItems * (kBlock / kWave)];
@@ -335,7 +335,7 @@ __global__ void __launch_bounds__(kBlock)
             const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
             keep[j] = false;
             if (rel < n_candidates) {
-                cand[j] = draw_candidate(r, centers, levels, cdf, s_tree, n_leaves, initial_size);
+                cand[j] = draw_candidate(r, boxes, cdf, s_tree, n_leaves);
                 keep[j] = sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
                 r.state = pcg_apply(step, r.state);
             }
@@ -577,13 +577,16 @@ using namespace inpc;
 extern "C" {
 
 int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* weights, const float* w2c,
-                      float* out, uint32_t n_leaves, const inpc_camera* cam, float initial_size, void* stream) {
+                      float* out, float* boxes_out, uint32_t n_leaves, const inpc_camera* cam, float initial_size,
+                      void* stream) {
     if (!cam) return fail(INPC_E_INVALID_ARGUMENT, "inpc_leaf_weights: camera is null");
     if (n_leaves == 0) return INPC_OK;
     if (!centers || !levels || !weights || !w2c || !out)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_leaf_weights: null pointer");
+    if (((uintptr_t)boxes_out & 15u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_leaf_weights: boxes_out must be 16-byte aligned");
     INPC_LAUNCH("leaf_weights", k_leaf_weights, dim3(div_up(n_leaves, kBlock)), dim3(kBlock), (hipStream_t)stream,
-                centers, levels, weights, w2c, out, n_leaves, to_device_camera(*cam), initial_size);
+                centers, levels, weights, w2c, out, (float4*)boxes_out, n_leaves, to_device_camera(*cam), initial_size);
     return INPC_OK;
 }
 
@@ -626,16 +629,16 @@ int inpc_build_cdf(float* w, float* sum_out, void* workspace, size_t workspace_b
     return INPC_OK;
 }
 
-int inpc_sample(const float* centers, const int32_t* levels, const float* cdf, const float* sum_dev,
-                float* positions_out, int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves,
-                float initial_size, uint64_t* rng_dev, void* stream_) {
+int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, float* positions_out,
+                int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves, uint64_t* rng_dev, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (n_samples == 0) return INPC_OK;
     if (n_samples >= (1u << 30)) return fail(INPC_E_UNSUPPORTED, "inpc_sample: n_samples must be below 2^30");
-    if (n_leaves == 0 || !centers || !levels || !cdf || !sum_dev || !positions_out || !rng_dev)
+    if (n_leaves == 0 || !boxes || !cdf || !sum_dev || !positions_out || !rng_dev)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: null pointer or no leaves");
-    INPC_LAUNCH("sample", k_sample, dim3(div_up(n_samples, kSampleTile)), dim3(kBlock), stream, centers, levels, cdf,
-                sum_dev, positions_out, leaf_ids_out, n_samples, n_leaves, initial_size, (const uint64_t*)rng_dev);
+    if (((uintptr_t)boxes & 15u) != 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: boxes must be 16-byte aligned");
+    INPC_LAUNCH("sample", k_sample, dim3(div_up(n_samples, kSampleTile)), dim3(kBlock), stream, (const float4*)boxes, cdf,
+                sum_dev, positions_out, leaf_ids_out, n_samples, n_leaves, (const uint64_t*)rng_dev);
     INPC_LAUNCH("rng_advance", k_rng_advance, dim3(1), dim3(64), stream, rng_dev, sum_dev, 4ull * n_samples);
     return INPC_OK;
 }
@@ -650,16 +653,17 @@ int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream) {
     return fill_u32(workspace, 0u, kCullHeaderWords, (hipStream_t)stream);
 }
 
-int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const float* cdf, const float* sum_dev,
-                             const float* w2c, float* positions_out, int32_t* leaf_ids_out, uint32_t capacity,
-                             uint32_t k0, uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam,
-                             float initial_size, const uint64_t* rng_dev, void* workspace, size_t workspace_bytes,
-                             void* stream_) {
+int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* sum_dev, const float* w2c,
+                             float* positions_out, int32_t* leaf_ids_out, uint32_t capacity, uint32_t k0,
+                             uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam, const uint64_t* rng_dev,
+                             void* workspace, size_t workspace_bytes, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (n_candidates == 0) return INPC_OK;
-    if (!cam || n_leaves == 0 || !centers || !levels || !cdf || !sum_dev || !w2c || !positions_out || !leaf_ids_out ||
-        !rng_dev || !workspace)
+    if (!cam || n_leaves == 0 || !boxes || !cdf || !sum_dev || !w2c || !positions_out || !leaf_ids_out || !rng_dev ||
+        !workspace)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample_cull_compact: null pointer or no leaves");
+    if (((uintptr_t)boxes & 15u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample_cull_compact: boxes must be 16-byte aligned");
     if ((uint64_t)k0 + n_candidates >= (1ull << 30))
         return fail(INPC_E_UNSUPPORTED, "inpc_sample_cull_compact: candidate index must stay below 2^30");
     if (workspace_bytes < inpc_cull_workspace_bytes(n_candidates))
@@ -674,9 +678,9 @@ int inpc_sample_cull_compact(const float* centers, const int32_t* levels, const 
     uint32_t resident = 0;
     const int rc = resident_blocks((const void*)k_sample_cull, kBlock, resident);
     if (rc != INPC_OK) return rc;
-    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(std::min(n_blocks, resident)), dim3(kBlock), stream, centers, levels, cdf,
-                sum_dev, w2c, positions_out, leaf_ids_out, capacity, k0, n_candidates, n_blocks, n_leaves,
-                to_device_camera(*cam), initial_size, rng_dev, st, status);
+    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(std::min(n_blocks, resident)), dim3(kBlock), stream,
+                (const float4*)boxes, cdf, sum_dev, w2c, positions_out, leaf_ids_out, capacity, k0, n_candidates, n_blocks,
+                n_leaves, to_device_camera(*cam), rng_dev, st, status);
     return INPC_OK;
 }
 

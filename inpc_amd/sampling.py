@@ -53,7 +53,7 @@ def compute_viewpoint_weights(centers: torch.Tensor, levels: torch.Tensor, weigh
     out = torch.empty(n, dtype=torch.float32, device=centers.device)
     cam = _lib.make_camera(view.camera)
     _lib.check(_lib.lib().inpc_leaf_weights(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(w2c),
-                                            _lib.ptr(out), n, C.byref(cam), float(initial_size),
+                                            _lib.ptr(out), None, n, C.byref(cam), float(initial_size),
                                             _lib.current_stream()), "inpc_leaf_weights")
     return out
 
@@ -96,21 +96,22 @@ class ProbabilityFieldSampler(torch.nn.Module):
         stream = _lib.current_stream()
         cam = _lib.make_camera(view.camera)
         vw = torch.empty(max(n, 1), dtype=torch.float32, device=centers.device)
+        boxes = torch.empty((max(n, 1), 4), dtype=torch.float32, device=centers.device)  # centre, edge length
         _lib.check(lib.inpc_leaf_weights(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(w2c),
-                                         _lib.ptr(vw), n, C.byref(cam), float(initial_size), stream),
+                                         _lib.ptr(vw), _lib.ptr(boxes), n, C.byref(cam), float(initial_size), stream),
                    "inpc_leaf_weights")
         ws_bytes = int(lib.inpc_sampler_workspace_bytes(max(n, 1)))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=centers.device)
         total = torch.zeros(_lib.CDF_HEAD_FLOATS, dtype=torch.float32, device=centers.device)  # CDF head; [0] = total
-        return vw, ws, ws_bytes, total, cam, stream
+        return vw, boxes, ws, ws_bytes, total, cam, stream
 
     def _cdf(self, centers, levels, weights, w2c, view, initial_size):
-        vw, ws, ws_bytes, total, cam, stream = self._weights(centers, levels, weights, w2c, view, initial_size)
+        vw, boxes, ws, ws_bytes, total, cam, stream = self._weights(centers, levels, weights, w2c, view, initial_size)
         n = centers.shape[0]
         if n > 0:
             _lib.check(_lib.lib().inpc_build_cdf(_lib.ptr(vw), _lib.ptr(total), _lib.ptr(ws), ws_bytes, n, stream),
                        "inpc_build_cdf")
-        return vw, total, cam, stream
+        return vw, boxes, total, cam, stream
 
     # -- API ---------------------------------------------------------------------------------------------
     def generate_training_samples(self, centers, levels, weights, view, n_samples: int,
@@ -132,7 +133,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
             positions.zero_()
             ids64.fill_(-1)
             return positions, ids64
-        cdf, total, cam, stream = self._cdf(centers, levels, weights, w2c, view, initial_size)
+        cdf, boxes, total, cam, stream = self._cdf(centers, levels, weights, w2c, view, initial_size)
         rng = self._rng_dev(device)
         first = min(int(n_samples / max(self._acceptance, 1e-3) * self.OVERSAMPLE) + 4096, (1 << 30) - 1)
         cull_bytes = int(lib.inpc_cull_workspace_bytes(first))
@@ -141,11 +142,10 @@ class ProbabilityFieldSampler(torch.nn.Module):
         k0, accepted, consumed = 0, C.c_uint32(0), C.c_uint32(0)
         n_round = first
         while True:
-            _lib.check(lib.inpc_sample_cull_compact(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(cdf),
-                                                    _lib.ptr(total), _lib.ptr(w2c), _lib.ptr(positions),
-                                                    _lib.ptr(ids32), n_samples, k0, n_round, n_leaves, C.byref(cam),
-                                                    float(initial_size), _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes,
-                                                    stream), "inpc_sample_cull_compact")
+            _lib.check(lib.inpc_sample_cull_compact(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(w2c),
+                                                    _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0, n_round,
+                                                    n_leaves, C.byref(cam), _lib.ptr(rng), _lib.ptr(cull_ws),
+                                                    cull_bytes, stream), "inpc_sample_cull_compact")
             k0 += n_round
             _lib.check(lib.inpc_cull_read_counts(_lib.ptr(cull_ws), C.byref(accepted), C.byref(consumed), stream),
                        "inpc_cull_read_counts")
@@ -179,14 +179,13 @@ class ProbabilityFieldSampler(torch.nn.Module):
         n_leaves = centers.shape[0]
         if n_leaves == 0:
             return torch.empty((0, 3), dtype=torch.float32, device=device)
-        cdf, total, cam, stream = self._cdf(centers, levels, weights, w2c, view, initial_size)
+        cdf, boxes, total, cam, stream = self._cdf(centers, levels, weights, w2c, view, initial_size)
         if not float(total[0].item()) > 0.0:  # the reference reads the sum back here as well
             return torch.empty((0, 3), dtype=torch.float32, device=device)
         n_samples = int(n_samples)
         positions = torch.empty((n_samples, 3), dtype=torch.float32, device=device)
-        _lib.check(_lib.lib().inpc_sample(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(cdf), _lib.ptr(total),
-                                          _lib.ptr(positions), None, n_samples, n_leaves, float(initial_size),
-                                          _lib.ptr(self._rng_dev(device)), stream), "inpc_sample")
+        _lib.check(_lib.lib().inpc_sample(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(positions), None,
+                                          n_samples, n_leaves, _lib.ptr(self._rng_dev(device)), stream), "inpc_sample")
         return positions
 
     def generate_expected_samples(self, centers, levels, weights, view, n_samples: int, n_multi: int,
@@ -200,7 +199,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
         n_leaves = centers.shape[0]
         if n_leaves == 0:
             return torch.empty((0, 3), dtype=torch.float32, device=device)
-        vw, ws, ws_bytes, total, cam, stream = self._weights(centers, levels, weights, w2c, view, initial_size)
+        vw, _, ws, ws_bytes, total, cam, stream = self._weights(centers, levels, weights, w2c, view, initial_size)
         offsets = torch.empty(n_leaves, dtype=torch.int32, device=device)
         _lib.check(lib.inpc_expected_counts(_lib.ptr(vw), _lib.ptr(total), _lib.ptr(offsets), int(n_samples),
                                             _lib.ptr(ws), ws_bytes, n_leaves, stream), "inpc_expected_counts")

@@ -42,8 +42,28 @@ def leaf_weights(oct, hv, device="cuda:0"):
     # keep the uploads alive until the launch is queued: a temporary's memory is recycled at once
     centers, levels, weights, w2c = dev(oct.centers), dev(oct.levels), dev(oct.weights), dev(hv.w2c)
     _lib.check(lib.inpc_leaf_weights(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(w2c),
-                                     _lib.ptr(out), n, C.byref(cam), oct.initial_size, stream()), "inpc_leaf_weights")
+                                     _lib.ptr(out), None, n, C.byref(cam), oct.initial_size, stream()),
+               "inpc_leaf_weights")
     return out
+
+
+def leaf_boxes(oct, hv=None, device="cuda:0"):
+    """(L, 4) device tensor {centre, edge length} as inpc_leaf_weights writes it for the sampling calls
+    (the camera does not enter it)."""
+    from inpc_amd import synthetic
+
+    if hv is None:
+        hv = synthetic.camera_on_z(8, 8, 8.0, 1.0)
+    lib = _lib.lib()
+    n = len(oct.levels)
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    boxes = torch.full((n, 4), float("nan"), dtype=torch.float32, device=device)
+    cam = cam_struct(hv.camera)
+    centers, levels, weights, w2c = dev(oct.centers), dev(oct.levels), dev(oct.weights), dev(hv.w2c)
+    _lib.check(lib.inpc_leaf_weights(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(weights), _lib.ptr(w2c),
+                                     _lib.ptr(out), _lib.ptr(boxes), n, C.byref(cam), oct.initial_size, stream()),
+               "inpc_leaf_weights")
+    return boxes
 
 
 def build_cdf(w_dev):
@@ -63,10 +83,9 @@ def sample(oct, cdf, total, n_samples, rng_dev):
     device = cdf.device
     pos = torch.full((n_samples, 3), float("nan"), dtype=torch.float32, device=device)
     ids = torch.full((n_samples,), -7, dtype=torch.int32, device=device)
-    centers, levels = dev(oct.centers), dev(oct.levels)
-    _lib.check(lib.inpc_sample(_lib.ptr(centers), _lib.ptr(levels), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(pos),
-                               _lib.ptr(ids), n_samples, len(oct.levels), oct.initial_size, _lib.ptr(rng_dev),
-                               stream()), "inpc_sample")
+    boxes = leaf_boxes(oct)
+    _lib.check(lib.inpc_sample(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(pos), _lib.ptr(ids), n_samples,
+                               len(oct.levels), _lib.ptr(rng_dev), stream()), "inpc_sample")
     return pos.cpu().numpy(), ids.cpu().numpy()
 
 
@@ -78,7 +97,7 @@ class CullDraw:
         self.oct, self.hv, self.cdf, self.total, self.rng = oct, hv, cdf, total, rng_dev
         self.capacity = capacity
         device = cdf.device
-        self.centers, self.levels, self.w2c = dev(oct.centers), dev(oct.levels), dev(hv.w2c)
+        self.boxes, self.w2c = leaf_boxes(oct, hv), dev(hv.w2c)
         self.pos = torch.full((capacity, 3), float("nan"), dtype=torch.float32, device=device)
         self.ids = torch.full((capacity,), -7, dtype=torch.int32, device=device)
         self.ws_bytes = int(self.lib.inpc_cull_workspace_bytes(max_round))
@@ -89,9 +108,9 @@ class CullDraw:
 
     def round(self, n_candidates):
         _lib.check(self.lib.inpc_sample_cull_compact(
-            _lib.ptr(self.centers), _lib.ptr(self.levels), _lib.ptr(self.cdf), _lib.ptr(self.total), _lib.ptr(self.w2c),
-            _lib.ptr(self.pos), _lib.ptr(self.ids), self.capacity, self.k0, n_candidates, len(self.oct.levels),
-            C.byref(self.cam), self.oct.initial_size, _lib.ptr(self.rng), _lib.ptr(self.ws), self.ws_bytes, stream()),
+            _lib.ptr(self.boxes), _lib.ptr(self.cdf), _lib.ptr(self.total), _lib.ptr(self.w2c), _lib.ptr(self.pos),
+            _lib.ptr(self.ids), self.capacity, self.k0, n_candidates, len(self.oct.levels), C.byref(self.cam),
+            _lib.ptr(self.rng), _lib.ptr(self.ws), self.ws_bytes, stream()),
             "inpc_sample_cull_compact")
         self.k0 += n_candidates
         return self.counts()
