@@ -29,19 +29,16 @@ __device__ __forceinline__ float ordered_value(uint32_t k) {
 constexpr uint32_t kNoMax = 0u;           // below the key of every float
 constexpr uint32_t kNoMin = 0xFFFFFFFFu;  // above the key of every float
 
-__global__ void __launch_bounds__(kBlock) k_field_reset(uint32_t* __restrict__ max_key, uint32_t* __restrict__ min_key,
-                                                        uint32_t n_leaves) {
+// keys[leaf] = {key of the maximum, key of the minimum}: one 8-byte word, so that the look before the atomics is
+// one gather (a divergent load costs the same whatever its width).
+__global__ void __launch_bounds__(kBlock) k_field_reset(uint2* __restrict__ keys, uint32_t n_leaves) {
     const uint32_t stride = gridDim.x * kBlock;
-    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_leaves; i += stride) {
-        max_key[i] = kNoMax;
-        min_key[i] = kNoMin;
-    }
+    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_leaves; i += stride) keys[i] = make_uint2(kNoMax, kNoMin);
 }
 
 __global__ void __launch_bounds__(kBlock) k_field_scatter(const int64_t* __restrict__ indices,
                                                           const float* __restrict__ weights, uint32_t n_samples,
-                                                          uint32_t* max_key, uint32_t* min_key, uint32_t n_leaves,
-                                                          uint32_t* error_flag) {
+                                                          uint2* keys, uint32_t n_leaves, uint32_t* error_flag) {
     const uint32_t stride = gridDim.x * kBlock;
     for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_samples; i += stride) {
         const int64_t leaf = indices[i];
@@ -50,20 +47,22 @@ __global__ void __launch_bounds__(kBlock) k_field_scatter(const int64_t* __restr
             continue;
         }
         const uint32_t key = ordered_key(weights[i]);
-        // most samples of a leaf do not change its extrema: look before paying for the atomic
-        if (key > __hip_atomic_load(&max_key[leaf], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&max_key[leaf], key);
-        if (key < __hip_atomic_load(&min_key[leaf], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMin(&min_key[leaf], key);
+        // most samples of a leaf do not change its extrema: look before paying for the atomics. The look may see
+        // an older value of either half; the atomics decide.
+        unsigned long long* word = (unsigned long long*)(keys + leaf);
+        const unsigned long long seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (key > (uint32_t)seen) atomicMax(&keys[leaf].x, key);
+        if (key < (uint32_t)(seen >> 32)) atomicMin(&keys[leaf].y, key);
     }
 }
 
-__global__ void __launch_bounds__(kBlock) k_field_finish(const uint32_t* __restrict__ max_key,
-                                                         const uint32_t* __restrict__ min_key, float* __restrict__ leaf_weights,
+__global__ void __launch_bounds__(kBlock) k_field_finish(const uint2* __restrict__ keys, float* __restrict__ leaf_weights,
                                                          float* __restrict__ leaf_scores, uint32_t n_leaves, float decay) {
     const uint32_t stride = gridDim.x * kBlock;
     for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n_leaves; i += stride) {
-        const uint32_t kmax = max_key[i], kmin = min_key[i];
-        const float max_sampled = kmax == kNoMax ? 0.0f : ordered_value(kmax);
-        const float min_sampled = kmin == kNoMin ? 0.0f : ordered_value(kmin);
+        const uint2 k = keys[i];
+        const float max_sampled = k.x == kNoMax ? 0.0f : ordered_value(k.x);
+        const float min_sampled = k.y == kNoMin ? 0.0f : ordered_value(k.y);
         leaf_weights[i] = fmaxf(leaf_weights[i] * decay, max_sampled);
         leaf_scores[i] = fmaxf(leaf_scores[i] * decay, fminf(fmaxf(max_sampled - min_sampled, 0.0f), 1.0f));
     }
@@ -362,20 +361,18 @@ int inpc_field_update(const int64_t* indices, const float* weights, uint32_t n_s
     if (n_samples > 0 && (!indices || !weights)) return fail(INPC_E_INVALID_ARGUMENT, "field_update: null samples");
     if (!workspace || workspace_bytes < inpc_field_update_workspace_bytes(n_leaves))
         return fail(INPC_E_WORKSPACE, "field_update: workspace too small");
-    if (((uintptr_t)workspace & 3u) != 0) return fail(INPC_E_WORKSPACE, "field_update: workspace must be 4-byte aligned");
+    if (((uintptr_t)workspace & 7u) != 0) return fail(INPC_E_WORKSPACE, "field_update: workspace must be 8-byte aligned");
     uint32_t* error_flag = (uint32_t*)workspace;
-    uint32_t* max_key = (uint32_t*)workspace + 64;
-    uint32_t* min_key = max_key + n_leaves;
+    uint2* keys = (uint2*)((uint32_t*)workspace + 64);
     int rc = fill_u32(error_flag, 0u, 1, stream);
     if (rc != INPC_OK) return rc;
     const uint32_t leaf_blocks = std::min<uint32_t>(div_up(n_leaves, kBlock), 4096u);
-    INPC_LAUNCH("field_reset", k_field_reset, dim3(leaf_blocks), dim3(kBlock), stream, max_key, min_key, n_leaves);
-    if (n_samples > 0) {
+    INPC_LAUNCH("field_reset", k_field_reset, dim3(leaf_blocks), dim3(kBlock), stream, keys, n_leaves);
+    if (n_samples > 0)
         INPC_LAUNCH("field_scatter", k_field_scatter, dim3(std::min<uint32_t>(div_up(n_samples, kBlock), 8192u)),
-                    dim3(kBlock), stream, indices, weights, n_samples, max_key, min_key, n_leaves, error_flag);
-    }
-    INPC_LAUNCH("field_finish", k_field_finish, dim3(leaf_blocks), dim3(kBlock), stream, (const uint32_t*)max_key,
-                (const uint32_t*)min_key, leaf_weights, leaf_scores, n_leaves, decay);
+                    dim3(kBlock), stream, indices, weights, n_samples, keys, n_leaves, error_flag);
+    INPC_LAUNCH("field_finish", k_field_finish, dim3(leaf_blocks), dim3(kBlock), stream, (const uint2*)keys, leaf_weights,
+                leaf_scores, n_leaves, decay);
     return INPC_OK;
 }
 
