@@ -271,6 +271,96 @@ int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* workspa
                               uint32_t counters_host[3], void* stream);
 
 /* =========================================================================================
+ * Rasterizer, Gaussian footprint (RasterizerMode.GAUSSIAN of
+ * B/torch_bindings/rasterization.py:15-18; B/rasterization/src/gaussian/)
+ * ======================================================================================= */
+
+/* A point is drawn as a screen-space Gaussian: covariance from an isotropic world-space variance
+ * through the Jacobian of the projection plus a dilation of 0.16, cut where it falls below a
+ * threshold (B/rasterization/src/gaussian/kernels.cu:57-91, include/gaussian/config.h:19).
+ *   training (base.flags without INPC_RASTER_INFERENCE): variance (0.3 * 0.5)^2 / (fx * fy),
+ *     3-sigma tile bounds, threshold 0.01110899653 (kernels.cu:57-60,80-81,452); sigma_world and
+ *     sigma_cutoff are ignored;
+ *   inference: variance sigma_world^2, or scales[i]^2 when a scales array is passed; tile bounds
+ *     sigma_cutoff * sigma - 0.5, threshold exp(-sigma_cutoff^2 / 2)
+ *     (kernels.cu:166,186-187,268-273; inference.cu:170-171).
+ * A point touches any number of tiles, so the instance buffers have a capacity the caller
+ * chooses: max_instances (0: 4 * n_points + 65536). */
+typedef struct inpc_gaussian_config {
+    inpc_raster_config base;
+    float sigma_world;
+    float sigma_cutoff;
+    uint32_t max_instances;
+    uint32_t reserved;
+} inpc_gaussian_config;
+
+/* Offsets (bytes from the workspace base) of the buffers a caller may want to inspect. */
+typedef struct inpc_gaussian_layout {
+    size_t total_bytes;
+    size_t counters;         /* u32[16]: [0] n_visible, [1] n_instances, [2] error flag,
+                                [4] instances drawn (n_instances, or 0 when they do not fit)   */
+    size_t point_touched;    /* (N) u32: tiles a point touches, 0 when it is not drawn          */
+    size_t point_bounds;     /* (N) 4 x u16: x_min, x_max, y_min, y_max in tiles, half open     */
+    size_t point_record;     /* (N) records of record_stride bytes, in point order:
+                                float sx, sy, opacity, conic.x, conic.y, conic.z, depth,
+                                u32 (point id | bit 31: touches more than one tile); then the
+                                view features as fp32                                           */
+    size_t depth_order;      /* (N) u32 point ids in (depth, point id) order, n_visible valid   */
+    size_t depth_keys;       /* (N) u32 matching depth keys                                     */
+    size_t instance_keys;    /* (max_instances) u16 tile id per instance in final order         */
+    size_t instance_points;  /* (max_instances) u32 point id per instance in final order        */
+    size_t tile_ranges;      /* (n_tiles) {u32 begin, end}                                      */
+    uint32_t record_stride;
+    uint32_t grid_width;
+    uint32_t grid_height;
+    uint32_t n_tiles;
+    uint32_t end_bit;
+    uint32_t depth_key_bias;
+    uint32_t max_instances;  /* the capacity in effect                                          */
+    uint32_t reserved;
+} inpc_gaussian_layout;
+
+/* Workspace size and layout. Replaces the growable blobs of
+ * B/rasterization/include/gaussian/buffer_utils.h:24-117 with one caller-owned buffer. */
+int inpc_gaussian_layout_query(const inpc_gaussian_config* cfg, inpc_gaussian_layout* out);
+
+/* Forward pass with the Gaussian footprint. Replaces the gaussian branches of forward_wrapper /
+ * inference_wrapper / inference_preextracted_wrapper
+ * (B/rasterization/src/rasterization_api.cu:79-100,248-269,336-360), gaussian::forward /
+ * inference / inference_preextracted (B/rasterization/src/gaussian/forward.cu:12-172,
+ * inference.cu:12-175, inference_preextracted.cu:11-177) and the kernels of
+ * B/rasterization/src/gaussian/kernels.cu:11-324,346-474,581-660.
+ *   Arguments as for inpc_raster_forward; scales (N,) f32 or NULL (inference only).
+ *   blending_weights receive sum over pixels of G * blending weight (kernels.cu:456).
+ * When the points touch more tiles than max_instances, counter [1] exceeds the capacity, no
+ * instance is drawn (the images show the background) and inpc_gaussian_read_counters reports
+ * it. No host synchronisation. */
+int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* positions,
+                          const void* features, const float* opacities, const float* scales,
+                          const float* w2c, const float* cam_position, float* image, float* alpha,
+                          float* blending_weights, float* depth_image, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* Backward pass of the Gaussian footprint. Replaces the gaussian branch of backward_wrapper
+ * (B/rasterization/src/rasterization_api.cu:165-184), gaussian::backward
+ * (B/rasterization/src/gaussian/backward.cu:9-68), blend_backward_cu and preprocess_backward_cu
+ * (B/rasterization/src/gaussian/kernels.cu:326-344,476-579). Arguments as for
+ * inpc_raster_backward. Gradients of points that touch several tiles are summed with float
+ * atomics, so their last bits depend on scheduling, as in the reference. */
+int inpc_gaussian_backward(const inpc_gaussian_config* cfg, const float* grad_image,
+                           const float* grad_alpha, const float* image, const float* alpha,
+                           const float* positions, const float* cam_position, void* grad_features,
+                           float* grad_opacities, float* grad_view_scratch, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* Copy {n_visible, n_instances, error flag, instances drawn} to the host; synchronises `stream`.
+ * Returns INPC_E_DEVICE if the error flag is set and INPC_E_WORKSPACE if n_instances exceeds
+ * max_instances (the images of that call are incomplete: call again with a larger capacity; the
+ * reference reads the count back and resizes, B/rasterization/src/gaussian/forward.cu:87-90,118-119). */
+int inpc_gaussian_read_counters(const inpc_gaussian_config* cfg, const void* workspace,
+                                uint32_t counters_host[4], void* stream);
+
+/* =========================================================================================
  * Probability-field statistics (the consumer of the sampler's leaf indices and the
  * rasterizer's blending weights, once per training iteration)
  * ======================================================================================= */

@@ -64,6 +64,39 @@ class RasterLayout(C.Structure):
     ]
 
 
+class GaussianConfig(C.Structure):
+    _fields_ = [
+        ("base", RasterConfig),
+        ("sigma_world", C.c_float),
+        ("sigma_cutoff", C.c_float),
+        ("max_instances", C.c_uint32),
+        ("reserved", C.c_uint32),
+    ]
+
+
+class GaussianLayout(C.Structure):
+    _fields_ = [
+        ("total_bytes", C.c_size_t),
+        ("counters", C.c_size_t),
+        ("point_touched", C.c_size_t),
+        ("point_bounds", C.c_size_t),
+        ("point_record", C.c_size_t),
+        ("depth_order", C.c_size_t),
+        ("depth_keys", C.c_size_t),
+        ("instance_keys", C.c_size_t),
+        ("instance_points", C.c_size_t),
+        ("tile_ranges", C.c_size_t),
+        ("record_stride", C.c_uint32),
+        ("grid_width", C.c_uint32),
+        ("grid_height", C.c_uint32),
+        ("n_tiles", C.c_uint32),
+        ("end_bit", C.c_uint32),
+        ("depth_key_bias", C.c_uint32),
+        ("max_instances", C.c_uint32),
+        ("reserved", C.c_uint32),
+    ]
+
+
 class TimingRecord(C.Structure):
     _fields_ = [("name", C.c_char_p), ("ms", C.c_float)]
 
@@ -75,6 +108,7 @@ _F = C.c_float
 _SZ = C.c_size_t
 _CAM = C.POINTER(Camera)
 _CFG = C.POINTER(RasterConfig)
+_GCFG = C.POINTER(GaussianConfig)
 SIGNATURES = {
     "inpc_last_error": (C.c_char_p, []),
     "inpc_abi_version": (C.c_int, []),
@@ -98,6 +132,10 @@ SIGNATURES = {
     "inpc_raster_forward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "inpc_raster_backward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "inpc_raster_read_counters": (C.c_int, [_CFG, _P, C.POINTER(_U32 * 3), _P]),
+    "inpc_gaussian_layout_query": (C.c_int, [_GCFG, C.POINTER(GaussianLayout)]),
+    "inpc_gaussian_forward": (C.c_int, [_GCFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "inpc_gaussian_backward": (C.c_int, [_GCFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "inpc_gaussian_read_counters": (C.c_int, [_GCFG, _P, C.POINTER(_U32 * 4), _P]),
     "inpc_field_update_workspace_bytes": (_SZ, [_U32]),
     "inpc_field_update": (C.c_int, [_P, _P, _U32, _P, _P, _U32, _F, _P, _SZ, _P]),
     "inpc_field_update_check": (C.c_int, [_P, _P]),

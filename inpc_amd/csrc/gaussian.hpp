@@ -1,0 +1,562 @@
+// gaussian.hpp — the rasterizer's Gaussian footprint (RasterizerMode.GAUSSIAN; B/rasterization/src/gaussian/).
+// Included by raster.hip after blend.hpp; shares the projection, SH and sort helpers with the bilinear path.
+//
+// A point is drawn as a screen-space Gaussian and touches any number of tiles, so this path keeps the reference's
+// structure: per-point records in point order, depth sort, instances expanded in depth order, stable tile sort,
+// ranges, blend (B/rasterization/src/gaussian/forward.cu:12-172).
+//   k_preprocess        project, covariance -> conic, tile bounds, record, depth key and digit histograms
+//                       (kernels.cu:11-324)
+//   radix sort          by depth key, culled points dropped (forward.cu:92-100)
+//   k_touch_sums / k_touch_scan   exclusive prefix of the touched-tile counts in depth order (forward.cu:102-116)
+//   k_create_instances  every block expands 1024 depth-ordered points; the instances, not the points, are spread
+//                       over the threads, so a point that covers the screen costs no more per instance than one
+//                       that covers a tile (kernels.cu:358-380); tile-key histograms for the sort
+//   radix sort          by tile key, stable (forward.cu:133-141)
+//   k_ranges            [begin, end) per tile (kernels.cu:382-399)
+//   k_blend_*           one block per tile, one thread per pixel, a wave owns an 8 x 8 pixel block; per batch of
+//                       T*T staged instances a wave first finds, 64 instances at a time, the ones whose footprint
+//                       reaches its pixel block and evaluates only those (kernels.cu:401-660)
+#pragma once
+
+namespace gaussian {
+
+constexpr float kDilation = 0.16f;                  // gaussian/config.h:19
+constexpr float kTrainThreshold = 0.01110899653f;   // kernels.cu:452
+constexpr float kTrainCutoff = 3.0f;                // kernels.cu:80-81
+constexpr uint32_t kMultiTile = 1u << 31;           // record word: the point touches more than one tile
+constexpr uint32_t kPointMask = kMultiTile - 1u;
+constexpr int kCntKept = 4;                         // instances that are sorted and drawn (0 when they do not fit)
+constexpr int kCntInstances64 = 6;                  // u64 at words 6, 7: exact instance count
+constexpr int kPointsPerBlock = 1024;               // depth-ordered points per block of the instance kernels
+
+inline uint32_t record_stride(int channels) { return (uint32_t)align_up(32 + (size_t)channels * 4, 32); }
+
+// exp(x) for x <= 0 by one fixed sequence of fp32 operations (the reference calls expf / __expf, kernels.cu:451,
+// 548,634): n = rint(x log2 e), r = x - n ln 2 in two parts, a degree-7 polynomial (Cephes' expf coefficients),
+// scaling by 2^n. Within one ulp of exp on [-87, 0], 0 below; a CPU evaluates the same sequence to the same bits,
+// so the cut at the footprint's threshold falls on the same pixels.
+__device__ __forceinline__ float footprint_exp(float x) {
+    if (!(x >= -87.0f)) return 0.0f;
+    const float n = __builtin_rintf(x * 1.44269504088896341f);
+    const float r = (x - n * 0.693359375f) - n * -2.12194440e-4f;
+    float p = 1.9875691500e-4f;
+    p = p * r + 1.3981999507e-3f;
+    p = p * r + 8.3334519073e-3f;
+    p = p * r + 4.1665795894e-2f;
+    p = p * r + 1.6666665459e-1f;
+    p = p * r + 5.0000001201e-1f;
+    const float y = (p * (r * r) + r) + 1.0f;
+    return ldexpf(y, (int)n);
+}
+
+struct Params {
+    float variance;    // world-space variance of a point without a scale of its own
+    float cutoff;      // the tile bounds reach cutoff * sigma - 0.5 pixels
+    float threshold;   // smallest footprint value that is drawn
+    float reach2;      // -2 ln(threshold): |dx| <= sqrt(reach2 * cov_x) wherever the footprint passes the threshold
+    uint32_t capacity; // instances the buffers hold
+};
+
+// ---- preprocess (kernels.cu:11-324) -------------------------------------------------------------------------------
+template <int FMODE, int C>
+__global__ void __launch_bounds__(kBlock)
+    k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
+                 const float* __restrict__ opacities, const float* __restrict__ scales, const float* __restrict__ w2c,
+                 const float* __restrict__ cam_position, char* __restrict__ records, uint32_t* __restrict__ touched_out,
+                 uint2* __restrict__ bounds_out, uint32_t* __restrict__ keys, uint32_t* __restrict__ vals,
+                 float* __restrict__ blending_weights, uint32_t* counters, uint32_t* g_hist, Geometry g, Params prm,
+                 float tile_edge, radix::DevicePlan plan) {
+    __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
+    __shared__ uint32_t s_visible;
+    __shared__ unsigned long long s_instances;
+    for (int i = threadIdx.x; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
+    if (threadIdx.x == 0) {
+        s_visible = 0u;
+        s_instances = 0ull;
+    }
+    __syncthreads();
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t touched = 0u;
+    if (i < g.n) {
+        uint32_t key = radix::kInvalidKey;
+        const ViewRows m = load_view_rows(w2c);
+        const float px = positions[3 * (size_t)i], py = positions[3 * (size_t)i + 1], pz = positions[3 * (size_t)i + 2];
+        const float depth = affine_row(m.r3, px, py, pz);
+        if (!(depth < g.cam.near_plane || depth > g.cam.far_plane)) {
+            const float x = affine_row(m.r1, px, py, pz) / depth;
+            const float y = affine_row(m.r2, px, py, pz) / depth;
+            const float sx = x * g.cam.fx + g.cam.cx;
+            const float sy = y * g.cam.fy + g.cam.cy;
+            float variance = prm.variance;
+            if (scales) variance = scales[i] * scales[i];
+            const float j00 = g.cam.fx / depth;
+            const float j02 = -j00 * fmaxf(-1.3f * g.cam.cx / g.cam.fx, fminf(x, 1.3f * g.cam.cx / g.cam.fx));
+            const float j11 = g.cam.fy / depth;
+            const float j12 = -j11 * fmaxf(-1.3f * g.cam.cy / g.cam.fy, fminf(y, 1.3f * g.cam.cy / g.cam.fy));
+            float cov_x = variance * (j00 * j00 + j02 * j02);
+            const float cov_y = variance * (j02 * j12);
+            float cov_z = variance * (j11 * j11 + j12 * j12);
+            cov_x += kDilation;
+            cov_z += kDilation;
+            const float det = cov_x * cov_z - cov_y * cov_y;
+            if (det != 0.0f) {
+                const float rcp = 1.0f / det;
+                const float conic_x = cov_z * rcp, conic_y = -cov_y * rcp, conic_z = cov_x * rcp;
+                const float reach_x = prm.cutoff * sqrtf(cov_x) - 0.5f;
+                const float reach_y = prm.cutoff * sqrtf(cov_z) - 0.5f;
+                const float fgw = (float)g.gw, fgh = (float)g.gh;
+                const uint32_t x0 = (uint32_t)fminf(fgw, fmaxf(0.0f, floorf((sx - reach_x) / tile_edge)));
+                const uint32_t x1 = (uint32_t)fminf(fgw, fmaxf(0.0f, ceilf((sx + reach_x) / tile_edge)));
+                const uint32_t y0 = (uint32_t)fminf(fgh, fmaxf(0.0f, floorf((sy - reach_y) / tile_edge)));
+                const uint32_t y1 = (uint32_t)fminf(fgh, fmaxf(0.0f, ceilf((sy + reach_y) / tile_edge)));
+                if (x1 > x0 && y1 > y0) {
+                    touched = (x1 - x0) * (y1 - y0);
+                    bounds_out[i] = make_uint2(x0 | (x1 << 16), y0 | (y1 << 16));
+                    float opacity = FMODE == INPC_FEAT_RAW37_F16 ? 0.0f : opacities[i];
+                    float4* rec = (float4*)(records + (size_t)i * g.stride);
+                    if (FMODE == INPC_FEAT_DIRECT_F32) {
+                        const float4* src = (const float4*)features + (size_t)i * (C / 4);
+#pragma unroll
+                        for (int q = 0; q < C / 4; ++q) rec[2 + q] = src[q];
+                    } else if (FMODE == INPC_FEAT_DIRECT_F16) {
+                        const __half* src = (const __half*)features + (size_t)i * C;
+#pragma unroll
+                        for (int q = 0; q < C / 4; ++q)
+                            rec[2 + q] = make_float4(__half2float(src[4 * q]), __half2float(src[4 * q + 1]),
+                                                     __half2float(src[4 * q + 2]), __half2float(src[4 * q + 3]));
+                    } else {
+                        const ShBasis sb = sh_basis(px, py, pz, cam_position);
+                        if (FMODE == INPC_FEAT_SH36_F16) {
+                            rec[2] = sh_to_view(sb, (const __half*)features + 36 * (size_t)i);
+                        } else {
+                            const __half* raw = (const __half*)features + 37 * (size_t)i;
+                            rec[2] = sh_to_view(sb, raw + 1);
+                            opacity = 1.0f - expf(-expf(__half2float(raw[0])));  // kernels.cu:154
+                        }
+                    }
+                    rec[0] = make_float4(sx, sy, opacity, conic_x);
+                    rec[1] = make_float4(conic_y, conic_z, depth, __uint_as_float(i | (touched > 1u ? kMultiTile : 0u)));
+                    key = __float_as_uint(depth) - g.key_bias;
+                    radix::hist_add(s_hist, plan, key);
+                }
+            }
+        }
+        touched_out[i] = touched;
+        keys[i] = key;
+        vals[i] = i;
+        if (blending_weights) blending_weights[i] = 0.0f;
+    }
+    const uint32_t visible = (uint32_t)__popcll(__ballot(touched != 0u));
+    uint32_t sum = touched;
+    for (int s = 32; s > 0; s >>= 1) sum += __shfl_down(sum, s, 64);
+    if ((threadIdx.x & 63u) == 0u) {
+        if (visible) atomicAdd(&s_visible, visible);
+        if (sum) atomicAdd(&s_instances, (unsigned long long)sum);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (s_visible) atomicAdd(&counters[kCntVisible], s_visible);
+        if (s_instances) atomicAdd((unsigned long long*)(counters + kCntInstances64), s_instances);
+    }
+    radix::hist_flush(s_hist, plan, g_hist);
+}
+
+// ---- instance offsets: exclusive prefix of touched[order[j]] (kernels.cu:346-356, forward.cu:110-116) ------------
+__global__ void __launch_bounds__(kBlock)
+    k_touch_sums(const uint32_t* __restrict__ order, const uint32_t* __restrict__ touched,
+                 const uint32_t* __restrict__ counters, uint32_t* __restrict__ block_sums) {
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    const uint32_t n_visible = counters[kCntVisible];
+    const uint32_t base = blockIdx.x * kPointsPerBlock;
+    uint32_t sum = 0;
+    for (uint32_t k = threadIdx.x; k < (uint32_t)kPointsPerBlock; k += kBlock) {
+        const uint32_t j = base + k;
+        if (j < n_visible) sum += touched[order[j]];
+    }
+    for (int s = 32; s > 0; s >>= 1) sum += __shfl_down(sum, s, 64);
+    if ((threadIdx.x & 63u) == 0u) s_wave[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t total = 0;
+        for (int w = 0; w < kBlock / kWave; ++w) total += s_wave[w];
+        block_sums[blockIdx.x] = total;
+    }
+}
+
+// One block: block_sums -> exclusive prefix in place; decides whether the instances fit. When they do not, nothing
+// is expanded or drawn (the 32-bit offsets could not even address them) and the count tells the caller.
+__global__ void __launch_bounds__(kScanBlock) k_touch_scan(uint32_t* __restrict__ block_sums, uint32_t n_blocks,
+                                                           uint32_t* counters, uint32_t capacity) {
+    __shared__ uint32_t s_wave[kScanBlock / kWave];
+    __shared__ uint32_t s_fits;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    if (tid == 0) {
+        const unsigned long long total = *(const unsigned long long*)(counters + kCntInstances64);
+        const bool fits = total <= (unsigned long long)capacity;
+        s_fits = fits ? 1u : 0u;
+        counters[kCntKept] = fits ? (uint32_t)total : 0u;
+        counters[kCntInstances] = total > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)total;
+    }
+    __syncthreads();
+    if (!s_fits) return;
+    const uint32_t per = (n_blocks + kScanBlock - 1) / kScanBlock;
+    const uint32_t begin = min(tid * per, n_blocks), end = min(begin + per, n_blocks);
+    uint32_t mine = 0;
+    for (uint32_t b = begin; b < end; ++b) mine += block_sums[b];
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s, 64);
+        if (lane >= (uint32_t)s) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - mine;
+    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
+    for (uint32_t b = begin; b < end; ++b) {
+        const uint32_t c = block_sums[b];
+        block_sums[b] = run;
+        run += c;
+    }
+}
+
+// Instances of the block's 1024 depth-ordered points, in depth order, row-major over each point's tiles
+// (kernels.cu:358-380). Output slot s of the block belongs to the last point whose offset is <= s.
+__global__ void __launch_bounds__(kBlock)
+    k_create_instances(const uint32_t* __restrict__ order, const uint32_t* __restrict__ touched,
+                       const uint2* __restrict__ bounds, const uint32_t* __restrict__ block_base,
+                       const uint32_t* __restrict__ counters, uint16_t* __restrict__ inst_keys,
+                       uint32_t* __restrict__ inst_points, uint32_t* g_hist, uint32_t gw, radix::DevicePlan plan) {
+    constexpr int kPer = kPointsPerBlock / kBlock;   // consecutive points per thread
+    __shared__ uint32_t s_offset[kPointsPerBlock + 1];
+    __shared__ uint32_t s_point[kPointsPerBlock];
+    __shared__ uint2 s_bounds[kPointsPerBlock];
+    __shared__ uint32_t s_wave[kBlock / kWave];
+    __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
+    if (counters[kCntKept] == 0u) return;
+    const uint32_t n_visible = counters[kCntVisible];
+    const uint32_t base = blockIdx.x * kPointsPerBlock;
+    if (base >= n_visible) return;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    for (int i = tid; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
+    uint32_t count[kPer], mine = 0;
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        const uint32_t k = tid * kPer + u, j = base + k;
+        count[u] = 0u;
+        if (j < n_visible) {
+            const uint32_t p = order[j];
+            count[u] = touched[p];
+            s_point[k] = p;
+            s_bounds[k] = bounds[p];
+        }
+        mine += count[u];
+    }
+    uint32_t incl = mine;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s, 64);
+        if (lane >= (uint32_t)s) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - mine;
+    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        s_offset[tid * kPer + u] = run;
+        run += count[u];
+    }
+    if (tid == kBlock - 1) s_offset[kPointsPerBlock] = run;
+    __syncthreads();
+    const uint32_t total = s_offset[kPointsPerBlock];
+    const uint32_t out = block_base[blockIdx.x];
+    for (uint32_t s = tid; s < total; s += kBlock) {
+        uint32_t lo = 0, hi = kPointsPerBlock;   // last k with s_offset[k] <= s
+        while (hi - lo > 1u) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_offset[mid] <= s) lo = mid;
+            else hi = mid;
+        }
+        const uint2 b = s_bounds[lo];
+        const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
+        const uint32_t r = s - s_offset[lo];
+        const uint32_t tile = (y0 + r / nx) * gw + x0 + r % nx;
+        inst_keys[out + s] = (uint16_t)tile;
+        inst_points[out + s] = s_point[lo];
+        radix::hist_add(s_hist, plan, tile);
+    }
+    __syncthreads();
+    radix::hist_flush(s_hist, plan, g_hist);
+}
+
+// [begin, end) of every tile's instances (kernels.cu:382-399); tiles without instances keep (0, 0).
+__global__ void __launch_bounds__(kBlock) k_ranges(const uint16_t* __restrict__ inst_keys,
+                                                   const uint32_t* __restrict__ counters, uint2* __restrict__ ranges) {
+    const uint32_t n = counters[kCntKept];
+    const uint32_t stride = gridDim.x * kBlock;
+    for (uint32_t k = blockIdx.x * kBlock + threadIdx.x; k < n; k += stride) {
+        const uint32_t t = inst_keys[k];
+        if (k == 0u) {
+            ranges[t].x = 0u;
+        } else {
+            const uint32_t before = inst_keys[k - 1];
+            if (before != t) {
+                ranges[before].y = k;
+                ranges[t].x = k;
+            }
+        }
+        if (k == n - 1u) ranges[t].y = n;
+    }
+}
+
+// ---- blend -----------------------------------------------------------------------------------------------------------
+// A staged instance: header words, features, and the pixel box (tile-local, conservative) its footprint can reach.
+template <int T, int C>
+struct Stage {
+    static constexpr int TT = T * T;
+    float4 head0[TT];   // sx, sy, opacity, conic.x
+    float4 head1[TT];   // conic.y, conic.z, depth, point id | kMultiTile
+    float4 feat[TT * (C / 4)];
+    uint32_t box[TT];   // bytes: first column, one past the last column, first row, one past the last row
+};
+
+// Thread `slot` stages instance `slot` of the batch.
+template <int T, int C>
+__device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, const char* __restrict__ record,
+                                               int tile_x0, int tile_y0, float reach2) {
+    const float4* src = (const float4*)record;
+    const float4 h0 = src[0], h1 = src[1];
+    st.head0[slot] = h0;
+    st.head1[slot] = h1;
+#pragma unroll
+    for (int q = 0; q < C / 4; ++q) st.feat[slot * (C / 4) + q] = src[2 + q];
+    // cov = conic^-1; the footprint passes the threshold only where |dx| <= sqrt(reach2 * cov_x) (same in y).
+    // Taken a little wider; anything odd (non-positive determinant, non-finite values) selects the whole tile.
+    const float det = h0.w * h1.y - h1.x * h1.x;
+    float x_lo = 0.0f, x_hi = (float)T, y_lo = 0.0f, y_hi = (float)T;
+    if (det > 0.0f) {
+        const float rx = sqrtf(reach2 * (h1.y / det)) * 1.01f + 0.01f;
+        const float ry = sqrtf(reach2 * (h0.w / det)) * 1.01f + 0.01f;
+        if (rx < 1e6f && ry < 1e6f) {
+            x_lo = fminf(fmaxf(ceilf(h0.x - rx - 0.5f) - (float)tile_x0, 0.0f), (float)T);
+            x_hi = fminf(fmaxf(floorf(h0.x + rx - 0.5f) + 1.0f - (float)tile_x0, 0.0f), (float)T);
+            y_lo = fminf(fmaxf(ceilf(h0.y - ry - 0.5f) - (float)tile_y0, 0.0f), (float)T);
+            y_hi = fminf(fmaxf(floorf(h0.y + ry - 0.5f) + 1.0f - (float)tile_y0, 0.0f), (float)T);
+        }
+    }
+    st.box[slot] = (uint32_t)x_lo | ((uint32_t)x_hi << 8) | ((uint32_t)y_lo << 16) | ((uint32_t)y_hi << 24);
+}
+
+// Does the box reach the 8 x 8 pixel block at (qx0, qy0)?
+__device__ __forceinline__ bool box_reaches(uint32_t box, int qx0, int qy0) {
+    const int x_lo = box & 0xFF, x_hi = (box >> 8) & 0xFF, y_lo = (box >> 16) & 0xFF, y_hi = box >> 24;
+    return x_lo < qx0 + 8 && x_hi > qx0 && y_lo < qy0 + 8 && y_hi > qy0;
+}
+
+// Footprint value of a staged instance at the pixel centre (kernels.cu:447-452); false when the pixel is skipped.
+__device__ __forceinline__ bool footprint_value(const float4 h0, const float4 h1, float cx, float cy, float threshold,
+                                                float& G) {
+    const float dx = h0.x - cx, dy = h0.y - cy;
+    const float exponent = -0.5f * (h0.w * dx * dx + h1.y * dy * dy) - h1.x * dx * dy;
+    if (exponent > 0.0f) return false;
+    G = footprint_exp(exponent);
+    return !(G < threshold);
+}
+
+struct Pixel {
+    int x, y;       // image coordinates
+    int qx0, qy0;   // tile-local origin of the wave's pixel block
+    bool inside;
+};
+
+template <int T>
+__device__ __forceinline__ Pixel pixel_of_thread(uint32_t tile, uint32_t gw, int W, int H) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    Pixel p;
+    p.qx0 = T == 16 ? (int)(wave & 1u) * 8 : 0;
+    p.qy0 = T == 16 ? (int)(wave >> 1) * 8 : 0;
+    p.x = (int)(tile % gw) * T + p.qx0 + (int)(lane & 7u);
+    p.y = (int)(tile / gw) * T + p.qy0 + (int)(lane >> 3);
+    p.inside = p.x < W && p.y < H;
+    return p;
+}
+
+template <int T, int C, bool INFERENCE>
+__global__ void __launch_bounds__(T * T)
+    k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ order,
+                    const uint32_t* __restrict__ inst_points, const char* __restrict__ records, uint32_t stride,
+                    float* __restrict__ image, float* __restrict__ alpha_image, float* blending_weights,
+                    float* __restrict__ depth_image, int W, int H, uint32_t gw, float threshold, float reach2) {
+    constexpr int TT = T * T;
+    __shared__ Stage<T, C> st;
+    __shared__ float s_weight[TT];   // per staged instance: sum over the tile's pixels of G * blending weight
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t tile = order[blockIdx.x];
+    const Pixel px = pixel_of_thread<T>(tile, gw, W, H);
+    const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
+    const float cx = (float)px.x + 0.5f, cy = (float)px.y + 0.5f;
+    float acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) acc[c] = 0.0f;
+    float depth_acc = 0.0f, tr = 1.0f;
+    bool done = !px.inside;
+    const uint2 range = ranges[tile];
+    for (uint32_t base = range.x; base < range.y; base += TT) {
+        if (__syncthreads_count(done) == TT) break;
+        const uint32_t count = min((uint32_t)TT, range.y - base);
+        if (tid < count) {
+            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2);
+            if (!INFERENCE) s_weight[tid] = 0.0f;
+        }
+        __syncthreads();
+        if (__ballot(!done) != 0ull) {
+            for (uint32_t first = 0; first < count; first += 64u) {
+                const uint32_t mine = first + lane;
+                uint64_t todo = __ballot(mine < count && box_reaches(st.box[mine], px.qx0, px.qy0));
+                while (todo) {
+                    const uint32_t j = first + (uint32_t)__builtin_ctzll(todo);
+                    todo &= todo - 1ull;
+                    if (done) continue;
+                    const float4 h0 = st.head0[j], h1 = st.head1[j];
+                    float G;
+                    if (!footprint_value(h0, h1, cx, cy, threshold, G)) continue;
+                    const float a = h0.z * G;
+                    const float bw = tr * a;
+                    if (!INFERENCE && bw > 0.0f) atomicAdd(&s_weight[j], G * bw);
+#pragma unroll
+                    for (int q = 0; q < C / 4; ++q) {
+                        const float4 f = st.feat[j * (C / 4) + q];
+                        acc[4 * q] += bw * f.x;
+                        acc[4 * q + 1] += bw * f.y;
+                        acc[4 * q + 2] += bw * f.z;
+                        acc[4 * q + 3] += bw * f.w;
+                    }
+                    if (INFERENCE) depth_acc += bw * h1.z;
+                    tr *= 1.0f - a;
+                    if (tr < kTransmittanceThreshold) done = true;
+                }
+            }
+        }
+        if (!INFERENCE) {
+            __syncthreads();
+            if (tid < count) {
+                const float w = s_weight[tid];
+                if (w != 0.0f) {
+                    const uint32_t word = __float_as_uint(st.head1[tid].w);
+                    if (word & kMultiTile) atomicAdd(&blending_weights[word & kPointMask], w);
+                    else blending_weights[word] = w;   // the point's only instance
+                }
+            }
+        }
+    }
+    if (px.inside) {
+        const size_t n_pixels = (size_t)W * H, pix = (size_t)px.y * W + px.x;
+#pragma unroll
+        for (int c = 0; c < C; ++c) image[c * n_pixels + pix] = acc[c];
+        const float alpha_px = 1.0f - tr;
+        alpha_image[pix] = tr < kTransmittanceThreshold ? 1.0f : alpha_px;
+        if (INFERENCE) depth_image[pix] = alpha_px > 0.0f ? depth_acc / alpha_px : 0.0f;
+    }
+}
+
+// Backward: the same walk with the saved final image (kernels.cu:476-579). Per staged instance the tile's
+// contributions are summed in LDS and leave the block once: a plain store for a point with a single instance,
+// float atomics for the others.
+template <int T, int C>
+__global__ void __launch_bounds__(T * T)
+    k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ order,
+                     const uint32_t* __restrict__ inst_points, const char* __restrict__ records, uint32_t stride,
+                     const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
+                     const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_features,
+                     float* grad_opacities, int W, int H, uint32_t gw, float threshold, float reach2) {
+    constexpr int TT = T * T;
+    __shared__ Stage<T, C> st;
+    __shared__ float s_grad[TT][C + 1];   // per staged instance: feature gradient, opacity gradient
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t tile = order[blockIdx.x];
+    const Pixel px = pixel_of_thread<T>(tile, gw, W, H);
+    const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
+    const float cx = (float)px.x + 0.5f, cy = (float)px.y + 0.5f;
+    float g[C], final_px[C], fresh[C];
+    float common = 0.0f;
+#pragma unroll
+    for (int c = 0; c < C; ++c) g[c] = final_px[c] = fresh[c] = 0.0f;
+    if (px.inside) {
+        const size_t n_pixels = (size_t)W * H, pix = (size_t)px.y * W + px.x;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            g[c] = grad_image[c * n_pixels + pix];
+            final_px[c] = image[c * n_pixels + pix];
+        }
+        common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
+    }
+    float tr = 1.0f;
+    bool done = !px.inside;
+    const uint2 range = ranges[tile];
+    for (uint32_t base = range.x; base < range.y; base += TT) {
+        if (__syncthreads_count(done) == TT) break;
+        const uint32_t count = min((uint32_t)TT, range.y - base);
+        if (tid < count) {
+            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2);
+#pragma unroll
+            for (int c = 0; c <= C; ++c) s_grad[tid][c] = 0.0f;
+        }
+        __syncthreads();
+        if (__ballot(!done) != 0ull) {
+            for (uint32_t first = 0; first < count; first += 64u) {
+                const uint32_t mine = first + lane;
+                uint64_t todo = __ballot(mine < count && box_reaches(st.box[mine], px.qx0, px.qy0));
+                while (todo) {
+                    const uint32_t j = first + (uint32_t)__builtin_ctzll(todo);
+                    todo &= todo - 1ull;
+                    if (done) continue;
+                    const float4 h0 = st.head0[j], h1 = st.head1[j];
+                    float G;
+                    if (!footprint_value(h0, h1, cx, cy, threshold, G)) continue;
+                    const float a = h0.z * G;
+                    const float bw = tr * a;
+                    const float one_minus_a = 1.0f - a;
+                    const float rcp = 1.0f / fmaxf(one_minus_a, kOneMinusAlphaEps);
+                    float dot = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < C / 4; ++q) {
+                        const float4 f4 = st.feat[j * (C / 4) + q];
+                        const float f[4] = {f4.x, f4.y, f4.z, f4.w};
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int c = 4 * q + k;
+                            if (bw > 0.0f) atomicAdd(&s_grad[j][c], bw * g[c]);
+                            fresh[c] += bw * f[k];
+                            const float term = (tr * f[k] + (fresh[c] - final_px[c]) * rcp) * g[c];
+                            dot = c == 0 ? term : dot + term;
+                        }
+                    }
+                    const float d_alpha = dot + common * rcp;
+                    const float d_opacity = d_alpha * G;
+                    if (d_opacity != 0.0f) atomicAdd(&s_grad[j][C], d_opacity);
+                    tr *= one_minus_a;
+                    if (tr < kTransmittanceThreshold) done = true;
+                }
+            }
+        }
+        __syncthreads();
+        if (tid < count) {
+            const uint32_t word = __float_as_uint(st.head1[tid].w);
+            const uint32_t point = word & kPointMask;
+            float* gf = grad_features + (size_t)point * C;
+            if (word & kMultiTile) {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                    if (s_grad[tid][c] != 0.0f) atomicAdd(&gf[c], s_grad[tid][c]);
+                if (s_grad[tid][C] != 0.0f) atomicAdd(&grad_opacities[point], s_grad[tid][C]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < C; ++c) gf[c] = s_grad[tid][c];
+                grad_opacities[point] = s_grad[tid][C];
+            }
+        }
+    }
+}
+
+}  // namespace gaussian

@@ -609,6 +609,7 @@ __device__ unsigned long long g_blend_profile[8];
 #endif
 
 #include "blend.hpp"
+#include "gaussian.hpp"
 
 // view-space feature gradient -> (N,36) fp16; a point that was not drawn has a zero view gradient and
 // gets zeros (kernels.cu:95)
@@ -897,6 +898,218 @@ int dispatch_preprocess(const Layout& L, const float* positions, const void* fea
     return fail(INPC_E_UNSUPPORTED, "raster: unsupported preprocess configuration");
 }
 
+// ---- Gaussian footprint: workspace layout and launches --------------------------------------------------------
+struct GaussianLayout {
+    inpc_gaussian_layout pub;
+    Geometry geo;
+    gaussian::Params prm;
+    radix::PassPlan depth_plan, tile_plan;
+    int T, C, fmode;
+    bool inference, sh;
+    uint32_t n_blocks;  // blocks of gaussian::kPointsPerBlock depth-ordered points
+    size_t zero_begin, zero_words;
+    size_t hist_depth, hist_tile, status_depth, status_tile, bases_depth, bases_tile, tile_order, block_sums;
+    size_t keys_a, keys_b, vals_a, vals_b, inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
+};
+
+int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
+    if (!gcfg) return fail(INPC_E_INVALID_ARGUMENT, "gaussian: config is null");
+    const inpc_raster_config* cfg = &gcfg->base;
+    const inpc_camera& cam = cfg->cam;
+    if (cfg->tile != 8 && cfg->tile != 16) return fail(INPC_E_INVALID_ARGUMENT, "gaussian: tile must be 8 or 16");
+    if (cam.width <= 0 || cam.height <= 0) return fail(INPC_E_INVALID_ARGUMENT, "gaussian: empty image");
+    if (cfg->n_points >= (1u << 28)) return fail(INPC_E_UNSUPPORTED, "gaussian: n_points must be below 2^28");
+    L.T = cfg->tile;
+    L.fmode = cfg->feature_mode;
+    if (L.fmode < 0 || L.fmode > 3) return fail(INPC_E_UNSUPPORTED, "gaussian: unknown feature mode %d", L.fmode);
+    L.sh = L.fmode == INPC_FEAT_SH36_F16 || L.fmode == INPC_FEAT_RAW37_F16;
+    L.C = L.sh ? 4 : cfg->channels;
+    if (L.C != 4 && L.C != 8 && L.C != 16) return fail(INPC_E_INVALID_ARGUMENT, "gaussian: channels must be 4, 8 or 16");
+    L.inference = (cfg->flags & INPC_RASTER_INFERENCE) != 0;
+    if (L.fmode == INPC_FEAT_RAW37_F16 && !L.inference)
+        return fail(INPC_E_INVALID_ARGUMENT, "gaussian: raw (N,37) features are an inference input");
+    gaussian::Params& prm = L.prm;
+    if (L.inference) {
+        if (!(gcfg->sigma_cutoff > 0.0f) || !(gcfg->sigma_cutoff < 64.0f) || !(gcfg->sigma_world >= 0.0f) ||
+            !(gcfg->sigma_world < INFINITY))
+            return fail(INPC_E_INVALID_ARGUMENT, "gaussian: sigma_world must be >= 0 and sigma_cutoff in (0, 64)");
+        prm.variance = gcfg->sigma_world * gcfg->sigma_world;                // kernels.cu:166
+        prm.cutoff = gcfg->sigma_cutoff;                                     // kernels.cu:186-187
+        prm.threshold = expf(-0.5f * gcfg->sigma_cutoff * gcfg->sigma_cutoff);  // inference.cu:171
+    } else {
+        constexpr float numerator = 0.3f * 0.3f * 0.5f * 0.5f;               // kernels.cu:57-59
+        prm.variance = numerator / (cam.focal_x * cam.focal_y);
+        prm.cutoff = gaussian::kTrainCutoff;
+        prm.threshold = gaussian::kTrainThreshold;
+    }
+    prm.reach2 = -2.0f * logf(prm.threshold);
+    Geometry& g = L.geo;
+    g.n = cfg->n_points;
+    g.W = cam.width;
+    g.H = cam.height;
+    g.gw = (uint32_t)((cam.width + L.T - 1) / L.T);
+    g.gh = (uint32_t)((cam.height + L.T - 1) / L.T);
+    g.n_tiles = g.gw * g.gh;
+    if (g.n_tiles > 65536u)
+        return fail(INPC_E_UNSUPPORTED, "gaussian: %u tiles exceed the 16-bit tile key (65536)", g.n_tiles);
+    g.cam = to_device_camera(cam);
+    g.stride = gaussian::record_stride(L.C);
+    int depth_bits = 32;
+    g.key_bias = 0u;
+    if (cam.near_plane > 0.0f && cam.far_plane >= cam.near_plane && cam.far_plane < INFINITY) {
+        g.key_bias = float_bits(cam.near_plane);
+        depth_bits = std::max(1, bit_length(float_bits(cam.far_plane) - g.key_bias));
+    }
+    L.depth_plan = radix::make_plan(depth_bits);
+    const int end_bit = bit_length(g.n_tiles - 1);
+    L.tile_plan = radix::make_plan(std::max(end_bit, 1));
+    const size_t n = std::max<size_t>(g.n, 1);
+    uint64_t capacity = gcfg->max_instances ? gcfg->max_instances : 4ull * g.n + 65536ull;
+    if (capacity >= (1ull << 31)) return fail(INPC_E_UNSUPPORTED, "gaussian: max_instances must be below 2^31");
+    prm.capacity = (uint32_t)capacity;
+    L.n_blocks = div_up((uint32_t)n, gaussian::kPointsPerBlock);
+
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t o = off;
+        off += align_up(bytes, 256);
+        return o;
+    };
+    inpc_gaussian_layout& P = L.pub;
+    memset(&P, 0, sizeof(P));
+    L.zero_begin = off;
+    P.counters = take(kCntWords * 4);
+    L.hist_depth = take(radix::kMaxPasses * radix::kRadix * 4);
+    L.hist_tile = take(radix::kMaxPasses * radix::kRadix * 4);
+    L.status_depth = take(L.depth_plan.n_passes * radix::status_words(g.n) * 4);
+    L.status_tile = take(L.tile_plan.n_passes * radix::status_words(prm.capacity) * 4);
+    P.tile_ranges = take((size_t)g.n_tiles * 8);
+    L.zero_words = (off - L.zero_begin) / 4;
+    L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
+    L.bases_tile = take(radix::kMaxPasses * radix::kRadix * 4);
+    L.tile_order = take((size_t)g.n_tiles * 4);
+    L.block_sums = take((size_t)L.n_blocks * 4);
+    P.point_touched = take(n * 4);
+    P.point_bounds = take(n * 8);
+    P.point_record = take(n * g.stride);
+    L.keys_a = take(n * 4);
+    L.keys_b = take(n * 4);
+    L.vals_a = take(n * 4);
+    L.vals_b = take(n * 4);
+    L.inst_keys_a = take(capacity * 2);
+    L.inst_keys_b = take(capacity * 2);
+    L.inst_vals_a = take(capacity * 4);
+    L.inst_vals_b = take(capacity * 4);
+    const bool depth_in_a = (L.depth_plan.n_passes % 2) == 0, tile_in_a = (L.tile_plan.n_passes % 2) == 0;
+    P.depth_keys = depth_in_a ? L.keys_a : L.keys_b;
+    P.depth_order = depth_in_a ? L.vals_a : L.vals_b;
+    P.instance_keys = tile_in_a ? L.inst_keys_a : L.inst_keys_b;
+    P.instance_points = tile_in_a ? L.inst_vals_a : L.inst_vals_b;
+    P.total_bytes = off;
+    P.record_stride = g.stride;
+    P.grid_width = g.gw;
+    P.grid_height = g.gh;
+    P.n_tiles = g.n_tiles;
+    P.end_bit = (uint32_t)end_bit;
+    P.depth_key_bias = g.key_bias;
+    P.max_instances = prm.capacity;
+    return INPC_OK;
+}
+
+template <int FMODE, int C>
+int launch_gaussian_preprocess(const GaussianLayout& L, const float* positions, const void* features,
+                               const float* opacities, const float* scales, const float* w2c, const float* cam_position,
+                               float* blending_weights, void* ws, hipStream_t stream) {
+    INPC_LAUNCH("gaussian_preprocess", (gaussian::k_preprocess<FMODE, C>), dim3(div_up(L.geo.n, kBlock)), dim3(kBlock),
+                stream, positions, features, opacities, scales, w2c, cam_position, at<char>(ws, L.pub.point_record),
+                at<uint32_t>(ws, L.pub.point_touched), at<uint2>(ws, L.pub.point_bounds), at<uint32_t>(ws, L.keys_a),
+                at<uint32_t>(ws, L.vals_a), blending_weights, at<uint32_t>(ws, L.pub.counters),
+                at<uint32_t>(ws, L.hist_depth), L.geo, L.prm, (float)L.T, radix::to_device_plan(L.depth_plan));
+    return INPC_OK;
+}
+
+int dispatch_gaussian_preprocess(const GaussianLayout& L, const float* positions, const void* features,
+                                 const float* opacities, const float* scales, const float* w2c,
+                                 const float* cam_position, float* bw, void* ws, hipStream_t stream) {
+#define CALL_GPRE(FM_, C_) \
+    launch_gaussian_preprocess<FM_, C_>(L, positions, features, opacities, scales, w2c, cam_position, bw, ws, stream)
+    switch (L.fmode) {
+        case INPC_FEAT_SH36_F16: return CALL_GPRE(INPC_FEAT_SH36_F16, 4);
+        case INPC_FEAT_RAW37_F16: return CALL_GPRE(INPC_FEAT_RAW37_F16, 4);
+        case INPC_FEAT_DIRECT_F32:
+            if (L.C == 4) return CALL_GPRE(INPC_FEAT_DIRECT_F32, 4);
+            if (L.C == 8) return CALL_GPRE(INPC_FEAT_DIRECT_F32, 8);
+            if (L.C == 16) return CALL_GPRE(INPC_FEAT_DIRECT_F32, 16);
+            break;
+        case INPC_FEAT_DIRECT_F16:
+            if (L.C == 4) return CALL_GPRE(INPC_FEAT_DIRECT_F16, 4);
+            if (L.C == 8) return CALL_GPRE(INPC_FEAT_DIRECT_F16, 8);
+            if (L.C == 16) return CALL_GPRE(INPC_FEAT_DIRECT_F16, 16);
+            break;
+    }
+#undef CALL_GPRE
+    return fail(INPC_E_UNSUPPORTED, "gaussian: unsupported preprocess configuration");
+}
+
+template <int T, int C>
+int launch_gaussian_blend_forward(const GaussianLayout& L, float* image, float* alpha, float* blending_weights,
+                                  float* depth_image, void* ws, hipStream_t stream) {
+    const uint2* ranges = at<uint2>(ws, L.pub.tile_ranges);
+    const uint32_t* order = at<uint32_t>(ws, L.tile_order);
+    const uint32_t* inst = at<uint32_t>(ws, L.pub.instance_points);
+    const char* records = at<char>(ws, L.pub.point_record);
+    if (L.inference) {
+        INPC_LAUNCH("gaussian_blend_inference", (gaussian::k_blend_forward<T, C, true>), dim3(L.geo.n_tiles), dim3(T * T),
+                    stream, ranges, order, inst, records, L.geo.stride, image, alpha, (float*)nullptr, depth_image,
+                    L.geo.W, L.geo.H, L.geo.gw, L.prm.threshold, L.prm.reach2);
+    } else {
+        INPC_LAUNCH("gaussian_blend_forward", (gaussian::k_blend_forward<T, C, false>), dim3(L.geo.n_tiles), dim3(T * T),
+                    stream, ranges, order, inst, records, L.geo.stride, image, alpha, blending_weights, (float*)nullptr,
+                    L.geo.W, L.geo.H, L.geo.gw, L.prm.threshold, L.prm.reach2);
+    }
+    return INPC_OK;
+}
+
+template <int T, int C>
+int launch_gaussian_blend_backward(const GaussianLayout& L, const float* grad_image, const float* grad_alpha,
+                                   const float* image, const float* alpha, float* grad_view, float* grad_opacities,
+                                   void* ws, hipStream_t stream) {
+    INPC_LAUNCH("gaussian_blend_backward", (gaussian::k_blend_backward<T, C>), dim3(L.geo.n_tiles), dim3(T * T), stream,
+                at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
+                (const uint32_t*)at<uint32_t>(ws, L.pub.instance_points), (const char*)at<char>(ws, L.pub.point_record),
+                L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, L.geo.W, L.geo.H, L.geo.gw,
+                L.prm.threshold, L.prm.reach2);
+    return INPC_OK;
+}
+
+#define INPC_DISPATCH_TC(CALL)                       \
+    do {                                             \
+        if (L.T == 8 && L.C == 4) return CALL(8, 4);    \
+        if (L.T == 8 && L.C == 8) return CALL(8, 8);    \
+        if (L.T == 8 && L.C == 16) return CALL(8, 16);  \
+        if (L.T == 16 && L.C == 4) return CALL(16, 4);  \
+        if (L.T == 16 && L.C == 8) return CALL(16, 8);  \
+        if (L.T == 16 && L.C == 16) return CALL(16, 16); \
+    } while (0)
+
+int dispatch_gaussian_blend_forward(const GaussianLayout& L, float* image, float* alpha, float* bw, float* depth_image,
+                                    void* ws, hipStream_t stream) {
+#define CALL_GFWD(T_, C_) launch_gaussian_blend_forward<T_, C_>(L, image, alpha, bw, depth_image, ws, stream)
+    INPC_DISPATCH_TC(CALL_GFWD);
+#undef CALL_GFWD
+    return fail(INPC_E_UNSUPPORTED, "gaussian: unsupported blend configuration");
+}
+
+int dispatch_gaussian_blend_backward(const GaussianLayout& L, const float* grad_image, const float* grad_alpha,
+                                     const float* image, const float* alpha, float* grad_view, float* grad_opacities,
+                                     void* ws, hipStream_t stream) {
+#define CALL_GBWD(T_, C_) \
+    launch_gaussian_blend_backward<T_, C_>(L, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, ws, stream)
+    INPC_DISPATCH_TC(CALL_GBWD);
+#undef CALL_GBWD
+    return fail(INPC_E_UNSUPPORTED, "gaussian: unsupported backward configuration");
+}
+
 }  // namespace
 }  // namespace inpc
 
@@ -1059,6 +1272,138 @@ int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* ws, uin
     INPC_HIP_CHECK(hipStreamSynchronize(stream));
     if (counters_host) memcpy(counters_host, host, sizeof(host));
     if (host[2]) return fail(INPC_E_DEVICE, "rasterizer look-back gave up waiting (device error flag set)");
+    return INPC_OK;
+}
+
+int inpc_gaussian_layout_query(const inpc_gaussian_config* cfg, inpc_gaussian_layout* out) {
+    GaussianLayout L;
+    const int rc = make_gaussian_layout(cfg, L);
+    if (rc != INPC_OK) return rc;
+    if (out) *out = L.pub;
+    return INPC_OK;
+}
+
+int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* positions, const void* features,
+                          const float* opacities, const float* scales, const float* w2c, const float* cam_position,
+                          float* image, float* alpha, float* blending_weights, float* depth_image, void* ws,
+                          size_t ws_bytes, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    GaussianLayout L;
+    int rc = make_gaussian_layout(cfg, L);
+    if (rc != INPC_OK) return rc;
+    if (!ws || ws_bytes < L.pub.total_bytes)
+        return fail(INPC_E_WORKSPACE, "inpc_gaussian_forward: workspace has %zu bytes, needs %zu", ws_bytes,
+                    L.pub.total_bytes);
+    if (((uintptr_t)ws & 255u) != 0)
+        return fail(INPC_E_WORKSPACE, "inpc_gaussian_forward: workspace must be 256-byte aligned");
+    if (!w2c || !image || !alpha) return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: null pointer");
+    if (L.geo.n > 0 && (!positions || !features)) return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: null input");
+    if (L.fmode != INPC_FEAT_RAW37_F16 && L.geo.n > 0 && !opacities)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: opacities are null");
+    if (L.sh && !cam_position) return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: cam_position is null");
+    if (L.inference && !depth_image) return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: depth image is null");
+    if (!L.inference && L.geo.n > 0 && !blending_weights)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: blending weights are null");
+    if (!L.inference && scales)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: per-point scales are an inference input");
+    if (L.fmode == INPC_FEAT_DIRECT_F32 && ((uintptr_t)features & 15u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: fp32 features must be 16-byte aligned");
+
+    rc = fill_u32(at<uint32_t>(ws, L.zero_begin), 0u, L.zero_words, stream);
+    if (rc != INPC_OK) return rc;
+    uint32_t* counters = at<uint32_t>(ws, L.pub.counters);
+    if (L.geo.n > 0) {
+        rc = dispatch_gaussian_preprocess(L, positions, features, opacities, scales, w2c, cam_position,
+                                          L.inference ? nullptr : blending_weights, ws, stream);
+        if (rc != INPC_OK) return rc;
+        rc = radix::sort_pairs<uint32_t>(L.depth_plan, radix::kSkipInvalid, at<uint32_t>(ws, L.keys_a),
+                                         at<uint32_t>(ws, L.vals_a), at<uint32_t>(ws, L.keys_b),
+                                         at<uint32_t>(ws, L.vals_b), counters + kCntVisible, L.geo.n,
+                                         at<uint32_t>(ws, L.hist_depth), at<uint32_t>(ws, L.bases_depth),
+                                         at<uint32_t>(ws, L.status_depth), counters + kCntError, stream,
+                                         "gaussian_depth_sort");
+        if (rc != INPC_OK) return rc;
+        const uint32_t* order = at<uint32_t>(ws, L.pub.depth_order);
+        const uint32_t* touched = at<uint32_t>(ws, L.pub.point_touched);
+        INPC_LAUNCH("gaussian_touch_sums", gaussian::k_touch_sums, dim3(L.n_blocks), dim3(kBlock), stream, order, touched,
+                    (const uint32_t*)counters, at<uint32_t>(ws, L.block_sums));
+        INPC_LAUNCH("gaussian_touch_scan", gaussian::k_touch_scan, dim3(1), dim3(kScanBlock), stream,
+                    at<uint32_t>(ws, L.block_sums), L.n_blocks, counters, L.prm.capacity);
+        INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(L.n_blocks), dim3(kBlock), stream,
+                    order, touched, (const uint2*)at<uint2>(ws, L.pub.point_bounds),
+                    (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,
+                    at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), at<uint32_t>(ws, L.hist_tile),
+                    L.geo.gw, radix::to_device_plan(L.tile_plan));
+        rc = radix::sort_pairs<uint16_t>(L.tile_plan, radix::kPlain, at<uint16_t>(ws, L.inst_keys_a),
+                                         at<uint32_t>(ws, L.inst_vals_a), at<uint16_t>(ws, L.inst_keys_b),
+                                         at<uint32_t>(ws, L.inst_vals_b), counters + gaussian::kCntKept, L.prm.capacity,
+                                         at<uint32_t>(ws, L.hist_tile), at<uint32_t>(ws, L.bases_tile),
+                                         at<uint32_t>(ws, L.status_tile), counters + kCntError, stream,
+                                         "gaussian_tile_sort");
+        if (rc != INPC_OK) return rc;
+        INPC_LAUNCH("gaussian_ranges", gaussian::k_ranges, dim3(std::min(div_up(L.prm.capacity, kBlock), 4096u)),
+                    dim3(kBlock), stream, (const uint16_t*)at<uint16_t>(ws, L.pub.instance_keys),
+                    (const uint32_t*)counters, at<uint2>(ws, L.pub.tile_ranges));
+    }
+    INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
+                (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
+    return dispatch_gaussian_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
+}
+
+int inpc_gaussian_backward(const inpc_gaussian_config* cfg, const float* grad_image, const float* grad_alpha,
+                           const float* image, const float* alpha, const float* positions, const float* cam_position,
+                           void* grad_features, float* grad_opacities, float* grad_view_scratch, void* ws,
+                           size_t ws_bytes, void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    GaussianLayout L;
+    int rc = make_gaussian_layout(cfg, L);
+    if (rc != INPC_OK) return rc;
+    if (L.inference) return fail(INPC_E_UNSUPPORTED, "inpc_gaussian_backward: inference configurations have no backward pass");
+    if (!ws || ws_bytes < L.pub.total_bytes) return fail(INPC_E_WORKSPACE, "inpc_gaussian_backward: workspace too small");
+    if (L.geo.n == 0) return INPC_OK;
+    if (!grad_image || !grad_alpha || !image || !alpha || !grad_features || !grad_opacities)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: null pointer");
+    const bool direct32 = L.fmode == INPC_FEAT_DIRECT_F32;
+    float* grad_view = direct32 ? (float*)grad_features : grad_view_scratch;
+    if (!grad_view) return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: this feature mode needs grad_view_scratch");
+    if (L.sh && (!cam_position || !positions))
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: positions / cam_position are null");
+    rc = fill_u32(grad_view, 0u, (size_t)L.geo.n * L.C, stream);
+    if (rc != INPC_OK) return rc;
+    rc = fill_u32(grad_opacities, 0u, L.geo.n, stream);
+    if (rc != INPC_OK) return rc;
+    rc = dispatch_gaussian_blend_backward(L, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, ws, stream);
+    if (rc != INPC_OK) return rc;
+    if (L.fmode == INPC_FEAT_SH36_F16) {
+        INPC_LAUNCH("raster_sh_backward", k_sh_backward, dim3(div_up(L.geo.n, kBlock)), dim3(kBlock), stream, positions,
+                    cam_position, (const float4*)grad_view, (__half*)grad_features, L.geo.n);
+    } else if (L.fmode == INPC_FEAT_DIRECT_F16) {
+        const size_t total = (size_t)L.geo.n * L.C;
+        INPC_LAUNCH("raster_grad_to_half", k_float_to_half, dim3((uint32_t)std::min<size_t>((total + 255) / 256, 8192)),
+                    dim3(kBlock), stream, (const float*)grad_view, (__half*)grad_features, total);
+    }
+    return INPC_OK;
+}
+
+int inpc_gaussian_read_counters(const inpc_gaussian_config* cfg, const void* ws, uint32_t counters_host[4],
+                                void* stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    GaussianLayout L;
+    const int rc = make_gaussian_layout(cfg, L);
+    if (rc != INPC_OK) return rc;
+    uint32_t host[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    INPC_HIP_CHECK(hipMemcpyAsync(host, (const char*)ws + L.pub.counters, sizeof(host), hipMemcpyDeviceToHost, stream));
+    INPC_HIP_CHECK(hipStreamSynchronize(stream));
+    if (counters_host) {
+        counters_host[0] = host[kCntVisible];
+        counters_host[1] = host[kCntInstances];
+        counters_host[2] = host[kCntError];
+        counters_host[3] = host[gaussian::kCntKept];
+    }
+    if (host[kCntError]) return fail(INPC_E_DEVICE, "rasterizer look-back gave up waiting (device error flag set)");
+    if (host[kCntInstances] > L.prm.capacity)
+        return fail(INPC_E_WORKSPACE, "gaussian: %u instances do not fit max_instances = %u; nothing was drawn",
+                    host[kCntInstances], L.prm.capacity);
     return INPC_OK;
 }
 

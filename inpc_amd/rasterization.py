@@ -4,6 +4,11 @@ Same names, arguments and error behaviour as B/torch_bindings/rasterization.py:1
 side is libinpc_hip.so instead of the pybind11 module `_C`. On top of the reference's fixed shape
 (8x8 tiles, (N,36) fp16 SH features -> 4 channels) the constructor accepts the tile size, and
 `rasterize_points` exposes the direct-feature variants (C in {4, 8, 16}, fp32 or fp16 storage).
+
+Both footprints of the reference are there: BILINEAR (2x2 splat) and GAUSSIAN (screen-space Gaussian,
+B/rasterization/src/gaussian/). A Gaussian point touches any number of tiles, so that mode reads the
+instance count back after the forward pass, as the reference does, and repeats the pass with larger
+buffers in the rare case that they were too small.
 """
 from __future__ import annotations
 
@@ -52,12 +57,14 @@ _FEATURE_MODES = {"sh36": _lib.FEAT_SH36_F16, "f32": _lib.FEAT_DIRECT_F32, "f16"
                   "raw37": _lib.FEAT_RAW37_F16}
 
 
-def _require_bilinear(settings: RasterizerSettings) -> None:
-    if settings.mode != RasterizerMode.BILINEAR:
-        # the reference throws std::runtime_error("unsupported rasterizer mode") for modes its
-        # native side does not know (B/rasterization/src/rasterization_api.cu:102-103); the
-        # Gaussian footprint is not part of this library
+def _require_known_mode(settings: RasterizerSettings) -> None:
+    if settings.mode not in (RasterizerMode.BILINEAR, RasterizerMode.GAUSSIAN):
+        # std::runtime_error("unsupported rasterizer mode"), B/rasterization/src/rasterization_api.cu:102-103
         raise RuntimeError("unsupported rasterizer mode")
+
+
+# instances per point the Gaussian buffers are sized for beyond the default, learnt from earlier calls
+_gaussian_capacity_hint = {"per_point": 0.0}
 
 
 def _config(settings: RasterizerSettings, n_points: int, tile: int, channels: int, feature_mode: int,
@@ -95,11 +102,64 @@ def _checked_inputs(positions, features, opacities, feature_mode: int, channels:
     return positions, features, opacities
 
 
+def _forward_gaussian(settings: RasterizerSettings, positions, features, opacities, tile: int, channels: int,
+                      feature_mode: int, inference: bool, scales, sigma_world: float, sigma_cutoff: float):
+    """Runs inpc_gaussian_forward; same return value as _forward_native, cfg is a GaussianConfig."""
+    n = positions.shape[0]
+    device = positions.device
+    sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
+    out_channels = 4 if sh else channels
+    H, W = settings.height, settings.width
+    image = torch.empty((out_channels, H, W), dtype=torch.float32, device=device)
+    alpha = torch.empty((1, H, W), dtype=torch.float32, device=device)
+    weights = None if inference else torch.empty(n, dtype=torch.float32, device=device)
+    depth = torch.empty((1, H, W), dtype=torch.float32, device=device) if inference else None
+    w2c = settings.w2c.contiguous()
+    cam_position = settings.cam_position.contiguous()
+    if scales is not None:
+        scales = scales.contiguous()
+        if scales.dtype != torch.float32:
+            raise RuntimeError("expected scalar type Float")
+        if scales.numel() != n:
+            raise RuntimeError("scales must hold one value per point")
+    capacity = int(4 * n + 65536 + _gaussian_capacity_hint["per_point"] * n)
+    lib = _lib.lib()
+    for _ in range(3):
+        capacity = min(capacity, 2**31 - 1)
+        cfg = _lib.GaussianConfig(_config(settings, n, tile, out_channels, feature_mode, inference),
+                                  float(sigma_world), float(sigma_cutoff), capacity, 0)
+        layout = _lib.GaussianLayout()
+        _lib.check(lib.inpc_gaussian_layout_query(C.byref(cfg), C.byref(layout)), "inpc_gaussian_layout_query")
+        workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+        stream = _lib.current_stream()
+        _lib.check(lib.inpc_gaussian_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
+                                             _lib.ptr(scales), _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image),
+                                             _lib.ptr(alpha), _lib.ptr(weights), _lib.ptr(depth), _lib.ptr(workspace),
+                                             layout.total_bytes, stream), "inpc_gaussian_forward")
+        counters = (C.c_uint32 * 4)()
+        rc = lib.inpc_gaussian_read_counters(C.byref(cfg), _lib.ptr(workspace), C.byref(counters), stream)
+        if rc == 0:
+            return image, alpha, (depth if inference else weights), workspace, cfg
+        if counters[1] <= capacity:
+            _lib.check(rc, "inpc_gaussian_read_counters")
+        # the instances did not fit: remember the density and go again with room for all of them
+        _gaussian_capacity_hint["per_point"] = max(_gaussian_capacity_hint["per_point"], 1.25 * counters[1] / max(n, 1))
+        if counters[1] >= 2**32 - 1:
+            break
+        capacity = int(counters[1]) + 65536
+        del workspace
+    raise _lib.BackendError("the points touch more tiles than the instance buffers can index (2^31)")
+
+
 def _forward_native(settings: RasterizerSettings, positions, features, opacities, tile: int, channels: int,
-                    feature_mode: int, inference: bool):
-    """Runs inpc_raster_forward. Returns (image, alpha, third, workspace, cfg) where `third` is the
-    blending weights (training) or the depth image (inference)."""
-    _require_bilinear(settings)
+                    feature_mode: int, inference: bool, scales=None, sigma_world: float = 0.0,
+                    sigma_cutoff: float = 3.0):
+    """Runs inpc_raster_forward (or inpc_gaussian_forward). Returns (image, alpha, third, workspace, cfg) where
+    `third` is the blending weights (training) or the depth image (inference)."""
+    _require_known_mode(settings)
+    if settings.mode == RasterizerMode.GAUSSIAN:
+        return _forward_gaussian(settings, positions, features, opacities, tile, channels, feature_mode, inference,
+                                 scales, sigma_world, sigma_cutoff)
     n = positions.shape[0]
     device = positions.device
     sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
@@ -129,7 +189,7 @@ class _Rasterize(torch.autograd.Function):
     def forward(ctx: Any, positions: torch.Tensor, features: torch.Tensor, opacities: torch.Tensor,
                 rasterizer_settings: RasterizerSettings, tile: int = 8, feature_mode: int = _lib.FEAT_SH36_F16,
                 channels: int = 4):
-        _require_bilinear(rasterizer_settings)
+        _require_known_mode(rasterizer_settings)
         positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)
         image, alpha, blending_weights, workspace, cfg = _forward_native(
             rasterizer_settings, positions, features, opacities, tile, channels, feature_mode, inference=False)
@@ -146,6 +206,8 @@ class _Rasterize(torch.autograd.Function):
     def backward(ctx: Any, grad_image: Optional[torch.Tensor], grad_alpha: Optional[torch.Tensor], _):
         image, alpha, positions, workspace = ctx.saved_tensors
         cfg = ctx.cfg
+        gaussian = isinstance(cfg, _lib.GaussianConfig)
+        base = cfg.base if gaussian else cfg
         settings = ctx.rasterizer_settings
         n = positions.shape[0]
         device = positions.device
@@ -154,24 +216,24 @@ class _Rasterize(torch.autograd.Function):
         grad_alpha = torch.zeros_like(alpha) if grad_alpha is None else grad_alpha.contiguous()
         if grad_image.dtype != torch.float32 or grad_alpha.dtype != torch.float32:
             raise RuntimeError("expected scalar type Float")
-        mode = cfg.feature_mode
+        mode = base.feature_mode
         scratch = None
         if mode == _lib.FEAT_SH36_F16:
             grad_features = torch.empty((n, 36), dtype=torch.float16, device=device)
             scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
         elif mode == _lib.FEAT_DIRECT_F16:
-            grad_features = torch.empty((n, cfg.channels), dtype=torch.float16, device=device)
-            scratch = torch.empty((n, cfg.channels), dtype=torch.float32, device=device)
+            grad_features = torch.empty((n, base.channels), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, base.channels), dtype=torch.float32, device=device)
         else:
-            grad_features = torch.empty((n, cfg.channels), dtype=torch.float32, device=device)
+            grad_features = torch.empty((n, base.channels), dtype=torch.float32, device=device)
         grad_opacities = torch.empty((n, 1), dtype=torch.float32, device=device)
         cam_position = settings.cam_position.contiguous()
-        _lib.check(_lib.lib().inpc_raster_backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha),
-                                                   _lib.ptr(image), _lib.ptr(alpha), _lib.ptr(positions),
-                                                   _lib.ptr(cam_position), _lib.ptr(grad_features),
-                                                   _lib.ptr(grad_opacities),
-                                                   _lib.ptr(scratch), _lib.ptr(workspace), workspace.numel(),
-                                                   _lib.current_stream()), "inpc_raster_backward")
+        backward = _lib.lib().inpc_gaussian_backward if gaussian else _lib.lib().inpc_raster_backward
+        _lib.check(backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha), _lib.ptr(image), _lib.ptr(alpha),
+                            _lib.ptr(positions), _lib.ptr(cam_position), _lib.ptr(grad_features),
+                            _lib.ptr(grad_opacities), _lib.ptr(scratch), _lib.ptr(workspace), workspace.numel(),
+                            _lib.current_stream()),
+                   "inpc_gaussian_backward" if gaussian else "inpc_raster_backward")
         grad_features = grad_features.view(ctx.features_shape)
         grad_opacities = grad_opacities.view(ctx.opacities_shape)
         return None, grad_features, grad_opacities, None, None, None, None
@@ -220,10 +282,12 @@ class INPCRasterizer(torch.nn.Module):
         """(image, depth, alpha) from raw (N,37) fp16 appearance output; the sigma arguments only
         concern the Gaussian footprint and are ignored by the bilinear one, as in the reference."""
         settings = self.extract_settings(view, mode)
-        _require_bilinear(settings)
+        _require_known_mode(settings)
         positions, features_raw, _ = _checked_inputs(positions, features_raw, None, _lib.FEAT_RAW37_F16, 4)
+        sigma_world = sigma_world_scale * self.extract_base_sigma_world(view.camera)
         image, alpha, depth, _, _ = _forward_native(settings, positions, features_raw, None, self.tile, 4,
-                                                    _lib.FEAT_RAW37_F16, inference=True)
+                                                    _lib.FEAT_RAW37_F16, inference=True, sigma_world=sigma_world,
+                                                    sigma_cutoff=sigma_cutoff)
         return image, depth, alpha
 
     def render_preextracted(self, view, mode: int, positions: torch.Tensor, features: torch.Tensor,
@@ -231,19 +295,25 @@ class INPCRasterizer(torch.nn.Module):
                             sigma_world_scale: float = 1.0,
                             sigma_cutoff: float = 3.0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         settings = self.extract_settings(view, mode)
-        _require_bilinear(settings)
+        _require_known_mode(settings)
         positions, features, opacities = _checked_inputs(positions, features, opacities, _lib.FEAT_SH36_F16, 4)
+        if scales is not None and scales.numel() == 0:   # the reference passes an empty tensor for "no scales"
+            scales = None
+        sigma_world = sigma_world_scale * self.extract_base_sigma_world(view.camera)
         image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, self.tile, 4,
-                                                    _lib.FEAT_SH36_F16, inference=True)
+                                                    _lib.FEAT_SH36_F16, inference=True, scales=scales,
+                                                    sigma_world=sigma_world, sigma_cutoff=sigma_cutoff)
         return image, depth, alpha
 
 
 def rasterize_points(view, positions: torch.Tensor, features: torch.Tensor, opacities: torch.Tensor, tile: int = 16,
-                     inference: bool = False):
+                     inference: bool = False, mode: int = RasterizerMode.BILINEAR.value,
+                     scales: Optional[torch.Tensor] = None, sigma_world: float = 0.0, sigma_cutoff: float = 3.0):
     """Direct-feature rasterization: features (N,C), C in {4, 8, 16}, fp32 or fp16 storage, blended as
     they are. Training: (image (C,H,W), alpha, blending_weights), differentiable in features and
-    opacities. Inference: (image, depth, alpha)."""
-    settings = INPCRasterizer.extract_settings(view, RasterizerMode.BILINEAR.value)
+    opacities. Inference: (image, depth, alpha); scales, sigma_world and sigma_cutoff concern the Gaussian
+    footprint's inference variant only."""
+    settings = INPCRasterizer.extract_settings(view, mode)
     channels = features.shape[-1]
     if features.dtype not in (torch.float32, torch.float16):
         raise RuntimeError("expected scalar type Float or Half")
@@ -251,6 +321,7 @@ def rasterize_points(view, positions: torch.Tensor, features: torch.Tensor, opac
     if inference:
         positions, features, opacities = _checked_inputs(positions, features, opacities, feature_mode, channels)
         image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, tile, channels,
-                                                    feature_mode, inference=True)
+                                                    feature_mode, inference=True, scales=scales,
+                                                    sigma_world=sigma_world, sigma_cutoff=sigma_cutoff)
         return image, depth, alpha
     return _Rasterize.apply(positions, features, opacities, settings, tile, feature_mode, channels)

@@ -18,6 +18,8 @@
 //   sort / instances / ranges  B/rasterization/src/bilinear/forward.cu:91-152, kernels.cu:186-239
 //   blend forward / inference  B/rasterization/src/bilinear/kernels.cu:241-313,422-495
 //   blend backward             B/rasterization/src/bilinear/kernels.cu:315-420
+//   Gaussian footprint         B/rasterization/src/gaussian/kernels.cu:11-324 (preprocess),
+//                              :401-474 (blend), :476-579 (backward), :581-660 (inference)
 //
 // Where the reference leaves a result to scheduling (atomic compaction order, atomic sample
 // slots, the association order of cub's float reduce/scan) this file fixes one canonical
@@ -181,6 +183,25 @@ inline uint16_t float_to_half(float f) {
 }
 
 inline float saturate(float v) { return v < 0.0f ? 0.0f : (v > 1.0f ? 1.0f : v); }
+
+// exp(x) for x <= 0 as the Gaussian footprint evaluates it (the reference calls expf / __expf,
+// B/rasterization/src/gaussian/kernels.cu:451,548,634, whose last bits are the CUDA library's). One fixed
+// sequence of fp32 operations instead, so that the cut at the footprint's threshold falls on the same
+// pixels everywhere: n = rint(x * log2 e), r = x - n * ln 2 in two parts, a degree-7 polynomial
+// (Cephes' expf coefficients) and a scaling by 2^n. Within 2 ulp of exp on [-88, 0]; 0 below.
+inline float footprint_exp(float x) {
+    if (!(x >= -87.0f)) return 0.0f;
+    const float n = std::nearbyint(x * 1.44269504088896341f);
+    const float r = (x - n * 0.693359375f) - n * -2.12194440e-4f;
+    float p = 1.9875691500e-4f;
+    p = p * r + 1.3981999507e-3f;
+    p = p * r + 8.3334519073e-3f;
+    p = p * r + 4.1665795894e-2f;
+    p = p * r + 1.6666665459e-1f;
+    p = p * r + 5.0000001201e-1f;
+    const float y = (p * (r * r) + r) + 1.0f;
+    return std::ldexp(y, (int)n);
+}
 
 // ---------------------------------------------------------------------------------------------
 // canonical float reduce / scan: chunks of 64, left to right inside a chunk, chunk totals
@@ -389,6 +410,10 @@ struct RasterState {
     std::vector<float> depth;         // (N)
     std::vector<float> opacity;       // (N) as blended
     std::vector<float> feat;          // (N,C) as blended
+    bool gaussian = false;
+    std::vector<float> conic;         // (N,3), Gaussian footprint only
+    std::vector<float> reach;         // (N,2): no pixel further than this from the point (x, y) passes the threshold
+    float threshold = 0.0f;           // smallest footprint value that is drawn
     uint32_t n_visible = 0, n_instances = 0;
     std::vector<uint32_t> depth_keys;   // (V) sorted
     std::vector<uint32_t> depth_order;  // (V) point ids in (depth, id) order
@@ -397,8 +422,16 @@ struct RasterState {
     std::vector<uint32_t> ranges;       // (n_tiles,2)
 };
 
+// Parameters of the Gaussian footprint; null = bilinear.
+struct FootprintParams {
+    bool training;
+    float sigma_world, sigma_cutoff;
+    const float* scales;
+};
+
 int raster_prepare(RasterState& st, const inpc_raster_config* cfg, const float* positions, const void* features,
-                   const float* opacities, const float* w2c, const float* cam_position) {
+                   const float* opacities, const float* w2c, const float* cam_position,
+                   const FootprintParams* fp = nullptr) {
     const inpc_camera& cam = cfg->cam;
     const uint32_t n = cfg->n_points;
     const int T = cfg->tile, mode = cfg->feature_mode;
@@ -420,6 +453,13 @@ int raster_prepare(RasterState& st, const inpc_raster_config* cfg, const float* 
     st.depth.assign(n, 0.0f);
     st.opacity.assign(n, 0.0f);
     st.feat.assign((size_t)n * C, 0.0f);
+    st.gaussian = fp != nullptr;
+    if (fp) {
+        st.conic.assign((size_t)n * 3, 0.0f);
+        st.reach.assign((size_t)n * 2, 0.0f);
+        // kernels.cu:452 (training); inference.cu:171 (host expf)
+        st.threshold = fp->training ? 0.01110899653f : std::exp(-0.5f * fp->sigma_cutoff * fp->sigma_cutoff);
+    }
     const float fT = (float)T, fgw = (float)st.gw, fgh = (float)st.gh;
 
     // preprocess (B/rasterization/src/bilinear/kernels.cu:36-76)
@@ -433,12 +473,47 @@ int raster_prepare(RasterState& st, const inpc_raster_config* cfg, const float* 
         const float y = affine_row(w2c + 4, px, py, pz) / depth;
         const float sx = x * cam.focal_x + cam.center_x;
         const float sy = y * cam.focal_y + cam.center_y;
-        // min(grid, max(0, floor/ceil((s -+ 0.5) / T))), clamped in float so that huge or
+        float reach_x = 0.5f, reach_y = 0.5f;  // half extent of the tile bounds
+        float conic[3] = {0.0f, 0.0f, 0.0f};
+        float cov_x = 0.0f, cov_z = 0.0f;
+        if (fp) {
+            // B/rasterization/src/gaussian/kernels.cu:57-81 (training), :166-187, :268-294 (inference)
+            float variance;
+            if (fp->training) {
+                constexpr float numerator = 0.3f * 0.3f * 0.5f * 0.5f;
+                variance = numerator / (cam.focal_x * cam.focal_y);
+            } else if (fp->scales) {
+                variance = fp->scales[i] * fp->scales[i];
+            } else {
+                variance = fp->sigma_world * fp->sigma_world;
+            }
+            const float j00 = cam.focal_x / depth;
+            const float lim_x = 1.3f * cam.center_x / cam.focal_x, nlim_x = -1.3f * cam.center_x / cam.focal_x;
+            const float j02 = -j00 * std::fmax(nlim_x, std::fmin(x, lim_x));  // clamp of B/utils/helper_math.h
+            const float j11 = cam.focal_y / depth;
+            const float lim_y = 1.3f * cam.center_y / cam.focal_y, nlim_y = -1.3f * cam.center_y / cam.focal_y;
+            const float j12 = -j11 * std::fmax(nlim_y, std::fmin(y, lim_y));
+            cov_x = variance * (j00 * j00 + j02 * j02);
+            const float cov_y = variance * (j02 * j12);
+            cov_z = variance * (j11 * j11 + j12 * j12);
+            cov_x += 0.16f;
+            cov_z += 0.16f;
+            const float det = cov_x * cov_z - cov_y * cov_y;
+            if (det == 0.0f) continue;
+            const float rcp = 1.0f / det;
+            conic[0] = cov_z * rcp;
+            conic[1] = -cov_y * rcp;
+            conic[2] = cov_x * rcp;
+            const float cutoff = fp->training ? 3.0f : fp->sigma_cutoff;
+            reach_x = cutoff * std::sqrt(cov_x) - 0.5f;
+            reach_y = cutoff * std::sqrt(cov_z) - 0.5f;
+        }
+        // min(grid, max(0, floor/ceil((s -+ reach) / T))), clamped in float so that huge or
         // non-finite coordinates behave like the saturating __float2int_rd / _ru.
-        const float x0 = std::fmin(fgw, std::fmax(0.0f, std::floor((sx - 0.5f) / fT)));
-        const float x1 = std::fmin(fgw, std::fmax(0.0f, std::ceil((sx + 0.5f) / fT)));
-        const float y0 = std::fmin(fgh, std::fmax(0.0f, std::floor((sy - 0.5f) / fT)));
-        const float y1 = std::fmin(fgh, std::fmax(0.0f, std::ceil((sy + 0.5f) / fT)));
+        const float x0 = std::fmin(fgw, std::fmax(0.0f, std::floor((sx - reach_x) / fT)));
+        const float x1 = std::fmin(fgw, std::fmax(0.0f, std::ceil((sx + reach_x) / fT)));
+        const float y0 = std::fmin(fgh, std::fmax(0.0f, std::floor((sy - reach_y) / fT)));
+        const float y1 = std::fmin(fgh, std::fmax(0.0f, std::ceil((sy + reach_y) / fT)));
         const uint32_t ux0 = (uint32_t)x0, ux1 = (uint32_t)x1, uy0 = (uint32_t)y0, uy1 = (uint32_t)y1;
         const uint32_t touched = (ux1 - ux0) * (uy1 - uy0);  // unsigned, as in the reference
         if (touched == 0 || ux1 < ux0 || uy1 < uy0) continue;
@@ -450,6 +525,14 @@ int raster_prepare(RasterState& st, const inpc_raster_config* cfg, const float* 
         st.xy[2 * i] = sx;
         st.xy[2 * i + 1] = sy;
         st.depth[i] = depth;
+        if (fp) {
+            for (int k = 0; k < 3; ++k) st.conic[3 * i + k] = conic[k];
+            // G >= threshold implies |dx| <= sqrt(-2 ln(threshold) cov_x): a bound for the pixel loops only,
+            // taken generously; the exact test decides
+            const float l2 = -2.0f * std::log(st.threshold);
+            st.reach[2 * i] = std::sqrt(l2 * cov_x) * 1.01f + 1.0f;
+            st.reach[2 * i + 1] = std::sqrt(l2 * cov_z) * 1.01f + 1.0f;
+        }
         float* f = &st.feat[i * C];
         if (mode == INPC_FEAT_SH36_F16) {
             sh_to_view(sh_basis(positions + 3 * i, cam_position), (const uint16_t*)features + 36 * i, f);
@@ -537,6 +620,36 @@ inline PixelWindow pixel_window(float sx, float sy, int tx, int ty, int T, int W
     w.y_begin = (int)lo_y;
     w.y_end = (int)hi_y;
     return w;
+}
+
+// The pixels of tile (tx,ty) whose centre lies within (rx, ry) of (sx, sy).
+inline PixelWindow footprint_window(float sx, float sy, float rx, float ry, int tx, int ty, int T, int W, int H) {
+    PixelWindow w;
+    const int tile_x0 = tx * T, tile_y0 = ty * T;
+    const int tile_x1 = std::min(tile_x0 + T, W), tile_y1 = std::min(tile_y0 + T, H);
+    const float lo_x = std::fmax(std::ceil(sx - rx - 0.5f), (float)tile_x0);
+    const float hi_x = std::fmin(std::floor(sx + rx - 0.5f) + 1.0f, (float)tile_x1);
+    const float lo_y = std::fmax(std::ceil(sy - ry - 0.5f), (float)tile_y0);
+    const float hi_y = std::fmin(std::floor(sy + ry - 0.5f) + 1.0f, (float)tile_y1);
+    if (!(hi_x > lo_x) || !(hi_y > lo_y)) {
+        w.x_begin = w.x_end = w.y_begin = w.y_end = 0;
+        return w;
+    }
+    w.x_begin = (int)lo_x;
+    w.x_end = (int)hi_x;
+    w.y_begin = (int)lo_y;
+    w.y_end = (int)hi_y;
+    return w;
+}
+
+// Footprint value of a point at a pixel centre (B/rasterization/src/gaussian/kernels.cu:447-452); false when
+// the pixel is skipped.
+inline bool footprint_value(const float* conic, float sx, float sy, float cx, float cy, float threshold, float& G) {
+    const float dx = sx - cx, dy = sy - cy;
+    const float exponent = -0.5f * (conic[0] * dx * dx + conic[2] * dy * dy) - conic[1] * dx * dy;
+    if (exponent > 0.0f) return false;
+    G = footprint_exp(exponent);
+    return !(G < threshold);
 }
 
 }  // namespace
@@ -785,6 +898,7 @@ struct oracle_raster_debug {
     uint16_t* instance_keys;
     uint32_t* instance_points;
     uint32_t* tile_ranges;
+    float* conic;          // (N,3), Gaussian footprint only
 };
 
 // Forward / inference (B/rasterization/src/bilinear/forward.cu:12-170, kernels.cu:241-313,422-495).
@@ -812,15 +926,24 @@ static int raster_forward_with_state(const RasterState& st, const inpc_raster_co
                 const float sx = st.xy[2 * (size_t)p], sy = st.xy[2 * (size_t)p + 1];
                 const float op = st.opacity[p];
                 const float* f = &st.feat[(size_t)p * C];
-                const PixelWindow w = pixel_window(sx, sy, tx, ty, T, W, H);
+                const PixelWindow w = st.gaussian ? footprint_window(sx, sy, st.reach[2 * (size_t)p],
+                                                                     st.reach[2 * (size_t)p + 1], tx, ty, T, W, H)
+                                                  : pixel_window(sx, sy, tx, ty, T, W, H);
                 for (int py = w.y_begin; py < w.y_end; ++py)
                     for (int px = w.x_begin; px < w.x_end; ++px) {
                         const int lp = (py - ty * T) * T + (px - tx * T);
                         if (done[lp]) continue;
-                        const float dx = std::fabs(sx - ((float)px + 0.5f));
-                        const float dy = std::fabs(sy - ((float)py + 0.5f));
-                        if (dx >= 1.0f || dy >= 1.0f) continue;
-                        const float wgt = saturate(1.0f - dx) * saturate(1.0f - dy);
+                        float wgt;
+                        if (st.gaussian) {
+                            if (!footprint_value(&st.conic[3 * (size_t)p], sx, sy, (float)px + 0.5f, (float)py + 0.5f,
+                                                 st.threshold, wgt))
+                                continue;
+                        } else {
+                            const float dx = std::fabs(sx - ((float)px + 0.5f));
+                            const float dy = std::fabs(sy - ((float)py + 0.5f));
+                            if (dx >= 1.0f || dy >= 1.0f) continue;
+                            wgt = saturate(1.0f - dx) * saturate(1.0f - dy);
+                        }
                         const float a = op * wgt;
                         const float bw = Tr[lp] * a;
                         if (bw > 0.0f && blending_weights) {
@@ -868,6 +991,7 @@ static int raster_forward_with_state(const RasterState& st, const inpc_raster_co
         if (dbg->instance_points)
             std::copy(st.inst_points.begin(), st.inst_points.begin() + st.n_instances, dbg->instance_points);
         if (dbg->tile_ranges) std::copy(st.ranges.begin(), st.ranges.end(), dbg->tile_ranges);
+        if (dbg->conic && st.gaussian) std::copy(st.conic.begin(), st.conic.end(), dbg->conic);
         (void)n;
     }
     return INPC_OK;
@@ -901,16 +1025,25 @@ static int raster_backward_with_state(const RasterState& st, const inpc_raster_c
                 const float sx = st.xy[2 * (size_t)p], sy = st.xy[2 * (size_t)p + 1];
                 const float op = st.opacity[p];
                 const float* f = &st.feat[(size_t)p * C];
-                const PixelWindow w = pixel_window(sx, sy, tx, ty, T, W, H);
+                const PixelWindow w = st.gaussian ? footprint_window(sx, sy, st.reach[2 * (size_t)p],
+                                                                     st.reach[2 * (size_t)p + 1], tx, ty, T, W, H)
+                                                  : pixel_window(sx, sy, tx, ty, T, W, H);
                 for (int py = w.y_begin; py < w.y_end; ++py)
                     for (int px = w.x_begin; px < w.x_end; ++px) {
                         const int lp = (py - ty * T) * T + (px - tx * T);
                         if (done[lp]) continue;
-                        const float dx = std::fabs(sx - ((float)px + 0.5f));
-                        const float dy = std::fabs(sy - ((float)py + 0.5f));
-                        if (dx >= 1.0f || dy >= 1.0f) continue;
+                        float wgt;
+                        if (st.gaussian) {
+                            if (!footprint_value(&st.conic[3 * (size_t)p], sx, sy, (float)px + 0.5f, (float)py + 0.5f,
+                                                 st.threshold, wgt))
+                                continue;
+                        } else {
+                            const float dx = std::fabs(sx - ((float)px + 0.5f));
+                            const float dy = std::fabs(sy - ((float)py + 0.5f));
+                            if (dx >= 1.0f || dy >= 1.0f) continue;
+                            wgt = saturate(1.0f - dx) * saturate(1.0f - dy);
+                        }
                         const size_t pix = (size_t)py * W + px;
-                        const float wgt = saturate(1.0f - dx) * saturate(1.0f - dy);
                         const float a = op * wgt;
                         const float tr = Tr[lp];
                         const float bw = tr * a;
@@ -1005,6 +1138,43 @@ int oracle_raster_forward_backward(const inpc_raster_config* cfg, const float* p
     return raster_backward_with_state(st, cfg, grad_image, grad_alpha, image, alpha, positions, cam_position,
                                       grad_features, grad_opacities, nullptr);
 }
+
+// Gaussian footprint (B/rasterization/src/gaussian/): same pipeline, a point covers the pixels where its
+// screen-space Gaussian stays above the threshold. The instance buffers of `dbg` must hold n_instances entries
+// (dbg->counts reports them; call once with null instance pointers to size them).
+static FootprintParams footprint_params(const inpc_gaussian_config* cfg, const float* scales) {
+    FootprintParams fp;
+    fp.training = (cfg->base.flags & INPC_RASTER_INFERENCE) == 0;
+    fp.sigma_world = cfg->sigma_world;
+    fp.sigma_cutoff = cfg->sigma_cutoff;
+    fp.scales = fp.training ? nullptr : scales;
+    return fp;
+}
+
+int oracle_gaussian_forward(const inpc_gaussian_config* cfg, const float* positions, const void* features,
+                            const float* opacities, const float* scales, const float* w2c, const float* cam_position,
+                            float* image, float* alpha, float* blending_weights, float* depth_image,
+                            oracle_raster_debug* dbg) {
+    RasterState st;
+    const FootprintParams fp = footprint_params(cfg, scales);
+    const int rc = raster_prepare(st, &cfg->base, positions, features, opacities, w2c, cam_position, &fp);
+    if (rc != INPC_OK) return rc;
+    return raster_forward_with_state(st, &cfg->base, image, alpha, blending_weights, depth_image, dbg);
+}
+
+int oracle_gaussian_backward(const inpc_gaussian_config* cfg, const float* grad_image, const float* grad_alpha,
+                             const float* image, const float* alpha, const float* positions, const void* features,
+                             const float* opacities, const float* w2c, const float* cam_position,
+                             void* grad_features, float* grad_opacities, float* grad_view_out) {
+    RasterState st;
+    const FootprintParams fp = footprint_params(cfg, nullptr);
+    const int rc = raster_prepare(st, &cfg->base, positions, features, opacities, w2c, cam_position, &fp);
+    if (rc != INPC_OK) return rc;
+    return raster_backward_with_state(st, &cfg->base, grad_image, grad_alpha, image, alpha, positions, cam_position,
+                                      grad_features, grad_opacities, grad_view_out);
+}
+
+float oracle_footprint_exp(float x) { return footprint_exp(x); }
 
 // Wall-clock helper for benchmarks: seconds since an arbitrary origin.
 double oracle_now(void) {

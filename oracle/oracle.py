@@ -71,6 +71,17 @@ class _RasterDebug(C.Structure):
         ("instance_keys", C.c_void_p),
         ("instance_points", C.c_void_p),
         ("tile_ranges", C.c_void_p),
+        ("conic", C.c_void_p),
+    ]
+
+
+class GaussianConfig(C.Structure):
+    _fields_ = [
+        ("base", RasterConfig),
+        ("sigma_world", C.c_float),
+        ("sigma_cutoff", C.c_float),
+        ("max_instances", C.c_uint32),
+        ("reserved", C.c_uint32),
     ]
 
 
@@ -96,6 +107,8 @@ def lib() -> C.CDLL:
         _lib.oracle_half_to_float.argtypes = [C.c_uint16]
         _lib.oracle_now.restype = C.c_double
         _lib.oracle_num_threads.restype = C.c_int
+        _lib.oracle_footprint_exp.restype = C.c_float
+        _lib.oracle_footprint_exp.argtypes = [C.c_float]
     return _lib
 
 
@@ -267,8 +280,10 @@ def _features_array(features, feature_mode):
     return np.ascontiguousarray(features, dtype=np.float16)
 
 
-def raster_forward(cfg: RasterConfig, positions, features, opacities, w2c, cam_position=None, debug: bool = False):
-    """Returns dict(image (C,H,W), alpha (1,H,W), blending_weights (N,) | depth_image (1,H,W), + debug buffers)."""
+def raster_forward(cfg: RasterConfig, positions, features, opacities, w2c, cam_position=None, debug: bool = False,
+                   gaussian: "GaussianConfig | None" = None, scales=None, n_instances_hint: int = 0):
+    """Returns dict(image (C,H,W), alpha (1,H,W), blending_weights (N,) | depth_image (1,H,W), + debug buffers).
+    With `gaussian` (whose base is `cfg`) the Gaussian footprint is drawn instead of the bilinear one."""
     n = cfg.n_points
     W, H = cfg.cam.width, cfg.cam.height
     sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
@@ -297,17 +312,24 @@ def raster_forward(cfg: RasterConfig, positions, features, opacities, w2c, cam_p
             "counts": np.zeros(2, np.uint32),
             "depth_keys": np.zeros(n, np.uint32),
             "depth_order": np.zeros(n, np.uint32),
-            "instance_keys": np.zeros(4 * n, np.uint16),
-            "instance_points": np.zeros(4 * n, np.uint32),
+            "instance_keys": np.zeros(max(4 * n, n_instances_hint), np.uint16),
+            "instance_points": np.zeros(max(4 * n, n_instances_hint), np.uint32),
             "tile_ranges": np.zeros((n_tiles, 2), np.uint32),
+            "conic": np.zeros((n, 3), np.float32),
         }
         dbg = _RasterDebug(*[_p(bufs[name]) for name, _ in _RasterDebug._fields_])
         dbg_ptr = C.byref(dbg)
         out.update(bufs)
-    rc = lib().oracle_raster_forward(C.byref(cfg), _p(positions), _p(features), _p(opacities), _p(w2c),
-                                     _p(cam_position), _p(image), _p(alpha), _p(bw), _p(depth_image), dbg_ptr)
+    if gaussian is not None:
+        scales = None if scales is None else _f32(scales).reshape(-1)
+        rc = lib().oracle_gaussian_forward(C.byref(gaussian), _p(positions), _p(features), _p(opacities), _p(scales),
+                                           _p(w2c), _p(cam_position), _p(image), _p(alpha), _p(bw), _p(depth_image),
+                                           dbg_ptr)
+    else:
+        rc = lib().oracle_raster_forward(C.byref(cfg), _p(positions), _p(features), _p(opacities), _p(w2c),
+                                         _p(cam_position), _p(image), _p(alpha), _p(bw), _p(depth_image), dbg_ptr)
     if rc != 0:
-        raise RuntimeError(f"oracle_raster_forward failed with {rc}")
+        raise RuntimeError(f"oracle raster forward failed with {rc}")
     if debug:
         v, i = int(out["counts"][0]), int(out["counts"][1])
         out["n_visible"], out["n_instances"] = v, i
@@ -318,8 +340,44 @@ def raster_forward(cfg: RasterConfig, positions, features, opacities, w2c, cam_p
     return out
 
 
+def gaussian_instance_count(gcfg: GaussianConfig, positions, w2c, scales=None) -> int:
+    """Number of (point, tile) instances of a Gaussian-footprint call (sizes the debug buffers)."""
+    cfg = gcfg.base
+    n = cfg.n_points
+    counts = np.zeros(2, np.uint32)
+    fields = {name: None for name, _ in _RasterDebug._fields_}
+    fields["counts"] = counts
+    dbg = _RasterDebug(*[_p(fields[name]) for name, _ in _RasterDebug._fields_])
+    W, H = cfg.cam.width, cfg.cam.height
+    sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
+    Cn = 4 if sh else cfg.channels
+    width = {FEAT_SH36_F16: 36, FEAT_RAW37_F16: 37}.get(cfg.feature_mode, Cn)
+    feats = np.zeros((n, width), np.float32 if cfg.feature_mode == FEAT_DIRECT_F32 else np.float16)
+    image = np.zeros((Cn, H, W), np.float32)
+    alpha = np.zeros((1, H, W), np.float32)
+    third = np.zeros(max(n, H * W), np.float32)
+    scales = None if scales is None else _f32(scales).reshape(-1)
+    rc = lib().oracle_gaussian_forward(C.byref(gcfg), _p(_f32(positions)), _p(feats), _p(np.zeros(n, np.float32)),
+                                       _p(scales), _p(_f32(w2c)), _p(np.zeros(3, np.float32)), _p(image), _p(alpha),
+                                       _p(third), _p(third), C.byref(dbg))
+    if rc != 0:
+        raise RuntimeError(f"oracle_gaussian_forward failed with {rc}")
+    return int(counts[1])
+
+
+def footprint_exp(x):
+    """exp(x), x <= 0, as the Gaussian footprint evaluates it (elementwise, float32)."""
+    x = np.asarray(x, np.float32)
+    out = np.empty_like(x)
+    f = lib().oracle_footprint_exp
+    flat_in, flat_out = x.reshape(-1), out.reshape(-1)
+    for i in range(flat_in.size):
+        flat_out[i] = f(float(flat_in[i]))
+    return out
+
+
 def raster_backward(cfg: RasterConfig, grad_image, grad_alpha, image, alpha, positions, features, opacities, w2c,
-                    cam_position=None):
+                    cam_position=None, gaussian: "GaussianConfig | None" = None):
     """Returns (grad_features, grad_opacities (N,), grad_view (N,C))."""
     n = cfg.n_points
     sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
@@ -337,9 +395,9 @@ def raster_backward(cfg: RasterConfig, grad_image, grad_alpha, image, alpha, pos
         gf = np.zeros((n, Cn), dtype=np.float32)
     go = np.zeros(n, dtype=np.float32)
     gv = np.zeros((n, Cn), dtype=np.float32)
-    rc = lib().oracle_raster_backward(C.byref(cfg), _p(grad_image), _p(grad_alpha), _p(image), _p(alpha),
-                                      _p(positions), _p(features), _p(opacities), _p(w2c), _p(cam_position), _p(gf),
-                                      _p(go), _p(gv))
+    fn = lib().oracle_raster_backward if gaussian is None else lib().oracle_gaussian_backward
+    rc = fn(C.byref(cfg if gaussian is None else gaussian), _p(grad_image), _p(grad_alpha), _p(image), _p(alpha),
+            _p(positions), _p(features), _p(opacities), _p(w2c), _p(cam_position), _p(gf), _p(go), _p(gv))
     if rc != 0:
         raise RuntimeError(f"oracle_raster_backward failed with {rc}")
     return gf, go, gv

@@ -257,6 +257,115 @@ class RasterRun:
         return gf.cpu().numpy(), go.cpu().numpy()
 
 
+class GaussianRun:
+    """inpc_gaussian_forward (+ backward) through the C ABI on numpy inputs."""
+
+    def __init__(self, hv, positions, features, opacities, tile=8, channels=4, feature_mode=_lib.FEAT_DIRECT_F32,
+                 inference=False, scales=None, sigma_world=0.0, sigma_cutoff=3.0, max_instances=0, device="cuda:0"):
+        self.lib = _lib.lib()
+        self.n = len(positions)
+        sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
+        self.C = 4 if sh else channels
+        base = _lib.RasterConfig(self.n, tile, self.C, feature_mode, _lib.RASTER_INFERENCE if inference else 0,
+                                 cam_struct(hv.camera))
+        self.cfg = _lib.GaussianConfig(base, sigma_world, sigma_cutoff, max_instances, 0)
+        self.layout = _lib.GaussianLayout()
+        _lib.check(self.lib.inpc_gaussian_layout_query(C.byref(self.cfg), C.byref(self.layout)), "layout")
+        self.inference = inference
+        self.device = device
+        self.positions = dev(np.asarray(positions, np.float32).reshape(-1, 3), device)
+        self.features = dev(np.asarray(features, FEATURE_DTYPES[feature_mode]), device)
+        self.opacities = None if opacities is None else dev(np.asarray(opacities, np.float32).reshape(-1), device)
+        self.scales = None if scales is None else dev(np.asarray(scales, np.float32).reshape(-1), device)
+        self.w2c = dev(hv.w2c, device)
+        self.cam_position = dev(hv.position, device)
+        H, W = hv.camera.height, hv.camera.width
+        self.image = torch.full((self.C, H, W), float("nan"), dtype=torch.float32, device=device)
+        self.alpha = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device)
+        self.bw = None if inference else torch.full((max(self.n, 1),), float("nan"), dtype=torch.float32, device=device)
+        self.depth_image = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device) if inference else None
+        # poisoned: nothing may depend on what the workspace held before the call
+        self.ws = torch.randint(0, 256, (self.layout.total_bytes,), dtype=torch.uint8, device=device)
+
+    def forward(self):
+        _lib.check(self.lib.inpc_gaussian_forward(
+            C.byref(self.cfg), _lib.ptr(self.positions), _lib.ptr(self.features), _lib.ptr(self.opacities),
+            _lib.ptr(self.scales), _lib.ptr(self.w2c), _lib.ptr(self.cam_position), _lib.ptr(self.image),
+            _lib.ptr(self.alpha), _lib.ptr(self.bw), _lib.ptr(self.depth_image), _lib.ptr(self.ws),
+            self.layout.total_bytes, stream()), "inpc_gaussian_forward")
+        return self
+
+    def counters(self, check=True):
+        """(return code, [n_visible, n_instances, error flag, instances drawn])"""
+        out = (C.c_uint32 * 4)()
+        rc = self.lib.inpc_gaussian_read_counters(C.byref(self.cfg), _lib.ptr(self.ws), C.byref(out), stream())
+        if check:
+            _lib.check(rc, "inpc_gaussian_read_counters")
+        return rc, [int(v) for v in out]
+
+    def _buf(self, offset, count, dtype):
+        nbytes = count * np.dtype(dtype).itemsize
+        return self.ws[offset:offset + nbytes].cpu().numpy().view(dtype)
+
+    def debug(self):
+        """Intermediate buffers in the oracle's shapes."""
+        L, n = self.layout, self.n
+        _, (v, i, _, kept) = self.counters()
+        assert kept == i
+        touched = self._buf(L.point_touched, n, np.uint32).copy()
+        vis = touched > 0
+        packed = self._buf(L.point_bounds, 2 * n, np.uint32).reshape(n, 2)
+        bounds = np.stack([packed[:, 0] & 0xFFFF, packed[:, 0] >> 16, packed[:, 1] & 0xFFFF, packed[:, 1] >> 16],
+                          axis=1).astype(np.uint16)
+        bounds[~vis] = 0
+        stride = L.record_stride
+        raw = self._buf(L.point_record, n * stride, np.uint8).reshape(n, stride)
+        head = raw[:, :32].copy().view(np.float32).reshape(n, 8)
+        word = head.view(np.uint32)[:, 7]
+        assert (word[vis] & 0x7FFFFFFF == np.flatnonzero(vis)).all(), "a record names another point"
+        assert ((word[vis] >> 31) == (touched[vis] > 1)).all(), "the several-tiles flag differs from the tile count"
+        feats = raw[:, 32:32 + 4 * self.C].copy().view(np.float32).reshape(n, self.C)
+
+        def drawn(a):
+            a = a.copy()
+            a[~vis] = 0
+            return a
+
+        return {
+            "n_visible": v, "n_instances": i, "n_touched": touched, "bounds": bounds,
+            "screen_xy": drawn(head[:, :2]), "opacity": drawn(head[:, 2]), "conic": drawn(head[:, 3:6]),
+            "depth": drawn(head[:, 6]), "features_view": drawn(feats),
+            "depth_keys": (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32),
+            "depth_order": self._buf(L.depth_order, n, np.uint32)[:v].copy(),
+            "instance_keys": self._buf(L.instance_keys, i, np.uint16).copy(),
+            "instance_points": self._buf(L.instance_points, i, np.uint32).copy(),
+            "tile_ranges": self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2),
+        }
+
+    outputs = RasterRun.outputs
+
+    def backward(self, grad_image, grad_alpha):
+        mode = self.cfg.base.feature_mode
+        n, Cn = self.n, self.C
+        device = self.device
+        scratch = None
+        if mode == _lib.FEAT_SH36_F16:
+            gf = torch.full((n, 36), float("nan"), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
+        elif mode == _lib.FEAT_DIRECT_F16:
+            gf = torch.full((n, Cn), float("nan"), dtype=torch.float16, device=device)
+            scratch = torch.empty((n, Cn), dtype=torch.float32, device=device)
+        else:
+            gf = torch.full((n, Cn), float("nan"), dtype=torch.float32, device=device)
+        go = torch.full((n,), float("nan"), dtype=torch.float32, device=device)
+        gi, ga = dev(np.asarray(grad_image, np.float32), device), dev(np.asarray(grad_alpha, np.float32), device)
+        _lib.check(self.lib.inpc_gaussian_backward(
+            C.byref(self.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(self.image), _lib.ptr(self.alpha),
+            _lib.ptr(self.positions), _lib.ptr(self.cam_position), _lib.ptr(gf), _lib.ptr(go), _lib.ptr(scratch),
+            _lib.ptr(self.ws), self.layout.total_bytes, stream()), "inpc_gaussian_backward")
+        return gf.cpu().numpy(), go.cpu().numpy()
+
+
 def assert_close(actual, expected, rtol=1e-4, atol=1e-6, what=""):
     """allclose with a report of the worst element."""
     actual, expected = np.asarray(actual, np.float64), np.asarray(expected, np.float64)

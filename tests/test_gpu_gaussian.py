@@ -1,0 +1,266 @@
+"""GPU parity of the rasterizer's Gaussian footprint against the CPU oracle, through the C ABI.
+
+Bit-exact: tile bounds, screen coordinates, conics, depth order, instance order, tile ranges, and (because the
+footprint's exponential is one fixed sequence of fp32 operations on both sides) image, alpha and depth image.
+Within 1e-4 relative: blending weights and gradients, which both sides sum in an order of their own.
+"""
+import numpy as np
+import pytest
+import torch
+
+from inpc_amd import _lib, synthetic
+from tests import helpers as H
+from tests.test_oracle_gaussian import gcfg_of, near_camera_points
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+
+
+def oracle_run(O, hv, pos, feats, opac, tile, channels, mode=None, inference=False, scales=None, sigma_world=0.0,
+               sigma_cutoff=3.0, cam_position=None):
+    n = len(pos)
+    g = gcfg_of(O, hv, n, tile, channels, mode, inference, sigma_world, sigma_cutoff)
+    count = O.gaussian_instance_count(g, pos, hv.w2c, scales)
+    ref = O.raster_forward(g.base, pos, feats, opac, hv.w2c, cam_position, debug=True, gaussian=g, scales=scales,
+                           n_instances_hint=count)
+    return g, ref
+
+
+def check_structure(dbg, ref):
+    assert dbg["n_visible"] == ref["n_visible"]
+    assert dbg["n_instances"] == ref["n_instances"]
+    np.testing.assert_array_equal(dbg["n_touched"], ref["n_touched"])
+    np.testing.assert_array_equal(dbg["bounds"], ref["bounds"])
+    for name in ("screen_xy", "conic", "depth"):
+        np.testing.assert_array_equal(dbg[name].view(np.uint32), ref[name].view(np.uint32), err_msg=name)
+    np.testing.assert_array_equal(dbg["depth_keys"], ref["depth_keys"])
+    np.testing.assert_array_equal(dbg["depth_order"], ref["depth_order"])
+    np.testing.assert_array_equal(dbg["instance_keys"], ref["instance_keys"])
+    np.testing.assert_array_equal(dbg["instance_points"], ref["instance_points"])
+    np.testing.assert_array_equal(dbg["tile_ranges"], ref["tile_ranges"])
+
+
+def scene(n, channels, seed, width=251, height=163, focal=230.0, near=400):
+    hv = synthetic.rotated_camera(width, height, focal, 2.4, 0.2, -0.1)
+    pos = synthetic.cube_points(n, 1.6, seed)
+    if near:
+        pos[:near] = near_camera_points(hv, near, seed + 7)   # footprints of many tiles
+    feats, opac = synthetic.point_attributes(n, channels, "normal", seed + 1)
+    return hv, pos, feats, opac
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+@pytest.mark.parametrize("channels", [4, 8, 16])
+def test_forward_direct_f32(gpu, oracle, tile, channels):
+    n = 40000
+    hv, pos, feats, opac = scene(n, channels, seed=tile + channels)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, channels).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, channels)
+    assert ref["n_touched"].max() > 16
+    dbg = run.debug()
+    check_structure(dbg, ref)
+    np.testing.assert_array_equal(dbg["features_view"], ref["features_view"])
+    out = run.outputs()
+    np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_forward_backward_dense_opaque_scene(gpu, oracle, tile):
+    # many nearly opaque points per pixel: early termination, tiles of many batches
+    n = 120000
+    hv = synthetic.camera_on_z(97, 61, 90.0, 2.4)
+    pos = synthetic.cube_points(n, 1.2, 5)
+    feats, _ = synthetic.point_attributes(n, 8, "uniform", 6)
+    opac = np.random.default_rng(7).uniform(0.3, 0.999, n).astype(np.float32)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, 8).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, 8)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    assert (ref["alpha"] == 1.0).mean() > 0.3
+    np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+    rng = np.random.default_rng(8)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                               gaussian=g)
+    H.assert_close(gf, gf_ref, RTOL, 1e-7, "feature gradients")
+    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+
+
+@pytest.mark.parametrize("tile", [8, 16])
+def test_forward_sh36_and_backward(gpu, oracle, tile):
+    n = 30000
+    hv = synthetic.rotated_camera(233, 171, 210.0, 2.6, yaw=0.5, pitch=-0.3)
+    pos = synthetic.cube_points(n, 1.5, 11)
+    pos[:300] = near_camera_points(hv, 300, 3)
+    feats = synthetic.sh_features(n, 12)
+    _, opac = synthetic.point_attributes(n, 4, "normal", 13)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_SH36_F16).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, 4, oracle.FEAT_SH36_F16, cam_position=hv.position)
+    dbg = run.debug()
+    check_structure(dbg, ref)
+    vis = ref["n_touched"] > 0
+    H.assert_close(dbg["features_view"][vis], ref["features_view"][vis], RTOL, 1e-5, "SH view features")
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    rng = np.random.default_rng(14)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    image_gpu, alpha_gpu = out["image"], out["alpha"]
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, image_gpu, alpha_gpu, pos, feats, opac, hv.w2c,
+                                               hv.position, gaussian=g)
+    assert (gf[~vis] == 0).all() and (go[~vis] == 0).all()
+    H.assert_close(gf.astype(np.float32), gf_ref.astype(np.float32), 2e-3, 1e-7, "SH gradients")
+    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+
+
+@pytest.mark.parametrize("mode", ["f16", "f32"])
+def test_backward_direct(gpu, oracle, mode):
+    n, tile, channels = 50000, 16, 4
+    hv, pos, feats, opac = scene(n, channels, seed=21)
+    fmode = _lib.FEAT_DIRECT_F16 if mode == "f16" else _lib.FEAT_DIRECT_F32
+    if mode == "f16":
+        feats = feats.astype(np.float16)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, channels, fmode).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, channels, fmode)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+    rng = np.random.default_rng(22)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                               gaussian=g)
+    if mode == "f16":
+        H.assert_close(gf.astype(np.float32), gf_ref.astype(np.float32), 2e-3, 1e-7, "feature gradients")
+    else:
+        H.assert_close(gf, gf_ref, RTOL, 1e-7, "feature gradients")
+    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+
+
+@pytest.mark.parametrize("with_scales", [False, True])
+@pytest.mark.parametrize("tile", [8, 16])
+def test_inference_preextracted(gpu, oracle, tile, with_scales):
+    n = 30000
+    hv, pos, _, opac = scene(n, 4, seed=31, near=0)
+    feats = synthetic.sh_features(n, 32)
+    scales = (np.random.default_rng(5).random(n) * 0.01).astype(np.float32) if with_scales else None
+    kw = dict(inference=True, scales=scales, sigma_world=0.006, sigma_cutoff=2.5)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_SH36_F16, **kw).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, 4, oracle.FEAT_SH36_F16, cam_position=hv.position, **kw)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(out["depth_image"], ref["depth_image"], RTOL, 1e-6, "depth image")
+
+
+def test_inference_raw37(gpu, oracle):
+    n, tile = 20000, 8
+    hv, pos, _, _ = scene(n, 4, seed=41, near=0)
+    rng = np.random.default_rng(42)
+    raw = np.concatenate([rng.normal(-1.0, 1.0, (n, 1)), synthetic.sh_features(n, 43).astype(np.float64)], axis=1)
+    raw = raw.astype(np.float16)
+    kw = dict(inference=True, sigma_world=0.004, sigma_cutoff=3.0)
+    run = H.GaussianRun(hv, pos, raw, None, tile, 4, _lib.FEAT_RAW37_F16, **kw).forward()
+    g, ref = oracle_run(oracle, hv, pos, raw, None, tile, 4, oracle.FEAT_RAW37_F16, cam_position=hv.position, **kw)
+    dbg = run.debug()
+    np.testing.assert_array_equal(dbg["instance_points"], ref["instance_points"])
+    vis = ref["n_touched"] > 0
+    H.assert_close(dbg["opacity"][vis], ref["opacity"][vis], RTOL, 1e-7, "activated opacity")
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], 2e-4, 1e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], 2e-4, 1e-6, "alpha")
+    H.assert_close(out["depth_image"], ref["depth_image"], 2e-4, 1e-5, "depth image")
+
+
+def test_edge_cases(gpu, oracle):
+    hv = synthetic.camera_on_z(64, 48, 60.0, 2.0)
+    # no points at all: background images
+    run = H.GaussianRun(hv, np.zeros((0, 3), np.float32), np.zeros((0, 4), np.float32), np.zeros(0, np.float32)).forward()
+    out = run.outputs()
+    assert (out["image"] == 0).all() and (out["alpha"] == 0).all()
+    # every point behind the camera
+    n = 1000
+    pos = synthetic.cube_points(n, 1.0, 1)
+    pos[:, 2] -= 10.0
+    feats, opac = synthetic.point_attributes(n, 4, "uniform", 2)
+    run = H.GaussianRun(hv, pos, feats, opac).forward()
+    _, counters = run.counters()
+    assert counters[:2] == [0, 0]
+    out = run.outputs()
+    assert (out["image"] == 0).all() and (out["alpha"] == 0).all() and (out["blending_weights"] == 0).all()
+    gf, go = run.backward(np.ones((4, 48, 64), np.float32), np.ones((1, 48, 64), np.float32))
+    assert (gf == 0).all() and (go == 0).all()
+    # a single point
+    one = np.array([[0.01, -0.02, 0.0]], np.float32)
+    run = H.GaussianRun(hv, one, np.ones((1, 4), np.float32), np.array([0.7], np.float32)).forward()
+    g, ref = oracle_run(oracle, hv, one, np.ones((1, 4), np.float32), np.array([0.7], np.float32), 8, 4)
+    np.testing.assert_array_equal(run.outputs()["image"].view(np.uint32), ref["image"].view(np.uint32))
+
+
+def test_instances_beyond_the_capacity_are_reported(gpu, oracle):
+    n = 5000
+    hv, pos, feats, opac = scene(n, 4, seed=51, near=500)
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, 8, 4)
+    need = ref["n_instances"]
+    small = H.GaussianRun(hv, pos, feats, opac, 8, 4, max_instances=need - 1).forward()
+    rc, counters = small.counters(check=False)
+    assert rc == -2 and counters[1] == need and counters[3] == 0      # INPC_E_WORKSPACE, nothing drawn
+    out = small.outputs()
+    assert (out["image"] == 0).all() and (out["alpha"] == 0).all()
+    exact = H.GaussianRun(hv, pos, feats, opac, 8, 4, max_instances=need).forward()
+    rc, counters = exact.counters()
+    assert counters[1] == need and counters[3] == need
+    np.testing.assert_array_equal(exact.outputs()["image"].view(np.uint32), ref["image"].view(np.uint32))
+
+
+def test_python_api(gpu, oracle):
+    from inpc_amd import INPCRasterizer, rasterize_points
+
+    n = 20000
+    hv = synthetic.rotated_camera(160, 120, 140.0, 2.5, 0.3, 0.1)
+    view = hv.to_view(gpu)
+    pos = synthetic.cube_points(n, 1.5, 61)
+    pos[:200] = near_camera_points(hv, 200, 5)
+    feats = synthetic.sh_features(n, 62)
+    _, opac = synthetic.point_attributes(n, 4, "normal", 63)
+    rasterizer = INPCRasterizer()
+    positions = H.dev(pos)
+    features = H.dev(feats).requires_grad_(True)
+    opacities = H.dev(opac.reshape(-1, 1)).requires_grad_(True)
+    image, alpha, weights = rasterizer(view, 1, positions, features, opacities)
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, 8, 4, oracle.FEAT_SH36_F16, cam_position=hv.position)
+    H.assert_close(image.detach().cpu().numpy(), ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(weights.cpu().numpy(), ref["blending_weights"], RTOL, 1e-7, "blending weights")
+    (image.sum() + alpha.sum()).backward()
+    ones_i, ones_a = np.ones_like(ref["image"]), np.ones_like(ref["alpha"])
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, ones_i, ones_a, image.detach().cpu().numpy(),
+                                               alpha.detach().cpu().numpy(), pos, feats, opac, hv.w2c, hv.position,
+                                               gaussian=g)
+    H.assert_close(features.grad.float().cpu().numpy(), gf_ref.astype(np.float32), 2e-3, 1e-6, "SH gradients")
+    H.assert_close(opacities.grad.cpu().numpy().reshape(-1), go_ref, RTOL, 1e-6, "opacity gradients")
+    # render_preextracted: sigma_world = scale * 0.05 / focal_y (B/torch_bindings/rasterization.py:130-134)
+    img2, depth2, alpha2 = rasterizer.render_preextracted(view, 1, positions, features.detach(), opacities.detach(),
+                                                          None, 2.0, 2.5)
+    g2, ref2 = oracle_run(oracle, hv, pos, feats, opac, 8, 4, oracle.FEAT_SH36_F16, inference=True,
+                          sigma_world=float(np.float32(2.0 * 0.05 / hv.camera.focal_y)), sigma_cutoff=2.5,
+                          cam_position=hv.position)
+    H.assert_close(img2.cpu().numpy(), ref2["image"], RTOL, 1e-5, "preextracted image")
+    H.assert_close(depth2.cpu().numpy(), ref2["depth_image"], RTOL, 1e-6, "preextracted depth")
+    # a second call with far more instances than the default buffers hold: the wrapper sizes them and goes again
+    pos_near = near_camera_points(hv, 10000, 9)
+    f8, o8 = synthetic.point_attributes(10000, 8, "normal", 64)
+    img8, alpha8, w8 = rasterize_points(view, H.dev(pos_near), H.dev(f8), H.dev(o8), tile=8, mode=1)
+    g8, ref8 = oracle_run(oracle, hv, pos_near, f8, o8, 8, 8)
+    assert ref8["n_instances"] > 4 * 10000 + 65536
+    np.testing.assert_array_equal(img8.cpu().numpy().view(np.uint32), ref8["image"].view(np.uint32))

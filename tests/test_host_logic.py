@@ -81,12 +81,14 @@ def test_base_sigma_world():
     assert INPCRasterizer.extract_base_sigma_world(PerspectiveCamera(8, 8, 100.0, 200.0, 4, 4)) == 0.05 / 200.0
 
 
-def test_gaussian_mode_is_refused_like_an_unknown_native_mode():
+def test_gaussian_mode_is_a_known_mode():
+    # both footprints get as far as the device check (B/torch_bindings/rasterization.py:15-18)
     r = INPCRasterizer()
     n = 4
     args = (torch.zeros(n, 3), torch.zeros(n, 36, dtype=torch.float16), torch.zeros(n))
-    with pytest.raises(RuntimeError, match="unsupported rasterizer mode"):
-        r(cpu_view(), RasterizerMode.GAUSSIAN.value, *args)
+    for mode in (RasterizerMode.BILINEAR.value, RasterizerMode.GAUSSIAN.value):
+        with pytest.raises(RuntimeError, match="expected tensors on the GPU"):
+            r(cpu_view(), mode, *args)
 
 
 def test_tile_argument():
