@@ -14,8 +14,9 @@
 //   radix sort          by tile key, stable (forward.cu:133-141)
 //   k_ranges            [begin, end) per tile (kernels.cu:382-399)
 //   k_blend_*           one block per tile, one thread per pixel, a wave owns an 8 x 8 pixel block; per batch of
-//                       T*T staged instances a wave first finds, 64 instances at a time, the ones whose footprint
-//                       reaches its pixel block and evaluates only those (kernels.cu:401-660)
+//                       T*T staged instances and 64 instances at a time, every lane first collects the instances
+//                       whose pixel box contains its pixel (a few integer operations each) and then evaluates only
+//                       those, each lane its own list in depth order (kernels.cu:401-660)
 #pragma once
 
 namespace gaussian {
@@ -311,6 +312,27 @@ __global__ void __launch_bounds__(kBlock) k_ranges(const uint16_t* __restrict__ 
 }
 
 // ---- blend -----------------------------------------------------------------------------------------------------------
+// An instance whose pixel box has at most kSlots pixels owns one slot per pixel of the box. The instance's own thread
+// fills the slots with the footprint values (0: pixel skipped) when the instance is staged, so that the per-pixel
+// walk, which is sequential where many points pile up on a few pixels, only has the blend itself left to do. A pixel
+// that has blended the instance replaces the value (positive) by minus its contribution (forward: G * blending
+// weight; backward: the blending weight, next to the opacity gradient in a second array); after the batch the
+// instance's thread adds up the negative slots, in slot order: no atomics.
+// Larger boxes (points close to the camera) are evaluated by the pixels and add to global memory directly.
+constexpr int kSlots = 9;
+constexpr int kSlotStride = kSlots;   // odd: rows of neighbouring instances spread over the LDS banks
+
+// Footprint value of a staged instance at the pixel centre (kernels.cu:447-452); false when the pixel is skipped.
+// Without branches, so that the values of several instances are computed side by side.
+__device__ __forceinline__ bool footprint_value(const float4 h0, const float4 h1, float cx, float cy, float threshold,
+                                                float& G) {
+    const float dx = h0.x - cx, dy = h0.y - cy;
+    const float exponent = -0.5f * (h0.w * dx * dx + h1.y * dy * dy) - h1.x * dx * dy;
+    const bool positive = exponent > 0.0f;
+    G = footprint_exp(positive ? 0.0f : exponent);   // a NaN exponent stays NaN and gives 0: skipped, as in the reference
+    return !positive && !(G < threshold);
+}
+
 // A staged instance: header words, features, and the pixel box (tile-local, conservative) its footprint can reach.
 template <int T, int C>
 struct Stage {
@@ -318,13 +340,14 @@ struct Stage {
     float4 head0[TT];   // sx, sy, opacity, conic.x
     float4 head1[TT];   // conic.y, conic.z, depth, point id | kMultiTile
     float4 feat[TT * (C / 4)];
-    uint32_t box[TT];   // bytes: first column, one past the last column, first row, one past the last row
+    uint32_t box[TT];   // bits 0-15: columns of the tile the footprint can reach, bits 16-31: rows
+    float value[TT][kSlotStride];   // footprint value per pixel of the box (boxes of at most kSlots pixels)
 };
 
 // Thread `slot` stages instance `slot` of the batch.
 template <int T, int C>
 __device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, const char* __restrict__ record,
-                                               int tile_x0, int tile_y0, float reach2) {
+                                               int tile_x0, int tile_y0, float reach2, float threshold) {
     const float4* src = (const float4*)record;
     const float4 h0 = src[0], h1 = src[1];
     st.head0[slot] = h0;
@@ -345,27 +368,35 @@ __device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, c
             y_hi = fminf(fmaxf(floorf(h0.y + ry - 0.5f) + 1.0f - (float)tile_y0, 0.0f), (float)T);
         }
     }
-    st.box[slot] = (uint32_t)x_lo | ((uint32_t)x_hi << 8) | ((uint32_t)y_lo << 16) | ((uint32_t)y_hi << 24);
+    // columns and rows of the tile as bit masks
+    const uint32_t cols = ((1u << (uint32_t)x_hi) - 1u) & ~((1u << (uint32_t)x_lo) - 1u);
+    const uint32_t rows = ((1u << (uint32_t)y_hi) - 1u) & ~((1u << (uint32_t)y_lo) - 1u);
+    st.box[slot] = cols | (rows << 16);
+    const int w = __popc(cols), h = __popc(rows);
+    if (w * h <= kSlots) {
+        const int px0 = tile_x0 + __ffs(cols) - 1, py0 = tile_y0 + __ffs(rows) - 1;
+        int k = 0;
+        for (int yy = 0; yy < h; ++yy) {
+            for (int xx = 0; xx < w; ++xx, ++k) {
+                float G;
+                const bool hit = footprint_value(h0, h1, (float)(px0 + xx) + 0.5f, (float)(py0 + yy) + 0.5f, threshold, G);
+                st.value[slot][k] = hit ? G : 0.0f;
+            }
+        }
+    }
 }
 
-// Does the box reach the 8 x 8 pixel block at (qx0, qy0)?
-__device__ __forceinline__ bool box_reaches(uint32_t box, int qx0, int qy0) {
-    const int x_lo = box & 0xFF, x_hi = (box >> 8) & 0xFF, y_lo = (box >> 16) & 0xFF, y_hi = box >> 24;
-    return x_lo < qx0 + 8 && x_hi > qx0 && y_lo < qy0 + 8 && y_hi > qy0;
-}
-
-// Footprint value of a staged instance at the pixel centre (kernels.cu:447-452); false when the pixel is skipped.
-__device__ __forceinline__ bool footprint_value(const float4 h0, const float4 h1, float cx, float cy, float threshold,
-                                                float& G) {
-    const float dx = h0.x - cx, dy = h0.y - cy;
-    const float exponent = -0.5f * (h0.w * dx * dx + h1.y * dy * dy) - h1.x * dx * dy;
-    if (exponent > 0.0f) return false;
-    G = footprint_exp(exponent);
-    return !(G < threshold);
+// Slot of tile-local pixel (lx, ly), which lies in the box; -1 when the box has no slots.
+__device__ __forceinline__ int slot_of(uint32_t box, int lx, int ly) {
+    const uint32_t cols = box & 0xFFFFu, rows = box >> 16;
+    const int w = __popc(cols), h = __popc(rows);
+    if (w * h > kSlots) return -1;
+    return (ly - (__ffs(rows) - 1)) * w + (lx - (__ffs(cols) - 1));
 }
 
 struct Pixel {
     int x, y;       // image coordinates
+    int lx, ly;     // tile-local coordinates
     int qx0, qy0;   // tile-local origin of the wave's pixel block
     bool inside;
 };
@@ -376,11 +407,34 @@ __device__ __forceinline__ Pixel pixel_of_thread(uint32_t tile, uint32_t gw, int
     Pixel p;
     p.qx0 = T == 16 ? (int)(wave & 1u) * 8 : 0;
     p.qy0 = T == 16 ? (int)(wave >> 1) * 8 : 0;
-    p.x = (int)(tile % gw) * T + p.qx0 + (int)(lane & 7u);
-    p.y = (int)(tile / gw) * T + p.qy0 + (int)(lane >> 3);
+    p.lx = p.qx0 + (int)(lane & 7u);
+    p.ly = p.qy0 + (int)(lane >> 3);
+    p.x = (int)(tile % gw) * T + p.lx;
+    p.y = (int)(tile / gw) * T + p.ly;
     p.inside = p.x < W && p.y < H;
     return p;
 }
+
+// Bits of a pixel in a box word, and of a wave's 8 x 8 pixel block.
+__device__ __forceinline__ uint32_t pixel_bits(const Pixel& p) { return (1u << p.lx) | (1u << (16 + p.ly)); }
+__device__ __forceinline__ bool box_reaches(uint32_t box, const Pixel& p) {
+    return (box & (0xFFu << p.qx0)) != 0u && (box & (0xFF0000u << p.qy0)) != 0u;
+}
+
+// Of the instances first + k, k a bit of `reach`, the ones whose box contains the pixel with bits `mine`.
+template <int T, int C>
+__device__ __forceinline__ uint64_t instances_over_pixel(const Stage<T, C>& st, uint32_t first, uint64_t reach, uint32_t mine) {
+    uint64_t over = 0ull;
+    for (uint64_t t = reach; t; t &= t - 1ull) {
+        const uint32_t k = (uint32_t)__builtin_ctzll(t);
+        if ((st.box[first + k] & mine) == mine) over |= 1ull << k;
+    }
+    return over;
+}
+
+#ifdef INPC_GS_PROFILE
+__device__ unsigned long long g_gs_profile[65536 * 4];
+#endif
 
 template <int T, int C, bool INFERENCE>
 __global__ void __launch_bounds__(T * T)
@@ -390,40 +444,60 @@ __global__ void __launch_bounds__(T * T)
                     float* __restrict__ depth_image, int W, int H, uint32_t gw, float threshold, float reach2) {
     constexpr int TT = T * T;
     __shared__ Stage<T, C> st;
-    __shared__ float s_weight[TT];   // per staged instance: sum over the tile's pixels of G * blending weight
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t tile = order[blockIdx.x];
     const Pixel px = pixel_of_thread<T>(tile, gw, W, H);
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     const float cx = (float)px.x + 0.5f, cy = (float)px.y + 0.5f;
+    const uint32_t mine = pixel_bits(px);
     float acc[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) acc[c] = 0.0f;
     float depth_acc = 0.0f, tr = 1.0f;
     bool done = !px.inside;
     const uint2 range = ranges[tile];
+#ifdef INPC_GS_PROFILE
+    const unsigned long long prof_t0 = wall_clock64();
+    unsigned long long prof_iters = 0, prof_batches = 0;
+#endif
     for (uint32_t base = range.x; base < range.y; base += TT) {
         if (__syncthreads_count(done) == TT) break;
+#ifdef INPC_GS_PROFILE
+        ++prof_batches;
+#endif
         const uint32_t count = min((uint32_t)TT, range.y - base);
         if (tid < count) {
-            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2);
-            if (!INFERENCE) s_weight[tid] = 0.0f;
+            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2, threshold);
         }
         __syncthreads();
         if (__ballot(!done) != 0ull) {
             for (uint32_t first = 0; first < count; first += 64u) {
-                const uint32_t mine = first + lane;
-                uint64_t todo = __ballot(mine < count && box_reaches(st.box[mine], px.qx0, px.qy0));
-                while (todo) {
-                    const uint32_t j = first + (uint32_t)__builtin_ctzll(todo);
-                    todo &= todo - 1ull;
-                    if (done) continue;
-                    const float4 h0 = st.head0[j], h1 = st.head1[j];
+                const uint32_t at = first + lane;
+                const uint64_t reach = __ballot(at < count && box_reaches(st.box[at], px));
+                uint64_t over = instances_over_pixel<T, C>(st, first, reach, mine);
+                if (done) over = 0ull;
+                while (__ballot(over != 0ull) != 0ull) {
+#ifdef INPC_GS_PROFILE
+                    ++prof_iters;
+#endif
+                    if (over == 0ull) continue;
+                    const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
+                    over &= over - 1ull;
+                    const int slot = slot_of(st.box[j], px.lx, px.ly);
                     float G;
-                    if (!footprint_value(h0, h1, cx, cy, threshold, G)) continue;
-                    const float a = h0.z * G;
+                    if (slot >= 0) {
+                        G = st.value[j][slot];
+                        if (G == 0.0f) continue;
+                    } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
+                        continue;
+                    }
+                    const float a = st.head0[j].z * G;
                     const float bw = tr * a;
-                    if (!INFERENCE && bw > 0.0f) atomicAdd(&s_weight[j], G * bw);
+                    if (!INFERENCE) {
+                        const float part = bw > 0.0f ? G * bw : 0.0f;
+                        if (slot >= 0) st.value[j][slot] = -part;
+                        else if (part != 0.0f) atomicAdd(&blending_weights[__float_as_uint(st.head1[j].w) & kPointMask], part);
+                    }
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q) {
                         const float4 f = st.feat[j * (C / 4) + q];
@@ -432,16 +506,28 @@ __global__ void __launch_bounds__(T * T)
                         acc[4 * q + 2] += bw * f.z;
                         acc[4 * q + 3] += bw * f.w;
                     }
-                    if (INFERENCE) depth_acc += bw * h1.z;
+                    if (INFERENCE) depth_acc += bw * st.head1[j].z;
                     tr *= 1.0f - a;
-                    if (tr < kTransmittanceThreshold) done = true;
+                    if (tr < kTransmittanceThreshold) {
+                        done = true;
+                        over = 0ull;
+                    }
                 }
             }
         }
         if (!INFERENCE) {
             __syncthreads();
             if (tid < count) {
-                const float w = s_weight[tid];
+                float w = 0.0f;
+                const uint32_t box = st.box[tid];
+                const int used = __popc(box & 0xFFFFu) * __popc(box >> 16);
+                if (used <= kSlots) {
+#pragma unroll
+                    for (int k = 0; k < kSlots; ++k) {
+                        const float v = st.value[tid][k];
+                        if (k < used && v < 0.0f) w -= v;   // slots no pixel has blended still hold the footprint value
+                    }
+                }
                 if (w != 0.0f) {
                     const uint32_t word = __float_as_uint(st.head1[tid].w);
                     if (word & kMultiTile) atomicAdd(&blending_weights[word & kPointMask], w);
@@ -450,6 +536,19 @@ __global__ void __launch_bounds__(T * T)
             }
         }
     }
+#ifdef INPC_GS_PROFILE
+    if (lane == 0) {
+        unsigned long long* out = g_gs_profile + (size_t)blockIdx.x * 4;
+        if (tid == 0) {
+            out[0] = wall_clock64() - prof_t0;
+            out[1] = range.y - range.x;
+            out[2] = prof_batches;
+            out[3] = 0;
+        }
+        __threadfence();
+        atomicMax(&out[3], prof_iters);
+    }
+#endif
     if (px.inside) {
         const size_t n_pixels = (size_t)W * H, pix = (size_t)px.y * W + px.x;
 #pragma unroll
@@ -460,9 +559,10 @@ __global__ void __launch_bounds__(T * T)
     }
 }
 
-// Backward: the same walk with the saved final image (kernels.cu:476-579). Per staged instance the tile's
-// contributions are summed in LDS and leave the block once: a plain store for a point with a single instance,
-// float atomics for the others.
+// Backward: the same walk with the saved final image (kernels.cu:476-579). A pixel leaves its blending weight and
+// opacity gradient in the instance's slot; after the batch the instance's thread multiplies the weights with the
+// pixels' image gradients (kept in LDS) and adds everything up: a plain store for a point with a single
+// instance, float atomics for the others.
 template <int T, int C>
 __global__ void __launch_bounds__(T * T)
     k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ order,
@@ -472,12 +572,14 @@ __global__ void __launch_bounds__(T * T)
                      float* grad_opacities, int W, int H, uint32_t gw, float threshold, float reach2) {
     constexpr int TT = T * T;
     __shared__ Stage<T, C> st;
-    __shared__ float s_grad[TT][C + 1];   // per staged instance: feature gradient, opacity gradient
+    __shared__ float s_d_opacity[TT][kSlotStride];   // per staged instance and box pixel: d loss / d opacity
+    __shared__ float s_grad_px[TT][C + 1];       // image gradient of every pixel of the tile (padded rows)
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t tile = order[blockIdx.x];
     const Pixel px = pixel_of_thread<T>(tile, gw, W, H);
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     const float cx = (float)px.x + 0.5f, cy = (float)px.y + 0.5f;
+    const uint32_t mine = pixel_bits(px);
     float g[C], final_px[C], fresh[C];
     float common = 0.0f;
 #pragma unroll
@@ -491,6 +593,8 @@ __global__ void __launch_bounds__(T * T)
         }
         common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
     }
+#pragma unroll
+    for (int c = 0; c < C; ++c) s_grad_px[px.ly * T + px.lx][c] = g[c];
     float tr = 1.0f;
     bool done = !px.inside;
     const uint2 range = ranges[tile];
@@ -498,23 +602,28 @@ __global__ void __launch_bounds__(T * T)
         if (__syncthreads_count(done) == TT) break;
         const uint32_t count = min((uint32_t)TT, range.y - base);
         if (tid < count) {
-            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2);
-#pragma unroll
-            for (int c = 0; c <= C; ++c) s_grad[tid][c] = 0.0f;
+            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2, threshold);
         }
         __syncthreads();
         if (__ballot(!done) != 0ull) {
             for (uint32_t first = 0; first < count; first += 64u) {
-                const uint32_t mine = first + lane;
-                uint64_t todo = __ballot(mine < count && box_reaches(st.box[mine], px.qx0, px.qy0));
-                while (todo) {
-                    const uint32_t j = first + (uint32_t)__builtin_ctzll(todo);
-                    todo &= todo - 1ull;
-                    if (done) continue;
-                    const float4 h0 = st.head0[j], h1 = st.head1[j];
+                const uint32_t at = first + lane;
+                const uint64_t reach = __ballot(at < count && box_reaches(st.box[at], px));
+                uint64_t over = instances_over_pixel<T, C>(st, first, reach, mine);
+                if (done) over = 0ull;
+                while (__ballot(over != 0ull) != 0ull) {
+                    if (over == 0ull) continue;
+                    const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
+                    over &= over - 1ull;
+                    const int slot = slot_of(st.box[j], px.lx, px.ly);
                     float G;
-                    if (!footprint_value(h0, h1, cx, cy, threshold, G)) continue;
-                    const float a = h0.z * G;
+                    if (slot >= 0) {
+                        G = st.value[j][slot];
+                        if (G == 0.0f) continue;
+                    } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
+                        continue;
+                    }
+                    const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     const float one_minus_a = 1.0f - a;
                     const float rcp = 1.0f / fmaxf(one_minus_a, kOneMinusAlphaEps);
@@ -524,36 +633,69 @@ __global__ void __launch_bounds__(T * T)
                         const float4 f4 = st.feat[j * (C / 4) + q];
                         const float f[4] = {f4.x, f4.y, f4.z, f4.w};
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            const int c = 4 * q + k;
-                            if (bw > 0.0f) atomicAdd(&s_grad[j][c], bw * g[c]);
-                            fresh[c] += bw * f[k];
-                            const float term = (tr * f[k] + (fresh[c] - final_px[c]) * rcp) * g[c];
+                        for (int e = 0; e < 4; ++e) {
+                            const int c = 4 * q + e;
+                            fresh[c] += bw * f[e];
+                            const float term = (tr * f[e] + (fresh[c] - final_px[c]) * rcp) * g[c];
                             dot = c == 0 ? term : dot + term;
                         }
                     }
                     const float d_alpha = dot + common * rcp;
                     const float d_opacity = d_alpha * G;
-                    if (d_opacity != 0.0f) atomicAdd(&s_grad[j][C], d_opacity);
+                    const float weight = bw > 0.0f ? bw : 0.0f;
+                    if (slot >= 0) {
+                        st.value[j][slot] = -weight;
+                        s_d_opacity[j][slot] = d_opacity;
+                    } else {
+                        const uint32_t point = __float_as_uint(st.head1[j].w) & kPointMask;
+                        if (weight > 0.0f) {
+#pragma unroll
+                            for (int c = 0; c < C; ++c) atomicAdd(&grad_features[(size_t)point * C + c], weight * g[c]);
+                        }
+                        if (d_opacity != 0.0f) atomicAdd(&grad_opacities[point], d_opacity);
+                    }
                     tr *= one_minus_a;
-                    if (tr < kTransmittanceThreshold) done = true;
+                    if (tr < kTransmittanceThreshold) {
+                        done = true;
+                        over = 0ull;
+                    }
                 }
             }
         }
         __syncthreads();
         if (tid < count) {
-            const uint32_t word = __float_as_uint(st.head1[tid].w);
-            const uint32_t point = word & kPointMask;
-            float* gf = grad_features + (size_t)point * C;
-            if (word & kMultiTile) {
+            const uint32_t box = st.box[tid];
+            const uint32_t cols = box & 0xFFFFu, rows = box >> 16;
+            const int w = __popc(cols), h = __popc(rows), x_lo = __ffs(cols) - 1, y_lo = __ffs(rows) - 1;
+            if (w * h <= kSlots && w * h > 0) {
+                float sum[C + 1];
 #pragma unroll
-                for (int c = 0; c < C; ++c)
-                    if (s_grad[tid][c] != 0.0f) atomicAdd(&gf[c], s_grad[tid][c]);
-                if (s_grad[tid][C] != 0.0f) atomicAdd(&grad_opacities[point], s_grad[tid][C]);
-            } else {
+                for (int c = 0; c <= C; ++c) sum[c] = 0.0f;
+                int slot = 0;
+                for (int yy = 0; yy < h; ++yy) {
+                    for (int xx = 0; xx < w; ++xx, ++slot) {
+                        const float v = st.value[tid][slot];
+                        if (!(__float_as_uint(v) >> 31)) continue;   // no pixel has blended it: still the footprint value
+                        const float weight = -v;
+                        const float* gp = s_grad_px[(y_lo + yy) * T + x_lo + xx];
 #pragma unroll
-                for (int c = 0; c < C; ++c) gf[c] = s_grad[tid][c];
-                grad_opacities[point] = s_grad[tid][C];
+                        for (int c = 0; c < C; ++c) sum[c] += weight * gp[c];
+                        sum[C] += s_d_opacity[tid][slot];
+                    }
+                }
+                const uint32_t word = __float_as_uint(st.head1[tid].w);
+                const uint32_t point = word & kPointMask;
+                float* gf = grad_features + (size_t)point * C;
+                if (word & kMultiTile) {
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                        if (sum[c] != 0.0f) atomicAdd(&gf[c], sum[c]);
+                    if (sum[C] != 0.0f) atomicAdd(&grad_opacities[point], sum[C]);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < C; ++c) gf[c] = sum[c];
+                    grad_opacities[point] = sum[C];
+                }
             }
         }
     }
