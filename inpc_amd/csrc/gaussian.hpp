@@ -67,6 +67,11 @@ __global__ void __launch_bounds__(kBlock)
                  uint2* __restrict__ bounds_out, uint32_t* __restrict__ keys, uint32_t* __restrict__ vals,
                  float* __restrict__ blending_weights, uint32_t* counters, uint32_t* g_hist, Geometry g, Params prm,
                  float tile_edge, radix::DevicePlan plan) {
+    // A record leaves the block through LDS: every lane assembles its record in the wave's staging rows, then the
+    // wave writes its 64 records, which are neighbours in memory, as one contiguous run of 16-byte words (a lane
+    // storing its own record would put 16 bytes into each of 64 different lines per instruction).
+    constexpr uint32_t kWords = (32u + 4u * C + 31u) / 32u * 2u, kRow = kWords + 1u;   // 16-byte words per record; padded row
+    __shared__ float4 s_stage[kBlock * kRow];
     __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
     __shared__ uint32_t s_visible;
     __shared__ unsigned long long s_instances;
@@ -76,11 +81,19 @@ __global__ void __launch_bounds__(kBlock)
         s_instances = 0ull;
     }
     __syncthreads();
-    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u;
+    float4* stage = s_stage + (threadIdx.x >> 6) * (64u * kRow);
+    const ViewRows m = load_view_rows(w2c);
+    uint32_t my_visible = 0u;
+    unsigned long long my_instances = 0ull;
+    // the grid is a few blocks per CU and walks over the points: histograms and counts leave a block once
+    for (uint32_t first = blockIdx.x * kBlock; first < g.n; first += gridDim.x * kBlock) {
+    const uint32_t i = first + threadIdx.x;
+#pragma unroll
+    for (uint32_t w = 0; w < kWords; ++w) stage[lane * kRow + w] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     uint32_t touched = 0u;
     if (i < g.n) {
         uint32_t key = radix::kInvalidKey;
-        const ViewRows m = load_view_rows(w2c);
         const float px = positions[3 * (size_t)i], py = positions[3 * (size_t)i + 1], pz = positions[3 * (size_t)i + 2];
         const float depth = affine_row(m.r3, px, py, pz);
         if (!(depth < g.cam.near_plane || depth > g.cam.far_plane)) {
@@ -114,7 +127,7 @@ __global__ void __launch_bounds__(kBlock)
                     touched = (x1 - x0) * (y1 - y0);
                     bounds_out[i] = make_uint2(x0 | (x1 << 16), y0 | (y1 << 16));
                     float opacity = FMODE == INPC_FEAT_RAW37_F16 ? 0.0f : opacities[i];
-                    float4* rec = (float4*)(records + (size_t)i * g.stride);
+                    float4* rec = stage + lane * kRow;
                     if (FMODE == INPC_FEAT_DIRECT_F32) {
                         const float4* src = (const float4*)features + (size_t)i * (C / 4);
 #pragma unroll
@@ -147,12 +160,27 @@ __global__ void __launch_bounds__(kBlock)
         vals[i] = i;
         if (blending_weights) blending_weights[i] = 0.0f;
     }
-    const uint32_t visible = (uint32_t)__popcll(__ballot(touched != 0u));
-    uint32_t sum = touched;
-    for (int s = 32; s > 0; s >>= 1) sum += __shfl_down(sum, s, 64);
+    wave_sync();
+    {
+        const uint32_t wave_first = i - lane;   // first point of this wave
+        float4* out = (float4*)(records + (size_t)wave_first * g.stride);
+#pragma unroll
+        for (uint32_t k = 0; k < kWords; ++k) {
+            const uint32_t flat = k * 64u + lane, r = flat / kWords, w = flat % kWords;
+            if (wave_first + r < g.n) out[flat] = stage[r * kRow + w];
+        }
+    }
+    wave_sync();   // the staging rows are reused by the next round
+    my_visible += touched != 0u ? 1u : 0u;
+    my_instances += touched;
+    }
+    for (int s = 32; s > 0; s >>= 1) {
+        my_visible += __shfl_down(my_visible, s, 64);
+        my_instances += __shfl_down(my_instances, s, 64);
+    }
     if ((threadIdx.x & 63u) == 0u) {
-        if (visible) atomicAdd(&s_visible, visible);
-        if (sum) atomicAdd(&s_instances, (unsigned long long)sum);
+        if (my_visible) atomicAdd(&s_visible, my_visible);
+        if (my_instances) atomicAdd(&s_instances, my_instances);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -162,17 +190,28 @@ __global__ void __launch_bounds__(kBlock)
     radix::hist_flush(s_hist, plan, g_hist);
 }
 
-// ---- instance offsets: exclusive prefix of touched[order[j]] (kernels.cu:346-356, forward.cu:110-116) ------------
+// ---- instance offsets: exclusive prefix of the touched-tile counts in depth order (kernels.cu:346-356,
+// forward.cu:110-116). The tile bounds are gathered once, here, and kept in depth order for k_create_instances;
+// the count follows from them.
+__device__ __forceinline__ uint32_t tiles_of(uint2 b) {
+    return ((b.x >> 16) - (b.x & 0xFFFFu)) * ((b.y >> 16) - (b.y & 0xFFFFu));
+}
+
 __global__ void __launch_bounds__(kBlock)
-    k_touch_sums(const uint32_t* __restrict__ order, const uint32_t* __restrict__ touched,
-                 const uint32_t* __restrict__ counters, uint32_t* __restrict__ block_sums) {
+    k_touch_sums(const uint32_t* __restrict__ order, const uint2* __restrict__ bounds,
+                 const uint32_t* __restrict__ counters, uint2* __restrict__ sorted_bounds,
+                 uint32_t* __restrict__ block_sums) {
     __shared__ uint32_t s_wave[kBlock / kWave];
     const uint32_t n_visible = counters[kCntVisible];
     const uint32_t base = blockIdx.x * kPointsPerBlock;
     uint32_t sum = 0;
     for (uint32_t k = threadIdx.x; k < (uint32_t)kPointsPerBlock; k += kBlock) {
         const uint32_t j = base + k;
-        if (j < n_visible) sum += touched[order[j]];
+        if (j < n_visible) {
+            const uint2 b = bounds[order[j]];
+            sorted_bounds[j] = b;
+            sum += tiles_of(b);
+        }
     }
     for (int s = 32; s > 0; s >>= 1) sum += __shfl_down(sum, s, 64);
     if ((threadIdx.x & 63u) == 0u) s_wave[threadIdx.x >> 6] = sum;
@@ -224,8 +263,8 @@ __global__ void __launch_bounds__(kScanBlock) k_touch_scan(uint32_t* __restrict_
 // Instances of the block's 1024 depth-ordered points, in depth order, row-major over each point's tiles
 // (kernels.cu:358-380). Output slot s of the block belongs to the last point whose offset is <= s.
 __global__ void __launch_bounds__(kBlock)
-    k_create_instances(const uint32_t* __restrict__ order, const uint32_t* __restrict__ touched,
-                       const uint2* __restrict__ bounds, const uint32_t* __restrict__ block_base,
+    k_create_instances(const uint32_t* __restrict__ order, const uint2* __restrict__ sorted_bounds,
+                       const uint32_t* __restrict__ block_base,
                        const uint32_t* __restrict__ counters, uint16_t* __restrict__ inst_keys,
                        uint32_t* __restrict__ inst_points, uint32_t* g_hist, uint32_t gw, radix::DevicePlan plan) {
     constexpr int kPer = kPointsPerBlock / kBlock;   // consecutive points per thread
@@ -246,10 +285,10 @@ __global__ void __launch_bounds__(kBlock)
         const uint32_t k = tid * kPer + u, j = base + k;
         count[u] = 0u;
         if (j < n_visible) {
-            const uint32_t p = order[j];
-            count[u] = touched[p];
-            s_point[k] = p;
-            s_bounds[k] = bounds[p];
+            const uint2 b = sorted_bounds[j];
+            count[u] = tiles_of(b);
+            s_point[k] = order[j];
+            s_bounds[k] = b;
         }
         mine += count[u];
     }
@@ -386,6 +425,8 @@ __device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, c
     }
 }
 
+__device__ __forceinline__ bool has_slots(uint32_t box) { return __popc(box & 0xFFFFu) * __popc(box >> 16) <= kSlots; }
+
 // Slot of tile-local pixel (lx, ly), which lies in the box; -1 when the box has no slots.
 __device__ __forceinline__ int slot_of(uint32_t box, int lx, int ly) {
     const uint32_t cols = box & 0xFFFFu, rows = box >> 16;
@@ -473,24 +514,13 @@ __global__ void __launch_bounds__(T * T)
         if (__ballot(!done) != 0ull) {
             for (uint32_t first = 0; first < count; first += 64u) {
                 const uint32_t at = first + lane;
-                const uint64_t reach = __ballot(at < count && box_reaches(st.box[at], px));
+                const uint32_t my_box = at < count ? st.box[at] : 0u;
+                const uint64_t reach = __ballot(box_reaches(my_box, px));
+                const bool all_slots = __ballot(box_reaches(my_box, px) && !has_slots(my_box)) == 0ull;
                 uint64_t over = instances_over_pixel<T, C>(st, first, reach, mine);
                 if (done) over = 0ull;
-                while (__ballot(over != 0ull) != 0ull) {
-#ifdef INPC_GS_PROFILE
-                    ++prof_iters;
-#endif
-                    if (over == 0ull) continue;
-                    const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
-                    over &= over - 1ull;
-                    const int slot = slot_of(st.box[j], px.lx, px.ly);
-                    float G;
-                    if (slot >= 0) {
-                        G = st.value[j][slot];
-                        if (G == 0.0f) continue;
-                    } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
-                        continue;
-                    }
+                // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
+                auto blend = [&](uint32_t j, int slot, float G) {
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     if (!INFERENCE) {
@@ -511,6 +541,35 @@ __global__ void __launch_bounds__(T * T)
                     if (tr < kTransmittanceThreshold) {
                         done = true;
                         over = 0ull;
+                    }
+                };
+                if (all_slots) {   // the usual case, without the branches of the other one
+                    while (__ballot(over != 0ull) != 0ull) {
+#ifdef INPC_GS_PROFILE
+                        ++prof_iters;
+#endif
+                        if (over != 0ull) {
+                            const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
+                            over &= over - 1ull;
+                            const int slot = slot_of(st.box[j], px.lx, px.ly);
+                            const float G = st.value[j][slot];
+                            if (G != 0.0f) blend(j, slot, G);
+                        }
+                    }
+                } else {
+                    while (__ballot(over != 0ull) != 0ull) {
+                        if (over == 0ull) continue;
+                        const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
+                        over &= over - 1ull;
+                        const int slot = slot_of(st.box[j], px.lx, px.ly);
+                        float G;
+                        if (slot >= 0) {
+                            G = st.value[j][slot];
+                            if (G == 0.0f) continue;
+                        } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
+                            continue;
+                        }
+                        blend(j, slot, G);
                     }
                 }
             }
@@ -608,21 +667,13 @@ __global__ void __launch_bounds__(T * T)
         if (__ballot(!done) != 0ull) {
             for (uint32_t first = 0; first < count; first += 64u) {
                 const uint32_t at = first + lane;
-                const uint64_t reach = __ballot(at < count && box_reaches(st.box[at], px));
+                const uint32_t my_box = at < count ? st.box[at] : 0u;
+                const uint64_t reach = __ballot(box_reaches(my_box, px));
+                const bool all_slots = __ballot(box_reaches(my_box, px) && !has_slots(my_box)) == 0ull;
                 uint64_t over = instances_over_pixel<T, C>(st, first, reach, mine);
                 if (done) over = 0ull;
-                while (__ballot(over != 0ull) != 0ull) {
-                    if (over == 0ull) continue;
-                    const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
-                    over &= over - 1ull;
-                    const int slot = slot_of(st.box[j], px.lx, px.ly);
-                    float G;
-                    if (slot >= 0) {
-                        G = st.value[j][slot];
-                        if (G == 0.0f) continue;
-                    } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
-                        continue;
-                    }
+                // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
+                auto blend = [&](uint32_t j, int slot, float G) {
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     const float one_minus_a = 1.0f - a;
@@ -658,6 +709,32 @@ __global__ void __launch_bounds__(T * T)
                     if (tr < kTransmittanceThreshold) {
                         done = true;
                         over = 0ull;
+                    }
+                };
+                if (all_slots) {   // the usual case, without the branches of the other one
+                    while (__ballot(over != 0ull) != 0ull) {
+                        if (over != 0ull) {
+                            const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
+                            over &= over - 1ull;
+                            const int slot = slot_of(st.box[j], px.lx, px.ly);
+                            const float G = st.value[j][slot];
+                            if (G != 0.0f) blend(j, slot, G);
+                        }
+                    }
+                } else {
+                    while (__ballot(over != 0ull) != 0ull) {
+                        if (over == 0ull) continue;
+                        const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
+                        over &= over - 1ull;
+                        const int slot = slot_of(st.box[j], px.lx, px.ly);
+                        float G;
+                        if (slot >= 0) {
+                            G = st.value[j][slot];
+                            if (G == 0.0f) continue;
+                        } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
+                            continue;
+                        }
+                        blend(j, slot, G);
                     }
                 }
             }

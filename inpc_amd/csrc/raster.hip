@@ -909,6 +909,7 @@ struct GaussianLayout {
     uint32_t n_blocks;  // blocks of gaussian::kPointsPerBlock depth-ordered points
     size_t zero_begin, zero_words;
     size_t hist_depth, hist_tile, status_depth, status_tile, bases_depth, bases_tile, tile_order, block_sums;
+    size_t sorted_bounds;
     size_t keys_a, keys_b, vals_a, vals_b, inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
 };
 
@@ -991,6 +992,7 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
     L.block_sums = take((size_t)L.n_blocks * 4);
     P.point_touched = take(n * 4);
     P.point_bounds = take(n * 8);
+    L.sorted_bounds = take(n * 8);
     P.point_record = take(n * g.stride);
     L.keys_a = take(n * 4);
     L.keys_b = take(n * 4);
@@ -1020,7 +1022,7 @@ template <int FMODE, int C>
 int launch_gaussian_preprocess(const GaussianLayout& L, const float* positions, const void* features,
                                const float* opacities, const float* scales, const float* w2c, const float* cam_position,
                                float* blending_weights, void* ws, hipStream_t stream) {
-    INPC_LAUNCH("gaussian_preprocess", (gaussian::k_preprocess<FMODE, C>), dim3(div_up(L.geo.n, kBlock)), dim3(kBlock),
+    INPC_LAUNCH("gaussian_preprocess", (gaussian::k_preprocess<FMODE, C>), dim3(std::min(div_up(L.geo.n, kBlock), 2048u)), dim3(kBlock),
                 stream, positions, features, opacities, scales, w2c, cam_position, at<char>(ws, L.pub.point_record),
                 at<uint32_t>(ws, L.pub.point_touched), at<uint2>(ws, L.pub.point_bounds), at<uint32_t>(ws, L.keys_a),
                 at<uint32_t>(ws, L.vals_a), blending_weights, at<uint32_t>(ws, L.pub.counters),
@@ -1331,13 +1333,13 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
                                          "gaussian_depth_sort");
         if (rc != INPC_OK) return rc;
         const uint32_t* order = at<uint32_t>(ws, L.pub.depth_order);
-        const uint32_t* touched = at<uint32_t>(ws, L.pub.point_touched);
-        INPC_LAUNCH("gaussian_touch_sums", gaussian::k_touch_sums, dim3(L.n_blocks), dim3(kBlock), stream, order, touched,
-                    (const uint32_t*)counters, at<uint32_t>(ws, L.block_sums));
+        INPC_LAUNCH("gaussian_touch_sums", gaussian::k_touch_sums, dim3(L.n_blocks), dim3(kBlock), stream, order,
+                    (const uint2*)at<uint2>(ws, L.pub.point_bounds), (const uint32_t*)counters,
+                    at<uint2>(ws, L.sorted_bounds), at<uint32_t>(ws, L.block_sums));
         INPC_LAUNCH("gaussian_touch_scan", gaussian::k_touch_scan, dim3(1), dim3(kScanBlock), stream,
                     at<uint32_t>(ws, L.block_sums), L.n_blocks, counters, L.prm.capacity);
         INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(L.n_blocks), dim3(kBlock), stream,
-                    order, touched, (const uint2*)at<uint2>(ws, L.pub.point_bounds),
+                    order, (const uint2*)at<uint2>(ws, L.sorted_bounds),
                     (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,
                     at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), at<uint32_t>(ws, L.hist_tile),
                     L.geo.gw, radix::to_device_plan(L.tile_plan));
