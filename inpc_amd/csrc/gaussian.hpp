@@ -462,15 +462,30 @@ __device__ __forceinline__ bool box_reaches(uint32_t box, const Pixel& p) {
     return (box & (0xFFu << p.qx0)) != 0u && (box & (0xFF0000u << p.qy0)) != 0u;
 }
 
-// Of the instances first + k, k a bit of `reach`, the ones whose box contains the pixel with bits `mine`.
-template <int T, int C>
-__device__ __forceinline__ uint64_t instances_over_pixel(const Stage<T, C>& st, uint32_t first, uint64_t reach, uint32_t mine) {
-    uint64_t over = 0ull;
-    for (uint64_t t = reach; t; t &= t - 1ull) {
-        const uint32_t k = (uint32_t)__builtin_ctzll(t);
-        if ((st.box[first + k] & mine) == mine) over |= 1ull << k;
+// Lane k holds row k of a 64 x 64 bit matrix; afterwards lane k holds column k (bit p of the result = bit k of lane
+// p's input). Six exchange steps: in step j the two off-diagonal j x j blocks of every 2j x 2j block change places.
+__device__ __forceinline__ uint64_t wave_transpose_bits(uint64_t x) {
+    const uint32_t lane = lane_id();
+    uint64_t keep = 0x00000000FFFFFFFFull;   // bit positions p with (p & j) == 0
+#pragma unroll
+    for (int j = 32; j > 0; j >>= 1) {
+        const uint64_t other = __shfl_xor((unsigned long long)x, j, 64);
+        x = (lane & (uint32_t)j) == 0u ? (x & keep) | ((other & keep) << j) : (x & ~keep) | ((other & ~keep) >> j);
+        keep ^= keep << (j >> 1);
     }
-    return over;
+    return x;
+}
+
+// Per lane: of the instances first + k (lane k looks at instance first + k, `box` is its box word, 0 for none), the
+// ones whose box contains this lane's pixel, as a bit mask over k. Every lane marks the pixels of the wave's 8 x 8
+// block that its instance's box covers (lane l owns pixel l of the block), and a bit transpose hands every pixel its
+// column.
+__device__ __forceinline__ uint64_t instances_over_pixel(uint32_t box, const Pixel& p) {
+    const uint32_t cols = (box >> p.qx0) & 0xFFu, rows = (box >> (16 + p.qy0)) & 0xFFu;
+    // byte r of a half = cols when row r is in the box: the row bits spread to one per byte, times cols
+    const uint32_t lo = (((rows & 15u) * 0x00204081u) & 0x01010101u) * cols;
+    const uint32_t hi = (((rows >> 4) * 0x00204081u) & 0x01010101u) * cols;
+    return wave_transpose_bits((uint64_t)lo | ((uint64_t)hi << 32));
 }
 
 #ifdef INPC_GS_PROFILE
@@ -517,7 +532,7 @@ __global__ void __launch_bounds__(T * T)
                 const uint32_t my_box = at < count ? st.box[at] : 0u;
                 const uint64_t reach = __ballot(box_reaches(my_box, px));
                 const bool all_slots = __ballot(box_reaches(my_box, px) && !has_slots(my_box)) == 0ull;
-                uint64_t over = instances_over_pixel<T, C>(st, first, reach, mine);
+                uint64_t over = reach != 0ull ? instances_over_pixel(my_box, px) : 0ull;
                 if (done) over = 0ull;
                 // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
                 auto blend = [&](uint32_t j, int slot, float G) {
@@ -670,7 +685,7 @@ __global__ void __launch_bounds__(T * T)
                 const uint32_t my_box = at < count ? st.box[at] : 0u;
                 const uint64_t reach = __ballot(box_reaches(my_box, px));
                 const bool all_slots = __ballot(box_reaches(my_box, px) && !has_slots(my_box)) == 0ull;
-                uint64_t over = instances_over_pixel<T, C>(st, first, reach, mine);
+                uint64_t over = reach != 0ull ? instances_over_pixel(my_box, px) : 0ull;
                 if (done) over = 0ull;
                 // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
                 auto blend = [&](uint32_t j, int slot, float G) {
