@@ -266,7 +266,8 @@ __global__ void __launch_bounds__(kBlock)
     k_create_instances(const uint32_t* __restrict__ order, const uint2* __restrict__ sorted_bounds,
                        const uint32_t* __restrict__ block_base,
                        const uint32_t* __restrict__ counters, uint16_t* __restrict__ inst_keys,
-                       uint32_t* __restrict__ inst_points, uint32_t* g_hist, uint32_t gw, radix::DevicePlan plan) {
+                       uint32_t* __restrict__ inst_points, uint32_t* __restrict__ sorted_first,
+                       uint32_t* __restrict__ point_first, uint32_t* g_hist, uint32_t gw, radix::DevicePlan plan) {
     constexpr int kPer = kPointsPerBlock / kBlock;   // consecutive points per thread
     __shared__ uint32_t s_offset[kPointsPerBlock + 1];
     __shared__ uint32_t s_point[kPointsPerBlock];
@@ -311,6 +312,18 @@ __global__ void __launch_bounds__(kBlock)
     __syncthreads();
     const uint32_t total = s_offset[kPointsPerBlock];
     const uint32_t out = block_base[blockIdx.x];
+    if (sorted_first) {   // where a point's instances start, in the order they are created in: the backward pass
+                          // collects the gradient of a point that touches several tiles in rows numbered that way
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            const uint32_t k = tid * kPer + u;
+            if (base + k < n_visible) {
+                const uint32_t at = out + s_offset[k];
+                sorted_first[base + k] = at;
+                if (count[u] > 1u) point_first[s_point[k]] = at;
+            }
+        }
+    }
     for (uint32_t s = tid; s < total; s += kBlock) {
         uint32_t lo = 0, hi = kPointsPerBlock;   // last k with s_offset[k] <= s
         while (hi - lo > 1u) {
@@ -456,8 +469,7 @@ __device__ __forceinline__ Pixel pixel_of_thread(uint32_t tile, uint32_t gw, int
     return p;
 }
 
-// Bits of a pixel in a box word, and of a wave's 8 x 8 pixel block.
-__device__ __forceinline__ uint32_t pixel_bits(const Pixel& p) { return (1u << p.lx) | (1u << (16 + p.ly)); }
+// Does the box reach the wave's 8 x 8 pixel block?
 __device__ __forceinline__ bool box_reaches(uint32_t box, const Pixel& p) {
     return (box & (0xFFu << p.qx0)) != 0u && (box & (0xFF0000u << p.qy0)) != 0u;
 }
@@ -505,7 +517,6 @@ __global__ void __launch_bounds__(T * T)
     const Pixel px = pixel_of_thread<T>(tile, gw, W, H);
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     const float cx = (float)px.x + 0.5f, cy = (float)px.y + 0.5f;
-    const uint32_t mine = pixel_bits(px);
     float acc[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) acc[c] = 0.0f;
@@ -633,6 +644,59 @@ __global__ void __launch_bounds__(T * T)
     }
 }
 
+// Gradient rows of the points that touch several tiles: one row per instance, numbered in the order the instances
+// are created in (a point's instances are neighbours), C + 1 values padded to whole 16-byte words. A block that
+// ends early (every pixel saturated) leaves the rows of its remaining instances unwritten: `written` says which
+// rows count (cleared before the blend).
+struct GradRows {
+    float* values;
+    uint8_t* written;
+    const uint2* bounds;           // per point: tile bounds
+    const uint32_t* point_first;   // per point that touches several tiles: its first row
+    __host__ __device__ static constexpr uint32_t words(int channels) { return (uint32_t)(channels + 4) / 4u * 4u; }
+};
+
+// Gradient of a point that touches several tiles = sum of its rows, in row order; one thread per depth-ordered point.
+template <int C>
+__global__ void __launch_bounds__(kBlock)
+    k_grad_reduce(const uint32_t* __restrict__ order, const uint2* __restrict__ sorted_bounds,
+                  const uint32_t* __restrict__ sorted_first, const uint32_t* __restrict__ counters, GradRows rows,
+                  float* __restrict__ grad_features, float* __restrict__ grad_opacities) {
+    const uint32_t n_visible = counters[kCntVisible];
+    if (counters[kCntKept] == 0u) return;
+    const uint32_t stride = gridDim.x * kBlock;
+    for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < n_visible; j += stride) {
+        const uint32_t n_rows = tiles_of(sorted_bounds[j]);
+        if (n_rows < 2u) continue;
+        const uint32_t first = sorted_first[j];
+        float sum[C + 1];
+#pragma unroll
+        for (int c = 0; c <= C; ++c) sum[c] = 0.0f;
+        for (uint32_t r = first; r < first + n_rows; ++r) {
+            if (!rows.written[r]) continue;
+            const float4* in = (const float4*)(rows.values + (size_t)r * GradRows::words(C));
+#pragma unroll
+            for (int q = 0; q < C / 4; ++q) {
+                const float4 v = in[q];
+                sum[4 * q] += v.x;
+                sum[4 * q + 1] += v.y;
+                sum[4 * q + 2] += v.z;
+                sum[4 * q + 3] += v.w;
+            }
+            sum[C] += in[C / 4].x;
+        }
+        // added to what is there: instances without slots have put their share into the arrays directly
+        const uint32_t point = order[j];
+        float4* gf = (float4*)(grad_features + (size_t)point * C);
+#pragma unroll
+        for (int q = 0; q < C / 4; ++q) {
+            const float4 old = gf[q];
+            gf[q] = make_float4(old.x + sum[4 * q], old.y + sum[4 * q + 1], old.z + sum[4 * q + 2], old.w + sum[4 * q + 3]);
+        }
+        grad_opacities[point] += sum[C];
+    }
+}
+
 // Backward: the same walk with the saved final image (kernels.cu:476-579). A pixel leaves its blending weight and
 // opacity gradient in the instance's slot; after the batch the instance's thread multiplies the weights with the
 // pixels' image gradients (kept in LDS) and adds everything up: a plain store for a point with a single
@@ -643,7 +707,7 @@ __global__ void __launch_bounds__(T * T)
                      const uint32_t* __restrict__ inst_points, const char* __restrict__ records, uint32_t stride,
                      const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
                      const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_features,
-                     float* grad_opacities, int W, int H, uint32_t gw, float threshold, float reach2) {
+                     float* grad_opacities, GradRows grad_rows, int W, int H, uint32_t gw, float threshold, float reach2) {
     constexpr int TT = T * T;
     __shared__ Stage<T, C> st;
     __shared__ float s_d_opacity[TT][kSlotStride];   // per staged instance and box pixel: d loss / d opacity
@@ -653,20 +717,24 @@ __global__ void __launch_bounds__(T * T)
     const Pixel px = pixel_of_thread<T>(tile, gw, W, H);
     const int tile_x0 = (int)(tile % gw) * T, tile_y0 = (int)(tile / gw) * T;
     const float cx = (float)px.x + 0.5f, cy = (float)px.y + 0.5f;
-    const uint32_t mine = pixel_bits(px);
-    float g[C], final_px[C], fresh[C];
-    float common = 0.0f;
+    // With s = features . grad of an instance, R the running sum of blending weight x s of the pixel and S its final
+    // value, the reference's dot(T f + (F_running - F_final) / (1 - a), grad) + grad_alpha (1 - alpha_final) / (1 - a)
+    // is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the walk carries two scalars, not 2C.
+    float g[C];
+    float offset = 0.0f;   // grad_alpha (1 - alpha_final) - S
 #pragma unroll
-    for (int c = 0; c < C; ++c) g[c] = final_px[c] = fresh[c] = 0.0f;
+    for (int c = 0; c < C; ++c) g[c] = 0.0f;
     if (px.inside) {
         const size_t n_pixels = (size_t)W * H, pix = (size_t)px.y * W + px.x;
+        float final_dot = 0.0f;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             g[c] = grad_image[c * n_pixels + pix];
-            final_px[c] = image[c * n_pixels + pix];
+            final_dot = fmaf(image[c * n_pixels + pix], g[c], final_dot);
         }
-        common = grad_alpha[pix] * (1.0f - alpha_image[pix]);
+        offset = grad_alpha[pix] * (1.0f - alpha_image[pix]) - final_dot;
     }
+    float running = 0.0f;
 #pragma unroll
     for (int c = 0; c < C; ++c) s_grad_px[px.ly * T + px.lx][c] = g[c];
     float tr = 1.0f;
@@ -693,20 +761,17 @@ __global__ void __launch_bounds__(T * T)
                     const float bw = tr * a;
                     const float one_minus_a = 1.0f - a;
                     const float rcp = 1.0f / fmaxf(one_minus_a, kOneMinusAlphaEps);
-                    float dot = 0.0f;
+                    float sd = 0.0f;
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q) {
-                        const float4 f4 = st.feat[j * (C / 4) + q];
-                        const float f[4] = {f4.x, f4.y, f4.z, f4.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int c = 4 * q + e;
-                            fresh[c] += bw * f[e];
-                            const float term = (tr * f[e] + (fresh[c] - final_px[c]) * rcp) * g[c];
-                            dot = c == 0 ? term : dot + term;
-                        }
+                        const float4 f = st.feat[j * (C / 4) + q];
+                        sd = fmaf(f.x, g[4 * q], sd);
+                        sd = fmaf(f.y, g[4 * q + 1], sd);
+                        sd = fmaf(f.z, g[4 * q + 2], sd);
+                        sd = fmaf(f.w, g[4 * q + 3], sd);
                     }
-                    const float d_alpha = dot + common * rcp;
+                    running = fmaf(bw, sd, running);
+                    const float d_alpha = fmaf(tr, sd, (running + offset) * rcp);
                     const float d_opacity = d_alpha * G;
                     const float weight = bw > 0.0f ? bw : 0.0f;
                     if (slot >= 0) {
@@ -779,13 +844,20 @@ __global__ void __launch_bounds__(T * T)
                 const uint32_t point = word & kPointMask;
                 float* gf = grad_features + (size_t)point * C;
                 if (word & kMultiTile) {
+                    // the point's row for this tile: its instances were created row-major over its tile bounds
+                    const uint2 b = grad_rows.bounds[point];
+                    const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
+                    const uint32_t row = grad_rows.point_first[point] + (tile / gw - y0) * nx + (tile % gw - x0);
+                    float4* out = (float4*)(grad_rows.values + (size_t)row * GradRows::words(C));
 #pragma unroll
-                    for (int c = 0; c < C; ++c)
-                        if (sum[c] != 0.0f) atomicAdd(&gf[c], sum[c]);
-                    if (sum[C] != 0.0f) atomicAdd(&grad_opacities[point], sum[C]);
+                    for (int q = 0; q < C / 4; ++q)
+                        out[q] = make_float4(sum[4 * q], sum[4 * q + 1], sum[4 * q + 2], sum[4 * q + 3]);
+                    out[C / 4] = make_float4(sum[C], 0.0f, 0.0f, 0.0f);
+                    grad_rows.written[row] = 1u;
                 } else {
 #pragma unroll
-                    for (int c = 0; c < C; ++c) gf[c] = sum[c];
+                    for (int q = 0; q < C / 4; ++q)   // the rows are 16-byte aligned (checked by the host)
+                        ((float4*)gf)[q] = make_float4(sum[4 * q], sum[4 * q + 1], sum[4 * q + 2], sum[4 * q + 3]);
                     grad_opacities[point] = sum[C];
                 }
             }

@@ -909,7 +909,7 @@ struct GaussianLayout {
     uint32_t n_blocks;  // blocks of gaussian::kPointsPerBlock depth-ordered points
     size_t zero_begin, zero_words;
     size_t hist_depth, hist_tile, status_depth, status_tile, bases_depth, bases_tile, tile_order, block_sums;
-    size_t sorted_bounds;
+    size_t sorted_bounds, sorted_first, point_first, grad_rows, row_flags;
     size_t keys_a, keys_b, vals_a, vals_b, inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
 };
 
@@ -993,6 +993,13 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
     P.point_touched = take(n * 4);
     P.point_bounds = take(n * 8);
     L.sorted_bounds = take(n * 8);
+    L.sorted_first = L.point_first = L.grad_rows = L.row_flags = 0;
+    if (!L.inference) {   // configurations with a backward pass
+        L.sorted_first = take(n * 4);
+        L.point_first = take(n * 4);
+        L.grad_rows = take(capacity * gaussian::GradRows::words(L.C) * 4);
+        L.row_flags = take(capacity);
+    }
     P.point_record = take(n * g.stride);
     L.keys_a = take(n * 4);
     L.keys_b = take(n * 4);
@@ -1076,11 +1083,20 @@ template <int T, int C>
 int launch_gaussian_blend_backward(const GaussianLayout& L, const float* grad_image, const float* grad_alpha,
                                    const float* image, const float* alpha, float* grad_view, float* grad_opacities,
                                    void* ws, hipStream_t stream) {
+    const gaussian::GradRows rows{at<float>(ws, L.grad_rows), at<uint8_t>(ws, L.row_flags),
+                                  (const uint2*)at<uint2>(ws, L.pub.point_bounds),
+                                  (const uint32_t*)at<uint32_t>(ws, L.point_first)};
+    int rc = fill_u32(rows.written, 0u, align_up(L.prm.capacity, 4) / 4, stream);
+    if (rc != INPC_OK) return rc;
     INPC_LAUNCH("gaussian_blend_backward", (gaussian::k_blend_backward<T, C>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 (const uint32_t*)at<uint32_t>(ws, L.pub.instance_points), (const char*)at<char>(ws, L.pub.point_record),
-                L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, L.geo.W, L.geo.H, L.geo.gw,
-                L.prm.threshold, L.prm.reach2);
+                L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, rows, L.geo.W, L.geo.H,
+                L.geo.gw, L.prm.threshold, L.prm.reach2);
+    INPC_LAUNCH("gaussian_grad_reduce", gaussian::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, kBlock), 4096u)),
+                dim3(kBlock), stream, (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order),
+                (const uint2*)at<uint2>(ws, L.sorted_bounds), (const uint32_t*)at<uint32_t>(ws, L.sorted_first),
+                (const uint32_t*)at<uint32_t>(ws, L.pub.counters), rows, grad_view, grad_opacities);
     return INPC_OK;
 }
 
@@ -1341,7 +1357,9 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
         INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(L.n_blocks), dim3(kBlock), stream,
                     order, (const uint2*)at<uint2>(ws, L.sorted_bounds),
                     (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,
-                    at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a), at<uint32_t>(ws, L.hist_tile),
+                    at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a),
+                    L.inference ? (uint32_t*)nullptr : at<uint32_t>(ws, L.sorted_first),
+                    L.inference ? (uint32_t*)nullptr : at<uint32_t>(ws, L.point_first), at<uint32_t>(ws, L.hist_tile),
                     L.geo.gw, radix::to_device_plan(L.tile_plan));
         rc = radix::sort_pairs<uint16_t>(L.tile_plan, radix::kPlain, at<uint16_t>(ws, L.inst_keys_a),
                                          at<uint32_t>(ws, L.inst_vals_a), at<uint16_t>(ws, L.inst_keys_b),
@@ -1375,6 +1393,8 @@ int inpc_gaussian_backward(const inpc_gaussian_config* cfg, const float* grad_im
     const bool direct32 = L.fmode == INPC_FEAT_DIRECT_F32;
     float* grad_view = direct32 ? (float*)grad_features : grad_view_scratch;
     if (!grad_view) return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: this feature mode needs grad_view_scratch");
+    if (((uintptr_t)grad_view & 15u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: the fp32 gradient buffer must be 16-byte aligned");
     if (L.sh && (!cam_position || !positions))
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: positions / cam_position are null");
     rc = fill_u32(grad_view, 0u, (size_t)L.geo.n * L.C, stream);

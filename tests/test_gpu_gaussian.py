@@ -2,7 +2,10 @@
 
 Bit-exact: tile bounds, screen coordinates, conics, depth order, instance order, tile ranges, and (because the
 footprint's exponential is one fixed sequence of fp32 operations on both sides) image, alpha and depth image.
-Within 1e-4 relative: blending weights and gradients, which both sides sum in an order of their own.
+Within 1e-4 relative: blending weights and gradients, which both sides sum in an order of their own. The opacity
+gradient contains the difference between the running and the final pixel value, which cancels towards the end of a
+pixel's list; the kernel carries that difference as one scalar, the oracle per channel as the reference writes it,
+so a single small element can differ by 1e-4 of the largest gradient rather than of itself (`grad_atol`).
 """
 import numpy as np
 import pytest
@@ -15,6 +18,10 @@ from tests.test_oracle_gaussian import gcfg_of, near_camera_points
 pytestmark = pytest.mark.gpu
 
 RTOL = 1e-4
+
+
+def grad_atol(ref):
+    return 1e-4 * float(np.abs(ref).max()) + 2e-7
 
 
 def oracle_run(O, hv, pos, feats, opac, tile, channels, mode=None, inference=False, scales=None, sigma_world=0.0,
@@ -90,7 +97,7 @@ def test_forward_backward_dense_opaque_scene(gpu, oracle, tile):
     gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
                                                gaussian=g)
     H.assert_close(gf, gf_ref, RTOL, 1e-7, "feature gradients")
-    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
 
 
 @pytest.mark.parametrize("tile", [8, 16])
@@ -119,7 +126,7 @@ def test_forward_sh36_and_backward(gpu, oracle, tile):
                                                hv.position, gaussian=g)
     assert (gf[~vis] == 0).all() and (go[~vis] == 0).all()
     H.assert_close(gf.astype(np.float32), gf_ref.astype(np.float32), 2e-3, 1e-7, "SH gradients")
-    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
 
 
 @pytest.mark.parametrize("mode", ["f16", "f32"])
@@ -144,7 +151,7 @@ def test_backward_direct(gpu, oracle, mode):
         H.assert_close(gf.astype(np.float32), gf_ref.astype(np.float32), 2e-3, 1e-7, "feature gradients")
     else:
         H.assert_close(gf, gf_ref, RTOL, 1e-7, "feature gradients")
-    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
 
 
 @pytest.mark.parametrize("with_scales", [False, True])
@@ -248,7 +255,7 @@ def test_python_api(gpu, oracle):
                                                alpha.detach().cpu().numpy(), pos, feats, opac, hv.w2c, hv.position,
                                                gaussian=g)
     H.assert_close(features.grad.float().cpu().numpy(), gf_ref.astype(np.float32), 2e-3, 1e-6, "SH gradients")
-    H.assert_close(opacities.grad.cpu().numpy().reshape(-1), go_ref, RTOL, 1e-6, "opacity gradients")
+    H.assert_close(opacities.grad.cpu().numpy().reshape(-1), go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
     # render_preextracted: sigma_world = scale * 0.05 / focal_y (B/torch_bindings/rasterization.py:130-134)
     img2, depth2, alpha2 = rasterizer.render_preextracted(view, 1, positions, features.detach(), opacities.detach(),
                                                           None, 2.0, 2.5)
