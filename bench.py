@@ -227,6 +227,56 @@ def main() -> int:
     field_ms = time_calls(lambda: update_probability_field(field_weights, field_scores, leaf_ids, blending_weights),
                           args.steps)
 
+    # the same points through the Gaussian footprint (the reference's other rasterizer mode), 8x8 tiles as in the
+    # reference: a side measurement, not part of `value`
+    gaussian = None
+    try:
+        gcfg = _lib.GaussianConfig(_lib.RasterConfig(n, 8, channels, _lib.FEAT_DIRECT_F32, 0,
+                                                     _lib.make_camera(hv.camera)), 0.0, 3.0, 0, 0)
+        glayout = _lib.GaussianLayout()
+        _lib.check(lib.inpc_gaussian_layout_query(C.byref(gcfg), C.byref(glayout)), "gaussian layout")
+        gws = torch.empty(glayout.total_bytes, dtype=torch.uint8, device=device)
+        g_image, g_alpha, g_weights = torch.empty_like(image), torch.empty_like(alpha), torch.empty_like(blending_weights)
+        g_gf, g_go = torch.empty_like(grad_features), torch.empty_like(grad_opacities)
+
+        def gaussian_forward():
+            _lib.check(lib.inpc_gaussian_forward(C.byref(gcfg), _lib.ptr(positions), _lib.ptr(features),
+                                                 _lib.ptr(opacities), None, _lib.ptr(w2c), _lib.ptr(cam_position),
+                                                 _lib.ptr(g_image), _lib.ptr(g_alpha), _lib.ptr(g_weights), None,
+                                                 _lib.ptr(gws), glayout.total_bytes, stream), "inpc_gaussian_forward")
+
+        def gaussian_backward():
+            _lib.check(lib.inpc_gaussian_backward(C.byref(gcfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha),
+                                                  _lib.ptr(g_image), _lib.ptr(g_alpha), _lib.ptr(positions),
+                                                  _lib.ptr(cam_position), _lib.ptr(g_gf), _lib.ptr(g_go), None,
+                                                  _lib.ptr(gws), glayout.total_bytes, stream), "inpc_gaussian_backward")
+
+        def gaussian_step():
+            gaussian_forward()
+            gaussian_backward()
+
+        gaussian_step()
+        g_counters = (C.c_uint32 * 4)()
+        _lib.check(lib.inpc_gaussian_read_counters(C.byref(gcfg), _lib.ptr(gws), C.byref(g_counters), stream),
+                   "inpc_gaussian_read_counters")
+        g_step_ms = time_calls(gaussian_step, args.steps)
+        g_fwd_ms = time_calls(gaussian_forward, args.steps)
+        g_bwd_ms = time_calls(gaussian_backward, args.steps)
+        with _lib.KernelTimer() as g_timer:
+            for _ in range(args.steps):
+                gaussian_step()
+        g_kernels = {}
+        for name, ms in g_timer.records:
+            g_kernels[name] = g_kernels.get(name, 0.0) + ms / args.steps
+        gaussian = {"workload": "same points, Gaussian footprint (training variance), 8x8 tiles, forward+backward",
+                    "ms_per_step": round(g_step_ms, 4), "forward_ms": round(g_fwd_ms, 4),
+                    "backward_ms": round(g_bwd_ms, 4), "Mpoints_per_s": round(n / (g_step_ms * 1e-3) / 1e6, 1),
+                    "n_instances": int(g_counters[1]),
+                    "kernel_ms_per_step": {k: round(v, 4) for k, v in sorted(g_kernels.items(), key=lambda kv: -kv[1])}}
+        del gws, g_image, g_alpha, g_weights, g_gf, g_go
+    except Exception as exc:  # the figure is optional
+        print(f"bench.py: Gaussian footprint not measured: {exc}", file=sys.stderr)
+
     # ---- per-kernel durations: HIP events around every launch, on the launch stream, same steps ----------
     with _lib.KernelTimer() as timer:
         for _ in range(args.steps):
@@ -304,6 +354,7 @@ def main() -> int:
             "forward_ms": round(fwd_ms, 4), "backward_ms": round(bwd_ms, 4),
             "graph_replay_ms": None if graph_ms is None else round(graph_ms, 4), "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
             "field_update_ms": round(field_ms, 4),
+            "gaussian_footprint": gaussian,
             "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
             "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),
             "kernels": kernels,
