@@ -1,7 +1,7 @@
 /*
  * inpc_hip.h — C ABI of libinpc_hip.so, the MI355X (gfx950) implementation of the
  * INPCCudaBackend hot path: view-dependent octree point sampling and the tile-based
- * differentiable bilinear point rasterizer (forward, backward, inference).
+ * differentiable point rasterizer (forward, backward, inference; bilinear and Gaussian footprint).
  *
  * Conventions
  *   - every pointer marked "dev" is a device pointer on the current HIP device;
