@@ -10,7 +10,8 @@
  *     never throws; inpc_last_error() returns a thread-local message for the last failure;
  *   - the library never allocates or frees device memory: the caller provides the
  *     workspace whose size inpc_*_workspace_bytes() reports (sized for the worst case,
- *     so no count has to travel back to the host between kernels);
+ *     so no count has to travel back to the host between kernels; the Gaussian footprint,
+ *     whose worst case has no useful bound, takes a capacity and reports when it is exceeded);
  *   - all kernels are enqueued on `stream`; no call synchronises the host unless its
  *     comment says so.
  *

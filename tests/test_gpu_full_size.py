@@ -134,6 +134,42 @@ def test_config2_and_3_forward_backward_full_size(config1, oracle, tile):
     H.assert_close(go2, 2 * go, 1e-5, 1e-8, "opacity gradients, doubled input")
 
 
+def test_config3_points_gaussian_footprint_full_size(config1, oracle):
+    """The 8,388,608 points of config 3 through the Gaussian footprint (training variance), 8x8 tiles, forward and
+    backward, against the oracle: structure, image and alpha bit-exact, weights and gradients to tolerance."""
+    from tests.test_gpu_gaussian import check_structure as check_gaussian_structure, grad_atol, oracle_run
+
+    c = config1
+    n, hv = c["n"], c["hv"]
+    pos = c["pos_ref"]
+    feats, opac = synthetic.point_attributes(n, 8, "normal", 1)
+    run = H.GaussianRun(hv, pos, feats, opac, 8, 8).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, 8, 8)
+    dbg = run.debug()
+    check_gaussian_structure(dbg, ref)
+    assert (np.diff(dbg["instance_keys"].astype(np.int64)) >= 0).all()
+    r = dbg["tile_ranges"].astype(np.int64)
+    used = r[:, 1] > r[:, 0]
+    assert (r[used, 1] - r[used, 0]).sum() == dbg["n_instances"]
+    del dbg
+    out = run.outputs()
+    np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+    rng = np.random.default_rng(3)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                               gaussian=g)
+    H.assert_close(gf, gf_ref, RTOL, grad_atol(gf_ref), "feature gradients")
+    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
+    # the gradient sums have a fixed order: a second backward gives the same bits
+    gf2, go2 = run.backward(gi, ga)
+    np.testing.assert_array_equal(gf2.view(np.uint32), gf.view(np.uint32))
+    np.testing.assert_array_equal(go2.view(np.uint32), go.view(np.uint32))
+
+
 def test_config4_large_frame_inference(gpu, oracle):
     """2,097,152 leaves of the level-11 grid, 33,554,432 samples, 16 channels stored as fp16, 2473x1643, f = 2000,
     16x16 tiles: sampling + inference forward end to end."""
