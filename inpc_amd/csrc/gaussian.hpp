@@ -743,8 +743,18 @@ __global__ void __launch_bounds__(T * T)
     for (uint32_t base = range.x; base < range.y; base += TT) {
         if (__syncthreads_count(done) == TT) break;
         const uint32_t count = min((uint32_t)TT, range.y - base);
+        uint32_t my_row = 0u;
         if (tid < count) {
-            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2, threshold);
+            const uint32_t point = inst_points[base + tid];
+            const char* record = records + (size_t)point * stride;
+            // the row of a point that touches several tiles is looked up now, long before it is needed: its
+            // instances were created row-major over its tile bounds
+            if (((const uint32_t*)record)[7] & kMultiTile) {
+                const uint2 b = grad_rows.bounds[point];
+                const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
+                my_row = grad_rows.point_first[point] + (tile / gw - y0) * nx + (tile % gw - x0);
+            }
+            stage_instance<T, C>(st, tid, record, tile_x0, tile_y0, reach2, threshold);
         }
         __syncthreads();
         if (__ballot(!done) != 0ull) {
@@ -844,16 +854,12 @@ __global__ void __launch_bounds__(T * T)
                 const uint32_t point = word & kPointMask;
                 float* gf = grad_features + (size_t)point * C;
                 if (word & kMultiTile) {
-                    // the point's row for this tile: its instances were created row-major over its tile bounds
-                    const uint2 b = grad_rows.bounds[point];
-                    const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
-                    const uint32_t row = grad_rows.point_first[point] + (tile / gw - y0) * nx + (tile % gw - x0);
-                    float4* out = (float4*)(grad_rows.values + (size_t)row * GradRows::words(C));
+                    float4* out = (float4*)(grad_rows.values + (size_t)my_row * GradRows::words(C));
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q)
                         out[q] = make_float4(sum[4 * q], sum[4 * q + 1], sum[4 * q + 2], sum[4 * q + 3]);
                     out[C / 4] = make_float4(sum[C], 0.0f, 0.0f, 0.0f);
-                    grad_rows.written[row] = 1u;
+                    grad_rows.written[my_row] = 1u;
                 } else {
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q)   // the rows are 16-byte aligned (checked by the host)

@@ -271,3 +271,55 @@ def test_python_api(gpu, oracle):
     g8, ref8 = oracle_run(oracle, hv, pos_near, f8, o8, 8, 8)
     assert ref8["n_instances"] > 4 * 10000 + 65536
     np.testing.assert_array_equal(img8.cpu().numpy().view(np.uint32), ref8["image"].view(np.uint32))
+
+
+RANDOM_CASES = [
+    # seed, n, width, height, focal, tile, channels, opacity range, cluster share, share of points close to the camera
+    (201, 9000, 37, 29, 40.0, 8, 4, (0.0, 1.0), 0.0, 0.0),
+    (202, 30000, 130, 71, 110.0, 16, 8, (0.0, 0.2), 0.3, 0.01),
+    (203, 20000, 65, 65, 70.0, 16, 4, (0.9, 1.0), 0.5, 0.0),
+    (204, 25000, 129, 33, 95.0, 8, 8, (0.3, 0.7), 0.8, 0.02),
+    (205, 12000, 16, 16, 30.0, 16, 16, (0.0, 0.6), 0.2, 0.05),
+    (206, 40000, 200, 120, 150.0, 8, 16, (0.01, 0.05), 0.6, 0.0),
+]
+
+
+@pytest.mark.parametrize("case", RANDOM_CASES, ids=[f"seed{c[0]}" for c in RANDOM_CASES])
+def test_random_scenes_forward_backward(gpu, oracle, case):
+    # Odd image sizes, clusters of hundreds of points on single pixels (long per-pixel lists over several batches,
+    # early termination), opacities at exactly 0 and 1, footprints with and without slots side by side.
+    seed, n, width, height, focal, tile, channels, (lo, hi), cluster, near = case
+    rng = np.random.default_rng(seed)
+    hv = synthetic.camera_on_z(width, height, focal, 2.4)
+    pos = synthetic.cube_points(n, 1.4, seed)
+    n_cluster = int(n * cluster)
+    if n_cluster:
+        spots = rng.uniform(-0.5, 0.5, (7, 3)).astype(np.float32)
+        pos[:n_cluster] = spots[rng.integers(0, 7, n_cluster)] + rng.normal(0, 2e-3, (n_cluster, 3)).astype(np.float32)
+    n_near = int(n * near)
+    if n_near:
+        pos[n - n_near:] = near_camera_points(hv, n_near, seed + 2)
+    feats, _ = synthetic.point_attributes(n, channels, "normal", seed + 1)
+    opac = rng.uniform(lo, hi, n).astype(np.float32)
+    opac[::97] = 0.0
+    if hi >= 1.0:
+        opac[5::89] = 1.0
+    run = H.GaussianRun(hv, pos, feats, opac, tile, channels).forward()
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, channels)
+    check_structure(run.debug(), ref)
+    out = run.outputs()
+    np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7 + 1e-6 * float(ref["blending_weights"].max()),
+                   "blending weights")
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                               gaussian=g)
+    H.assert_close(gf, gf_ref, RTOL, grad_atol(gf_ref), "feature gradients")
+    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
+    # a second backward pass on the same saved state
+    gf2, go2 = run.backward(gi, ga)
+    H.assert_close(gf2, gf, 1e-5, grad_atol(gf_ref) * 0.1, "feature gradients, second pass")
+    H.assert_close(go2, go, 1e-5, grad_atol(go_ref) * 0.1, "opacity gradients, second pass")
