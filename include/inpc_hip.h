@@ -303,9 +303,11 @@ typedef struct inpc_gaussian_layout {
     size_t point_touched;    /* (N) u32: tiles a point touches, 0 when it is not drawn          */
     size_t point_bounds;     /* (N) 4 x u16: x_min, x_max, y_min, y_max in tiles, half open     */
     size_t point_record;     /* (N) records of record_stride bytes, in point order:
-                                float sx, sy, opacity, conic.x, conic.y, conic.z, depth,
-                                u32 (point id | bit 31: touches more than one tile); then the
-                                view features as fp32                                           */
+                                float sx, sy, opacity, conic.x, conic.y, conic.z, depth (training
+                                configurations, points that touch several tiles: u32 origin of
+                                the point's gradient rows instead), u32 (bits 0-27 point id,
+                                28-30 min(tile columns, 7), 31: touches more than one tile);
+                                then the view features as fp32                                  */
     size_t depth_order;      /* (N) u32 point ids in (depth, point id) order, n_visible valid   */
     size_t depth_keys;       /* (N) u32 matching depth keys                                     */
     size_t instance_keys;    /* (max_instances) u16 tile id per instance in final order         */

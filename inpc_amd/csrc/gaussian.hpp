@@ -24,10 +24,14 @@ namespace gaussian {
 constexpr float kDilation = 0.16f;                  // gaussian/config.h:19
 constexpr float kTrainThreshold = 0.01110899653f;   // kernels.cu:452
 constexpr float kTrainCutoff = 3.0f;                // kernels.cu:80-81
-constexpr uint32_t kMultiTile = 1u << 31;           // record word: the point touches more than one tile
-constexpr uint32_t kPointMask = kMultiTile - 1u;
+// Last header word of a record: point id (n < 2^28), then min(tile columns, 7), then "touches more than one tile".
+constexpr uint32_t kMultiTile = 1u << 31;
+constexpr uint32_t kPointMask = (1u << 28) - 1u;
+constexpr int kColumnsShift = 28;
+constexpr uint32_t kManyColumns = 7u;               // 7 or more tile columns: the count is looked up
 constexpr int kCntKept = 4;                         // instances that are sorted and drawn (0 when they do not fit)
 constexpr int kCntInstances64 = 6;                  // u64 at words 6, 7: exact instance count
+constexpr int kCntMulti = 8;                        // drawn points that touch more than one tile
 constexpr int kPointsPerBlock = 1024;               // depth-ordered points per block of the instance kernels
 
 inline uint32_t record_stride(int channels) { return (uint32_t)align_up(32 + (size_t)channels * 4, 32); }
@@ -149,7 +153,8 @@ __global__ void __launch_bounds__(kBlock)
                         }
                     }
                     rec[0] = make_float4(sx, sy, opacity, conic_x);
-                    rec[1] = make_float4(conic_y, conic_z, depth, __uint_as_float(i | (touched > 1u ? kMultiTile : 0u)));
+                    rec[1] = make_float4(conic_y, conic_z, depth,
+                                         __uint_as_float(i | (min(x1 - x0, kManyColumns) << kColumnsShift) | (touched > 1u ? kMultiTile : 0u)));
                     key = __float_as_uint(depth) - g.key_bias;
                     radix::hist_add(s_hist, plan, key);
                 }
@@ -265,21 +270,24 @@ __global__ void __launch_bounds__(kScanBlock) k_touch_scan(uint32_t* __restrict_
 __global__ void __launch_bounds__(kBlock)
     k_create_instances(const uint32_t* __restrict__ order, const uint2* __restrict__ sorted_bounds,
                        const uint32_t* __restrict__ block_base,
-                       const uint32_t* __restrict__ counters, uint16_t* __restrict__ inst_keys,
-                       uint32_t* __restrict__ inst_points, uint32_t* __restrict__ sorted_first,
-                       uint32_t* __restrict__ point_first, uint32_t* g_hist, uint32_t gw, radix::DevicePlan plan) {
+                       const uint32_t* counters, uint16_t* __restrict__ inst_keys,
+                       uint32_t* __restrict__ inst_points, uint4* __restrict__ multi_list, uint32_t* counters_out,
+                       char* __restrict__ records, uint32_t stride, uint32_t* g_hist, uint32_t gw,
+                       radix::DevicePlan plan) {
     constexpr int kPer = kPointsPerBlock / kBlock;   // consecutive points per thread
     __shared__ uint32_t s_offset[kPointsPerBlock + 1];
     __shared__ uint32_t s_point[kPointsPerBlock];
     __shared__ uint2 s_bounds[kPointsPerBlock];
     __shared__ uint32_t s_wave[kBlock / kWave];
     __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
+    __shared__ uint32_t s_multi, s_multi_base;
     if (counters[kCntKept] == 0u) return;
     const uint32_t n_visible = counters[kCntVisible];
     const uint32_t base = blockIdx.x * kPointsPerBlock;
     if (base >= n_visible) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     for (int i = tid; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
+    if (tid == 0) s_multi = 0u;
     uint32_t count[kPer], mine = 0;
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
@@ -312,15 +320,29 @@ __global__ void __launch_bounds__(kBlock)
     __syncthreads();
     const uint32_t total = s_offset[kPointsPerBlock];
     const uint32_t out = block_base[blockIdx.x];
-    if (sorted_first) {   // where a point's instances start, in the order they are created in: the backward pass
-                          // collects the gradient of a point that touches several tiles in rows numbered that way
+    if (multi_list) {
+        // Where a point's instances start, in the order they are created in: the backward pass collects the
+        // gradient of a point that touches several tiles in rows numbered that way. The instance of tile (tx, ty)
+        // has row origin + ty * columns + tx; the origin (modulo 2^32) replaces the depth in the point's record,
+        // which only the inference blend reads. The points themselves go on a list {first row, rows, point} for
+        // the pass that adds the rows up (in no particular order: every point is summed on its own).
+        uint32_t mine_multi = 0;
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) mine_multi += (base + tid * kPer + u < n_visible && count[u] > 1u) ? 1u : 0u;
+        uint32_t slot = mine_multi ? atomicAdd(&s_multi, mine_multi) : 0u;
+        __syncthreads();
+        if (tid == 0) s_multi_base = s_multi ? atomicAdd(&counters_out[kCntMulti], s_multi) : 0u;
+        __syncthreads();
+        slot += s_multi_base;
 #pragma unroll
         for (int u = 0; u < kPer; ++u) {
             const uint32_t k = tid * kPer + u;
-            if (base + k < n_visible) {
+            if (base + k < n_visible && count[u] > 1u) {
                 const uint32_t at = out + s_offset[k];
-                sorted_first[base + k] = at;
-                if (count[u] > 1u) point_first[s_point[k]] = at;
+                const uint2 b = s_bounds[k];
+                const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
+                ((uint32_t*)(records + (size_t)s_point[k] * stride))[6] = at - y0 * nx - x0;
+                multi_list[slot++] = make_uint4(at, count[u], s_point[k], 0u);
             }
         }
     }
@@ -390,7 +412,7 @@ template <int T, int C>
 struct Stage {
     static constexpr int TT = T * T;
     float4 head0[TT];   // sx, sy, opacity, conic.x
-    float4 head1[TT];   // conic.y, conic.z, depth, point id | kMultiTile
+    float4 head1[TT];   // conic.y, conic.z, depth (or row origin), point id with the column and several-tiles bits
     float4 feat[TT * (C / 4)];
     uint32_t box[TT];   // bits 0-15: columns of the tile the footprint can reach, bits 16-31: rows
     float value[TT][kSlotStride];   // footprint value per pixel of the box (boxes of at most kSlots pixels)
@@ -616,7 +638,7 @@ __global__ void __launch_bounds__(T * T)
                 if (w != 0.0f) {
                     const uint32_t word = __float_as_uint(st.head1[tid].w);
                     if (word & kMultiTile) atomicAdd(&blending_weights[word & kPointMask], w);
-                    else blending_weights[word] = w;   // the point's only instance
+                    else blending_weights[word & kPointMask] = w;   // the point's only instance
                 }
             }
         }
@@ -645,36 +667,35 @@ __global__ void __launch_bounds__(T * T)
 }
 
 // Gradient rows of the points that touch several tiles: one row per instance, numbered in the order the instances
-// are created in (a point's instances are neighbours), C + 1 values padded to whole 16-byte words. A block that
-// ends early (every pixel saturated) leaves the rows of its remaining instances unwritten: `written` says which
-// rows count (cleared before the blend).
+// are created in (a point's instances are neighbours): C + 1 values, then the two words of the call's stamp, padded
+// to whole 16-byte words. A block that ends early (every pixel saturated) leaves the rows of its remaining instances
+// unwritten: a row counts when it carries the stamp of this backward call (64 bits, unique per call and process),
+// so nothing has to be cleared.
 struct GradRows {
     float* values;
-    uint8_t* written;
-    const uint2* bounds;           // per point: tile bounds
-    const uint32_t* point_first;   // per point that touches several tiles: its first row
-    __host__ __device__ static constexpr uint32_t words(int channels) { return (uint32_t)(channels + 4) / 4u * 4u; }
+    const uint2* bounds;   // per point: tile bounds (looked up for points with kManyColumns or more tile columns)
+    uint32_t stamp_lo, stamp_hi;
+    __host__ __device__ static constexpr uint32_t words(int channels) { return (uint32_t)(channels + 6) / 4u * 4u; }
 };
 
-// Gradient of a point that touches several tiles = sum of its rows, in row order; one thread per depth-ordered point.
+// Gradient of a point that touches several tiles = sum of its rows, in row order; one thread per such point.
 template <int C>
 __global__ void __launch_bounds__(kBlock)
-    k_grad_reduce(const uint32_t* __restrict__ order, const uint2* __restrict__ sorted_bounds,
-                  const uint32_t* __restrict__ sorted_first, const uint32_t* __restrict__ counters, GradRows rows,
+    k_grad_reduce(const uint4* __restrict__ multi_list, const uint32_t* __restrict__ counters, GradRows rows,
                   float* __restrict__ grad_features, float* __restrict__ grad_opacities) {
-    const uint32_t n_visible = counters[kCntVisible];
     if (counters[kCntKept] == 0u) return;
+    const uint32_t n_multi = counters[kCntMulti];
     const uint32_t stride = gridDim.x * kBlock;
-    for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < n_visible; j += stride) {
-        const uint32_t n_rows = tiles_of(sorted_bounds[j]);
-        if (n_rows < 2u) continue;
-        const uint32_t first = sorted_first[j];
+    for (uint32_t m = blockIdx.x * kBlock + threadIdx.x; m < n_multi; m += stride) {
+        const uint4 entry = multi_list[m];
+        const uint32_t first = entry.x, n_rows = entry.y, point = entry.z;
         float sum[C + 1];
 #pragma unroll
         for (int c = 0; c <= C; ++c) sum[c] = 0.0f;
         for (uint32_t r = first; r < first + n_rows; ++r) {
-            if (!rows.written[r]) continue;
             const float4* in = (const float4*)(rows.values + (size_t)r * GradRows::words(C));
+            const float4 tail = in[C / 4];
+            if (__float_as_uint(tail.y) != rows.stamp_lo || __float_as_uint(tail.z) != rows.stamp_hi) continue;
 #pragma unroll
             for (int q = 0; q < C / 4; ++q) {
                 const float4 v = in[q];
@@ -683,10 +704,9 @@ __global__ void __launch_bounds__(kBlock)
                 sum[4 * q + 2] += v.z;
                 sum[4 * q + 3] += v.w;
             }
-            sum[C] += in[C / 4].x;
+            sum[C] += tail.x;
         }
         // added to what is there: instances without slots have put their share into the arrays directly
-        const uint32_t point = order[j];
         float4* gf = (float4*)(grad_features + (size_t)point * C);
 #pragma unroll
         for (int q = 0; q < C / 4; ++q) {
@@ -749,10 +769,14 @@ __global__ void __launch_bounds__(T * T)
             const char* record = records + (size_t)point * stride;
             // the row of a point that touches several tiles is looked up now, long before it is needed: its
             // instances were created row-major over its tile bounds
-            if (((const uint32_t*)record)[7] & kMultiTile) {
-                const uint2 b = grad_rows.bounds[point];
-                const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
-                my_row = grad_rows.point_first[point] + (tile / gw - y0) * nx + (tile % gw - x0);
+            const uint32_t word = ((const uint32_t*)record)[7];
+            if (word & kMultiTile) {
+                uint32_t columns = (word >> kColumnsShift) & kManyColumns;
+                if (columns == kManyColumns) {
+                    const uint2 b = grad_rows.bounds[point];
+                    columns = (b.x >> 16) - (b.x & 0xFFFFu);
+                }
+                my_row = ((const uint32_t*)record)[6] + (tile / gw) * columns + tile % gw;
             }
             stage_instance<T, C>(st, tid, record, tile_x0, tile_y0, reach2, threshold);
         }
@@ -858,8 +882,7 @@ __global__ void __launch_bounds__(T * T)
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q)
                         out[q] = make_float4(sum[4 * q], sum[4 * q + 1], sum[4 * q + 2], sum[4 * q + 3]);
-                    out[C / 4] = make_float4(sum[C], 0.0f, 0.0f, 0.0f);
-                    grad_rows.written[my_row] = 1u;
+                    out[C / 4] = make_float4(sum[C], __uint_as_float(grad_rows.stamp_lo), __uint_as_float(grad_rows.stamp_hi), 0.0f);
                 } else {
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q)   // the rows are 16-byte aligned (checked by the host)

@@ -27,7 +27,10 @@
 // bin of its tile; the blend of a tile then gathers from a few contiguous kilobytes instead of from the
 // whole point cloud, and every fetched line is used completely.
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cmath>
+#include <random>
 #include <cstring>
 #include <type_traits>
 
@@ -909,7 +912,7 @@ struct GaussianLayout {
     uint32_t n_blocks;  // blocks of gaussian::kPointsPerBlock depth-ordered points
     size_t zero_begin, zero_words;
     size_t hist_depth, hist_tile, status_depth, status_tile, bases_depth, bases_tile, tile_order, block_sums;
-    size_t sorted_bounds, sorted_first, point_first, grad_rows, row_flags;
+    size_t sorted_bounds, multi_list, grad_rows;
     size_t keys_a, keys_b, vals_a, vals_b, inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
 };
 
@@ -993,12 +996,10 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
     P.point_touched = take(n * 4);
     P.point_bounds = take(n * 8);
     L.sorted_bounds = take(n * 8);
-    L.sorted_first = L.point_first = L.grad_rows = L.row_flags = 0;
+    L.multi_list = L.grad_rows = 0;
     if (!L.inference) {   // configurations with a backward pass
-        L.sorted_first = take(n * 4);
-        L.point_first = take(n * 4);
+        L.multi_list = take(n * 16);
         L.grad_rows = take(capacity * gaussian::GradRows::words(L.C) * 4);
-        L.row_flags = take(capacity);
     }
     P.point_record = take(n * g.stride);
     L.keys_a = take(n * 4);
@@ -1079,23 +1080,30 @@ int launch_gaussian_blend_forward(const GaussianLayout& L, float* image, float* 
     return INPC_OK;
 }
 
+// A 64-bit value no other backward call of this or another process is likely to have used: a counter above a
+// start value drawn once per process.
+uint64_t next_stamp() {
+    static std::atomic<uint64_t> counter{[] {
+        std::random_device rd;
+        return ((uint64_t)rd() << 32) ^ ((uint64_t)rd() << 11) ^ (uint64_t)std::chrono::steady_clock::now().time_since_epoch().count();
+    }()};
+    return counter.fetch_add(0x9E3779B97F4A7C15ull) + 1u;
+}
+
 template <int T, int C>
 int launch_gaussian_blend_backward(const GaussianLayout& L, const float* grad_image, const float* grad_alpha,
                                    const float* image, const float* alpha, float* grad_view, float* grad_opacities,
                                    void* ws, hipStream_t stream) {
-    const gaussian::GradRows rows{at<float>(ws, L.grad_rows), at<uint8_t>(ws, L.row_flags),
-                                  (const uint2*)at<uint2>(ws, L.pub.point_bounds),
-                                  (const uint32_t*)at<uint32_t>(ws, L.point_first)};
-    int rc = fill_u32(rows.written, 0u, align_up(L.prm.capacity, 4) / 4, stream);
-    if (rc != INPC_OK) return rc;
+    const uint64_t stamp = next_stamp();
+    const gaussian::GradRows rows{at<float>(ws, L.grad_rows), (const uint2*)at<uint2>(ws, L.pub.point_bounds),
+                                  (uint32_t)stamp, (uint32_t)(stamp >> 32)};
     INPC_LAUNCH("gaussian_blend_backward", (gaussian::k_blend_backward<T, C>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 (const uint32_t*)at<uint32_t>(ws, L.pub.instance_points), (const char*)at<char>(ws, L.pub.point_record),
                 L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, rows, L.geo.W, L.geo.H,
                 L.geo.gw, L.prm.threshold, L.prm.reach2);
     INPC_LAUNCH("gaussian_grad_reduce", gaussian::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, kBlock), 4096u)),
-                dim3(kBlock), stream, (const uint32_t*)at<uint32_t>(ws, L.pub.depth_order),
-                (const uint2*)at<uint2>(ws, L.sorted_bounds), (const uint32_t*)at<uint32_t>(ws, L.sorted_first),
+                dim3(kBlock), stream, (const uint4*)at<uint4>(ws, L.multi_list),
                 (const uint32_t*)at<uint32_t>(ws, L.pub.counters), rows, grad_view, grad_opacities);
     return INPC_OK;
 }
@@ -1358,9 +1366,9 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
                     order, (const uint2*)at<uint2>(ws, L.sorted_bounds),
                     (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,
                     at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a),
-                    L.inference ? (uint32_t*)nullptr : at<uint32_t>(ws, L.sorted_first),
-                    L.inference ? (uint32_t*)nullptr : at<uint32_t>(ws, L.point_first), at<uint32_t>(ws, L.hist_tile),
-                    L.geo.gw, radix::to_device_plan(L.tile_plan));
+                    L.inference ? (uint4*)nullptr : at<uint4>(ws, L.multi_list), counters,
+                    at<char>(ws, L.pub.point_record), L.geo.stride, at<uint32_t>(ws, L.hist_tile), L.geo.gw,
+                    radix::to_device_plan(L.tile_plan));
         rc = radix::sort_pairs<uint16_t>(L.tile_plan, radix::kPlain, at<uint16_t>(ws, L.inst_keys_a),
                                          at<uint32_t>(ws, L.inst_vals_a), at<uint16_t>(ws, L.inst_keys_b),
                                          at<uint32_t>(ws, L.inst_vals_b), counters + gaussian::kCntKept, L.prm.capacity,

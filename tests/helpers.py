@@ -322,8 +322,10 @@ class GaussianRun:
         raw = self._buf(L.point_record, n * stride, np.uint8).reshape(n, stride)
         head = raw[:, :32].copy().view(np.float32).reshape(n, 8)
         word = head.view(np.uint32)[:, 7]
-        assert (word[vis] & 0x7FFFFFFF == np.flatnonzero(vis)).all(), "a record names another point"
+        assert (word[vis] & 0x0FFFFFFF == np.flatnonzero(vis)).all(), "a record names another point"
         assert ((word[vis] >> 31) == (touched[vis] > 1)).all(), "the several-tiles flag differs from the tile count"
+        columns = (bounds[:, 1].astype(np.int64) - bounds[:, 0])[vis]
+        assert (((word[vis] >> 28) & 7) == np.minimum(columns, 7)).all(), "the tile-column bits differ from the bounds"
         feats = raw[:, 32:32 + 4 * self.C].copy().view(np.float32).reshape(n, self.C)
 
         def drawn(a):
@@ -331,12 +333,22 @@ class GaussianRun:
             a[~vis] = 0
             return a
 
+        # the depth of a point as the sort saw it (the record's depth word of a point that touches several tiles is
+        # reused by the training configurations)
+        depth_keys = (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32)
+        depth_order = self._buf(L.depth_order, n, np.uint32)[:v].copy()
+        depth = np.zeros(n, np.float32)
+        depth[depth_order] = depth_keys.view(np.float32)
+        single = vis & (touched == 1)
+        assert (head[single, 6].view(np.uint32) == depth[single].view(np.uint32)).all(), "record depth differs from the key"
+        if self.inference:
+            assert (head[vis, 6].view(np.uint32) == depth[vis].view(np.uint32)).all(), "record depth differs from the key"
+
         return {
             "n_visible": v, "n_instances": i, "n_touched": touched, "bounds": bounds,
             "screen_xy": drawn(head[:, :2]), "opacity": drawn(head[:, 2]), "conic": drawn(head[:, 3:6]),
-            "depth": drawn(head[:, 6]), "features_view": drawn(feats),
-            "depth_keys": (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32),
-            "depth_order": self._buf(L.depth_order, n, np.uint32)[:v].copy(),
+            "depth": depth, "features_view": drawn(feats),
+            "depth_keys": depth_keys, "depth_order": depth_order,
             "instance_keys": self._buf(L.instance_keys, i, np.uint16).copy(),
             "instance_points": self._buf(L.instance_points, i, np.uint32).copy(),
             "tile_ranges": self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2),
