@@ -462,6 +462,12 @@ __device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, c
 
 __device__ __forceinline__ bool has_slots(uint32_t box) { return __popc(box & 0xFFFFu) * __popc(box >> 16) <= kSlots; }
 
+// Slot of tile-local pixel (lx, ly), which lies in the box, of a box that has slots.
+__device__ __forceinline__ int slot_in(uint32_t box, int lx, int ly) {
+    const uint32_t cols = box & 0xFFFFu, rows = box >> 16;
+    return (ly - (__ffs(rows) - 1)) * __popc(cols) + (lx - (__ffs(cols) - 1));
+}
+
 // Slot of tile-local pixel (lx, ly), which lies in the box; -1 when the box has no slots.
 __device__ __forceinline__ int slot_of(uint32_t box, int lx, int ly) {
     const uint32_t cols = box & 0xFFFFu, rows = box >> 16;
@@ -568,12 +574,12 @@ __global__ void __launch_bounds__(T * T)
                 uint64_t over = reach != 0ull ? instances_over_pixel(my_box, px) : 0ull;
                 if (done) over = 0ull;
                 // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
-                auto blend = [&](uint32_t j, int slot, float G) {
+                auto blend = [&](uint32_t j, int slot, float G, auto has_slot) {
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     if (!INFERENCE) {
                         const float part = bw > 0.0f ? G * bw : 0.0f;
-                        if (slot >= 0) st.value[j][slot] = -part;
+                        if (decltype(has_slot)::value || slot >= 0) st.value[j][slot] = -part;
                         else if (part != 0.0f) atomicAdd(&blending_weights[__float_as_uint(st.head1[j].w) & kPointMask], part);
                     }
 #pragma unroll
@@ -599,9 +605,9 @@ __global__ void __launch_bounds__(T * T)
                         if (over != 0ull) {
                             const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
                             over &= over - 1ull;
-                            const int slot = slot_of(st.box[j], px.lx, px.ly);
+                            const int slot = slot_in(st.box[j], px.lx, px.ly);
                             const float G = st.value[j][slot];
-                            if (G != 0.0f) blend(j, slot, G);
+                            if (G != 0.0f) blend(j, slot, G, std::true_type{});
                         }
                     }
                 } else {
@@ -617,7 +623,7 @@ __global__ void __launch_bounds__(T * T)
                         } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
                             continue;
                         }
-                        blend(j, slot, G);
+                        blend(j, slot, G, std::false_type{});
                     }
                 }
             }
@@ -790,7 +796,7 @@ __global__ void __launch_bounds__(T * T)
                 uint64_t over = reach != 0ull ? instances_over_pixel(my_box, px) : 0ull;
                 if (done) over = 0ull;
                 // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
-                auto blend = [&](uint32_t j, int slot, float G) {
+                auto blend = [&](uint32_t j, int slot, float G, auto has_slot) {
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     const float one_minus_a = 1.0f - a;
@@ -808,7 +814,7 @@ __global__ void __launch_bounds__(T * T)
                     const float d_alpha = fmaf(tr, sd, (running + offset) * rcp);
                     const float d_opacity = d_alpha * G;
                     const float weight = bw > 0.0f ? bw : 0.0f;
-                    if (slot >= 0) {
+                    if (decltype(has_slot)::value || slot >= 0) {
                         st.value[j][slot] = -weight;
                         s_d_opacity[j][slot] = d_opacity;
                     } else {
@@ -830,9 +836,9 @@ __global__ void __launch_bounds__(T * T)
                         if (over != 0ull) {
                             const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
                             over &= over - 1ull;
-                            const int slot = slot_of(st.box[j], px.lx, px.ly);
+                            const int slot = slot_in(st.box[j], px.lx, px.ly);
                             const float G = st.value[j][slot];
-                            if (G != 0.0f) blend(j, slot, G);
+                            if (G != 0.0f) blend(j, slot, G, std::true_type{});
                         }
                     }
                 } else {
@@ -848,7 +854,7 @@ __global__ void __launch_bounds__(T * T)
                         } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
                             continue;
                         }
-                        blend(j, slot, G);
+                        blend(j, slot, G, std::false_type{});
                     }
                 }
             }
