@@ -433,8 +433,10 @@ __device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, c
     const float det = h0.w * h1.y - h1.x * h1.x;
     float x_lo = 0.0f, x_hi = (float)T, y_lo = 0.0f, y_hi = (float)T;
     if (det > 0.0f) {
-        const float rx = sqrtf(reach2 * (h1.y / det)) * 1.01f + 0.01f;
-        const float ry = sqrtf(reach2 * (h0.w / det)) * 1.01f + 0.01f;
+        // hardware reciprocal and square root (1 ulp) are plenty for a bound that is widened by a percent
+        const float scale = reach2 * __builtin_amdgcn_rcpf(det);
+        const float rx = __builtin_amdgcn_sqrtf(scale * h1.y) * 1.01f + 0.01f;
+        const float ry = __builtin_amdgcn_sqrtf(scale * h0.w) * 1.01f + 0.01f;
         if (rx < 1e6f && ry < 1e6f) {
             x_lo = fminf(fmaxf(ceilf(h0.x - rx - 0.5f) - (float)tile_x0, 0.0f), (float)T);
             x_hi = fminf(fmaxf(floorf(h0.x + rx - 0.5f) + 1.0f - (float)tile_x0, 0.0f), (float)T);
