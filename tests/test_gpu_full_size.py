@@ -201,3 +201,17 @@ def test_config4_large_frame_inference(gpu, oracle):
     H.assert_close(image.cpu().numpy(), ref["image"], RTOL, 2e-5, "image")
     H.assert_close(alpha.cpu().numpy(), ref["alpha"], RTOL, 1e-6, "alpha")
     H.assert_close(depth.cpu().numpy(), ref["depth_image"], RTOL, 1e-5, "depth")
+    del image, depth, alpha, ref
+
+    # the same 33,554,432 points through the Gaussian footprint's inference variant (sigma_world 0.002, cut at 3 sigma),
+    # 8x8 tiles: 63,860 tiles, close to the limit of the 16-bit tile key
+    from tests.test_oracle_gaussian import gcfg_of
+
+    kw = dict(sigma_world=0.002, sigma_cutoff=3.0)
+    image, depth, alpha = rasterize_points(view, pos_dev, feats_dev, opac_dev, tile=8, inference=True, mode=1, **kw)
+    torch.cuda.synchronize()
+    g = gcfg_of(oracle, hv, n, 8, 16, oracle.FEAT_DIRECT_F16, inference=True, **kw)
+    ref = oracle.raster_forward(g.base, pos, feats, opac, hv.w2c, gaussian=g)
+    np.testing.assert_array_equal(image.cpu().numpy().view(np.uint32), ref["image"].view(np.uint32))
+    np.testing.assert_array_equal(alpha.cpu().numpy().view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(depth.cpu().numpy(), ref["depth_image"], RTOL, 1e-5, "Gaussian footprint depth")
