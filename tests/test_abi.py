@@ -51,6 +51,8 @@ def test_header_is_plain_c_and_structs_match_ctypes(tmp_path):
         "inpc_raster_config": (_lib.RasterConfig, [f for f, _ in _lib.RasterConfig._fields_]),
         "inpc_raster_layout": (_lib.RasterLayout, [f for f, _ in _lib.RasterLayout._fields_]),
         "inpc_timing_record": (_lib.TimingRecord, [f for f, _ in _lib.TimingRecord._fields_]),
+        "inpc_gaussian_config": (_lib.GaussianConfig, [f for f, _ in _lib.GaussianConfig._fields_]),
+        "inpc_gaussian_layout": (_lib.GaussianLayout, [f for f, _ in _lib.GaussianLayout._fields_]),
     }
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', "int main(void) {"]
     for struct, (_, names) in fields.items():
@@ -99,6 +101,39 @@ def test_layout_query_on_the_host():
     small = _lib.RasterLayout()
     assert lib.inpc_raster_layout_query(C.byref(make_cfg(0, 64, 64, 8, 4)), C.byref(small)) == 0
     assert small.total_bytes > 0 and small.n_tiles == 64
+
+
+def test_gaussian_layout_query_on_the_host():
+    lib = _lib.lib()
+    n = 8_388_608
+    layout = _lib.GaussianLayout()
+    cfg = _lib.GaussianConfig(make_cfg(n, 1237, 822, tile=8), 0.0, 3.0, 0, 0)
+    assert lib.inpc_gaussian_layout_query(C.byref(cfg), C.byref(layout)) == 0
+    assert (layout.grid_width, layout.grid_height, layout.n_tiles) == (155, 103, 155 * 103)
+    assert layout.record_stride == 64 and layout.total_bytes % 256 == 0 and layout.end_bit == 14
+    assert layout.max_instances == 4 * n + 65536          # the default capacity
+    offsets = [layout.counters, layout.point_touched, layout.point_bounds, layout.point_record, layout.depth_order,
+               layout.depth_keys, layout.instance_keys, layout.instance_points, layout.tile_ranges]
+    assert all(o % 256 == 0 and o < layout.total_bytes for o in offsets) and len(set(offsets)) == len(offsets)
+    # a capacity of the caller's choice sizes the instance buffers (and, in training configurations, the gradient rows)
+    small = _lib.GaussianLayout()
+    cfg_small = _lib.GaussianConfig(make_cfg(n, 1237, 822, tile=8), 0.0, 3.0, n, 0)
+    assert lib.inpc_gaussian_layout_query(C.byref(cfg_small), C.byref(small)) == 0
+    assert small.max_instances == n and small.total_bytes < layout.total_bytes
+    inference = _lib.GaussianLayout()
+    cfg_inf = _lib.GaussianConfig(make_cfg(n, 1237, 822, tile=8, flags=_lib.RASTER_INFERENCE), 0.003, 3.0, 0, 0)
+    assert lib.inpc_gaussian_layout_query(C.byref(cfg_inf), C.byref(inference)) == 0
+    assert inference.total_bytes < layout.total_bytes     # no gradient rows
+    # refused on the host: inference without a cut, raw features outside inference, a capacity of 2^31 or more
+    bad_cut = _lib.GaussianConfig(make_cfg(10, 64, 64, flags=_lib.RASTER_INFERENCE), 0.003, 0.0, 0, 0)
+    assert lib.inpc_gaussian_layout_query(C.byref(bad_cut), C.byref(small)) == -1
+    raw_training = _lib.GaussianConfig(make_cfg(10, 64, 64, channels=4, mode=_lib.FEAT_RAW37_F16), 0.0, 3.0, 0, 0)
+    assert lib.inpc_gaussian_layout_query(C.byref(raw_training), C.byref(small)) == -1
+    too_many = _lib.GaussianConfig(make_cfg(10, 64, 64), 0.0, 3.0, 2**31, 0)
+    assert lib.inpc_gaussian_layout_query(C.byref(too_many), C.byref(small)) == -3
+    assert lib.inpc_gaussian_forward(C.byref(cfg), None, None, None, None, None, None, None, None, None, None, None, 0,
+                                     None) in (-1, -2)
+    assert lib.inpc_gaussian_layout_query(None, None) == -1
 
 
 @pytest.mark.parametrize("cfg,code", [
