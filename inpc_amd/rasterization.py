@@ -2,7 +2,7 @@
 
 Same names, arguments and error behaviour as B/torch_bindings/rasterization.py:15-189; the native
 side is libinpc_hip.so instead of the pybind11 module `_C`. On top of the reference's fixed shape
-(8x8 tiles, (N,36) fp16 SH features -> 4 channels) the constructor accepts the tile size, and
+(8x8 tiles, (N,36) fp16 SH features -> 4 channels) the constructor accepts a tile size, and
 `rasterize_points` exposes the direct-feature variants (C in {4, 8, 16}, fp32 or fp16 storage).
 
 Both footprints of the reference are there: BILINEAR (2x2 splat) and GAUSSIAN (screen-space Gaussian,
@@ -240,14 +240,22 @@ class _Rasterize(torch.autograd.Function):
 
 
 class INPCRasterizer(torch.nn.Module):
-    """Counterpart of B/torch_bindings/rasterization.py:104-189. `tile` is 8 in the reference
-    (B/rasterization/include/bilinear/config.h:23-25); 16 is the other supported size."""
+    """Counterpart of B/torch_bindings/rasterization.py:104-189. The reference's tiles are 8x8
+    (B/rasterization/include/bilinear/config.h:23-25, gaussian/config.h:23-25). `tile` = 8 or 16 fixes the size;
+    left at None, every mode gets the size that is fastest here without changing its results: 16 for the bilinear
+    footprint (its image does not depend on the tile size: a point reaches the same pixels either way), 8 for the
+    Gaussian one (whose tile bounds decide which pixels at the rim of a footprint are drawn)."""
 
-    def __init__(self, tile: int = 8) -> None:
+    def __init__(self, tile: Optional[int] = None) -> None:
         super().__init__()
-        if tile not in (8, 16):
+        if tile not in (None, 8, 16):
             raise ValueError("tile must be 8 or 16")
         self.tile = tile
+
+    def tile_for(self, mode: RasterizerMode) -> int:
+        if self.tile is not None:
+            return self.tile
+        return 8 if mode == RasterizerMode.GAUSSIAN else 16
 
     @staticmethod
     def extract_settings(view, mode: int) -> RasterizerSettings:
@@ -274,7 +282,8 @@ class INPCRasterizer(torch.nn.Module):
                 opacities: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         """(image (4,H,W), alpha (1,H,W), blending_weights (N,)); differentiable in features and
         opacities, positions get no gradient."""
-        return _Rasterize.apply(positions, features, opacities, self.extract_settings(view, mode), self.tile,
+        settings = self.extract_settings(view, mode)
+        return _Rasterize.apply(positions, features, opacities, settings, self.tile_for(settings.mode),
                                 _lib.FEAT_SH36_F16, 4)
 
     def render(self, view, mode: int, positions: torch.Tensor, features_raw: torch.Tensor,
@@ -285,7 +294,7 @@ class INPCRasterizer(torch.nn.Module):
         _require_known_mode(settings)
         positions, features_raw, _ = _checked_inputs(positions, features_raw, None, _lib.FEAT_RAW37_F16, 4)
         sigma_world = sigma_world_scale * self.extract_base_sigma_world(view.camera)
-        image, alpha, depth, _, _ = _forward_native(settings, positions, features_raw, None, self.tile, 4,
+        image, alpha, depth, _, _ = _forward_native(settings, positions, features_raw, None, self.tile_for(settings.mode), 4,
                                                     _lib.FEAT_RAW37_F16, inference=True, sigma_world=sigma_world,
                                                     sigma_cutoff=sigma_cutoff)
         return image, depth, alpha
@@ -300,7 +309,7 @@ class INPCRasterizer(torch.nn.Module):
         if scales is not None and scales.numel() == 0:   # the reference passes an empty tensor for "no scales"
             scales = None
         sigma_world = sigma_world_scale * self.extract_base_sigma_world(view.camera)
-        image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, self.tile, 4,
+        image, alpha, depth, _, _ = _forward_native(settings, positions, features, opacities, self.tile_for(settings.mode), 4,
                                                     _lib.FEAT_SH36_F16, inference=True, scales=scales,
                                                     sigma_world=sigma_world, sigma_cutoff=sigma_cutoff)
         return image, depth, alpha

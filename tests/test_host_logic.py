@@ -92,7 +92,12 @@ def test_gaussian_mode_is_a_known_mode():
 
 
 def test_tile_argument():
-    assert INPCRasterizer().tile == 8 and INPCRasterizer(16).tile == 16
+    assert INPCRasterizer(8).tile == 8 and INPCRasterizer(16).tile == 16
+    # left open, the tile size follows the mode: the bilinear image does not depend on it, the Gaussian one keeps the
+    # reference's 8x8
+    auto = INPCRasterizer()
+    assert auto.tile_for(RasterizerMode.BILINEAR) == 16 and auto.tile_for(RasterizerMode.GAUSSIAN) == 8
+    assert INPCRasterizer(8).tile_for(RasterizerMode.BILINEAR) == 8
     with pytest.raises(ValueError):
         INPCRasterizer(32)
 
