@@ -34,14 +34,27 @@ class View:
     position: Any   # (3,) float32 tensor on the GPU: camera centre in world space
 
 
+_framework_camera = False   # False: not looked up yet; None: the framework is not importable
+
+
+def _framework_camera_class():
+    """The NeRFICG framework's PerspectiveCamera, or None; looked up once (a failing import is not cached by
+    Python and costs a walk over sys.path every time)."""
+    global _framework_camera
+    if _framework_camera is False:
+        try:  # pragma: no cover - only with the NeRFICG framework on the path
+            from Cameras.Perspective import PerspectiveCamera as FrameworkCamera
+
+            _framework_camera = FrameworkCamera
+        except ImportError:
+            _framework_camera = None
+    return _framework_camera
+
+
 def is_perspective(camera) -> bool:
     """True for a pinhole camera: the framework's PerspectiveCamera when it is importable, else any
     object that carries the pinhole scalars."""
-    try:  # pragma: no cover - only with the NeRFICG framework on the path
-        from Cameras.Perspective import PerspectiveCamera as FrameworkCamera
-
-        if isinstance(camera, FrameworkCamera):
-            return True
-    except ImportError:
-        pass
+    framework = _framework_camera_class()
+    if framework is not None and isinstance(camera, framework):
+        return True
     return all(hasattr(camera, f) for f in _CAMERA_FIELDS)
