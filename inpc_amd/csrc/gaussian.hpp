@@ -32,6 +32,7 @@ constexpr uint32_t kManyColumns = 7u;               // 7 or more tile columns: t
 constexpr int kCntKept = 4;                         // instances that are sorted and drawn (0 when they do not fit)
 constexpr int kCntInstances64 = 6;                  // u64 at words 6, 7: exact instance count
 constexpr int kCntMulti = 8;                        // drawn points that touch more than one tile
+constexpr int kCntDirect = 9;                       // set by a backward blend that added gradients to the arrays directly
 constexpr int kPointsPerBlock = 1024;               // depth-ordered points per block of the instance kernels
 
 inline uint32_t record_stride(int channels) { return (uint32_t)align_up(32 + (size_t)channels * 4, 32); }
@@ -693,6 +694,7 @@ __global__ void __launch_bounds__(kBlock)
                   float* __restrict__ grad_features, float* __restrict__ grad_opacities) {
     if (counters[kCntKept] == 0u) return;
     const uint32_t n_multi = counters[kCntMulti];
+    const bool add = counters[kCntDirect] != 0u;
     const uint32_t stride = gridDim.x * kBlock;
     for (uint32_t m = blockIdx.x * kBlock + threadIdx.x; m < n_multi; m += stride) {
         const uint4 entry = multi_list[m];
@@ -714,14 +716,14 @@ __global__ void __launch_bounds__(kBlock)
             }
             sum[C] += tail.x;
         }
-        // added to what is there: instances without slots have put their share into the arrays directly
+        // stored, or added to what is there when instances without slots have put their share into the arrays directly
         float4* gf = (float4*)(grad_features + (size_t)point * C);
 #pragma unroll
         for (int q = 0; q < C / 4; ++q) {
-            const float4 old = gf[q];
+            const float4 old = add ? gf[q] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             gf[q] = make_float4(old.x + sum[4 * q], old.y + sum[4 * q + 1], old.z + sum[4 * q + 2], old.w + sum[4 * q + 3]);
         }
-        grad_opacities[point] += sum[C];
+        grad_opacities[point] = (add ? grad_opacities[point] : 0.0f) + sum[C];
     }
 }
 
@@ -735,7 +737,8 @@ __global__ void __launch_bounds__(T * T)
                      const uint32_t* __restrict__ inst_points, const char* __restrict__ records, uint32_t stride,
                      const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
                      const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_features,
-                     float* grad_opacities, GradRows grad_rows, int W, int H, uint32_t gw, float threshold, float reach2) {
+                     float* grad_opacities, GradRows grad_rows, uint32_t* counters, int W, int H, uint32_t gw, float threshold,
+                     float reach2) {
     constexpr int TT = T * T;
     __shared__ Stage<T, C> st;
     __shared__ float s_d_opacity[TT][kSlotStride];   // per staged instance and box pixel: d loss / d opacity
@@ -763,6 +766,7 @@ __global__ void __launch_bounds__(T * T)
         offset = grad_alpha[pix] * (1.0f - alpha_image[pix]) - final_dot;
     }
     float running = 0.0f;
+    bool used_direct = false;   // this thread has added a gradient to the arrays directly (an instance without slots)
 #pragma unroll
     for (int c = 0; c < C; ++c) s_grad_px[px.ly * T + px.lx][c] = g[c];
     float tr = 1.0f;
@@ -826,6 +830,7 @@ __global__ void __launch_bounds__(T * T)
                             for (int c = 0; c < C; ++c) atomicAdd(&grad_features[(size_t)point * C + c], weight * g[c]);
                         }
                         if (d_opacity != 0.0f) atomicAdd(&grad_opacities[point], d_opacity);
+                        used_direct = true;
                     }
                     tr *= one_minus_a;
                     if (tr < kTransmittanceThreshold) {
@@ -900,6 +905,8 @@ __global__ void __launch_bounds__(T * T)
             }
         }
     }
+    // the pass that adds the rows up has to add to the arrays instead of storing into them
+    if (__ballot(used_direct) != 0ull && lane == 0u) atomicOr(&counters[kCntDirect], 1u);
 }
 
 }  // namespace gaussian
