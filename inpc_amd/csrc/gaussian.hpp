@@ -284,10 +284,11 @@ __global__ void __launch_bounds__(kBlock)
     __shared__ uint32_t s_multi, s_multi_base;
     if (counters[kCntKept] == 0u) return;
     const uint32_t n_visible = counters[kCntVisible];
-    const uint32_t base = blockIdx.x * kPointsPerBlock;
-    if (base >= n_visible) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     for (int i = tid; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
+    // a block takes the chunks of 1024 points chunk, chunk + grid, ...: the histograms leave it once
+    for (uint32_t chunk = blockIdx.x; chunk * kPointsPerBlock < n_visible; chunk += gridDim.x) {
+    const uint32_t base = chunk * kPointsPerBlock;
     if (tid == 0) s_multi = 0u;
     uint32_t count[kPer], mine = 0;
 #pragma unroll
@@ -320,7 +321,7 @@ __global__ void __launch_bounds__(kBlock)
     if (tid == kBlock - 1) s_offset[kPointsPerBlock] = run;
     __syncthreads();
     const uint32_t total = s_offset[kPointsPerBlock];
-    const uint32_t out = block_base[blockIdx.x];
+    const uint32_t out = block_base[chunk];
     if (multi_list) {
         // Where a point's instances start, in the order they are created in: the backward pass collects the
         // gradient of a point that touches several tiles in rows numbered that way. The instance of tile (tx, ty)
@@ -362,7 +363,8 @@ __global__ void __launch_bounds__(kBlock)
         inst_points[out + s] = s_point[lo];
         radix::hist_add(s_hist, plan, tile);
     }
-    __syncthreads();
+    __syncthreads();   // the LDS arrays are reused by the next chunk
+    }
     radix::hist_flush(s_hist, plan, g_hist);
 }
 

@@ -1362,7 +1362,7 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
                     at<uint2>(ws, L.sorted_bounds), at<uint32_t>(ws, L.block_sums));
         INPC_LAUNCH("gaussian_touch_scan", gaussian::k_touch_scan, dim3(1), dim3(kScanBlock), stream,
                     at<uint32_t>(ws, L.block_sums), L.n_blocks, counters, L.prm.capacity);
-        INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(L.n_blocks), dim3(kBlock), stream,
+        INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(std::min(L.n_blocks, 2048u)), dim3(kBlock), stream,
                     order, (const uint2*)at<uint2>(ws, L.sorted_bounds),
                     (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,
                     at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a),
