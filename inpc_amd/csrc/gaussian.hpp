@@ -808,7 +808,8 @@ __global__ void __launch_bounds__(T * T)
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     const float one_minus_a = 1.0f - a;
-                    const float rcp = 1.0f / fmaxf(one_minus_a, kOneMinusAlphaEps);
+                    // hardware reciprocal (1 ulp): the gradients are compared to 1e-4, not to the bit
+                    const float rcp = __builtin_amdgcn_rcpf(fmaxf(one_minus_a, kOneMinusAlphaEps));
                     float sd = 0.0f;
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q) {
@@ -885,7 +886,7 @@ __global__ void __launch_bounds__(T * T)
                         const float weight = -v;
                         const float* gp = s_grad_px[(y_lo + yy) * T + x_lo + xx];
 #pragma unroll
-                        for (int c = 0; c < C; ++c) sum[c] += weight * gp[c];
+                        for (int c = 0; c < C; ++c) sum[c] = fmaf(weight, gp[c], sum[c]);
                         sum[C] += s_d_opacity[tid][slot];
                     }
                 }
