@@ -1,11 +1,11 @@
 """Writes the golden fixtures of this directory from the CPU oracle.
 
 The reference ships no vectors for the sampling / rasterization path and cannot run here (CUDA sources), so these
-fixtures do not come from it: they freeze the oracle's answers on two small seeded cases, so that a later change of
+fixtures do not come from it: they freeze the oracle's answers on three small seeded cases, so that a later change of
 the oracle (or of the canonical rules it encodes) shows up as a diff of committed data, and so that the HIP path is
 checked against data as well as against the oracle built from today's sources.
 
-    python tests/golden/make_golden.py          # rewrites sampler_small.npz and raster_small.npz
+    python tests/golden/make_golden.py          # rewrites sampler_small.npz, raster_small.npz, gaussian_small.npz
 """
 from __future__ import annotations
 
@@ -81,10 +81,27 @@ def raster_answers():
     return out
 
 
+def gaussian_answers():
+    """The raster case through the Gaussian footprint (training variance), 8x8 tiles."""
+    p = RASTER
+    hv, pos, feats, opac, gi, ga = raster_case()
+    base = O.make_config(p["n"], oracle_camera(hv), 8, p["channels"], O.FEAT_DIRECT_F32, 0)
+    g = O.GaussianConfig(base, 0.0, 3.0, 0, 0)
+    count = O.gaussian_instance_count(g, pos, hv.w2c)
+    ref = O.raster_forward(base, pos, feats, opac, hv.w2c, debug=True, gaussian=g, n_instances_hint=count)
+    gf, go, _ = O.raster_backward(base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c, gaussian=g)
+    keep = ("n_visible", "n_instances", "n_touched", "bounds", "screen_xy", "conic", "depth_keys", "depth_order",
+            "instance_keys", "instance_points", "tile_ranges", "image", "alpha", "blending_weights")
+    out = {k: np.asarray(ref[k]) for k in keep}
+    out.update(grad_features=gf, grad_opacities=go)
+    return out
+
+
 def main():
     np.savez_compressed(HERE / "sampler_small.npz", **sampler_answers())
     np.savez_compressed(HERE / "raster_small.npz", **raster_answers())
-    for name in ("sampler_small.npz", "raster_small.npz"):
+    np.savez_compressed(HERE / "gaussian_small.npz", **gaussian_answers())
+    for name in ("sampler_small.npz", "raster_small.npz", "gaussian_small.npz"):
         print(name, (HERE / name).stat().st_size, "bytes")
 
 

@@ -1,4 +1,4 @@
-"""The committed fixtures of tests/golden (written by tests/golden/make_golden.py from the CPU oracle on two small
+"""The committed fixtures of tests/golden (written by tests/golden/make_golden.py from the CPU oracle on three small
 seeded cases): the oracle must still give them, and the HIP path must give them through the C ABI.
 
 Bit-exact: leaf weights, CDF, sample ids and positions, generator states, tile bounds, screen coordinates, depth
@@ -51,6 +51,39 @@ def test_oracle_reproduces_raster_fixture(oracle, maker):
         np.testing.assert_array_equal(_bits(np.asarray(got[key])), _bits(want[key]), err_msg=key)
     for key, atol in CLOSE_RASTER.items():
         np.testing.assert_allclose(got[key], want[key], rtol=RTOL, atol=atol, err_msg=key)
+
+
+EXACT_GAUSSIAN = EXACT_RASTER + ("conic", "image", "alpha")   # one fixed fp32 sequence for the footprint on both sides
+CLOSE_GAUSSIAN = {"blending_weights": 1e-7, "grad_features": 2e-7, "grad_opacities": 1e-6}
+
+
+def test_oracle_reproduces_gaussian_fixture(oracle, maker):
+    want = np.load(GOLDEN / "gaussian_small.npz")
+    got = maker.gaussian_answers()
+    for key in EXACT_GAUSSIAN:
+        np.testing.assert_array_equal(_bits(np.asarray(got[key])), _bits(want[key]), err_msg=key)
+    for key, atol in CLOSE_GAUSSIAN.items():
+        np.testing.assert_allclose(got[key], want[key], rtol=RTOL, atol=atol, err_msg=key)
+
+
+@pytest.mark.gpu
+def test_hip_gaussian_footprint_gives_fixture(gpu, maker):
+    from inpc_amd import _lib
+    from tests import helpers as H
+
+    want = np.load(GOLDEN / "gaussian_small.npz")
+    p = maker.RASTER
+    hv, pos, feats, opac, gi, ga = maker.raster_case()
+    run = H.GaussianRun(hv, pos, feats, opac, 8, p["channels"], _lib.FEAT_DIRECT_F32).forward()
+    dbg = run.debug()
+    out = run.outputs()
+    for key in EXACT_GAUSSIAN:
+        got = np.asarray(out[key] if key in out else dbg[key])
+        np.testing.assert_array_equal(_bits(got), _bits(want[key]), err_msg=key)
+    H.assert_close(out["blending_weights"], want["blending_weights"], RTOL, CLOSE_GAUSSIAN["blending_weights"], "weights")
+    gf, go = run.backward(gi, ga)
+    H.assert_close(gf, want["grad_features"], RTOL, CLOSE_GAUSSIAN["grad_features"], "feature gradients")
+    H.assert_close(go, want["grad_opacities"], RTOL, CLOSE_GAUSSIAN["grad_opacities"], "opacity gradients")
 
 
 @pytest.mark.gpu
