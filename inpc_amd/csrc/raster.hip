@@ -615,27 +615,39 @@ __device__ unsigned long long g_blend_profile[8];
 #include "gaussian.hpp"
 
 // view-space feature gradient -> (N,36) fp16; a point that was not drawn has a zero view gradient and
-// gets zeros (kernels.cu:95)
+// gets zeros (kernels.cu:95). A point's 72 bytes are nine 8-byte words (word k = the four channels of coefficient
+// k); the wave's 64 points leave through LDS as one contiguous run.
 __global__ void __launch_bounds__(kBlock)
     k_sh_backward(const float* __restrict__ positions, const float* __restrict__ cam_position,
                   const float4* __restrict__ grad_view, __half* __restrict__ grad_features, uint32_t n) {
-    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    __half* out = grad_features + 36 * (size_t)i;
-    const float4 g = grad_view[i];
-    if (g.x == 0.0f && g.y == 0.0f && g.z == 0.0f && g.w == 0.0f) {
+    __shared__ uint2 s_out[kBlock * 9];
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x, lane = threadIdx.x & 63u;
+    uint2* stage = s_out + (threadIdx.x >> 6) * (64u * 9u);
+    uint2 word[9];
 #pragma unroll
-        for (int k = 0; k < 36; ++k) out[k] = __float2half_rn(0.0f);
-        return;
+    for (int k = 0; k < 9; ++k) word[k] = make_uint2(0u, 0u);
+    if (i < n) {
+        const float4 g = grad_view[i];
+        if (!(g.x == 0.0f && g.y == 0.0f && g.z == 0.0f && g.w == 0.0f)) {
+            const ShBasis s = sh_basis(positions[3 * (size_t)i], positions[3 * (size_t)i + 1], positions[3 * (size_t)i + 2],
+                                       cam_position);
+#pragma unroll
+            for (int k = 0; k < 9; ++k) {
+                const __half2 lo = __halves2half2(__float2half_rn(s.b[k] * g.x), __float2half_rn(s.b[k] * g.y));
+                const __half2 hi = __halves2half2(__float2half_rn(s.b[k] * g.z), __float2half_rn(s.b[k] * g.w));
+                word[k] = make_uint2(*reinterpret_cast<const uint32_t*>(&lo), *reinterpret_cast<const uint32_t*>(&hi));
+            }
+        }
     }
-    const ShBasis s = sh_basis(positions[3 * (size_t)i], positions[3 * (size_t)i + 1], positions[3 * (size_t)i + 2],
-                               cam_position);
 #pragma unroll
-    for (int k = 0; k < 9; ++k) {
-        out[4 * k + 0] = __float2half_rn(s.b[k] * g.x);
-        out[4 * k + 1] = __float2half_rn(s.b[k] * g.y);
-        out[4 * k + 2] = __float2half_rn(s.b[k] * g.z);
-        out[4 * k + 3] = __float2half_rn(s.b[k] * g.w);
+    for (int k = 0; k < 9; ++k) stage[lane * 9u + k] = word[k];
+    wave_sync();
+    const uint32_t wave_first = i - lane;
+    uint2* out = (uint2*)grad_features + (size_t)wave_first * 9;
+#pragma unroll
+    for (uint32_t r = 0; r < 9; ++r) {
+        const uint32_t flat = r * 64u + lane;
+        if (wave_first + flat / 9u < n) out[flat] = stage[flat];
     }
 }
 
@@ -1248,6 +1260,8 @@ int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: the fp32 gradient buffer must be 16-byte aligned");
     if (L.sh && (!cam_position || !positions))
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: positions / cam_position are null");
+    if (L.fmode == INPC_FEAT_SH36_F16 && ((uintptr_t)grad_features & 7u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_backward: the fp16 gradient buffer must be 8-byte aligned");
     rc = fill_u32(grad_view, 0u, (size_t)L.geo.n * L.C, stream);
     if (rc != INPC_OK) return rc;
     rc = fill_u32(grad_opacities, 0u, L.geo.n, stream);
@@ -1405,6 +1419,8 @@ int inpc_gaussian_backward(const inpc_gaussian_config* cfg, const float* grad_im
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: the fp32 gradient buffer must be 16-byte aligned");
     if (L.sh && (!cam_position || !positions))
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: positions / cam_position are null");
+    if (L.fmode == INPC_FEAT_SH36_F16 && ((uintptr_t)grad_features & 7u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_backward: the fp16 gradient buffer must be 8-byte aligned");
     rc = fill_u32(grad_view, 0u, (size_t)L.geo.n * L.C, stream);
     if (rc != INPC_OK) return rc;
     rc = fill_u32(grad_opacities, 0u, L.geo.n, stream);
