@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(kBlock)
                     } else {
                         const ShBasis sb = sh_basis(px, py, pz, cam_position);
                         if (FMODE == INPC_FEAT_SH36_F16) {
-                            rec[2] = sh_to_view(sb, (const __half*)features + 36 * (size_t)i);
+                            rec[2] = sh_to_view_aligned(sb, (const __half*)features + 36 * (size_t)i);
                         } else {
                             const __half* raw = (const __half*)features + 37 * (size_t)i;
                             rec[2] = sh_to_view(sb, raw + 1);

@@ -115,6 +115,24 @@ __device__ __forceinline__ float4 sh_to_view(const ShBasis& s, const __half* __r
     return make_float4(acc[0], acc[1], acc[2], acc[3]);
 }
 
+// The same for 36 coefficients that start on an 8-byte boundary: nine 8-byte loads (word k = the four channels of
+// coefficient k) instead of 36 two-byte ones.
+__device__ __forceinline__ float4 sh_to_view_aligned(const ShBasis& s, const __half* __restrict__ coeffs) {
+    const uint2* src = (const uint2*)coeffs;
+    uint2 w[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k) w[k] = src[k];
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 9; ++k) {
+        const __half2 lo = *reinterpret_cast<const __half2*>(&w[k].x), hi = *reinterpret_cast<const __half2*>(&w[k].y);
+        const float f[4] = {__low2float(lo), __high2float(lo), __low2float(hi), __high2float(hi)};
+#pragma unroll
+        for (int ch = 0; ch < 4; ++ch) acc[ch] = k == 0 ? s.b[0] * f[ch] : acc[ch] + s.b[k] * f[ch];
+    }
+    return make_float4(acc[0], acc[1], acc[2], acc[3]);
+}
+
 // ---- projection (kernels.cu:40-64) ---------------------------------------------------------------------------
 struct Projected {
     float sx, sy, depth;
@@ -409,7 +427,7 @@ __global__ void __launch_bounds__(kBinThreads)
                     } else {
                         const ShBasis sb = sh_basis(px[u], py[u], pz[u], cam_position);
                         if (FMODE == INPC_FEAT_SH36_F16) {
-                            rec[2] = sh_to_view(sb, (const __half*)features + 36 * (size_t)i);
+                            rec[2] = sh_to_view_aligned(sb, (const __half*)features + 36 * (size_t)i);
                         } else {
                             const __half* raw = (const __half*)features + 37 * (size_t)i;
                             rec[2] = sh_to_view(sb, raw + 1);
@@ -1185,7 +1203,7 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: blending weights are null");
     if (L.fmode == INPC_FEAT_DIRECT_F32 && ((uintptr_t)features & 15u) != 0)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: fp32 features must be 16-byte aligned");
-    if (L.fmode == INPC_FEAT_DIRECT_F16 && ((uintptr_t)features & 7u) != 0)
+    if ((L.fmode == INPC_FEAT_DIRECT_F16 || L.fmode == INPC_FEAT_SH36_F16) && ((uintptr_t)features & 7u) != 0)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: fp16 features must be 8-byte aligned");
 
     rc = fill_u32(at<uint32_t>(ws, L.zero_begin), 0u, L.zero_words, stream);
@@ -1355,6 +1373,8 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: per-point scales are an inference input");
     if (L.fmode == INPC_FEAT_DIRECT_F32 && ((uintptr_t)features & 15u) != 0)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: fp32 features must be 16-byte aligned");
+    if (L.fmode == INPC_FEAT_SH36_F16 && ((uintptr_t)features & 7u) != 0)
+        return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: fp16 features must be 8-byte aligned");
 
     rc = fill_u32(at<uint32_t>(ws, L.zero_begin), 0u, L.zero_words, stream);
     if (rc != INPC_OK) return rc;
