@@ -281,6 +281,30 @@ def main() -> int:
     except Exception as exc:  # the figure is optional
         print(f"bench.py: Gaussian footprint not measured: {exc}", file=sys.stderr)
 
+    # the reference's own shape through the operator layer: (N,36) fp16 SH features -> 4 channels, autograd step
+    # (forward + backward including the SH gradient), both footprints with the tile size the layer picks
+    reference_shape = None
+    try:
+        from inpc_amd import INPCRasterizer
+
+        sh = (torch.randn((n, 36), generator=gen, device=device) * 0.2).half().requires_grad_(True)
+        op1 = opacities.reshape(n, 1).clone().requires_grad_(True)
+        gi4 = torch.randn((4, H, W), generator=gen, device=device) * 1e-2
+        rasterizer = INPCRasterizer()
+        reference_shape = {}
+        for mode_name, mode_value in (("bilinear", 0), ("gaussian", 1)):
+            def api_step():
+                sh.grad = None
+                op1.grad = None
+                img, alp, _ = rasterizer(view, mode_value, positions, sh, op1)
+                torch.autograd.backward([img, alp], [gi4, grad_alpha])
+
+            api_step()
+            reference_shape[f"{mode_name}_ms_per_step"] = round(time_calls(api_step, max(args.steps // 2, 1)), 4)
+        del sh, op1
+    except Exception as exc:  # the figure is optional
+        print(f"bench.py: reference-shaped step not measured: {exc}", file=sys.stderr)
+
     # ---- per-kernel durations: HIP events around every launch, on the launch stream, same steps ----------
     with _lib.KernelTimer() as timer:
         for _ in range(args.steps):
@@ -359,6 +383,7 @@ def main() -> int:
             "graph_replay_ms": None if graph_ms is None else round(graph_ms, 4), "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
             "field_update_ms": round(field_ms, 4),
             "gaussian_footprint": gaussian,
+            "sh36_autograd_step": reference_shape,
             "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
             "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),
             "kernels": kernels,
