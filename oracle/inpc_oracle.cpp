@@ -22,8 +22,9 @@
 //                              :401-474 (blend), :476-579 (backward), :581-660 (inference)
 //
 // Where the reference leaves a result to scheduling (atomic compaction order, atomic sample
-// slots, the association order of cub's float reduce/scan) this file fixes one canonical
-// choice, stated at the function. Those choices are "parity unpinned" by the reference: it
+// slots, the association order of cub's float reduce/scan) or to the CUDA math library (the last
+// bits of expf / __expf in the Gaussian footprint) this file fixes one canonical choice, stated
+// at the function. Those choices are "parity unpinned" by the reference: it
 // ships no test, golden vector or fixture for this path, and the cub association order is not
 // recoverable from its sources. Everything else is pinned by tests/test_oracle_*.py against
 // published known answers, float64 closed forms, numpy's sort/search routines and brute force.
