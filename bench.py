@@ -93,6 +93,9 @@ def main() -> int:
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also launch three 1 GiB plain copies (the yardstick for profiler byte counters)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target duration of the CPU baseline leg")
+    ap.add_argument("--with-config4", action="store_true",
+                    help="also time the large-frame inference configuration (33,554,432 points @2473x1643, 16 fp16 "
+                         "channels): training draw + inference forward, reported in extra.config4_inference")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
@@ -361,6 +364,35 @@ def main() -> int:
                "sample": f"first {n_cpu} of the {n} points, same camera/image/channels/tiles, forward+backward, "
                          f"{reps} repetitions, {spent:.1f} s"}
 
+    config4 = None
+    if args.with_config4:
+        # free the training workload first: this one needs about 12 GB
+        del workspace, image, alpha, blending_weights, grad_features, grad_opacities, features, opacities
+        torch.cuda.empty_cache()
+        n4, W4, H4 = 33_554_432, 2473, 1643
+        hv4 = synthetic.camera_on_z(W4, H4, 2000.0, 6.0)
+        view4 = hv4.to_view(device)
+        oct4 = synthetic.octree_leaves(2_097_152, 11, 4.0, seed=0)
+        c4, l4, w4 = (torch.from_numpy(a).to(device) for a in (oct4.centers, oct4.levels, oct4.weights))
+        sampler4 = ProbabilityFieldSampler(seed=0)
+        pos4, _ = sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size)
+        draw4_ms = time_calls(lambda: sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size), 5)
+        feats4 = torch.randn((n4, 16), generator=gen, device=device, dtype=torch.float32).half()
+        opac4 = torch.sigmoid(torch.randn(n4, generator=gen, device=device, dtype=torch.float32))
+        config4 = {"workload": "33,554,432 pts @2473x1643, 16 channels stored fp16, inference forward",
+                   "training_draw_ms": round(draw4_ms, 3)}
+        for label, mode, tile4, kw in (("bilinear", 0, 16, {}),
+                                       ("gaussian", 1, 8, dict(sigma_world=0.002, sigma_cutoff=3.0))):
+            from inpc_amd import rasterize_points
+
+            def infer():
+                rasterize_points(view4, pos4, feats4, opac4, tile=tile4, inference=True, mode=mode, **kw)
+
+            infer()
+            ms = time_calls(infer, 5)
+            config4[f"{label}_forward_ms"] = round(ms, 3)
+            config4[f"{label}_Mpoints_per_s"] = round(n4 / (ms * 1e-3) / 1e6, 1)
+
     out = {
         "metric": "Mpoints/s, rasterizer fwd+bwd, 8M pts @1237x822 (ms/frame in ms_per_step)",
         "value": round(n / (ms_per_step * 1e-3) / 1e6, 2),
@@ -384,6 +416,7 @@ def main() -> int:
             "field_update_ms": round(field_ms, 4),
             "gaussian_footprint": gaussian,
             "sh36_autograd_step": reference_shape,
+            "config4_inference": config4,
             "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
             "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),
             "kernels": kernels,
