@@ -533,9 +533,6 @@ __device__ __forceinline__ uint64_t instances_over_pixel(uint32_t box, const Pix
     return wave_transpose_bits((uint64_t)lo | ((uint64_t)hi << 32));
 }
 
-#ifdef INPC_GS_PROFILE
-__device__ unsigned long long g_gs_profile[65536 * 4];
-#endif
 
 template <int T, int C, bool INFERENCE>
 __global__ void __launch_bounds__(T * T)
@@ -556,15 +553,8 @@ __global__ void __launch_bounds__(T * T)
     float depth_acc = 0.0f, tr = 1.0f;
     bool done = !px.inside;
     const uint2 range = ranges[tile];
-#ifdef INPC_GS_PROFILE
-    const unsigned long long prof_t0 = wall_clock64();
-    unsigned long long prof_iters = 0, prof_batches = 0;
-#endif
     for (uint32_t base = range.x; base < range.y; base += TT) {
         if (__syncthreads_count(done) == TT) break;
-#ifdef INPC_GS_PROFILE
-        ++prof_batches;
-#endif
         const uint32_t count = min((uint32_t)TT, range.y - base);
         if (tid < count) {
             stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2, threshold);
@@ -604,9 +594,6 @@ __global__ void __launch_bounds__(T * T)
                 };
                 if (all_slots) {   // the usual case, without the branches of the other one
                     while (__ballot(over != 0ull) != 0ull) {
-#ifdef INPC_GS_PROFILE
-                        ++prof_iters;
-#endif
                         if (over != 0ull) {
                             const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
                             over &= over - 1ull;
@@ -654,19 +641,6 @@ __global__ void __launch_bounds__(T * T)
             }
         }
     }
-#ifdef INPC_GS_PROFILE
-    if (lane == 0) {
-        unsigned long long* out = g_gs_profile + (size_t)blockIdx.x * 4;
-        if (tid == 0) {
-            out[0] = wall_clock64() - prof_t0;
-            out[1] = range.y - range.x;
-            out[2] = prof_batches;
-            out[3] = 0;
-        }
-        __threadfence();
-        atomicMax(&out[3], prof_iters);
-    }
-#endif
     if (px.inside) {
         const size_t n_pixels = (size_t)W * H, pix = (size_t)px.y * W + px.x;
 #pragma unroll

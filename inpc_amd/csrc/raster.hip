@@ -1309,13 +1309,6 @@ int inpc_debug_blend_profile(unsigned long long out[8], int reset) {
 }
 #endif
 
-#ifdef INPC_GS_PROFILE
-int inpc_debug_gs_profile(unsigned long long* out, size_t words) {
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(gaussian::g_gs_profile), words * sizeof(unsigned long long)) != hipSuccess) return -1;
-    return 0;
-}
-#endif
-
 #ifdef INPC_SORT_PROFILE
 int inpc_debug_sort_profile(unsigned long long out[8], int reset) {
     if (hipMemcpyFromSymbol(out, HIP_SYMBOL(inpc::radix::g_sort_profile), 8 * sizeof(unsigned long long)) != hipSuccess) return -1;
