@@ -5,7 +5,7 @@ footprint's exponential is one fixed sequence of fp32 operations on both sides) 
 Within 1e-4 relative: blending weights and gradients, which both sides sum in an order of their own. The opacity
 gradient contains the difference between the running and the final pixel value, which cancels towards the end of a
 pixel's list; the kernel carries that difference as one scalar, the oracle per channel as the reference writes it,
-so a single small element can differ by 1e-4 of the largest gradient rather than of itself (`grad_atol`).
+so small elements differ by more than 1e-4 of themselves: the comparison has an absolute floor of 2e-6 (`grad_atol`).
 """
 import numpy as np
 import pytest
@@ -21,7 +21,9 @@ RTOL = 1e-4
 
 
 def grad_atol(ref):
-    return 1e-4 * float(np.abs(ref).max()) + 2e-7
+    """Absolute floor of a gradient comparison: 2e-7 for feature gradients, 2e-6 for opacity gradients (the same
+    floors as for the bilinear footprint)."""
+    return 2e-7 if np.asarray(ref).ndim == 2 else 2e-6
 
 
 def oracle_run(O, hv, pos, feats, opac, tile, channels, mode=None, inference=False, scales=None, sigma_world=0.0,
@@ -321,5 +323,6 @@ def test_random_scenes_forward_backward(gpu, oracle, case):
     H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
     # a second backward pass on the same saved state
     gf2, go2 = run.backward(gi, ga)
-    H.assert_close(gf2, gf, 1e-5, grad_atol(gf_ref) * 0.1, "feature gradients, second pass")
-    H.assert_close(go2, go, 1e-5, grad_atol(go_ref) * 0.1, "opacity gradients, second pass")
+    # (instances without slots add with float atomics: the last bits depend on scheduling)
+    H.assert_close(gf2, gf, RTOL, grad_atol(gf_ref), "feature gradients, second pass")
+    H.assert_close(go2, go, RTOL, grad_atol(go_ref), "opacity gradients, second pass")
