@@ -232,7 +232,8 @@ __global__ void __launch_bounds__(kBlock)
 // One block: block_sums -> exclusive prefix in place; decides whether the instances fit. When they do not, nothing
 // is expanded or drawn (the 32-bit offsets could not even address them) and the count tells the caller.
 __global__ void __launch_bounds__(kScanBlock) k_touch_scan(uint32_t* __restrict__ block_sums, uint32_t n_blocks,
-                                                           uint32_t* counters, uint32_t capacity) {
+                                                           uint32_t* counters, uint32_t capacity,
+                                                           unsigned long long* generation, unsigned long long seed) {
     __shared__ uint32_t s_wave[kScanBlock / kWave];
     __shared__ uint32_t s_fits;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -242,6 +243,10 @@ __global__ void __launch_bounds__(kScanBlock) k_touch_scan(uint32_t* __restrict_
         s_fits = fits ? 1u : 0u;
         counters[kCntKept] = fits ? (uint32_t)total : 0u;
         counters[kCntInstances] = total > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)total;
+        // The stamp the backward pass marks its gradient rows with: a new one per forward pass *execution* (a full-period
+        // congruential step in the workspace, increment from the host's per-call seed), so that a captured graph, whose
+        // kernel arguments never change, still gets a new stamp on every replay.
+        if (generation) *generation = *generation * 6364136223846793005ull + (seed | 1ull);
     }
     __syncthreads();
     if (!s_fits) return;
@@ -654,12 +659,13 @@ __global__ void __launch_bounds__(T * T)
 // Gradient rows of the points that touch several tiles: one row per instance, numbered in the order the instances
 // are created in (a point's instances are neighbours): C + 1 values, then the two words of the call's stamp, padded
 // to whole 16-byte words. A block that ends early (every pixel saturated) leaves the rows of its remaining instances
-// unwritten: a row counts when it carries the stamp of this backward call (64 bits, unique per call and process),
-// so nothing has to be cleared.
+// unwritten: a row counts when it carries the stamp of the forward pass the rows were laid out by (64 bits, a new
+// value per execution of k_touch_scan, kept in the workspace), so nothing has to be cleared. Backward passes of one
+// forward pass share the stamp: they write the same rows.
 struct GradRows {
     float* values;
     const uint2* bounds;   // per point: tile bounds (looked up for points with kManyColumns or more tile columns)
-    uint32_t stamp_lo, stamp_hi;
+    const uint2* stamp;    // the workspace's current stamp
     __host__ __device__ static constexpr uint32_t words(int channels) { return (uint32_t)(channels + 6) / 4u * 4u; }
 };
 
@@ -671,6 +677,7 @@ __global__ void __launch_bounds__(kBlock)
     if (counters[kCntKept] == 0u) return;
     const uint32_t n_multi = counters[kCntMulti];
     const bool add = counters[kCntDirect] != 0u;
+    const uint2 stamp = *rows.stamp;
     const uint32_t stride = gridDim.x * kBlock;
     for (uint32_t m = blockIdx.x * kBlock + threadIdx.x; m < n_multi; m += stride) {
         const uint4 entry = multi_list[m];
@@ -681,7 +688,7 @@ __global__ void __launch_bounds__(kBlock)
         for (uint32_t r = first; r < first + n_rows; ++r) {
             const float4* in = (const float4*)(rows.values + (size_t)r * GradRows::words(C));
             const float4 tail = in[C / 4];
-            if (__float_as_uint(tail.y) != rows.stamp_lo || __float_as_uint(tail.z) != rows.stamp_hi) continue;
+            if (__float_as_uint(tail.y) != stamp.x || __float_as_uint(tail.z) != stamp.y) continue;
 #pragma unroll
             for (int q = 0; q < C / 4; ++q) {
                 const float4 v = in[q];
@@ -742,6 +749,7 @@ __global__ void __launch_bounds__(T * T)
         offset = grad_alpha[pix] * (1.0f - alpha_image[pix]) - final_dot;
     }
     float running = 0.0f;
+    const uint2 stamp = *grad_rows.stamp;
     bool used_direct = false;   // this thread has added a gradient to the arrays directly (an instance without slots)
 #pragma unroll
     for (int c = 0; c < C; ++c) s_grad_px[px.ly * T + px.lx][c] = g[c];
@@ -872,7 +880,7 @@ __global__ void __launch_bounds__(T * T)
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q)
                         out[q] = make_float4(sum[4 * q], sum[4 * q + 1], sum[4 * q + 2], sum[4 * q + 3]);
-                    out[C / 4] = make_float4(sum[C], __uint_as_float(grad_rows.stamp_lo), __uint_as_float(grad_rows.stamp_hi), 0.0f);
+                    out[C / 4] = make_float4(sum[C], __uint_as_float(stamp.x), __uint_as_float(stamp.y), 0.0f);
                 } else {
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q)   // the rows are 16-byte aligned (checked by the host)

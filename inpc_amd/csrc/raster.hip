@@ -942,7 +942,7 @@ struct GaussianLayout {
     uint32_t n_blocks;  // blocks of gaussian::kPointsPerBlock depth-ordered points
     size_t zero_begin, zero_words;
     size_t hist_depth, hist_tile, status_depth, status_tile, bases_depth, bases_tile, tile_order, block_sums;
-    size_t sorted_bounds, multi_list, grad_rows;
+    size_t sorted_bounds, multi_list, grad_rows, generation;
     size_t keys_a, keys_b, vals_a, vals_b, inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
 };
 
@@ -1026,8 +1026,9 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
     P.point_touched = take(n * 4);
     P.point_bounds = take(n * 8);
     L.sorted_bounds = take(n * 8);
-    L.multi_list = L.grad_rows = 0;
+    L.multi_list = L.grad_rows = L.generation = 0;
     if (!L.inference) {   // configurations with a backward pass
+        L.generation = take(8);   // never cleared: the stamp of the gradient rows carries on from call to call
         L.multi_list = take(n * 16);
         L.grad_rows = take(capacity * gaussian::GradRows::words(L.C) * 4);
     }
@@ -1110,8 +1111,8 @@ int launch_gaussian_blend_forward(const GaussianLayout& L, float* image, float* 
     return INPC_OK;
 }
 
-// A 64-bit value no other backward call of this or another process is likely to have used: a counter above a
-// start value drawn once per process.
+// A 64-bit value no other forward call of this or another process is likely to have used: a counter above a
+// start value drawn once per process. It seeds the step of the workspace's gradient-row stamp.
 uint64_t next_stamp() {
     static std::atomic<uint64_t> counter{[] {
         std::random_device rd;
@@ -1124,9 +1125,8 @@ template <int T, int C>
 int launch_gaussian_blend_backward(const GaussianLayout& L, const float* grad_image, const float* grad_alpha,
                                    const float* image, const float* alpha, float* grad_view, float* grad_opacities,
                                    void* ws, hipStream_t stream) {
-    const uint64_t stamp = next_stamp();
     const gaussian::GradRows rows{at<float>(ws, L.grad_rows), (const uint2*)at<uint2>(ws, L.pub.point_bounds),
-                                  (uint32_t)stamp, (uint32_t)(stamp >> 32)};
+                                  (const uint2*)at<uint2>(ws, L.generation)};
     INPC_LAUNCH("gaussian_blend_backward", (gaussian::k_blend_backward<T, C>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 (const uint32_t*)at<uint32_t>(ws, L.pub.instance_points), (const char*)at<char>(ws, L.pub.point_record),
@@ -1388,7 +1388,9 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
                     (const uint2*)at<uint2>(ws, L.pub.point_bounds), (const uint32_t*)counters,
                     at<uint2>(ws, L.sorted_bounds), at<uint32_t>(ws, L.block_sums));
         INPC_LAUNCH("gaussian_touch_scan", gaussian::k_touch_scan, dim3(1), dim3(kScanBlock), stream,
-                    at<uint32_t>(ws, L.block_sums), L.n_blocks, counters, L.prm.capacity);
+                    at<uint32_t>(ws, L.block_sums), L.n_blocks, counters, L.prm.capacity,
+                    L.inference ? (unsigned long long*)nullptr : at<unsigned long long>(ws, L.generation),
+                    (unsigned long long)next_stamp());
         INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(std::min(L.n_blocks, 2048u)), dim3(kBlock), stream,
                     order, (const uint2*)at<uint2>(ws, L.sorted_bounds),
                     (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,

@@ -102,6 +102,71 @@ def test_forward_backward_dense_opaque_scene(gpu, oracle, tile):
     H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
 
 
+def test_forward_backward_replay_from_a_graph_with_new_inputs(gpu, oracle):
+    # A captured step keeps its kernel arguments, so whatever tells this pass's gradient rows from an earlier
+    # pass's has to change on the device. The scene saturates (tiles end early and leave rows unwritten) and has
+    # points over several tiles; every replay gets new points in place and is checked against the oracle.
+    import ctypes as C
+    n, tile, channels = 90000, 8, 8
+    hv = synthetic.camera_on_z(97, 61, 90.0, 2.4)
+    rng = np.random.default_rng(41)
+
+    def inputs(seed):
+        pos = synthetic.cube_points(n, 1.2, seed)
+        feats, _ = synthetic.point_attributes(n, channels, "uniform", seed + 1)
+        opac = np.random.default_rng(seed + 2).uniform(0.3, 0.999, n).astype(np.float32)
+        return pos, feats, opac
+
+    pos, feats, opac = inputs(500)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, channels)
+    lib = _lib.lib()
+    Hh, Ww = hv.camera.height, hv.camera.width
+    gf = torch.empty((n, channels), dtype=torch.float32, device="cuda:0")
+    go = torch.empty((n,), dtype=torch.float32, device="cuda:0")
+    gi = torch.zeros((channels, Hh, Ww), dtype=torch.float32, device="cuda:0")
+    ga = torch.zeros((1, Hh, Ww), dtype=torch.float32, device="cuda:0")
+
+    def step():
+        s = _lib.current_stream()
+        _lib.check(lib.inpc_gaussian_forward(
+            C.byref(run.cfg), _lib.ptr(run.positions), _lib.ptr(run.features), _lib.ptr(run.opacities), None,
+            _lib.ptr(run.w2c), _lib.ptr(run.cam_position), _lib.ptr(run.image), _lib.ptr(run.alpha), _lib.ptr(run.bw),
+            None, _lib.ptr(run.ws), run.layout.total_bytes, s), "forward")
+        _lib.check(lib.inpc_gaussian_backward(
+            C.byref(run.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(run.image), _lib.ptr(run.alpha),
+            _lib.ptr(run.positions), _lib.ptr(run.cam_position), _lib.ptr(gf), _lib.ptr(go), None, _lib.ptr(run.ws),
+            run.layout.total_bytes, s), "backward")
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        step()   # warm-up outside the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step()
+    for replay in range(3):
+        pos, feats, opac = inputs(510 + 10 * replay)
+        new_gi = rng.normal(0, 1e-2, (channels, Hh, Ww)).astype(np.float32)
+        new_ga = rng.normal(0, 1e-2, (1, Hh, Ww)).astype(np.float32)
+        run.positions.copy_(H.dev(pos))
+        run.features.copy_(H.dev(feats))
+        run.opacities.copy_(H.dev(opac))
+        gi.copy_(H.dev(new_gi))
+        ga.copy_(H.dev(new_ga))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, channels)
+        assert (ref["alpha"] == 1.0).mean() > 0.3 and (ref["n_touched"] > 1).mean() > 0.2
+        out = run.outputs()
+        np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+        np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+        gf_ref, go_ref, _ = oracle.raster_backward(g.base, new_gi, new_ga, ref["image"], ref["alpha"], pos, feats,
+                                                   opac, hv.w2c, gaussian=g)
+        H.assert_close(gf.cpu().numpy(), gf_ref, RTOL, grad_atol(gf_ref), f"feature gradients, replay {replay}")
+        H.assert_close(go.cpu().numpy(), go_ref, RTOL, grad_atol(go_ref), f"opacity gradients, replay {replay}")
+
+
 @pytest.mark.parametrize("tile", [8, 16])
 def test_forward_sh36_and_backward(gpu, oracle, tile):
     n = 30000
