@@ -292,6 +292,9 @@ def test_instances_beyond_the_capacity_are_reported(gpu, oracle):
     assert rc == -2 and counters[1] == need and counters[3] == 0      # INPC_E_WORKSPACE, nothing drawn
     out = small.outputs()
     assert (out["image"] == 0).all() and (out["alpha"] == 0).all()
+    # the backward pass of a call that drew nothing gives zero gradients
+    gf, go = small.backward(np.ones_like(out["image"]), np.ones_like(out["alpha"]))
+    assert (gf == 0).all() and (go == 0).all()
     exact = H.GaussianRun(hv, pos, feats, opac, 8, 4, max_instances=need).forward()
     rc, counters = exact.counters()
     assert counters[1] == need and counters[3] == need
