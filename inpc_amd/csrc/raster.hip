@@ -690,6 +690,7 @@ struct Layout {
     size_t keys_a, keys_b, vals_a, vals_b;
     size_t inst_keys_a, inst_vals_a;
     size_t split_count, split_points, split_features, split_opacities, split_flags;  // points that straddle tiles
+    size_t ordered_records, tile_end;   // 0: the configuration has no backward pass
 };
 
 uint32_t float_bits(float f) {
@@ -771,10 +772,14 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.split_count = take(kBinBlocks * 4);
     L.split_points = take(n * 4);
     L.split_flags = take(n * 4);
-    L.split_features = L.split_opacities = 0;
+    L.split_features = L.split_opacities = L.ordered_records = L.tile_end = 0;
     if (!L.inference && L.fmode != INPC_FEAT_RAW37_F16) {   // configurations with a backward pass
         L.split_features = take(4 * n * L.C * 4);
         L.split_opacities = take(4 * n * 4);
+        // the records once more, per instance and in the order of the tiles' lists, left by the forward blend for
+        // the backward blend; how far each tile's reach
+        L.ordered_records = take(ni * (2 + (size_t)L.C / 4) * 16);
+        L.tile_end = take((size_t)g.n_tiles * 4);
     }
     const bool depth_in_a = (L.depth_plan.n_passes % 2) == 0;
     P.depth_keys = depth_in_a ? L.keys_a : L.keys_b;
@@ -847,12 +852,13 @@ int launch_blend_forward(const Layout& L, float* image, float* alpha, float* ble
     const char* records = at<char>(ws, L.pub.point_record);
     if (L.inference) {
         INPC_LAUNCH("raster_blend_inference", (blend::k_blend_forward<T, C, HALF, true>), dim3(L.geo.n_tiles), dim3(T * T),
-                    stream, ranges, order, inst, records, L.geo.stride, image, alpha, (float*)nullptr, depth_image, L.geo.W,
-                    L.geo.H, L.geo.gw);
+                    stream, ranges, order, inst, records, L.geo.stride, image, alpha, (float*)nullptr, depth_image,
+                    (float4*)nullptr, (uint32_t*)nullptr, L.geo.W, L.geo.H, L.geo.gw);
     } else {
         INPC_LAUNCH("raster_blend_forward", (blend::k_blend_forward<T, C, HALF, false>), dim3(L.geo.n_tiles), dim3(T * T),
                     stream, ranges, order, inst, records, L.geo.stride, image, alpha, blending_weights, (float*)nullptr,
-                    L.geo.W, L.geo.H, L.geo.gw);
+                    L.tile_end ? at<float4>(ws, L.ordered_records) : (float4*)nullptr,
+                    L.tile_end ? at<uint32_t>(ws, L.tile_end) : (uint32_t*)nullptr, L.geo.W, L.geo.H, L.geo.gw);
     }
     return INPC_OK;
 }
@@ -865,7 +871,7 @@ int launch_blend_backward(const Layout& L, const float* grad_image, const float*
                                 (const uint32_t*)at<uint32_t>(ws, L.pub.counters) + kCntSplit};
     INPC_LAUNCH("raster_blend_backward", (blend::k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
-                at<uint32_t>(ws, L.pub.instance_slots), at<char>(ws, L.pub.point_record), L.geo.stride, grad_image,
+                (const float4*)at<float4>(ws, L.ordered_records), (const uint32_t*)at<uint32_t>(ws, L.tile_end), grad_image,
                 grad_alpha, image, alpha, grad_view,
                 grad_opacities, rows, L.geo.W, L.geo.H, L.geo.gw);
     INPC_LAUNCH("raster_grad_reduce", blend::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, 256u), 4096u)), dim3(256),
