@@ -426,16 +426,42 @@ struct Stage {
     float value[TT][kSlotStride];   // footprint value per pixel of the box (boxes of at most kSlots pixels)
 };
 
+// The record of this thread's instance of a coming batch, requested a batch ahead so that the gather (a line from
+// anywhere in the point records per instance) is under way while the current batch is blended; `after` is the point
+// of the thread's instance one batch further on.
+template <int C>
+struct Ahead {
+    float4 h0, h1, f[C / 4];
+    uint32_t after;
+    __device__ __forceinline__ void request(const char* __restrict__ record) {
+        const float4* src = (const float4*)record;
+        h0 = src[0];
+        h1 = src[1];
+#pragma unroll
+        for (int q = 0; q < C / 4; ++q) f[q] = src[2 + q];
+    }
+    // first batch and the point of the second
+    __device__ __forceinline__ void start(const uint32_t* __restrict__ inst_points, const char* __restrict__ records,
+                                          uint32_t stride, uint2 range, uint32_t block) {
+        h0 = h1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int q = 0; q < C / 4; ++q) f[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        after = 0u;
+        const uint32_t at = range.x + threadIdx.x;
+        if (at < range.y) request(records + (size_t)inst_points[at] * stride);
+        if (at + block < range.y) after = inst_points[at + block];
+    }
+};
+
 // Thread `slot` stages instance `slot` of the batch.
 template <int T, int C>
-__device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, const char* __restrict__ record,
-                                               int tile_x0, int tile_y0, float reach2, float threshold) {
-    const float4* src = (const float4*)record;
-    const float4 h0 = src[0], h1 = src[1];
+__device__ __forceinline__ void stage_instance(Stage<T, C>& st, uint32_t slot, const float4 h0, const float4 h1,
+                                               const float4 (&feat)[C / 4], int tile_x0, int tile_y0, float reach2,
+                                               float threshold) {
     st.head0[slot] = h0;
     st.head1[slot] = h1;
 #pragma unroll
-    for (int q = 0; q < C / 4; ++q) st.feat[slot * (C / 4) + q] = src[2 + q];
+    for (int q = 0; q < C / 4; ++q) st.feat[slot * (C / 4) + q] = feat[q];
     // cov = conic^-1; the footprint passes the threshold only where |dx| <= sqrt(reach2 * cov_x) (same in y).
     // Taken a little wider; anything odd (non-positive determinant, non-finite values) selects the whole tile.
     const float det = h0.w * h1.y - h1.x * h1.x;
@@ -558,11 +584,19 @@ __global__ void __launch_bounds__(T * T)
     float depth_acc = 0.0f, tr = 1.0f;
     bool done = !px.inside;
     const uint2 range = ranges[tile];
+    Ahead<C> ahead;
+    ahead.start(inst_points, records, stride, range, TT);
     for (uint32_t base = range.x; base < range.y; base += TT) {
         if (__syncthreads_count(done) == TT) break;
         const uint32_t count = min((uint32_t)TT, range.y - base);
-        if (tid < count) {
-            stage_instance<T, C>(st, tid, records + (size_t)inst_points[base + tid] * stride, tile_x0, tile_y0, reach2, threshold);
+        {
+            const float4 h0 = ahead.h0, h1 = ahead.h1;
+            float4 feat[C / 4];
+#pragma unroll
+            for (int q = 0; q < C / 4; ++q) feat[q] = ahead.f[q];
+            if (base + TT + tid < range.y) ahead.request(records + (size_t)ahead.after * stride);
+            if (base + 2u * TT + tid < range.y) ahead.after = inst_points[base + 2u * TT + tid];
+            if (tid < count) stage_instance<T, C>(st, tid, h0, h1, feat, tile_x0, tile_y0, reach2, threshold);
         }
         __syncthreads();
         if (__ballot(!done) != 0ull) {
@@ -769,25 +803,33 @@ __global__ void __launch_bounds__(T * T)
     float tr = 1.0f;
     bool done = !px.inside;
     const uint2 range = ranges[tile];
+    Ahead<C> ahead;
+    ahead.start(inst_points, records, stride, range, TT);
     for (uint32_t base = range.x; base < range.y; base += TT) {
         if (__syncthreads_count(done) == TT) break;
         const uint32_t count = min((uint32_t)TT, range.y - base);
         uint32_t my_row = 0u;
-        if (tid < count) {
-            const uint32_t point = inst_points[base + tid];
-            const char* record = records + (size_t)point * stride;
-            // the row of a point that touches several tiles is looked up now, long before it is needed: its
-            // instances were created row-major over its tile bounds
-            const uint32_t word = ((const uint32_t*)record)[7];
-            if (word & kMultiTile) {
-                uint32_t columns = (word >> kColumnsShift) & kManyColumns;
-                if (columns == kManyColumns) {
-                    const uint2 b = grad_rows.bounds[point];
-                    columns = (b.x >> 16) - (b.x & 0xFFFFu);
+        {
+            const float4 h0 = ahead.h0, h1 = ahead.h1;
+            float4 feat[C / 4];
+#pragma unroll
+            for (int q = 0; q < C / 4; ++q) feat[q] = ahead.f[q];
+            if (base + TT + tid < range.y) ahead.request(records + (size_t)ahead.after * stride);
+            if (base + 2u * TT + tid < range.y) ahead.after = inst_points[base + 2u * TT + tid];
+            if (tid < count) {
+                // the row of a point that touches several tiles is looked up now, long before it is needed: its
+                // instances were created row-major over its tile bounds
+                const uint32_t word = __float_as_uint(h1.w);
+                if (word & kMultiTile) {
+                    uint32_t columns = (word >> kColumnsShift) & kManyColumns;
+                    if (columns == kManyColumns) {
+                        const uint2 b = grad_rows.bounds[word & kPointMask];
+                        columns = (b.x >> 16) - (b.x & 0xFFFFu);
+                    }
+                    my_row = __float_as_uint(h1.z) + (tile / gw) * columns + tile % gw;
                 }
-                my_row = ((const uint32_t*)record)[6] + (tile / gw) * columns + tile % gw;
+                stage_instance<T, C>(st, tid, h0, h1, feat, tile_x0, tile_y0, reach2, threshold);
             }
-            stage_instance<T, C>(st, tid, record, tile_x0, tile_y0, reach2, threshold);
         }
         __syncthreads();
         if (__ballot(!done) != 0ull) {
