@@ -13,7 +13,9 @@
 //            lists); the results stay in the fragment list;
 //   write    thread t collects the results of instance t's fragments: a plain store when the point lies in
 //            one tile only, rows of its own when it straddles tiles (forward: atomics).
-// Two block barriers per batch; the record gather runs two batches ahead of the blend.
+// Two block barriers per batch. The forward pass gathers the records by slot, two batches ahead of the blend, and
+// (configurations with a backward pass) writes each record once more where its instance stands in the tile's list;
+// the backward pass reads those ordered records in contiguous runs, one batch ahead.
 #pragma once
 
 namespace blend {
