@@ -202,44 +202,103 @@ __device__ __forceinline__ void load_search_tree(float* s_tree, const float* __r
     __syncthreads();
 }
 
-__device__ __forceinline__ uint32_t cdf_search(const float* s_tree, const float* __restrict__ cdf, float sample,
-                                               uint32_t n) {
-    uint32_t first = 0, count = n, node = 1;
-    while (count > 0) {
-        const uint32_t step = count >> 1;
-        const uint32_t it = first + step;
-        const float v = node < kTreeNodes ? s_tree[node] : cdf[it];
-        if (v < sample) {
-            first = it + 1;
-            count -= step + 1;
-            node = 2u * node + 1u;
-        } else {
-            count = step;
-            node = 2u * node;
-        }
-    }
-    return min(first, n - 1);
-}
-
 struct Candidate {
     uint32_t leaf;
     float x, y, z;
 };
 
-// `r` stands at draw 4*k; leaves it at 4*k + 4. boxes[leaf] = {centre, edge length} (B/sampling/src/
-// sampling_kernels.cu:141-147: centre + (u - 0.5) * initial_size / 2^level).
-__device__ __forceinline__ Candidate draw_candidate(Pcg32& r, const float4* __restrict__ boxes,
-                                                    const float* __restrict__ cdf, const float* s_tree,
-                                                    uint32_t n_leaves) {
-    const float u = pcg_float(r);
-    const float ox = pcg_float(r), oy = pcg_float(r), oz = pcg_float(r);
-    Candidate c;
-    c.leaf = cdf_search(s_tree, cdf, u, n_leaves);
-    const float4 box = boxes[c.leaf];
-    c.x = box.x + (ox - 0.5f) * box.w;
-    c.y = box.y + (oy - 0.5f) * box.w;
-    c.z = box.z + (oz - 0.5f) * box.w;
-    return c;
+// A candidate k takes draws 4k .. 4k + 3 of the stream: u picks the leaf (lower_bound over the CDF, the probe
+// sequence of cdf_search above with the first kTreeDepth probes read from the tree), the other three place the
+// point in the leaf's cell; boxes[leaf] = {centre, edge length} (B/sampling/src/sampling_kernels.cu:141-147:
+// centre + (u - 0.5) * initial_size / 2^level).
+// ---- the kSampleItems candidates of a thread, side by side ---------------------------------------------------------
+// One candidate is a chain of dependent steps (four generator steps, up to 19 probes of the CDF, the box of the
+// leaf); a thread that takes its candidates one after the other spends its time waiting for the next link. Here the
+// chains of all its candidates advance together: every generator state comes from the thread's first one by a jump
+// of its own, and the searches run level by level for all candidates, without branches, so that the probes of one
+// level are in flight together. The values and comparisons are those of the sequential form.
+__device__ __forceinline__ float pcg_float_of(uint64_t state) {   // the output of the generator standing at `state`
+    const uint32_t xs = (uint32_t)(((state >> 18u) ^ state) >> 27u);
+    const uint32_t rot = (uint32_t)(state >> 59u);
+    const uint32_t v = (xs >> rot) | (xs << ((~rot + 1u) & 31u));
+    return __uint_as_float((v >> 9) | 0x3f800000u) - 1.0f;
+}
+
+struct TileJumps {
+    PcgJump row[kSampleItems];   // from the thread's first candidate of a tile to its j-th: 4 * kBlock * j draws
+    PcgJump draw[3];             // from a candidate's first draw to its second, third and fourth
+};
+
+__device__ __forceinline__ TileJumps make_tile_jumps(uint64_t inc) {
+    TileJumps t;
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) t.row[j] = pcg_jump(inc, 4ull * kBlock * (uint64_t)j);
+#pragma unroll
+    for (int d = 0; d < 3; ++d) t.draw[d] = pcg_jump(inc, (uint64_t)d + 1u);
+    return t;
+}
+
+// `state0`: the generator at the first draw of the thread's first candidate; live[j]: candidate j exists.
+__device__ __forceinline__ void draw_candidates(uint64_t state0, const TileJumps& jumps, const bool (&live)[kSampleItems],
+                                                const float4* __restrict__ boxes, const float* __restrict__ cdf,
+                                                const float* s_tree, uint32_t n_leaves, Candidate (&c)[kSampleItems]) {
+    float u[kSampleItems], ox[kSampleItems], oy[kSampleItems], oz[kSampleItems];
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) {
+        const uint64_t s = pcg_apply(jumps.row[j], state0);
+        u[j] = pcg_float_of(s);
+        ox[j] = pcg_float_of(pcg_apply(jumps.draw[0], s));
+        oy[j] = pcg_float_of(pcg_apply(jumps.draw[1], s));
+        oz[j] = pcg_float_of(pcg_apply(jumps.draw[2], s));
+    }
+    uint32_t first[kSampleItems], count[kSampleItems], node[kSampleItems];
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) {
+        first[j] = 0u;
+        count[j] = live[j] ? n_leaves : 0u;
+        node[j] = 1u;
+    }
+    // the probes whose element lies in the tree (a finished search keeps its node and reads it again)
+#pragma unroll 1
+    for (int level = 0; level < kTreeDepth; ++level) {
+#pragma unroll
+        for (int j = 0; j < kSampleItems; ++j) {
+            const bool active = count[j] > 0u;
+            const uint32_t step = count[j] >> 1;
+            const bool right = s_tree[node[j]] < u[j];
+            first[j] = active && right ? first[j] + step + 1u : first[j];
+            count[j] = !active ? 0u : right ? count[j] - (step + 1u) : step;
+            node[j] = active ? 2u * node[j] + (right ? 1u : 0u) : node[j];
+        }
+    }
+    // the probes below it read the CDF itself
+    bool more = false;
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) more = more || count[j] > 0u;
+    while (more) {
+        more = false;
+#pragma unroll
+        for (int j = 0; j < kSampleItems; ++j) {
+            const bool active = count[j] > 0u;
+            const uint32_t step = count[j] >> 1;
+            const bool right = cdf[min(first[j] + step, n_leaves - 1u)] < u[j];   // a finished search reads and drops
+            first[j] = active && right ? first[j] + step + 1u : first[j];
+            count[j] = !active ? 0u : right ? count[j] - (step + 1u) : step;
+            more = more || count[j] > 0u;
+        }
+    }
+    float4 box[kSampleItems];
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) {
+        c[j].leaf = min(first[j], n_leaves - 1u);
+        box[j] = boxes[c[j].leaf];
+    }
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) {
+        c[j].x = box[j].x + (ox[j] - 0.5f) * box[j].w;
+        c[j].y = box[j].y + (oy[j] - 0.5f) * box[j].w;
+        c[j].z = box[j].z + (oz[j] - 0.5f) * box[j].w;
+    }
 }
 
 // Generator of the first candidate of this thread: tile start (uniform jump) then 4*tid draws.
@@ -258,17 +317,21 @@ __global__ void __launch_bounds__(kBlock) k_sample(const float4* __restrict__ bo
     if (!(*sum_dev > 0.0f)) return;
     load_search_tree(s_tree, sum_dev);
     const uint64_t tile_first = (uint64_t)blockIdx.x * kSampleTile;
-    Pcg32 r = thread_generator(rng_dev, tile_first);
-    const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);  // from draw 4k+4 to 4(k+256)
+    const Pcg32 r = thread_generator(rng_dev, tile_first);
+    const TileJumps jumps = make_tile_jumps(r.inc);
+    bool live[kSampleItems];
+#pragma unroll
+    for (int j = 0; j < kSampleItems; ++j) live[j] = tile_first + (uint64_t)j * kBlock + threadIdx.x < n_samples;
+    Candidate c[kSampleItems];
+    draw_candidates(r.state, jumps, live, boxes, cdf, s_tree, n_leaves, c);
+#pragma unroll
     for (int j = 0; j < kSampleItems; ++j) {
         const uint64_t k = tile_first + (uint64_t)j * kBlock + threadIdx.x;
-        if (k < n_samples) {
-            const Candidate c = draw_candidate(r, boxes, cdf, s_tree, n_leaves);
-            positions[3 * k] = c.x;
-            positions[3 * k + 1] = c.y;
-            positions[3 * k + 2] = c.z;
-            if (leaf_ids) leaf_ids[k] = (int32_t)c.leaf;
-            r.state = pcg_apply(step, r.state);
+        if (live[j]) {
+            positions[3 * k] = c[j].x;
+            positions[3 * k + 1] = c[j].y;
+            positions[3 * k + 2] = c[j].z;
+            if (leaf_ids) leaf_ids[k] = (int32_t)c[j].leaf;
         }
     }
 }
@@ -305,10 +368,20 @@ __global__ void __launch_bounds__(kBlock)
     if (tid == 0) s_accepted0 = __hip_atomic_load(&st->accepted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     load_search_tree(s_tree, sum_dev);
     const Rows m = load_rows(w2c);
+    // The generator of a thread's first candidate of a tile = the tile's (start of the draw + 4 * first candidate of
+    // the tile) advanced by 4 * tid draws. The O(log) jumps are made once: by 4 * tid, from a candidate to the
+    // thread's j-th one of a tile, and from a tile of this block to its next one; per tile a few multiply-adds are left.
+    const uint64_t rng_inc = rng_dev[1];
+    const PcgJump jump_thread = pcg_jump(rng_inc, 4ull * tid);
+    const TileJumps jumps = make_tile_jumps(rng_inc);
+    const PcgJump jump_grid = pcg_jump(rng_inc, 4ull * (uint64_t)gridDim.x * kSampleTile);
+    uint64_t tile_state = pcg_apply(pcg_jump(rng_inc, 4ull * ((uint64_t)k0 + (uint64_t)blockIdx.x * kSampleTile)), rng_dev[0]);
     // Tiles in order: a tile waits (look-back) only for tiles in front of it, and those belong to blocks that are
     // running or to an earlier round of this grid, which stays resident as a whole (the host sizes it so):
     // no block has to end for another one to start.
     for (uint32_t bid = blockIdx.x; bid < n_blocks; bid += gridDim.x) {
+        const uint64_t state0 = pcg_apply(jump_thread, tile_state);
+        tile_state = pcg_apply(jump_grid, tile_state);
         if (tid == 0) {
             const uint32_t done = __hip_atomic_load(&st->consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
             s_done = done;
@@ -324,21 +397,16 @@ __global__ void __launch_bounds__(kBlock)
             continue;
         }
         const uint64_t tile_first = (uint64_t)bid * kSampleTile;  // relative to k0
-        Pcg32 r = thread_generator(rng_dev, (uint64_t)k0 + tile_first);
-        const PcgJump step = pcg_jump(r.inc, 4ull * kBlock - 4ull);
 
         Candidate cand[kSampleItems];
         uint32_t rank[kSampleItems];
         bool keep[kSampleItems];
 #pragma unroll
+        for (int j = 0; j < kSampleItems; ++j) keep[j] = tile_first + (uint64_t)j * kBlock + tid < n_candidates;
+        draw_candidates(state0, jumps, keep, boxes, cdf, s_tree, n_leaves, cand);
+#pragma unroll
         for (int j = 0; j < kSampleItems; ++j) {
-            const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
-            keep[j] = false;
-            if (rel < n_candidates) {
-                cand[j] = draw_candidate(r, boxes, cdf, s_tree, n_leaves);
-                keep[j] = sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
-                r.state = pcg_apply(step, r.state);
-            }
+            keep[j] = keep[j] && sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
             const uint64_t ballot = __ballot(keep[j]);
             rank[j] = mask_rank(ballot);
             if (lane == 0) s_count[j * (kBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
