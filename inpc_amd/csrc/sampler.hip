@@ -147,27 +147,18 @@ __global__ void __launch_bounds__(kBlock) k_chunk_add_prefix(float* data, uint32
     data[i] = inclusive_totals[c - 1] + data[i];
 }
 
-// std::lower_bound with the probe sequence of B/sampling/include/sampling_utils.h:49-69.
-__device__ __forceinline__ uint32_t cdf_search(const float* __restrict__ cdf, float sample, uint32_t n) {
-    uint32_t first = 0, count = n;
-    while (count > 0) {
-        const uint32_t step = count >> 1;
-        const uint32_t it = first + step;
-        if (cdf[it] < sample) {
-            first = it + 1;
-            count -= step + 1;
-        } else {
-            count = step;
-        }
-    }
-    return min(first, n - 1);
-}
-
-// The same search with the top of its decision tree in LDS. Which element the k-th probe reads depends only on
+// The leaf of a sample is std::lower_bound over the CDF with the probe sequence of
+// B/sampling/include/sampling_utils.h:49-69:
+//     first = 0, count = n;  while (count > 0) { step = count / 2; it = first + step;
+//         if (cdf[it] < sample) { first = it + 1; count -= step + 1; } else count = step; }
+//     leaf = min(first, n - 1)
+// draw_candidates below makes exactly these probes, level by level for all candidates of a thread.
+//
+// The top of the decision tree of that search lives in LDS. Which element the k-th probe reads depends only on
 // the outcomes of the probes before it, so the first kTreeDepth probes can only touch 2^kTreeDepth - 1 fixed
 // elements. inpc_build_cdf leaves those, in heap order (node 1 = first probe, node 2n / 2n + 1 = the probe after
 // going left / right), behind the total in the CDF head; a block copies them into LDS and reads the CDF itself
-// only below that depth. The comparisons are exactly those of cdf_search, so the result is the same even
+// only below that depth. The comparisons are exactly those of the sequence above, so the result is the same even
 // where rounding leaves the CDF not perfectly monotone; for 262,144 leaves 13 of the 18 dependent cache round
 // trips of a sample become LDS reads and the other five fall into one 128-byte line.
 constexpr int kTreeDepth = 13;
@@ -208,9 +199,10 @@ struct Candidate {
 };
 
 // A candidate k takes draws 4k .. 4k + 3 of the stream: u picks the leaf (lower_bound over the CDF, the probe
-// sequence of cdf_search above with the first kTreeDepth probes read from the tree), the other three place the
+// sequence above with the first kTreeDepth probes read from the tree), the other three place the
 // point in the leaf's cell; boxes[leaf] = {centre, edge length} (B/sampling/src/sampling_kernels.cu:141-147:
 // centre + (u - 0.5) * initial_size / 2^level).
+
 // ---- the kSampleItems candidates of a thread, side by side ---------------------------------------------------------
 // One candidate is a chain of dependent steps (four generator steps, up to 19 probes of the CDF, the box of the
 // leaf); a thread that takes its candidates one after the other spends its time waiting for the next link. Here the
