@@ -93,8 +93,8 @@ int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* 
 /* Bytes of scratch the CDF / counting passes need for n_leaves leaves. */
 size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
 
-/* Floats in the head of a CDF: the total and the top 13 levels of the search tree. */
-#define INPC_CDF_HEAD_FLOATS 8192
+/* Floats in the head of a CDF: the total and the top 14 levels of the search tree. */
+#define INPC_CDF_HEAD_FLOATS 16384
 
 /* Normalise the leaf weights and turn them into an inclusive CDF, in place.
  * Replaces compute_cdf (B/sampling/src/sampling.cu:150-186): cub::DeviceReduce::Sum, the
@@ -104,7 +104,7 @@ size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
  * `sum_out` (dev, INPC_CDF_HEAD_FLOATS floats, 16-byte aligned) is the head of the CDF: [0]
  * receives the un-normalised total; when it is <= 0 the weights are left un-normalised and later
  * sampling kernels take the failure path themselves. [1 .. INPC_CDF_HEAD_FLOATS - 1] receive
- * the CDF elements that the first 13 probes of the binary search of B/sampling/src/
+ * the CDF elements that the first 14 probes of the binary search of B/sampling/src/
  * sampling_kernels.cu:101-126 can read, in heap order; the sampling kernels keep them in LDS.
  * Every later call that takes `sum_dev` takes this buffer. No host synchronisation. */
 int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t workspace_bytes,

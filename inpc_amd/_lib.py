@@ -17,7 +17,7 @@ FEAT_DIRECT_F32 = 1
 FEAT_DIRECT_F16 = 2
 FEAT_RAW37_F16 = 3
 RASTER_INFERENCE = 1
-CDF_HEAD_FLOATS = 8192  # INPC_CDF_HEAD_FLOATS: total + the top of the CDF search tree
+CDF_HEAD_FLOATS = 16384  # INPC_CDF_HEAD_FLOATS: total + the top of the CDF search tree
 
 
 class Camera(C.Structure):

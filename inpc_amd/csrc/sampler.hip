@@ -26,7 +26,9 @@ constexpr int kChunk = 64;
 constexpr int kChunksPerBlock = 64;                      // one wave scans 64 chunks
 constexpr int kChunkTile = kChunk * kChunksPerBlock;     // 4096 floats per block
 constexpr int kSampleItems = 8;                          // candidates per thread
-constexpr int kSampleTile = kBlock * kSampleItems;       // candidates per block
+constexpr int kSampleTile = kBlock * kSampleItems;       // candidates per block (expected-count sampler)
+constexpr int kDrawBlock = 512;                          // threads per block of the sampling kernels that search the CDF
+constexpr int kDrawTile = kDrawBlock * kSampleItems;     // candidates per block of those
 
 struct Rows {
     float4 r1, r2, r3;
@@ -159,11 +161,15 @@ __global__ void __launch_bounds__(kBlock) k_chunk_add_prefix(float* data, uint32
 // elements. inpc_build_cdf leaves those, in heap order (node 1 = first probe, node 2n / 2n + 1 = the probe after
 // going left / right), behind the total in the CDF head; a block copies them into LDS and reads the CDF itself
 // only below that depth. The comparisons are exactly those of the sequence above, so the result is the same even
-// where rounding leaves the CDF not perfectly monotone; for 262,144 leaves 13 of the 18 dependent cache round
-// trips of a sample become LDS reads and the other five fall into one 128-byte line.
-constexpr int kTreeDepth = 13;
+// where rounding leaves the CDF not perfectly monotone; for 262,144 leaves 14 of the 18 dependent cache round
+// trips of a sample become LDS reads and the other four fall into one 64-byte stretch. The tree takes 64 KB of LDS,
+// shared by the 512 threads of a block (two blocks per CU); every probe that still reads the CDF itself is a load
+// whose 64 lanes touch 64 different lines and costs the kernel as much as all its arithmetic (13 levels for 256
+// threads: cull kernel 0.32 instead of 0.27 ms).
+constexpr int kTreeDepth = 14;
 constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNodes - 1; index 0 of the head: the total
 static_assert(kTreeNodes == INPC_CDF_HEAD_FLOATS, "the CDF head holds the total and the search tree");
+static_assert(kSampleItems * (kDrawBlock / kWave) <= kWave, "one wave scans the (round, wave) counts of a tile");
 
 // head[node] for every node of the tree (one thread per node).
 __global__ void __launch_bounds__(kBlock) k_build_search_tree(const float* __restrict__ cdf, float* __restrict__ head,
@@ -218,14 +224,14 @@ __device__ __forceinline__ float pcg_float_of(uint64_t state) {   // the output 
 }
 
 struct TileJumps {
-    PcgJump row[kSampleItems];   // from the thread's first candidate of a tile to its j-th: 4 * kBlock * j draws
+    PcgJump row[kSampleItems];   // from the thread's first candidate of a tile to its j-th: 4 * kDrawBlock * j draws
     PcgJump draw[3];             // from a candidate's first draw to its second, third and fourth
 };
 
 __device__ __forceinline__ TileJumps make_tile_jumps(uint64_t inc) {
     TileJumps t;
 #pragma unroll
-    for (int j = 0; j < kSampleItems; ++j) t.row[j] = pcg_jump(inc, 4ull * kBlock * (uint64_t)j);
+    for (int j = 0; j < kSampleItems; ++j) t.row[j] = pcg_jump(inc, 4ull * kDrawBlock * (uint64_t)j);
 #pragma unroll
     for (int d = 0; d < 3; ++d) t.draw[d] = pcg_jump(inc, (uint64_t)d + 1u);
     return t;
@@ -302,24 +308,24 @@ __device__ __forceinline__ Pcg32 thread_generator(const uint64_t* rng_dev, uint6
     return r;
 }
 
-__global__ void __launch_bounds__(kBlock) k_sample(const float4* __restrict__ boxes, const float* __restrict__ cdf,
+__global__ void __launch_bounds__(kDrawBlock) k_sample(const float4* __restrict__ boxes, const float* __restrict__ cdf,
                                                    const float* __restrict__ sum_dev, float* __restrict__ positions,
                                                    int32_t* __restrict__ leaf_ids, uint32_t n_samples, uint32_t n_leaves,
                                                    const uint64_t* __restrict__ rng_dev) {
     __shared__ __align__(16) float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
     load_search_tree(s_tree, sum_dev);
-    const uint64_t tile_first = (uint64_t)blockIdx.x * kSampleTile;
+    const uint64_t tile_first = (uint64_t)blockIdx.x * kDrawTile;
     const Pcg32 r = thread_generator(rng_dev, tile_first);
     const TileJumps jumps = make_tile_jumps(r.inc);
     bool live[kSampleItems];
 #pragma unroll
-    for (int j = 0; j < kSampleItems; ++j) live[j] = tile_first + (uint64_t)j * kBlock + threadIdx.x < n_samples;
+    for (int j = 0; j < kSampleItems; ++j) live[j] = tile_first + (uint64_t)j * kDrawBlock + threadIdx.x < n_samples;
     Candidate c[kSampleItems];
     draw_candidates(r.state, jumps, live, boxes, cdf, s_tree, n_leaves, c);
 #pragma unroll
     for (int j = 0; j < kSampleItems; ++j) {
-        const uint64_t k = tile_first + (uint64_t)j * kBlock + threadIdx.x;
+        const uint64_t k = tile_first + (uint64_t)j * kDrawBlock + threadIdx.x;
         if (live[j]) {
             positions[3 * k] = c[j].x;
             positions[3 * k + 1] = c[j].y;
@@ -346,13 +352,13 @@ struct CullState {
 };
 constexpr size_t kCullHeaderWords = sizeof(CullState) / 4;
 
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kDrawBlock)
     k_sample_cull(const float4* __restrict__ boxes, const float* __restrict__ cdf, const float* __restrict__ sum_dev,
                   const float* __restrict__ w2c, float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
                   uint32_t capacity, uint32_t k0, uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam,
                   const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
     __shared__ uint32_t s_accepted0, s_exclusive, s_done;
-    __shared__ uint32_t s_count[kSampleItems * (kBlock / kWave)];
+    __shared__ uint32_t s_count[kSampleItems * (kDrawBlock / kWave)];
     __shared__ __align__(16) float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
@@ -367,8 +373,8 @@ __global__ void __launch_bounds__(kBlock)
     const uint64_t rng_inc = rng_dev[1];
     const PcgJump jump_thread = pcg_jump(rng_inc, 4ull * tid);
     const TileJumps jumps = make_tile_jumps(rng_inc);
-    const PcgJump jump_grid = pcg_jump(rng_inc, 4ull * (uint64_t)gridDim.x * kSampleTile);
-    uint64_t tile_state = pcg_apply(pcg_jump(rng_inc, 4ull * ((uint64_t)k0 + (uint64_t)blockIdx.x * kSampleTile)), rng_dev[0]);
+    const PcgJump jump_grid = pcg_jump(rng_inc, 4ull * (uint64_t)gridDim.x * kDrawTile);
+    uint64_t tile_state = pcg_apply(pcg_jump(rng_inc, 4ull * ((uint64_t)k0 + (uint64_t)blockIdx.x * kDrawTile)), rng_dev[0]);
     // Tiles in order: a tile waits (look-back) only for tiles in front of it, and those belong to blocks that are
     // running or to an earlier round of this grid, which stays resident as a whole (the host sizes it so):
     // no block has to end for another one to start.
@@ -389,32 +395,32 @@ __global__ void __launch_bounds__(kBlock)
             __syncthreads();   // s_done is rewritten by the next tile
             continue;
         }
-        const uint64_t tile_first = (uint64_t)bid * kSampleTile;  // relative to k0
+        const uint64_t tile_first = (uint64_t)bid * kDrawTile;  // relative to k0
 
         Candidate cand[kSampleItems];
         uint32_t rank[kSampleItems];
         bool keep[kSampleItems];
 #pragma unroll
-        for (int j = 0; j < kSampleItems; ++j) keep[j] = tile_first + (uint64_t)j * kBlock + tid < n_candidates;
+        for (int j = 0; j < kSampleItems; ++j) keep[j] = tile_first + (uint64_t)j * kDrawBlock + tid < n_candidates;
         draw_candidates(state0, jumps, keep, boxes, cdf, s_tree, n_leaves, cand);
 #pragma unroll
         for (int j = 0; j < kSampleItems; ++j) {
             keep[j] = keep[j] && sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
             const uint64_t ballot = __ballot(keep[j]);
             rank[j] = mask_rank(ballot);
-            if (lane == 0) s_count[j * (kBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
+            if (lane == 0) s_count[j * (kDrawBlock / kWave) + wave] = (uint32_t)__popcll(ballot);
         }
         __syncthreads();
         if (wave == 0) {
             // exclusive scan of the 32 (round, wave) counts by the first lanes, then the block-level look-back
-            uint32_t c = lane < (uint32_t)(kSampleItems * (kBlock / kWave)) ? s_count[lane] : 0u;
+            uint32_t c = lane < (uint32_t)(kSampleItems * (kDrawBlock / kWave)) ? s_count[lane] : 0u;
             uint32_t incl = c;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
                 const uint32_t up = __shfl_up(incl, d, 64);
                 if (lane >= (uint32_t)d) incl += up;
             }
-            if (lane < (uint32_t)(kSampleItems * (kBlock / kWave))) s_count[lane] = incl - c;
+            if (lane < (uint32_t)(kSampleItems * (kDrawBlock / kWave))) s_count[lane] = incl - c;
             const uint32_t run = __shfl(incl, 63, 64);
             const uint32_t exclusive = lookback_exclusive_wave(status, bid, run, &st->error);
             if (lane == 0) {
@@ -427,14 +433,14 @@ __global__ void __launch_bounds__(kBlock)
 #pragma unroll
         for (int j = 0; j < kSampleItems; ++j) {
             if (!keep[j]) continue;
-            const uint64_t slot = base + s_count[j * (kBlock / kWave) + wave] + rank[j];
+            const uint64_t slot = base + s_count[j * (kDrawBlock / kWave) + wave] + rank[j];
             if (slot >= capacity) continue;
             positions[3 * slot] = cand[j].x;
             positions[3 * slot + 1] = cand[j].y;
             positions[3 * slot + 2] = cand[j].z;
             leaf_ids[slot] = (int32_t)cand[j].leaf;
             if (slot + 1 == capacity) {
-                const uint64_t rel = tile_first + (uint64_t)j * kBlock + tid;
+                const uint64_t rel = tile_first + (uint64_t)j * kDrawBlock + tid;
                 __hip_atomic_store(&st->consumed, (uint32_t)(k0 + rel + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
@@ -698,14 +704,14 @@ int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, floa
     if (n_leaves == 0 || !boxes || !cdf || !sum_dev || !positions_out || !rng_dev)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: null pointer or no leaves");
     if (((uintptr_t)boxes & 15u) != 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: boxes must be 16-byte aligned");
-    INPC_LAUNCH("sample", k_sample, dim3(div_up(n_samples, kSampleTile)), dim3(kBlock), stream, (const float4*)boxes, cdf,
+    INPC_LAUNCH("sample", k_sample, dim3(div_up(n_samples, kDrawTile)), dim3(kDrawBlock), stream, (const float4*)boxes, cdf,
                 sum_dev, positions_out, leaf_ids_out, n_samples, n_leaves, (const uint64_t*)rng_dev);
     INPC_LAUNCH("rng_advance", k_rng_advance, dim3(1), dim3(64), stream, rng_dev, sum_dev, 4ull * n_samples);
     return INPC_OK;
 }
 
 size_t inpc_cull_workspace_bytes(uint32_t n_candidates) {
-    return align_up((kCullHeaderWords + div_up(std::max(n_candidates, 1u), kSampleTile)) * 4, 256);
+    return align_up((kCullHeaderWords + div_up(std::max(n_candidates, 1u), kDrawTile)) * 4, 256);
 }
 
 int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream) {
@@ -732,14 +738,14 @@ int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* 
                     inpc_cull_workspace_bytes(n_candidates));
     CullState* st = (CullState*)workspace;
     uint32_t* status = (uint32_t*)workspace + kCullHeaderWords;
-    const uint32_t n_blocks = div_up(n_candidates, kSampleTile);
+    const uint32_t n_blocks = div_up(n_candidates, kDrawTile);
     INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(n_blocks, kBlock)), dim3(kBlock), stream, status,
                 n_blocks);
     // the whole grid must be resident at once: its blocks wait for each other's tiles
     uint32_t resident = 0;
-    const int rc = resident_blocks((const void*)k_sample_cull, kBlock, resident);
+    const int rc = resident_blocks((const void*)k_sample_cull, kDrawBlock, resident);
     if (rc != INPC_OK) return rc;
-    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(std::min(n_blocks, resident)), dim3(kBlock), stream,
+    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(std::min(n_blocks, resident)), dim3(kDrawBlock), stream,
                 (const float4*)boxes, cdf, sum_dev, w2c, positions_out, leaf_ids_out, capacity, k0, n_candidates, n_blocks,
                 n_leaves, to_device_camera(*cam), rng_dev, st, status);
     return INPC_OK;
