@@ -111,11 +111,16 @@ __global__ void __launch_bounds__(kWave) k_chunk_pass(float* data, uint32_t n, f
     float norm = 1.0f;
     const bool normalise = SCAN && norm_sum != nullptr;
     if (normalise) norm = 1.0f / *norm_sum;
-    for (int r = 0; r < kChunksPerBlock; ++r) {
-        const size_t i = base + (size_t)r * kChunk + lane;
-        float v = i < n ? data[i] : 0.0f;
-        if (normalise) v *= norm;
-        tile[r * (kChunk + 1) + lane] = v;
+    // the loads of sixteen rows are issued together (one row at a time left the wave waiting on every load)
+    for (int r0 = 0; r0 < kChunksPerBlock; r0 += 16) {
+        float v[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const size_t i = base + (size_t)(r0 + k) * kChunk + lane;
+            v[k] = i < n ? data[i] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k) tile[(r0 + k) * (kChunk + 1) + lane] = normalise ? v[k] * norm : v[k];
     }
     __syncthreads();
     const size_t chunk_base = base + (size_t)lane * kChunk;
@@ -131,6 +136,7 @@ __global__ void __launch_bounds__(kWave) k_chunk_pass(float* data, uint32_t n, f
     }
     if (SCAN) {
         __syncthreads();
+#pragma unroll 16
         for (int r = 0; r < kChunksPerBlock; ++r) {
             const size_t i = base + (size_t)r * kChunk + lane;
             if (i < n) data[i] = tile[r * (kChunk + 1) + lane];
