@@ -30,6 +30,14 @@ def test_header_functions_are_exported_and_bound():
         assert hasattr(handle, name), f"{name} is declared but not exported"
 
 
+def test_header_constants_match_the_binder():
+    # the CDF head the callers allocate: the header's size is the one the Python layer uses
+    text = HEADER.read_text()
+    assert int(re.search(r"#define\s+INPC_CDF_HEAD_FLOATS\s+(\d+)", text).group(1)) == _lib.CDF_HEAD_FLOATS
+    for name in ("DIRECT_F32", "DIRECT_F16", "SH36_F16", "RAW37_F16"):
+        assert int(re.search(rf"#define\s+INPC_FEAT_{name}\s+(\d+)", text).group(1)) == getattr(_lib, f"FEAT_{name}")
+
+
 def test_every_entry_point_cites_the_interface_it_replaces():
     text = HEADER.read_text()
     # the comment block in front of each declaration names a file of the reference with line numbers
