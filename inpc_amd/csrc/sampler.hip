@@ -462,13 +462,14 @@ __global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks) {
 // Failure pattern of B/sampling/src/sampling.cu:107-111 when the weight sum is not positive.
 __global__ void __launch_bounds__(kBlock) k_cull_failure_fill(const float* __restrict__ sum_dev, float* positions,
                                                               int32_t* leaf_ids, uint32_t capacity) {
-    if (*sum_dev > 0.0f) return;
-    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= capacity) return;
-    positions[3 * (size_t)i] = 0.0f;
-    positions[3 * (size_t)i + 1] = 0.0f;
-    positions[3 * (size_t)i + 2] = 0.0f;
-    leaf_ids[i] = -1;
+    if (*sum_dev > 0.0f) return;   // the usual case: a small grid, so that returning costs next to nothing
+    const uint32_t stride = gridDim.x * kBlock;
+    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < capacity; i += stride) {
+        positions[3 * (size_t)i] = 0.0f;
+        positions[3 * (size_t)i + 1] = 0.0f;
+        positions[3 * (size_t)i + 2] = 0.0f;
+        leaf_ids[i] = -1;
+    }
 }
 
 __global__ void k_cull_finish(const float* sum_dev, uint64_t* rng_dev, const CullState* st, uint32_t capacity,
@@ -775,7 +776,7 @@ int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_i
     if (!sum_dev || !rng_dev || !workspace || workspace_bytes < sizeof(CullState))
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_cull_finish: null pointer");
     if (capacity > 0 && positions_out && leaf_ids_out)
-        INPC_LAUNCH("cull_failure_fill", k_cull_failure_fill, dim3(div_up(capacity, kBlock)), dim3(kBlock), stream,
+        INPC_LAUNCH("cull_failure_fill", k_cull_failure_fill, dim3(std::min(div_up(capacity, kBlock), 1024u)), dim3(kBlock), stream,
                     sum_dev, positions_out, leaf_ids_out, capacity);
     INPC_LAUNCH("cull_finish", k_cull_finish, dim3(1), dim3(64), stream, sum_dev, rng_dev, (const CullState*)workspace,
                 capacity, total_candidates);
