@@ -106,6 +106,13 @@ def test_layout_query_on_the_host():
     assert layout.total_bytes >= 8_388_608 * (64 + 4 * 6)
     # bits the tile sort has to look at
     assert layout.end_bit == (layout.n_tiles - 1).bit_length() == 12
+    # a configuration with a backward pass also holds one ordered record (64 bytes here) and one gradient row per
+    # possible instance; an inference configuration holds neither
+    inference = _lib.RasterLayout()
+    cfg_inf = make_cfg(8_388_608, 1237, 822)
+    cfg_inf.flags = _lib.RASTER_INFERENCE
+    assert lib.inpc_raster_layout_query(C.byref(cfg_inf), C.byref(inference)) == 0
+    assert layout.total_bytes - inference.total_bytes >= 4 * 8_388_608 * (64 + 4 * 8 + 4)
     small = _lib.RasterLayout()
     assert lib.inpc_raster_layout_query(C.byref(make_cfg(0, 64, 64, 8, 4)), C.byref(small)) == 0
     assert small.total_bytes > 0 and small.n_tiles == 64
