@@ -110,6 +110,17 @@ size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
 int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t workspace_bytes,
                    uint32_t n_leaves, void* stream);
 
+/* The same as inpc_build_cdf without a workspace argument: the chunk totals live in a scratch array
+ * built into the library (about 261 KB of device memory per GPU the library runs on, held until the
+ * process ends), so the call allocates nothing and takes nothing but inputs and outputs. It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory or size a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid allocation).
+ * At most INPC_BUILD_CDF_STATIC_MAX_LEAVES leaves (INPC_E_UNSUPPORTED beyond). All calls on one GPU
+ * share the one scratch array: calls that overlap on one GPU (different streams or threads) race;
+ * calls ordered on one stream do not. Nothing in the scratch has to be cleared between calls. */
+#define INPC_BUILD_CDF_STATIC_MAX_LEAVES 4194304u
+int inpc_build_cdf_static(float* weights_inout, float* sum_out, uint32_t n_leaves, void* stream);
+
 /* Multinomial leaf pick + uniform in-leaf jitter, no culling.
  * Replaces create_samples (B/sampling/src/sampling.cu:188-209) and create_samples_cu
  * (B/sampling/src/sampling_kernels.cu:128-150). Sample i uses the generator `rng_dev`

@@ -119,6 +119,7 @@ SIGNATURES = {
     "inpc_leaf_weights": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _CAM, _F, _P]),
     "inpc_sampler_workspace_bytes": (_SZ, [_U32]),
     "inpc_build_cdf": (C.c_int, [_P, _P, _P, _SZ, _U32, _P]),
+    "inpc_build_cdf_static": (C.c_int, [_P, _P, _U32, _P]),
     "inpc_sample": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _P, _P]),
     "inpc_cull_workspace_bytes": (_SZ, [_U32]),
     "inpc_cull_begin": (C.c_int, [_P, _SZ, _P]),

@@ -13,6 +13,7 @@
 // Candidate k always uses the sampler's generator advanced by 4*k draws. A thread walks candidates
 // 256 apart, so it pays one O(log k) jump at the start and one constant affine step per candidate.
 #include <algorithm>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -636,6 +637,64 @@ int launch_blocked_total(const float* data, uint32_t n, float* totals, float* su
     return INPC_OK;
 }
 
+// Sum, normalisation and inclusive scan of the n leaf weights in place; the head of the CDF into sum_out.
+// `totals` is scratch of plan_levels(n).total_floats floats; every element that is read has been written
+// by an earlier launch of the same call, so it needs no clearing.
+int launch_build_cdf(float* w, float* sum_out, float* totals, uint32_t n_leaves, hipStream_t stream) {
+    const LevelPlan plan = plan_levels(n_leaves);
+    int rc = launch_blocked_total(w, n_leaves, totals, sum_out, plan, stream);
+    if (rc != INPC_OK) return rc;
+    // down: local scans, level 0 normalises; stops once a level has a single chunk
+    float* cur = w;
+    uint32_t m = n_leaves;
+    int depth = 0;
+    for (;;) {
+        float* tot = totals + plan.offset[depth];
+        INPC_LAUNCH("chunk_scan", k_chunk_pass<true>, dim3(div_up(m, kChunkTile)), dim3(kWave), stream, cur, m, tot,
+                    (const float*)sum_out, depth == 0 ? (const float*)sum_out : (const float*)nullptr);
+        if (plan.size[depth] == 1) break;
+        cur = tot;
+        m = plan.size[depth];
+        ++depth;
+    }
+    // up: add the scanned chunk totals of level d+1 to level d
+    for (int d = depth - 1; d >= 0; --d) {
+        float* dst = d == 0 ? w : totals + plan.offset[d - 1];
+        const uint32_t dn = d == 0 ? n_leaves : plan.size[d - 1];
+        INPC_LAUNCH("chunk_add_prefix", k_chunk_add_prefix, dim3(div_up(dn, kBlock)), dim3(kBlock), stream, dst, dn,
+                    (const float*)(totals + plan.offset[d]), (const float*)sum_out);
+    }
+    INPC_LAUNCH("search_tree", k_build_search_tree, dim3(kTreeNodes / kBlock), dim3(kBlock), stream, (const float*)w,
+                sum_out, n_leaves);
+    return INPC_OK;
+}
+
+// ---- built-in scratch of inpc_build_cdf_static ------------------------------------------------------------------
+// Chunk totals for up to INPC_BUILD_CDF_STATIC_MAX_LEAVES leaves (levels of 65536, 1024, 64 and 64 floats). The
+// array's name is only a handle in host code: the address kernels can use comes from hipGetSymbolAddress,
+// once per device (every device holds its own copy).
+constexpr size_t kStaticTotalsFloats = 65536 + 1024 + 64 + 64;
+__device__ __align__(256) float g_static_totals[kStaticTotalsFloats];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+float* g_static_totals_ptr[kMaxDevices] = {};
+
+int static_totals(float*& out) {
+    int device = 0;
+    INPC_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(INPC_E_UNSUPPORTED, "device index %d out of range", device);
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_totals_ptr[device]) {
+        void* p = nullptr;
+        INPC_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_totals)));
+        if (!p) return fail(INPC_E_HIP, "hipGetSymbolAddress returned a null address for the built-in scratch");
+        g_static_totals_ptr[device] = (float*)p;
+    }
+    out = g_static_totals_ptr[device];
+    return INPC_OK;
+}
+
 }  // namespace
 
 size_t sampler_workspace_bytes(uint32_t n_leaves) {
@@ -668,39 +727,26 @@ size_t inpc_sampler_workspace_bytes(uint32_t n_leaves) { return sampler_workspac
 
 int inpc_build_cdf(float* w, float* sum_out, void* workspace, size_t workspace_bytes, uint32_t n_leaves,
                    void* stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
     if (n_leaves == 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: no leaves");
     if (!w || !sum_out || !workspace) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: null pointer");
     if (workspace_bytes < sampler_workspace_bytes(n_leaves))
         return fail(INPC_E_WORKSPACE, "inpc_build_cdf: workspace has %zu bytes, needs %zu", workspace_bytes,
                     sampler_workspace_bytes(n_leaves));
-    const LevelPlan plan = plan_levels(n_leaves);
-    float* totals = (float*)workspace;
-    int rc = launch_blocked_total(w, n_leaves, totals, sum_out, plan, stream);
+    return launch_build_cdf(w, sum_out, (float*)workspace, n_leaves, (hipStream_t)stream_);
+}
+
+int inpc_build_cdf_static(float* w, float* sum_out, uint32_t n_leaves, void* stream_) {
+    if (n_leaves == 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf_static: no leaves");
+    if (!w || !sum_out) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf_static: null pointer");
+    if (n_leaves > INPC_BUILD_CDF_STATIC_MAX_LEAVES)
+        return fail(INPC_E_UNSUPPORTED, "inpc_build_cdf_static: %u leaves exceed the %u the built-in scratch holds",
+                    n_leaves, (unsigned)INPC_BUILD_CDF_STATIC_MAX_LEAVES);
+    if (plan_levels(n_leaves).total_floats > kStaticTotalsFloats)
+        return fail(INPC_E_UNSUPPORTED, "inpc_build_cdf_static: the built-in scratch is too small for %u leaves", n_leaves);
+    float* totals = nullptr;
+    const int rc = static_totals(totals);
     if (rc != INPC_OK) return rc;
-    // down: local scans, level 0 normalises; stops once a level has a single chunk
-    float* cur = w;
-    uint32_t m = n_leaves;
-    int depth = 0;
-    for (;;) {
-        float* tot = totals + plan.offset[depth];
-        INPC_LAUNCH("chunk_scan", k_chunk_pass<true>, dim3(div_up(m, kChunkTile)), dim3(kWave), stream, cur, m, tot,
-                    (const float*)sum_out, depth == 0 ? (const float*)sum_out : (const float*)nullptr);
-        if (plan.size[depth] == 1) break;
-        cur = tot;
-        m = plan.size[depth];
-        ++depth;
-    }
-    // up: add the scanned chunk totals of level d+1 to level d
-    for (int d = depth - 1; d >= 0; --d) {
-        float* dst = d == 0 ? w : totals + plan.offset[d - 1];
-        const uint32_t dn = d == 0 ? n_leaves : plan.size[d - 1];
-        INPC_LAUNCH("chunk_add_prefix", k_chunk_add_prefix, dim3(div_up(dn, kBlock)), dim3(kBlock), stream, dst, dn,
-                    (const float*)(totals + plan.offset[d]), (const float*)sum_out);
-    }
-    INPC_LAUNCH("search_tree", k_build_search_tree, dim3(kTreeNodes / kBlock), dim3(kBlock), stream, (const float*)w,
-                sum_out, n_leaves);
-    return INPC_OK;
+    return launch_build_cdf(w, sum_out, totals, n_leaves, (hipStream_t)stream_);
 }
 
 int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, float* positions_out,
