@@ -58,8 +58,11 @@ typedef struct inpc_camera {
                                   (B/rasterization/src/bilinear/kernels.cu:106-184)        */
 
 /* ---- rasterizer flags ------------------------------------------------------------------ */
-#define INPC_RASTER_INFERENCE 1u /* write a depth image, no blending weights
-                                    (B/rasterization/src/bilinear/kernels.cu:422-495)      */
+#define INPC_RASTER_INFERENCE 1u     /* write a depth image, no blending weights
+                                        (B/rasterization/src/bilinear/kernels.cu:422-495)  */
+#define INPC_RASTER_KEEP_GEOMETRY 2u /* bilinear footprint: also keep every point's screen position, depth
+                                        and tile bounds in the workspace (layout field debug_geometry),
+                                        for callers that want to inspect the projection             */
 
 const char* inpc_last_error(void);
 int inpc_abi_version(void);
@@ -206,35 +209,43 @@ typedef struct inpc_raster_config {
     int32_t feature_mode; /* INPC_FEAT_*                                                           */
     uint32_t flags;       /* INPC_RASTER_*                                                         */
     inpc_camera cam;
+    uint32_t max_instances; /* bilinear footprint: (point, touched tile) pairs the workspace holds; 0: about
+                               1.06 (1 + 1/tile)^2 per point + 65536, what evenly spread points need with a
+                               margin; 4 * n_points can never be exceeded. Ignored by the Gaussian footprint,
+                               which takes its own (inpc_gaussian_config)                              */
 } inpc_raster_config;
 
 /* Offsets (bytes from the workspace base) of the buffers a caller may want to inspect.
  * The layout is private otherwise. Counts live in device memory.
  *
- * A drawn point owns one blend record of `record_stride` bytes; the records of the points whose first
- * touched tile is t occupy slots bin_start[t] .. bin_start[t+1]-1, in no particular order. Sorted
- * orders refer to record slots; the header of a record names its point:
- *   float sx, sy, opacity; u32 point id; u32 tile info; float depth; 2 unused words; then the view
- *   features (fp32, or fp16 for INPC_FEAT_DIRECT_F16).
- *   tile info: bits 0-15 first tile id, bit 16 spans two tiles in x, bit 17 in y, bit 18 drawn. */
+ * A drawn point owns the blend record at its own index in the record array (record_stride bytes):
+ *   float wx0, wx1, wy0, wy1: interpolation weights of the pixel columns Lx, Lx + 1 and rows Ly, Ly + 1 that
+ *     can lie closer than 1 to the point's screen position (L = floor(s - 0.5)), 0 where a pixel centre is 1
+ *     or more away; float opacity; u32 point index | bit 28: touches several tiles | bit 29 / 30: two tiles in
+ *     x / y; u32 (Lx + 1) | (Ly + 1) << 16; u32 first gradient row (training) or float depth (inference);
+ *     then the view features (fp32, or fp16 for INPC_FEAT_DIRECT_F16).
+ * The instances (point, touched tile) of tile t are instance_points[bin_start[t] .. bin_start[t + 1] - 1], in
+ * (depth bits, point index) order. */
 typedef struct inpc_raster_layout {
     size_t total_bytes;
-    size_t counters;        /* u32[16]: [0] n_visible, [1] n_instances, [2] error flag          */
-    size_t bin_start;       /* u32[n_tiles + 1]                                                 */
-    size_t point_record;    /* n_visible records of record_stride bytes, binned by first tile   */
-    size_t depth_order;     /* (N) u32: (record slot << 2 | span bits) in (depth, point id)
-                               order, first n_visible valid                                     */
-    size_t depth_keys;      /* (N) u32: matching depth keys, first n_visible valid              */
-    size_t instance_keys;   /* (4N) u16: tile id per instance in final order                    */
-    size_t instance_slots;  /* (4N) u32: record slot per instance in final order                */
-    size_t tile_ranges;     /* (n_tiles) {u32 begin, end}                                       */
+    size_t counters;        /* u32[16]: [0] n_visible, [1] n_instances, [2] error flag,
+                               [5] the instances do not fit max_instances: nothing was drawn      */
+    size_t bin_start;       /* u32[n_tiles + 1]: first instance of every tile                      */
+    size_t point_record;    /* (N) records of record_stride bytes, valid for drawn points          */
+    size_t instance_points; /* (max_instances) u32: point index per instance in final order        */
+    size_t tile_ranges;     /* (n_tiles) {u32 begin, end}; {0, 0} for a tile without instances      */
+    size_t debug_geometry;  /* (N) {float sx, sy, depth; u32 tile info} with INPC_RASTER_KEEP_GEOMETRY,
+                               else 0. tile info: bits 0-15 first tile, bit 16 / 17: two tiles in x / y,
+                               bit 18: drawn                                                        */
     uint32_t record_stride;
     uint32_t grid_width;
     uint32_t grid_height;
     uint32_t n_tiles;
     uint32_t end_bit;       /* bit length of n_tiles-1
                                (B/rasterization/include/rasterization_utils.h:3-13)             */
-    uint32_t depth_key_bias; /* depth_keys hold (float bits of the depth) - depth_key_bias       */
+    uint32_t depth_key_bias; /* instances are ordered by (float bits of the depth) - depth_key_bias */
+    uint32_t max_instances; /* the capacity in effect                                            */
+    uint32_t reserved;
 } inpc_raster_layout;
 
 /* Workspace size and layout for a configuration. Replaces the three growable blobs of
@@ -278,7 +289,10 @@ int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
                          size_t workspace_bytes, void* stream);
 
 /* Copy the rasterizer counters {n_visible, n_instances, error flag} to the host.
- * Synchronises `stream`. Returns INPC_E_DEVICE if the error flag is set. */
+ * Synchronises `stream`. Returns INPC_E_DEVICE if the error flag is set and INPC_E_WORKSPACE if the
+ * instances did not fit max_instances (the images of that call show the background: call again
+ * with a larger capacity; the reference reads the count back and resizes on every call,
+ * B/rasterization/src/bilinear/forward.cu:86-89,118-119). */
 int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* workspace,
                               uint32_t counters_host[3], void* stream);
 

@@ -12,11 +12,13 @@ PKG_DIR = Path(__file__).resolve().parent
 LIB_PATH = PKG_DIR / "libinpc_hip.so"
 
 INPC_OK = 0
+E_INVALID_ARGUMENT, E_WORKSPACE, E_UNSUPPORTED, E_HIP, E_DEVICE = -1, -2, -3, -4, -5
 FEAT_SH36_F16 = 0
 FEAT_DIRECT_F32 = 1
 FEAT_DIRECT_F16 = 2
 FEAT_RAW37_F16 = 3
 RASTER_INFERENCE = 1
+RASTER_KEEP_GEOMETRY = 2
 CDF_HEAD_FLOATS = 16384  # INPC_CDF_HEAD_FLOATS: total + the top of the CDF search tree
 
 
@@ -41,6 +43,7 @@ class RasterConfig(C.Structure):
         ("feature_mode", C.c_int32),
         ("flags", C.c_uint32),
         ("cam", Camera),
+        ("max_instances", C.c_uint32),
     ]
 
 
@@ -50,17 +53,17 @@ class RasterLayout(C.Structure):
         ("counters", C.c_size_t),
         ("bin_start", C.c_size_t),
         ("point_record", C.c_size_t),
-        ("depth_order", C.c_size_t),
-        ("depth_keys", C.c_size_t),
-        ("instance_keys", C.c_size_t),
-        ("instance_slots", C.c_size_t),
+        ("instance_points", C.c_size_t),
         ("tile_ranges", C.c_size_t),
+        ("debug_geometry", C.c_size_t),
         ("record_stride", C.c_uint32),
         ("grid_width", C.c_uint32),
         ("grid_height", C.c_uint32),
         ("n_tiles", C.c_uint32),
         ("end_bit", C.c_uint32),
         ("depth_key_bias", C.c_uint32),
+        ("max_instances", C.c_uint32),
+        ("reserved", C.c_uint32),
     ]
 
 

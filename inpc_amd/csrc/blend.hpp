@@ -13,24 +13,18 @@
 //            lists); the results stay in the fragment list;
 //   write    thread t collects the results of instance t's fragments: a plain store when the point lies in
 //            one tile only, rows of its own when it straddles tiles (forward: atomics).
-// Two block barriers per batch. The forward pass gathers the records by slot, two batches ahead of the blend, and
-// (configurations with a backward pass) writes each record once more where its instance stands in the tile's list;
-// the backward pass reads those ordered records in contiguous runs, one batch ahead.
+// Two block barriers per batch. The forward pass gathers the records by point index, two batches ahead of the blend,
+// and (configurations with a backward pass) writes each record once more where its instance stands in the tile's
+// list; the backward pass reads those ordered records in contiguous runs, one batch ahead.
+// A record carries the footprint of its point as preprocess computed it: the left / top candidate pixel and the
+// interpolation weights of the two candidate columns and rows, so a wave finds the fragment of an instance with a
+// few integer operations.
 #pragma once
 
 namespace blend {
 
 constexpr int kQuad = 8;             // a wave's pixel quad is 8 x 8
-#ifndef INPC_LONG_LIST
-#define INPC_LONG_LIST 32
-#endif
-constexpr uint32_t kLongList = INPC_LONG_LIST;
-#ifndef INPC_FWD_WAVES
-#define INPC_FWD_WAVES 1
-#endif
-#ifndef INPC_BWD_WAVES
-#define INPC_BWD_WAVES 1
-#endif  // lists longer than this are evaluated by the whole wave
+constexpr uint32_t kLongList = 32;   // lists longer than this are evaluated by the whole wave
 
 __device__ __forceinline__ uint64_t lanes_below() {
     const uint32_t lane = __lane_id();
@@ -125,7 +119,8 @@ struct Stage {
     static constexpr int NQ = TT / 64;
     float4 feat[TT * (C / 4)];
     float depth[WITH_DEPTH ? TT : 1];
-    float4 point[TT];                   // sx, sy, opacity of the staged instance
+    float4 weights[TT];                 // wx0, wx1, wy0, wy1 of the staged instance
+    float2 place[TT];                   // opacity, (Lx + 1) | (Ly + 1) << 16
     alignas(8) uint16_t frag[TT][4];    // per slot: the fragment field, written by the wave that placed the fragment
 };
 
@@ -139,14 +134,14 @@ struct QuadScratch {
 
 // The record header as the kernels use it.
 struct Header {
-    float sx, sy, opacity;
-    uint32_t point;
-    uint32_t tiles;  // raw word; see multi()
-    float depth;
-    uint32_t split;  // index among the points that touch several tiles
-    // the point touches more than one tile (kept as the raw word until the write phase: a flag derived
-    // at the load would make the gather wait for its own first reply)
-    __device__ __forceinline__ bool multi() const { return ((tiles >> 16) & 3u) != 0u; }
+    float wx0, wx1, wy0, wy1;   // weights of the candidate columns Lx, Lx + 1 and rows Ly, Ly + 1
+    float opacity;
+    uint32_t tag;     // point index | kRecordMulti | span bits (kept as the raw word until the write phase: a
+                      // flag derived at the load would make the gather wait for its own first reply)
+    uint32_t cell;    // (Lx + 1) | (Ly + 1) << 16
+    uint32_t extra;   // first gradient row (training, points that touch several tiles) or depth bits (inference)
+    __device__ __forceinline__ bool multi() const { return (tag & kRecordMulti) != 0u; }
+    __device__ __forceinline__ uint32_t point() const { return tag & kRecordIdMask; }
 };
 
 // Makes the value available here: the wait for an outstanding load that produces it lands at this point and not
@@ -154,56 +149,50 @@ struct Header {
 __device__ __forceinline__ void arrive(float& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void arrive(uint32_t& v) { asm volatile("" : "+v"(v)); }
 
-__device__ __forceinline__ Header read_header(const char* __restrict__ record) {
-    const float4 h0 = ((const float4*)record)[0];
-    const float4 h1 = ((const float4*)record)[1];
+__device__ __forceinline__ void arrive(Header& h) {
+    arrive(h.wx0);
+    arrive(h.wx1);
+    arrive(h.wy0);
+    arrive(h.wy1);
+    arrive(h.opacity);
+    arrive(h.tag);
+    arrive(h.cell);
+    arrive(h.extra);
+}
+
+__device__ __forceinline__ Header make_header(const float4 h0, const float4 h1) {
     Header h;
-    h.sx = h0.x;
-    h.sy = h0.y;
-    h.opacity = h0.z;
-    h.point = __float_as_uint(h0.w);
-    h.tiles = __float_as_uint(h1.x);
-    h.depth = h1.y;
-    h.split = __float_as_uint(h1.z);
+    h.wx0 = h0.x;
+    h.wx1 = h0.y;
+    h.wy0 = h0.z;
+    h.wy1 = h0.w;
+    h.opacity = h1.x;
+    h.tag = __float_as_uint(h1.y);
+    h.cell = __float_as_uint(h1.z);
+    h.extra = __float_as_uint(h1.w);
     return h;
 }
 
-// One candidate pixel of one axis: the one of the two candidates (left_pixel, left_pixel + 1) whose tile-local
-// index has parity `odd`; the float test of B/rasterization/src/bilinear/kernels.cu:284-285 and the
-// interpolation weight of :286-287, the same arithmetic as cover_axis.
-struct AxisCandidate {
-    int index;     // tile-local
-    bool hit;
-    float weight;
-};
-
-template <int T>
-__device__ __forceinline__ AxisCandidate candidate_of_parity(float s, int tile_origin, bool odd) {
-    AxisCandidate a;
-    const int first = left_pixel<T>(s, tile_origin);
-    a.index = first + ((((first & 1) != 0) != odd) ? 1 : 0);
-    const float d = fabsf(s - ((float)(tile_origin + a.index) + 0.5f));
-    a.hit = a.index >= 0 && a.index < T && !(d >= 1.0f);
-    a.weight = __saturatef(1.0f - d);
-    return a;
+__device__ __forceinline__ Header read_header(const char* __restrict__ record) {
+    return make_header(((const float4*)record)[0], ((const float4*)record)[1]);
 }
 
-// Interpolation weights of the four fragment slots of a point (whether the fragment exists or not).
+// Tile-local index of the left / top candidate pixel of a record.
+__device__ __forceinline__ int local_left(uint32_t cell_half, int tile_origin) { return (int)cell_half - 1 - tile_origin; }
+
+// The candidate (0: L, 1: L + 1) of one axis whose tile-local index has the parity `odd` (tiles start at even pixels).
+__device__ __forceinline__ int candidate_of_parity(int left, uint32_t odd) { return (left ^ (int)odd) & 1; }
+
+// Interpolation weights of the four fragment slots of a point in a tile (whether the fragment exists or not):
+// 16x16 tiles: slot = parity class (x parity | y parity << 1); 8x8 tiles: slot = candidate (kx | ky << 1).
 template <int T>
-__device__ __forceinline__ void slot_weights(float sx, float sy, int tile_x0, int tile_y0, float (&weight)[4]) {
-    if (T == 16) {
-        float wx[2], wy[2];
+__device__ __forceinline__ void slot_weights(const Header& h, int tile_x0, int tile_y0, float (&weight)[4]) {
+    const int lx = local_left(h.cell & 0xFFFFu, tile_x0), ly = local_left(h.cell >> 16, tile_y0);
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            wx[b] = candidate_of_parity<T>(sx, tile_x0, b != 0).weight;
-            wy[b] = candidate_of_parity<T>(sy, tile_y0, b != 0).weight;
-        }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) weight[c] = wx[c & 1] * wy[c >> 1];
-    } else {
-        const AxisCover ax = cover_axis<T>(sx, tile_x0), ay = cover_axis<T>(sy, tile_y0);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) weight[c] = ax.weight[c & 1] * ay.weight[c >> 1];
+    for (int c = 0; c < 4; ++c) {
+        const int kx = T == 16 ? candidate_of_parity(lx, c & 1) : (c & 1);
+        const int ky = T == 16 ? candidate_of_parity(ly, c >> 1) : (c >> 1);
+        weight[c] = (kx ? h.wx1 : h.wx0) * (ky ? h.wy1 : h.wy0);
     }
 }
 
@@ -216,8 +205,9 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
     if (!valid) return;
 #pragma unroll
     for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
-    if (WITH_DEPTH) st.depth[t] = h.depth;
-    st.point[t] = make_float4(h.sx, h.sy, h.opacity, 0.0f);
+    if (WITH_DEPTH) st.depth[t] = __uint_as_float(h.extra);
+    st.weights[t] = make_float4(h.wx0, h.wx1, h.wy0, h.wy1);
+    st.place[t] = make_float2(h.opacity, __uint_as_float(h.cell));
     const uint2 nothing_placed = make_uint2(0u, 0u);
     __builtin_memcpy(st.frag[t], &nothing_placed, 8);
 }
@@ -243,32 +233,35 @@ __device__ __forceinline__ void load_entries(const Stage<T, C, WITH_DEPTH>& st, 
         const uint32_t j = k * 64u + lane;
         const bool live = j < count;
         e.j[k] = j;
-        const float4 p = st.point[live ? j : 0u];
+        const float4 w4 = st.weights[live ? j : 0u];
+        const float2 place = st.place[live ? j : 0u];
+        const uint32_t cell = __float_as_uint(place.y);
+        const int lx = local_left(cell & 0xFFFFu, tile_x0), ly = local_left(cell >> 16, tile_y0);
         bool hit[NF];
         uint32_t pix[NF];
         float weight[NF];
         if (T == 16) {
             // the fragment of this wave's parity class (x parity = quad & 1, y parity = quad >> 1)
-            const AxisCandidate cx = candidate_of_parity<T>(p.x, tile_x0, (quad & 1u) != 0u);
-            const AxisCandidate cy = candidate_of_parity<T>(p.y, tile_y0, (quad >> 1) != 0u);
-            hit[0] = cx.hit && cy.hit;
-            pix[0] = (uint32_t)((cy.index >> 1) * 8 + (cx.index >> 1));
-            weight[0] = cx.weight * cy.weight;
+            const int kx = candidate_of_parity(lx, quad & 1u), ky = candidate_of_parity(ly, quad >> 1);
+            const int cx = lx + kx, cy = ly + ky;
+            weight[0] = (kx ? w4.y : w4.x) * (ky ? w4.w : w4.z);
+            hit[0] = (uint32_t)(cx | cy) < (uint32_t)T && weight[0] > 0.0f;   // inside the tile, closer than 1 in x and y
+            pix[0] = (uint32_t)((cy >> 1) * 8 + (cx >> 1));
         } else {
-            const AxisCover ax = cover_axis<T>(p.x, tile_x0), ay = cover_axis<T>(p.y, tile_y0);
 #pragma unroll
             for (int q = 0; q < NF; ++q) {
                 const int ky = q >> 1, kx = q & 1;
-                hit[q] = ax.hit[kx] && ay.hit[ky];
-                pix[q] = (uint32_t)((ay.first + ky) * 8 + (ax.first + kx));
-                weight[q] = ax.weight[kx] * ay.weight[ky];
+                const int cx = lx + kx, cy = ly + ky;
+                weight[q] = (kx ? w4.y : w4.x) * (ky ? w4.w : w4.z);
+                hit[q] = (uint32_t)(cx | cy) < (uint32_t)T && weight[q] > 0.0f;
+                pix[q] = (uint32_t)(cy * 8 + cx);
             }
         }
 #pragma unroll
         for (int q = 0; q < NF; ++q) {
             const bool open = live && hit[q] && ((finished >> (pix[q] & kPixelMask)) & 1ull) == 0ull;
             e.pixel[k][q] = open ? pix[q] : kNoPixel;
-            e.alpha[k][q] = p.z * weight[q];
+            e.alpha[k][q] = place.x * weight[q];
         }
     }
 }
@@ -341,7 +334,7 @@ struct Gather {
 };
 
 template <int T, int C, bool HALF>
-__device__ __forceinline__ void start_gather(Gather<C>& g, const uint32_t* __restrict__ inst_slots,
+__device__ __forceinline__ void start_gather(Gather<C>& g, const uint32_t* __restrict__ inst_points,
                                              const char* __restrict__ records, uint32_t stride, uint2 range) {
     constexpr uint32_t TT = T * T;
     const uint32_t at = range.x + threadIdx.x;
@@ -351,9 +344,9 @@ __device__ __forceinline__ void start_gather(Gather<C>& g, const uint32_t* __res
     for (int c = 0; c < C; ++c) g.f[c] = g.f_next[c] = 0.0f;
     g.next_slot = 0u;
     uint32_t slot0 = 0u, slot1 = 0u;
-    if (at < range.y) slot0 = inst_slots[at];
-    if (at + TT < range.y) slot1 = inst_slots[at + TT];
-    if (at + 2u * TT < range.y) g.next_slot = inst_slots[at + 2u * TT];
+    if (at < range.y) slot0 = inst_points[at];
+    if (at + TT < range.y) slot1 = inst_points[at + TT];
+    if (at + 2u * TT < range.y) g.next_slot = inst_points[at + 2u * TT];
     if (at < range.y) {
         const char* record = records + (size_t)slot0 * stride;
         g.h = read_header(record);
@@ -370,18 +363,12 @@ __device__ __forceinline__ void start_gather(Gather<C>& g, const uint32_t* __res
 // waiting for the gather never waits for those stores: takes the record of the next batch (requested a whole
 // batch ago) and requests the record of the batch after it and the slot of the one after that.
 template <int T, int C, bool HALF>
-__device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __restrict__ inst_slots,
+__device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __restrict__ inst_points,
                                                const char* __restrict__ records, uint32_t stride, uint32_t begin,
                                                uint32_t end) {
     constexpr uint32_t TT = T * T;
     const uint32_t at = begin + threadIdx.x;
-    arrive(g.h_next.sx);
-    arrive(g.h_next.sy);
-    arrive(g.h_next.opacity);
-    arrive(g.h_next.point);
-    arrive(g.h_next.tiles);
-    arrive(g.h_next.depth);
-    arrive(g.h_next.split);
+    arrive(g.h_next);
 #pragma unroll
     for (int c = 0; c < C; ++c) arrive(g.f_next[c]);
     arrive(g.next_slot);
@@ -393,7 +380,7 @@ __device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __r
         g.h_next = read_header(record);
         load_record_features<C, HALF>(g.f_next, record);
     }
-    if (at + 3u * TT < end) g.next_slot = inst_slots[at + 3u * TT];
+    if (at + 3u * TT < end) g.next_slot = inst_points[at + 3u * TT];
 }
 
 // ---- ordered records: what the forward blend leaves for the backward blend ------------------------------------------
@@ -410,8 +397,9 @@ struct Ordered {
     }
     __device__ static __forceinline__ void store(float4* __restrict__ ordered, uint32_t begin, uint32_t count,
                                                  const Header& h, const float (&f)[C]) {
-        ordered[word(begin, count, 0)] = make_float4(h.sx, h.sy, h.opacity, __uint_as_float(h.point));
-        ordered[word(begin, count, 1)] = make_float4(__uint_as_float(h.tiles), h.depth, __uint_as_float(h.split), 0.0f);
+        ordered[word(begin, count, 0)] = make_float4(h.wx0, h.wx1, h.wy0, h.wy1);
+        ordered[word(begin, count, 1)] = make_float4(h.opacity, __uint_as_float(h.tag), __uint_as_float(h.cell),
+                                                     __uint_as_float(h.extra));
 #pragma unroll
         for (int q = 0; q < C / 4; ++q)
             ordered[word(begin, count, 2 + q)] = make_float4(f[4 * q], f[4 * q + 1], f[4 * q + 2], f[4 * q + 3]);
@@ -422,14 +410,7 @@ struct Ordered {
         if (begin >= end) return;
         const uint32_t count = min((uint32_t)blockDim.x, end - begin);
         if (threadIdx.x >= count) return;
-        const float4 h0 = ordered[word(begin, count, 0)], h1 = ordered[word(begin, count, 1)];
-        h.sx = h0.x;
-        h.sy = h0.y;
-        h.opacity = h0.z;
-        h.point = __float_as_uint(h0.w);
-        h.tiles = __float_as_uint(h1.x);
-        h.depth = h1.y;
-        h.split = __float_as_uint(h1.z);
+        h = make_header(ordered[word(begin, count, 0)], ordered[word(begin, count, 1)]);
 #pragma unroll
         for (int q = 0; q < C / 4; ++q) {
             const float4 v = ordered[word(begin, count, 2 + q)];
@@ -456,13 +437,7 @@ __device__ __forceinline__ void start_ordered(Gather<C>& g, const float4* __rest
 template <int T, int C>
 __device__ __forceinline__ void advance_ordered(Gather<C>& g, const float4* __restrict__ ordered, uint32_t begin,
                                                 uint32_t end) {
-    arrive(g.h_next.sx);
-    arrive(g.h_next.sy);
-    arrive(g.h_next.opacity);
-    arrive(g.h_next.point);
-    arrive(g.h_next.tiles);
-    arrive(g.h_next.depth);
-    arrive(g.h_next.split);
+    arrive(g.h_next);
 #pragma unroll
     for (int c = 0; c < C; ++c) arrive(g.f_next[c]);
     g.h = g.h_next;
@@ -473,9 +448,9 @@ __device__ __forceinline__ void advance_ordered(Gather<C>& g, const float4* __re
 
 // ---- forward ------------------------------------------------------------------------------------------------------
 template <int T, int C, bool HALF, bool INFERENCE>
-__global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1)
+__global__ void __launch_bounds__(T* T)
     k_blend_forward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
-                    const uint32_t* __restrict__ inst_slots,
+                    const uint32_t* __restrict__ inst_points,
                     const char* __restrict__ records, uint32_t stride, float* __restrict__ image,
                     float* __restrict__ alpha_image, float* blending_weights, float* __restrict__ depth_image,
                     float4* __restrict__ ordered_records, uint32_t* __restrict__ tile_end, int W, int H, uint32_t gw) {
@@ -499,23 +474,15 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
     bool done = !inside;
 
     const uint2 range = ranges[tile];
-#ifdef INPC_PROFILE_BACKWARD
-#define FWD_MARK(i)
-#else
-    INPC_PROF_DECL;
-#define FWD_MARK(i) INPC_PROF_MARK(i)
-#endif
     Gather<C> g;
-    start_gather<T, C, HALF>(g, inst_slots, records, stride, range);
+    start_gather<T, C, HALF>(g, inst_points, records, stride, range);
     uint32_t staged_end = range.x;   // the tile's instances in front of this one have been staged
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
         staged_end = begin + count;
         stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f);
-        FWD_MARK(0);
         __syncthreads();
-        FWD_MARK(1);
 
         // ---- consume: this wave's list
         uint32_t my_start = 0, my_count = 0, n_fragments = 0;
@@ -525,7 +492,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
             build_fragment_lists<T, C, INFERENCE>(qs, st, wave, e, my_start, my_count, n_fragments,
                                                   [&](int k, int) { return __uint_as_float(e.j[k]); });
         }
-        FWD_MARK(2);
         if (n_fragments != 0u) {
             // ---- pixels with short lists: the reference's sequential walk (kernels.cu:281-299)
             if (my_count <= kLongList) {
@@ -549,7 +515,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
                     done = done || Tr < kTransmittanceThreshold;
                 }
             }
-            FWD_MARK(3);
             // ---- pixels with long lists, one after the other, 64 fragments at a time over the wave
             uint64_t long_pixels = __ballot(my_count > kLongList);
             while (long_pixels) {
@@ -606,29 +571,21 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
                     done = Tr < kTransmittanceThreshold;
                 }
             }
-            FWD_MARK(4);
         }
-        FWD_MARK(2);
         const bool all_done = __syncthreads_and(done) != 0;
-        FWD_MARK(5);
-#if defined(INPC_BLEND_PROFILE) && !defined(INPC_PROFILE_BACKWARD)
-        ++prof_batches;
-#endif
         // ---- the gather moves on in front of the stores of the write phase
-        const uint32_t point = g.h.point;
-        const bool multi = g.h.multi();
-        const float sx = g.h.sx, sy = g.h.sy;
-        // the backward pass reads the records of this batch in runs (the gather by slot pulls a 128-byte line per
+        const Header mine = g.h;
+        // the backward pass reads the records of this batch in runs (a gather pulls a 128-byte line per
         // 64-byte record and was 0.13 ms of the backward blend)
         if (!INFERENCE && ordered_records && valid) Ordered<C>::store(ordered_records, begin, count, g.h, g.f);
-        advance_gather<T, C, HALF>(g, inst_slots, records, stride, begin, range.y);
+        advance_gather<T, C, HALF>(g, inst_points, records, stride, begin, range.y);
         // ---- write: thread t owns staged instance t (kernels.cu:291-295): its blending weight is the sum over
         // the fragments the waves placed
         if (!INFERENCE && valid) {
             uint32_t field[4];
             load_fields<T, C, INFERENCE>(st, tid, field);
             float weight[4];
-            slot_weights<T>(sx, sy, tile_x0, tile_y0, weight);
+            slot_weights<T>(mine, tile_x0, tile_y0, weight);
             float w = 0.0f;
 #pragma unroll
             for (int c = 0; c < 4; ++c)
@@ -637,16 +594,12 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
                     if (bw > 0.0f) w = fmaf(bw, weight[c], w);
                 }
             if (w > 0.0f) {
-                if (multi) atomicAdd(&blending_weights[point], w);
-                else blending_weights[point] = w;
+                if (mine.multi()) atomicAdd(&blending_weights[mine.point()], w);
+                else blending_weights[mine.point()] = w;
             }
         }
         if (all_done) break;
     }
-#ifndef INPC_PROFILE_BACKWARD
-    INPC_PROF_FLUSH;
-#endif
-#undef FWD_MARK
     // how far the ordered records of the tile reach: the backward pass goes no further
     if (!INFERENCE && tile_end && tid == 0) tile_end[tile] = staged_end;
     if (inside) {
@@ -660,50 +613,57 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_FWD_WAVES : 1
 }
 
 // ---- gradients of points that straddle tiles --------------------------------------------------------------------
-// A point that touches several tiles has an index s among such points (record header) and four rows, one per
-// tile: features[4 s + part][C], opacities[4 s + part], and a flag byte per row in flags[s]: the row has been
-// written. The flags are zero after the forward pass and after k_grad_reduce.
+// A point that touches several tiles has a list entry {point | touched tiles << 28, first row} and one gradient row
+// per touched tile, in the row-major order of its tiles: features[row][C], opacities[row], and a flag byte per
+// row: the row has been written. The flags are zero after the forward pass and after k_grad_reduce.
 struct SplitRows {
     float* features;
     float* opacities;
-    uint32_t* flags;
-    const uint32_t* points;   // points[s]: the point
-    const uint32_t* count;    // number of such points
+    uint8_t* flags;
+    const uint2* list;
+    const uint32_t* count;    // number of list entries
 };
 
-// Which of the (at most 2 x 2) tiles of a point `tile` is: 0 the first (top left), 1 its right neighbour,
-// 2 the one below, 3 the one below right. `info` is the tile word of the record.
-__device__ __forceinline__ uint32_t tile_part(uint32_t tile, uint32_t info, uint32_t gw) {
-    const uint32_t delta = tile - (info & 0xFFFFu);
-    return delta >= gw ? 2u + (delta - gw) : delta;
+// Which of the (at most 2 x 2) tiles of a point the tile at (tile_x, tile_y) is, counted row-major.
+__device__ __forceinline__ uint32_t tile_rank(const Header& h, uint32_t tile_x, uint32_t tile_y, uint32_t tile_shift) {
+    const int left = (int)(h.cell & 0xFFFFu) - 1, top = (int)(h.cell >> 16) - 1;
+    const uint32_t x0 = (uint32_t)max(left, 0) >> tile_shift, y0 = (uint32_t)max(top, 0) >> tile_shift;
+    return (tile_y - y0) * ((h.tag & kRecordSpanX) ? 2u : 1u) + (tile_x - x0);
 }
 
-// gradient of the point = sum of its rows, in row order (the gradient buffers are zero before). All four rows are
+// gradient of the point = sum of its rows, in row order (the gradient buffers are zero before). All rows are
 // read whether written or not (stale rows are dropped by their flag): the reads are dense and independent.
 template <int C>
 __global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __restrict__ grad_view,
                                                      float* __restrict__ grad_opacities) {
     const uint32_t n = *rows.count;
     for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < n; s += gridDim.x * 256u) {
-        const uint32_t flags = rows.flags[s];
-        const uint32_t i = rows.points[s];
-        const float4* row = (const float4*)(rows.features + (size_t)s * 4u * C);
+        const uint2 entry = rows.list[s];
+        const uint32_t i = entry.x & kRecordIdMask, touched = entry.x >> 28, first = entry.y;
+        const float4* row = (const float4*)(rows.features + (size_t)first * C);
         float4 part[4][C / 4];
+        float part_opacity[4];
+        bool written[4];
+        bool any = false;
 #pragma unroll
-        for (int p = 0; p < 4; ++p)
+        for (int p = 0; p < 4; ++p) {
+            const bool exists = (uint32_t)p < touched;
+            written[p] = exists && rows.flags[first + (exists ? p : 0)] != 0;
+            any = any || written[p];
 #pragma unroll
-            for (int q4 = 0; q4 < C / 4; ++q4) part[p][q4] = row[p * (C / 4) + q4];
-        const float4 op = ((const float4*)rows.opacities)[s];
-        if (flags == 0u) continue;
-        rows.flags[s] = 0u;
-        const float part_opacity[4] = {op.x, op.y, op.z, op.w};
+            for (int q4 = 0; q4 < C / 4; ++q4)
+                part[p][q4] = exists ? row[p * (C / 4) + q4] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            part_opacity[p] = exists ? rows.opacities[first + p] : 0.0f;
+        }
+        if (!any) continue;
         float4 acc[C / 4];
 #pragma unroll
         for (int q4 = 0; q4 < C / 4; ++q4) acc[q4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         float opacity = 0.0f;
 #pragma unroll
         for (int p = 0; p < 4; ++p)
-            if ((flags >> (8 * p)) & 0xFFu) {
+            if (written[p]) {
+                rows.flags[first + p] = 0;
 #pragma unroll
                 for (int q4 = 0; q4 < C / 4; ++q4) {
                     acc[q4].x += part[p][q4].x;
@@ -725,12 +685,12 @@ __global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __re
 //   dot(T f + (F_running - F_final) / (1 - a), grad) + grad_alpha (1 - alpha_final) / (1 - a),
 // is T s + (R - S + grad_alpha (1 - alpha_final)) / (1 - a): the pixel walk carries two scalars, not 2C.
 template <int T, int C, bool HALF>
-__global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1)   // 16x16 tiles: registers for four blocks per CU
+__global__ void __launch_bounds__(T* T)
     k_blend_backward(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order,
                      const float4* __restrict__ ordered_records, const uint32_t* __restrict__ tile_end,
                      const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
                      const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_view,
-                     float* grad_opacities, SplitRows rows, int W, int H, uint32_t gw) {
+                     float* grad_opacities, SplitRows rows, int W, int H, uint32_t gw, uint32_t tile_shift) {
     constexpr int TT = T * T;
     constexpr int NQ = TT / 64;
     constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
@@ -770,12 +730,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
     float Tr = 1.0f, running = 0.0f;
     bool done = !inside;
 
-#ifdef INPC_PROFILE_BACKWARD
-    INPC_PROF_DECL;
-#define BWD_MARK(i) INPC_PROF_MARK(i)
-#else
-#define BWD_MARK(i)
-#endif
     // the records as the forward pass staged them, in the order of the tile's list; only as far as it got
     uint2 range = ranges[tile];
     range.y = min(range.y, tile_end[tile]);
@@ -785,9 +739,7 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
         stage_instance<T, C, false>(st, valid, g.h, g.f);
-        BWD_MARK(0);
         __syncthreads();
-        BWD_MARK(1);
 
         // ---- consume: this wave's list
         uint32_t my_start = 0, my_count = 0, n_fragments = 0;
@@ -819,7 +771,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
             build_fragment_lists<T, C, false>(qs, st, wave, e, my_start, my_count, n_fragments,
                                               [&](int k, int q) { return dots[k][q]; });
         }
-        BWD_MARK(2);
         if (n_fragments != 0u) {
             // ---- pixels with short lists: the sequential walk (kernels.cu:383-417)
             if (my_count <= kLongList) {
@@ -837,7 +788,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
                     done = done || Tr < kTransmittanceThreshold;
                 }
             }
-            BWD_MARK(3);
             // ---- pixels with long lists, one after the other, 64 fragments at a time over the wave
             uint64_t long_pixels = __ballot(my_count > kLongList);
             while (long_pixels) {
@@ -874,25 +824,17 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
                     done = Tr < kTransmittanceThreshold;
                 }
             }
-            BWD_MARK(4);
         }
-        BWD_MARK(2);
         const bool all_done = __syncthreads_and(done) != 0;
-        BWD_MARK(5);
-#if defined(INPC_PROFILE_BACKWARD) && defined(INPC_BLEND_PROFILE)
-        ++prof_batches;
-#endif
         // ---- the gather moves on in front of the stores of the write phase (see the forward kernel)
-        const uint32_t point = g.h.point, tiles = g.h.tiles, split = g.h.split;
-        const bool multi = g.h.multi();
-        const float sx = g.h.sx, sy = g.h.sy;
+        const Header mine = g.h;
         advance_ordered<T, C>(g, ordered_records, begin, range.y);
         // ---- write: thread t owns staged instance t: gradient of the point from the fragments the waves placed
         if (valid) {
             uint32_t field[4];
             load_fields<T, C, false>(st, tid, field);
             float weight[4];
-            slot_weights<T>(sx, sy, tile_x0, tile_y0, weight);
+            slot_weights<T>(mine, tile_x0, tile_y0, weight);
             float gf[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) gf[c] = 0.0f;
@@ -920,14 +862,13 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
             if (any_weight || gop != 0.0f) {
                 // a point that straddles tiles gets its gradient from up to four blocks: each writes a row of
                 // its own (summed up by k_grad_reduce); no atomics, and the sum has a fixed order
-                float* dst = grad_view + (size_t)point * C;
-                float* dst_opacity = grad_opacities + point;
-                if (multi) {
-                    const uint32_t part = tile_part(tile, tiles, gw);
-                    const size_t row = (size_t)split * 4u + part;
+                float* dst = grad_view + (size_t)mine.point() * C;
+                float* dst_opacity = grad_opacities + mine.point();
+                if (mine.multi()) {
+                    const size_t row = (size_t)mine.extra + tile_rank(mine, tile % gw, tile / gw, tile_shift);
                     dst = rows.features + row * C;
                     dst_opacity = rows.opacities + row;
-                    ((uint8_t*)(rows.flags + split))[part] = 1;
+                    rows.flags[row] = 1;
                 }
 #pragma unroll
                 for (int q4 = 0; q4 < C / 4; ++q4)
@@ -937,10 +878,6 @@ __global__ void __launch_bounds__(T* T, (T == 16 && C <= 8) ? INPC_BWD_WAVES : 1
         }
         if (all_done) break;
     }
-#ifdef INPC_PROFILE_BACKWARD
-    INPC_PROF_FLUSH;
-#endif
-#undef BWD_MARK
 }
 
 }  // namespace blend

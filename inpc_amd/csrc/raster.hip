@@ -1,31 +1,21 @@
 // raster.hip — tile-based differentiable bilinear point rasterizer for gfx950.
 //
 // Pipeline (all on the caller's stream, counts stay on the device):
-//   k_bin_count      project every point and count the drawn ones per first touched tile
-//   k_bin_offsets    per tile: exclusive prefix of the counts over the chunks of points
-//   k_bin_scan       exclusive scan of the counts: start of every tile's record bin
-//   k_bin_coarse     tile of every 256th record slot (a slot's tile is then found with a short search)
-//   k_preprocess     project, cull, tile bounds, depth key, depth-digit histograms; the blend record of a
-//                    drawn point (screen position, opacity, point id, view features) is written into the
-//                    bin of its first tile (B/rasterization/src/bilinear/kernels.cu:11-84,106-184)
-//   radix sort       stable sort of the drawn points by depth key; the first pass drops the culled
-//                    points, ties keep ascending point id (forward.cu:91-98)
-//   instances.hpp    depth-ordered points -> every tile's instances in depth order and its [begin, end):
-//                    per-chunk instance counts per tile, prefix sums, then a block per chunk sorts a few
-//                    thousand instances by tile inside LDS and appends the runs at the tiles' cursors
-//                    (kernels.cu:186-239, forward.cu:101-143)
-//   k_tile_order     schedule of the blend blocks: tiles with the longest instance lists first
+//   k_bin_count      project every point; per chunk of points count the instances (point, touched tile) per tile
+//   k_bin_offsets    per tile: exclusive prefix of the counts over the chunks
+//   k_bin_scan       exclusive scan over the tiles: [begin, end) of every tile's instances
+//                    (B/rasterization/src/bilinear/kernels.cu:222-239); decides whether they fit the buffers
+//   k_tile_order     schedule of the per-tile blocks: tiles with the longest instance lists first
+//   k_preprocess     project, cull, tile bounds, depth key; the blend record of a drawn point (footprint weights,
+//                    opacity, view features) goes to the point's place in the record array, a (depth key, point)
+//                    pair per instance into the bin of its tile (kernels.cu:11-84,106-184,198-220)
+//   tilesort.hpp     one block per tile sorts its bin by (depth key, point index) inside LDS: the order the
+//                    reference gets from its two device-wide sorts (forward.cu:91-141)
 //   blend.hpp        k_blend_forward: front-to-back bilinear 2x2 splat blend, one block per tile
 //                    (kernels.cu:241-313,422-495); k_blend_backward: replay of the blend with the saved
 //                    final image (kernels.cu:315-420)
 //   k_sh_backward    view-space feature gradient -> 36 fp16 SH coefficient gradients
 //                    (kernels.cu:86-104, sh_utils.cuh:44-62)
-//
-// Why the records are binned: the points arrive in no spatial order, and on this memory system a random
-// gather costs a whole 128-byte line whatever it uses of it, while a random aligned 64-byte store costs
-// 64 bytes. So the one pass that already reads every point scatters a 64-byte record per point into the
-// bin of its tile; the blend of a tile then gathers from a few contiguous kilobytes instead of from the
-// whole point cloud, and every fetched line is used completely.
 #include <algorithm>
 #include <atomic>
 #include <chrono>
@@ -53,20 +43,29 @@ enum Counter : int {
     kCntInstances = 1,
     kCntError = 2,
     kCntSplit = 3,         // drawn points that touch more than one tile
+    kCntOverflow = 5,      // the instances (or the gradient rows) do not fit the buffers: nothing is drawn
+    kCntRows = 10,         // instances of the points that touch more than one tile
     kCntWords = 16
 };
 
-// tile info word: first tile id, spans, valid
+// tile info word of a projected point: first tile id, spans, valid
 constexpr uint32_t kInfoValid = 1u << 18;
 __device__ __forceinline__ uint32_t info_tile0(uint32_t info) { return info & 0xFFFFu; }
 __device__ __forceinline__ uint32_t info_nx(uint32_t info) { return ((info >> 16) & 1u) + 1u; }
 __device__ __forceinline__ uint32_t info_ny(uint32_t info) { return ((info >> 17) & 1u) + 1u; }
 
-// Blend record of a drawn point: a 32-byte header followed by the view features, padded to a multiple
-// of 32 bytes (64 bytes for every configuration but 16 fp32 channels).
-//   header: float sx, sy, opacity; u32 point id; u32 tile info; float depth; u32 index among the points that
-//           touch several tiles (0 for the others); 1 word unused
+// Blend record of a drawn point, at the point's index in the record array: a 32-byte header followed by the view
+// features, padded to a multiple of 32 bytes (64 bytes for every configuration but 16 fp32 channels).
+//   header: float wx0, wx1, wy0, wy1   interpolation weights of the two candidate pixel columns Lx, Lx + 1 and rows
+//                                      Ly, Ly + 1 (L = floor(s - 0.5)); 0 where the pixel centre is 1 or more away
+//                                      (kernels.cu:284-287)
+//           float opacity
+//           u32   point index | kRecordMulti when the point touches several tiles | span bits
+//           u32   (Lx + 1) | (Ly + 1) << 16
+//           u32   training: first gradient row of a point that touches several tiles; inference: depth
 constexpr uint32_t kRecordHeader = 32;
+constexpr uint32_t kRecordIdMask = (1u << 28) - 1u;
+constexpr uint32_t kRecordMulti = 1u << 28, kRecordSpanX = 1u << 29;   // bit 30: two tiles in y
 inline uint32_t record_stride(int channels, bool half_features) {
     return (uint32_t)align_up(kRecordHeader + (size_t)channels * (half_features ? 2 : 4), 32);
 }
@@ -76,8 +75,11 @@ struct Geometry {
     int W, H;
     uint32_t gw, gh, n_tiles;
     Camera cam;
-    uint32_t key_bias;  // depth key = float bits - key_bias
-    uint32_t stride;    // record stride in bytes
+    uint32_t key_bias;      // depth key = float bits - key_bias
+    uint32_t stride;        // record stride in bytes
+    uint32_t capacity;      // instances the buffers hold
+    uint32_t row_capacity;  // gradient rows (instances of points that touch several tiles)
+    uint32_t tile_shift;    // log2 of the tile size
 };
 
 // ---- SH degree 2 (sh_utils.cuh:6-23) ---------------------------------------------------------------------
@@ -175,35 +177,63 @@ __device__ __forceinline__ Projected project_point(const ViewRows& m, const Geom
     return o;
 }
 
-// ---- record bins ------------------------------------------------------------------------------------------------
+// The two pixels of one axis that can lie closer than 1 to screen coordinate s: L = floor(s - 0.5) and L + 1.
+// Their interpolation weights as the reference's blend computes them per pixel (kernels.cu:284-287):
+// d = |s - (pixel + 0.5)|, skipped when d >= 1 (weight 0 here), else saturate(1 - d).
+struct AxisWeights {
+    int left;         // L, clamped to [-1, 65534]
+    float w0, w1;
+};
+
+__device__ __forceinline__ AxisWeights axis_weights(float s) {
+    AxisWeights a;
+    a.left = (int)fminf(fmaxf(floorf(s - 0.5f), -1.0f), 65534.0f);
+    const float d0 = fabsf(s - ((float)a.left + 0.5f));
+    const float d1 = fabsf(s - ((float)(a.left + 1) + 0.5f));
+    a.w0 = !(d0 >= 1.0f) ? __saturatef(1.0f - d0) : 0.0f;
+    a.w1 = !(d1 >= 1.0f) ? __saturatef(1.0f - d1) : 0.0f;
+    return a;
+}
+
+// ---- instance bins ----------------------------------------------------------------------------------------------
 // The points are cut into kBinBlocks contiguous chunks, one per block, the same way in k_bin_count and in
-// k_preprocess. k_bin_count leaves, per (chunk, tile), the number of drawn points of the chunk whose first
-// tile it is; k_bin_offsets turns that table into the exclusive prefix over the chunks of every tile and
-// k_bin_scan into the start of every tile's bin. k_preprocess then hands out slots from LDS cursors
-// seeded with bin_start[tile] + prefix[chunk][tile]: no global atomic anywhere (they run at about
-// 10 G/s on this machine, far below what 8M points need).
-#ifndef INPC_BIN_BLOCKS
-#define INPC_BIN_BLOCKS 512
-#endif
-constexpr int kBinBlocks = INPC_BIN_BLOCKS;
+// k_preprocess. k_bin_count leaves, per (chunk, tile), the number of instances the chunk's points have in the
+// tile; k_bin_offsets turns that table into the exclusive prefix over the chunks of every tile and k_bin_scan
+// into the start of every tile's bin. k_preprocess then hands out bin slots from LDS cursors seeded with
+// bin_start[tile] + prefix[chunk][tile]: no global atomic anywhere (they run at about 10 G/s on this machine,
+// far below what 8M points need).
+constexpr int kBinBlocks = 512;
 constexpr int kBinThreads = 512;
-constexpr uint32_t kMaxLdsTiles = 16384;  // tile counters a block keeps in LDS (64 KiB)
+constexpr uint32_t kMaxLdsTiles = 16384;  // tiles whose counters a block keeps as 32-bit words in LDS (64 KiB)
 
 __host__ __device__ inline uint32_t bin_chunk_size(uint32_t n) {
     const uint32_t per = (n + kBinBlocks - 1) / kBinBlocks;
     return (per + kBinThreads - 1) / kBinThreads * kBinThreads;
 }
 
+// For every touched tile of a projected point, in the row-major order of the reference's create_instances_cu
+// (kernels.cu:208-217).
+template <typename F>
+__device__ __forceinline__ void for_each_tile(uint32_t info, uint32_t gw, F f) {
+    const uint32_t tile0 = info_tile0(info);
+    f(tile0);
+    if (info & (1u << 16)) f(tile0 + 1u);
+    if (info & (1u << 17)) {
+        f(tile0 + gw);
+        if (info & (1u << 16)) f(tile0 + gw + 1u);
+    }
+}
+
 template <int T>
 __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restrict__ positions,
                                                            const float* __restrict__ w2c, uint32_t* __restrict__ table,
-                                                           uint32_t* __restrict__ split_count, Geometry g) {
+                                                           uint2* __restrict__ split_count, Geometry g) {
     extern __shared__ uint32_t s_count[];
-    __shared__ uint32_t s_split;   // drawn points of the chunk that touch more than one tile
+    __shared__ uint32_t s_split, s_rows;   // the chunk's points that touch several tiles, and their instances
     for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_count[t] = 0u;
-    if (threadIdx.x == 0) s_split = 0u;
+    if (threadIdx.x == 0) s_split = s_rows = 0u;
     __syncthreads();
-    uint32_t my_split = 0;
+    uint32_t my_split = 0, my_rows = 0;
     const ViewRows m = load_view_rows(w2c);
     const uint32_t chunk = bin_chunk_size(g.n);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
@@ -222,16 +252,25 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
         for (int u = 0; u < kUnroll; ++u) {
             if (base + u * kBinThreads + threadIdx.x >= end) continue;
             const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
-            if (p.info) atomicAdd(&s_count[info_tile0(p.info)], 1u);
-            if (p.touched > 1u) my_split += 1u;
+            if (p.info) for_each_tile(p.info, g.gw, [&](uint32_t tile) { atomicAdd(&s_count[tile], 1u); });
+            if (p.touched > 1u) {
+                my_split += 1u;
+                my_rows += p.touched;
+            }
         }
     }
-    for (int sh = 32; sh > 0; sh >>= 1) my_split += __shfl_down(my_split, sh, 64);
-    if ((threadIdx.x & 63u) == 0u && my_split) atomicAdd(&s_split, my_split);
+    for (int sh = 32; sh > 0; sh >>= 1) {
+        my_split += __shfl_down(my_split, sh, 64);
+        my_rows += __shfl_down(my_rows, sh, 64);
+    }
+    if ((threadIdx.x & 63u) == 0u && my_split) {
+        atomicAdd(&s_split, my_split);
+        atomicAdd(&s_rows, my_rows);
+    }
     __syncthreads();
     uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
     for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) row[t] = s_count[t];
-    if (threadIdx.x == 0) split_count[blockIdx.x] = s_split;
+    if (threadIdx.x == 0) split_count[blockIdx.x] = make_uint2(s_split, s_rows);
 }
 
 // table[c][t] <- sum of table[c'][t] over c' < c; total[t] <- sum over all chunks.
@@ -273,31 +312,65 @@ __global__ void __launch_bounds__(kOffsetWaves * kWave) k_bin_offsets(uint32_t* 
     }
 }
 
-// bin_start[t] = number of records in bins before t (n_tiles + 1 entries).
+// One block. bin_start[t] = number of instances in the bins before t (n_tiles + 1 entries) and the tiles'
+// [begin, end) ranges, (0, 0) for a tile without instances as the reference's cleared buffer leaves it
+// (forward.cu:52). split_base[c] = {points that touch several tiles, their instances} in the chunks before c.
+// When the instances or the gradient rows exceed the buffers, every bin is left empty and the overflow counter set:
+// the later kernels then draw nothing.
 constexpr int kScanBlock = 1024;
-__global__ void __launch_bounds__(kScanBlock) k_bin_scan(const uint32_t* __restrict__ bin_count,
-                                                         uint32_t* __restrict__ bin_start, uint32_t n_tiles) {
-    __shared__ uint32_t s_wave[kScanBlock / kWave];
+static_assert(kBinBlocks <= kScanBlock, "one thread per chunk in k_bin_scan");
+__global__ void __launch_bounds__(kScanBlock)
+    k_bin_scan(const uint32_t* __restrict__ bin_count, uint32_t* __restrict__ bin_start, uint2* __restrict__ ranges,
+               const uint2* __restrict__ split_count, uint2* __restrict__ split_base, uint32_t* __restrict__ counters,
+               uint32_t n_tiles, uint32_t capacity, uint32_t row_capacity) {
+    __shared__ uint32_t s_wave[3][kScanBlock / kWave];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t per = (n_tiles + kScanBlock - 1) / kScanBlock;
     const uint32_t begin = min(tid * per, n_tiles), end = min(begin + per, n_tiles);
-    uint32_t mine = 0;
-    for (uint32_t t = begin; t < end; ++t) mine += bin_count[t];
-    uint32_t incl = mine;
+    uint32_t mine[3] = {0u, 0u, 0u};
+    for (uint32_t t = begin; t < end; ++t) mine[0] += bin_count[t];
+    if (tid < (uint32_t)kBinBlocks) {
+        const uint2 c = split_count[tid];
+        mine[1] = c.x;
+        mine[2] = c.y;
+    }
+    uint32_t incl[3] = {mine[0], mine[1], mine[2]};
 #pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s, 64);
-        if (lane >= (uint32_t)s) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
+    for (int s = 1; s < 64; s <<= 1)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const uint32_t up = __shfl_up(incl[k], s, 64);
+            if (lane >= (uint32_t)s) incl[k] += up;
+        }
+    if (lane == 63)
+        for (int k = 0; k < 3; ++k) s_wave[k][wave] = incl[k];
     __syncthreads();
-    uint32_t run = incl - mine;
-    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
-    for (uint32_t t = begin; t < end; ++t) {
-        bin_start[t] = run;
-        run += bin_count[t];
+    uint32_t run[3], total[3] = {0u, 0u, 0u};
+    for (int k = 0; k < 3; ++k) {
+        run[k] = incl[k] - mine[k];
+        for (uint32_t w = 0; w < (uint32_t)(kScanBlock / kWave); ++w) {
+            const uint32_t s = s_wave[k][w];
+            if (w < wave) run[k] += s;
+            total[k] += s;
+        }
     }
-    if (end == n_tiles && begin < n_tiles) bin_start[n_tiles] = run;
+    const bool overflow = total[0] > capacity || total[2] > row_capacity;
+    for (uint32_t t = begin; t < end; ++t) {
+        const uint32_t c = overflow ? 0u : bin_count[t];
+        bin_start[t] = overflow ? 0u : run[0];
+        ranges[t] = c ? make_uint2(run[0], run[0] + c) : make_uint2(0u, 0u);
+        run[0] += c;
+    }
+    if (tid < (uint32_t)kBinBlocks) split_base[tid] = make_uint2(run[1], run[2]);
+    if (tid == 0) {
+        bin_start[n_tiles] = overflow ? 0u : total[0];
+        counters[kCntVisible] = 0u;   // counted by k_preprocess
+        counters[kCntError] = 0u;
+        counters[kCntInstances] = total[0];
+        counters[kCntSplit] = total[1];
+        counters[kCntRows] = total[2];
+        counters[kCntOverflow] = overflow ? 1u : 0u;
+    }
 }
 
 // ---- preprocess -------------------------------------------------------------------------------------------
@@ -311,52 +384,46 @@ struct PreprocessShape {
     static constexpr size_t kStageBytes = (size_t)kBinThreads * (kStrideWords + 1) * 16;   // padded rows, per block
 };
 
+// What a training configuration keeps of the points that touch several tiles: a list entry
+// {point | touched tiles << 28, first gradient row} per such point, and a flag byte per gradient row.
+struct SplitOut {
+    const uint2* base;      // per chunk: {such points, their instances} in the chunks before
+    uint2* list;
+    uint8_t* row_flags;
+};
+
 template <int T, int FMODE, int C>
 __global__ void __launch_bounds__(kBinThreads)
     k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
                  const float* __restrict__ opacities, const float* __restrict__ w2c,
                  const float* __restrict__ cam_position, char* __restrict__ records,
                  const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start,
-                 uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, float* __restrict__ blending_weights,
-                 const uint32_t* __restrict__ split_count, uint32_t* __restrict__ split_points,
-                 uint32_t* __restrict__ split_flags, uint32_t* counters, uint32_t* g_hist, Geometry g,
-                 radix::DevicePlan plan) {
+                 uint64_t* __restrict__ pairs, float* __restrict__ blending_weights, SplitOut split,
+                 float4* __restrict__ debug_geometry, uint32_t* counters, Geometry g) {
     extern __shared__ __align__(16) uint32_t s_dyn[];
     float4* s_stage = (float4*)s_dyn;                                           // record staging, 64 rows per wave
     uint32_t* s_cursor = s_dyn + PreprocessShape<FMODE, C>::kStageBytes / 4;     // n_tiles
-    uint32_t* s_hist = s_cursor + g.n_tiles;                                    // kMaxPasses * kRadix
-    __shared__ uint32_t s_visible, s_instances;
-    __shared__ uint32_t s_split;   // next index for a point of this chunk that touches more than one tile
+    __shared__ uint32_t s_visible;
+    __shared__ uint32_t s_split, s_rows;   // next list entry / gradient row for a point of this chunk
+    const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then no instance is stored
     {
         const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
         for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_cursor[t] = bin_start[t] + row[t];
     }
-    for (int i = threadIdx.x; i < plan.n_passes * radix::kRadix; i += kBinThreads) s_hist[i] = 0u;
     if (threadIdx.x == 0) {
         s_visible = 0u;
-        s_instances = 0u;
-        s_split = 0u;
+        const uint2 first = split.base ? split.base[blockIdx.x] : make_uint2(0u, 0u);
+        s_split = first.x;
+        s_rows = first.y;
     }
     __syncthreads();
-    {
-        // the points that touch several tiles are numbered chunk by chunk (inside a chunk in no particular
-        // order): the index only names the rows their gradient is collected in
-        uint32_t before = 0;
-        for (uint32_t b = threadIdx.x; b < blockIdx.x; b += kBinThreads) before += split_count[b];
-        for (int sh = 32; sh > 0; sh >>= 1) before += __shfl_down(before, sh, 64);
-        if ((threadIdx.x & 63u) == 0u && before) atomicAdd(&s_split, before);
-        __syncthreads();
-        const uint32_t first = s_split;
-        __syncthreads();
-        if (threadIdx.x == 0 && blockIdx.x == gridDim.x - 1u) counters[kCntSplit] = first + split_count[blockIdx.x];
-    }
     const ViewRows m = load_view_rows(w2c);
-    uint32_t my_visible = 0, my_instances = 0;
+    uint32_t my_visible = 0;
     const uint32_t chunk = bin_chunk_size(g.n);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
     // kUnroll points per thread and round, their loads issued together. A record leaves the block through LDS:
     // every lane assembles its record in the wave's staging rows, then neighbouring lanes write the 16-byte
-    // words of one record, so that a store instruction covers whole records (contiguous 64 bytes and more)
+    // words of one record, so that a store instruction covers a contiguous stretch of the record array
     // instead of one word of 64 different records.
     constexpr bool kDirect = FMODE == INPC_FEAT_DIRECT_F32 || FMODE == INPC_FEAT_DIRECT_F16;
     constexpr int kUnroll = kDirect ? 4 : 2;
@@ -364,7 +431,6 @@ __global__ void __launch_bounds__(kBinThreads)
     constexpr int kWords = kDirect ? C / 4 : 1;
     constexpr int kPer = sizeof(Word) / 4;   // 32-bit registers per word
     constexpr uint32_t kStrideWords = PreprocessShape<FMODE, C>::kStrideWords, kRow = kStrideWords + 1;  // padded row
-    constexpr uint32_t kNoSlot = 0xFFFFFFFFu;
     const uint32_t lane = threadIdx.x & 63u;
     float4* stage = s_stage + (threadIdx.x >> 6) * (64u * kRow);
     for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
@@ -396,17 +462,14 @@ __global__ void __launch_bounds__(kBinThreads)
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const uint32_t i = base + u * kBinThreads + threadIdx.x;
-            uint32_t slot = kNoSlot;
+            bool drawn = false;
             if (i < end) {
                 const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
-                uint32_t key = radix::kInvalidKey, val = 0u;
-                if (p.info) {
-                    key = __float_as_uint(p.depth) - g.key_bias;
+                drawn = p.info != 0u;
+                if (drawn) {
                     my_visible += 1u;
-                    my_instances += p.touched;
-                    radix::hist_add(s_hist, plan, key);
-                    slot = atomicAdd(&s_cursor[info_tile0(p.info)], 1u);
-                    val = (slot << 2) | ((p.info >> 16) & 3u);
+                    const uint64_t pair = ((uint64_t)(__float_as_uint(p.depth) - g.key_bias) << 32) | (uint64_t)i;
+                    if (!overflow) for_each_tile(p.info, g.gw, [&](uint32_t tile) { pairs[atomicAdd(&s_cursor[tile], 1u)] = pair; });
                     float4* rec = stage + lane * kRow;
                     float opacity = op[u];
 #pragma unroll
@@ -434,76 +497,45 @@ __global__ void __launch_bounds__(kBinThreads)
                             opacity = 1.0f - expf(-expf(__half2float(raw[0])));  // kernels.cu:142
                         }
                     }
-                    uint32_t split = 0u;
-                    if (p.touched > 1u) {
-                        split = atomicAdd(&s_split, 1u);
-                        split_points[split] = i;
-                        split_flags[split] = 0u;
+                    uint32_t tag = i | (((p.info >> 16) & 3u) << 29);
+                    uint32_t extra = __float_as_uint(p.depth);
+                    if (split.list) {   // training configurations
+                        extra = 0u;
+                        if (p.touched > 1u && !overflow) {
+                            tag |= kRecordMulti;
+                            extra = atomicAdd(&s_rows, p.touched);
+                            split.list[atomicAdd(&s_split, 1u)] = make_uint2(i | (p.touched << 28), extra);
+                            for (uint32_t r = 0; r < p.touched; ++r) split.row_flags[extra + r] = 0;
+                        }
                     }
-                    rec[0] = make_float4(p.sx, p.sy, opacity, __uint_as_float(i));
-                    rec[1] = make_float4(__uint_as_float(p.info), p.depth, __uint_as_float(split), 0.0f);
+                    const AxisWeights ax = axis_weights(p.sx), ay = axis_weights(p.sy);
+                    rec[0] = make_float4(ax.w0, ax.w1, ay.w0, ay.w1);
+                    rec[1] = make_float4(opacity, __uint_as_float(tag),
+                                         __uint_as_float((uint32_t)(ax.left + 1) | ((uint32_t)(ay.left + 1) << 16)),
+                                         __uint_as_float(extra));
                 }
-                keys[i] = key;
-                vals[i] = val;
                 if (blending_weights) blending_weights[i] = 0.0f;
+                if (debug_geometry) debug_geometry[i] = make_float4(p.sx, p.sy, p.depth, __uint_as_float(p.info));
             }
             wave_sync();
+            // the wave's 64 points are consecutive: their records are one contiguous stretch
+            const uint32_t wave_first = base + u * kBinThreads + (threadIdx.x & ~63u);
+            const uint64_t drawn_lanes = __ballot(drawn);
+            float4* out = (float4*)(records + (size_t)wave_first * g.stride);
 #pragma unroll
             for (uint32_t k = 0; k < kStrideWords; ++k) {
                 const uint32_t flat = k * 64u + lane, r = flat / kStrideWords, w = flat % kStrideWords;
-                const uint32_t to = __shfl(slot, r, 64);
-                if (to != kNoSlot) ((float4*)(records + (size_t)to * g.stride))[w] = stage[r * kRow + w];
+                if ((drawn_lanes >> r) & 1ull) out[flat] = stage[r * kRow + w];
             }
             wave_sync();
         }
     }
-    // block totals -> one global atomic each
-    for (int s = 32; s > 0; s >>= 1) {
-        my_visible += __shfl_down(my_visible, s, 64);
-        my_instances += __shfl_down(my_instances, s, 64);
-    }
-    if ((threadIdx.x & 63u) == 0u) {
-        atomicAdd(&s_visible, my_visible);
-        atomicAdd(&s_instances, my_instances);
-    }
+    // block total -> one global atomic
+    for (int s = 32; s > 0; s >>= 1) my_visible += __shfl_down(my_visible, s, 64);
+    if ((threadIdx.x & 63u) == 0u) atomicAdd(&s_visible, my_visible);
     __syncthreads();
-    if (threadIdx.x == 0) {
-        if (s_visible) atomicAdd(&counters[kCntVisible], s_visible);
-        if (s_instances) atomicAdd(&counters[kCntInstances], s_instances);
-    }
-    radix::hist_flush(s_hist, plan, g_hist);
+    if (threadIdx.x == 0 && s_visible) atomicAdd(&counters[kCntVisible], s_visible);
 }
-
-// ---- record slot -> tile ------------------------------------------------------------------------------------------
-constexpr int kCoarseShift = 8;     // one coarse entry per 256 record slots
-
-inline uint32_t coarse_entries(uint32_t n) { return (n >> kCoarseShift) + 2u; }
-
-// Tile whose record bin holds `slot`: the last t in [lo, hi) with bin_start[t] <= slot.
-// Requires bin_start[lo] <= slot < bin_start[hi].
-__device__ __forceinline__ uint32_t tile_of_slot(const uint32_t* __restrict__ bin_start, uint32_t lo, uint32_t hi,
-                                                 uint32_t slot) {
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (bin_start[mid] <= slot) lo = mid;
-        else hi = mid;
-    }
-    return lo;
-}
-
-// coarse[b] = tile of record slot b << kCoarseShift (the last tile for slots behind the last record), so
-// that the tile of any slot is found between two neighbouring entries.
-__global__ void __launch_bounds__(kBlock) k_bin_coarse(const uint32_t* __restrict__ bin_start, uint16_t* __restrict__ coarse,
-                                                       uint32_t n_tiles, uint32_t n_entries) {
-    const uint32_t b = blockIdx.x * kBlock + threadIdx.x;
-    if (b >= n_entries) return;
-    const uint64_t slot = (uint64_t)b << kCoarseShift;
-    uint32_t t = n_tiles - 1u;
-    if (slot < bin_start[n_tiles]) t = tile_of_slot(bin_start, 0u, n_tiles, (uint32_t)slot);
-    coarse[b] = (uint16_t)t;
-}
-
-#include "instances.hpp"
 
 // ---- tile schedule -----------------------------------------------------------------------------------------------
 // Blocks of the blend kernels take their tiles from this list: longest instance list first, so that the
@@ -577,59 +609,8 @@ __device__ __forceinline__ void load_record_features(float* dst, const char* __r
     }
 }
 
-// Tile-local index of the last pixel whose centre is not right of (not below) coordinate s, clamped so
-// that the conversion is safe for any float. Only this pixel and the next one can be closer than 1 to s.
-template <int T>
-__device__ __forceinline__ int left_pixel(float s, int tile_origin) {
-    return (int)fminf(fmaxf(floorf(s - 0.5f) - (float)tile_origin, -4.0f), (float)(T + 4));
-}
-
-// The two candidate pixels of one axis: which of them lie in the tile and pass the float test of
-// B/rasterization/src/bilinear/kernels.cu:284-285, and their interpolation weights (kernels.cu:286-287).
-struct AxisCover {
-    int first;      // tile-local index of candidate 0
-    bool hit[2];
-    float weight[2];
-};
-
-template <int T>
-__device__ __forceinline__ AxisCover cover_axis(float s, int tile_origin) {
-    AxisCover a;
-    a.first = left_pixel<T>(s, tile_origin);
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        const int c = a.first + k;
-        const float d = fabsf(s - ((float)(tile_origin + c) + 0.5f));
-        a.hit[k] = c >= 0 && c < T && !(d >= 1.0f);
-        a.weight[k] = __saturatef(1.0f - d);
-    }
-    return a;
-}
-
-#ifdef INPC_BLEND_PROFILE
-// development aid: per-phase shader clocks of k_blend_forward, summed over blocks (thread 0 of each)
-__device__ unsigned long long g_blend_profile[8];
-#define INPC_PROF_DECL unsigned long long prof_t = clock64(), prof_acc[6] = {0, 0, 0, 0, 0, 0}, prof_batches = 0
-#define INPC_PROF_MARK(i)                          \
-    do {                                           \
-        const unsigned long long now_ = clock64(); \
-        prof_acc[i] += now_ - prof_t;              \
-        prof_t = now_;                             \
-    } while (0)
-#define INPC_PROF_FLUSH                                                         \
-    do {                                                                        \
-        if (threadIdx.x == 0) {                                                 \
-            for (int i_ = 0; i_ < 6; ++i_) atomicAdd(&g_blend_profile[i_], prof_acc[i_]); \
-            atomicAdd(&g_blend_profile[6], prof_batches);                       \
-        }                                                                       \
-    } while (0)
-#else
-#define INPC_PROF_DECL
-#define INPC_PROF_MARK(i)
-#define INPC_PROF_FLUSH
-#endif
-
 #include "blend.hpp"
+#include "tilesort.hpp"
 #include "gaussian.hpp"
 
 // view-space feature gradient -> (N,36) fp16; a point that was not drawn has a zero view gradient and
@@ -679,24 +660,24 @@ __global__ void __launch_bounds__(kBlock) k_float_to_half(const float* __restric
 struct Layout {
     inpc_raster_layout pub;
     Geometry geo;
-    radix::PassPlan depth_plan;
-    int T, C, fmode;
+    int T, C, fmode, key_bits;
     bool inference, sh, half_features;
     // private offsets
-    size_t zero_begin, zero_words;  // region cleared at the start of every forward
-    size_t hist_depth, bases_depth;
-    size_t status_depth, bin_coarse;
-    size_t bin_table, bin_total, tile_order, inst_start;
-    size_t keys_a, keys_b, vals_a, vals_b;
-    size_t inst_keys_a, inst_vals_a;
-    size_t split_count, split_points, split_features, split_opacities, split_flags;  // points that straddle tiles
-    size_t ordered_records, tile_end;   // 0: the configuration has no backward pass
+    size_t bin_table, bin_total, tile_order, split_count, split_base;
+    size_t pairs, pairs_scratch;
+    size_t split_list, row_flags, row_features, row_opacities;   // points that straddle tiles (0: no backward pass)
+    size_t ordered_records, tile_end;                            // 0: the configuration has no backward pass
 };
 
 uint32_t float_bits(float f) {
     uint32_t u;
     memcpy(&u, &f, 4);
     return u;
+}
+
+template <typename Tp>
+Tp* at(void* ws, size_t off) {
+    return (Tp*)((char*)ws + off);
 }
 
 int make_layout(const inpc_raster_config* cfg, Layout& L) {
@@ -713,6 +694,8 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     L.C = L.sh ? 4 : cfg->channels;
     if (L.C != 4 && L.C != 8 && L.C != 16) return fail(INPC_E_INVALID_ARGUMENT, "raster: channels must be 4, 8 or 16");
     L.inference = (cfg->flags & INPC_RASTER_INFERENCE) != 0;
+    const bool training = !L.inference && L.fmode != INPC_FEAT_RAW37_F16;   // configurations with a backward pass
+    const bool debug = (cfg->flags & INPC_RASTER_KEEP_GEOMETRY) != 0;
     Geometry& g = L.geo;
     g.n = cfg->n_points;
     g.W = cam.width;
@@ -720,6 +703,9 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     g.gw = (uint32_t)((cam.width + L.T - 1) / L.T);
     g.gh = (uint32_t)((cam.height + L.T - 1) / L.T);
     g.n_tiles = g.gw * g.gh;
+    g.tile_shift = L.T == 16 ? 4u : 3u;
+    if (cam.width > 65000 || cam.height > 65000)
+        return fail(INPC_E_UNSUPPORTED, "raster: images beyond 65000 pixels per side are not supported");
     if (g.n_tiles > 65536u)
         return fail(INPC_E_UNSUPPORTED, "raster: %u tiles exceed the 16-bit tile key (65536)", g.n_tiles);
     if (g.n_tiles > kMaxLdsTiles)
@@ -728,16 +714,32 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     g.cam = to_device_camera(cam);
     g.stride = record_stride(L.C, L.half_features);
     // depth keys of drawn points lie in [bits(near), bits(far)] when 0 < near <= far: sort on the offset
-    int depth_bits = 32;
+    L.key_bits = 32;
     g.key_bias = 0u;
     if (cam.near_plane > 0.0f && cam.far_plane >= cam.near_plane && cam.far_plane < INFINITY) {
         g.key_bias = float_bits(cam.near_plane);
-        depth_bits = std::max(1, bit_length(float_bits(cam.far_plane) - g.key_bias));
+        L.key_bits = std::max(1, bit_length(float_bits(cam.far_plane) - g.key_bias));
     }
-    L.depth_plan = radix::make_plan(depth_bits);
     const int end_bit = bit_length(g.n_tiles - 1);
 
-    const size_t n = std::max<size_t>(g.n, 1), ni = 4 * n;
+    // A point has at most four instances; evenly spread points have (1 + 1 / tile)^2 on average, which the default
+    // capacity covers with a margin. k_bin_scan decides on the device whether a call fits.
+    const size_t n = std::max<size_t>(g.n, 1);
+    const uint64_t most = 4ull * g.n;
+    uint64_t capacity = cfg->max_instances;
+    if (capacity == 0) {
+        const double per_point = (1.0 + 1.0 / L.T) * (1.0 + 1.0 / L.T);
+        capacity = (uint64_t)std::ceil((double)g.n * per_point * 1.0625) + 65536ull;
+    }
+    capacity = std::max<uint64_t>(std::min(capacity, most), 1);
+    g.capacity = (uint32_t)capacity;
+    // gradient rows: the instances of the points that touch several tiles, at most twice the instances beyond one per point
+    g.row_capacity = 0xFFFFFFFFu;
+    if (training) {
+        const uint64_t beyond = capacity > g.n ? capacity - g.n : 0;
+        g.row_capacity = (uint32_t)std::min<uint64_t>(capacity, 2 * beyond + (capacity < most ? 262144ull : 0ull));
+    }
+
     size_t off = 0;
     auto take = [&](size_t bytes) {
         const size_t o = off;
@@ -746,46 +748,34 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     };
     inpc_raster_layout& P = L.pub;
     memset(&P, 0, sizeof(P));
-    // zeroed region: counters, histograms, look-back status, bin counts, tile ranges
-    L.zero_begin = off;
     P.counters = take(kCntWords * 4);
-    L.hist_depth = take(radix::kMaxPasses * radix::kRadix * 4);
-    L.status_depth = take(L.depth_plan.n_passes * radix::status_words(g.n) * 4);
     P.tile_ranges = take((size_t)g.n_tiles * 8);
-    L.zero_words = (off - L.zero_begin) / 4;
-    L.bin_table = take((size_t)std::max<int>(kBinBlocks, instances::kChunks) * g.n_tiles * 4);
+    L.bin_table = take((size_t)kBinBlocks * g.n_tiles * 4);
     L.bin_total = take((size_t)g.n_tiles * 4);
     L.tile_order = take((size_t)g.n_tiles * 4);
-    L.inst_start = take((size_t)(g.n_tiles + 1) * 4);
     P.bin_start = take((size_t)(g.n_tiles + 1) * 4);
-    L.bin_coarse = take((size_t)coarse_entries(g.n) * 2);
-    L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
+    L.split_count = take(kBinBlocks * 8);
+    L.split_base = take(kBinBlocks * 8);
     P.point_record = take(n * g.stride);
-    L.keys_a = take(n * 4);
-    L.keys_b = take(n * 4);
-    L.vals_a = take(n * 4);
-    L.vals_b = take(n * 4);
-    L.inst_keys_a = take(ni * 2);
-    L.inst_vals_a = take(ni * 4);
-    // gradient rows of the points that touch several tiles, four per point; sized for the worst case
-    // (every point), touched only as far as such points exist
-    L.split_count = take(kBinBlocks * 4);
-    L.split_points = take(n * 4);
-    L.split_flags = take(n * 4);
-    L.split_features = L.split_opacities = L.ordered_records = L.tile_end = 0;
-    if (!L.inference && L.fmode != INPC_FEAT_RAW37_F16) {   // configurations with a backward pass
-        L.split_features = take(4 * n * L.C * 4);
-        L.split_opacities = take(4 * n * 4);
+    L.pairs = take(capacity * 8);
+    P.instance_points = take(capacity * 4);
+    L.split_list = L.row_flags = L.row_features = L.row_opacities = L.ordered_records = L.tile_end = 0;
+    if (training) {
+        const size_t rows = std::max<size_t>(g.row_capacity, 1);
+        L.split_list = take((rows / 2 + 1) * 8);
+        L.row_flags = take(rows);
+        L.row_features = take(rows * L.C * 4);
+        L.row_opacities = take(rows * 4);
         // the records once more, per instance and in the order of the tiles' lists, left by the forward blend for
-        // the backward blend; how far each tile's reach
-        L.ordered_records = take(ni * (2 + (size_t)L.C / 4) * 16);
+        // the backward blend; how far each tile's reach. Until the forward blend runs the block is free and the
+        // merges of the tile sort use it.
+        L.ordered_records = take(capacity * (2 + (size_t)L.C / 4) * 16);
         L.tile_end = take((size_t)g.n_tiles * 4);
+        L.pairs_scratch = L.ordered_records;
+    } else {
+        L.pairs_scratch = take(capacity * 8);
     }
-    const bool depth_in_a = (L.depth_plan.n_passes % 2) == 0;
-    P.depth_keys = depth_in_a ? L.keys_a : L.keys_b;
-    P.depth_order = depth_in_a ? L.vals_a : L.vals_b;
-    P.instance_keys = L.inst_keys_a;
-    P.instance_slots = L.inst_vals_a;
+    P.debug_geometry = debug ? take(n * 16) : 0;
     P.total_bytes = off;
     P.record_stride = g.stride;
     P.grid_width = g.gw;
@@ -793,12 +783,8 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     P.n_tiles = g.n_tiles;
     P.end_bit = (uint32_t)end_bit;
     P.depth_key_bias = g.key_bias;
+    P.max_instances = g.capacity;
     return INPC_OK;
-}
-
-template <typename Tp>
-Tp* at(void* ws, size_t off) {
-    return (Tp*)((char*)ws + off);
 }
 
 // Launch with `lds_bytes` of dynamic LDS; above 64 KiB the kernel has to be told once.
@@ -822,7 +808,7 @@ template <int T>
 int launch_bin_count(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
     const size_t lds = (size_t)L.geo.n_tiles * 4;
     INPC_LAUNCH_LDS("raster_bin_count", (k_bin_count<T>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream, positions,
-                    w2c, at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.split_count), L.geo);
+                    w2c, at<uint32_t>(ws, L.bin_table), at<uint2>(ws, L.split_count), L.geo);
     return INPC_OK;
 }
 
@@ -830,16 +816,17 @@ template <int T, int FMODE, int C>
 int launch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
                       const float* w2c, const float* cam_position, float* blending_weights, void* ws,
                       hipStream_t stream) {
-    const size_t lds = PreprocessShape<FMODE, C>::kStageBytes + ((size_t)L.geo.n_tiles + radix::kMaxPasses * radix::kRadix) * 4;
+    const size_t lds = PreprocessShape<FMODE, C>::kStageBytes + (size_t)L.geo.n_tiles * 4;
     if (L.pub.record_stride != PreprocessShape<FMODE, C>::kStrideWords * 16u)
         return fail(INPC_E_UNSUPPORTED, "record stride %u does not match the preprocess kernel", L.pub.record_stride);
+    SplitOut split{nullptr, nullptr, nullptr};
+    if (L.split_list) split = SplitOut{at<uint2>(ws, L.split_base), at<uint2>(ws, L.split_list), at<uint8_t>(ws, L.row_flags)};
     INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream,
                     positions, features, opacities, w2c, cam_position, at<char>(ws, L.pub.point_record),
                     (const uint32_t*)at<uint32_t>(ws, L.bin_table), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
-                    at<uint32_t>(ws, L.keys_a), at<uint32_t>(ws, L.vals_a), blending_weights,
-                    (const uint32_t*)at<uint32_t>(ws, L.split_count), at<uint32_t>(ws, L.split_points),
-                    at<uint32_t>(ws, L.split_flags), at<uint32_t>(ws, L.pub.counters), at<uint32_t>(ws, L.hist_depth), L.geo,
-                    radix::to_device_plan(L.depth_plan));
+                    at<uint64_t>(ws, L.pairs), blending_weights, split,
+                    L.pub.debug_geometry ? at<float4>(ws, L.pub.debug_geometry) : (float4*)nullptr,
+                    at<uint32_t>(ws, L.pub.counters), L.geo);
     return INPC_OK;
 }
 
@@ -848,7 +835,7 @@ int launch_blend_forward(const Layout& L, float* image, float* alpha, float* ble
                          void* ws, hipStream_t stream) {
     const uint2* ranges = at<uint2>(ws, L.pub.tile_ranges);
     const uint32_t* order = at<uint32_t>(ws, L.tile_order);
-    const uint32_t* inst = at<uint32_t>(ws, L.pub.instance_slots);
+    const uint32_t* inst = at<uint32_t>(ws, L.pub.instance_points);
     const char* records = at<char>(ws, L.pub.point_record);
     if (L.inference) {
         INPC_LAUNCH("raster_blend_inference", (blend::k_blend_forward<T, C, HALF, true>), dim3(L.geo.n_tiles), dim3(T * T),
@@ -866,14 +853,14 @@ int launch_blend_forward(const Layout& L, float* image, float* alpha, float* ble
 template <int T, int C, bool HALF>
 int launch_blend_backward(const Layout& L, const float* grad_image, const float* grad_alpha, const float* image,
                           const float* alpha, float* grad_view, float* grad_opacities, void* ws, hipStream_t stream) {
-    const blend::SplitRows rows{at<float>(ws, L.split_features), at<float>(ws, L.split_opacities),
-                                at<uint32_t>(ws, L.split_flags), (const uint32_t*)at<uint32_t>(ws, L.split_points),
+    const blend::SplitRows rows{at<float>(ws, L.row_features), at<float>(ws, L.row_opacities),
+                                at<uint8_t>(ws, L.row_flags), (const uint2*)at<uint2>(ws, L.split_list),
                                 (const uint32_t*)at<uint32_t>(ws, L.pub.counters) + kCntSplit};
     INPC_LAUNCH("raster_blend_backward", (blend::k_blend_backward<T, C, HALF>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 (const float4*)at<float4>(ws, L.ordered_records), (const uint32_t*)at<uint32_t>(ws, L.tile_end), grad_image,
                 grad_alpha, image, alpha, grad_view,
-                grad_opacities, rows, L.geo.W, L.geo.H, L.geo.gw);
+                grad_opacities, rows, L.geo.W, L.geo.H, L.geo.gw, L.geo.tile_shift);
     INPC_LAUNCH("raster_grad_reduce", blend::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, 256u), 4096u)), dim3(256),
                 stream, rows, grad_view, grad_opacities);
     return INPC_OK;
@@ -1212,54 +1199,33 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
     if ((L.fmode == INPC_FEAT_DIRECT_F16 || L.fmode == INPC_FEAT_SH36_F16) && ((uintptr_t)features & 7u) != 0)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_raster_forward: fp16 features must be 8-byte aligned");
 
-    rc = fill_u32(at<uint32_t>(ws, L.zero_begin), 0u, L.zero_words, stream);
-    if (rc != INPC_OK) return rc;
     uint32_t* counters = at<uint32_t>(ws, L.pub.counters);
     if (L.geo.n > 0) {
         rc = L.T == 8 ? launch_bin_count<8>(L, positions, w2c, ws, stream) : launch_bin_count<16>(L, positions, w2c, ws, stream);
         if (rc != INPC_OK) return rc;
         INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<kBinBlocks>, dim3(div_up(L.geo.n_tiles, kWave)), dim3(kOffsetWaves * kWave), stream,
                     at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
-        INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
-                    (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start), L.geo.n_tiles);
-        INPC_LAUNCH("raster_bin_coarse", k_bin_coarse, dim3(div_up(coarse_entries(L.geo.n), kBlock)), dim3(kBlock),
-                    stream, (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start), at<uint16_t>(ws, L.bin_coarse),
-                    L.geo.n_tiles, coarse_entries(L.geo.n));
+    } else {
+        rc = fill_u32(at<uint32_t>(ws, L.bin_total), 0u, L.geo.n_tiles, stream);
+        if (rc != INPC_OK) return rc;
+        rc = fill_u32(at<uint32_t>(ws, L.split_count), 0u, 2 * kBinBlocks, stream);
+        if (rc != INPC_OK) return rc;
+    }
+    INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
+                (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start),
+                at<uint2>(ws, L.pub.tile_ranges), (const uint2*)at<uint2>(ws, L.split_count),
+                at<uint2>(ws, L.split_base), counters, L.geo.n_tiles, L.geo.capacity, L.geo.row_capacity);
+    INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
+                (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
+    if (L.geo.n > 0) {
         rc = dispatch_preprocess(L, positions, features, opacities, w2c, cam_position,
                                  L.inference ? nullptr : blending_weights, ws, stream);
         if (rc != INPC_OK) return rc;
-        rc = radix::sort_pairs<uint32_t>(L.depth_plan, radix::kSkipInvalid, at<uint32_t>(ws, L.keys_a),
-                                         at<uint32_t>(ws, L.vals_a), at<uint32_t>(ws, L.keys_b),
-                                         at<uint32_t>(ws, L.vals_b), counters + kCntVisible, L.geo.n,
-                                         at<uint32_t>(ws, L.hist_depth), at<uint32_t>(ws, L.bases_depth),
-                                         at<uint32_t>(ws, L.status_depth),
-                                         counters + kCntError, stream, "raster_depth_sort");
-        if (rc != INPC_OK) return rc;
-        {
-            // depth-ordered points -> per-tile instance lists (instances.hpp); the bin table is free again
-            const uint32_t* order = at<uint32_t>(ws, L.pub.depth_order);
-            const uint32_t* bin_start = at<uint32_t>(ws, L.pub.bin_start);
-            const uint16_t* coarse = at<uint16_t>(ws, L.bin_coarse);
-            INPC_LAUNCH_LDS("raster_inst_count", instances::k_inst_count, dim3(instances::kChunks), dim3(kBinThreads),
-                            (size_t)L.geo.n_tiles * 4, stream, order, bin_start, coarse, (const uint32_t*)counters,
-                            at<uint32_t>(ws, L.bin_table), L.geo.n, L.geo.gw, L.geo.n_tiles);
-            INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<instances::kChunks>, dim3(div_up(L.geo.n_tiles, kWave)),
-                        dim3(kOffsetWaves * kWave), stream, at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total),
-                        L.geo.n_tiles);
-            INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
-                        (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.inst_start), L.geo.n_tiles);
-            INPC_LAUNCH("raster_tile_ranges", instances::k_ranges_from_starts, dim3(div_up(L.geo.n_tiles, kBlock)),
-                        dim3(kBlock), stream, (const uint32_t*)at<uint32_t>(ws, L.inst_start),
-                        at<uint2>(ws, L.pub.tile_ranges), L.geo.n_tiles);
-            INPC_LAUNCH_LDS("raster_inst_emit", instances::k_inst_emit, dim3(instances::kChunks), dim3(instances::kEmitThreads),
-                            (size_t)L.geo.n_tiles * 4, stream, order, bin_start, coarse, (const uint32_t*)counters,
-                            (const uint32_t*)at<uint32_t>(ws, L.bin_table),
-                            (const uint32_t*)at<uint32_t>(ws, L.inst_start), at<uint16_t>(ws, L.inst_keys_a),
-                            at<uint32_t>(ws, L.inst_vals_a), L.geo.n, L.geo.gw, L.geo.n_tiles, (int)L.pub.end_bit);
-        }
+        INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort, dim3(L.geo.n_tiles), dim3(tilesort::kThreads),
+                        tilesort::kSharedBytes, stream, (const uint2*)at<uint2>(ws, L.pub.tile_ranges),
+                        (const uint32_t*)at<uint32_t>(ws, L.tile_order), at<uint64_t>(ws, L.pairs),
+                        at<uint64_t>(ws, L.pairs_scratch), at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
     }
-    INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
-                (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
     return dispatch_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }
 
@@ -1303,39 +1269,25 @@ int inpc_raster_backward(const inpc_raster_config* cfg, const float* grad_image,
     return INPC_OK;
 }
 
-#ifdef INPC_BLEND_PROFILE
-// development aid: per-phase shader clocks of k_blend_forward, summed over blocks (thread 0 of each)
-int inpc_debug_blend_profile(unsigned long long out[8], int reset) {
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(g_blend_profile), 8 * sizeof(unsigned long long)) != hipSuccess) return -1;
-    if (reset) {
-        unsigned long long zero[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (hipMemcpyToSymbol(HIP_SYMBOL(g_blend_profile), zero, sizeof(zero)) != hipSuccess) return -1;
-    }
-    return 0;
-}
-#endif
-
-#ifdef INPC_SORT_PROFILE
-int inpc_debug_sort_profile(unsigned long long out[8], int reset) {
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(inpc::radix::g_sort_profile), 8 * sizeof(unsigned long long)) != hipSuccess) return -1;
-    if (reset) {
-        unsigned long long zero[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (hipMemcpyToSymbol(HIP_SYMBOL(inpc::radix::g_sort_profile), zero, sizeof(zero)) != hipSuccess) return -1;
-    }
-    return 0;
-}
-#endif
-
 int inpc_raster_read_counters(const inpc_raster_config* cfg, const void* ws, uint32_t counters_host[3], void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     Layout L;
     const int rc = make_layout(cfg, L);
     if (rc != INPC_OK) return rc;
-    uint32_t host[3] = {0, 0, 0};
+    uint32_t host[kCntWords] = {};
     INPC_HIP_CHECK(hipMemcpyAsync(host, (const char*)ws + L.pub.counters, sizeof(host), hipMemcpyDeviceToHost, stream));
     INPC_HIP_CHECK(hipStreamSynchronize(stream));
-    if (counters_host) memcpy(counters_host, host, sizeof(host));
-    if (host[2]) return fail(INPC_E_DEVICE, "rasterizer look-back gave up waiting (device error flag set)");
+    if (counters_host) {
+        counters_host[0] = host[kCntVisible];
+        counters_host[1] = host[kCntInstances];
+        counters_host[2] = host[kCntError];
+    }
+    if (host[kCntError]) return fail(INPC_E_DEVICE, "rasterizer raised its device error flag");
+    if (host[kCntOverflow])
+        return fail(INPC_E_WORKSPACE,
+                    "raster: %u instances (%u of them of points that touch several tiles) do not fit max_instances = %u "
+                    "(%u of those); nothing was drawn",
+                    host[kCntInstances], host[kCntRows], L.geo.capacity, L.geo.row_capacity);
     return INPC_OK;
 }
 

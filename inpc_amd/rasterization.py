@@ -68,9 +68,16 @@ _gaussian_capacity_hint = {"per_point": 0.0}
 
 
 def _config(settings: RasterizerSettings, n_points: int, tile: int, channels: int, feature_mode: int,
-            inference: bool) -> _lib.RasterConfig:
+            inference: bool, max_instances: int = 0) -> _lib.RasterConfig:
     return _lib.RasterConfig(int(n_points), int(tile), int(channels), int(feature_mode),
-                             _lib.RASTER_INFERENCE if inference else 0, settings.camera())
+                             _lib.RASTER_INFERENCE if inference else 0, settings.camera(), int(max_instances))
+
+
+# Up to this many points the bilinear workspace is sized for four instances per point, which no input can exceed;
+# beyond it the library's default capacity (what evenly spread points need, with a margin) is used and the
+# instance count is read back after the forward pass, as the reference reads it back to size its buffers
+# (B/rasterization/src/bilinear/forward.cu:86-89).
+_ALWAYS_FITS_POINTS = 1 << 20
 
 
 def query_layout(cfg: _lib.RasterConfig) -> _lib.RasterLayout:
@@ -97,9 +104,25 @@ def _checked_inputs(positions, features, opacities, feature_mode: int, channels:
             raise RuntimeError("expected scalar type Float")
         if opacities.numel() != n:
             raise RuntimeError("opacities must hold one value per point")
-    if not positions.is_cuda or not features.is_cuda:
+    if not positions.is_cuda or not features.is_cuda or (opacities is not None and not opacities.is_cuda):
         raise RuntimeError("expected tensors on the GPU")
+    if features.device != positions.device or (opacities is not None and opacities.device != positions.device):
+        raise RuntimeError("expected all tensors on the same device")
     return positions, features, opacities
+
+
+def _checked_camera_tensor(t: torch.Tensor, numel: int, name: str, device) -> torch.Tensor:
+    """The camera tensors reach the kernels as raw float pointers: they must be fp32 on the points' device
+    (the reference's data_ptr<float>() raises for another dtype, B/rasterization/src/rasterization_api.cu:61-65)."""
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a tensor")
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"expected scalar type Float for {name}")
+    if not t.is_cuda or t.device != device:
+        raise RuntimeError(f"expected {name} on the device of the points ({device})")
+    if t.numel() != numel:
+        raise RuntimeError(f"{name} must hold {numel} values")
+    return t.contiguous()
 
 
 def _forward_gaussian(settings: RasterizerSettings, positions, features, opacities, tile: int, channels: int,
@@ -114,12 +137,14 @@ def _forward_gaussian(settings: RasterizerSettings, positions, features, opaciti
     alpha = torch.empty((1, H, W), dtype=torch.float32, device=device)
     weights = None if inference else torch.empty(n, dtype=torch.float32, device=device)
     depth = torch.empty((1, H, W), dtype=torch.float32, device=device) if inference else None
-    w2c = settings.w2c.contiguous()
-    cam_position = settings.cam_position.contiguous()
+    w2c = _checked_camera_tensor(settings.w2c, 16, "w2c", device)
+    cam_position = _checked_camera_tensor(settings.cam_position, 3, "cam_position", device)
     if scales is not None:
         scales = scales.contiguous()
         if scales.dtype != torch.float32:
             raise RuntimeError("expected scalar type Float")
+        if not scales.is_cuda or scales.device != device:
+            raise RuntimeError("expected scales on the device of the points")
         if scales.numel() != n:
             raise RuntimeError("scales must hold one value per point")
     capacity = int(4 * n + 65536 + _gaussian_capacity_hint["per_point"] * n)
@@ -164,21 +189,36 @@ def _forward_native(settings: RasterizerSettings, positions, features, opacities
     device = positions.device
     sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
     out_channels = 4 if sh else channels
-    cfg = _config(settings, n, tile, out_channels, feature_mode, inference)
-    layout = query_layout(cfg)
-    workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
     H, W = settings.height, settings.width
     image = torch.empty((out_channels, H, W), dtype=torch.float32, device=device)
     alpha = torch.empty((1, H, W), dtype=torch.float32, device=device)
     weights = None if inference else torch.empty(n, dtype=torch.float32, device=device)
     depth = torch.empty((1, H, W), dtype=torch.float32, device=device) if inference else None
-    w2c = settings.w2c.contiguous()
-    cam_position = settings.cam_position.contiguous()
-    _lib.check(_lib.lib().inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features),
-                                              _lib.ptr(opacities), _lib.ptr(w2c), _lib.ptr(cam_position),
-                                              _lib.ptr(image), _lib.ptr(alpha), _lib.ptr(weights), _lib.ptr(depth),
-                                              _lib.ptr(workspace), layout.total_bytes, _lib.current_stream()),
-               "inpc_raster_forward")
+    w2c = _checked_camera_tensor(settings.w2c, 16, "w2c", device)
+    cam_position = _checked_camera_tensor(settings.cam_position, 3, "cam_position", device)
+    lib = _lib.lib()
+    everything = max(4 * n, 1)
+    capacity = everything if n <= _ALWAYS_FITS_POINTS else 0
+    for _ in range(2):
+        cfg = _config(settings, n, tile, out_channels, feature_mode, inference, capacity)
+        layout = query_layout(cfg)
+        workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+        stream = _lib.current_stream()
+        _lib.check(lib.inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
+                                           _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image), _lib.ptr(alpha),
+                                           _lib.ptr(weights), _lib.ptr(depth), _lib.ptr(workspace), layout.total_bytes,
+                                           stream), "inpc_raster_forward")
+        if layout.max_instances >= everything:
+            break
+        counters = (C.c_uint32 * 3)()
+        rc = lib.inpc_raster_read_counters(C.byref(cfg), _lib.ptr(workspace), C.byref(counters), stream)
+        if rc == 0:
+            break
+        if rc != _lib.E_WORKSPACE:
+            _lib.check(rc, "inpc_raster_read_counters")
+        # the points touch more tiles than the default capacity holds: once more with room for all of them
+        capacity = everything
+        del workspace
     return image, alpha, (depth if inference else weights), workspace, cfg
 
 
@@ -216,6 +256,10 @@ class _Rasterize(torch.autograd.Function):
         grad_alpha = torch.zeros_like(alpha) if grad_alpha is None else grad_alpha.contiguous()
         if grad_image.dtype != torch.float32 or grad_alpha.dtype != torch.float32:
             raise RuntimeError("expected scalar type Float")
+        if grad_image.device != device or grad_alpha.device != device:
+            raise RuntimeError("expected the gradients on the device of the points")
+        if grad_image.shape != image.shape or grad_alpha.shape != alpha.shape:
+            raise RuntimeError("gradient shapes differ from the outputs")
         mode = base.feature_mode
         scratch = None
         if mode == _lib.FEAT_SH36_F16:
@@ -227,7 +271,7 @@ class _Rasterize(torch.autograd.Function):
         else:
             grad_features = torch.empty((n, base.channels), dtype=torch.float32, device=device)
         grad_opacities = torch.empty((n, 1), dtype=torch.float32, device=device)
-        cam_position = settings.cam_position.contiguous()
+        cam_position = _checked_camera_tensor(settings.cam_position, 3, "cam_position", device)
         backward = _lib.lib().inpc_gaussian_backward if gaussian else _lib.lib().inpc_raster_backward
         _lib.check(backward(C.byref(cfg), _lib.ptr(grad_image), _lib.ptr(grad_alpha), _lib.ptr(image), _lib.ptr(alpha),
                             _lib.ptr(positions), _lib.ptr(cam_position), _lib.ptr(grad_features),

@@ -54,6 +54,7 @@ class RasterConfig(C.Structure):
         ("feature_mode", C.c_int32),
         ("flags", C.c_uint32),
         ("cam", Camera),
+        ("max_instances", C.c_uint32),   # capacity of the HIP library's buffers; the oracle ignores it
     ]
 
 

@@ -135,14 +135,16 @@ class RasterRun:
     """inpc_raster_forward (+ backward) through the C ABI on numpy inputs."""
 
     def __init__(self, hv, positions, features, opacities, tile=16, channels=4, feature_mode=_lib.FEAT_DIRECT_F32,
-                 inference=False, device="cuda:0"):
+                 inference=False, device="cuda:0", max_instances=None, keep_geometry=True):
         self.lib = _lib.lib()
         self.hv = hv
         self.n = len(positions)
         sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
         self.C = 4 if sh else channels
-        self.cfg = _lib.RasterConfig(self.n, tile, self.C, feature_mode, _lib.RASTER_INFERENCE if inference else 0,
-                                     cam_struct(hv.camera))
+        flags = (_lib.RASTER_INFERENCE if inference else 0) | (_lib.RASTER_KEEP_GEOMETRY if keep_geometry else 0)
+        # room for every possible instance unless a test asks for less
+        capacity = max(4 * self.n, 1) if max_instances is None else max_instances
+        self.cfg = _lib.RasterConfig(self.n, tile, self.C, feature_mode, flags, cam_struct(hv.camera), capacity)
         self.layout = _lib.RasterLayout()
         _lib.check(self.lib.inpc_raster_layout_query(C.byref(self.cfg), C.byref(self.layout)), "layout")
         self.inference = inference
@@ -179,50 +181,59 @@ class RasterRun:
         return self.ws[offset:offset + nbytes].cpu().numpy().view(dtype)
 
     def debug(self):
-        """Intermediate buffers decoded into the oracle's shapes (record slots mapped back to point ids)."""
+        """Intermediate buffers decoded into the oracle's shapes. Needs keep_geometry."""
         L, n = self.layout, self.n
         v, i = self.counters()
-        stride = L.record_stride
-        raw = self._buf(L.point_record, v * stride, np.uint8).reshape(v, stride)
-        head = raw[:, :32].copy().view(np.float32).reshape(v, 8)
-        head_u = head.view(np.uint32)
-        orig = head_u[:, 3].astype(np.int64)          # point id of every record slot
-        info = head_u[:, 4]
-        assert len(np.unique(orig)) == v, "two records name the same point"
-        assert ((info >> 18) & 1).all(), "a record of a point that is not drawn"
+        assert L.debug_geometry != 0, "RasterRun(keep_geometry=True) keeps the projection for inspection"
+        geo = self._buf(L.debug_geometry, 4 * n, np.float32).reshape(n, 4)
+        info = geo.view(np.uint32)[:, 3]
+        drawn = ((info >> 18) & 1).astype(bool)
+        assert int(drawn.sum()) == v, "the visible count differs from the number of drawn points"
         tile0 = info & 0xFFFF
         nx = ((info >> 16) & 1) + 1
         ny = ((info >> 17) & 1) + 1
-        bin_start = self._buf(L.bin_start, L.n_tiles + 1, np.uint32)
-        assert bin_start[0] == 0 and bin_start[-1] == v and (np.diff(bin_start.astype(np.int64)) >= 0).all()
-        # every record lies in the bin of its first tile
-        slot_tile = np.searchsorted(bin_start, np.arange(v), side="right") - 1
-        assert (slot_tile == tile0).all(), "a record outside the bin of its first tile"
         x0, y0 = tile0 % L.grid_width, tile0 // L.grid_width
-        n_touched = np.zeros(n, np.uint32)
-        bounds = np.zeros((n, 4), np.uint16)
-        xy = np.zeros((n, 2), np.float32)
-        opacity = np.zeros(n, np.float32)
-        depth = np.zeros(n, np.float32)
-        n_touched[orig] = nx * ny
-        bounds[orig] = np.stack([x0, x0 + nx, y0, y0 + ny], axis=1)
-        xy[orig] = head[:, :2]
-        opacity[orig] = head[:, 2]
-        depth[orig] = head[:, 5]
-        order_vals = self._buf(L.depth_order, n, np.uint32)[:v]
-        span = order_vals & 3
-        assert (span == ((info >> 16) & 3)[order_vals >> 2]).all(), "span bits of the sort value differ from the record"
+        n_touched = np.where(drawn, nx * ny, 0).astype(np.uint32)
+        bounds = np.where(drawn[:, None], np.stack([x0, x0 + nx, y0, y0 + ny], axis=1), 0).astype(np.uint16)
+        xy = np.where(drawn[:, None], geo[:, :2], 0).astype(np.float32)
+        depth = np.where(drawn, geo[:, 2], 0).astype(np.float32)
+        assert int(n_touched.sum()) == i, "the instance count differs from the sum of the touched tiles"
+        # blend records: one per drawn point, at the point's index
+        stride = L.record_stride
+        raw = self._buf(L.point_record, n * stride, np.uint8).reshape(n, stride)
+        head = raw[:, :32].copy().view(np.float32).reshape(n, 8)
+        head_u = head.view(np.uint32)
+        tag = head_u[:, 5]
+        assert ((tag & 0x0FFFFFFF)[drawn] == np.nonzero(drawn)[0]).all(), "a record does not name its own point"
+        assert ((((tag >> 29) & 3) == ((info >> 16) & 3)) | ~drawn).all(), "span bits of a record differ from its bounds"
+        if not self.inference:
+            assert ((((tag >> 28) & 1) == (n_touched > 1)) | ~drawn).all(), "several-tiles flag of a record is wrong"
+        # footprint weights against the float expressions of the reference's blend (kernels.cu:284-287) at the two
+        # candidate pixels per axis, from the kept screen position
+        left = (head_u[:, 6] & 0xFFFF).astype(np.int64) - 1
+        top = (head_u[:, 6] >> 16).astype(np.int64) - 1
+        for axis, first, w0, w1 in ((0, left, head[:, 0], head[:, 1]), (1, top, head[:, 2], head[:, 3])):
+            s_ = geo[:, axis]
+            expect_first = np.floor((s_ - np.float32(0.5)).astype(np.float32)).astype(np.int64)
+            assert (first[drawn] == expect_first[drawn]).all(), "left / top candidate pixel of a record is wrong"
+            for k, w in ((0, w0), (1, w1)):
+                d = np.abs(s_ - ((first + k).astype(np.float32) + np.float32(0.5))).astype(np.float32)
+                expect = np.where(d >= 1, np.float32(0), np.clip(np.float32(1) - d, 0, 1)).astype(np.float32)
+                assert (w.view(np.uint32)[drawn] == expect.view(np.uint32)[drawn]).all(), "footprint weight of a record is wrong"
+        opacity = np.where(drawn, head[:, 4], 0).astype(np.float32)
         feat_dtype = np.float16 if self.cfg.feature_mode == _lib.FEAT_DIRECT_F16 else np.float32
-        feats = raw[:, 32:32 + self.C * np.dtype(feat_dtype).itemsize].copy().view(feat_dtype).reshape(v, self.C)
-        features_view = np.zeros((n, self.C), np.float32)
-        features_view[orig] = feats.astype(np.float32)
+        feats = raw[:, 32:32 + self.C * np.dtype(feat_dtype).itemsize].copy().view(feat_dtype).reshape(n, self.C)
+        features_view = np.where(drawn[:, None], feats.astype(np.float32), 0).astype(np.float32)
+        bin_start = self._buf(L.bin_start, L.n_tiles + 1, np.uint32)
+        assert bin_start[0] == 0 and bin_start[-1] == i and (np.diff(bin_start.astype(np.int64)) >= 0).all()
+        points = self._buf(L.instance_points, max(i, 1), np.uint32)[:i]
+        keys = np.repeat(np.arange(L.n_tiles, dtype=np.uint16), np.diff(bin_start.astype(np.int64)))
         return {
             "n_visible": v, "n_instances": i, "n_touched": n_touched, "bounds": bounds, "screen_xy": xy,
             "opacity": opacity, "depth": depth, "features_view": features_view,
-            "depth_keys": (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32),
-            "depth_order": orig[order_vals >> 2].astype(np.uint32),
-            "instance_keys": self._buf(L.instance_keys, 4 * n, np.uint16)[:i],
-            "instance_points": orig[self._buf(L.instance_slots, 4 * n, np.uint32)[:i]].astype(np.uint32),
+            "instance_keys": keys, "instance_points": points,
+            # depth key of every instance, in final order: what the per-tile sort ordered by
+            "instance_depth_keys": geo.view(np.uint32)[points, 2],
             "tile_ranges": self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2),
         }
 

@@ -86,33 +86,44 @@ def test_header_is_plain_c_and_structs_match_ctypes(tmp_path):
                            f"{_lib.FEAT_RAW37_F16} {_lib.RASTER_INFERENCE}"
 
 
-def make_cfg(n, w, h, tile=16, channels=8, mode=_lib.FEAT_DIRECT_F32, flags=0):
-    return _lib.RasterConfig(n, tile, channels, mode, flags, _lib.Camera(w, h, 1000.0, 1000.0, w / 2, h / 2, 0.01, 100.0))
+def make_cfg(n, w, h, tile=16, channels=8, mode=_lib.FEAT_DIRECT_F32, flags=0, max_instances=0):
+    return _lib.RasterConfig(n, tile, channels, mode, flags, _lib.Camera(w, h, 1000.0, 1000.0, w / 2, h / 2, 0.01, 100.0),
+                             max_instances)
 
 
 def test_layout_query_on_the_host():
     lib = _lib.lib()
-    assert lib.inpc_abi_version() >= 1
+    assert lib.inpc_abi_version() >= 2
+    n = 8_388_608
     layout = _lib.RasterLayout()
-    cfg = make_cfg(8_388_608, 1237, 822)
+    cfg = make_cfg(n, 1237, 822)
     assert lib.inpc_raster_layout_query(C.byref(cfg), C.byref(layout)) == 0
     assert (layout.grid_width, layout.grid_height, layout.n_tiles) == (78, 52, 78 * 52)
     assert layout.record_stride == 64 and layout.total_bytes % 256 == 0
     assert layout.depth_key_bias == int(np.float32(0.01).view(np.uint32))
-    offsets = [layout.counters, layout.bin_start, layout.point_record, layout.depth_order, layout.depth_keys,
-               layout.instance_keys, layout.instance_slots, layout.tile_ranges]
+    offsets = [layout.counters, layout.bin_start, layout.point_record, layout.instance_points, layout.tile_ranges]
     assert all(o % 256 == 0 and o < layout.total_bytes for o in offsets) and len(set(offsets)) == len(offsets)
-    # every point can touch four tiles: the workspace holds at least 4 N instances of 6 bytes and N records
-    assert layout.total_bytes >= 8_388_608 * (64 + 4 * 6)
-    # bits the tile sort has to look at
+    assert layout.debug_geometry == 0
+    # default capacity: what evenly spread points need, (1 + 1/16)^2 instances per point, with a margin
+    assert 1.129 * n < layout.max_instances < 1.25 * n
+    # one record per point, per instance a sort pair, a list entry and (training) an ordered record
+    assert layout.total_bytes >= n * 64 + layout.max_instances * (8 + 4 + 64)
+    assert layout.total_bytes < 1.5e9
     assert layout.end_bit == (layout.n_tiles - 1).bit_length() == 12
-    # a configuration with a backward pass also holds one ordered record (64 bytes here) and one gradient row per
-    # possible instance; an inference configuration holds neither
+    # the caller may ask for room for every possible instance, and never gets more
+    for asked, got in ((4 * n, 4 * n), (0xFFFFFFFF, 4 * n), (n, n)):
+        sized = _lib.RasterLayout()
+        assert lib.inpc_raster_layout_query(C.byref(make_cfg(n, 1237, 822, max_instances=asked)), C.byref(sized)) == 0
+        assert sized.max_instances == got
+    # keeping the projection costs 16 bytes per point
+    kept = _lib.RasterLayout()
+    assert lib.inpc_raster_layout_query(C.byref(make_cfg(n, 1237, 822, flags=_lib.RASTER_KEEP_GEOMETRY)), C.byref(kept)) == 0
+    assert kept.debug_geometry != 0 and kept.total_bytes - layout.total_bytes == n * 16
+    # a configuration with a backward pass also holds one ordered record (64 bytes here) per instance and the
+    # gradient rows of the points that straddle tiles; an inference configuration holds neither
     inference = _lib.RasterLayout()
-    cfg_inf = make_cfg(8_388_608, 1237, 822)
-    cfg_inf.flags = _lib.RASTER_INFERENCE
-    assert lib.inpc_raster_layout_query(C.byref(cfg_inf), C.byref(inference)) == 0
-    assert layout.total_bytes - inference.total_bytes >= 4 * 8_388_608 * (64 + 4 * 8 + 4)
+    assert lib.inpc_raster_layout_query(C.byref(make_cfg(n, 1237, 822, flags=_lib.RASTER_INFERENCE)), C.byref(inference)) == 0
+    assert layout.total_bytes - inference.total_bytes >= layout.max_instances * (64 - 8)
     small = _lib.RasterLayout()
     assert lib.inpc_raster_layout_query(C.byref(make_cfg(0, 64, 64, 8, 4)), C.byref(small)) == 0
     assert small.total_bytes > 0 and small.n_tiles == 64

@@ -39,10 +39,13 @@ def check_structure(dbg, ref):
     np.testing.assert_array_equal(dbg["screen_xy"].view(np.uint32), ref["screen_xy"].view(np.uint32))
     vis = ref["n_touched"] > 0
     np.testing.assert_array_equal(dbg["depth"][vis].view(np.uint32), ref["depth"][vis].view(np.uint32))
-    np.testing.assert_array_equal(dbg["depth_keys"], ref["depth_keys"])
-    np.testing.assert_array_equal(dbg["depth_order"], ref["depth_order"])
+    # the oracle's depth keys are those of its depth-ordered points; here every tile is sorted on its own, so the
+    # comparison is per instance, in final (tile, depth bits, point index) order
+    key_of_point = np.zeros(len(ref["n_touched"]), np.uint32)
+    key_of_point[ref["depth_order"]] = ref["depth_keys"]
     np.testing.assert_array_equal(dbg["instance_keys"], ref["instance_keys"])
     np.testing.assert_array_equal(dbg["instance_points"], ref["instance_points"])
+    np.testing.assert_array_equal(dbg["instance_depth_keys"], key_of_point[ref["instance_points"]])
     np.testing.assert_array_equal(dbg["tile_ranges"], ref["tile_ranges"])
 
 
