@@ -8,11 +8,11 @@
 // (depth key, point index) pair per instance into the bin of its tile, and one block per tile sorts its bin.
 //
 //   elements   u64 = depth key << 32 | point index: the order wanted is plain ascending u64 order
-//   in LDS     least-significant-digit radix sort, 4-bit digits, over the key bits. A thread owns kPer
-//              consecutive elements and counts their digits in sixteen 4-bit fields of one 64-bit register; the
-//              16 x kThreads counts are scanned in digit-major order, which is a stable ranking. Digits
-//              that are the same for all elements of the tile are skipped (the depths of one tile mostly share
-//              their leading bits).
+//   in LDS     least-significant-digit radix sort, 4-bit digits, over the key bits. A thread owns up to 15
+//              consecutive elements, holds them in registers during a pass (so the pass works in place) and
+//              counts their digits in sixteen 4-bit fields of one 64-bit register; the 16 x threads counts are
+//              scanned in digit-major order, which is a stable ranking. Digits that are the same for all
+//              elements of the tile are skipped (the depths of one tile mostly share their leading bits).
 //   ties       elements with equal keys come out in the order they were binned, which is arbitrary: a few
 //              ties are put right in place (rank by point index inside the run of equal keys); a tile with
 //              many is sorted again over all 64 bits.
@@ -25,14 +25,15 @@ namespace tilesort {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / kWave;
-constexpr int kMaxPer = 7;                  // elements per thread: 1, 3, 5 or 7 (odd: conflict-free LDS rows)
+constexpr int kMaxPer = 15;                 // elements per thread: 3, 7, 11 or 15 (odd: conflict-free LDS rows; at
+                                            // most 15: a thread's digit counts fit 4-bit fields)
 constexpr int kCap = kThreads * kMaxPer;    // elements sorted in LDS at a time
 constexpr int kDigits = 16;
 constexpr uint64_t kPad = ~0ull;            // sorts behind every element
 constexpr uint32_t kFewTies = 16;           // threads with tied elements up to which ties are fixed in place
 
 struct Shared {
-    uint64_t buf[2][kCap];
+    uint64_t buf[kCap];
     alignas(16) uint16_t count[kDigits * kThreads];   // [digit][thread], scanned in this order
     uint32_t wave_sum[kWaves];
     uint32_t bits_or[2], bits_and[2];                 // over the tile's elements: [0] point index, [1] key
@@ -52,69 +53,85 @@ __device__ __forceinline__ uint32_t wave_inclusive_u32(uint32_t v) {
     return v;
 }
 
-// One stable counting pass on the 4-bit digit at bit `shift`, from sh.buf[src] to sh.buf[1 - src]. All
-// kThreads threads call it; kPer * kThreads elements (padding included) take part. Ends with a barrier.
+// The 4-bit digit at bit `shift` (a multiple of 4) of a 64-bit element.
+__device__ __forceinline__ uint32_t digit_of(uint64_t v, int shift) {
+    const uint32_t word = shift >= 32 ? hi32(v) : lo32(v);
+    return (word >> (shift & 31)) & 15u;
+}
+
+// One stable counting pass, in place, on the 4-bit digit at bit `shift`. The first `active` threads (a multiple
+// of 64) own kPer consecutive elements each; every thread of the block calls it (the others only meet the
+// barriers). All elements are in registers before the first one is stored, so one buffer suffices.
 template <int kPer>
-__device__ __forceinline__ void digit_pass(Shared& sh, int src, int shift) {
+__device__ __forceinline__ void digit_pass(Shared& sh, uint32_t active, int shift) {
     const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
-    const uint64_t* from = sh.buf[src];
-    uint64_t* to = sh.buf[1 - src];
+    const bool on = t < active;
     uint64_t v[kPer];
     uint64_t fields = 0ull;   // sixteen 4-bit counters: kPer <= 15 elements per thread cannot overflow one
+    if (on) {
 #pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-        v[e] = from[t * kPer + e];
-        fields += 1ull << (4u * (uint32_t)((v[e] >> shift) & 15ull));
+        for (int e = 0; e < kPer; ++e) {
+            v[e] = sh.buf[t * kPer + e];
+            fields += 1ull << (4u * digit_of(v[e], shift));
+        }
+#pragma unroll
+        for (int d = 0; d < kDigits; ++d) sh.count[d * active + t] = (uint16_t)((fields >> (4 * d)) & 15ull);
     }
-#pragma unroll
-    for (int d = 0; d < kDigits; ++d) sh.count[d * kThreads + t] = (uint16_t)((fields >> (4 * d)) & 15ull);
     __syncthreads();
-    // exclusive scan of the 16 * kThreads counts in storage order; thread t owns entries [16 t, 16 t + 16)
+    // exclusive scan of the 16 * active counts in storage order; thread t owns entries [16 t, 16 t + 16)
+    uint32_t w[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};   // two counts per word
+    uint32_t sum = 0, incl = 0;
     uint4* mine = (uint4*)(sh.count + 16u * t);
-    uint4 a = mine[0], b = mine[1];
-    uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};   // two counts per word
-    uint32_t sum = 0;
+    if (on) {
+        const uint4 a = mine[0], b = mine[1];
+        w[0] = a.x, w[1] = a.y, w[2] = a.z, w[3] = a.w, w[4] = b.x, w[5] = b.y, w[6] = b.z, w[7] = b.w;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sum += (w[i] & 0xFFFFu) + (w[i] >> 16);
-    const uint32_t incl = wave_inclusive_u32(sum);
-    if (lane == 63u) sh.wave_sum[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - sum;
-#pragma unroll
-    for (int k = 0; k < kWaves; ++k) run += (uint32_t)k < wave ? sh.wave_sum[k] : 0u;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t c0 = w[i] & 0xFFFFu, c1 = w[i] >> 16;
-        w[i] = run | ((run + c0) << 16);
-        run += c0 + c1;
+        for (int i = 0; i < 8; ++i) sum += (w[i] & 0xFFFFu) + (w[i] >> 16);
+        incl = wave_inclusive_u32(sum);
+        if (lane == 63u) sh.wave_sum[wave] = incl;
     }
-    mine[0] = make_uint4(w[0], w[1], w[2], w[3]);
-    mine[1] = make_uint4(w[4], w[5], w[6], w[7]);
     __syncthreads();
-    uint64_t seen = 0ull;     // how many of this thread's earlier elements had the same digit
+    if (on) {
+        uint32_t run = incl - sum;
 #pragma unroll
-    for (int e = 0; e < kPer; ++e) {
-        const uint32_t d = (uint32_t)((v[e] >> shift) & 15ull);
-        const uint32_t at = (uint32_t)sh.count[d * kThreads + t] + (uint32_t)((seen >> (4u * d)) & 15ull);
-        seen += 1ull << (4u * d);
-        to[at] = v[e];
+        for (int k = 0; k < kWaves; ++k) run += (uint32_t)k < wave ? sh.wave_sum[k] : 0u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t c0 = w[i] & 0xFFFFu, c1 = w[i] >> 16;
+            w[i] = run | ((run + c0) << 16);
+            run += c0 + c1;
+        }
+        mine[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        mine[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    }
+    __syncthreads();
+    if (on) {
+        uint64_t seen = 0ull;     // how many of this thread's earlier elements had the same digit
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) {
+            const uint32_t d = digit_of(v[e], shift);
+            const uint32_t at = (uint32_t)sh.count[d * active + t] + (uint32_t)((seen >> (4u * d)) & 15ull);
+            seen += 1ull << (4u * d);
+            sh.buf[at] = v[e];
+        }
     }
     __syncthreads();
 }
 
-// Sorts the n <= kPer * kThreads elements in sh.buf[0] ascending as u64 (the slots behind them hold kPad);
-// returns the buffer that holds the result. All threads call it.
+// Sorts the n <= kPer * active elements in sh.buf ascending as u64 (the slots behind them, up to
+// kPer * active, hold kPad). All threads of the block call it.
 template <int kPer>
-__device__ int sort_run(Shared& sh, uint32_t n, int key_bits) {
+__device__ void sort_run(Shared& sh, uint32_t n, uint32_t active, int key_bits) {
     const uint32_t t = threadIdx.x, lane = t & 63u;
+    const bool on = t < active;
     // bits that differ between the elements
     {
         uint32_t or_lo = 0u, or_hi = 0u, and_lo = ~0u, and_hi = ~0u;
 #pragma unroll
         for (int e = 0; e < kPer; ++e) {
             const uint32_t p = t * kPer + e;
-            if (p < n) {
-                const uint64_t v = sh.buf[0][p];
+            if (on && p < n) {
+                const uint64_t v = sh.buf[p];
                 or_lo |= lo32(v);
                 or_hi |= hi32(v);
                 and_lo &= lo32(v);
@@ -132,7 +149,7 @@ __device__ int sort_run(Shared& sh, uint32_t n, int key_bits) {
             sh.bits_and[t] = ~0u;
         }
         __syncthreads();
-        if (lane == 0u) {
+        if (lane == 0u && on) {
             atomicOr(&sh.bits_or[0], or_lo);
             atomicOr(&sh.bits_or[1], or_hi);
             atomicAnd(&sh.bits_and[0], and_lo);
@@ -141,83 +158,78 @@ __device__ int sort_run(Shared& sh, uint32_t n, int key_bits) {
         __syncthreads();
     }
     const uint32_t vary_lo = sh.bits_or[0] ^ sh.bits_and[0], vary_hi = sh.bits_or[1] ^ sh.bits_and[1];
-    int cur = 0;
     auto key_passes = [&]() {
         for (int shift = 0; shift < key_bits; shift += 4)
-            if ((vary_hi >> shift) & 15u) {
-                digit_pass<kPer>(sh, cur, 32 + shift);
-                cur ^= 1;
-            }
+            if ((vary_hi >> shift) & 15u) digit_pass<kPer>(sh, active, 32 + shift);
     };
     key_passes();
     // elements with equal keys stand in the order they were binned; the order wanted is by point index
     bool tied[kPer];
     bool any = false;
-    {
-        const uint64_t* b = sh.buf[cur];
 #pragma unroll
-        for (int e = 0; e < kPer; ++e) {
-            const uint32_t p = t * kPer + e;
-            tied[e] = false;
-            if (p < n) {
-                const uint32_t key = hi32(b[p]);
-                tied[e] = (p > 0u && hi32(b[p - 1u]) == key) || (p + 1u < n && hi32(b[p + 1u]) == key);
-            }
-            any = any || tied[e];
+    for (int e = 0; e < kPer; ++e) {
+        const uint32_t p = t * kPer + e;
+        tied[e] = false;
+        if (on && p < n) {
+            const uint32_t key = hi32(sh.buf[p]);
+            tied[e] = (p > 0u && hi32(sh.buf[p - 1u]) == key) || (p + 1u < n && hi32(sh.buf[p + 1u]) == key);
         }
+        any = any || tied[e];
     }
     const uint32_t threads_tied = (uint32_t)__syncthreads_count(any);
-    if (threads_tied == 0u) return cur;
+    if (threads_tied == 0u) return;
     if (threads_tied <= kFewTies) {
-        // few ties (runs of at most kFewTies * kPer elements): every tied element finds its run and its rank in it
-        const uint64_t* b = sh.buf[cur];
-        uint64_t* to = sh.buf[cur ^ 1];
+        // few ties (runs of at most kFewTies * kPer elements): every tied element finds its run and its rank in
+        // it; all of them are read before the first one is stored
+        uint32_t at[kPer];
+        uint64_t v[kPer];
 #pragma unroll
         for (int e = 0; e < kPer; ++e) {
+            if (!tied[e]) continue;
             const uint32_t p = t * kPer + e;
-            const uint64_t v = b[p];
-            uint32_t at = p;
-            if (tied[e]) {
-                const uint32_t key = hi32(v);
-                uint32_t first = p, last = p + 1u;
-                while (first > 0u && hi32(b[first - 1u]) == key) --first;
-                while (last < n && hi32(b[last]) == key) ++last;
-                uint32_t smaller = 0;
-                for (uint32_t q = first; q < last; ++q) smaller += lo32(b[q]) < lo32(v) ? 1u : 0u;
-                at = first + smaller;
-            }
-            to[at] = v;
+            v[e] = sh.buf[p];
+            const uint32_t key = hi32(v[e]);
+            uint32_t first = p, last = p + 1u;
+            while (first > 0u && hi32(sh.buf[first - 1u]) == key) --first;
+            while (last < n && hi32(sh.buf[last]) == key) ++last;
+            uint32_t smaller = 0;
+            for (uint32_t q = first; q < last; ++q) smaller += lo32(sh.buf[q]) < lo32(v[e]) ? 1u : 0u;
+            at[e] = first + smaller;
         }
         __syncthreads();
-        return cur ^ 1;
+#pragma unroll
+        for (int e = 0; e < kPer; ++e)
+            if (tied[e]) sh.buf[at[e]] = v[e];
+        __syncthreads();
+        return;
     }
     // many ties: sort over all 64 bits, least significant digit first
     for (int shift = 0; shift < 32; shift += 4)
-        if ((vary_lo >> shift) & 15u) {
-            digit_pass<kPer>(sh, cur, shift);
-            cur ^= 1;
-        }
+        if ((vary_lo >> shift) & 15u) digit_pass<kPer>(sh, active, shift);
     key_passes();
-    return cur;
 }
 
-// Loads `n` elements from `src` into sh.buf[0], pads, sorts; returns the buffer holding the result.
-__device__ __forceinline__ int load_and_sort(Shared& sh, const uint64_t* __restrict__ src, uint32_t n, int key_bits) {
+// Loads `n` <= kCap elements from `src` into sh.buf and sorts them there.
+__device__ __forceinline__ void load_and_sort(Shared& sh, const uint64_t* __restrict__ src, uint32_t n, int key_bits) {
     const uint32_t t = threadIdx.x;
-    const uint32_t per = (n + kThreads - 1u) / kThreads;            // 1 .. kMaxPer
-    const uint32_t padded = (per <= 1u ? 1u : per <= 3u ? 3u : per <= 5u ? 5u : 7u) * kThreads;
-    for (uint32_t p = t; p < padded; p += kThreads) sh.buf[0][p] = p < n ? src[p] : kPad;
+    // as few threads as hold the elements with at most kMaxPer each: the per-thread cost of a pass does not
+    // depend on the number of its elements
+    uint32_t active = kWave;
+    while (active < (uint32_t)kThreads && active * kMaxPer < n) active <<= 1;
+    const uint32_t need = (n + active - 1u) / active;
+    const uint32_t per = need <= 3u ? 3u : need <= 7u ? 7u : need <= 11u ? 11u : 15u;
+    for (uint32_t p = t; p < per * active; p += kThreads) sh.buf[p] = p < n ? src[p] : kPad;
     __syncthreads();
-    if (per <= 1u) return sort_run<1>(sh, n, key_bits);
-    if (per <= 3u) return sort_run<3>(sh, n, key_bits);
-    if (per <= 5u) return sort_run<5>(sh, n, key_bits);
-    return sort_run<7>(sh, n, key_bits);
+    if (per == 3u) sort_run<3>(sh, n, active, key_bits);
+    else if (per == 7u) sort_run<7>(sh, n, active, key_bits);
+    else if (per == 11u) sort_run<11>(sh, n, active, key_bits);
+    else sort_run<15>(sh, n, active, key_bits);
 }
 
 // One block per tile, longest bins first. pairs[begin .. end) of a tile are its elements in no particular order;
 // afterwards points[begin .. end) holds their point indices in ascending element order. `pairs` and `scratch`
 // (same size) are clobbered for tiles with more than kCap elements.
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kThreads, 4)   // four waves per SIMD (two blocks per CU): 128 registers
     k_tile_sort(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order, uint64_t* pairs,
                 uint64_t* scratch, uint32_t* __restrict__ points, int key_bits) {
     extern __shared__ __align__(16) unsigned char s_raw[];
@@ -227,22 +239,22 @@ __global__ void __launch_bounds__(kThreads)
     const uint32_t begin = range.x, n = range.y - range.x;
     if (n == 0u) return;
     if (n <= (uint32_t)kCap) {
-        const int res = load_and_sort(sh, pairs + begin, n, key_bits);
-        for (uint32_t p = t; p < n; p += kThreads) points[begin + p] = lo32(sh.buf[res][p]);
+        load_and_sort(sh, pairs + begin, n, key_bits);
+        for (uint32_t p = t; p < n; p += kThreads) points[begin + p] = lo32(sh.buf[p]);
         return;
     }
     // runs of kCap elements, each sorted in LDS and written back in place
     for (uint32_t first = 0; first < n; first += kCap) {
         const uint32_t len = min((uint32_t)kCap, n - first);
-        const int res = load_and_sort(sh, pairs + begin + first, len, key_bits);
-        for (uint32_t p = t; p < len; p += kThreads) pairs[begin + first + p] = sh.buf[res][p];
+        load_and_sort(sh, pairs + begin + first, len, key_bits);
+        for (uint32_t p = t; p < len; p += kThreads) pairs[begin + first + p] = sh.buf[p];
         __syncthreads();
     }
     // pairwise merges; the global stores of a level are visible to the whole block behind the barrier
     uint64_t* from = pairs + begin;
     uint64_t* to = scratch + begin;
     for (uint32_t width = kCap; width < n; width <<= 1) {
-        constexpr int kAhead = 4;   // independent searches per thread
+        constexpr int kAhead = 8;   // independent searches per thread
         for (uint32_t base = 0; base < n; base += kAhead * kThreads) {
             uint64_t v[kAhead];
             uint32_t lo[kAhead], hi[kAhead];   // the part of the partner run still searched
