@@ -187,12 +187,15 @@ __device__ __forceinline__ int candidate_of_parity(int left, uint32_t odd) { ret
 // 16x16 tiles: slot = parity class (x parity | y parity << 1); 8x8 tiles: slot = candidate (kx | ky << 1).
 template <int T>
 __device__ __forceinline__ void slot_weights(const Header& h, int tile_x0, int tile_y0, float (&weight)[4]) {
+    // plain scalars: a choice between two members of the record would otherwise be made through memory
+    const float wx0 = h.wx0, wx1 = h.wx1, wy0 = h.wy0, wy1 = h.wy1;
     const int lx = local_left(h.cell & 0xFFFFu, tile_x0), ly = local_left(h.cell >> 16, tile_y0);
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        const int kx = T == 16 ? candidate_of_parity(lx, c & 1) : (c & 1);
-        const int ky = T == 16 ? candidate_of_parity(ly, c >> 1) : (c >> 1);
-        weight[c] = (kx ? h.wx1 : h.wx0) * (ky ? h.wy1 : h.wy0);
+        const bool kx = (T == 16 ? candidate_of_parity(lx, c & 1) : (c & 1)) != 0;
+        const bool ky = (T == 16 ? candidate_of_parity(ly, c >> 1) : (c >> 1)) != 0;
+        const float wx = kx ? wx1 : wx0, wy = ky ? wy1 : wy0;
+        weight[c] = wx * wy;
     }
 }
 

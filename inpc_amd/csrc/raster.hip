@@ -844,7 +844,7 @@ int launch_blend_forward(const Layout& L, float* image, float* alpha, float* ble
     } else {
         INPC_LAUNCH("raster_blend_forward", (blend::k_blend_forward<T, C, HALF, false>), dim3(L.geo.n_tiles), dim3(T * T),
                     stream, ranges, order, inst, records, L.geo.stride, image, alpha, blending_weights, (float*)nullptr,
-                    L.tile_end ? at<float4>(ws, L.ordered_records) : (float4*)nullptr,
+                    L.ordered_records ? at<float4>(ws, L.ordered_records) : (float4*)nullptr,
                     L.tile_end ? at<uint32_t>(ws, L.tile_end) : (uint32_t*)nullptr, L.geo.W, L.geo.H, L.geo.gw);
     }
     return INPC_OK;
