@@ -1221,10 +1221,17 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
         rc = dispatch_preprocess(L, positions, features, opacities, w2c, cam_position,
                                  L.inference ? nullptr : blending_weights, ws, stream);
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort, dim3(L.geo.n_tiles), dim3(tilesort::kThreads),
-                        tilesort::kSharedBytes, stream, (const uint2*)at<uint2>(ws, L.pub.tile_ranges),
-                        (const uint32_t*)at<uint32_t>(ws, L.tile_order), at<uint64_t>(ws, L.pairs),
-                        at<uint64_t>(ws, L.pairs_scratch), at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
+        // tiles of more than tilesort::kSmallTile instances, then the others with small blocks
+        INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort<tilesort::kLargeThreads>, dim3(L.geo.n_tiles),
+                        dim3(tilesort::kLargeThreads), sizeof(tilesort::Shared<tilesort::kLargeThreads>), stream,
+                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
+                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
+                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
+        INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort<tilesort::kSmallThreads>, dim3(L.geo.n_tiles),
+                        dim3(tilesort::kSmallThreads), sizeof(tilesort::Shared<tilesort::kSmallThreads>), stream,
+                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
+                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
+                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
     }
     return dispatch_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }

@@ -23,22 +23,23 @@
 
 namespace tilesort {
 
-constexpr int kThreads = 512;
-constexpr int kWaves = kThreads / kWave;
 constexpr int kMaxPer = 15;                 // elements per thread: 3, 7, 11 or 15 (odd: conflict-free LDS rows; at
                                             // most 15: a thread's digit counts fit 4-bit fields)
-constexpr int kCap = kThreads * kMaxPer;    // elements sorted in LDS at a time
 constexpr int kDigits = 16;
-constexpr uint64_t kPad = ~0ull;            // sorts behind every element
 constexpr uint32_t kFewTies = 16;           // threads with tied elements up to which ties are fixed in place
+constexpr uint64_t kPad = ~0ull;            // sorts behind every element
+constexpr int kLargeThreads = 512, kSmallThreads = 128;   // block sizes of the two kernels
+constexpr uint32_t kSmallTile = kSmallThreads * kMaxPer;  // tiles up to this size go to the small blocks
 
+// LDS of a block of THREADS threads.
+template <int THREADS>
 struct Shared {
+    static constexpr int kCap = THREADS * kMaxPer;        // elements sorted in LDS at a time
     uint64_t buf[kCap];
-    alignas(16) uint16_t count[kDigits * kThreads];   // [digit][thread], scanned in this order
-    uint32_t wave_sum[kWaves];
-    uint32_t bits_or[2], bits_and[2];                 // over the tile's elements: [0] point index, [1] key
+    alignas(16) uint16_t count[kDigits * THREADS];        // [digit][thread], scanned in this order
+    uint32_t wave_sum[THREADS / kWave];
+    uint32_t bits_or[2], bits_and[2];                     // over the tile's elements: [0] point index, [1] key
 };
-constexpr size_t kSharedBytes = sizeof(Shared);
 
 __device__ __forceinline__ uint32_t hi32(uint64_t v) { return (uint32_t)(v >> 32); }
 __device__ __forceinline__ uint32_t lo32(uint64_t v) { return (uint32_t)v; }
@@ -62,8 +63,8 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t v, int shift) {
 // One stable counting pass, in place, on the 4-bit digit at bit `shift`. The first `active` threads (a multiple
 // of 64) own kPer consecutive elements each; every thread of the block calls it (the others only meet the
 // barriers). All elements are in registers before the first one is stored, so one buffer suffices.
-template <int kPer>
-__device__ __forceinline__ void digit_pass(Shared& sh, uint32_t active, int shift) {
+template <int THREADS, int kPer>
+__device__ __forceinline__ void digit_pass(Shared<THREADS>& sh, uint32_t active, int shift) {
     const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
     const bool on = t < active;
     uint64_t v[kPer];
@@ -94,7 +95,7 @@ __device__ __forceinline__ void digit_pass(Shared& sh, uint32_t active, int shif
     if (on) {
         uint32_t run = incl - sum;
 #pragma unroll
-        for (int k = 0; k < kWaves; ++k) run += (uint32_t)k < wave ? sh.wave_sum[k] : 0u;
+        for (int k = 0; k < THREADS / kWave; ++k) run += (uint32_t)k < wave ? sh.wave_sum[k] : 0u;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t c0 = w[i] & 0xFFFFu, c1 = w[i] >> 16;
@@ -120,8 +121,8 @@ __device__ __forceinline__ void digit_pass(Shared& sh, uint32_t active, int shif
 
 // Sorts the n <= kPer * active elements in sh.buf ascending as u64 (the slots behind them, up to
 // kPer * active, hold kPad). All threads of the block call it.
-template <int kPer>
-__device__ void sort_run(Shared& sh, uint32_t n, uint32_t active, int key_bits) {
+template <int THREADS, int kPer>
+__device__ void sort_run(Shared<THREADS>& sh, uint32_t n, uint32_t active, int key_bits) {
     const uint32_t t = threadIdx.x, lane = t & 63u;
     const bool on = t < active;
     // bits that differ between the elements
@@ -160,7 +161,7 @@ __device__ void sort_run(Shared& sh, uint32_t n, uint32_t active, int key_bits) 
     const uint32_t vary_lo = sh.bits_or[0] ^ sh.bits_and[0], vary_hi = sh.bits_or[1] ^ sh.bits_and[1];
     auto key_passes = [&]() {
         for (int shift = 0; shift < key_bits; shift += 4)
-            if ((vary_hi >> shift) & 15u) digit_pass<kPer>(sh, active, 32 + shift);
+            if ((vary_hi >> shift) & 15u) digit_pass<THREADS, kPer>(sh, active, 32 + shift);
     };
     key_passes();
     // elements with equal keys stand in the order they were binned; the order wanted is by point index
@@ -205,48 +206,53 @@ __device__ void sort_run(Shared& sh, uint32_t n, uint32_t active, int key_bits) 
     }
     // many ties: sort over all 64 bits, least significant digit first
     for (int shift = 0; shift < 32; shift += 4)
-        if ((vary_lo >> shift) & 15u) digit_pass<kPer>(sh, active, shift);
+        if ((vary_lo >> shift) & 15u) digit_pass<THREADS, kPer>(sh, active, shift);
     key_passes();
 }
 
-// Loads `n` <= kCap elements from `src` into sh.buf and sorts them there.
-__device__ __forceinline__ void load_and_sort(Shared& sh, const uint64_t* __restrict__ src, uint32_t n, int key_bits) {
+// Loads `n` <= THREADS * kMaxPer elements from `src` into sh.buf and sorts them there.
+template <int THREADS>
+__device__ __forceinline__ void load_and_sort(Shared<THREADS>& sh, const uint64_t* __restrict__ src, uint32_t n, int key_bits) {
     const uint32_t t = threadIdx.x;
     // as few threads as hold the elements with at most kMaxPer each: the per-thread cost of a pass does not
     // depend on the number of its elements
     uint32_t active = kWave;
-    while (active < (uint32_t)kThreads && active * kMaxPer < n) active <<= 1;
+    while (active < (uint32_t)THREADS && active * kMaxPer < n) active <<= 1;
     const uint32_t need = (n + active - 1u) / active;
     const uint32_t per = need <= 3u ? 3u : need <= 7u ? 7u : need <= 11u ? 11u : 15u;
-    for (uint32_t p = t; p < per * active; p += kThreads) sh.buf[p] = p < n ? src[p] : kPad;
+    for (uint32_t p = t; p < per * active; p += THREADS) sh.buf[p] = p < n ? src[p] : kPad;
     __syncthreads();
-    if (per == 3u) sort_run<3>(sh, n, active, key_bits);
-    else if (per == 7u) sort_run<7>(sh, n, active, key_bits);
-    else if (per == 11u) sort_run<11>(sh, n, active, key_bits);
-    else sort_run<15>(sh, n, active, key_bits);
+    if (per == 3u) sort_run<THREADS, 3>(sh, n, active, key_bits);
+    else if (per == 7u) sort_run<THREADS, 7>(sh, n, active, key_bits);
+    else if (per == 11u) sort_run<THREADS, 11>(sh, n, active, key_bits);
+    else sort_run<THREADS, 15>(sh, n, active, key_bits);
 }
 
 // One block per tile, longest bins first. pairs[begin .. end) of a tile are its elements in no particular order;
 // afterwards points[begin .. end) holds their point indices in ascending element order. `pairs` and `scratch`
-// (same size) are clobbered for tiles with more than kCap elements.
-__global__ void __launch_bounds__(kThreads, 4)   // four waves per SIMD (two blocks per CU): 128 registers
+// (same size) are clobbered for tiles with more than THREADS * kMaxPer elements. Two launches cover the tiles:
+// blocks of kSmallThreads threads take the tiles of at most kSmallTile elements (many blocks per CU), blocks of
+// kLargeThreads threads the others; a block whose tile belongs to the other launch ends at once.
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS, 4)   // four waves per SIMD: 128 registers
     k_tile_sort(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order, uint64_t* pairs,
                 uint64_t* scratch, uint32_t* __restrict__ points, int key_bits) {
     extern __shared__ __align__(16) unsigned char s_raw[];
-    Shared& sh = *reinterpret_cast<Shared*>(s_raw);
+    Shared<THREADS>& sh = *reinterpret_cast<Shared<THREADS>*>(s_raw);
+    constexpr uint32_t kThreads = THREADS, kCap = Shared<THREADS>::kCap;
     const uint32_t t = threadIdx.x;
     const uint2 range = ranges[tile_order[blockIdx.x]];
     const uint32_t begin = range.x, n = range.y - range.x;
-    if (n == 0u) return;
-    if (n <= (uint32_t)kCap) {
-        load_and_sort(sh, pairs + begin, n, key_bits);
+    if (n == 0u || (n <= kSmallTile) != (THREADS == kSmallThreads)) return;
+    if (n <= kCap) {
+        load_and_sort<THREADS>(sh, pairs + begin, n, key_bits);
         for (uint32_t p = t; p < n; p += kThreads) points[begin + p] = lo32(sh.buf[p]);
         return;
     }
     // runs of kCap elements, each sorted in LDS and written back in place
     for (uint32_t first = 0; first < n; first += kCap) {
         const uint32_t len = min((uint32_t)kCap, n - first);
-        load_and_sort(sh, pairs + begin + first, len, key_bits);
+        load_and_sort<THREADS>(sh, pairs + begin + first, len, key_bits);
         for (uint32_t p = t; p < len; p += kThreads) pairs[begin + first + p] = sh.buf[p];
         __syncthreads();
     }
