@@ -119,8 +119,8 @@ struct Stage {
     static constexpr int NQ = TT / 64;
     float4 feat[TT * (C / 4)];
     float depth[WITH_DEPTH ? TT : 1];
-    float4 weights[TT];                 // wx0, wx1, wy0, wy1 of the staged instance
-    float2 place[TT];                   // opacity, (Lx + 1) | (Ly + 1) << 16
+    float4 alpha[T == 16 ? TT : 1];     // per fragment slot of the staged instance: opacity * interpolation weight
+    uint32_t pixel[T == 16 ? TT : 1];   // per slot, one byte: pixel in the owning wave's grid, kNoPixel: no fragment
     alignas(8) uint16_t frag[TT][4];    // per slot: the fragment field, written by the wave that placed the fragment
 };
 
@@ -183,34 +183,47 @@ __device__ __forceinline__ int local_left(uint32_t cell_half, int tile_origin) {
 // The candidate (0: L, 1: L + 1) of one axis whose tile-local index has the parity `odd` (tiles start at even pixels).
 __device__ __forceinline__ int candidate_of_parity(int left, uint32_t odd) { return (left ^ (int)odd) & 1; }
 
-// Interpolation weights of the four fragment slots of a point in a tile (whether the fragment exists or not):
-// 16x16 tiles: slot = parity class (x parity | y parity << 1); 8x8 tiles: slot = candidate (kx | ky << 1).
+// The four fragment slots of a point in a tile. 16x16 tiles: slot = parity class (x parity | y parity << 1) of the
+// candidate pixel, i.e. the wave that owns it; 8x8 tiles: slot = candidate (kx | ky << 1). Per slot: the
+// interpolation weight (whether the fragment exists or not) and the pixel in the owning wave's 8 x 8 grid, kNoPixel
+// when the candidate lies outside the tile or a pixel centre is 1 or more away (B/rasterization/src/bilinear/
+// kernels.cu:284-285: weight 0).
 template <int T>
-__device__ __forceinline__ void slot_weights(const Header& h, int tile_x0, int tile_y0, float (&weight)[4]) {
+__device__ __forceinline__ void fragment_slots(const Header& h, int tile_x0, int tile_y0, float (&weight)[4],
+                                               uint32_t (&pixel)[4]) {
     // plain scalars: a choice between two members of the record would otherwise be made through memory
     const float wx0 = h.wx0, wx1 = h.wx1, wy0 = h.wy0, wy1 = h.wy1;
     const int lx = local_left(h.cell & 0xFFFFu, tile_x0), ly = local_left(h.cell >> 16, tile_y0);
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        const bool kx = (T == 16 ? candidate_of_parity(lx, c & 1) : (c & 1)) != 0;
-        const bool ky = (T == 16 ? candidate_of_parity(ly, c >> 1) : (c >> 1)) != 0;
+        const int kx = T == 16 ? candidate_of_parity(lx, c & 1) : (c & 1);
+        const int ky = T == 16 ? candidate_of_parity(ly, c >> 1) : (c >> 1);
+        const int cx = lx + kx, cy = ly + ky;
         const float wx = kx ? wx1 : wx0, wy = ky ? wy1 : wy0;
         weight[c] = wx * wy;
+        const bool hit = (uint32_t)(cx | cy) < (uint32_t)T && weight[c] > 0.0f;
+        const uint32_t pix = T == 16 ? (uint32_t)((cy >> 1) * 8 + (cx >> 1)) : (uint32_t)(cy * 8 + cx);
+        pixel[c] = hit ? (pix & kPixelMask) : kNoPixel;
     }
 }
 
-// Stage instance `t` (thread t). `valid` is false for the threads behind the end of the batch. Must be followed
-// by a block barrier.
+// Stage instance `t` (thread t): features, and per fragment slot the blend's alpha and the pixel, so that the waves
+// only look their fragments up. `weight` receives the slots' interpolation weights (for the write phase of the same
+// thread). `valid` is false for the threads behind the end of the batch. Must be followed by a block barrier.
 template <int T, int C, bool WITH_DEPTH>
 __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool valid, const Header& h,
-                                               const float (&f)[C]) {
+                                               const float (&f)[C], int tile_x0, int tile_y0, float (&weight)[4],
+                                               uint32_t (&pixel)[4]) {
     const uint32_t t = threadIdx.x;
+    fragment_slots<T>(h, tile_x0, tile_y0, weight, pixel);
     if (!valid) return;
 #pragma unroll
     for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
     if (WITH_DEPTH) st.depth[t] = __uint_as_float(h.extra);
-    st.weights[t] = make_float4(h.wx0, h.wx1, h.wy0, h.wy1);
-    st.place[t] = make_float2(h.opacity, __uint_as_float(h.cell));
+    if (T == 16) {   // 8x8 tiles: the staging thread's wave is the only consumer and takes them from its registers
+        st.alpha[t] = make_float4(h.opacity * weight[0], h.opacity * weight[1], h.opacity * weight[2], h.opacity * weight[3]);
+        st.pixel[t] = pixel[0] | (pixel[1] << 8) | (pixel[2] << 16) | (pixel[3] << 24);
+    }
     const uint2 nothing_placed = make_uint2(0u, 0u);
     __builtin_memcpy(st.frag[t], &nothing_placed, 8);
 }
@@ -225,46 +238,35 @@ struct Entries {
     float alpha[K][NF];
 };
 
-// `count`: staged instances of the batch; `finished`: this wave's pixels that are done.
+// `count`: staged instances of the batch; `finished`: this wave's pixels that are done. 16x16 tiles: the wave looks
+// up slot `quad` of all staged instances; 8x8 tiles: lane l staged instance l itself and passes its slots
+// (`opacity`, `weight`, `pixel`).
 template <int T, int C, bool WITH_DEPTH>
 __device__ __forceinline__ void load_entries(const Stage<T, C, WITH_DEPTH>& st, uint32_t count, uint32_t quad,
-                                             int tile_x0, int tile_y0, uint64_t finished, Entries<T>& e) {
+                                             uint64_t finished, float opacity, const float (&weight)[4],
+                                             const uint32_t (&pixel)[4], Entries<T>& e) {
     constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
     const uint32_t lane = __lane_id();
+    if (T == 16) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const uint32_t j = k * 64u + lane;
-        const bool live = j < count;
-        e.j[k] = j;
-        const float4 w4 = st.weights[live ? j : 0u];
-        const float2 place = st.place[live ? j : 0u];
-        const uint32_t cell = __float_as_uint(place.y);
-        const int lx = local_left(cell & 0xFFFFu, tile_x0), ly = local_left(cell >> 16, tile_y0);
-        bool hit[NF];
-        uint32_t pix[NF];
-        float weight[NF];
-        if (T == 16) {
-            // the fragment of this wave's parity class (x parity = quad & 1, y parity = quad >> 1)
-            const int kx = candidate_of_parity(lx, quad & 1u), ky = candidate_of_parity(ly, quad >> 1);
-            const int cx = lx + kx, cy = ly + ky;
-            weight[0] = (kx ? w4.y : w4.x) * (ky ? w4.w : w4.z);
-            hit[0] = (uint32_t)(cx | cy) < (uint32_t)T && weight[0] > 0.0f;   // inside the tile, closer than 1 in x and y
-            pix[0] = (uint32_t)((cy >> 1) * 8 + (cx >> 1));
-        } else {
-#pragma unroll
-            for (int q = 0; q < NF; ++q) {
-                const int ky = q >> 1, kx = q & 1;
-                const int cx = lx + kx, cy = ly + ky;
-                weight[q] = (kx ? w4.y : w4.x) * (ky ? w4.w : w4.z);
-                hit[q] = (uint32_t)(cx | cy) < (uint32_t)T && weight[q] > 0.0f;
-                pix[q] = (uint32_t)(cy * 8 + cx);
-            }
+        for (int k = 0; k < K; ++k) {
+            const uint32_t j = k * 64u + lane;
+            const bool live = j < count;
+            e.j[k] = j;
+            const uint32_t at = live ? j : 0u;
+            const uint32_t pix = ((const uint8_t*)&st.pixel[at])[quad];
+            const bool open = live && pix != kNoPixel && ((finished >> (pix & kPixelMask)) & 1ull) == 0ull;
+            e.pixel[k][0] = open ? pix : kNoPixel;
+            e.alpha[k][0] = ((const float*)&st.alpha[at])[quad];
         }
+    } else {
+        const bool live = lane < count;
+        e.j[0] = lane;
 #pragma unroll
         for (int q = 0; q < NF; ++q) {
-            const bool open = live && hit[q] && ((finished >> (pix[q] & kPixelMask)) & 1ull) == 0ull;
-            e.pixel[k][q] = open ? pix[q] : kNoPixel;
-            e.alpha[k][q] = place.x * weight[q];
+            const bool open = live && pixel[q] != kNoPixel && ((finished >> (pixel[q] & kPixelMask)) & 1ull) == 0ull;
+            e.pixel[0][q] = open ? pixel[q] : kNoPixel;
+            e.alpha[0][q] = opacity * weight[q];
         }
     }
 }
@@ -484,14 +486,16 @@ __global__ void __launch_bounds__(T* T)
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
         staged_end = begin + count;
-        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f);
+        float weight[4];   // of this thread's staged instance, per fragment slot
+        uint32_t slot_pixel[4];
+        stage_instance<T, C, INFERENCE>(st, valid, g.h, g.f, tile_x0, tile_y0, weight, slot_pixel);
         __syncthreads();
 
         // ---- consume: this wave's list
         uint32_t my_start = 0, my_count = 0, n_fragments = 0;
         {
             Entries<T> e;
-            load_entries<T, C, INFERENCE>(st, count, wave, tile_x0, tile_y0, __ballot(done), e);
+            load_entries<T, C, INFERENCE>(st, count, wave, __ballot(done), g.h.opacity, weight, slot_pixel, e);
             build_fragment_lists<T, C, INFERENCE>(qs, st, wave, e, my_start, my_count, n_fragments,
                                                   [&](int k, int) { return __uint_as_float(e.j[k]); });
         }
@@ -587,8 +591,6 @@ __global__ void __launch_bounds__(T* T)
         if (!INFERENCE && valid) {
             uint32_t field[4];
             load_fields<T, C, INFERENCE>(st, tid, field);
-            float weight[4];
-            slot_weights<T>(mine, tile_x0, tile_y0, weight);
             float w = 0.0f;
 #pragma unroll
             for (int c = 0; c < 4; ++c)
@@ -741,14 +743,16 @@ __global__ void __launch_bounds__(T* T)
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
-        stage_instance<T, C, false>(st, valid, g.h, g.f);
+        float weight[4];   // of this thread's staged instance, per fragment slot
+        uint32_t slot_pixel[4];
+        stage_instance<T, C, false>(st, valid, g.h, g.f, tile_x0, tile_y0, weight, slot_pixel);
         __syncthreads();
 
         // ---- consume: this wave's list
         uint32_t my_start = 0, my_count = 0, n_fragments = 0;
         {
             Entries<T> e;
-            load_entries<T, C, false>(st, count, wave, tile_x0, tile_y0, __ballot(done), e);
+            load_entries<T, C, false>(st, count, wave, __ballot(done), g.h.opacity, weight, slot_pixel, e);
             float dots[K][NF];   // features . grad of the fragment's pixel
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -836,8 +840,6 @@ __global__ void __launch_bounds__(T* T)
         if (valid) {
             uint32_t field[4];
             load_fields<T, C, false>(st, tid, field);
-            float weight[4];
-            slot_weights<T>(mine, tile_x0, tile_y0, weight);
             float gf[C];
 #pragma unroll
             for (int c = 0; c < C; ++c) gf[c] = 0.0f;
