@@ -80,6 +80,7 @@ struct Geometry {
     uint32_t capacity;      // instances the buffers hold
     uint32_t row_capacity;  // gradient rows (instances of points that touch several tiles)
     uint32_t tile_shift;    // log2 of the tile size
+    uint32_t n_chunks;      // contiguous chunks the points are cut into for binning (one block each)
 };
 
 // ---- SH degree 2 (sh_utils.cuh:6-23) ---------------------------------------------------------------------
@@ -202,13 +203,25 @@ __device__ __forceinline__ AxisWeights axis_weights(float s) {
 // into the start of every tile's bin. k_preprocess then hands out bin slots from LDS cursors seeded with
 // bin_start[tile] + prefix[chunk][tile]: no global atomic anywhere (they run at about 10 G/s on this machine,
 // far below what 8M points need).
-constexpr int kBinBlocks = 512;
-constexpr int kBinThreads = 512;
-constexpr uint32_t kMaxLdsTiles = 16384;  // tiles whose counters a block keeps as 32-bit words in LDS (64 KiB)
+//
+// Up to kMaxLdsTiles tiles a block keeps its per-tile counters / cursors as 32-bit words in LDS. Beyond that (the
+// reference's 8x8 tiles on large images, up to the 65536 tiles of its 16-bit tile key, kernels.cu:204,214) they are
+// 16-bit halves of LDS words counting within the chunk, which a chunk of at most kWideChunk points cannot
+// overflow, and a cursor's base comes from the table in memory (the WIDE variants of the two kernels).
+constexpr int kBinBlocks = 512, kBinBlocksWide = 1024;   // chunks: normally; for many tiles and many points
+constexpr int kBinThreads = 512, kBinThreadsWide = 256;   // the WIDE kernels leave the LDS to the counters
+constexpr uint32_t kMaxLdsTiles = 16384;  // 64 KiB of 32-bit counters
+constexpr uint32_t kWideChunk = 65024;    // points per chunk with 16-bit counters (a multiple of kBinThreads)
 
-__host__ __device__ inline uint32_t bin_chunk_size(uint32_t n) {
-    const uint32_t per = (n + kBinBlocks - 1) / kBinBlocks;
+__host__ __device__ inline uint32_t bin_chunk_size(uint32_t n, uint32_t n_chunks) {
+    const uint32_t per = (n + n_chunks - 1) / n_chunks;
     return (per + kBinThreads - 1) / kBinThreads * kBinThreads;
+}
+
+// 16-bit counters, two per LDS word: add one to the counter of `tile`, return its value before.
+__device__ __forceinline__ uint32_t packed_counter_next(uint32_t* counters, uint32_t tile) {
+    const uint32_t shift = (tile & 1u) * 16u;
+    return (atomicAdd(&counters[tile >> 1], 1u << shift) >> shift) & 0xFFFFu;
 }
 
 // For every touched tile of a projected point, in the row-major order of the reference's create_instances_cu
@@ -224,25 +237,27 @@ __device__ __forceinline__ void for_each_tile(uint32_t info, uint32_t gw, F f) {
     }
 }
 
-template <int T>
-__global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restrict__ positions,
+template <int T, bool WIDE>
+__global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads) k_bin_count(const float* __restrict__ positions,
                                                            const float* __restrict__ w2c, uint32_t* __restrict__ table,
                                                            uint2* __restrict__ split_count, Geometry g) {
+    constexpr int kThreads = WIDE ? kBinThreadsWide : kBinThreads;
     extern __shared__ uint32_t s_count[];
     __shared__ uint32_t s_split, s_rows;   // the chunk's points that touch several tiles, and their instances
-    for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_count[t] = 0u;
+    const uint32_t n_words = WIDE ? (g.n_tiles + 1u) / 2u : g.n_tiles;
+    for (uint32_t t = threadIdx.x; t < n_words; t += kThreads) s_count[t] = 0u;
     if (threadIdx.x == 0) s_split = s_rows = 0u;
     __syncthreads();
     uint32_t my_split = 0, my_rows = 0;
     const ViewRows m = load_view_rows(w2c);
-    const uint32_t chunk = bin_chunk_size(g.n);
+    const uint32_t chunk = bin_chunk_size(g.n, g.n_chunks);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
     constexpr int kUnroll = 4;   // points per thread and round, their loads issued together
-    for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
+    for (uint32_t base = begin; base < end; base += kUnroll * kThreads) {
         float px[kUnroll], py[kUnroll], pz[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const uint32_t at = base + u * kBinThreads + threadIdx.x;
+            const uint32_t at = base + u * kThreads + threadIdx.x;
             const size_t i = at < end ? at : begin;
             px[u] = positions[3 * i];
             py[u] = positions[3 * i + 1];
@@ -250,9 +265,13 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            if (base + u * kBinThreads + threadIdx.x >= end) continue;
+            if (base + u * kThreads + threadIdx.x >= end) continue;
             const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
-            if (p.info) for_each_tile(p.info, g.gw, [&](uint32_t tile) { atomicAdd(&s_count[tile], 1u); });
+            if (p.info)
+                for_each_tile(p.info, g.gw, [&](uint32_t tile) {
+                    if (WIDE) packed_counter_next(s_count, tile);
+                    else atomicAdd(&s_count[tile], 1u);
+                });
             if (p.touched > 1u) {
                 my_split += 1u;
                 my_rows += p.touched;
@@ -269,7 +288,8 @@ __global__ void __launch_bounds__(kBinThreads) k_bin_count(const float* __restri
     }
     __syncthreads();
     uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
-    for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) row[t] = s_count[t];
+    for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kThreads)
+        row[t] = WIDE ? (s_count[t >> 1] >> ((t & 1u) * 16u)) & 0xFFFFu : s_count[t];
     if (threadIdx.x == 0) split_count[blockIdx.x] = make_uint2(s_split, s_rows);
 }
 
@@ -318,18 +338,18 @@ __global__ void __launch_bounds__(kOffsetWaves * kWave) k_bin_offsets(uint32_t* 
 // When the instances or the gradient rows exceed the buffers, every bin is left empty and the overflow counter set:
 // the later kernels then draw nothing.
 constexpr int kScanBlock = 1024;
-static_assert(kBinBlocks <= kScanBlock, "one thread per chunk in k_bin_scan");
+static_assert(kBinBlocksWide <= kScanBlock, "one thread per chunk in k_bin_scan");
 __global__ void __launch_bounds__(kScanBlock)
     k_bin_scan(const uint32_t* __restrict__ bin_count, uint32_t* __restrict__ bin_start, uint2* __restrict__ ranges,
                const uint2* __restrict__ split_count, uint2* __restrict__ split_base, uint32_t* __restrict__ counters,
-               uint32_t n_tiles, uint32_t capacity, uint32_t row_capacity) {
+               uint32_t n_tiles, uint32_t n_chunks, uint32_t capacity, uint32_t row_capacity) {
     __shared__ uint32_t s_wave[3][kScanBlock / kWave];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t per = (n_tiles + kScanBlock - 1) / kScanBlock;
     const uint32_t begin = min(tid * per, n_tiles), end = min(begin + per, n_tiles);
     uint32_t mine[3] = {0u, 0u, 0u};
     for (uint32_t t = begin; t < end; ++t) mine[0] += bin_count[t];
-    if (tid < (uint32_t)kBinBlocks) {
+    if (tid < n_chunks) {
         const uint2 c = split_count[tid];
         mine[1] = c.x;
         mine[2] = c.y;
@@ -361,13 +381,13 @@ __global__ void __launch_bounds__(kScanBlock)
         ranges[t] = c ? make_uint2(run[0], run[0] + c) : make_uint2(0u, 0u);
         run[0] += c;
     }
-    if (tid < (uint32_t)kBinBlocks) split_base[tid] = make_uint2(run[1], run[2]);
+    if (tid < n_chunks) split_base[tid] = make_uint2(run[1], run[2]);
     if (tid == 0) {
         bin_start[n_tiles] = overflow ? 0u : total[0];
         counters[kCntVisible] = 0u;   // counted by k_preprocess
         counters[kCntError] = 0u;
         counters[kCntInstances] = total[0];
-        counters[kCntSplit] = total[1];
+        counters[kCntSplit] = overflow ? 0u : total[1];   // no list entry is written when nothing is drawn
         counters[kCntRows] = total[2];
         counters[kCntOverflow] = overflow ? 1u : 0u;
     }
@@ -381,7 +401,7 @@ struct PreprocessShape {
     static constexpr bool kDirect = FMODE == INPC_FEAT_DIRECT_F32 || kHalf;
     static constexpr uint32_t kBytes = kRecordHeader + (kDirect ? C * (kHalf ? 2 : 4) : 16);
     static constexpr uint32_t kStrideWords = (kBytes + 31u) / 32u * 2u;
-    static constexpr size_t kStageBytes = (size_t)kBinThreads * (kStrideWords + 1) * 16;   // padded rows, per block
+    static constexpr size_t stage_bytes(int threads) { return (size_t)threads * (kStrideWords + 1) * 16; }   // padded rows
 };
 
 // What a training configuration keeps of the points that touch several tiles: a list entry
@@ -392,24 +412,32 @@ struct SplitOut {
     uint8_t* row_flags;
 };
 
-template <int T, int FMODE, int C>
-__global__ void __launch_bounds__(kBinThreads)
+template <int T, int FMODE, int C, bool WIDE>
+__global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
     k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
                  const float* __restrict__ opacities, const float* __restrict__ w2c,
                  const float* __restrict__ cam_position, char* __restrict__ records,
                  const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start,
                  uint64_t* __restrict__ pairs, float* __restrict__ blending_weights, SplitOut split,
                  float4* __restrict__ debug_geometry, uint32_t* counters, Geometry g) {
+    constexpr int kThreads = WIDE ? kBinThreadsWide : kBinThreads;
     extern __shared__ __align__(16) uint32_t s_dyn[];
     float4* s_stage = (float4*)s_dyn;                                           // record staging, 64 rows per wave
-    uint32_t* s_cursor = s_dyn + PreprocessShape<FMODE, C>::kStageBytes / 4;     // n_tiles
+    uint32_t* s_cursor = s_dyn + PreprocessShape<FMODE, C>::stage_bytes(kThreads) / 4;   // n_tiles (WIDE: 16-bit halves)
     __shared__ uint32_t s_visible;
     __shared__ uint32_t s_split, s_rows;   // next list entry / gradient row for a point of this chunk
     const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then no instance is stored
-    {
-        const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;
-        for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kBinThreads) s_cursor[t] = bin_start[t] + row[t];
+    const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;   // instances of the chunks before, per tile
+    if (WIDE) {
+        for (uint32_t t = threadIdx.x; t < (g.n_tiles + 1u) / 2u; t += kThreads) s_cursor[t] = 0u;
+    } else {
+        for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kThreads) s_cursor[t] = bin_start[t] + row[t];
     }
+    // next bin slot of `tile`
+    auto take_slot = [&](uint32_t tile) -> uint32_t {
+        if (WIDE) return bin_start[tile] + row[tile] + packed_counter_next(s_cursor, tile);
+        return atomicAdd(&s_cursor[tile], 1u);
+    };
     if (threadIdx.x == 0) {
         s_visible = 0u;
         const uint2 first = split.base ? split.base[blockIdx.x] : make_uint2(0u, 0u);
@@ -419,7 +447,7 @@ __global__ void __launch_bounds__(kBinThreads)
     __syncthreads();
     const ViewRows m = load_view_rows(w2c);
     uint32_t my_visible = 0;
-    const uint32_t chunk = bin_chunk_size(g.n);
+    const uint32_t chunk = bin_chunk_size(g.n, g.n_chunks);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
     // kUnroll points per thread and round, their loads issued together. A record leaves the block through LDS:
     // every lane assembles its record in the wave's staging rows, then neighbouring lanes write the 16-byte
@@ -433,13 +461,13 @@ __global__ void __launch_bounds__(kBinThreads)
     constexpr uint32_t kStrideWords = PreprocessShape<FMODE, C>::kStrideWords, kRow = kStrideWords + 1;  // padded row
     const uint32_t lane = threadIdx.x & 63u;
     float4* stage = s_stage + (threadIdx.x >> 6) * (64u * kRow);
-    for (uint32_t base = begin; base < end; base += kUnroll * kBinThreads) {
+    for (uint32_t base = begin; base < end; base += kUnroll * kThreads) {
         float px[kUnroll], py[kUnroll], pz[kUnroll], op[kUnroll];
         uint32_t fw[kUnroll][kWords * kPer];   // plain registers (an array of vector types ends up in scratch memory)
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             // a thread behind the end reads the chunk's first point and drops it
-            const uint32_t at = base + u * kBinThreads + threadIdx.x;
+            const uint32_t at = base + u * kThreads + threadIdx.x;
             const size_t i = at < end ? at : begin;
             px[u] = positions[3 * i];
             py[u] = positions[3 * i + 1];
@@ -461,7 +489,7 @@ __global__ void __launch_bounds__(kBinThreads)
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            const uint32_t i = base + u * kBinThreads + threadIdx.x;
+            const uint32_t i = base + u * kThreads + threadIdx.x;
             bool drawn = false;
             if (i < end) {
                 const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
@@ -469,7 +497,7 @@ __global__ void __launch_bounds__(kBinThreads)
                 if (drawn) {
                     my_visible += 1u;
                     const uint64_t pair = ((uint64_t)(__float_as_uint(p.depth) - g.key_bias) << 32) | (uint64_t)i;
-                    if (!overflow) for_each_tile(p.info, g.gw, [&](uint32_t tile) { pairs[atomicAdd(&s_cursor[tile], 1u)] = pair; });
+                    if (!overflow) for_each_tile(p.info, g.gw, [&](uint32_t tile) { pairs[take_slot(tile)] = pair; });
                     float4* rec = stage + lane * kRow;
                     float opacity = op[u];
 #pragma unroll
@@ -519,7 +547,7 @@ __global__ void __launch_bounds__(kBinThreads)
             }
             wave_sync();
             // the wave's 64 points are consecutive: their records are one contiguous stretch
-            const uint32_t wave_first = base + u * kBinThreads + (threadIdx.x & ~63u);
+            const uint32_t wave_first = base + u * kThreads + (threadIdx.x & ~63u);
             const uint64_t drawn_lanes = __ballot(drawn);
             float4* out = (float4*)(records + (size_t)wave_first * g.stride);
 #pragma unroll
@@ -662,6 +690,7 @@ struct Layout {
     Geometry geo;
     int T, C, fmode, key_bits;
     bool inference, sh, half_features;
+    bool wide;   // more tiles than a block keeps 32-bit counters for: the WIDE binning kernels
     // private offsets
     size_t bin_table, bin_total, tile_order, split_count, split_base;
     size_t pairs, pairs_scratch;
@@ -708,9 +737,12 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
         return fail(INPC_E_UNSUPPORTED, "raster: images beyond 65000 pixels per side are not supported");
     if (g.n_tiles > 65536u)
         return fail(INPC_E_UNSUPPORTED, "raster: %u tiles exceed the 16-bit tile key (65536)", g.n_tiles);
-    if (g.n_tiles > kMaxLdsTiles)
-        return fail(INPC_E_UNSUPPORTED, "raster: %u tiles exceed the %u this build keeps counters for", g.n_tiles,
-                    kMaxLdsTiles);
+    L.wide = g.n_tiles > kMaxLdsTiles;
+    g.n_chunks = kBinBlocks;
+    if (L.wide && bin_chunk_size(g.n, kBinBlocks) > kWideChunk) g.n_chunks = kBinBlocksWide;
+    if (L.wide && bin_chunk_size(g.n, g.n_chunks) > kWideChunk)
+        return fail(INPC_E_UNSUPPORTED, "raster: more than %u points with more than %u tiles are not supported",
+                    kBinBlocksWide * kWideChunk, kMaxLdsTiles);
     g.cam = to_device_camera(cam);
     g.stride = record_stride(L.C, L.half_features);
     // depth keys of drawn points lie in [bits(near), bits(far)] when 0 < near <= far: sort on the offset
@@ -750,12 +782,12 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     memset(&P, 0, sizeof(P));
     P.counters = take(kCntWords * 4);
     P.tile_ranges = take((size_t)g.n_tiles * 8);
-    L.bin_table = take((size_t)kBinBlocks * g.n_tiles * 4);
+    L.bin_table = take((size_t)g.n_chunks * g.n_tiles * 4);
     L.bin_total = take((size_t)g.n_tiles * 4);
     L.tile_order = take((size_t)g.n_tiles * 4);
     P.bin_start = take((size_t)(g.n_tiles + 1) * 4);
-    L.split_count = take(kBinBlocks * 8);
-    L.split_base = take(kBinBlocks * 8);
+    L.split_count = take(kBinBlocksWide * 8);
+    L.split_base = take(kBinBlocksWide * 8);
     P.point_record = take(n * g.stride);
     L.pairs = take(capacity * 8);
     P.instance_points = take(capacity * 4);
@@ -806,9 +838,15 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
 
 template <int T>
 int launch_bin_count(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
-    const size_t lds = (size_t)L.geo.n_tiles * 4;
-    INPC_LAUNCH_LDS("raster_bin_count", (k_bin_count<T>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream, positions,
-                    w2c, at<uint32_t>(ws, L.bin_table), at<uint2>(ws, L.split_count), L.geo);
+    if (L.wide) {
+        const size_t lds = (size_t)(L.geo.n_tiles + 1) / 2 * 4;
+        INPC_LAUNCH_LDS("raster_bin_count", (k_bin_count<T, true>), dim3(L.geo.n_chunks), dim3(kBinThreadsWide), lds, stream,
+                        positions, w2c, at<uint32_t>(ws, L.bin_table), at<uint2>(ws, L.split_count), L.geo);
+    } else {
+        const size_t lds = (size_t)L.geo.n_tiles * 4;
+        INPC_LAUNCH_LDS("raster_bin_count", (k_bin_count<T, false>), dim3(L.geo.n_chunks), dim3(kBinThreads), lds, stream,
+                        positions, w2c, at<uint32_t>(ws, L.bin_table), at<uint2>(ws, L.split_count), L.geo);
+    }
     return INPC_OK;
 }
 
@@ -816,17 +854,25 @@ template <int T, int FMODE, int C>
 int launch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
                       const float* w2c, const float* cam_position, float* blending_weights, void* ws,
                       hipStream_t stream) {
-    const size_t lds = PreprocessShape<FMODE, C>::kStageBytes + (size_t)L.geo.n_tiles * 4;
     if (L.pub.record_stride != PreprocessShape<FMODE, C>::kStrideWords * 16u)
         return fail(INPC_E_UNSUPPORTED, "record stride %u does not match the preprocess kernel", L.pub.record_stride);
     SplitOut split{nullptr, nullptr, nullptr};
     if (L.split_list) split = SplitOut{at<uint2>(ws, L.split_base), at<uint2>(ws, L.split_list), at<uint8_t>(ws, L.row_flags)};
-    INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C>), dim3(kBinBlocks), dim3(kBinThreads), lds, stream,
-                    positions, features, opacities, w2c, cam_position, at<char>(ws, L.pub.point_record),
-                    (const uint32_t*)at<uint32_t>(ws, L.bin_table), (const uint32_t*)at<uint32_t>(ws, L.pub.bin_start),
-                    at<uint64_t>(ws, L.pairs), blending_weights, split,
-                    L.pub.debug_geometry ? at<float4>(ws, L.pub.debug_geometry) : (float4*)nullptr,
-                    at<uint32_t>(ws, L.pub.counters), L.geo);
+    char* records = at<char>(ws, L.pub.point_record);
+    const uint32_t* table = at<uint32_t>(ws, L.bin_table);
+    const uint32_t* bin_start = at<uint32_t>(ws, L.pub.bin_start);
+    float4* debug = L.pub.debug_geometry ? at<float4>(ws, L.pub.debug_geometry) : (float4*)nullptr;
+    if (L.wide) {
+        const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kBinThreadsWide) + (size_t)(L.geo.n_tiles + 1) / 2 * 4;
+        INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C, true>), dim3(L.geo.n_chunks), dim3(kBinThreadsWide),
+                        lds, stream, positions, features, opacities, w2c, cam_position, records, table, bin_start,
+                        at<uint64_t>(ws, L.pairs), blending_weights, split, debug, at<uint32_t>(ws, L.pub.counters), L.geo);
+    } else {
+        const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kBinThreads) + (size_t)L.geo.n_tiles * 4;
+        INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C, false>), dim3(L.geo.n_chunks), dim3(kBinThreads),
+                        lds, stream, positions, features, opacities, w2c, cam_position, records, table, bin_start,
+                        at<uint64_t>(ws, L.pairs), blending_weights, split, debug, at<uint32_t>(ws, L.pub.counters), L.geo);
+    }
     return INPC_OK;
 }
 
@@ -1203,18 +1249,25 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
     if (L.geo.n > 0) {
         rc = L.T == 8 ? launch_bin_count<8>(L, positions, w2c, ws, stream) : launch_bin_count<16>(L, positions, w2c, ws, stream);
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<kBinBlocks>, dim3(div_up(L.geo.n_tiles, kWave)), dim3(kOffsetWaves * kWave), stream,
-                    at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
+        if (L.geo.n_chunks == (uint32_t)kBinBlocks) {
+            INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<kBinBlocks>, dim3(div_up(L.geo.n_tiles, kWave)),
+                        dim3(kOffsetWaves * kWave), stream, at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total),
+                        L.geo.n_tiles);
+        } else {
+            INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<kBinBlocksWide>, dim3(div_up(L.geo.n_tiles, kWave)),
+                        dim3(kOffsetWaves * kWave), stream, at<uint32_t>(ws, L.bin_table), at<uint32_t>(ws, L.bin_total),
+                        L.geo.n_tiles);
+        }
     } else {
         rc = fill_u32(at<uint32_t>(ws, L.bin_total), 0u, L.geo.n_tiles, stream);
         if (rc != INPC_OK) return rc;
-        rc = fill_u32(at<uint32_t>(ws, L.split_count), 0u, 2 * kBinBlocks, stream);
+        rc = fill_u32(at<uint32_t>(ws, L.split_count), 0u, 2 * kBinBlocksWide, stream);
         if (rc != INPC_OK) return rc;
     }
     INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
                 (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start),
                 at<uint2>(ws, L.pub.tile_ranges), (const uint2*)at<uint2>(ws, L.split_count),
-                at<uint2>(ws, L.split_base), counters, L.geo.n_tiles, L.geo.capacity, L.geo.row_capacity);
+                at<uint2>(ws, L.split_base), counters, L.geo.n_tiles, L.geo.n_chunks, L.geo.capacity, L.geo.row_capacity);
     INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
                 (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
     if (L.geo.n > 0) {

@@ -224,10 +224,92 @@ def test_edge_cases(gpu, oracle, tile):
 
 
 def test_too_many_tiles_is_rejected(gpu):
-    hv = synthetic.camera_on_z(8 * 300, 8 * 300, 500.0, 3.0)
+    # 65,536 tiles are the reference's limit (16-bit tile key, kernels.cu:204,214); one more is refused
+    hv = synthetic.camera_on_z(8 * 257, 8 * 256, 500.0, 3.0)
     with pytest.raises(_lib.BackendError, match="16-bit tile key"):
         H.RasterRun(hv, np.zeros((4, 3), np.float32), np.zeros((4, 4), np.float32), np.ones(4, np.float32), 8, 4,
                     _lib.FEAT_DIRECT_F32)
+    hv = synthetic.camera_on_z(8 * 256, 8 * 256, 500.0, 3.0)   # exactly 65,536
+    run = H.RasterRun(hv, np.zeros((4, 3), np.float32), np.zeros((4, 4), np.float32), np.ones(4, np.float32), 8, 4,
+                      _lib.FEAT_DIRECT_F32)
+    assert run.layout.n_tiles == 65536
+
+
+@pytest.mark.parametrize("width,height,focal", [(1920, 1080, 1500.0), (2473, 1643, 2000.0)],
+                         ids=["1920x1080", "2473x1643"])
+def test_reference_tile_size_on_large_images(gpu, oracle, width, height, focal):
+    # the reference's 8x8 tiles on images of more than 16,384 tiles (32,400 and 63,860): per-tile counters as 16-bit
+    # halves in LDS; structure bit-exact, images and gradients to tolerance
+    n, channels = 300000, 4
+    hv = synthetic.camera_on_z(width, height, focal, 2.6)
+    pos = synthetic.cube_points(n, 2.4, 71)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", 72)
+    run = H.RasterRun(hv, pos, feats, opac, 8, channels, _lib.FEAT_DIRECT_F32).forward()
+    assert run.layout.n_tiles > 16384
+    cfg = oracle_cfg(oracle, hv, n, 8, channels, oracle.FEAT_DIRECT_F32)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    dbg = run.debug()
+    assert dbg["n_visible"] > 0.5 * n
+    check_structure(dbg, ref)
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+    rng = np.random.default_rng(73)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
+    H.assert_close(gf, gf_ref, RTOL, 1e-7, "feature gradients")
+    H.assert_close(go, go_ref, RTOL, 2e-7, "opacity gradients")
+
+
+def test_instances_beyond_the_capacity_are_reported_and_nothing_is_drawn(gpu, oracle):
+    # every point on a tile corner: four instances per point, more than a capacity of 2 N holds
+    n, tile = 5000, 16
+    hv = synthetic.camera_on_z(320, 240, 300.0, 3.0)
+    c = hv.camera
+    rng = np.random.default_rng(5)
+    z = rng.uniform(0.5, 2.0, n).astype(np.float32)
+    gx, gy = rng.integers(1, 320 // tile, n), rng.integers(1, 240 // tile, n)
+    wx = ((gx * tile - c.center_x) / c.focal_x * (z + 3.0)).astype(np.float32)
+    wy = ((gy * tile - c.center_y) / c.focal_y * (z + 3.0)).astype(np.float32)
+    pos = np.stack([wx, wy, z], 1)
+    feats, opac = synthetic.point_attributes(n, 4, "normal", 6)
+    cfg = oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_DIRECT_F32)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    assert ref["n_instances"] > 3 * n
+    small = H.RasterRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_DIRECT_F32, max_instances=2 * n).forward()
+    assert small.layout.max_instances == 2 * n
+    with pytest.raises(_lib.BackendError, match="do not fit max_instances"):
+        small.counters()
+    out = small.outputs()
+    assert (out["image"] == 0).all() and (out["alpha"] == 0).all() and (out["blending_weights"] == 0).all()
+    gf, go = small.backward(np.ones_like(ref["image"]), np.ones_like(ref["alpha"]))
+    assert (gf == 0).all() and (go == 0).all()
+    # the same workspace size is enough for a call that fits, and a capacity of 4 N always is
+    run = H.RasterRun(hv, pos, feats, opac, tile, 4, _lib.FEAT_DIRECT_F32).forward()
+    check_structure(run.debug(), ref)
+    H.assert_close(run.outputs()["image"], ref["image"], RTOL, 1e-5, "image")
+
+
+def test_operator_layer_grows_the_workspace_when_the_default_capacity_is_exceeded(gpu, oracle, monkeypatch):
+    from inpc_amd import rasterization, rasterize_points
+
+    n, tile = 5000, 16
+    hv = synthetic.camera_on_z(320, 240, 300.0, 3.0)
+    c = hv.camera
+    rng = np.random.default_rng(8)
+    z = rng.uniform(0.5, 2.0, n).astype(np.float32)
+    gx, gy = rng.integers(1, 320 // tile, n), rng.integers(1, 240 // tile, n)
+    pos = np.stack([((gx * tile - c.center_x) / c.focal_x * (z + 3.0)).astype(np.float32),
+                    ((gy * tile - c.center_y) / c.focal_y * (z + 3.0)).astype(np.float32), z], 1)
+    feats, opac = synthetic.point_attributes(n, 4, "normal", 9)
+    monkeypatch.setattr(rasterization, "_ALWAYS_FITS_POINTS", 0)   # take the library's default capacity
+    image, alpha, weights = rasterize_points(hv.to_view(gpu), H.dev(pos), H.dev(feats), H.dev(opac), tile=tile)
+    ref = oracle.raster_forward(oracle_cfg(oracle, hv, n, tile, 4, oracle.FEAT_DIRECT_F32), pos, feats, opac, hv.w2c)
+    H.assert_close(image.cpu().numpy(), ref["image"], RTOL, 1e-5, "image")
+    H.assert_close(weights.cpu().numpy(), ref["blending_weights"], RTOL, 1e-7, "blending weights")
 
 
 def test_autograd_api_sh_and_direct(gpu, oracle):
