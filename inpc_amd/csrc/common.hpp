@@ -137,11 +137,11 @@ __host__ __device__ __forceinline__ uint64_t pcg_apply(const PcgJump& j, uint64_
 }
 
 // ---- decoupled look-back --------------------------------------------------------------------------
-// A status word is {2 flag bits, 30 value bits}. A block must only ever wait on blocks that are running. The
-// large kernels get that by running as one resident grid whose blocks take the tiles in order (block index,
-// + grid size, ...); the small ones by taking their tile index from an atomic ticket (thousands of blocks
-// taking tickets from one address at the start of a kernel cost more than the look-back itself). The wait is
-// bounded and raises the error flag instead of spinning forever.
+// A status word is {2 flag bits, 30 value bits}. A block must only ever wait on blocks that are running: every
+// kernel with a look-back hands its tiles out through an atomic ticket, taken when a block starts a tile, so a
+// tile that is waited for has always been taken by a block that was running then, whatever else occupies the GPU
+// (other streams, other kernels). The grids are sized to what fits the GPU at once, so a block takes many tiles
+// and the tickets stay few. The wait is bounded all the same and raises the error flag instead of spinning forever.
 constexpr uint32_t kFlagAggregate = 1u << 30;
 constexpr uint32_t kFlagInclusive = 2u << 30;
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
@@ -172,10 +172,7 @@ __device__ __forceinline__ uint32_t lookback_walk(uint32_t* status, uint32_t str
     if (bid == 0) return 0u;
     // Several predecessors are fetched per round trip and consumed nearest first; the walk ends at the
     // first one that carries an inclusive prefix and waits at the first one that has nothing yet.
-#ifndef INPC_LOOKBACK_AHEAD
-#define INPC_LOOKBACK_AHEAD 8
-#endif
-    constexpr int kAhead = INPC_LOOKBACK_AHEAD;
+    constexpr int kAhead = 8;
     uint32_t exclusive = 0u, spins = 0u;
     int64_t p = (int64_t)bid - 1;
     bool finished = false;

@@ -17,17 +17,11 @@ namespace radix {
 
 // Digits of up to 8 bits. (9-bit digits save a pass on 27-bit depth keys, but a pass then leaves the block in runs
 // of 8 keys instead of 32 and takes a third longer: measured 3 x 88 us against 4 x 66 us.)
-#ifndef INPC_RADIX_BITS
-#define INPC_RADIX_BITS 8
-#endif
-constexpr int kMaxBits = INPC_RADIX_BITS;
+constexpr int kMaxBits = 8;
 constexpr int kRadix = 1 << kMaxBits;
 constexpr int kBlock = kRadix;          // thread d owns digit d
 constexpr int kWaves = kBlock / kWave;
-#ifndef INPC_RADIX_ITEMS
-#define INPC_RADIX_ITEMS (4096 / (1 << INPC_RADIX_BITS))
-#endif
-constexpr int kItems = INPC_RADIX_ITEMS;
+constexpr int kItems = 4096 / kRadix;
 constexpr int kTile = kBlock * kItems;  // keys per block
 constexpr int kMaxPasses = 4;
 static_assert(kMaxBits * kMaxPasses >= 32, "every 32-bit key must fit the passes");
@@ -108,29 +102,6 @@ enum FirstPass : int {
                        // the drawn points for free
 };
 
-#ifdef INPC_SORT_PROFILE
-// development aid: per-phase shader clocks of k_scatter, summed over blocks (thread 0 of each)
-__device__ unsigned long long g_sort_profile[8];
-#define INPC_SORT_PROF_DECL unsigned long long sp_t = clock64(), sp_acc[7] = {0, 0, 0, 0, 0, 0, 0}
-#define INPC_SORT_PROF_MARK(i)                    \
-    do {                                          \
-        const unsigned long long now_ = clock64(); \
-        sp_acc[i] += now_ - sp_t;                 \
-        sp_t = now_;                              \
-    } while (0)
-#define INPC_SORT_PROF_FLUSH                                                        \
-    do {                                                                            \
-        if (threadIdx.x == 0) {                                                     \
-            for (int i_ = 0; i_ < 7; ++i_) atomicAdd(&g_sort_profile[i_], sp_acc[i_]); \
-            atomicAdd(&g_sort_profile[7], 1ull);                                    \
-        }                                                                           \
-    } while (0)
-#else
-#define INPC_SORT_PROF_DECL
-#define INPC_SORT_PROF_MARK(i)
-#define INPC_SORT_PROF_FLUSH
-#endif
-
 // One digit pass. FIRST: n comes from the host and keys equal to kInvalidKey are dropped.
 // Order of work inside a block: load -> digit histogram (LDS atomics) -> publish the aggregates -> stable
 // ranking -> look-back walk -> LDS staging -> coalesced write. Publishing before the expensive ranking means
@@ -148,21 +119,24 @@ __global__ void __launch_bounds__(kBlock)
     __shared__ KeyT s_keys[kTile];
     __shared__ uint32_t s_vals[kTile];
     __shared__ uint32_t s_wave[kWaves];
+    __shared__ uint32_t s_bid;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    INPC_SORT_PROF_DECL;
     uint32_t n = n_host;
     if (!FIRST) n = min(n_host, *n_dev);
-    // Tiles in order, bid = blockIdx.x, + gridDim.x, ...: a tile waits (look-back) only for tiles in front of it,
-    // and those belong to blocks that are running or to an earlier round of this grid, which the host sizes
-    // so that all of it is resident at once: no block has to end for another one to start.
-    for (uint32_t bid = blockIdx.x;; bid += gridDim.x) {
+    // A block takes its tiles from a ticket counter, in order: a tile waits (look-back) only for tiles in front of
+    // it, and each of those was taken by a block that was running when it took it. So nothing ever waits for a
+    // block that has not started, whatever else occupies the GPU; the grid only needs as many blocks as fit.
+    uint32_t* ticket = status + (size_t)((n_host + kTile - 1u) / kTile) * kRadix;
+    for (;;) {
+    if (tid == 0) s_bid = atomicAdd(ticket, 1u);
+    __syncthreads();
+    const uint32_t bid = s_bid;
     const uint64_t tile_base = (uint64_t)bid * kTile;
     if (tile_base >= n) break;
     for (int i = tid; i < kWaves * kRadix; i += kBlock) (&s_cnt[0][0])[i] = 0u;
     s_hist[tid] = 0u;
     __syncthreads();
-    INPC_SORT_PROF_MARK(0);
 
     KeyT key[kItems];
     uint32_t val[kItems];
@@ -193,7 +167,6 @@ __global__ void __launch_bounds__(kBlock)
         if (lane >= (uint32_t)s) incl += up;
     }
     if (lane == 63) s_wave[wave] = incl;
-    INPC_SORT_PROF_MARK(1);
 
     // stable rank of every key among the keys of its wave with the same digit
     uint32_t rank[kItems];
@@ -215,7 +188,6 @@ __global__ void __launch_bounds__(kBlock)
         }
         __builtin_amdgcn_wave_barrier();
     }
-    INPC_SORT_PROF_MARK(2);
     __syncthreads();
 
     // per-wave offsets inside the digit's run, block-level exclusive scan over the digits
@@ -237,13 +209,11 @@ __global__ void __launch_bounds__(kBlock)
     }
     const uint32_t local_base = wave_off + incl - total;
     s_local_base[tid] = local_base;
-    INPC_SORT_PROF_MARK(3);
     if (tid <= digit_mask) {  // one look-back per digit in use
         const uint32_t exclusive = lookback_walk(status + tid, kRadix, bid, total, error_flag);
         s_global[tid] = digit_base[tid] + exclusive - local_base;
     }
     __syncthreads();
-    INPC_SORT_PROF_MARK(4);
 
 #pragma unroll
     for (int r = 0; r < kItems; ++r) {
@@ -255,7 +225,6 @@ __global__ void __launch_bounds__(kBlock)
         }
     }
     __syncthreads();
-    INPC_SORT_PROF_MARK(5);
 #pragma unroll
     for (int j = 0; j < kItems; ++j) {
         const uint32_t idx = j * kBlock + tid;
@@ -267,14 +236,12 @@ __global__ void __launch_bounds__(kBlock)
             vals_out[out] = s_vals[idx];
         }
     }
-    INPC_SORT_PROF_MARK(6);
     __syncthreads();   // the LDS arrays are reused by the next tile
     }
-    INPC_SORT_PROF_FLUSH;
 }
 
-// Status words one pass needs for up to n_max keys.
-inline size_t status_words(uint32_t n_max) { return (size_t)div_up(n_max, kTile) * kRadix; }
+// Status words one pass needs for up to n_max keys: a word per (tile, digit), then the pass's ticket counter.
+inline size_t status_words(uint32_t n_max) { return (size_t)div_up(n_max, kTile) * kRadix + kRadix; }
 
 // Enqueue every pass of a sort. Buffers ping-pong: pass 0 reads keys_a / vals_a, the result ends in the
 // a-buffers when the pass count is even, else in the b-buffers.

@@ -354,17 +354,19 @@ struct CullState {
     uint32_t accepted;   // samples accepted so far in this draw (a lower bound once `consumed` is set)
     uint32_t consumed;   // candidates consumed when the capacity-th sample was accepted, else 0
     uint32_t error;      // look-back gave up
-    uint32_t unused;
+    uint32_t ticket;     // next tile of the round that is running (cleared with the round's status words)
     uint32_t pad[12];
 };
 constexpr size_t kCullHeaderWords = sizeof(CullState) / 4;
+constexpr int kTileJumpBits = 20;   // a round has fewer than 2^20 tiles (candidate indices stay below 2^30)
 
 __global__ void __launch_bounds__(kDrawBlock)
     k_sample_cull(const float4* __restrict__ boxes, const float* __restrict__ cdf, const float* __restrict__ sum_dev,
                   const float* __restrict__ w2c, float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
                   uint32_t capacity, uint32_t k0, uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam,
                   const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
-    __shared__ uint32_t s_accepted0, s_exclusive, s_done;
+    __shared__ uint32_t s_accepted0, s_exclusive, s_done, s_bid;
+    __shared__ PcgJump s_tile_jump[kTileJumpBits];   // generator step over 2^b tiles
     __shared__ uint32_t s_count[kSampleItems * (kDrawBlock / kWave)];
     __shared__ __align__(16) float s_tree[kTreeNodes];
     if (!(*sum_dev > 0.0f)) return;
@@ -380,14 +382,21 @@ __global__ void __launch_bounds__(kDrawBlock)
     const uint64_t rng_inc = rng_dev[1];
     const PcgJump jump_thread = pcg_jump(rng_inc, 4ull * tid);
     const TileJumps jumps = make_tile_jumps(rng_inc);
-    const PcgJump jump_grid = pcg_jump(rng_inc, 4ull * (uint64_t)gridDim.x * kDrawTile);
-    uint64_t tile_state = pcg_apply(pcg_jump(rng_inc, 4ull * ((uint64_t)k0 + (uint64_t)blockIdx.x * kDrawTile)), rng_dev[0]);
-    // Tiles in order: a tile waits (look-back) only for tiles in front of it, and those belong to blocks that are
-    // running or to an earlier round of this grid, which stays resident as a whole (the host sizes it so):
-    // no block has to end for another one to start.
-    for (uint32_t bid = blockIdx.x; bid < n_blocks; bid += gridDim.x) {
+    if (tid < (uint32_t)kTileJumpBits) s_tile_jump[tid] = pcg_jump(rng_inc, (4ull * kDrawTile) << tid);
+    uint64_t tile_state = pcg_apply(pcg_jump(rng_inc, 4ull * (uint64_t)k0), rng_dev[0]);   // of tile `at`
+    uint32_t at = 0;
+    // A block takes its tiles from a ticket counter, in order: a tile waits (look-back) only for tiles in front of
+    // it, and each of those was taken by a block that was running then. Nothing ever waits for a block that has
+    // not started, whatever else occupies the GPU.
+    for (;;) {
+        if (tid == 0) s_bid = atomicAdd(&st->ticket, 1u);
+        __syncthreads();   // also: s_tile_jump is complete
+        const uint32_t bid = s_bid;
+        if (bid >= n_blocks) break;
+        for (uint32_t step = bid - at, b = 0; step != 0u; step >>= 1, ++b)
+            if (step & 1u) tile_state = pcg_apply(s_tile_jump[b], tile_state);
+        at = bid;
         const uint64_t state0 = pcg_apply(jump_thread, tile_state);
-        tile_state = pcg_apply(jump_grid, tile_state);
         if (tid == 0) {
             const uint32_t done = __hip_atomic_load(&st->consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
             s_done = done;
@@ -451,13 +460,14 @@ __global__ void __launch_bounds__(kDrawBlock)
                 __hip_atomic_store(&st->consumed, (uint32_t)(k0 + rel + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        __syncthreads();   // s_count, s_exclusive and s_done are reused by the next tile
+        __syncthreads();   // s_count, s_exclusive, s_done and s_bid are reused by the next tile
     }
 }
 
-__global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks) {
+__global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks, CullState* st) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n_blocks) status[i] = 0u;
+    if (i == 0) st->ticket = 0u;
 }
 
 // Failure pattern of B/sampling/src/sampling.cu:107-111 when the weight sum is not positive.
@@ -793,8 +803,8 @@ int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* 
     uint32_t* status = (uint32_t*)workspace + kCullHeaderWords;
     const uint32_t n_blocks = div_up(n_candidates, kDrawTile);
     INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(n_blocks, kBlock)), dim3(kBlock), stream, status,
-                n_blocks);
-    // the whole grid must be resident at once: its blocks wait for each other's tiles
+                n_blocks, st);
+    // as many blocks as the GPU holds at once; each takes tiles until none is left
     uint32_t resident = 0;
     const int rc = resident_blocks((const void*)k_sample_cull, kDrawBlock, resident);
     if (rc != INPC_OK) return rc;

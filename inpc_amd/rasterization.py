@@ -118,7 +118,7 @@ def _checked_camera_tensor(t: torch.Tensor, numel: int, name: str, device) -> to
         raise RuntimeError(f"{name} must be a tensor")
     if t.dtype != torch.float32:
         raise RuntimeError(f"expected scalar type Float for {name}")
-    if not t.is_cuda or t.device != device:
+    if t.device != device:
         raise RuntimeError(f"expected {name} on the device of the points ({device})")
     if t.numel() != numel:
         raise RuntimeError(f"{name} must hold {numel} values")

@@ -165,8 +165,13 @@ class ProbabilityFieldSampler(torch.nn.Module):
         _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0,
                                         _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream), "inpc_cull_finish")
         if consumed.value == 0 and accepted.value < n_samples and float(total[0].item()) > 0.0:
-            _log.warning("sampler accepted only %d of %d samples; the rest is uninitialised", accepted.value,
-                         n_samples)
+            # the draw gave up (the frustum is hardly ever hit, or the candidate limit was reached): the slots behind
+            # the accepted samples get the failure pattern of B/sampling/src/sampling.cu:107-111, positions 0 and
+            # index -1, instead of whatever the buffers held (the reference's kernel would not return here)
+            _log.warning("sampler accepted only %d of %d samples; the rest is filled with position 0 / index -1",
+                         accepted.value, n_samples)
+            positions[accepted.value:].zero_()
+            ids32[accepted.value:].fill_(-1)
         _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
         return positions, ids64
 

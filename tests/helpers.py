@@ -245,26 +245,34 @@ class RasterRun:
             out["blending_weights"] = self.bw.cpu().numpy()[:self.n]
         return out
 
-    def backward(self, grad_image, grad_alpha):
+    def backward_async(self, gi, ga):
+        """Enqueues the backward pass on the current stream; device tensors in, device tensors out. The scratch
+        buffer is kept on the object so that it outlives the call."""
         mode = self.cfg.feature_mode
         n, Cn = self.n, self.C
         device = self.device
-        scratch = None
+        self._scratch = None
         if mode == _lib.FEAT_SH36_F16:
             gf = torch.full((n, 36), float("nan"), dtype=torch.float16, device=device)
-            scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
+            self._scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
         elif mode == _lib.FEAT_DIRECT_F16:
             gf = torch.full((n, Cn), float("nan"), dtype=torch.float16, device=device)
-            scratch = torch.empty((n, Cn), dtype=torch.float32, device=device)
+            self._scratch = torch.empty((n, Cn), dtype=torch.float32, device=device)
         else:
             gf = torch.full((n, Cn), float("nan"), dtype=torch.float32, device=device)
         go = torch.full((n,), float("nan"), dtype=torch.float32, device=device)
-        gi, ga = dev(np.asarray(grad_image, np.float32), device), dev(np.asarray(grad_alpha, np.float32), device)
+        self._grads_in = (gi, ga)
         _lib.check(self.lib.inpc_raster_backward(
             C.byref(self.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(self.image), _lib.ptr(self.alpha),
-            _lib.ptr(self.positions), _lib.ptr(self.cam_position), _lib.ptr(gf), _lib.ptr(go), _lib.ptr(scratch),
+            _lib.ptr(self.positions), _lib.ptr(self.cam_position), _lib.ptr(gf), _lib.ptr(go), _lib.ptr(self._scratch),
             _lib.ptr(self.ws), self.layout.total_bytes, stream()),
             "inpc_raster_backward")
+        return gf, go
+
+    def backward(self, grad_image, grad_alpha):
+        device = self.device
+        gf, go = self.backward_async(dev(np.asarray(grad_image, np.float32), device),
+                                     dev(np.asarray(grad_alpha, np.float32), device))
         return gf.cpu().numpy(), go.cpu().numpy()
 
 
@@ -367,25 +375,32 @@ class GaussianRun:
 
     outputs = RasterRun.outputs
 
-    def backward(self, grad_image, grad_alpha):
+    def backward_async(self, gi, ga):
+        """Enqueues the backward pass on the current stream; device tensors in, device tensors out."""
         mode = self.cfg.base.feature_mode
         n, Cn = self.n, self.C
         device = self.device
-        scratch = None
+        self._scratch = None
         if mode == _lib.FEAT_SH36_F16:
             gf = torch.full((n, 36), float("nan"), dtype=torch.float16, device=device)
-            scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
+            self._scratch = torch.empty((n, 4), dtype=torch.float32, device=device)
         elif mode == _lib.FEAT_DIRECT_F16:
             gf = torch.full((n, Cn), float("nan"), dtype=torch.float16, device=device)
-            scratch = torch.empty((n, Cn), dtype=torch.float32, device=device)
+            self._scratch = torch.empty((n, Cn), dtype=torch.float32, device=device)
         else:
             gf = torch.full((n, Cn), float("nan"), dtype=torch.float32, device=device)
         go = torch.full((n,), float("nan"), dtype=torch.float32, device=device)
-        gi, ga = dev(np.asarray(grad_image, np.float32), device), dev(np.asarray(grad_alpha, np.float32), device)
+        self._grads_in = (gi, ga)
         _lib.check(self.lib.inpc_gaussian_backward(
             C.byref(self.cfg), _lib.ptr(gi), _lib.ptr(ga), _lib.ptr(self.image), _lib.ptr(self.alpha),
-            _lib.ptr(self.positions), _lib.ptr(self.cam_position), _lib.ptr(gf), _lib.ptr(go), _lib.ptr(scratch),
+            _lib.ptr(self.positions), _lib.ptr(self.cam_position), _lib.ptr(gf), _lib.ptr(go), _lib.ptr(self._scratch),
             _lib.ptr(self.ws), self.layout.total_bytes, stream()), "inpc_gaussian_backward")
+        return gf, go
+
+    def backward(self, grad_image, grad_alpha):
+        device = self.device
+        gf, go = self.backward_async(dev(np.asarray(grad_image, np.float32), device),
+                                     dev(np.asarray(grad_alpha, np.float32), device))
         return gf.cpu().numpy(), go.cpu().numpy()
 
 

@@ -202,3 +202,22 @@ def test_non_perspective_and_distorted_cameras_are_rejected(gpu):
     view.camera.distortion = object()
     with pytest.raises(NotImplementedError):
         ProbabilityFieldSampler(0).generate_samples(*args, view, 10, 4.0)
+
+
+def test_training_draw_that_never_hits_the_frustum_is_filled_with_the_failure_pattern(gpu):
+    # One leaf whose far face lies exactly on the near plane: its corners are visible, so its weight is positive, but
+    # every jittered position inside it is nearer than the near plane and is culled. The draw gives up and the
+    # samples it could not produce are position 0 / index -1, not whatever the buffers held.
+    from inpc_amd import ProbabilityFieldSampler, synthetic
+
+    hv = synthetic.camera_on_z(400, 300, 100.0, 0.0, near=1.0, far=50.0)   # camera at the origin, looking along +z
+    centers = np.array([[0.0, 0.0, 0.5]], np.float32)                        # cube [-0.5, 0.5]^2 x [0, 1]
+    levels = np.zeros(1, np.int32)
+    weights = np.ones(1, np.float32)
+    sampler = ProbabilityFieldSampler(seed=3)
+    view = hv.to_view(gpu)
+    w = H.leaf_weights(synthetic.Octree(centers, levels, weights, 1.0), hv)
+    assert float(w[0].item()) > 0.0
+    pos, ids = sampler.generate_training_samples(H.dev(centers), H.dev(levels), H.dev(weights), view, 1000, 1.0)
+    assert pos.shape == (1000, 3) and ids.shape == (1000,)
+    assert (pos == 0).all() and (ids == -1).all()

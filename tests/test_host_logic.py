@@ -160,3 +160,21 @@ def test_synthetic_scene_helpers_are_deterministic():
     np.testing.assert_allclose(rot @ rot.T, np.eye(3), atol=1e-6)
     # the stored camera position is the point the world-to-camera transform maps to the origin
     np.testing.assert_allclose(rot @ hv.position + hv.w2c[:3, 3], 0, atol=1e-5)
+
+
+def test_camera_tensors_must_be_fp32_on_the_points_device():
+    # w2c and cam_position reach the kernels as raw float pointers: another dtype would be reinterpreted, a host
+    # tensor would hand a host address to a kernel. Both are refused before anything is launched.
+    from inpc_amd.rasterization import _checked_camera_tensor
+
+    device = torch.device("cuda:0")
+    with pytest.raises(RuntimeError, match="Float"):
+        _checked_camera_tensor(torch.eye(4, dtype=torch.float64), 16, "w2c", device)
+    with pytest.raises(RuntimeError, match="on the device of the points"):
+        _checked_camera_tensor(torch.eye(4), 16, "w2c", device)
+    with pytest.raises(RuntimeError, match="must hold 3 values"):
+        _checked_camera_tensor(torch.zeros(4), 3, "cam_position", torch.device("cpu"))
+    with pytest.raises(RuntimeError, match="must be a tensor"):
+        _checked_camera_tensor(np.eye(4, dtype=np.float32), 16, "w2c", device)
+    ok = _checked_camera_tensor(torch.eye(4).t(), 16, "w2c", torch.device("cpu"))   # made contiguous, otherwise as given
+    assert ok.is_contiguous() and ok.dtype == torch.float32
