@@ -290,3 +290,52 @@ def test_backward_against_central_differences(oracle):
     # points that are not drawn get exact zeros
     hidden = ref["n_touched"] == 0
     assert np.all(gf[hidden] == 0) and np.all(go[hidden] == 0)
+
+
+def test_backward_on_saturating_pixels(oracle):
+    # The branch the smooth scene above never takes: pixels whose transmittance falls below 1e-4. The fragment that
+    # crosses the threshold still gets its gradient, the ones behind it get none
+    # (B/rasterization/src/gaussian/kernels.cu:476-579); the brute force ends a pixel's list the same way, so its
+    # central differences are those of the truncated blend.
+    hv, pos, feats, opac = small_scene(41, n=1100)
+    for k in range(60):   # sixty spots with sixteen nearly opaque points each
+        pos[16 * k: 16 * (k + 1)] = pos[1000 + k]
+    opac[:960] = 0.97
+    n, tile = len(pos), 8
+    g = gcfg_of(oracle, hv, n, tile, 4)
+    count = oracle.gaussian_instance_count(g, pos, hv.w2c)
+    ref = oracle.raster_forward(g.base, pos, feats, opac, hv.w2c, debug=True, gaussian=g, n_instances_hint=count)
+    saturated = ref["alpha"][0] == 1.0
+    assert saturated.sum() >= 40, "the scene must saturate many pixels"
+    rng = np.random.default_rng(5)
+    gi = rng.standard_normal(ref["image"].shape).astype(np.float32)
+    ga = rng.standard_normal(ref["alpha"].shape).astype(np.float32)
+    gf, go, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c, gaussian=g)
+    assert np.isfinite(gf).all() and np.isfinite(go).all()
+    geom = (ref["screen_xy"][:, 0].astype(np.float64), ref["screen_xy"][:, 1].astype(np.float64),
+            ref["depth"].astype(np.float64), ref["conic"].astype(np.float64), ref["bounds"], ref["n_touched"])
+
+    def loss(f, o):
+        img, alpha, _, _ = brute_force(hv, *geom, f, o, ref["depth_order"], tile, TRAIN_THRESHOLD)
+        return float((img * gi).sum() + (alpha * ga[0]).sum())
+
+    # The sixteen points of a spot coincide, so they are drawn in index order: the first ones are reached on every
+    # pixel of their footprint, the last ones lie behind the cut on the spot's saturated centre pixel and are only
+    # reached on the pixels around it. Both kinds must have the truncated blend's derivative.
+    _, alpha_bf, _, _ = brute_force(hv, *geom, feats, opac, ref["depth_order"], tile, TRAIN_THRESHOLD)
+    np.testing.assert_array_equal(alpha_bf == 1.0, saturated)
+    spots = [k for k in range(60) if ref["n_touched"][16 * k] > 0]
+    reached = np.array([16 * k + j for k in spots[::6] for j in (0, 15)])
+    assert len(reached) >= 10
+    eps = 1e-6
+    for i in reached:
+        o_hi, o_lo = opac.astype(np.float64), opac.astype(np.float64)
+        o_hi[i] += eps
+        o_lo[i] -= eps
+        d = (loss(feats.astype(np.float64), o_hi) - loss(feats.astype(np.float64), o_lo)) / (2 * eps)
+        np.testing.assert_allclose(go[i], d, rtol=5e-3, atol=5e-4)
+        f_hi, f_lo = feats.astype(np.float64), feats.astype(np.float64)
+        f_hi[i, 1] += 1e-4
+        f_lo[i, 1] -= 1e-4
+        d = (loss(f_hi, opac.astype(np.float64)) - loss(f_lo, opac.astype(np.float64))) / 2e-4
+        np.testing.assert_allclose(gf[i, 1], d, rtol=2e-3, atol=2e-4)

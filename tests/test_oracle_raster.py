@@ -304,6 +304,90 @@ def test_backward_against_autograd_and_finite_differences(oracle, tile, channels
         assert go[i] == pytest.approx((vals[0] - vals[1]) / (2 * eps), rel=2e-2, abs=2e-3)
 
 
+def truncated_forward_torch(hv, ref, feats, opac):
+    """Float64 restatement of the blend *with* the reference's early termination (kernels.cu:281-299,383-417): a
+    pixel's list ends behind the fragment that takes its transmittance below 1e-4 (that fragment included). Which
+    fragment that is is decided in fp32, from the fp32 screen positions and in the order the oracle reports, exactly
+    as the kernel decides it; the values are float64 and differentiable. A saturated pixel's alpha is the constant 1.
+    Returns image, alpha and, per point, whether any of its fragments was reached."""
+    c = hv.camera
+    xy = ref["screen_xy"]
+    C_ = feats.shape[1]
+    img = [[torch.zeros(C_, dtype=torch.float64) for _ in range(c.width)] for _ in range(c.height)]
+    Tr = [[torch.ones((), dtype=torch.float64) for _ in range(c.width)] for _ in range(c.height)]
+    T32 = np.ones((c.height, c.width), np.float32)
+    done = np.zeros((c.height, c.width), bool)
+    reached = np.zeros(len(xy), bool)
+    opac32 = opac.detach().numpy().astype(np.float32)
+    for i in ref["depth_order"]:
+        sx, sy = xy[i]
+        for py in range(int(np.floor(sy - 1.5)), int(np.floor(sy + 0.5)) + 2):
+            for px in range(int(np.floor(sx - 1.5)), int(np.floor(sx + 0.5)) + 2):
+                if not (0 <= px < c.width and 0 <= py < c.height) or done[py, px]:
+                    continue
+                dx32, dy32 = np.abs(sx - np.float32(px + 0.5)), np.abs(sy - np.float32(py + 0.5))
+                if dx32 >= 1 or dy32 >= 1:
+                    continue
+                w32 = np.float32(np.float32(1) - dx32) * np.float32(np.float32(1) - dy32)
+                a32 = np.float32(opac32[i] * w32)
+                T32[py, px] = np.float32(T32[py, px] * np.float32(np.float32(1) - a32))
+                done[py, px] = T32[py, px] < np.float32(1e-4)
+                reached[i] = True
+                a = opac[i] * ((1 - float(dx32)) * (1 - float(dy32)))
+                img[py][px] = img[py][px] + Tr[py][px] * a * feats[i]
+                Tr[py][px] = Tr[py][px] * (1 - a)
+    image = torch.stack([torch.stack(row) for row in img]).permute(2, 0, 1)
+    T = torch.stack([torch.stack(row) for row in Tr])
+    alpha = torch.where(torch.from_numpy(done), torch.ones_like(T), 1 - T)
+    return image, alpha[None], reached, done
+
+
+@pytest.mark.parametrize("tile,channels", [(8, 4), (16, 8)])
+def test_backward_on_saturating_pixels_and_opaque_fragments(oracle, tile, channels):
+    # The two branches the smooth scene above never takes: pixels whose transmittance falls below 1e-4 (the fragment
+    # that crosses the threshold still gets its gradient, the ones behind it get none, kernels.cu:383-417) and
+    # fragments with alpha exactly 1, where the reference divides by max(1 - alpha, 1e-8) (kernels.cu:400).
+    n = 900
+    hv = synthetic.camera_on_z(16, 12, 16.0, 2.0)   # focal 16 at depth 2: screen x = 8 x + 8 exactly
+    rng = np.random.default_rng(41)
+    pos = synthetic.cube_points(n, 1.0, 42)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", 43)
+    opac = rng.uniform(0.3, 0.98, n).astype(np.float32)
+    # forty points exactly on pixel centres (depth exactly 2) with opacity exactly 1: alpha = 1, transmittance 0
+    k = 40
+    px, py = rng.integers(2, 14, k), rng.integers(2, 10, k)
+    pos[:k, 0] = ((px + 0.5) - 8.0) / 8.0
+    pos[:k, 1] = ((py + 0.5) - 6.0) / 8.0
+    pos[:k, 2] = 0.0
+    opac[:k] = 1.0
+    cfg = cfg_of(oracle, hv, n, tile, channels)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    assert (ref["alpha"] == 1.0).sum() >= 50, "the scene must saturate many pixels"
+    assert np.array_equal(ref["screen_xy"][:k, 0], (px + 0.5).astype(np.float32))   # exactly on the centres
+    gi = rng.normal(0, 1.0, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1.0, ref["alpha"].shape).astype(np.float32)
+    gf, go, _ = oracle.raster_backward(cfg, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c)
+    assert np.isfinite(gf).all() and np.isfinite(go).all()
+    f_t = torch.tensor(feats.astype(np.float64), requires_grad=True)
+    o_t = torch.tensor(opac.astype(np.float64), requires_grad=True)
+    image, alpha, reached, done = truncated_forward_torch(hv, ref, f_t, o_t)
+    np.testing.assert_array_equal(done[None], ref["alpha"] == 1.0)           # the same pixels saturate
+    np.testing.assert_allclose(image.detach().numpy(), ref["image"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(alpha.detach().numpy(), ref["alpha"], rtol=1e-4, atol=1e-6)
+    loss = (image * torch.tensor(gi, dtype=torch.float64)).sum() + (alpha * torch.tensor(ga, dtype=torch.float64)).sum()
+    loss.backward()
+    np.testing.assert_allclose(gf, f_t.grad.numpy(), rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(go, o_t.grad.numpy(), rtol=2e-4, atol=2e-5)
+    # points whose every fragment lies behind a cut get exactly nothing
+    hidden = (ref["n_touched"] > 0) & ~reached
+    assert hidden.sum() > 10
+    assert (gf[hidden] == 0).all() and (go[hidden] == 0).all()
+    # an opaque fragment on a pixel centre that is reached: its opacity gradient is T f . g (nothing behind it)
+    front = [i for i in range(k) if reached[i]]
+    assert len(front) >= 5
+    assert np.abs(go[front]).max() > 0
+
+
 def test_combined_step_equals_separate_calls(oracle):
     n = 20000
     hv = synthetic.camera_on_z(120, 80, 100.0, 2.4)
