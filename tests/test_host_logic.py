@@ -178,3 +178,23 @@ def test_camera_tensors_must_be_fp32_on_the_points_device():
         _checked_camera_tensor(np.eye(4, dtype=np.float32), 16, "w2c", device)
     ok = _checked_camera_tensor(torch.eye(4).t(), 16, "w2c", torch.device("cpu"))   # made contiguous, otherwise as given
     assert ok.is_contiguous() and ok.dtype == torch.float32
+
+
+def test_c_module_has_the_eleven_names_with_the_reference_parameter_lists():
+    """Names and parameter counts of B/torch_bindings/bindings.cpp:10-29 with rasterization_api.h:8-86,
+    sampling_api.h:11-82 and misc_api.h:7-25."""
+    import inspect
+
+    from inpc_amd import _C
+
+    expected = {"forward": 14, "backward": 22, "render": 15, "render_preextracted": 17,
+                "compute_viewpoint_weights_cuda": 13, "compute_normalized_weight_decay_grads_cuda": 1,
+                "add_normalized_weight_decay_grads_cuda": 2, "spherical_contraction_cuda": 1, "cauchy_loss_cuda": 2,
+                "cauchy_loss_backward_cuda": 3}
+    for name, count in expected.items():
+        assert len(inspect.signature(getattr(_C, name)).parameters) == count, name
+    sampler = _C.ProbabilityFieldSamplerCUDA
+    assert len(inspect.signature(sampler.__init__).parameters) == 2          # self, seed
+    assert len(inspect.signature(sampler.generate_training_samples).parameters) == 15
+    assert len(inspect.signature(sampler.generate_samples).parameters) == 15
+    assert len(inspect.signature(sampler.generate_expected_samples).parameters) == 16
