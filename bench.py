@@ -9,7 +9,9 @@ before the timed region.
 
 Prints ONE JSON line. `value` is Mpoints/s of forward+backward; `roofline` describes the kernel with the
 largest share of the step (algorithmic bytes per launch / HIP-event duration on the launch stream);
-`cpu_baseline` is the CPU oracle running the same step on a bounded sample with all host threads.
+`cpu_baseline` is the CPU oracle running the same step on a bounded sample, with all host threads and with one.
+`extra` carries the sampler's figures, the Gaussian footprint, the reference-shaped autograd step and the
+large-frame inference configuration (33,554,432 points @2473x1643).
 """
 from __future__ import annotations
 
@@ -37,20 +39,21 @@ WORKLOADS = {
 }
 
 
-def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, depth_passes, tile_passes, end_bit):
-    """Algorithmic bytes one launch of `kernel` moves: each array of the pipeline touched the minimum
-    number of times its structure requires. F = feature bytes per point, R = blend record
-    (8 xy + 4 opacity + 4C features)."""
+def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, end_bit):
+    """Algorithmic bytes that all launches of `kernel` in one step move together: every array of the reference's
+    pipeline structure touched the minimum number of times that structure requires, booked on the kernel that does
+    that part of the work here. F = feature bytes per point, R = blend record (8 xy + 4 opacity + 4C features).
+    Kernels that only exist in this pipeline (bin offsets, the gradient reduction) carry no algorithmic bytes."""
     F = 4 * channels
     R = 8 + 4 + 4 * channels
     table = {
-        "raster_bin_count": n * 12,
-        "raster_preprocess": n * (16 + F) + v * (R + 8),
-        "raster_depth_sort": v * 68 / max(depth_passes, 1),
-        # expansion reads + instance emission + tile sort + range scan of the reference structure, done here by
-        # raster_inst_count (reads the sort values once more) and raster_inst_emit
-        "raster_inst_count": v * 4,
-        "raster_inst_emit": v * 36 + i * (6 + 2 + 12 * ((end_bit + 7) // 8) + 2),
+        # the count/scan in front of the instance expansion
+        "raster_bin_count": v * 20,
+        # point in (xyz, features, opacity), record + key/index out, instance emission (expansion reads + 6 B each)
+        "raster_preprocess": n * (16 + F) + v * (R + 8 + 16) + i * 6,
+        # what the reference structure spends on ordering: depth sort of the visible points (4 B histogram read +
+        # 4 passes x 16 B), tile sort of the instances and the range scan
+        "raster_tile_sort": v * 68 + i * (2 + 12 * ((end_bit + 7) // 8) + 2),
         "raster_blend_forward": i * (4 + R) + pixels * 4 * (channels + 1) + n * 4,
         "raster_blend_backward": i * (4 + R) + pixels * 8 * (channels + 1) + n * (4 * channels + 4),
         "fill_u32": n * (4 * channels + 4),
@@ -58,11 +61,16 @@ def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, depth_passes, tile
     return float(table.get(kernel, 0.0))
 
 
+def traffic_file(workload: str) -> Path:
+    return ROOT / "profiles" / f"hbm_traffic_{workload}.txt"
+
+
 def measured_traffic(kernel: str, workload: str):
     """HBM bytes per launch of `kernel` from the committed profiler-counter summary of this workload
     (profiles/hbm_traffic_<workload>.txt, lines `<kernel> fetch_bytes=F write_bytes=W total_bytes=T`),
-    or None when no such measurement is on file."""
-    path = ROOT / "profiles" / f"hbm_traffic_{workload}.txt"
+    or None when no such measurement is on file. The figure comes from that earlier profiler run of the same
+    command, not from the run that prints it."""
+    path = traffic_file(workload)
     if not path.exists():
         return None
     for line in path.read_text().splitlines():
@@ -93,9 +101,12 @@ def main() -> int:
     ap.add_argument("--pmc-copy", action="store_true",
                     help="also launch three 1 GiB plain copies (the yardstick for profiler byte counters)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target duration of the CPU baseline leg")
-    ap.add_argument("--with-config4", action="store_true",
-                    help="also time the large-frame inference configuration (33,554,432 points @2473x1643, 16 fp16 "
-                         "channels): training draw + inference forward, reported in extra.config4_inference")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="only the timed step, its per-kernel durations and the sampler draw: no graph replay, field "
+                         "update, Gaussian footprint, reference-shaped step or large-frame leg (for profiler runs)")
+    ap.add_argument("--no-config4", action="store_true",
+                    help="skip the large-frame inference configuration (33,554,432 points @2473x1643, 16 fp16 "
+                         "channels: training draw + inference forward, reported in extra.config4_inference)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
@@ -132,6 +143,12 @@ def main() -> int:
         torch.cuda.synchronize()
         draws.append((time.perf_counter() - t0) * 1e3)
     sampler_ms = sorted(draws[1:])[len(draws[1:]) // 2]
+    with _lib.KernelTimer() as draw_timer:   # the kernels of one more draw, HIP events on the launch stream
+        sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)
+    draw_kernels = {}
+    for name, ms in draw_timer.records:
+        draw_kernels[name] = draw_kernels.get(name, 0.0) + ms
+    draw_candidates = int(sampler.last_consumed)
     sampler = ProbabilityFieldSampler(seed=0)   # the benchmark's points: the first draw of seed 0
     positions, leaf_ids = sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)
     torch.cuda.synchronize()
@@ -209,6 +226,8 @@ def main() -> int:
     # what is left of the step when the host's launch work is taken away
     graph_ms = None
     try:
+        if args.no_extras:
+            raise RuntimeError("skipped (--no-extras)")
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
@@ -229,15 +248,19 @@ def main() -> int:
     # the step that closes the loop: leaf statistics from this frame's leaf indices and blending weights
     from inpc_amd import update_probability_field
 
-    field_weights = weights.clone()
-    field_scores = torch.zeros_like(weights)
-    field_ms = time_calls(lambda: update_probability_field(field_weights, field_scores, leaf_ids, blending_weights),
-                          args.steps)
+    field_ms = None
+    if not args.no_extras:
+        field_weights = weights.clone()
+        field_scores = torch.zeros_like(weights)
+        field_ms = time_calls(lambda: update_probability_field(field_weights, field_scores, leaf_ids, blending_weights),
+                              args.steps)
 
     # the same points through the Gaussian footprint (the reference's other rasterizer mode), 8x8 tiles as in the
     # reference: a side measurement, not part of `value`
     gaussian = None
     try:
+        if args.no_extras:
+            raise RuntimeError("skipped (--no-extras)")
         gcfg = _lib.GaussianConfig(_lib.RasterConfig(n, 8, channels, _lib.FEAT_DIRECT_F32, 0,
                                                      _lib.make_camera(hv.camera)), 0.0, 3.0, 0, 0)
         glayout = _lib.GaussianLayout()
@@ -288,6 +311,8 @@ def main() -> int:
     # (forward + backward including the SH gradient), both footprints with the tile size the layer picks
     reference_shape = None
     try:
+        if args.no_extras:
+            raise RuntimeError("skipped (--no-extras)")
         from inpc_amd import INPCRasterizer
 
         sh = (torch.randn((n, 36), generator=gen, device=device) * 0.2).half().requires_grad_(True)
@@ -316,24 +341,25 @@ def main() -> int:
     for name, ms in timer.records:
         tot, cnt = per_kernel.get(name, (0.0, 0))
         per_kernel[name] = (tot + ms, cnt + 1)
-    depth_passes = max(per_kernel.get("raster_depth_sort", (0, 0))[1] // args.steps, 1)
-    tile_passes = max(per_kernel.get("raster_tile_sort", (0, 0))[1] // args.steps, 1)
     pixels = H * W
     kernels = []
     for name, (tot, cnt) in sorted(per_kernel.items(), key=lambda kv: -kv[1][0]):
         avg_ms = tot / cnt
-        alg = algorithmic_bytes(name, n, n_visible, n_instances, pixels, channels, depth_passes, tile_passes,
-                                layout.end_bit)
-        kernels.append({"kernel": name, "launches_per_step": cnt / args.steps, "avg_ms": round(avg_ms, 5),
+        launches = cnt / args.steps
+        alg = algorithmic_bytes(name, n, n_visible, n_instances, pixels, channels, layout.end_bit) / launches
+        kernels.append({"kernel": name, "launches_per_step": launches, "avg_ms": round(avg_ms, 5),
                         "ms_per_step": round(tot / args.steps, 5),
-                        "algorithmic_GBps": round(alg / (avg_ms * 1e-3) / 1e9, 1) if avg_ms > 0 else None})
+                        "algorithmic_GBps": round(alg / (avg_ms * 1e-3) / 1e9, 1) if alg > 0 and avg_ms > 0 else None})
     dominant = kernels[0]
-    dom_alg = algorithmic_bytes(dominant["kernel"], n, n_visible, n_instances, pixels, channels, depth_passes,
-                                tile_passes, layout.end_bit)
+    dom_alg = algorithmic_bytes(dominant["kernel"], n, n_visible, n_instances, pixels, channels, layout.end_bit) \
+        / dominant["launches_per_step"]
     achieved = dom_alg / (dominant["avg_ms"] * 1e-3) / 1e9
+    traffic = measured_traffic(dominant["kernel"], args.workload)
     roofline = {"bound": "hbm", "kernel": dominant["kernel"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": measured_traffic(dominant["kernel"], args.workload),
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_source": None if traffic is None else
+                f"{traffic_file(args.workload).relative_to(ROOT)} (profiler counters of an earlier run of this "
+                "command, not measured by this run)",
                 "algorithmic_bytes_per_launch": dom_alg, "avg_launch_ms": dominant["avg_ms"]}
     fwd_bytes, bwd_bytes = step_algorithmic_bytes(n, n_visible, n_instances, pixels, channels, layout.end_bit)
     step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
@@ -353,19 +379,30 @@ def main() -> int:
         opac_h = opacities[:n_cpu].cpu().numpy()
         gi_h, ga_h = grad_image.cpu().numpy(), grad_alpha.cpu().numpy()
         O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)  # warm-up
-        reps, spent = 0, 0.0
-        while spent < args.cpu_seconds and reps < 1000:
-            t = O.now()
-            O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)
-            spent += O.now() - t
-            reps += 1
-        cpu = {"value": round(n_cpu * reps / spent / 1e6, 3), "unit": "Mpoints/s", "cores": O.num_threads(),
+
+        def cpu_leg(seconds):
+            reps, spent = 0, 0.0
+            while spent < seconds and reps < 1000:
+                t = O.now()
+                O.raster_forward_backward(ocfg, pos_h, feat_h, opac_h, hv.w2c, gi_h, ga_h)
+                spent += O.now() - t
+                reps += 1
+            return reps, spent
+
+        all_threads = O.num_threads()
+        reps, spent = cpu_leg(args.cpu_seconds)
+        O.set_num_threads(1)
+        reps1, spent1 = cpu_leg(args.cpu_seconds / 2)
+        O.set_num_threads(all_threads)
+        cpu = {"value": round(n_cpu * reps / spent / 1e6, 3), "unit": "Mpoints/s", "cores": all_threads,
                "kind": "port",
                "sample": f"first {n_cpu} of the {n} points, same camera/image/channels/tiles, forward+backward, "
-                         f"{reps} repetitions, {spent:.1f} s"}
+                         f"{reps} repetitions, {spent:.1f} s",
+               "single_thread": {"value": round(n_cpu * reps1 / spent1 / 1e6, 3), "unit": "Mpoints/s", "cores": 1,
+                                 "sample": f"same sample, {reps1} repetitions, {spent1:.1f} s"}}
 
     config4 = None
-    if args.with_config4:
+    if not args.no_config4 and not args.no_extras and args.workload.startswith("config3"):
         # free the training workload first: this one needs about 12 GB
         del workspace, image, alpha, blending_weights, grad_features, grad_opacities, features, opacities
         torch.cuda.empty_cache()
@@ -393,6 +430,22 @@ def main() -> int:
             config4[f"{label}_forward_ms"] = round(ms, 3)
             config4[f"{label}_Mpoints_per_s"] = round(n4 / (ms * 1e-3) / 1e6, 1)
 
+    # the sampler (training draw of the same n points): 32 B per leaf (20 in, 4 out, 8 scan) and 32 B per candidate
+    # (16 B of leaf data gathered, 12 B position + 4 B index written); the CDF probes are cache traffic and not counted
+    draw_kernel_ms = sum(draw_kernels.values())
+    draw_bytes = 32.0 * wl["leaves"] + 32.0 * draw_candidates
+    sampler_extra = {
+        "workload": f"training draw of {n} samples from {wl['leaves']} leaves (level {wl['level']}), same camera",
+        "call_ms": round(sampler_ms, 3), "kernels_ms": round(draw_kernel_ms, 4),
+        "candidates": draw_candidates,
+        "Msamples_per_s": round(n / (sampler_ms * 1e-3) / 1e6, 1),
+        "Msamples_per_s_kernels_only": round(n / (draw_kernel_ms * 1e-3) / 1e6, 1) if draw_kernel_ms > 0 else None,
+        "algorithmic_bytes": draw_bytes,
+        "algorithmic_GBps": round(draw_bytes / (draw_kernel_ms * 1e-3) / 1e9, 1) if draw_kernel_ms > 0 else None,
+        "hbm_frac": round(draw_bytes / (draw_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if draw_kernel_ms > 0 else None,
+        "kernel_ms": {k: round(v, 4) for k, v in sorted(draw_kernels.items(), key=lambda kv: -kv[1])},
+    }
+
     out = {
         "metric": "Mpoints/s, rasterizer fwd+bwd, 8M pts @1237x822 (ms/frame in ms_per_step)",
         "value": round(n / (ms_per_step * 1e-3) / 1e6, 2),
@@ -412,8 +465,9 @@ def main() -> int:
         "cpu_baseline": cpu,
         "extra": {
             "forward_ms": round(fwd_ms, 4), "backward_ms": round(bwd_ms, 4),
-            "graph_replay_ms": None if graph_ms is None else round(graph_ms, 4), "sampler_training_draw_ms": round(sampler_ms, 3), "sampler_candidates": sampler.last_consumed,
-            "field_update_ms": round(field_ms, 4),
+            "graph_replay_ms": None if graph_ms is None else round(graph_ms, 4),
+            "sampler": sampler_extra,
+            "field_update_ms": None if field_ms is None else round(field_ms, 4),
             "gaussian_footprint": gaussian,
             "sh36_autograd_step": reference_shape,
             "config4_inference": config4,
