@@ -49,8 +49,10 @@ def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, end_bit):
     table = {
         # the count/scan in front of the instance expansion
         "raster_bin_count": v * 20,
-        # point in (xyz, features, opacity), record + key/index out, instance emission (expansion reads + 6 B each)
-        "raster_preprocess": n * (16 + F) + v * (R + 8 + 16) + i * 6,
+        # point in (xyz, features, opacity), record out
+        "raster_records": n * (16 + F) + v * R,
+        # key/index out, instance emission (expansion reads + 6 B each)
+        "raster_bin_fill": v * (8 + 16) + i * 6,
         # what the reference structure spends on ordering: depth sort of the visible points (4 B histogram read +
         # 4 passes x 16 B), tile sort of the instances and the range scan
         "raster_tile_sort": v * 68 + i * (2 + 12 * ((end_bit + 7) // 8) + 2),

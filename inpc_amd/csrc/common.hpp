@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 
 #include "../../include/inpc_hip.h"
 
@@ -20,6 +21,20 @@ int fail(int code, const char* fmt, ...);
 // Optional per-launch timing (HIP events on the launch stream), see inpc_timing_enable().
 void timing_begin(const char* name, hipStream_t stream);
 void timing_end(hipStream_t stream);
+bool timing_enabled();   // for the calling thread
+
+// A second stream of the current device for work that does not depend on what the caller's stream is doing at the
+// moment, with the two events that tie it to the caller's stream: `fork` is recorded on the caller's stream and
+// awaited by `stream`, `join` the other way round. Created on first use (non-blocking, default priority) and kept
+// until the process ends; nullptr when it does not exist and `may_create` is false or it cannot be created (the caller
+// then keeps the work on its own stream). Record `fork` and make `stream` wait for it under side_lane_mutex(): the
+// lane is shared by all calls on the device.
+struct SideLane {
+    hipStream_t stream;
+    hipEvent_t fork, join;
+};
+SideLane* side_lane(bool may_create);
+std::mutex& side_lane_mutex();
 
 #define INPC_HIP_CHECK(expr)                                                                        \
     do {                                                                                            \

@@ -1,14 +1,16 @@
 // raster.hip — tile-based differentiable bilinear point rasterizer for gfx950.
 //
-// Pipeline (all on the caller's stream, counts stay on the device):
+// Pipeline (on the caller's stream but for k_records; counts stay on the device):
 //   k_bin_count      project every point; per chunk of points count the instances (point, touched tile) per tile
 //   k_bin_offsets    per tile: exclusive prefix of the counts over the chunks
 //   k_bin_scan       exclusive scan over the tiles: [begin, end) of every tile's instances
 //                    (B/rasterization/src/bilinear/kernels.cu:222-239); decides whether they fit the buffers
 //   k_tile_order     schedule of the per-tile blocks: tiles with the longest instance lists first
-//   k_preprocess     project, cull, tile bounds, depth key; the blend record of a drawn point (footprint weights,
-//                    opacity, view features) goes to the point's place in the record array, a (depth key, point)
-//                    pair per instance into the bin of its tile (kernels.cu:11-84,106-184,198-220)
+//   k_bin_fill       project, cull, tile bounds, depth key: a (depth key, point) pair per instance into the bin of
+//                    its tile (kernels.cu:11-84,198-220)
+//   k_records        (on a second stream, beside k_bin_fill and the tile sort) the blend record of a drawn point:
+//                    footprint weights, opacity, view features, at the point's place in the record array
+//                    (kernels.cu:11-84,106-184)
 //   tilesort.hpp     one block per tile sorts its bin by (depth key, point index) inside LDS: the order the
 //                    reference gets from its two device-wide sorts (forward.cu:91-141)
 //   blend.hpp        k_blend_forward: front-to-back bilinear 2x2 splat blend, one block per tile
@@ -197,10 +199,10 @@ __device__ __forceinline__ AxisWeights axis_weights(float s) {
 }
 
 // ---- instance bins ----------------------------------------------------------------------------------------------
-// The points are cut into kBinBlocks contiguous chunks, one per block, the same way in k_bin_count and in
-// k_preprocess. k_bin_count leaves, per (chunk, tile), the number of instances the chunk's points have in the
+// The points are cut into kBinBlocks contiguous chunks, one per block, the same way in k_bin_count,
+// k_bin_fill and k_records. k_bin_count leaves, per (chunk, tile), the number of instances the chunk's points have in the
 // tile; k_bin_offsets turns that table into the exclusive prefix over the chunks of every tile and k_bin_scan
-// into the start of every tile's bin. k_preprocess then hands out bin slots from LDS cursors seeded with
+// into the start of every tile's bin. k_bin_fill then hands out bin slots from LDS cursors seeded with
 // bin_start[tile] + prefix[chunk][tile]: no global atomic anywhere (they run at about 10 G/s on this machine,
 // far below what 8M points need).
 //
@@ -384,7 +386,7 @@ __global__ void __launch_bounds__(kScanBlock)
     if (tid < n_chunks) split_base[tid] = make_uint2(run[1], run[2]);
     if (tid == 0) {
         bin_start[n_tiles] = overflow ? 0u : total[0];
-        counters[kCntVisible] = 0u;   // counted by k_preprocess
+        counters[kCntVisible] = 0u;   // counted by k_bin_fill
         counters[kCntError] = 0u;
         counters[kCntInstances] = total[0];
         counters[kCntSplit] = overflow ? 0u : total[1];   // no list entry is written when nothing is drawn
@@ -412,22 +414,19 @@ struct SplitOut {
     uint8_t* row_flags;
 };
 
-template <int T, int FMODE, int C, bool WIDE>
+// Preprocess is two kernels that do not depend on each other: k_bin_fill drops the (depth key, point) pairs into
+// the tiles' bins, which is all the tile sort needs; k_records writes the blend records. The host runs the second
+// beside the first and the tile sort (which leaves the memory system idle) on a stream of its own.
+template <int T, bool WIDE>
 __global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
-    k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
-                 const float* __restrict__ opacities, const float* __restrict__ w2c,
-                 const float* __restrict__ cam_position, char* __restrict__ records,
-                 const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start,
-                 uint64_t* __restrict__ pairs, float* __restrict__ blending_weights, SplitOut split,
-                 float4* __restrict__ debug_geometry, uint32_t* counters, Geometry g) {
+    k_bin_fill(const float* __restrict__ positions, const float* __restrict__ w2c, const uint32_t* __restrict__ table,
+               const uint32_t* __restrict__ bin_start, uint64_t* __restrict__ pairs, uint32_t* counters, Geometry g) {
     constexpr int kThreads = WIDE ? kBinThreadsWide : kBinThreads;
-    extern __shared__ __align__(16) uint32_t s_dyn[];
-    float4* s_stage = (float4*)s_dyn;                                           // record staging, 64 rows per wave
-    uint32_t* s_cursor = s_dyn + PreprocessShape<FMODE, C>::stage_bytes(kThreads) / 4;   // n_tiles (WIDE: 16-bit halves)
+    extern __shared__ __align__(16) uint32_t s_cursor[];   // n_tiles (WIDE: 16-bit halves)
     __shared__ uint32_t s_visible;
-    __shared__ uint32_t s_split, s_rows;   // next list entry / gradient row for a point of this chunk
     const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then no instance is stored
-    const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;   // instances of the chunks before, per tile
+    const uint32_t chunk_id = blockIdx.x;
+    const uint32_t* row = table + (size_t)chunk_id * g.n_tiles;   // instances of the chunks before, per tile
     if (WIDE) {
         for (uint32_t t = threadIdx.x; t < (g.n_tiles + 1u) / 2u; t += kThreads) s_cursor[t] = 0u;
     } else {
@@ -438,15 +437,61 @@ __global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
         if (WIDE) return bin_start[tile] + row[tile] + packed_counter_next(s_cursor, tile);
         return atomicAdd(&s_cursor[tile], 1u);
     };
+    if (threadIdx.x == 0) s_visible = 0u;
+    __syncthreads();
+    const ViewRows m = load_view_rows(w2c);
+    uint32_t my_visible = 0;
+    const uint32_t chunk = bin_chunk_size(g.n, g.n_chunks);
+    const uint32_t begin = min(chunk_id * chunk, g.n), end = min(begin + chunk, g.n);
+    constexpr int kUnroll = 4;   // points per thread and round, their loads issued together
+    for (uint32_t base = begin; base < end; base += kUnroll * kThreads) {
+        float px[kUnroll], py[kUnroll], pz[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            // a thread behind the end reads the chunk's first point and drops it
+            const uint32_t at = base + u * kThreads + threadIdx.x;
+            const size_t i = at < end ? at : begin;
+            px[u] = positions[3 * i];
+            py[u] = positions[3 * i + 1];
+            pz[u] = positions[3 * i + 2];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t i = base + u * kThreads + threadIdx.x;
+            if (i >= end) continue;
+            const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
+            if (p.info == 0u) continue;
+            my_visible += 1u;
+            const uint64_t pair = ((uint64_t)(__float_as_uint(p.depth) - g.key_bias) << 32) | (uint64_t)i;
+            if (!overflow) for_each_tile(p.info, g.gw, [&](uint32_t tile) { pairs[take_slot(tile)] = pair; });
+        }
+    }
+    // block total -> one global atomic
+    for (int s = 32; s > 0; s >>= 1) my_visible += __shfl_down(my_visible, s, 64);
+    if ((threadIdx.x & 63u) == 0u) atomicAdd(&s_visible, my_visible);
+    __syncthreads();
+    if (threadIdx.x == 0 && s_visible) atomicAdd(&counters[kCntVisible], s_visible);
+}
+
+template <int T, int FMODE, int C>
+__global__ void __launch_bounds__(kBinThreads)
+    k_records(const float* __restrict__ positions, const void* __restrict__ features,
+              const float* __restrict__ opacities, const float* __restrict__ w2c,
+              const float* __restrict__ cam_position, char* __restrict__ records,
+              float* __restrict__ blending_weights, SplitOut split, float4* __restrict__ debug_geometry,
+              const uint32_t* __restrict__ counters, Geometry g) {
+    constexpr int kThreads = kBinThreads;
+    extern __shared__ __align__(16) uint32_t s_dyn[];
+    float4* s_stage = (float4*)s_dyn;      // record staging, 64 rows per wave
+    __shared__ uint32_t s_split, s_rows;   // next list entry / gradient row for a point of this chunk
+    const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then nothing is drawn
     if (threadIdx.x == 0) {
-        s_visible = 0u;
         const uint2 first = split.base ? split.base[blockIdx.x] : make_uint2(0u, 0u);
         s_split = first.x;
         s_rows = first.y;
     }
     __syncthreads();
     const ViewRows m = load_view_rows(w2c);
-    uint32_t my_visible = 0;
     const uint32_t chunk = bin_chunk_size(g.n, g.n_chunks);
     const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
     // kUnroll points per thread and round, their loads issued together. A record leaves the block through LDS:
@@ -495,9 +540,6 @@ __global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
                 const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
                 drawn = p.info != 0u;
                 if (drawn) {
-                    my_visible += 1u;
-                    const uint64_t pair = ((uint64_t)(__float_as_uint(p.depth) - g.key_bias) << 32) | (uint64_t)i;
-                    if (!overflow) for_each_tile(p.info, g.gw, [&](uint32_t tile) { pairs[take_slot(tile)] = pair; });
                     float4* rec = stage + lane * kRow;
                     float opacity = op[u];
 #pragma unroll
@@ -558,11 +600,6 @@ __global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
             wave_sync();
         }
     }
-    // block total -> one global atomic
-    for (int s = 32; s > 0; s >>= 1) my_visible += __shfl_down(my_visible, s, 64);
-    if ((threadIdx.x & 63u) == 0u) atomicAdd(&s_visible, my_visible);
-    __syncthreads();
-    if (threadIdx.x == 0 && s_visible) atomicAdd(&counters[kCntVisible], s_visible);
 }
 
 // ---- tile schedule -----------------------------------------------------------------------------------------------
@@ -850,29 +887,35 @@ int launch_bin_count(const Layout& L, const float* positions, const float* w2c, 
     return INPC_OK;
 }
 
+template <int T>
+int launch_bin_fill(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
+    const uint32_t* table = at<uint32_t>(ws, L.bin_table);
+    const uint32_t* bin_start = at<uint32_t>(ws, L.pub.bin_start);
+    if (L.wide) {
+        const size_t lds = (size_t)(L.geo.n_tiles + 1) / 2 * 4;
+        INPC_LAUNCH_LDS("raster_bin_fill", (k_bin_fill<T, true>), dim3(L.geo.n_chunks), dim3(kBinThreadsWide), lds, stream,
+                        positions, w2c, table, bin_start, at<uint64_t>(ws, L.pairs), at<uint32_t>(ws, L.pub.counters), L.geo);
+    } else {
+        const size_t lds = (size_t)L.geo.n_tiles * 4;
+        INPC_LAUNCH_LDS("raster_bin_fill", (k_bin_fill<T, false>), dim3(L.geo.n_chunks), dim3(kBinThreads), lds, stream,
+                        positions, w2c, table, bin_start, at<uint64_t>(ws, L.pairs), at<uint32_t>(ws, L.pub.counters), L.geo);
+    }
+    return INPC_OK;
+}
+
 template <int T, int FMODE, int C>
-int launch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
-                      const float* w2c, const float* cam_position, float* blending_weights, void* ws,
-                      hipStream_t stream) {
+int launch_records(const Layout& L, const float* positions, const void* features, const float* opacities,
+                   const float* w2c, const float* cam_position, float* blending_weights, void* ws, hipStream_t stream) {
     if (L.pub.record_stride != PreprocessShape<FMODE, C>::kStrideWords * 16u)
-        return fail(INPC_E_UNSUPPORTED, "record stride %u does not match the preprocess kernel", L.pub.record_stride);
+        return fail(INPC_E_UNSUPPORTED, "record stride %u does not match the record kernel", L.pub.record_stride);
     SplitOut split{nullptr, nullptr, nullptr};
     if (L.split_list) split = SplitOut{at<uint2>(ws, L.split_base), at<uint2>(ws, L.split_list), at<uint8_t>(ws, L.row_flags)};
     char* records = at<char>(ws, L.pub.point_record);
-    const uint32_t* table = at<uint32_t>(ws, L.bin_table);
-    const uint32_t* bin_start = at<uint32_t>(ws, L.pub.bin_start);
     float4* debug = L.pub.debug_geometry ? at<float4>(ws, L.pub.debug_geometry) : (float4*)nullptr;
-    if (L.wide) {
-        const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kBinThreadsWide) + (size_t)(L.geo.n_tiles + 1) / 2 * 4;
-        INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C, true>), dim3(L.geo.n_chunks), dim3(kBinThreadsWide),
-                        lds, stream, positions, features, opacities, w2c, cam_position, records, table, bin_start,
-                        at<uint64_t>(ws, L.pairs), blending_weights, split, debug, at<uint32_t>(ws, L.pub.counters), L.geo);
-    } else {
-        const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kBinThreads) + (size_t)L.geo.n_tiles * 4;
-        INPC_LAUNCH_LDS("raster_preprocess", (k_preprocess<T, FMODE, C, false>), dim3(L.geo.n_chunks), dim3(kBinThreads),
-                        lds, stream, positions, features, opacities, w2c, cam_position, records, table, bin_start,
-                        at<uint64_t>(ws, L.pairs), blending_weights, split, debug, at<uint32_t>(ws, L.pub.counters), L.geo);
-    }
+    const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kBinThreads);
+    INPC_LAUNCH_LDS("raster_records", (k_records<T, FMODE, C>), dim3(L.geo.n_chunks), dim3(kBinThreads), lds, stream,
+                    positions, features, opacities, w2c, cam_position, records, blending_weights, split, debug,
+                    (const uint32_t*)at<uint32_t>(ws, L.pub.counters), L.geo);
     return INPC_OK;
 }
 
@@ -941,10 +984,10 @@ int dispatch_blend_backward(const Layout& L, const float* grad_image, const floa
     return fail(INPC_E_UNSUPPORTED, "raster: unsupported backward configuration");
 }
 
-int dispatch_preprocess(const Layout& L, const float* positions, const void* features, const float* opacities,
-                        const float* w2c, const float* cam_position, float* bw, void* ws, hipStream_t stream) {
+int dispatch_records(const Layout& L, const float* positions, const void* features, const float* opacities,
+                     const float* w2c, const float* cam_position, float* bw, void* ws, hipStream_t stream) {
 #define CALL_PRE(T_, FM_, C_) \
-    launch_preprocess<T_, FM_, C_>(L, positions, features, opacities, w2c, cam_position, bw, ws, stream)
+    launch_records<T_, FM_, C_>(L, positions, features, opacities, w2c, cam_position, bw, ws, stream)
 #define CALL_PRE_C(T_, FM_)                    \
     do {                                       \
         if (L.C == 4) return CALL_PRE(T_, FM_, 4);   \
@@ -967,7 +1010,7 @@ int dispatch_preprocess(const Layout& L, const float* positions, const void* fea
     }
 #undef CALL_PRE_C
 #undef CALL_PRE
-    return fail(INPC_E_UNSUPPORTED, "raster: unsupported preprocess configuration");
+    return fail(INPC_E_UNSUPPORTED, "raster: unsupported record configuration");
 }
 
 // ---- Gaussian footprint: workspace layout and launches --------------------------------------------------------
@@ -1271,8 +1314,48 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
     INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
                 (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
     if (L.geo.n > 0) {
-        rc = dispatch_preprocess(L, positions, features, opacities, w2c, cam_position,
-                                 L.inference ? nullptr : blending_weights, ws, stream);
+        rc = L.T == 8 ? launch_bin_fill<8>(L, positions, w2c, ws, stream) : launch_bin_fill<16>(L, positions, w2c, ws, stream);
+        if (rc != INPC_OK) return rc;
+        // The records are not needed before the blend, and writing them is bound by memory while the tile sort hardly
+        // touches memory: they are written on the device's second stream, beside the tile sort (not beside
+        // k_bin_fill, which is bound by memory itself). With the
+        // per-launch timing on, everything stays on the caller's stream, so that each duration is that of a kernel
+        // that has the device to itself.
+        // (a stream that is being captured into a graph takes the second stream along, but the second stream is not
+        // created during a capture)
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        const bool capture_known = hipStreamIsCapturing(stream, &capture) == hipSuccess;
+        if (!capture_known) (void)hipGetLastError();
+        SideLane* lane = nullptr;
+        if (!timing_enabled() && capture_known) lane = side_lane(capture == hipStreamCaptureStatusNone);
+        hipStream_t record_stream = stream;
+        if (lane) {
+            std::lock_guard<std::mutex> lock(side_lane_mutex());
+            if (hipEventRecord(lane->fork, stream) == hipSuccess &&
+                hipStreamWaitEvent(lane->stream, lane->fork, 0) == hipSuccess) {
+                record_stream = lane->stream;
+            } else {
+                (void)hipGetLastError();
+                lane = nullptr;
+            }
+        }
+        rc = dispatch_records(L, positions, features, opacities, w2c, cam_position,
+                              L.inference ? nullptr : blending_weights, ws, record_stream);
+        // the caller's stream takes the second stream's work in again behind the tile sort, or wherever this
+        // function is left before
+        struct Join {
+            hipStream_t stream;
+            SideLane* lane;
+            ~Join() {
+                if (lane) (void)hipStreamWaitEvent(stream, lane->join, 0);
+            }
+        } join{stream, lane};
+        if (lane && hipEventRecord(lane->join, lane->stream) != hipSuccess) {
+            join.lane = nullptr;
+            (void)hipStreamSynchronize(lane->stream);   // no event to wait for: wait on the host
+            return fail(INPC_E_HIP, "inpc_raster_forward: cannot record on the record stream: %s",
+                        hipGetErrorString(hipGetLastError()));
+        }
         if (rc != INPC_OK) return rc;
         // tiles of more than tilesort::kSmallTile instances, then the others with small blocks
         INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort<tilesort::kLargeThreads>, dim3(L.geo.n_tiles),

@@ -47,6 +47,38 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+bool timing_enabled() { return g_timing_on; }
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_lane_mutex;
+SideLane g_lanes[kMaxDevices] = {};
+bool g_lane_ready[kMaxDevices] = {};
+}  // namespace
+
+std::mutex& side_lane_mutex() { return g_lane_mutex; }
+
+SideLane* side_lane(bool may_create) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_lane_mutex);
+    if (g_lane_ready[device]) return &g_lanes[device];
+    if (!may_create) return nullptr;
+    SideLane lane{nullptr, nullptr, nullptr};
+    // no timing data in the events: they only order the two streams
+    if (hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&lane.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&lane.join, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();   // the failure is handled here: the caller works without the lane
+        if (lane.fork) (void)hipEventDestroy(lane.fork);
+        if (lane.stream) (void)hipStreamDestroy(lane.stream);
+        return nullptr;
+    }
+    g_lanes[device] = lane;
+    g_lane_ready[device] = true;
+    return &g_lanes[device];
+}
+
 void timing_begin(const char* name, hipStream_t stream) {
     if (!g_timing_on) return;
     g_open.name = name;
