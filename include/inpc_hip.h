@@ -264,7 +264,10 @@ int inpc_raster_layout_query(const inpc_raster_config* cfg, inpc_raster_layout* 
  *   INPC_FEAT_RAW37_F16); w2c (4,4) f32; cam_position (3,) f32 (SH modes only);
  *   image (C,H,W) f32; alpha (1,H,W) f32;
  *   blending_weights (N,) f32 (training) or NULL; depth_image (1,H,W) f32 (inference) or NULL.
- * The workspace is the saved state the backward pass needs. No host synchronisation. */
+ * The workspace is the saved state the backward pass needs. No host synchronisation. Everything is enqueued on
+ * `stream` except the kernel that writes the blend records, which runs beside the tile sort on a second stream of
+ * the device (created by the library on first use, default priority); `stream` waits for it before the blend, so
+ * to the caller the call is ordered on `stream` like any other. */
 int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, const void* features,
                         const float* opacities, const float* w2c, const float* cam_position,
                         float* image, float* alpha, float* blending_weights, float* depth_image,

@@ -48,7 +48,8 @@ __device__ __forceinline__ uint32_t dpp_take(uint32_t old, uint32_t v) {
 }
 
 // T_i = (...((t_in * m_0) * m_1)...) * m_i for the lanes i < n, multiplied strictly left to right: the result is
-// bit-identical to a sequential walk. Every step, every lane takes its left neighbour's value (lane 0: t_in) times
+// bit-identical to a sequential walk, which the early-out test against the transmittance threshold needs
+// (a product taken in tree order may land on the other side of the threshold). Every step, every lane takes its left neighbour's value (lane 0: t_in) times
 // its own factor: after step s the lanes 0..s hold their final value, and computing a final value again from a
 // final neighbour reproduces it. One multiply per step, no LDS. (Steps beyond n only recompute final values, so
 // the loop runs in unrolled groups of eight.)
@@ -59,29 +60,6 @@ __device__ __forceinline__ float wave_sequential_product(float m, float t_in, ui
         for (int u = 0; u < 8; ++u) x = dpp_take<kDppWaveShr1, 0xf>(t_in, x) * m;
     }
     return x;
-}
-
-// m_0 * ... * m_i in every lane i, multiplied in tree order: six steps.
-__device__ __forceinline__ float wave_inclusive_product(float v) {
-    v *= dpp_take<kDppRowShr1, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowShr2, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowShr4, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowShr8, 0xf>(1.0f, v);
-    v *= dpp_take<kDppRowBcast15, 0xa>(1.0f, v);
-    v *= dpp_take<kDppRowBcast31, 0xc>(1.0f, v);
-    return v;
-}
-
-// Transmittance behind each of the n <= 64 fragments of a list (lane i: fragment i, m = 1 - alpha), t_in in front of
-// the first. The walk ends where the transmittance falls below kTransmittanceThreshold, and a product taken in
-// another order than the sequential walk's may land on the other side of the threshold: the tree-order products
-// (at most 64 roundings apart from the sequential ones, i.e. 4e-6 relative) are used only when none of them comes
-// closer to the threshold than 1e-5 relative; otherwise the sequential products are computed.
-__device__ __forceinline__ float wave_transmittance(float m, float t_in, uint32_t n) {
-    const float t = t_in * wave_inclusive_product(m);
-    const bool close = fabsf(t - kTransmittanceThreshold) < kTransmittanceThreshold * 1e-5f;
-    if (__ballot(close) == 0ull) return t;
-    return wave_sequential_product(m, t_in, n);
 }
 
 __device__ __forceinline__ float wave_inclusive_sum(float v) {
@@ -561,7 +539,7 @@ __global__ void __launch_bounds__(T* T)
                     float2 e = make_float2(0.0f, 0.0f);
                     if (here) e = qs.fragment[pos];
                     const float a = e.x;
-                    const float t_after = wave_transmittance(1.0f - a, p_T, min(64u, p_count - base));
+                    const float t_after = wave_sequential_product(1.0f - a, p_T, min(64u, p_count - base));
                     const float t_before = wave_previous(t_after, p_T);
                     const bool reached = here && !(t_before < kTransmittanceThreshold);
                     const float bw = reached ? t_before * a : 0.0f;
@@ -831,7 +809,7 @@ __global__ void __launch_bounds__(T* T)
                     float2 e = make_float2(0.0f, 0.0f);
                     if (here) e = qs.fragment[pos];
                     const float a = e.x, sd = e.y;
-                    const float t_after = wave_transmittance(1.0f - a, p_T, min(64u, p_count - base));
+                    const float t_after = wave_sequential_product(1.0f - a, p_T, min(64u, p_count - base));
                     const float t_before = wave_previous(t_after, p_T);
                     const bool reached = here && !(t_before < kTransmittanceThreshold);
                     const float bw = reached ? t_before * a : 0.0f;
