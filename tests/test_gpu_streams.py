@@ -97,3 +97,58 @@ def test_training_draws_on_two_streams_at_once(gpu, oracle):
                                                       oct.initial_size, oracle.Pcg32(11 + k), n)
         np.testing.assert_array_equal(ids.cpu().numpy(), ids_ref.astype(np.int64))
         np.testing.assert_array_equal(pos.cpu().numpy().view(np.uint32), pos_ref.view(np.uint32))
+
+
+def test_bilinear_steps_from_four_host_threads_share_the_second_stream(gpu, oracle):
+    """The bilinear forward pass writes its records on a second stream that all calls on the device share: four
+    host threads, a stream and a workspace each, several steps each, all in flight together."""
+    import threading
+
+    n, channels, steps = 150000, 8, 4
+    cases = []
+    for k in range(4):
+        hv = synthetic.rotated_camera(320 + 16 * k, 240, 300.0, 2.6, 0.07 * k, -0.04 * k)
+        pos = synthetic.cube_points(n, 1.8, 70 + k)
+        feats, opac = synthetic.point_attributes(n, channels, "normal", 80 + k)
+        rng = np.random.default_rng(90 + k)
+        gi = rng.normal(0, 1e-2, (channels, hv.camera.height, hv.camera.width)).astype(np.float32)
+        ga = rng.normal(0, 1e-2, (1, hv.camera.height, hv.camera.width)).astype(np.float32)
+        cases.append((hv, pos, feats, opac, gi, ga))
+    H.RasterRun(*cases[0][:4], 16, channels, _lib.FEAT_DIRECT_F32).forward()   # the second stream exists from here on
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in cases]
+    results = [None] * len(cases)
+    errors = []
+
+    def work(k):
+        try:
+            hv, pos, feats, opac, gi, ga = cases[k]
+            with torch.cuda.stream(streams[k]):
+                run = H.RasterRun(hv, pos, feats, opac, 16 if k % 2 == 0 else 8, channels, _lib.FEAT_DIRECT_F32)
+                gi_dev, ga_dev = H.dev(gi), H.dev(ga)
+                for _ in range(steps):
+                    run.forward()
+                    grads = run.backward_async(gi_dev, ga_dev)
+                streams[k].synchronize()
+            results[k] = (run, grads)
+        except Exception as exc:   # reported by the main thread
+            errors.append((k, exc))
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for k, ((run, (gf, go)), (hv, pos, feats, opac, gi, ga)) in enumerate(zip(results, cases)):
+        tile = 16 if k % 2 == 0 else 8
+        cfg = oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32)
+        ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+        check_structure(run.debug(), ref)
+        out = run.outputs()
+        H.assert_close(out["image"], ref["image"], RTOL, 1e-5, f"image {k}")
+        H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, f"blending weights {k}")
+        gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
+        H.assert_close(gf.cpu().numpy(), gf_ref, RTOL, grad_atol(gf_ref), f"feature gradients {k}")
+        H.assert_close(go.cpu().numpy(), go_ref, RTOL, grad_atol(go_ref), f"opacity gradients {k}")
