@@ -636,17 +636,23 @@ __device__ __forceinline__ uint32_t tile_rank(const Header& h, uint32_t tile_x, 
     return (tile_y - y0) * ((h.tag & kRecordSpanX) ? 2u : 1u) + (tile_x - x0);
 }
 
-// gradient of the point = sum of its rows, in row order (the gradient buffers are zero before). All rows are
-// read whether written or not (stale rows are dropped by their flag): the reads are dense and independent.
+// gradient of the point = sum of its rows that were written, in row order (the gradient buffers are zero before). A
+// group of kGroup neighbouring lanes takes one point, lane j the j-th 16-byte word of each feature row (the last lane
+// of the group also the opacity gradients), so that a wave reads the rows of neighbouring points in whole lines; one
+// lane per point walked its rows 16 bytes at a time and fetched every line several times. All rows are read whether
+// written or not (stale rows are dropped by their flag): the reads are dense and independent.
 template <int C>
 __global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __restrict__ grad_view,
                                                      float* __restrict__ grad_opacities) {
+    constexpr uint32_t kGroup = C / 4;   // 1, 2 or 4 lanes per point
     const uint32_t n = *rows.count;
-    for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < n; s += gridDim.x * 256u) {
+    const uint32_t gtid = blockIdx.x * 256u + threadIdx.x, word = gtid % kGroup;
+    const uint32_t stride = gridDim.x * 256u / kGroup;
+    for (uint32_t s = gtid / kGroup; s < n; s += stride) {   // the lanes of a group stay together
         const uint2 entry = rows.list[s];
         const uint32_t i = entry.x & kRecordIdMask, touched = entry.x >> 28, first = entry.y;
-        const float4* row = (const float4*)(rows.features + (size_t)first * C);
-        float4 part[4][C / 4];
+        const float4* row = (const float4*)(rows.features + (size_t)first * C) + word;
+        float4 part[4];
         float part_opacity[4];
         bool written[4];
         bool any = false;
@@ -655,32 +661,30 @@ __global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __re
             const bool exists = (uint32_t)p < touched;
             written[p] = exists && rows.flags[first + (exists ? p : 0)] != 0;
             any = any || written[p];
-#pragma unroll
-            for (int q4 = 0; q4 < C / 4; ++q4)
-                part[p][q4] = exists ? row[p * (C / 4) + q4] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            part_opacity[p] = exists ? rows.opacities[first + p] : 0.0f;
+            part[p] = exists ? row[p * (C / 4)] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            part_opacity[p] = exists && word == kGroup - 1u ? rows.opacities[first + p] : 0.0f;
         }
-        if (!any) continue;
-        float4 acc[C / 4];
-#pragma unroll
-        for (int q4 = 0; q4 < C / 4; ++q4) acc[q4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (!any) continue;   // the same for all lanes of the group
+        float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         float opacity = 0.0f;
 #pragma unroll
         for (int p = 0; p < 4; ++p)
             if (written[p]) {
-                rows.flags[first + p] = 0;
-#pragma unroll
-                for (int q4 = 0; q4 < C / 4; ++q4) {
-                    acc[q4].x += part[p][q4].x;
-                    acc[q4].y += part[p][q4].y;
-                    acc[q4].z += part[p][q4].z;
-                    acc[q4].w += part[p][q4].w;
-                }
+                acc.x += part[p].x;
+                acc.y += part[p].y;
+                acc.z += part[p].z;
+                acc.w += part[p].w;
                 opacity += part_opacity[p];
             }
+        ((float4*)(grad_view + (size_t)i * C))[word] = acc;
+        if (word == kGroup - 1u) grad_opacities[i] = opacity;
+        // the flags go back to zero for the next pass; the other lanes of the group have read them: they run in
+        // lockstep with this one (same wave, same control flow)
+        if (word == 0u) {
 #pragma unroll
-        for (int q4 = 0; q4 < C / 4; ++q4) ((float4*)(grad_view + (size_t)i * C))[q4] = acc[q4];
-        grad_opacities[i] = opacity;
+            for (int p = 0; p < 4; ++p)
+                if (written[p]) rows.flags[first + p] = 0;
+        }
     }
 }
 
