@@ -132,6 +132,22 @@ struct QuadScratch {
     float2 fragment[256];            // per fragment, pixel by pixel, in depth order
 };
 
+// Block barrier that also tells whether `done` holds for every thread of the block. The waves leave their verdicts
+// in the first hit mask of their scratch, which is idle between the list building of one batch and that of the next
+// (the block barrier in front of the next list building separates the reads here from its clearing). The library's
+// __syncthreads_and keeps LDS of its own, which kept the fourth block of the 16-channel inference kernel off a CU.
+template <int T>
+__device__ __forceinline__ bool barrier_all_done(QuadScratch<T>* s_quad, bool done) {
+    constexpr int NQ = Shape<T>::NQ;
+    const bool wave_done = __ballot(done) == ~0ull;   // every wave of the block is full
+    if (__lane_id() == 0u) s_quad[threadIdx.x >> 6].hits[0][0] = wave_done ? 1ull : 0ull;
+    __syncthreads();
+    bool all = true;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) all = all && s_quad[q].hits[0][0] != 0ull;
+    return all;
+}
+
 // The record header as the kernels use it.
 struct Header {
     float wx0, wx1, wy0, wy1;   // weights of the candidate columns Lx, Lx + 1 and rows Ly, Ly + 1
@@ -579,7 +595,7 @@ __global__ void __launch_bounds__(T* T)
                 }
             }
         }
-        const bool all_done = __syncthreads_and(done) != 0;
+        const bool all_done = barrier_all_done<T>(s_quad, done);
         // ---- the gather moves on in front of the stores of the write phase
         const Header mine = g.h;
         // the backward pass reads the records of this batch in runs (a gather pulls a 128-byte line per
@@ -838,7 +854,7 @@ __global__ void __launch_bounds__(T* T)
                 }
             }
         }
-        const bool all_done = __syncthreads_and(done) != 0;
+        const bool all_done = barrier_all_done<T>(s_quad, done);
         // ---- the gather moves on in front of the stores of the write phase (see the forward kernel)
         const Header mine = g.h;
         advance_ordered<T, C>(g, ordered_records, begin, range.y);
