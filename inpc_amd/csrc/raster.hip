@@ -5,7 +5,7 @@
 //   k_bin_offsets    per tile: exclusive prefix of the counts over the chunks
 //   k_bin_scan       exclusive scan over the tiles: [begin, end) of every tile's instances
 //                    (B/rasterization/src/bilinear/kernels.cu:222-239); decides whether they fit the buffers
-//   k_tile_order     schedule of the per-tile blocks: tiles with the longest instance lists first
+//                    and the schedule of the per-tile blocks: tiles with the longest instance lists first
 //   k_bin_fill       project, cull, tile bounds, depth key: a (depth key, point) pair per instance into the bin of
 //                    its tile (kernels.cu:11-84,198-220)
 //   k_records        (on a second stream, beside k_bin_fill and the tile sort) the blend record of a drawn point:
@@ -339,58 +339,147 @@ __global__ void __launch_bounds__(kOffsetWaves * kWave) k_bin_offsets(uint32_t* 
 // (forward.cu:52). split_base[c] = {points that touch several tiles, their instances} in the chunks before c.
 // When the instances or the gradient rows exceed the buffers, every bin is left empty and the overflow counter set:
 // the later kernels then draw nothing.
+// order[] = the schedule of the per-tile blocks of the sort and blend kernels: longest instance list first, so that
+// the few very long tiles do not start last and run on alone. The order only affects scheduling, not results (tiles
+// are independent); ties inside a bucket of 64 instances are in no particular order.
+// The tiles go through LDS in segments of kScanSegment, so that every access to memory is coalesced and the time
+// does not grow with the serial part of a thread (65,536 tiles are 16 segments).
 constexpr int kScanBlock = 1024;
+constexpr int kScanPer = 4;                            // consecutive tiles of a thread in a segment
+constexpr int kScanSegment = kScanBlock * kScanPer;
+constexpr int kOrderBuckets = 4096;
 static_assert(kBinBlocksWide <= kScanBlock, "one thread per chunk in k_bin_scan");
-__global__ void __launch_bounds__(kScanBlock)
-    k_bin_scan(const uint32_t* __restrict__ bin_count, uint32_t* __restrict__ bin_start, uint2* __restrict__ ranges,
-               const uint2* __restrict__ split_count, uint2* __restrict__ split_base, uint32_t* __restrict__ counters,
-               uint32_t n_tiles, uint32_t n_chunks, uint32_t capacity, uint32_t row_capacity) {
-    __shared__ uint32_t s_wave[3][kScanBlock / kWave];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t per = (n_tiles + kScanBlock - 1) / kScanBlock;
-    const uint32_t begin = min(tid * per, n_tiles), end = min(begin + per, n_tiles);
-    uint32_t mine[3] = {0u, 0u, 0u};
-    for (uint32_t t = begin; t < end; ++t) mine[0] += bin_count[t];
-    if (tid < n_chunks) {
-        const uint2 c = split_count[tid];
-        mine[1] = c.x;
-        mine[2] = c.y;
+
+// bucket 0 holds the longest lists
+__device__ __forceinline__ uint32_t order_bucket(uint32_t count) {
+    return (uint32_t)(kOrderBuckets - 1) - min(count >> 6, (uint32_t)(kOrderBuckets - 1));
+}
+
+// Exclusive prefix of `v` over the threads of a kScanBlock block, in thread order; `total` = the block's sum.
+// s_wave: kScanBlock / kWave words. Two block barriers; may be called again right away.
+__device__ __forceinline__ uint32_t scan_block_exclusive(uint32_t v, uint32_t* s_wave, uint32_t& total) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t incl = v;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const uint32_t up = __shfl_up(incl, s, 64);
+        if (lane >= (uint32_t)s) incl += up;
     }
-    uint32_t incl[3] = {mine[0], mine[1], mine[2]};
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1)
-#pragma unroll
-        for (int k = 0; k < 3; ++k) {
-            const uint32_t up = __shfl_up(incl[k], s, 64);
-            if (lane >= (uint32_t)s) incl[k] += up;
-        }
-    if (lane == 63)
-        for (int k = 0; k < 3; ++k) s_wave[k][wave] = incl[k];
+    __syncthreads();   // s_wave is free again
+    if (lane == 63u) s_wave[wave] = incl;
     __syncthreads();
-    uint32_t run[3], total[3] = {0u, 0u, 0u};
-    for (int k = 0; k < 3; ++k) {
-        run[k] = incl[k] - mine[k];
-        for (uint32_t w = 0; w < (uint32_t)(kScanBlock / kWave); ++w) {
-            const uint32_t s = s_wave[k][w];
-            if (w < wave) run[k] += s;
-            total[k] += s;
+    uint32_t before = incl - v;
+    total = 0u;
+#pragma unroll
+    for (uint32_t w = 0; w < (uint32_t)(kScanBlock / kWave); ++w) {
+        const uint32_t c = s_wave[w];
+        if (w < wave) before += c;
+        total += c;
+    }
+    return before;
+}
+
+__global__ void __launch_bounds__(kScanBlock)
+    k_bin_scan(const uint32_t* __restrict__ bin_count, uint32_t* __restrict__ bin_start, uint2* ranges,
+               const uint2* __restrict__ split_count, uint2* __restrict__ split_base, uint32_t* __restrict__ order,
+               uint32_t* __restrict__ counters, uint32_t n_tiles, uint32_t n_chunks, uint32_t capacity,
+               uint32_t row_capacity) {
+    __shared__ uint32_t s_count[kScanSegment], s_start[kScanSegment];
+    __shared__ uint32_t s_bucket[kOrderBuckets];
+    __shared__ uint32_t s_wave[kScanBlock / kWave];
+    const uint32_t tid = threadIdx.x;
+    // totals first: they decide whether anything is drawn
+    uint32_t mine = 0u;
+    constexpr int kAhead = 8;   // loads of a thread in flight together: a single block has little else to hide them behind
+    for (uint32_t first = 0; first < n_tiles; first += kAhead * kScanBlock) {
+        uint32_t v[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const uint32_t t = first + u * kScanBlock + tid;
+            v[u] = t < n_tiles ? bin_count[t] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) mine += v[u];
+    }
+    uint2 split = make_uint2(0u, 0u);
+    if (tid < n_chunks) split = split_count[tid];
+    uint32_t n_instances, n_split, n_rows;
+    (void)scan_block_exclusive(mine, s_wave, n_instances);
+    const uint32_t split_before = scan_block_exclusive(split.x, s_wave, n_split);
+    const uint32_t rows_before = scan_block_exclusive(split.y, s_wave, n_rows);
+    const bool overflow = n_instances > capacity || n_rows > row_capacity;
+    if (tid < n_chunks) split_base[tid] = make_uint2(split_before, rows_before);
+    for (int i = tid; i < kOrderBuckets; i += kScanBlock) s_bucket[i] = 0u;
+    uint32_t carry = 0u;
+    for (uint32_t first = 0; first < n_tiles; first += kScanSegment) {
+        __syncthreads();   // the segment buffers are free (and, the first time, the buckets are cleared)
+#pragma unroll
+        for (int k = 0; k < kScanPer; ++k) {
+            const uint32_t i = k * kScanBlock + tid, t = first + i;
+            s_count[i] = t < n_tiles && !overflow ? bin_count[t] : 0u;
+        }
+        __syncthreads();
+        uint32_t c[kScanPer], sum = 0u;
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) {
+            c[j] = s_count[tid * kScanPer + j];
+            sum += c[j];
+        }
+        uint32_t segment_total;
+        uint32_t run = carry + scan_block_exclusive(sum, s_wave, segment_total);
+#pragma unroll
+        for (int j = 0; j < kScanPer; ++j) {
+            s_start[tid * kScanPer + j] = run;
+            run += c[j];
+        }
+        carry += segment_total;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < kScanPer; ++k) {
+            const uint32_t i = k * kScanBlock + tid, t = first + i;
+            if (t < n_tiles) {
+                const uint32_t count = s_count[i], start = s_start[i];
+                bin_start[t] = overflow ? 0u : start;
+                ranges[t] = count ? make_uint2(start, start + count) : make_uint2(0u, 0u);
+                atomicAdd(&s_bucket[order_bucket(count)], 1u);
+            }
         }
     }
-    const bool overflow = total[0] > capacity || total[2] > row_capacity;
-    for (uint32_t t = begin; t < end; ++t) {
-        const uint32_t c = overflow ? 0u : bin_count[t];
-        bin_start[t] = overflow ? 0u : run[0];
-        ranges[t] = c ? make_uint2(run[0], run[0] + c) : make_uint2(0u, 0u);
-        run[0] += c;
+    __syncthreads();
+    // the buckets' first places in the schedule, then every tile takes the next place of its bucket
+    constexpr int kPer = kOrderBuckets / kScanBlock;
+    uint32_t in_buckets = 0u;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) in_buckets += s_bucket[tid * kPer + i];
+    uint32_t all;
+    uint32_t place = scan_block_exclusive(in_buckets, s_wave, all);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+        const uint32_t c = s_bucket[tid * kPer + i];
+        s_bucket[tid * kPer + i] = place;
+        place += c;
     }
-    if (tid < n_chunks) split_base[tid] = make_uint2(run[1], run[2]);
+    __syncthreads();   // also: the ranges written above are visible to the whole block
+    for (uint32_t first = 0; first < n_tiles; first += kAhead * kScanBlock) {
+        uint2 r[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const uint32_t t = first + u * kScanBlock + tid;
+            r[u] = t < n_tiles ? ranges[t] : make_uint2(0u, 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const uint32_t t = first + u * kScanBlock + tid;
+            if (t < n_tiles) order[atomicAdd(&s_bucket[order_bucket(r[u].y - r[u].x)], 1u)] = t;
+        }
+    }
     if (tid == 0) {
-        bin_start[n_tiles] = overflow ? 0u : total[0];
+        bin_start[n_tiles] = overflow ? 0u : n_instances;
         counters[kCntVisible] = 0u;   // counted by k_bin_fill
         counters[kCntError] = 0u;
-        counters[kCntInstances] = total[0];
-        counters[kCntSplit] = overflow ? 0u : total[1];   // no list entry is written when nothing is drawn
-        counters[kCntRows] = total[2];
+        counters[kCntInstances] = n_instances;
+        counters[kCntSplit] = overflow ? 0u : n_split;   // no list entry is written when nothing is drawn
+        counters[kCntRows] = n_rows;
         counters[kCntOverflow] = overflow ? 1u : 0u;
     }
 }
@@ -603,10 +692,7 @@ __global__ void __launch_bounds__(kBinThreads)
 }
 
 // ---- tile schedule -----------------------------------------------------------------------------------------------
-// Blocks of the blend kernels take their tiles from this list: longest instance list first, so that the
-// few very long tiles do not start last and run on alone. The order only affects scheduling, not results
-// (tiles are independent); ties inside a bucket of 64 instances are in no particular order.
-constexpr int kOrderBuckets = 4096;
+// The schedule of k_bin_scan for ranges that are already there (the Gaussian footprint's).
 __global__ void __launch_bounds__(kScanBlock) k_tile_order(const uint2* __restrict__ ranges, uint32_t* __restrict__ order,
                                                            uint32_t n_tiles) {
     __shared__ uint32_t s_bucket[kOrderBuckets];
@@ -614,10 +700,9 @@ __global__ void __launch_bounds__(kScanBlock) k_tile_order(const uint2* __restri
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     for (int i = tid; i < kOrderBuckets; i += kScanBlock) s_bucket[i] = 0u;
     __syncthreads();
-    // bucket 0 holds the longest lists
     auto bucket_of = [&](uint32_t t) {
         const uint2 r = ranges[t];
-        return (uint32_t)(kOrderBuckets - 1) - min((r.y - r.x) >> 6, (uint32_t)(kOrderBuckets - 1));
+        return order_bucket(r.y - r.x);
     };
     for (uint32_t t = tid; t < n_tiles; t += kScanBlock) atomicAdd(&s_bucket[bucket_of(t)], 1u);
     __syncthreads();
@@ -1310,9 +1395,8 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
     INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
                 (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start),
                 at<uint2>(ws, L.pub.tile_ranges), (const uint2*)at<uint2>(ws, L.split_count),
-                at<uint2>(ws, L.split_base), counters, L.geo.n_tiles, L.geo.n_chunks, L.geo.capacity, L.geo.row_capacity);
-    INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
-                (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
+                at<uint2>(ws, L.split_base), at<uint32_t>(ws, L.tile_order), counters, L.geo.n_tiles, L.geo.n_chunks,
+                L.geo.capacity, L.geo.row_capacity);
     if (L.geo.n > 0) {
         rc = L.T == 8 ? launch_bin_fill<8>(L, positions, w2c, ws, stream) : launch_bin_fill<16>(L, positions, w2c, ws, stream);
         if (rc != INPC_OK) return rc;
