@@ -207,11 +207,12 @@ __device__ __forceinline__ AxisWeights axis_weights(float s) {
 // far below what 8M points need).
 //
 // Up to kMaxLdsTiles tiles a block keeps its per-tile counters / cursors as 32-bit words in LDS. Beyond that (the
-// reference's 8x8 tiles on large images, up to the 65536 tiles of its 16-bit tile key, kernels.cu:204,214) they are
-// 16-bit halves of LDS words counting within the chunk, which a chunk of at most kWideChunk points cannot
-// overflow, and a cursor's base comes from the table in memory (the WIDE variants of the two kernels).
+// reference's 8x8 tiles on large images, up to the 65536 tiles of its 16-bit tile key, kernels.cu:204,214)
+// k_bin_count counts in 16-bit halves of LDS words, which a chunk of at most kWideChunk points cannot overflow (its
+// WIDE variant: one block of 1024 threads per CU, the counters fill the LDS), and k_bin_fill is launched once per
+// window of kMaxLdsTiles tiles.
 constexpr int kBinBlocks = 512, kBinBlocksWide = 1024;   // chunks: normally; for many tiles and many points
-constexpr int kBinThreads = 512, kBinThreadsWide = 256;   // the WIDE kernels leave the LDS to the counters
+constexpr int kBinThreads = 512, kBinThreadsWide = 1024;
 constexpr uint32_t kMaxLdsTiles = 16384;  // 64 KiB of 32-bit counters
 constexpr uint32_t kWideChunk = 65024;    // points per chunk with 16-bit counters (a multiple of kBinThreads)
 
@@ -506,32 +507,27 @@ struct SplitOut {
 // Preprocess is two kernels that do not depend on each other: k_bin_fill drops the (depth key, point) pairs into
 // the tiles' bins, which is all the tile sort needs; k_records writes the blend records. The host runs the second
 // beside the first and the tile sort (which leaves the memory system idle) on a stream of its own.
-template <int T, bool WIDE>
-__global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
+// One launch fills the bins of the tiles [tile_first, tile_first + tile_count), at most kMaxLdsTiles of them, so that a
+// block keeps a 32-bit cursor per tile in LDS; with more tiles the host launches it once per window of tiles (the
+// points are projected again in every launch, which costs less than taking each slot's base from the tables in
+// memory: 1.0 against 1.6 ms for 33,554,432 points and 63,860 tiles).
+template <int T>
+__global__ void __launch_bounds__(kBinThreads)
     k_bin_fill(const float* __restrict__ positions, const float* __restrict__ w2c, const uint32_t* __restrict__ table,
-               const uint32_t* __restrict__ bin_start, uint64_t* __restrict__ pairs, uint32_t* counters, Geometry g) {
-    constexpr int kThreads = WIDE ? kBinThreadsWide : kBinThreads;
-    extern __shared__ __align__(16) uint32_t s_cursor[];   // n_tiles (WIDE: 16-bit halves)
+               const uint32_t* __restrict__ bin_start, uint64_t* __restrict__ pairs, uint32_t* counters,
+               uint32_t tile_first, uint32_t tile_count, Geometry g) {
+    constexpr int kThreads = kBinThreads;
+    extern __shared__ __align__(16) uint32_t s_cursor[];   // tile_count
     __shared__ uint32_t s_visible;
     const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then no instance is stored
-    const uint32_t chunk_id = blockIdx.x;
-    const uint32_t* row = table + (size_t)chunk_id * g.n_tiles;   // instances of the chunks before, per tile
-    if (WIDE) {
-        for (uint32_t t = threadIdx.x; t < (g.n_tiles + 1u) / 2u; t += kThreads) s_cursor[t] = 0u;
-    } else {
-        for (uint32_t t = threadIdx.x; t < g.n_tiles; t += kThreads) s_cursor[t] = bin_start[t] + row[t];
-    }
-    // next bin slot of `tile`
-    auto take_slot = [&](uint32_t tile) -> uint32_t {
-        if (WIDE) return bin_start[tile] + row[tile] + packed_counter_next(s_cursor, tile);
-        return atomicAdd(&s_cursor[tile], 1u);
-    };
+    const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;   // instances of the chunks before, per tile
+    for (uint32_t t = threadIdx.x; t < tile_count; t += kThreads) s_cursor[t] = bin_start[tile_first + t] + row[tile_first + t];
     if (threadIdx.x == 0) s_visible = 0u;
     __syncthreads();
     const ViewRows m = load_view_rows(w2c);
     uint32_t my_visible = 0;
     const uint32_t chunk = bin_chunk_size(g.n, g.n_chunks);
-    const uint32_t begin = min(chunk_id * chunk, g.n), end = min(begin + chunk, g.n);
+    const uint32_t begin = min(blockIdx.x * chunk, g.n), end = min(begin + chunk, g.n);
     constexpr int kUnroll = 4;   // points per thread and round, their loads issued together
     for (uint32_t base = begin; base < end; base += kUnroll * kThreads) {
         float px[kUnroll], py[kUnroll], pz[kUnroll];
@@ -552,9 +548,14 @@ __global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads)
             if (p.info == 0u) continue;
             my_visible += 1u;
             const uint64_t pair = ((uint64_t)(__float_as_uint(p.depth) - g.key_bias) << 32) | (uint64_t)i;
-            if (!overflow) for_each_tile(p.info, g.gw, [&](uint32_t tile) { pairs[take_slot(tile)] = pair; });
+            if (!overflow)
+                for_each_tile(p.info, g.gw, [&](uint32_t tile) {
+                    const uint32_t local = tile - tile_first;   // wraps around for a tile in front of the window
+                    if (local < tile_count) pairs[atomicAdd(&s_cursor[local], 1u)] = pair;
+                });
         }
     }
+    if (tile_first != 0u) return;   // the drawn points are counted by the first launch
     // block total -> one global atomic
     for (int s = 32; s > 0; s >>= 1) my_visible += __shfl_down(my_visible, s, 64);
     if ((threadIdx.x & 63u) == 0u) atomicAdd(&s_visible, my_visible);
@@ -812,7 +813,7 @@ struct Layout {
     Geometry geo;
     int T, C, fmode, key_bits;
     bool inference, sh, half_features;
-    bool wide;   // more tiles than a block keeps 32-bit counters for: the WIDE binning kernels
+    bool wide;   // more tiles than a block keeps 32-bit counters for
     // private offsets
     size_t bin_table, bin_total, tile_order, split_count, split_base;
     size_t pairs, pairs_scratch;
@@ -976,14 +977,12 @@ template <int T>
 int launch_bin_fill(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
     const uint32_t* table = at<uint32_t>(ws, L.bin_table);
     const uint32_t* bin_start = at<uint32_t>(ws, L.pub.bin_start);
-    if (L.wide) {
-        const size_t lds = (size_t)(L.geo.n_tiles + 1) / 2 * 4;
-        INPC_LAUNCH_LDS("raster_bin_fill", (k_bin_fill<T, true>), dim3(L.geo.n_chunks), dim3(kBinThreadsWide), lds, stream,
-                        positions, w2c, table, bin_start, at<uint64_t>(ws, L.pairs), at<uint32_t>(ws, L.pub.counters), L.geo);
-    } else {
-        const size_t lds = (size_t)L.geo.n_tiles * 4;
-        INPC_LAUNCH_LDS("raster_bin_fill", (k_bin_fill<T, false>), dim3(L.geo.n_chunks), dim3(kBinThreads), lds, stream,
-                        positions, w2c, table, bin_start, at<uint64_t>(ws, L.pairs), at<uint32_t>(ws, L.pub.counters), L.geo);
+    for (uint32_t first = 0; first < L.geo.n_tiles; first += kMaxLdsTiles) {
+        const uint32_t count = std::min(kMaxLdsTiles, L.geo.n_tiles - first);
+        const size_t lds = (size_t)count * 4;
+        INPC_LAUNCH_LDS("raster_bin_fill", (k_bin_fill<T>), dim3(L.geo.n_chunks), dim3(kBinThreads), lds, stream, positions,
+                        w2c, table, bin_start, at<uint64_t>(ws, L.pairs), at<uint32_t>(ws, L.pub.counters), first, count,
+                        L.geo);
     }
     return INPC_OK;
 }
