@@ -257,6 +257,37 @@ def main() -> int:
         field_ms = time_calls(lambda: update_probability_field(field_weights, field_scores, leaf_ids, blending_weights),
                               args.steps)
 
+    # the same step with the other tile size (the reference's tiles are 8x8; the images do not depend on the tile size):
+    # a side measurement, not part of `value`
+    other_tile = None
+    if not args.no_extras:
+        t2 = 8 if tile == 16 else 16
+        cfg2 = _lib.RasterConfig(n, t2, channels, _lib.FEAT_DIRECT_F32, 0, _lib.make_camera(hv.camera), 0)
+        layout2 = _lib.RasterLayout()
+        _lib.check(lib.inpc_raster_layout_query(C.byref(cfg2), C.byref(layout2)), "layout")
+        ws2 = torch.empty(layout2.total_bytes, dtype=torch.uint8, device=device)
+        image2, alpha2, bw2 = torch.empty_like(image), torch.empty_like(alpha), torch.empty_like(blending_weights)
+        gf2, go2 = torch.empty_like(grad_features), torch.empty_like(grad_opacities)
+
+        def step2():
+            _lib.check(lib.inpc_raster_forward(C.byref(cfg2), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
+                                               _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image2), _lib.ptr(alpha2),
+                                               _lib.ptr(bw2), None, _lib.ptr(ws2), layout2.total_bytes, stream),
+                       "inpc_raster_forward")
+            _lib.check(lib.inpc_raster_backward(C.byref(cfg2), _lib.ptr(grad_image), _lib.ptr(grad_alpha), _lib.ptr(image2),
+                                                _lib.ptr(alpha2), _lib.ptr(positions), _lib.ptr(cam_position), _lib.ptr(gf2),
+                                                _lib.ptr(go2), None, _lib.ptr(ws2), layout2.total_bytes, stream),
+                       "inpc_raster_backward")
+
+        step2()
+        step2_ms = time_calls(step2, args.steps)
+        counters2 = (C.c_uint32 * 3)()
+        _lib.check(lib.inpc_raster_read_counters(C.byref(cfg2), _lib.ptr(ws2), C.byref(counters2), stream), "counters")
+        other_tile = {"tile": t2, "ms_per_step": round(step2_ms, 4), "Mpoints_per_s": round(n / (step2_ms * 1e-3) / 1e6, 1),
+                      "n_instances": int(counters2[1]), "n_tiles": int(layout2.n_tiles),
+                      "max_abs_image_difference": float((image2 - image).abs().max())}
+        del ws2, image2, alpha2, bw2, gf2, go2
+
     # the same points through the Gaussian footprint (the reference's other rasterizer mode), 8x8 tiles as in the
     # reference: a side measurement, not part of `value`
     gaussian = None
@@ -470,6 +501,7 @@ def main() -> int:
             "graph_replay_ms": None if graph_ms is None else round(graph_ms, 4),
             "sampler": sampler_extra,
             "field_update_ms": None if field_ms is None else round(field_ms, 4),
+            "other_tile_size": other_tile,
             "gaussian_footprint": gaussian,
             "sh36_autograd_step": reference_shape,
             "config4_inference": config4,
