@@ -336,11 +336,11 @@ typedef struct inpc_gaussian_layout {
                                 the point's gradient rows instead), u32 (bits 0-27 point id,
                                 28-30 min(tile columns, 7), 31: touches more than one tile);
                                 then the view features as fp32                                  */
-    size_t depth_order;      /* (N) u32 point ids in (depth, point id) order, n_visible valid   */
-    size_t depth_keys;       /* (N) u32 matching depth keys                                     */
-    size_t instance_keys;    /* (max_instances) u16 tile id per instance in final order         */
-    size_t instance_points;  /* (max_instances) u32 point id per instance in final order        */
-    size_t tile_ranges;      /* (n_tiles) {u32 begin, end}                                      */
+    size_t depth_keys;       /* (N) u32, in point order: (float bits of the depth) - depth_key_bias,
+                                0xFFFFFFFF for a point that is not drawn                        */
+    size_t instance_points;  /* (max_instances) u32 point id per instance: the instances of tile
+                                t are [tile_ranges[t].begin, .end), in (depth key, point id) order */
+    size_t tile_ranges;      /* (n_tiles) {u32 begin, end}; {0, 0} for a tile without instances  */
     uint32_t record_stride;
     uint32_t grid_width;
     uint32_t grid_height;

@@ -84,9 +84,7 @@ class GaussianLayout(C.Structure):
         ("point_touched", C.c_size_t),
         ("point_bounds", C.c_size_t),
         ("point_record", C.c_size_t),
-        ("depth_order", C.c_size_t),
         ("depth_keys", C.c_size_t),
-        ("instance_keys", C.c_size_t),
         ("instance_points", C.c_size_t),
         ("tile_ranges", C.c_size_t),
         ("record_stride", C.c_uint32),

@@ -173,61 +173,9 @@ __device__ __forceinline__ uint32_t status_load(const uint32_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Publish this block's aggregate (block 0: its inclusive prefix). Doing this as early as the aggregate is
-// known lets the blocks behind finish their walk without waiting for this block's remaining work.
-__device__ __forceinline__ void lookback_publish(uint32_t* status, uint32_t stride, uint32_t bid, uint32_t aggregate) {
-    status_store(status + (size_t)bid * stride, (bid == 0 ? kFlagInclusive : kFlagAggregate) | aggregate);
-}
-
-// Exclusive prefix of the aggregates of blocks 0..bid-1; publishes this block's inclusive prefix.
-// `status` points at this stream's word of block 0; consecutive blocks are `stride` words apart.
-// lookback_publish must have been called for this block.
-__device__ __forceinline__ uint32_t lookback_walk(uint32_t* status, uint32_t stride, uint32_t bid, uint32_t aggregate,
-                                                  uint32_t* error_flag) {
-    if (bid == 0) return 0u;
-    // Several predecessors are fetched per round trip and consumed nearest first; the walk ends at the
-    // first one that carries an inclusive prefix and waits at the first one that has nothing yet.
-    constexpr int kAhead = 8;
-    uint32_t exclusive = 0u, spins = 0u;
-    int64_t p = (int64_t)bid - 1;
-    bool finished = false;
-    while (!finished && p >= 0) {
-        uint32_t word[kAhead];
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u) {
-            const int64_t q = p - u;
-            word[u] = q >= 0 ? status_load(status + (size_t)q * stride) : kFlagInclusive;  // before block 0: nothing
-        }
-        int consumed = 0;
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u) {
-            if (finished || consumed != u) continue;
-            if ((word[u] & ~kValueMask) == 0u) continue;  // not published yet: stop consuming here
-            exclusive += word[u] & kValueMask;
-            ++consumed;
-            finished = (word[u] & kFlagInclusive) != 0u;
-        }
-        p -= consumed;
-        if (consumed == 0) {
-            if (++spins > kSpinLimit) {
-                atomicOr(error_flag, 1u);  // give up: the result is wrong but the kernel ends
-                break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-        }
-    }
-    status_store(status + (size_t)bid * stride, kFlagInclusive | ((exclusive + aggregate) & kValueMask));
-    return exclusive;
-}
-
-__device__ __forceinline__ uint32_t lookback_exclusive(uint32_t* status, uint32_t stride, uint32_t bid,
-                                                       uint32_t aggregate, uint32_t* error_flag) {
-    lookback_publish(status, stride, bid, aggregate);
-    return lookback_walk(status, stride, bid, aggregate, error_flag);
-}
-
-// The same for a single value per block, walked by a whole wave: the 64 lanes look at 64 predecessors at
-// a time. Every lane of the calling wave must enter; all get the result.
+// Exclusive prefix of one value per block over blocks 0..bid-1, walked by a whole wave: the 64 lanes look at 64
+// predecessors at a time; publishes this block's aggregate first and its inclusive prefix at the end. Every lane of
+// the calling wave must enter; all get the result.
 __device__ __forceinline__ uint32_t lookback_exclusive_wave(uint32_t* status, uint32_t bid, uint32_t aggregate,
                                                             uint32_t* error_flag) {
     const uint32_t lane = lane_id();

@@ -1,18 +1,17 @@
 // gaussian.hpp — the rasterizer's Gaussian footprint (RasterizerMode.GAUSSIAN; B/rasterization/src/gaussian/).
 // Included by raster.hip after blend.hpp; shares the projection, SH and sort helpers with the bilinear path.
 //
-// A point is drawn as a screen-space Gaussian and touches any number of tiles, so this path keeps the reference's
-// structure: per-point records in point order, depth sort, instances expanded in depth order, stable tile sort,
-// ranges, blend (B/rasterization/src/gaussian/forward.cu:12-172).
-//   k_preprocess        project, covariance -> conic, tile bounds, record, depth key and digit histograms
-//                       (kernels.cu:11-324)
-//   radix sort          by depth key, culled points dropped (forward.cu:92-100)
-//   k_touch_sums / k_touch_scan   exclusive prefix of the touched-tile counts in depth order (forward.cu:102-116)
-//   k_create_instances  every block expands 1024 depth-ordered points; the instances, not the points, are spread
-//                       over the threads, so a point that covers the screen costs no more per instance than one
-//                       that covers a tile (kernels.cu:358-380); tile-key histograms for the sort
-//   radix sort          by tile key, stable (forward.cu:133-141)
-//   k_ranges            [begin, end) per tile (kernels.cu:382-399)
+// A point is drawn as a screen-space Gaussian and touches any number of tiles. Per-point records in point order;
+// the per-tile instance lists of the reference (depth sort, instances expanded in depth order, stable tile sort,
+// ranges: B/rasterization/src/gaussian/forward.cu:12-172) come from per-tile bins sorted in LDS, as for the bilinear
+// footprint.
+//   k_preprocess        project, covariance -> conic, tile bounds, record, depth key (kernels.cu:11-324)
+//   k_bin_count         per (chunk of points, tile): instances; a rectangle of many tiles is taken by the whole block,
+//                       so a point that covers the screen costs no more per instance than one that covers a tile
+//   k_bin_offsets, k_bin_scan (raster.hip)   prefix over the chunks; tile ranges, schedule, "do the instances fit"
+//   k_bin_fill          a (depth key, point) pair per instance into the bin of its tile; gradient rows of the points
+//                       that touch several tiles (kernels.cu:358-380)
+//   tilesort.hpp        every bin sorted by (depth key, point index): the order of forward.cu:92-141
 //   k_blend_*           one block per tile, one thread per pixel, a wave owns an 8 x 8 pixel block; per batch of
 //                       T*T staged instances and 64 instances at a time, every lane first collects the instances
 //                       whose pixel box contains its pixel (a few integer operations each) and then evaluates only
@@ -29,11 +28,7 @@ constexpr uint32_t kMultiTile = 1u << 31;
 constexpr uint32_t kPointMask = (1u << 28) - 1u;
 constexpr int kColumnsShift = 28;
 constexpr uint32_t kManyColumns = 7u;               // 7 or more tile columns: the count is looked up
-constexpr int kCntKept = 4;                         // instances that are sorted and drawn (0 when they do not fit)
-constexpr int kCntInstances64 = 6;                  // u64 at words 6, 7: exact instance count
-constexpr int kCntMulti = 8;                        // drawn points that touch more than one tile
-constexpr int kCntDirect = 9;                       // set by a backward blend that added gradients to the arrays directly
-constexpr int kPointsPerBlock = 1024;               // depth-ordered points per block of the instance kernels
+constexpr uint32_t kNoKey = 0xFFFFFFFFu;            // depth key of a point that is not drawn
 
 inline uint32_t record_stride(int channels) { return (uint32_t)align_up(32 + (size_t)channels * 4, 32); }
 
@@ -69,18 +64,15 @@ __global__ void __launch_bounds__(kBlock)
     k_preprocess(const float* __restrict__ positions, const void* __restrict__ features,
                  const float* __restrict__ opacities, const float* __restrict__ scales, const float* __restrict__ w2c,
                  const float* __restrict__ cam_position, char* __restrict__ records, uint32_t* __restrict__ touched_out,
-                 uint2* __restrict__ bounds_out, uint32_t* __restrict__ keys, uint32_t* __restrict__ vals,
-                 float* __restrict__ blending_weights, uint32_t* counters, uint32_t* g_hist, Geometry g, Params prm,
-                 float tile_edge, radix::DevicePlan plan) {
+                 uint2* __restrict__ bounds_out, uint32_t* __restrict__ keys,
+                 float* __restrict__ blending_weights, uint32_t* counters, Geometry g, Params prm, float tile_edge) {
     // A record leaves the block through LDS: every lane assembles its record in the wave's staging rows, then the
     // wave writes its 64 records, which are neighbours in memory, as one contiguous run of 16-byte words (a lane
     // storing its own record would put 16 bytes into each of 64 different lines per instruction).
     constexpr uint32_t kWords = (32u + 4u * C + 31u) / 32u * 2u, kRow = kWords + 1u;   // 16-byte words per record; padded row
     __shared__ float4 s_stage[kBlock * kRow];
-    __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
     __shared__ uint32_t s_visible;
     __shared__ unsigned long long s_instances;
-    for (int i = threadIdx.x; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
     if (threadIdx.x == 0) {
         s_visible = 0u;
         s_instances = 0ull;
@@ -91,14 +83,14 @@ __global__ void __launch_bounds__(kBlock)
     const ViewRows m = load_view_rows(w2c);
     uint32_t my_visible = 0u;
     unsigned long long my_instances = 0ull;
-    // the grid is a few blocks per CU and walks over the points: histograms and counts leave a block once
+    // the grid is a few blocks per CU and walks over the points: the counts leave a block once
     for (uint32_t first = blockIdx.x * kBlock; first < g.n; first += gridDim.x * kBlock) {
     const uint32_t i = first + threadIdx.x;
 #pragma unroll
     for (uint32_t w = 0; w < kWords; ++w) stage[lane * kRow + w] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     uint32_t touched = 0u;
     if (i < g.n) {
-        uint32_t key = radix::kInvalidKey;
+        uint32_t key = kNoKey;
         const float px = positions[3 * (size_t)i], py = positions[3 * (size_t)i + 1], pz = positions[3 * (size_t)i + 2];
         const float depth = affine_row(m.r3, px, py, pz);
         if (!(depth < g.cam.near_plane || depth > g.cam.far_plane)) {
@@ -157,13 +149,11 @@ __global__ void __launch_bounds__(kBlock)
                     rec[1] = make_float4(conic_y, conic_z, depth,
                                          __uint_as_float(i | (min(x1 - x0, kManyColumns) << kColumnsShift) | (touched > 1u ? kMultiTile : 0u)));
                     key = __float_as_uint(depth) - g.key_bias;
-                    radix::hist_add(s_hist, plan, key);
                 }
             }
         }
         touched_out[i] = touched;
         keys[i] = key;
-        vals[i] = i;
         if (blending_weights) blending_weights[i] = 0.0f;
     }
     wave_sync();
@@ -193,204 +183,137 @@ __global__ void __launch_bounds__(kBlock)
         if (s_visible) atomicAdd(&counters[kCntVisible], s_visible);
         if (s_instances) atomicAdd((unsigned long long*)(counters + kCntInstances64), s_instances);
     }
-    radix::hist_flush(s_hist, plan, g_hist);
 }
 
-// ---- instance offsets: exclusive prefix of the touched-tile counts in depth order (kernels.cu:346-356,
-// forward.cu:110-116). The tile bounds are gathered once, here, and kept in depth order for k_create_instances;
-// the count follows from them.
-__device__ __forceinline__ uint32_t tiles_of(uint2 b) {
-    return ((b.x >> 16) - (b.x & 0xFFFFu)) * ((b.y >> 16) - (b.y & 0xFFFFu));
-}
+// ---- instance bins (kernels.cu:346-399, forward.cu:87-160) --------------------------------------------------------
+// The reference sorts the drawn points by depth, expands them into (tile, point) instances and sorts those by tile
+// with a second stable device-wide sort: per tile the instances end up ordered by (depth key, point index). Here, as
+// for the bilinear footprint, the instances are counted per (chunk of points, tile), every tile gets its range, a
+// (depth key, point) pair per instance is dropped into the bin of its tile and one block per tile sorts its bin in LDS
+// (tilesort.hpp): the same lists, without any device-wide sort. A point touches any number of tiles: the owner thread
+// walks over a rectangle of up to kOwnTiles tiles itself, larger ones are queued and taken by the whole block.
+constexpr uint32_t kOwnTiles = 64;
+constexpr int kQueue = 512;   // queued points per block; further ones are walked by their owner after all
 
-__global__ void __launch_bounds__(kBlock)
-    k_touch_sums(const uint32_t* __restrict__ order, const uint2* __restrict__ bounds,
-                 const uint32_t* __restrict__ counters, uint2* __restrict__ sorted_bounds,
-                 uint32_t* __restrict__ block_sums) {
-    __shared__ uint32_t s_wave[kBlock / kWave];
-    const uint32_t n_visible = counters[kCntVisible];
-    const uint32_t base = blockIdx.x * kPointsPerBlock;
-    uint32_t sum = 0;
-    for (uint32_t k = threadIdx.x; k < (uint32_t)kPointsPerBlock; k += kBlock) {
-        const uint32_t j = base + k;
-        if (j < n_visible) {
-            const uint2 b = bounds[order[j]];
-            sorted_bounds[j] = b;
-            sum += tiles_of(b);
-        }
-    }
-    for (int s = 32; s > 0; s >>= 1) sum += __shfl_down(sum, s, 64);
-    if ((threadIdx.x & 63u) == 0u) s_wave[threadIdx.x >> 6] = sum;
+// Calls point(i, touched, bounds) once for every drawn point of the block's points [begin, end) and then visit(i, tile)
+// for the tiles of its rectangle in the rows that the window [tile_first, tile_first + tile_count) of tile ids reaches
+// into (the first and the last of these rows may lie partly outside the window: visit checks).
+template <int THREADS, typename Point, typename Visit>
+__device__ __forceinline__ void for_each_instance(const uint32_t* __restrict__ touched, const uint2* __restrict__ bounds,
+                                                  uint32_t begin, uint32_t end, uint32_t gw, uint32_t tile_first,
+                                                  uint32_t tile_count, uint32_t* s_queue, uint32_t* s_queued,
+                                                  Point point, Visit visit) {
+    constexpr uint32_t kThreads = THREADS;
+    const uint32_t band_y0 = tile_first / gw, band_y1 = (tile_first + tile_count + gw - 1u) / gw;
+    if (threadIdx.x == 0) *s_queued = 0u;
     __syncthreads();
+    for (uint32_t base = begin; base < end; base += kThreads) {
+        const uint32_t i = base + threadIdx.x;
+        const uint32_t count = i < end ? touched[i] : 0u;
+        if (count == 0u) continue;
+        const uint2 b = bounds[i];
+        point(i, count, b);
+        const uint32_t x0 = b.x & 0xFFFFu, x1 = b.x >> 16;
+        const uint32_t y0 = max(b.y & 0xFFFFu, band_y0), y1 = min(b.y >> 16, band_y1);
+        if (y0 >= y1) continue;
+        if ((x1 - x0) * (y1 - y0) > kOwnTiles) {
+            const uint32_t slot = atomicAdd(s_queued, 1u);
+            if (slot < (uint32_t)kQueue) {
+                s_queue[slot] = i;
+                continue;
+            }
+        }
+        for (uint32_t ty = y0; ty < y1; ++ty)
+            for (uint32_t tx = x0; tx < x1; ++tx) visit(i, ty * gw + tx);
+    }
+    __syncthreads();
+    const uint32_t queued = min(*s_queued, (uint32_t)kQueue);
+    for (uint32_t q = 0; q < queued; ++q) {
+        const uint32_t i = s_queue[q];
+        const uint2 b = bounds[i];
+        const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0;
+        const uint32_t y0 = max(b.y & 0xFFFFu, band_y0), ny = min(b.y >> 16, band_y1) - y0;
+        for (uint32_t r = threadIdx.x; r < nx * ny; r += kThreads) visit(i, (y0 + r / nx) * gw + x0 + r % nx);
+    }
+}
+
+// Per chunk of points and tile of the window: number of instances; per chunk (first window only): the points that
+// touch several tiles and their instances.
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS)
+    k_bin_count(const uint32_t* __restrict__ touched, const uint2* __restrict__ bounds, uint32_t* __restrict__ table,
+                uint2* __restrict__ split_count, uint32_t tile_first, uint32_t tile_count, uint32_t n, uint32_t n_chunks,
+                uint32_t n_tiles, uint32_t gw) {
+    extern __shared__ uint32_t s_count[];   // tile_count
+    __shared__ uint32_t s_queue[kQueue];
+    __shared__ uint32_t s_queued, s_split, s_rows;
+    for (uint32_t t = threadIdx.x; t < tile_count; t += THREADS) s_count[t] = 0u;
+    if (threadIdx.x == 0) s_split = s_rows = 0u;
+    const uint32_t chunk = bin_chunk_size(n, n_chunks);
+    const uint32_t begin = min(blockIdx.x * chunk, n), end = min(begin + chunk, n);
+    uint32_t my_split = 0u, my_rows = 0u;
+    for_each_instance<THREADS>(
+        touched, bounds, begin, end, gw, tile_first, tile_count, s_queue, &s_queued,
+        [&](uint32_t, uint32_t count, uint2) {
+            if (count > 1u) {
+                my_split += 1u;
+                my_rows += count;
+            }
+        },
+        [&](uint32_t, uint32_t tile) {
+            const uint32_t local = tile - tile_first;   // wraps around for a tile in front of the window
+            if (local < tile_count) atomicAdd(&s_count[local], 1u);
+        });
+    if (my_split) {
+        atomicAdd(&s_split, my_split);
+        atomicAdd(&s_rows, my_rows);
+    }
+    __syncthreads();
+    uint32_t* row = table + (size_t)blockIdx.x * n_tiles + tile_first;
+    for (uint32_t t = threadIdx.x; t < tile_count; t += THREADS) row[t] = s_count[t];
+    if (threadIdx.x == 0 && tile_first == 0u) split_count[blockIdx.x] = make_uint2(s_split, s_rows);
+}
+
+// Drops the pair (depth key, point) of every instance into the bin of its tile (window by window, like the counts).
+// First window only, training configurations: a point that touches several tiles gets its gradient rows, one per
+// tile in row-major order of its rectangle: the instance of tile (tx, ty) has row origin + ty * columns + tx, and the
+// origin (modulo 2^32) replaces the depth in the point's record, which only the inference blend reads. The points go
+// on a list {first row, rows, point} for the pass that adds the rows up.
+template <int THREADS>
+__global__ void __launch_bounds__(THREADS)
+    k_bin_fill(const uint32_t* __restrict__ touched, const uint2* __restrict__ bounds, const uint32_t* __restrict__ keys,
+               const uint32_t* __restrict__ table, const uint32_t* __restrict__ bin_start, uint64_t* __restrict__ pairs,
+               const uint2* __restrict__ split_base, uint4* __restrict__ multi_list, char* __restrict__ records,
+               uint32_t stride, const uint32_t* __restrict__ counters, uint32_t tile_first, uint32_t tile_count,
+               uint32_t n, uint32_t n_chunks, uint32_t n_tiles, uint32_t gw) {
+    extern __shared__ uint32_t s_cursor[];   // tile_count
+    __shared__ uint32_t s_queue[kQueue];
+    __shared__ uint32_t s_queued, s_split, s_rows;
+    if (counters[kCntKept] == 0u) return;   // nothing is drawn (no instances, or more than the buffers hold)
+    const uint32_t* row = table + (size_t)blockIdx.x * n_tiles + tile_first;
+    for (uint32_t t = threadIdx.x; t < tile_count; t += THREADS) s_cursor[t] = bin_start[tile_first + t] + row[t];
+    const bool lists = multi_list != nullptr && tile_first == 0u;
     if (threadIdx.x == 0) {
-        uint32_t total = 0;
-        for (int w = 0; w < kBlock / kWave; ++w) total += s_wave[w];
-        block_sums[blockIdx.x] = total;
+        const uint2 first = lists ? split_base[blockIdx.x] : make_uint2(0u, 0u);
+        s_split = first.x;
+        s_rows = first.y;
     }
-}
-
-// One block: block_sums -> exclusive prefix in place; decides whether the instances fit. When they do not, nothing
-// is expanded or drawn (the 32-bit offsets could not even address them) and the count tells the caller.
-__global__ void __launch_bounds__(kScanBlock) k_touch_scan(uint32_t* __restrict__ block_sums, uint32_t n_blocks,
-                                                           uint32_t* counters, uint32_t capacity,
-                                                           unsigned long long* generation, unsigned long long seed) {
-    __shared__ uint32_t s_wave[kScanBlock / kWave];
-    __shared__ uint32_t s_fits;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    if (tid == 0) {
-        const unsigned long long total = *(const unsigned long long*)(counters + kCntInstances64);
-        const bool fits = total <= (unsigned long long)capacity;
-        s_fits = fits ? 1u : 0u;
-        counters[kCntKept] = fits ? (uint32_t)total : 0u;
-        counters[kCntInstances] = total > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)total;
-        // The stamp the backward pass marks its gradient rows with: a new one per forward pass *execution* (a full-period
-        // congruential step in the workspace, increment from the host's per-call seed), so that a captured graph, whose
-        // kernel arguments never change, still gets a new stamp on every replay.
-        if (generation) *generation = *generation * 6364136223846793005ull + (seed | 1ull);
-    }
-    __syncthreads();
-    if (!s_fits) return;
-    const uint32_t per = (n_blocks + kScanBlock - 1) / kScanBlock;
-    const uint32_t begin = min(tid * per, n_blocks), end = min(begin + per, n_blocks);
-    uint32_t mine = 0;
-    for (uint32_t b = begin; b < end; ++b) mine += block_sums[b];
-    uint32_t incl = mine;
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s, 64);
-        if (lane >= (uint32_t)s) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - mine;
-    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
-    for (uint32_t b = begin; b < end; ++b) {
-        const uint32_t c = block_sums[b];
-        block_sums[b] = run;
-        run += c;
-    }
-}
-
-// Instances of the block's 1024 depth-ordered points, in depth order, row-major over each point's tiles
-// (kernels.cu:358-380). Output slot s of the block belongs to the last point whose offset is <= s.
-__global__ void __launch_bounds__(kBlock)
-    k_create_instances(const uint32_t* __restrict__ order, const uint2* __restrict__ sorted_bounds,
-                       const uint32_t* __restrict__ block_base,
-                       const uint32_t* counters, uint16_t* __restrict__ inst_keys,
-                       uint32_t* __restrict__ inst_points, uint4* __restrict__ multi_list, uint32_t* counters_out,
-                       char* __restrict__ records, uint32_t stride, uint32_t* g_hist, uint32_t gw,
-                       radix::DevicePlan plan) {
-    constexpr int kPer = kPointsPerBlock / kBlock;   // consecutive points per thread
-    __shared__ uint32_t s_offset[kPointsPerBlock + 1];
-    __shared__ uint32_t s_point[kPointsPerBlock];
-    __shared__ uint2 s_bounds[kPointsPerBlock];
-    __shared__ uint32_t s_wave[kBlock / kWave];
-    __shared__ uint32_t s_hist[radix::kMaxPasses * radix::kRadix];
-    __shared__ uint32_t s_multi, s_multi_base;
-    if (counters[kCntKept] == 0u) return;
-    const uint32_t n_visible = counters[kCntVisible];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    for (int i = tid; i < plan.n_passes * radix::kRadix; i += kBlock) s_hist[i] = 0u;
-    // a block takes the chunks of 1024 points chunk, chunk + grid, ...: the histograms leave it once
-    for (uint32_t chunk = blockIdx.x; chunk * kPointsPerBlock < n_visible; chunk += gridDim.x) {
-    const uint32_t base = chunk * kPointsPerBlock;
-    if (tid == 0) s_multi = 0u;
-    uint32_t count[kPer], mine = 0;
-#pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-        const uint32_t k = tid * kPer + u, j = base + k;
-        count[u] = 0u;
-        if (j < n_visible) {
-            const uint2 b = sorted_bounds[j];
-            count[u] = tiles_of(b);
-            s_point[k] = order[j];
-            s_bounds[k] = b;
-        }
-        mine += count[u];
-    }
-    uint32_t incl = mine;
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s, 64);
-        if (lane >= (uint32_t)s) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - mine;
-    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
-#pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-        s_offset[tid * kPer + u] = run;
-        run += count[u];
-    }
-    if (tid == kBlock - 1) s_offset[kPointsPerBlock] = run;
-    __syncthreads();
-    const uint32_t total = s_offset[kPointsPerBlock];
-    const uint32_t out = block_base[chunk];
-    if (multi_list) {
-        // Where a point's instances start, in the order they are created in: the backward pass collects the
-        // gradient of a point that touches several tiles in rows numbered that way. The instance of tile (tx, ty)
-        // has row origin + ty * columns + tx; the origin (modulo 2^32) replaces the depth in the point's record,
-        // which only the inference blend reads. The points themselves go on a list {first row, rows, point} for
-        // the pass that adds the rows up (in no particular order: every point is summed on its own).
-        uint32_t mine_multi = 0;
-#pragma unroll
-        for (int u = 0; u < kPer; ++u) mine_multi += (base + tid * kPer + u < n_visible && count[u] > 1u) ? 1u : 0u;
-        uint32_t slot = mine_multi ? atomicAdd(&s_multi, mine_multi) : 0u;
-        __syncthreads();
-        if (tid == 0) s_multi_base = s_multi ? atomicAdd(&counters_out[kCntMulti], s_multi) : 0u;
-        __syncthreads();
-        slot += s_multi_base;
-#pragma unroll
-        for (int u = 0; u < kPer; ++u) {
-            const uint32_t k = tid * kPer + u;
-            if (base + k < n_visible && count[u] > 1u) {
-                const uint32_t at = out + s_offset[k];
-                const uint2 b = s_bounds[k];
+    const uint32_t chunk = bin_chunk_size(n, n_chunks);
+    const uint32_t begin = min(blockIdx.x * chunk, n), end = min(begin + chunk, n);
+    for_each_instance<THREADS>(
+        touched, bounds, begin, end, gw, tile_first, tile_count, s_queue, &s_queued,
+        [&](uint32_t i, uint32_t count, uint2 b) {
+            if (lists && count > 1u) {
+                const uint32_t first_row = atomicAdd(&s_rows, count);
                 const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
-                ((uint32_t*)(records + (size_t)s_point[k] * stride))[6] = at - y0 * nx - x0;
-                multi_list[slot++] = make_uint4(at, count[u], s_point[k], 0u);
+                ((uint32_t*)(records + (size_t)i * stride))[6] = first_row - y0 * nx - x0;
+                multi_list[atomicAdd(&s_split, 1u)] = make_uint4(first_row, count, i, 0u);
             }
-        }
-    }
-    for (uint32_t s = tid; s < total; s += kBlock) {
-        uint32_t lo = 0, hi = kPointsPerBlock;   // last k with s_offset[k] <= s
-        while (hi - lo > 1u) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (s_offset[mid] <= s) lo = mid;
-            else hi = mid;
-        }
-        const uint2 b = s_bounds[lo];
-        const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0, y0 = b.y & 0xFFFFu;
-        const uint32_t r = s - s_offset[lo];
-        const uint32_t tile = (y0 + r / nx) * gw + x0 + r % nx;
-        inst_keys[out + s] = (uint16_t)tile;
-        inst_points[out + s] = s_point[lo];
-        radix::hist_add(s_hist, plan, tile);
-    }
-    __syncthreads();   // the LDS arrays are reused by the next chunk
-    }
-    radix::hist_flush(s_hist, plan, g_hist);
-}
-
-// [begin, end) of every tile's instances (kernels.cu:382-399); tiles without instances keep (0, 0).
-__global__ void __launch_bounds__(kBlock) k_ranges(const uint16_t* __restrict__ inst_keys,
-                                                   const uint32_t* __restrict__ counters, uint2* __restrict__ ranges) {
-    const uint32_t n = counters[kCntKept];
-    const uint32_t stride = gridDim.x * kBlock;
-    for (uint32_t k = blockIdx.x * kBlock + threadIdx.x; k < n; k += stride) {
-        const uint32_t t = inst_keys[k];
-        if (k == 0u) {
-            ranges[t].x = 0u;
-        } else {
-            const uint32_t before = inst_keys[k - 1];
-            if (before != t) {
-                ranges[before].y = k;
-                ranges[t].x = k;
-            }
-        }
-        if (k == n - 1u) ranges[t].y = n;
-    }
+        },
+        [&](uint32_t i, uint32_t tile) {
+            const uint32_t local = tile - tile_first;
+            if (local < tile_count) pairs[atomicAdd(&s_cursor[local], 1u)] = ((uint64_t)keys[i] << 32) | (uint64_t)i;
+        });
 }
 
 // ---- blend -----------------------------------------------------------------------------------------------------------
@@ -690,11 +613,11 @@ __global__ void __launch_bounds__(T * T)
     }
 }
 
-// Gradient rows of the points that touch several tiles: one row per instance, numbered in the order the instances
-// are created in (a point's instances are neighbours): C + 1 values, then the two words of the call's stamp, padded
+// Gradient rows of the points that touch several tiles: one row per instance, a point's rows one after the other in
+// the row-major order of its tiles: C + 1 values, then the two words of the call's stamp, padded
 // to whole 16-byte words. A block that ends early (every pixel saturated) leaves the rows of its remaining instances
 // unwritten: a row counts when it carries the stamp of the forward pass the rows were laid out by (64 bits, a new
-// value per execution of k_touch_scan, kept in the workspace), so nothing has to be cleared. Backward passes of one
+// value per execution of k_bin_scan, kept in the workspace), so nothing has to be cleared. Backward passes of one
 // forward pass share the stamp: they write the same rows.
 struct GradRows {
     float* values;

@@ -27,7 +27,6 @@
 #include <type_traits>
 
 #include "common.hpp"
-#include "radix.hpp"
 
 #include <hip/hip_fp16.h>
 
@@ -45,7 +44,11 @@ enum Counter : int {
     kCntInstances = 1,
     kCntError = 2,
     kCntSplit = 3,         // drawn points that touch more than one tile
+    kCntKept = 4,          // Gaussian footprint: instances that are sorted and drawn (0 when they do not fit)
     kCntOverflow = 5,      // the instances (or the gradient rows) do not fit the buffers: nothing is drawn
+    kCntInstances64 = 6,   // Gaussian footprint: u64 at words 6, 7: exact instance count
+    kCntMulti = 8,         // Gaussian footprint: drawn points that touch more than one tile
+    kCntDirect = 9,        // Gaussian footprint: set by a backward blend that added gradients to the arrays directly
     kCntRows = 10,         // instances of the points that touch more than one tile
     kCntWords = 16
 };
@@ -380,11 +383,17 @@ __device__ __forceinline__ uint32_t scan_block_exclusive(uint32_t v, uint32_t* s
     return before;
 }
 
+// GAUSSIAN: the counters of the Gaussian footprint's pipeline. Its exact instance count (a point touches any number
+// of tiles: the 32-bit sums may wrap around) has been added up by its preprocess pass, and it steps `generation`, the
+// stamp the backward pass marks its gradient rows with: a new one per forward pass *execution* (a full-period
+// congruential step in the workspace, increment from the host's per-call seed), so that a captured graph, whose
+// kernel arguments never change, still gets a new stamp on every replay.
+template <bool GAUSSIAN>
 __global__ void __launch_bounds__(kScanBlock)
     k_bin_scan(const uint32_t* __restrict__ bin_count, uint32_t* __restrict__ bin_start, uint2* ranges,
                const uint2* __restrict__ split_count, uint2* __restrict__ split_base, uint32_t* __restrict__ order,
-               uint32_t* __restrict__ counters, uint32_t n_tiles, uint32_t n_chunks, uint32_t capacity,
-               uint32_t row_capacity) {
+               uint32_t* counters, uint32_t n_tiles, uint32_t n_chunks, uint32_t capacity, uint32_t row_capacity,
+               unsigned long long* generation, unsigned long long seed) {
     __shared__ uint32_t s_count[kScanSegment], s_start[kScanSegment];
     __shared__ uint32_t s_bucket[kOrderBuckets];
     __shared__ uint32_t s_wave[kScanBlock / kWave];
@@ -408,7 +417,8 @@ __global__ void __launch_bounds__(kScanBlock)
     (void)scan_block_exclusive(mine, s_wave, n_instances);
     const uint32_t split_before = scan_block_exclusive(split.x, s_wave, n_split);
     const uint32_t rows_before = scan_block_exclusive(split.y, s_wave, n_rows);
-    const bool overflow = n_instances > capacity || n_rows > row_capacity;
+    bool overflow = n_instances > capacity || n_rows > row_capacity;
+    if (GAUSSIAN) overflow = *(const unsigned long long*)(counters + kCntInstances64) > (unsigned long long)capacity;
     if (tid < n_chunks) split_base[tid] = make_uint2(split_before, rows_before);
     for (int i = tid; i < kOrderBuckets; i += kScanBlock) s_bucket[i] = 0u;
     uint32_t carry = 0u;
@@ -476,12 +486,20 @@ __global__ void __launch_bounds__(kScanBlock)
     }
     if (tid == 0) {
         bin_start[n_tiles] = overflow ? 0u : n_instances;
-        counters[kCntVisible] = 0u;   // counted by k_bin_fill
-        counters[kCntError] = 0u;
-        counters[kCntInstances] = n_instances;
-        counters[kCntSplit] = overflow ? 0u : n_split;   // no list entry is written when nothing is drawn
-        counters[kCntRows] = n_rows;
-        counters[kCntOverflow] = overflow ? 1u : 0u;
+        if (GAUSSIAN) {
+            const unsigned long long total = *(const unsigned long long*)(counters + kCntInstances64);
+            counters[kCntKept] = overflow ? 0u : (uint32_t)total;
+            counters[kCntInstances] = total > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)total;
+            counters[kCntMulti] = overflow ? 0u : n_split;
+            if (generation) *generation = *generation * 6364136223846793005ull + (seed | 1ull);
+        } else {
+            counters[kCntVisible] = 0u;   // counted by k_bin_fill
+            counters[kCntError] = 0u;
+            counters[kCntInstances] = n_instances;
+            counters[kCntSplit] = overflow ? 0u : n_split;   // no list entry is written when nothing is drawn
+            counters[kCntRows] = n_rows;
+            counters[kCntOverflow] = overflow ? 1u : 0u;
+        }
     }
 }
 
@@ -690,45 +708,6 @@ __global__ void __launch_bounds__(kBinThreads)
             wave_sync();
         }
     }
-}
-
-// ---- tile schedule -----------------------------------------------------------------------------------------------
-// The schedule of k_bin_scan for ranges that are already there (the Gaussian footprint's).
-__global__ void __launch_bounds__(kScanBlock) k_tile_order(const uint2* __restrict__ ranges, uint32_t* __restrict__ order,
-                                                           uint32_t n_tiles) {
-    __shared__ uint32_t s_bucket[kOrderBuckets];
-    __shared__ uint32_t s_wave[kScanBlock / kWave];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    for (int i = tid; i < kOrderBuckets; i += kScanBlock) s_bucket[i] = 0u;
-    __syncthreads();
-    auto bucket_of = [&](uint32_t t) {
-        const uint2 r = ranges[t];
-        return order_bucket(r.y - r.x);
-    };
-    for (uint32_t t = tid; t < n_tiles; t += kScanBlock) atomicAdd(&s_bucket[bucket_of(t)], 1u);
-    __syncthreads();
-    constexpr int kPer = kOrderBuckets / kScanBlock;
-    uint32_t mine = 0;
-#pragma unroll
-    for (int i = 0; i < kPer; ++i) mine += s_bucket[tid * kPer + i];
-    uint32_t incl = mine;
-#pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-        const uint32_t up = __shfl_up(incl, s, 64);
-        if (lane >= (uint32_t)s) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - mine;
-    for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
-#pragma unroll
-    for (int i = 0; i < kPer; ++i) {
-        const uint32_t c = s_bucket[tid * kPer + i];
-        s_bucket[tid * kPer + i] = run;
-        run += c;
-    }
-    __syncthreads();
-    for (uint32_t t = tid; t < n_tiles; t += kScanBlock) order[atomicAdd(&s_bucket[bucket_of(t)], 1u)] = t;
 }
 
 // ---- blend: helpers shared with blend.hpp ---------------------------------------------------------------------
@@ -1100,16 +1079,13 @@ int dispatch_records(const Layout& L, const float* positions, const void* featur
 // ---- Gaussian footprint: workspace layout and launches --------------------------------------------------------
 struct GaussianLayout {
     inpc_gaussian_layout pub;
-    Geometry geo;
+    Geometry geo;   // geo.n_chunks: chunks of points of the binning kernels
     gaussian::Params prm;
-    radix::PassPlan depth_plan, tile_plan;
-    int T, C, fmode;
+    int T, C, fmode, key_bits;
     bool inference, sh;
-    uint32_t n_blocks;  // blocks of gaussian::kPointsPerBlock depth-ordered points
-    size_t zero_begin, zero_words;
-    size_t hist_depth, hist_tile, status_depth, status_tile, bases_depth, bases_tile, tile_order, block_sums;
-    size_t sorted_bounds, multi_list, grad_rows, generation;
-    size_t keys_a, keys_b, vals_a, vals_b, inst_keys_a, inst_keys_b, inst_vals_a, inst_vals_b;
+    size_t bin_table, bin_total, bin_start, tile_order, split_count, split_base;
+    size_t pairs, pairs_scratch;
+    size_t multi_list, grad_rows, generation;
 };
 
 int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
@@ -1160,14 +1136,13 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
         g.key_bias = float_bits(cam.near_plane);
         depth_bits = std::max(1, bit_length(float_bits(cam.far_plane) - g.key_bias));
     }
-    L.depth_plan = radix::make_plan(depth_bits);
+    L.key_bits = depth_bits;
     const int end_bit = bit_length(g.n_tiles - 1);
-    L.tile_plan = radix::make_plan(std::max(end_bit, 1));
     const size_t n = std::max<size_t>(g.n, 1);
     uint64_t capacity = gcfg->max_instances ? gcfg->max_instances : 4ull * g.n + 65536ull;
     if (capacity >= (1ull << 31)) return fail(INPC_E_UNSUPPORTED, "gaussian: max_instances must be below 2^31");
     prm.capacity = (uint32_t)capacity;
-    L.n_blocks = div_up((uint32_t)n, gaussian::kPointsPerBlock);
+    g.n_chunks = kBinBlocks;
 
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -1177,21 +1152,17 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
     };
     inpc_gaussian_layout& P = L.pub;
     memset(&P, 0, sizeof(P));
-    L.zero_begin = off;
-    P.counters = take(kCntWords * 4);
-    L.hist_depth = take(radix::kMaxPasses * radix::kRadix * 4);
-    L.hist_tile = take(radix::kMaxPasses * radix::kRadix * 4);
-    L.status_depth = take(L.depth_plan.n_passes * radix::status_words(g.n) * 4);
-    L.status_tile = take(L.tile_plan.n_passes * radix::status_words(prm.capacity) * 4);
+    P.counters = take(kCntWords * 4);   // cleared by the forward pass: the preprocess pass adds its counts up there
     P.tile_ranges = take((size_t)g.n_tiles * 8);
-    L.zero_words = (off - L.zero_begin) / 4;
-    L.bases_depth = take(radix::kMaxPasses * radix::kRadix * 4);
-    L.bases_tile = take(radix::kMaxPasses * radix::kRadix * 4);
+    L.bin_table = take((size_t)g.n_chunks * g.n_tiles * 4);
+    L.bin_total = take((size_t)g.n_tiles * 4);
+    L.bin_start = take((size_t)(g.n_tiles + 1) * 4);
     L.tile_order = take((size_t)g.n_tiles * 4);
-    L.block_sums = take((size_t)L.n_blocks * 4);
+    L.split_count = take(kBinBlocksWide * 8);
+    L.split_base = take(kBinBlocksWide * 8);
     P.point_touched = take(n * 4);
     P.point_bounds = take(n * 8);
-    L.sorted_bounds = take(n * 8);
+    P.depth_keys = take(n * 4);
     L.multi_list = L.grad_rows = L.generation = 0;
     if (!L.inference) {   // configurations with a backward pass
         L.generation = take(8);   // never cleared: the stamp of the gradient rows carries on from call to call
@@ -1199,19 +1170,9 @@ int make_gaussian_layout(const inpc_gaussian_config* gcfg, GaussianLayout& L) {
         L.grad_rows = take(capacity * gaussian::GradRows::words(L.C) * 4);
     }
     P.point_record = take(n * g.stride);
-    L.keys_a = take(n * 4);
-    L.keys_b = take(n * 4);
-    L.vals_a = take(n * 4);
-    L.vals_b = take(n * 4);
-    L.inst_keys_a = take(capacity * 2);
-    L.inst_keys_b = take(capacity * 2);
-    L.inst_vals_a = take(capacity * 4);
-    L.inst_vals_b = take(capacity * 4);
-    const bool depth_in_a = (L.depth_plan.n_passes % 2) == 0, tile_in_a = (L.tile_plan.n_passes % 2) == 0;
-    P.depth_keys = depth_in_a ? L.keys_a : L.keys_b;
-    P.depth_order = depth_in_a ? L.vals_a : L.vals_b;
-    P.instance_keys = tile_in_a ? L.inst_keys_a : L.inst_keys_b;
-    P.instance_points = tile_in_a ? L.inst_vals_a : L.inst_vals_b;
+    L.pairs = take(capacity * 8);
+    L.pairs_scratch = take(capacity * 8);
+    P.instance_points = take(capacity * 4);
     P.total_bytes = off;
     P.record_stride = g.stride;
     P.grid_width = g.gw;
@@ -1229,9 +1190,9 @@ int launch_gaussian_preprocess(const GaussianLayout& L, const float* positions, 
                                float* blending_weights, void* ws, hipStream_t stream) {
     INPC_LAUNCH("gaussian_preprocess", (gaussian::k_preprocess<FMODE, C>), dim3(std::min(div_up(L.geo.n, kBlock), 2048u)), dim3(kBlock),
                 stream, positions, features, opacities, scales, w2c, cam_position, at<char>(ws, L.pub.point_record),
-                at<uint32_t>(ws, L.pub.point_touched), at<uint2>(ws, L.pub.point_bounds), at<uint32_t>(ws, L.keys_a),
-                at<uint32_t>(ws, L.vals_a), blending_weights, at<uint32_t>(ws, L.pub.counters),
-                at<uint32_t>(ws, L.hist_depth), L.geo, L.prm, (float)L.T, radix::to_device_plan(L.depth_plan));
+                at<uint32_t>(ws, L.pub.point_touched), at<uint2>(ws, L.pub.point_bounds),
+                at<uint32_t>(ws, L.pub.depth_keys), blending_weights, at<uint32_t>(ws, L.pub.counters), L.geo, L.prm,
+                (float)L.T);
     return INPC_OK;
 }
 
@@ -1391,11 +1352,11 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
         rc = fill_u32(at<uint32_t>(ws, L.split_count), 0u, 2 * kBinBlocksWide, stream);
         if (rc != INPC_OK) return rc;
     }
-    INPC_LAUNCH("raster_bin_scan", k_bin_scan, dim3(1), dim3(kScanBlock), stream,
+    INPC_LAUNCH("raster_bin_scan", k_bin_scan<false>, dim3(1), dim3(kScanBlock), stream,
                 (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.pub.bin_start),
                 at<uint2>(ws, L.pub.tile_ranges), (const uint2*)at<uint2>(ws, L.split_count),
                 at<uint2>(ws, L.split_base), at<uint32_t>(ws, L.tile_order), counters, L.geo.n_tiles, L.geo.n_chunks,
-                L.geo.capacity, L.geo.row_capacity);
+                L.geo.capacity, L.geo.row_capacity, (unsigned long long*)nullptr, 0ull);
     if (L.geo.n > 0) {
         rc = L.T == 8 ? launch_bin_fill<8>(L, positions, w2c, ws, stream) : launch_bin_fill<16>(L, positions, w2c, ws, stream);
         if (rc != INPC_OK) return rc;
@@ -1553,48 +1514,75 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
     if (L.fmode == INPC_FEAT_SH36_F16 && ((uintptr_t)features & 7u) != 0)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_gaussian_forward: fp16 features must be 8-byte aligned");
 
-    rc = fill_u32(at<uint32_t>(ws, L.zero_begin), 0u, L.zero_words, stream);
-    if (rc != INPC_OK) return rc;
     uint32_t* counters = at<uint32_t>(ws, L.pub.counters);
+    rc = fill_u32(counters, 0u, kCntWords, stream);
+    if (rc != INPC_OK) return rc;
+    const uint32_t* touched = at<uint32_t>(ws, L.pub.point_touched);
+    const uint2* bounds = at<uint2>(ws, L.pub.point_bounds);
+    uint32_t* table = at<uint32_t>(ws, L.bin_table);
+    const bool big = L.geo.n_tiles > kMaxLdsTiles;
+    const uint32_t window = big ? 2u * kMaxLdsTiles : kMaxLdsTiles;
     if (L.geo.n > 0) {
         rc = dispatch_gaussian_preprocess(L, positions, features, opacities, scales, w2c, cam_position,
                                           L.inference ? nullptr : blending_weights, ws, stream);
         if (rc != INPC_OK) return rc;
-        rc = radix::sort_pairs<uint32_t>(L.depth_plan, radix::kSkipInvalid, at<uint32_t>(ws, L.keys_a),
-                                         at<uint32_t>(ws, L.vals_a), at<uint32_t>(ws, L.keys_b),
-                                         at<uint32_t>(ws, L.vals_b), counters + kCntVisible, L.geo.n,
-                                         at<uint32_t>(ws, L.hist_depth), at<uint32_t>(ws, L.bases_depth),
-                                         at<uint32_t>(ws, L.status_depth), counters + kCntError, stream,
-                                         "gaussian_depth_sort");
+        // a block keeps a 32-bit counter per tile in LDS: one launch per window of tiles (16,384 with two blocks of
+        // 512 threads per CU; with more tiles than that 32,768 with one block of 1024 threads)
+        for (uint32_t first = 0; first < L.geo.n_tiles; first += window) {
+            const uint32_t count = std::min(window, L.geo.n_tiles - first);
+            if (big) {
+                INPC_LAUNCH_LDS("gaussian_bin_count", gaussian::k_bin_count<1024>, dim3(L.geo.n_chunks), dim3(1024),
+                                (size_t)count * 4, stream, touched, bounds, table, at<uint2>(ws, L.split_count), first,
+                                count, L.geo.n, L.geo.n_chunks, L.geo.n_tiles, L.geo.gw);
+            } else {
+                INPC_LAUNCH_LDS("gaussian_bin_count", gaussian::k_bin_count<kBinThreads>, dim3(L.geo.n_chunks),
+                                dim3(kBinThreads), (size_t)count * 4, stream, touched, bounds, table,
+                                at<uint2>(ws, L.split_count), first, count, L.geo.n, L.geo.n_chunks, L.geo.n_tiles,
+                                L.geo.gw);
+            }
+        }
+        INPC_LAUNCH("raster_bin_offsets", k_bin_offsets<kBinBlocks>, dim3(div_up(L.geo.n_tiles, kWave)),
+                    dim3(kOffsetWaves * kWave), stream, table, at<uint32_t>(ws, L.bin_total), L.geo.n_tiles);
+    } else {
+        rc = fill_u32(at<uint32_t>(ws, L.bin_total), 0u, L.geo.n_tiles, stream);
         if (rc != INPC_OK) return rc;
-        const uint32_t* order = at<uint32_t>(ws, L.pub.depth_order);
-        INPC_LAUNCH("gaussian_touch_sums", gaussian::k_touch_sums, dim3(L.n_blocks), dim3(kBlock), stream, order,
-                    (const uint2*)at<uint2>(ws, L.pub.point_bounds), (const uint32_t*)counters,
-                    at<uint2>(ws, L.sorted_bounds), at<uint32_t>(ws, L.block_sums));
-        INPC_LAUNCH("gaussian_touch_scan", gaussian::k_touch_scan, dim3(1), dim3(kScanBlock), stream,
-                    at<uint32_t>(ws, L.block_sums), L.n_blocks, counters, L.prm.capacity,
-                    L.inference ? (unsigned long long*)nullptr : at<unsigned long long>(ws, L.generation),
-                    (unsigned long long)next_stamp());
-        INPC_LAUNCH("gaussian_create_instances", gaussian::k_create_instances, dim3(std::min(L.n_blocks, 2048u)), dim3(kBlock), stream,
-                    order, (const uint2*)at<uint2>(ws, L.sorted_bounds),
-                    (const uint32_t*)at<uint32_t>(ws, L.block_sums), (const uint32_t*)counters,
-                    at<uint16_t>(ws, L.inst_keys_a), at<uint32_t>(ws, L.inst_vals_a),
-                    L.inference ? (uint4*)nullptr : at<uint4>(ws, L.multi_list), counters,
-                    at<char>(ws, L.pub.point_record), L.geo.stride, at<uint32_t>(ws, L.hist_tile), L.geo.gw,
-                    radix::to_device_plan(L.tile_plan));
-        rc = radix::sort_pairs<uint16_t>(L.tile_plan, radix::kPlain, at<uint16_t>(ws, L.inst_keys_a),
-                                         at<uint32_t>(ws, L.inst_vals_a), at<uint16_t>(ws, L.inst_keys_b),
-                                         at<uint32_t>(ws, L.inst_vals_b), counters + gaussian::kCntKept, L.prm.capacity,
-                                         at<uint32_t>(ws, L.hist_tile), at<uint32_t>(ws, L.bases_tile),
-                                         at<uint32_t>(ws, L.status_tile), counters + kCntError, stream,
-                                         "gaussian_tile_sort");
+        rc = fill_u32(at<uint32_t>(ws, L.split_count), 0u, 2 * kBinBlocksWide, stream);
         if (rc != INPC_OK) return rc;
-        INPC_LAUNCH("gaussian_ranges", gaussian::k_ranges, dim3(std::min(div_up(L.prm.capacity, kBlock), 4096u)),
-                    dim3(kBlock), stream, (const uint16_t*)at<uint16_t>(ws, L.pub.instance_keys),
-                    (const uint32_t*)counters, at<uint2>(ws, L.pub.tile_ranges));
     }
-    INPC_LAUNCH("raster_tile_order", k_tile_order, dim3(1), dim3(kScanBlock), stream,
-                (const uint2*)at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), L.geo.n_tiles);
+    INPC_LAUNCH("gaussian_bin_scan", k_bin_scan<true>, dim3(1), dim3(kScanBlock), stream,
+                (const uint32_t*)at<uint32_t>(ws, L.bin_total), at<uint32_t>(ws, L.bin_start),
+                at<uint2>(ws, L.pub.tile_ranges), (const uint2*)at<uint2>(ws, L.split_count),
+                at<uint2>(ws, L.split_base), at<uint32_t>(ws, L.tile_order), counters, L.geo.n_tiles, L.geo.n_chunks,
+                L.prm.capacity, L.prm.capacity,
+                L.inference ? (unsigned long long*)nullptr : at<unsigned long long>(ws, L.generation),
+                (unsigned long long)next_stamp());
+    if (L.geo.n > 0) {
+        for (uint32_t first = 0; first < L.geo.n_tiles; first += window) {
+            const uint32_t count = std::min(window, L.geo.n_tiles - first);
+#define INPC_GAUSSIAN_FILL(THREADS_)                                                                                  \
+    INPC_LAUNCH_LDS("gaussian_bin_fill", gaussian::k_bin_fill<THREADS_>, dim3(L.geo.n_chunks), dim3(THREADS_),        \
+                    (size_t)count * 4, stream, touched, bounds, (const uint32_t*)at<uint32_t>(ws, L.pub.depth_keys), \
+                    (const uint32_t*)table, (const uint32_t*)at<uint32_t>(ws, L.bin_start), at<uint64_t>(ws, L.pairs), \
+                    (const uint2*)at<uint2>(ws, L.split_base),                                                        \
+                    L.inference ? (uint4*)nullptr : at<uint4>(ws, L.multi_list), at<char>(ws, L.pub.point_record),    \
+                    L.geo.stride, (const uint32_t*)counters, first, count, L.geo.n, L.geo.n_chunks, L.geo.n_tiles,    \
+                    L.geo.gw)
+            if (big) INPC_GAUSSIAN_FILL(1024);
+            else INPC_GAUSSIAN_FILL(kBinThreads);
+#undef INPC_GAUSSIAN_FILL
+        }
+        // the tiles with the most instances first (large blocks), then the others with small blocks
+        INPC_LAUNCH_LDS("gaussian_tile_sort", tilesort::k_tile_sort<tilesort::kLargeThreads>, dim3(L.geo.n_tiles),
+                        dim3(tilesort::kLargeThreads), sizeof(tilesort::Shared<tilesort::kLargeThreads>), stream,
+                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
+                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
+                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
+        INPC_LAUNCH_LDS("gaussian_tile_sort", tilesort::k_tile_sort<tilesort::kSmallThreads>, dim3(L.geo.n_tiles),
+                        dim3(tilesort::kSmallThreads), sizeof(tilesort::Shared<tilesort::kSmallThreads>), stream,
+                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
+                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
+                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
+    }
     return dispatch_gaussian_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }
 
@@ -1650,9 +1638,9 @@ int inpc_gaussian_read_counters(const inpc_gaussian_config* cfg, const void* ws,
         counters_host[0] = host[kCntVisible];
         counters_host[1] = host[kCntInstances];
         counters_host[2] = host[kCntError];
-        counters_host[3] = host[gaussian::kCntKept];
+        counters_host[3] = host[kCntKept];
     }
-    if (host[kCntError]) return fail(INPC_E_DEVICE, "rasterizer look-back gave up waiting (device error flag set)");
+    if (host[kCntError]) return fail(INPC_E_DEVICE, "rasterizer raised its device error flag");
     if (host[kCntInstances] > L.prm.capacity)
         return fail(INPC_E_WORKSPACE, "gaussian: %u instances do not fit max_instances = %u; nothing was drawn",
                     host[kCntInstances], L.prm.capacity);

@@ -161,7 +161,7 @@ int inpc_calibration_copy(const void* src, void* dst, size_t bytes, void* stream
 
 const char* inpc_last_error(void) { return inpc::g_error; }
 
-int inpc_abi_version(void) { return 2; }
+int inpc_abi_version(void) { return 3; }
 
 void inpc_timing_enable(int on) {
     inpc::g_timing_on = on != 0;

@@ -353,9 +353,11 @@ class GaussianRun:
             return a
 
         # the depth of a point as the sort saw it (the record's depth word of a point that touches several tiles is
-        # reused by the training configurations)
-        depth_keys = (self._buf(L.depth_keys, n, np.uint32)[:v] + np.uint32(L.depth_key_bias)).astype(np.uint32)
-        depth_order = self._buf(L.depth_order, n, np.uint32)[:v].copy()
+        # reused by the training configurations); the order the reference's depth sort would give: by (key, point)
+        point_keys = self._buf(L.depth_keys, n, np.uint32).copy()
+        assert (point_keys[~vis] == 0xFFFFFFFF).all(), "a point that is not drawn has a depth key"
+        depth_order = np.flatnonzero(vis)[np.argsort(point_keys[vis], kind="stable")].astype(np.uint32)
+        depth_keys = (point_keys[depth_order] + np.uint32(L.depth_key_bias)).astype(np.uint32)
         depth = np.zeros(n, np.float32)
         depth[depth_order] = depth_keys.view(np.float32)
         single = vis & (touched == 1)
@@ -363,14 +365,25 @@ class GaussianRun:
         if self.inference:
             assert (head[vis, 6].view(np.uint32) == depth[vis].view(np.uint32)).all(), "record depth differs from the key"
 
+        # the tiles' lists lie one after the other in tile order
+        ranges = self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2).copy()
+        lengths = (ranges[:, 1].astype(np.int64) - ranges[:, 0]).astype(np.int64)
+        filled = lengths > 0
+        assert int(lengths.sum()) == i, "the tile ranges do not add up to the instance count"
+        starts = np.concatenate([[0], np.cumsum(lengths)[:-1]])
+        assert (ranges[filled, 0] == starts[filled]).all(), "the tile ranges leave gaps or overlap"
+        instance_keys = np.repeat(np.arange(L.n_tiles, dtype=np.uint16), lengths)
+        points = self._buf(L.instance_points, max(i, 1), np.uint32)[:i].copy()
         return {
             "n_visible": v, "n_instances": i, "n_touched": touched, "bounds": bounds,
             "screen_xy": drawn(head[:, :2]), "opacity": drawn(head[:, 2]), "conic": drawn(head[:, 3:6]),
             "depth": depth, "features_view": drawn(feats),
             "depth_keys": depth_keys, "depth_order": depth_order,
-            "instance_keys": self._buf(L.instance_keys, i, np.uint16).copy(),
-            "instance_points": self._buf(L.instance_points, i, np.uint32).copy(),
-            "tile_ranges": self._buf(L.tile_ranges, 2 * L.n_tiles, np.uint32).reshape(-1, 2),
+            "instance_keys": instance_keys,
+            "instance_points": points,
+            # depth key of every instance, in final order: what the per-tile sort ordered by
+            "instance_depth_keys": (point_keys[points] + np.uint32(L.depth_key_bias)).astype(np.uint32),
+            "tile_ranges": ranges,
         }
 
     outputs = RasterRun.outputs

@@ -93,7 +93,7 @@ def make_cfg(n, w, h, tile=16, channels=8, mode=_lib.FEAT_DIRECT_F32, flags=0, m
 
 def test_layout_query_on_the_host():
     lib = _lib.lib()
-    assert lib.inpc_abi_version() >= 2
+    assert lib.inpc_abi_version() >= 3
     n = 8_388_608
     layout = _lib.RasterLayout()
     cfg = make_cfg(n, 1237, 822)
@@ -138,8 +138,8 @@ def test_gaussian_layout_query_on_the_host():
     assert (layout.grid_width, layout.grid_height, layout.n_tiles) == (155, 103, 155 * 103)
     assert layout.record_stride == 64 and layout.total_bytes % 256 == 0 and layout.end_bit == 14
     assert layout.max_instances == 4 * n + 65536          # the default capacity
-    offsets = [layout.counters, layout.point_touched, layout.point_bounds, layout.point_record, layout.depth_order,
-               layout.depth_keys, layout.instance_keys, layout.instance_points, layout.tile_ranges]
+    offsets = [layout.counters, layout.point_touched, layout.point_bounds, layout.point_record, layout.depth_keys,
+               layout.instance_points, layout.tile_ranges]
     assert all(o % 256 == 0 and o < layout.total_bytes for o in offsets) and len(set(offsets)) == len(offsets)
     # a capacity of the caller's choice sizes the instance buffers (and, in training configurations, the gradient rows)
     small = _lib.GaussianLayout()

@@ -282,6 +282,33 @@ def test_edge_cases(gpu, oracle):
     np.testing.assert_array_equal(run.outputs()["image"].view(np.uint32), ref["image"].view(np.uint32))
 
 
+@pytest.mark.parametrize("width,height,focal", [(1920, 1080, 1500.0), (2473, 1643, 2000.0)],
+                         ids=["1920x1080", "2473x1643"])
+def test_reference_tile_size_on_large_images(gpu, oracle, width, height, focal):
+    # 8x8 tiles on images of more than 16,384 tiles (32,400 and 63,860): the bins are counted and filled in windows
+    # of 32,768 tiles by blocks of 1024 threads; footprints that straddle the windows come from the near points
+    n, channels = 200000, 4
+    hv, pos, feats, opac = scene(n, channels, seed=81, width=width, height=height, focal=focal, near=300)
+    run = H.GaussianRun(hv, pos, feats, opac, 8, channels, _lib.FEAT_DIRECT_F32).forward()
+    assert run.layout.n_tiles > 16384
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, 8, channels)
+    dbg = run.debug()
+    assert dbg["n_visible"] > 0.5 * n
+    check_structure(dbg, ref)
+    out = run.outputs()
+    np.testing.assert_array_equal(out["image"].view(np.uint32), ref["image"].view(np.uint32))
+    np.testing.assert_array_equal(out["alpha"].view(np.uint32), ref["alpha"].view(np.uint32))
+    H.assert_close(out["blending_weights"], ref["blending_weights"], RTOL, 1e-7, "blending weights")
+    rng = np.random.default_rng(82)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                               gaussian=g)
+    H.assert_close(gf, gf_ref, RTOL, grad_atol(gf_ref), "feature gradients")
+    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
+
+
 def test_instances_beyond_the_capacity_are_reported(gpu, oracle):
     n = 5000
     hv, pos, feats, opac = scene(n, 4, seed=51, near=500)

@@ -1,7 +1,6 @@
 """Calls in flight on several streams at once, with a workspace each: the kernels that wait for each other's tiles
-(radix passes of the Gaussian footprint, the sampler's cull kernel) hand their tiles out through tickets, so they do
-not depend on owning the GPU; the bilinear footprint has no such kernel. Every result is compared with the oracle
-and every device error flag must be clear."""
+(the sampler's cull kernels) hand their tiles out through tickets, so they do not depend on owning the GPU; the
+rasterizer has no such kernel. Every result is compared with the oracle and every device error flag must be clear."""
 import numpy as np
 import pytest
 import torch
