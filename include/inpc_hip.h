@@ -483,15 +483,29 @@ int inpc_field_subdivide(const float* centers, const int32_t* levels, const floa
  * when the leaf has one sample. The radical inverses are accumulated in double precision as in
  * the reference's Python loop and rounded to float once, so the positions are bit-identical.
  * counts (L,) i64 dev as torch.bincount returns them; positions_out (n_samples, 3) f32 dev;
- * initial_size: 3 floats on the host. The multinomial draw in front (:130) and the optional Morton
- * order behind (:141-143, CudaUtils.MortonEncoding, not part of the reference tree) stay with the
- * caller. inpc_extract_global_check synchronises and fails unless the counts are in range and add
+ * initial_size: 3 floats on the host. The multinomial draw in front (:130) stays with the caller;
+ * inpc_morton_encode gives the codes of the optional order behind (:141-143).
+ * inpc_extract_global_check synchronises and fails unless the counts are in range and add
  * up to n_samples. */
 size_t inpc_extract_global_workspace_bytes(uint32_t n_leaves);
 int inpc_extract_global(const float* centers, const int32_t* levels, const int64_t* counts,
                         uint32_t n_leaves, const float initial_size[3], float* positions_out,
                         uint32_t n_samples, void* workspace, size_t workspace_bytes, void* stream);
 int inpc_extract_global_check(const void* workspace, uint32_t n_samples, void* stream);
+
+/* codes_out[i] = 63-bit Morton code of positions[i] in the bounding cube of all positions: with lo
+ * the per-axis minimum and e the largest per-axis extent, cell_a = min(uint((p_a - lo_a) *
+ * (2^21 / e)), 2^21 - 1) in fp32 (all cells 0 when e = 0), and bit k of cell_x / cell_y / cell_z
+ * is bit 3k / 3k + 1 / 3k + 2 of the code. Sorting by the code (torch.argsort, as the caller does)
+ * gives the order ProbabilityField.extract_global asks for with use_morton_order
+ * (Modules/ProbabilityField.py:141-143). The reference takes the codes from
+ * CudaUtils.MortonEncoding.morton_encode, an extension of its framework whose source is not part
+ * of the reference tree: this is the textbook Z-order code, equal to the reference's only as far
+ * as both are Morton orders of the same points. positions (n, 3) f32 dev, codes_out (n,) i64 dev,
+ * workspace: inpc_morton_workspace_bytes() bytes. No host synchronisation. */
+size_t inpc_morton_workspace_bytes(void);
+int inpc_morton_encode(const float* positions, uint32_t n, int64_t* codes_out, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* grads (= or +=, `add` != 0) factor(i) * weights[i], factor = 0.1 * 2 / (entries of the hash-grid
  * level that holds flat index i), 0 in front of index 6144. Replaces

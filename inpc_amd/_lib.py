@@ -152,6 +152,8 @@ SIGNATURES = {
     "inpc_extract_global_workspace_bytes": (C.c_size_t, [_U32]),
     "inpc_extract_global": (C.c_int, [_P, _P, _P, _U32, C.POINTER(C.c_float), _P, _U32, _P, C.c_size_t, _P]),
     "inpc_extract_global_check": (C.c_int, [_P, _U32, _P]),
+    "inpc_morton_workspace_bytes": (C.c_size_t, []),
+    "inpc_morton_encode": (C.c_int, [_P, _U32, _P, _P, C.c_size_t, _P]),
     "inpc_weight_decay_grads": (C.c_int, [_P, _P, _U32, C.c_int, _P]),
     "inpc_cauchy_loss": (C.c_int, [_P, _P, _P, _U32, _P]),
     "inpc_cauchy_loss_backward": (C.c_int, [_P, _P, _P, _P, _U32, _P]),

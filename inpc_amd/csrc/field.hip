@@ -335,6 +335,68 @@ __global__ void __launch_bounds__(kBlock) k_extract_global(const float* __restri
     positions[3 * (size_t)s + 2] = z;
 }
 
+// ---- Morton codes ------------------------------------------------------------------------------------
+// bounds[0..2] = ordered keys of the per-axis minima, bounds[3..5] of the maxima (set to kNoMin / kNoMax before).
+__global__ void __launch_bounds__(kBlock) k_morton_bounds(const float* __restrict__ positions, uint32_t n,
+                                                          uint32_t* __restrict__ bounds) {
+    uint32_t lo[3] = {kNoMin, kNoMin, kNoMin}, hi[3] = {kNoMax, kNoMax, kNoMax};
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            const uint32_t k = ordered_key(positions[3 * i + a]);
+            lo[a] = min(lo[a], k);
+            hi[a] = max(hi[a], k);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        for (int s = 32; s > 0; s >>= 1) {
+            lo[a] = min(lo[a], (uint32_t)__shfl_xor(lo[a], s, 64));
+            hi[a] = max(hi[a], (uint32_t)__shfl_xor(hi[a], s, 64));
+        }
+    }
+    if (lane_id() == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            atomicMin(bounds + a, lo[a]);
+            atomicMax(bounds + 3 + a, hi[a]);
+        }
+    }
+}
+
+// Bit k of v goes to bit 3 k (v < 2^21).
+__device__ __forceinline__ uint64_t spread3(uint32_t v) {
+    uint64_t x = v;
+    x = (x | (x << 32)) & 0x001F00000000FFFFull;
+    x = (x | (x << 16)) & 0x001F0000FF0000FFull;
+    x = (x | (x << 8)) & 0x100F00F00F00F00Full;
+    x = (x | (x << 4)) & 0x10C30C30C30C30C3ull;
+    x = (x | (x << 2)) & 0x1249249249249249ull;
+    return x;
+}
+
+constexpr uint32_t kMortonCells = 1u << 21;   // per axis: 63 bits in all
+
+__global__ void __launch_bounds__(kBlock) k_morton_encode(const float* __restrict__ positions, uint32_t n,
+                                                          const uint32_t* __restrict__ bounds,
+                                                          int64_t* __restrict__ codes) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const float lx = ordered_value(bounds[0]), ly = ordered_value(bounds[1]), lz = ordered_value(bounds[2]);
+    const float extent = fmaxf(fmaxf(ordered_value(bounds[3]) - lx, ordered_value(bounds[4]) - ly),
+                               ordered_value(bounds[5]) - lz);
+    const float scale = extent > 0.0f ? (float)kMortonCells / extent : 0.0f;
+    const float lo[3] = {lx, ly, lz};
+    uint64_t code = 0;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        const float q = (positions[3 * (size_t)i + a] - lo[a]) * scale;
+        const uint32_t cell = min((uint32_t)q, kMortonCells - 1u);   // q >= 0; the maximum lands on 2^21
+        code |= spread3(cell) << a;
+    }
+    codes[i] = (int64_t)code;
+}
+
 int select_offsets(const float* values, const int32_t* levels, uint32_t n, float threshold, int max_level,
                    uint32_t* block_offsets, uint32_t* counts, hipStream_t stream) {
     const uint32_t blocks = div_up(n, kSelectTile);
@@ -488,6 +550,28 @@ int inpc_extract_global_check(const void* workspace, uint32_t n_samples, void* s
     if (head[0] != n_samples)
         return fail(INPC_E_INVALID_ARGUMENT, "extract_global: the counts add up to %u, not to the %u samples asked for",
                     head[0], n_samples);
+    return INPC_OK;
+}
+
+size_t inpc_morton_workspace_bytes(void) { return 256; }
+
+int inpc_morton_encode(const float* positions, uint32_t n, int64_t* codes_out, void* workspace, size_t workspace_bytes,
+                       void* stream_) {
+    using namespace inpc;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n == 0) return INPC_OK;
+    if (!positions || !codes_out) return fail(INPC_E_INVALID_ARGUMENT, "morton_encode: null pointer");
+    if (!workspace || workspace_bytes < inpc_morton_workspace_bytes())
+        return fail(INPC_E_WORKSPACE, "morton_encode: workspace too small");
+    uint32_t* bounds = (uint32_t*)workspace;
+    int rc = fill_u32(bounds, kNoMin, 3, stream);
+    if (rc != INPC_OK) return rc;
+    rc = fill_u32(bounds + 3, kNoMax, 3, stream);
+    if (rc != INPC_OK) return rc;
+    INPC_LAUNCH("morton_bounds", k_morton_bounds, dim3(std::min(div_up(n, kBlock), 2048u)), dim3(kBlock), stream,
+                positions, n, bounds);
+    INPC_LAUNCH("morton_encode", k_morton_encode, dim3(div_up(n, kBlock)), dim3(kBlock), stream, positions, n,
+                (const uint32_t*)bounds, codes_out);
     return INPC_OK;
 }
 

@@ -127,11 +127,35 @@ def subdivide_probability_field(leaf_centers, leaf_levels, leaf_weights, leaf_su
 
 
 @torch.no_grad()
+def morton_encode(positions: torch.Tensor) -> torch.Tensor:
+    """(n,) int64 Morton codes of (n, 3) float positions in their bounding cube, 21 bits per axis, x in the lowest
+    bit: the role of `CudaUtils.MortonEncoding.morton_encode` in Modules/ProbabilityField.py:142 (that extension's
+    source is not part of the reference tree; this is the textbook Z-order code)."""
+    if positions.dtype != torch.float32:
+        raise RuntimeError("expected scalar type Float")
+    if positions.dim() != 2 or positions.shape[1] != 3:
+        raise RuntimeError("positions (n, 3) expected")
+    if not positions.is_cuda:
+        raise RuntimeError("expected tensors on the GPU")
+    positions = positions.contiguous()
+    n = positions.shape[0]
+    if n >= 2 ** 32:
+        raise RuntimeError("too many positions")
+    codes = torch.empty(n, dtype=torch.int64, device=positions.device)
+    lib = _lib.lib()
+    ws_bytes = int(lib.inpc_morton_workspace_bytes())
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=positions.device)
+    _lib.check(lib.inpc_morton_encode(_lib.ptr(positions), n, _lib.ptr(codes), _lib.ptr(ws), ws_bytes,
+                                      _lib.current_stream()), "inpc_morton_encode")
+    return codes
+
+
+@torch.no_grad()
 def extract_global_samples(leaf_centers: torch.Tensor, leaf_levels: torch.Tensor, initial_cell_size,
-                           counts: torch.Tensor) -> torch.Tensor:
+                           counts: torch.Tensor, use_morton_order: bool = False) -> torch.Tensor:
     """Quasi-random positions, counts[l] of them in leaf l, leaves in order: what ProbabilityField.extract_global
-    computes between its multinomial draw and its optional Morton ordering (Modules/ProbabilityField.py:131-140;
-    Halton points in the cell, the centre for a leaf with a single sample). `counts` is the result of
+    computes behind its multinomial draw (Modules/ProbabilityField.py:131-143; Halton points in the cell, the centre
+    for a leaf with a single sample; with `use_morton_order` sorted by `morton_encode`). `counts` is the result of
     `torch.bincount(indices, minlength=n_leaves)`."""
     if leaf_centers.dtype != torch.float32:
         raise RuntimeError("expected scalar type Float")
@@ -156,4 +180,6 @@ def extract_global_samples(leaf_centers: torch.Tensor, leaf_levels: torch.Tensor
                                        _host_size(initial_cell_size), _lib.ptr(positions), n_samples, _lib.ptr(ws),
                                        ws_bytes, stream), "inpc_extract_global")
     _lib.check(lib.inpc_extract_global_check(_lib.ptr(ws), n_samples, stream), "inpc_extract_global")
+    if use_morton_order:
+        positions = positions[torch.argsort(morton_encode(positions))].contiguous()
     return positions

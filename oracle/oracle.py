@@ -535,6 +535,26 @@ def extract_global_samples(centers, levels, initial_size, counts):
     return out
 
 
+def morton_encode(positions):
+    """63-bit Z-order codes of the positions in their bounding cube, bit by bit: cell = min(uint((p - lo) *
+    (2^21 / largest extent)), 2^21 - 1) per axis in float32, bit k of the x / y / z cell at bit 3k / 3k+1 / 3k+2.
+    Stands where Modules/ProbabilityField.py:142 calls CudaUtils.MortonEncoding.morton_encode, whose source is not in
+    the reference tree (parity with it unpinned; pinned as a Morton code by tests/test_oracle_field.py)."""
+    p = np.asarray(positions, np.float32).reshape(-1, 3)
+    if len(p) == 0:
+        return np.zeros(0, np.int64)
+    lo = p.min(0)
+    extent = np.float32((p.max(0) - lo).max())
+    scale = np.float32(2 ** 21) / extent if extent > 0 else np.float32(0.0)
+    q = ((p - lo) * np.float32(scale)).astype(np.float32)
+    cells = np.minimum(q.astype(np.uint64), np.uint64(2 ** 21 - 1))
+    codes = np.zeros(len(p), np.uint64)
+    for k in range(21):
+        for axis in range(3):
+            codes |= ((cells[:, axis] >> np.uint64(k)) & np.uint64(1)) << np.uint64(3 * k + axis)
+    return codes.astype(np.int64)
+
+
 def spherical_contraction(positions):
     """B/misc/src/misc_kernels.cu:49-66, every operation rounded to float32 in the written order."""
     p = np.asarray(positions, np.float32).reshape(-1, 3)

@@ -136,3 +136,29 @@ def test_extract_global_bit_exact(gpu, oracle):
         bad = counts.copy()
         bad[0] = -1
         extract_global_samples(H.dev(centers), H.dev(levels), size, H.dev(bad))
+
+
+def test_morton_codes_bit_exact_and_the_ordered_extraction(gpu, oracle):
+    from inpc_amd import extract_global_samples, morton_encode
+
+    rng = np.random.default_rng(41)
+    for n, spread in ((1, 1.0), (2, 1.0), (63, 1e-3), (200001, 3.0)):
+        p = (rng.normal(0, spread, (n, 3)) * np.array([1.0, 0.3, 2.0])).astype(np.float32)
+        got = morton_encode(H.dev(p)).cpu().numpy()
+        np.testing.assert_array_equal(got, oracle.morton_encode(p), err_msg=f"n = {n}")
+    assert morton_encode(H.dev(np.full((100, 3), -0.75, np.float32))).cpu().numpy().tolist() == [0] * 100
+    assert morton_encode(H.dev(np.zeros((0, 3), np.float32))).shape == (0,)
+    with pytest.raises(RuntimeError):
+        morton_encode(H.dev(np.zeros((4, 2), np.float32)))
+    # extract_global with use_morton_order: the same samples, in the order of their codes
+    n_leaves = 3000
+    centers = rng.uniform(-2, 2, (n_leaves, 3)).astype(np.float32)
+    levels = rng.integers(0, 7, n_leaves).astype(np.int32)
+    size = np.array([0.37, 0.37, 0.37], np.float32)
+    counts = np.bincount(rng.integers(0, n_leaves, 20000), minlength=n_leaves).astype(np.int64)
+    plain = oracle.extract_global_samples(centers, levels, size, counts)
+    got = extract_global_samples(H.dev(centers), H.dev(levels), size, H.dev(counts), use_morton_order=True).cpu().numpy()
+    codes = oracle.morton_encode(plain)
+    np.testing.assert_array_equal(oracle.morton_encode(got), np.sort(codes))   # the same cube, so the same codes
+    rows = lambda a: a[np.lexsort(a.T[::-1])]
+    np.testing.assert_array_equal(rows(got).view(np.uint32), rows(plain).view(np.uint32))

@@ -153,3 +153,36 @@ def test_extract_global_matches_the_references_torch_statements(oracle):
     # the first Halton points, as published: 1/2, 1/3, 1/5; 1/4, 2/3, 2/5; 3/4, 1/9, 3/5
     assert [oracle.halton_base(1, b) for b in (2, 3, 5)] == pytest.approx([1 / 2, 1 / 3, 1 / 5])
     assert [oracle.halton_base(3, b) for b in (2, 3, 5)] == pytest.approx([3 / 4, 1 / 9, 3 / 5])
+
+
+def test_morton_codes_are_the_z_order_of_the_bounding_cube(oracle):
+    # a lattice whose bounding cube is [0, 2^21]^3: the scale is exactly 1 and a cell is the coordinate itself
+    top = float(2 ** 21)
+    lattice = np.array([[0, 0, 0], [1, 0, 0], [0, 1, 0], [0, 0, 1], [1, 1, 1], [2, 0, 0], [3, 5, 6],
+                        [2 ** 21 - 1, 0, 0], [0, 2 ** 21 - 1, 2 ** 21 - 1], [top, top, top]], np.float32)
+    codes = oracle.morton_encode(lattice)
+    x_bits = sum(1 << (3 * k) for k in range(21))
+    assert codes.tolist() == [0, 1, 2, 4, 7, 8, 0b110_101_011, x_bits, 6 * x_bits, 7 * x_bits]   # the corner is clamped
+    assert codes.dtype == np.int64 and (codes >= 0).all()
+    # a 4 x 4 x 4 lattice sorted by code: octant by octant, x fastest inside each 2 x 2 x 2 block
+    g = np.stack(np.meshgrid(np.arange(4), np.arange(4), np.arange(4), indexing="ij"), -1).reshape(-1, 3)
+    pts = np.concatenate([g.astype(np.float32) * np.float32(2 ** 19), [[top, top, top]]]).astype(np.float32)
+    order = np.argsort(oracle.morton_encode(pts)[:-1], kind="stable")
+    walk = g[order]
+    first_block = [[0, 0, 0], [1, 0, 0], [0, 1, 0], [1, 1, 0], [0, 0, 1], [1, 0, 1], [0, 1, 1], [1, 1, 1]]
+    assert walk[:8].tolist() == first_block
+    assert (walk[8:16] - [2, 0, 0]).tolist() == first_block and (walk[16:24] - [0, 2, 0]).tolist() == first_block
+    assert (walk[56:] - [2, 2, 2]).tolist() == first_block
+    # a shift and a scaling by powers of two change no cell (every float operation stays exact)
+    rng = np.random.default_rng(31)
+    p = rng.integers(0, 2 ** 21, (5000, 3)).astype(np.float32)
+    p[0], p[1] = 0.0, top
+    np.testing.assert_array_equal(oracle.morton_encode(p * np.float32(0.25) - np.float32(1024.0)), oracle.morton_encode(p))
+    # the largest extent sets the cube: the short axes only use the lower cells
+    q = p * np.array([1.0, 0.5, 0.25], np.float32)
+    cells_y = sum(((oracle.morton_encode(q) >> (3 * k + 1)) & 1) << k for k in range(21))
+    assert cells_y.max() < 2 ** 20 + 1
+    # one point, identical points, no points
+    assert oracle.morton_encode(np.array([[1.5, -2.0, 3.0]], np.float32)).tolist() == [0]
+    assert oracle.morton_encode(np.full((7, 3), 0.25, np.float32)).tolist() == [0] * 7
+    assert oracle.morton_encode(np.zeros((0, 3), np.float32)).shape == (0,)
