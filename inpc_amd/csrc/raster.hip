@@ -581,14 +581,16 @@ __global__ void __launch_bounds__(kBinThreads)
     if (threadIdx.x == 0 && s_visible) atomicAdd(&counters[kCntVisible], s_visible);
 }
 
+constexpr int kRecordThreads = kBinThreads;
+
 template <int T, int FMODE, int C>
-__global__ void __launch_bounds__(kBinThreads)
+__global__ void __launch_bounds__(kRecordThreads)
     k_records(const float* __restrict__ positions, const void* __restrict__ features,
               const float* __restrict__ opacities, const float* __restrict__ w2c,
               const float* __restrict__ cam_position, char* __restrict__ records,
               float* __restrict__ blending_weights, SplitOut split, float4* __restrict__ debug_geometry,
               const uint32_t* __restrict__ counters, Geometry g) {
-    constexpr int kThreads = kBinThreads;
+    constexpr int kThreads = kRecordThreads;
     extern __shared__ __align__(16) uint32_t s_dyn[];
     float4* s_stage = (float4*)s_dyn;      // record staging, 64 rows per wave
     __shared__ uint32_t s_split, s_rows;   // next list entry / gradient row for a point of this chunk
@@ -952,6 +954,25 @@ int launch_bin_count(const Layout& L, const float* positions, const float* w2c, 
     return INPC_OK;
 }
 
+// One block per tile and launch; blocks of kSmallThreads threads sort the tiles of at most tilesort::kSmallTile
+// instances, blocks of kLargeThreads threads the others; a block whose tile belongs to the other launch ends at once.
+struct TileSortBuffers {
+    const uint2* ranges;
+    const uint32_t* order;
+    uint64_t* pairs;
+    uint64_t* scratch;
+    uint32_t* points;
+    uint32_t n_tiles;
+    int key_bits;
+};
+
+template <int THREADS>
+int launch_tile_sort(const char* name, const TileSortBuffers& b, hipStream_t stream) {
+    INPC_LAUNCH_LDS(name, tilesort::k_tile_sort<THREADS>, dim3(b.n_tiles), dim3(THREADS),
+                    sizeof(tilesort::Shared<THREADS>), stream, b.ranges, b.order, b.pairs, b.scratch, b.points, b.key_bits);
+    return INPC_OK;
+}
+
 template <int T>
 int launch_bin_fill(const Layout& L, const float* positions, const float* w2c, void* ws, hipStream_t stream) {
     const uint32_t* table = at<uint32_t>(ws, L.bin_table);
@@ -975,8 +996,8 @@ int launch_records(const Layout& L, const float* positions, const void* features
     if (L.split_list) split = SplitOut{at<uint2>(ws, L.split_base), at<uint2>(ws, L.split_list), at<uint8_t>(ws, L.row_flags)};
     char* records = at<char>(ws, L.pub.point_record);
     float4* debug = L.pub.debug_geometry ? at<float4>(ws, L.pub.debug_geometry) : (float4*)nullptr;
-    const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kBinThreads);
-    INPC_LAUNCH_LDS("raster_records", (k_records<T, FMODE, C>), dim3(L.geo.n_chunks), dim3(kBinThreads), lds, stream,
+    const size_t lds = PreprocessShape<FMODE, C>::stage_bytes(kRecordThreads);
+    INPC_LAUNCH_LDS("raster_records", (k_records<T, FMODE, C>), dim3(L.geo.n_chunks), dim3(kRecordThreads), lds, stream,
                     positions, features, opacities, w2c, cam_position, records, blending_weights, split, debug,
                     (const uint32_t*)at<uint32_t>(ws, L.pub.counters), L.geo);
     return INPC_OK;
@@ -1385,6 +1406,15 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
         }
         rc = dispatch_records(L, positions, features, opacities, w2c, cam_position,
                               L.inference ? nullptr : blending_weights, ws, record_stream);
+        // the two launches of the tile sort touch different tiles. Where most tiles are large (going by the mean number
+        // of instances per tile) the sort of the small ones runs behind the records, beside the sort of the large ones;
+        // where most are small, the few large ones would only start late that way
+        const bool small_beside = (uint64_t)L.geo.n * 5u / 4u > (uint64_t)L.geo.n_tiles * (tilesort::kSmallTile / 2u);
+        const TileSortBuffers sort{at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), at<uint64_t>(ws, L.pairs),
+                                   at<uint64_t>(ws, L.pairs_scratch), at<uint32_t>(ws, L.pub.instance_points),
+                                   L.geo.n_tiles, L.key_bits};
+        if (rc == INPC_OK && small_beside)
+            rc = launch_tile_sort<tilesort::kSmallThreads>("raster_tile_sort", sort, record_stream);
         // the caller's stream takes the second stream's work in again behind the tile sort, or wherever this
         // function is left before
         struct Join {
@@ -1401,17 +1431,9 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                         hipGetErrorString(hipGetLastError()));
         }
         if (rc != INPC_OK) return rc;
-        // tiles of more than tilesort::kSmallTile instances, then the others with small blocks
-        INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort<tilesort::kLargeThreads>, dim3(L.geo.n_tiles),
-                        dim3(tilesort::kLargeThreads), sizeof(tilesort::Shared<tilesort::kLargeThreads>), stream,
-                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
-                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
-                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
-        INPC_LAUNCH_LDS("raster_tile_sort", tilesort::k_tile_sort<tilesort::kSmallThreads>, dim3(L.geo.n_tiles),
-                        dim3(tilesort::kSmallThreads), sizeof(tilesort::Shared<tilesort::kSmallThreads>), stream,
-                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
-                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
-                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
+        rc = launch_tile_sort<tilesort::kLargeThreads>("raster_tile_sort", sort, stream);
+        if (rc == INPC_OK && !small_beside) rc = launch_tile_sort<tilesort::kSmallThreads>("raster_tile_sort", sort, stream);
+        if (rc != INPC_OK) return rc;
     }
     return dispatch_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }
@@ -1572,16 +1594,12 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
 #undef INPC_GAUSSIAN_FILL
         }
         // the tiles with the most instances first (large blocks), then the others with small blocks
-        INPC_LAUNCH_LDS("gaussian_tile_sort", tilesort::k_tile_sort<tilesort::kLargeThreads>, dim3(L.geo.n_tiles),
-                        dim3(tilesort::kLargeThreads), sizeof(tilesort::Shared<tilesort::kLargeThreads>), stream,
-                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
-                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
-                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
-        INPC_LAUNCH_LDS("gaussian_tile_sort", tilesort::k_tile_sort<tilesort::kSmallThreads>, dim3(L.geo.n_tiles),
-                        dim3(tilesort::kSmallThreads), sizeof(tilesort::Shared<tilesort::kSmallThreads>), stream,
-                        (const uint2*)at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
-                        at<uint64_t>(ws, L.pairs), at<uint64_t>(ws, L.pairs_scratch),
-                        at<uint32_t>(ws, L.pub.instance_points), L.key_bits);
+        const TileSortBuffers sort{at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), at<uint64_t>(ws, L.pairs),
+                                   at<uint64_t>(ws, L.pairs_scratch), at<uint32_t>(ws, L.pub.instance_points),
+                                   L.geo.n_tiles, L.key_bits};
+        rc = launch_tile_sort<tilesort::kLargeThreads>("gaussian_tile_sort", sort, stream);
+        if (rc == INPC_OK) rc = launch_tile_sort<tilesort::kSmallThreads>("gaussian_tile_sort", sort, stream);
+        if (rc != INPC_OK) return rc;
     }
     return dispatch_gaussian_blend_forward(L, image, alpha, blending_weights, depth_image, ws, stream);
 }
