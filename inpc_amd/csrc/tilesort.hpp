@@ -13,9 +13,9 @@
 //              counts their digits in sixteen 4-bit fields of one 64-bit register; the 16 x threads counts are
 //              scanned in digit-major order, which is a stable ranking. Digits that are the same for all
 //              elements of the tile are skipped (the depths of one tile mostly share their leading bits).
-//   ties       elements with equal keys come out in the order they were binned, which is arbitrary: a few
-//              ties are put right in place (rank by point index inside the run of equal keys); a tile with
-//              many is sorted again over all 64 bits.
+//   ties       elements with equal keys come out in the order they were binned, which is arbitrary: short runs
+//              of equal keys are put right in place (rank by point index inside the run); a tile with a long
+//              run is sorted again over all 64 bits.
 //   big tiles  more elements than fit LDS: runs of kCap elements are sorted as above and written back, then
 //              merged pairwise through global memory (rank of an element = its place in its own run + the
 //              number of smaller elements in the partner run, by binary search on the full 64 bits).
@@ -26,7 +26,8 @@ namespace tilesort {
 constexpr int kMaxPer = 15;                 // elements per thread: 3, 7, 11 or 15 (odd: conflict-free LDS rows; at
                                             // most 15: a thread's digit counts fit 4-bit fields)
 constexpr int kDigits = 16;
-constexpr uint32_t kFewTies = 16;           // threads with tied elements up to which ties are fixed in place
+constexpr uint32_t kShortRun = 16;          // ties are fixed in place while no run of equal keys reaches further than
+                                            // this from any of its elements
 constexpr uint64_t kPad = ~0ull;            // sorts behind every element
 constexpr int kLargeThreads = 512, kSmallThreads = 128;   // block sizes of the two kernels
 constexpr uint32_t kSmallTile = kSmallThreads * kMaxPer;  // tiles up to this size go to the small blocks
@@ -177,32 +178,51 @@ __device__ void sort_run(Shared<THREADS>& sh, uint32_t n, uint32_t active, int k
         }
         any = any || tied[e];
     }
-    const uint32_t threads_tied = (uint32_t)__syncthreads_count(any);
-    if (threads_tied == 0u) return;
-    if (threads_tied <= kFewTies) {
-        // few ties (runs of at most kFewTies * kPer elements): every tied element finds its run and its rank in
-        // it; all of them are read before the first one is stored
+    if (__syncthreads_or(any) == 0) return;
+    // Runs of equal keys are mostly short, however many there are: every tied element looks along its run, up to
+    // kShortRun elements to either side, and takes the place its point index gives it inside the run. All of them
+    // are read before the first one is stored. A longer run anywhere in the tile sends the tile to the sort over
+    // all 64 bits below (nothing has been stored by then).
+    {
         uint32_t at[kPer];
         uint64_t v[kPer];
+        bool long_run = false;
 #pragma unroll
         for (int e = 0; e < kPer; ++e) {
             if (!tied[e]) continue;
             const uint32_t p = t * kPer + e;
             v[e] = sh.buf[p];
-            const uint32_t key = hi32(v[e]);
-            uint32_t first = p, last = p + 1u;
-            while (first > 0u && hi32(sh.buf[first - 1u]) == key) --first;
-            while (last < n && hi32(sh.buf[last]) == key) ++last;
-            uint32_t smaller = 0;
-            for (uint32_t q = first; q < last; ++q) smaller += lo32(sh.buf[q]) < lo32(v[e]) ? 1u : 0u;
+            const uint32_t key = hi32(v[e]), mine = lo32(v[e]);
+            uint32_t first = p, last = p + 1u, smaller = 0u;
+            for (uint32_t step = 0; first > 0u; ++step) {
+                const uint64_t w = sh.buf[first - 1u];
+                if (hi32(w) != key) break;
+                if (step == kShortRun) {
+                    long_run = true;
+                    break;
+                }
+                --first;
+                smaller += lo32(w) < mine ? 1u : 0u;
+            }
+            for (uint32_t step = 0; last < n; ++step) {
+                const uint64_t w = sh.buf[last];
+                if (hi32(w) != key) break;
+                if (step == kShortRun) {
+                    long_run = true;
+                    break;
+                }
+                ++last;
+                smaller += lo32(w) < mine ? 1u : 0u;
+            }
             at[e] = first + smaller;
         }
-        __syncthreads();
+        if (__syncthreads_or(long_run) == 0) {
 #pragma unroll
-        for (int e = 0; e < kPer; ++e)
-            if (tied[e]) sh.buf[at[e]] = v[e];
-        __syncthreads();
-        return;
+            for (int e = 0; e < kPer; ++e)
+                if (tied[e]) sh.buf[at[e]] = v[e];
+            __syncthreads();
+            return;
+        }
     }
     // many ties: sort over all 64 bits, least significant digit first
     for (int shift = 0; shift < 32; shift += 4)
