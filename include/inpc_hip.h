@@ -138,8 +138,9 @@ int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, floa
 size_t inpc_cull_workspace_bytes(uint32_t n_candidates);
 
 /* Zero the round state (accepted count, consumed count) kept at the head of a cull
- * workspace. Call once before the first round of a draw. Replaces the zero-initialised
- * sample_counter tensor of B/sampling/src/sampling_api.cu:72. */
+ * workspace: the zero-initialised sample_counter tensor of B/sampling/src/sampling_api.cu:72.
+ * A round with k0 = 0 does the same by itself, so the call is only needed for a draw whose
+ * first round starts at another candidate. */
 int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream);
 
 /* One round of the training sampler: candidates k0 .. k0+n_candidates-1 of the counter-based
@@ -151,7 +152,7 @@ int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream);
  * scheduling-dependent atomic slot order is replaced by ascending candidate order.
  * The workspace records, once `capacity` entries exist, how many candidates were consumed
  * (index of the last accepted candidate + 1). The generator is NOT advanced here; see
- * inpc_cull_finish. */
+ * inpc_cull_finish. k0 = 0 starts a new draw: the state in the workspace is cleared first. */
 int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* sum_dev,
                              const float* w2c, float* positions_out, int32_t* leaf_ids_out,
                              uint32_t capacity, uint32_t k0, uint32_t n_candidates,

@@ -464,16 +464,28 @@ __global__ void __launch_bounds__(kDrawBlock)
     }
 }
 
-__global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks, CullState* st) {
+// Clears the status words of a round; the first round of a draw (k0 = 0) clears the whole state in front of them too.
+__global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks, CullState* st, bool new_draw) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n_blocks) status[i] = 0u;
-    if (i == 0) st->ticket = 0u;
+    if (new_draw && i < (uint32_t)kCullHeaderWords) ((uint32_t*)st)[i] = 0u;
+    if (!new_draw && i == 0) st->ticket = 0u;
 }
 
-// Failure pattern of B/sampling/src/sampling.cu:107-111 when the weight sum is not positive.
-__global__ void __launch_bounds__(kBlock) k_cull_failure_fill(const float* __restrict__ sum_dev, float* positions,
-                                                              int32_t* leaf_ids, uint32_t capacity) {
-    if (*sum_dev > 0.0f) return;   // the usual case: a small grid, so that returning costs next to nothing
+// End of a draw. A positive weight sum: the generator moves on by four draws per consumed candidate. Otherwise: the
+// failure pattern of B/sampling/src/sampling.cu:107-111 in the outputs (a small grid, so that the usual case costs
+// next to nothing) and the generator stays where it is.
+__global__ void __launch_bounds__(kBlock) k_cull_finish(const float* __restrict__ sum_dev, uint64_t* rng_dev,
+                                                        const CullState* st, float* positions, int32_t* leaf_ids,
+                                                        uint32_t capacity, uint32_t total_candidates) {
+    if (*sum_dev > 0.0f) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            const uint32_t consumed = st->consumed != 0u ? st->consumed : total_candidates;
+            rng_dev[0] = pcg_apply(pcg_jump(rng_dev[1], 4ull * consumed), rng_dev[0]);
+        }
+        return;
+    }
+    if (!positions || !leaf_ids) return;
     const uint32_t stride = gridDim.x * kBlock;
     for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < capacity; i += stride) {
         positions[3 * (size_t)i] = 0.0f;
@@ -481,15 +493,6 @@ __global__ void __launch_bounds__(kBlock) k_cull_failure_fill(const float* __res
         positions[3 * (size_t)i + 2] = 0.0f;
         leaf_ids[i] = -1;
     }
-}
-
-__global__ void k_cull_finish(const float* sum_dev, uint64_t* rng_dev, const CullState* st, uint32_t capacity,
-                              uint32_t total_candidates) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    if (!(*sum_dev > 0.0f)) return;
-    const uint32_t consumed = st->consumed != 0u ? st->consumed : total_candidates;
-    (void)capacity;
-    rng_dev[0] = pcg_apply(pcg_jump(rng_dev[1], 4ull * consumed), rng_dev[0]);
 }
 
 __global__ void __launch_bounds__(kBlock) k_widen_ids(const int32_t* __restrict__ ids, int64_t* __restrict__ out,
@@ -802,8 +805,8 @@ int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* 
     CullState* st = (CullState*)workspace;
     uint32_t* status = (uint32_t*)workspace + kCullHeaderWords;
     const uint32_t n_blocks = div_up(n_candidates, kDrawTile);
-    INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(n_blocks, kBlock)), dim3(kBlock), stream, status,
-                n_blocks, st);
+    INPC_LAUNCH("cull_round_reset", k_cull_round_reset, dim3(div_up(std::max(n_blocks, (uint32_t)kCullHeaderWords), kBlock)),
+                dim3(kBlock), stream, status, n_blocks, st, k0 == 0u);
     // as many blocks as the GPU holds at once; each takes tiles until none is left
     uint32_t resident = 0;
     const int rc = resident_blocks((const void*)k_sample_cull, kDrawBlock, resident);
@@ -831,11 +834,9 @@ int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_i
     hipStream_t stream = (hipStream_t)stream_;
     if (!sum_dev || !rng_dev || !workspace || workspace_bytes < sizeof(CullState))
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_cull_finish: null pointer");
-    if (capacity > 0 && positions_out && leaf_ids_out)
-        INPC_LAUNCH("cull_failure_fill", k_cull_failure_fill, dim3(std::min(div_up(capacity, kBlock), 1024u)), dim3(kBlock), stream,
-                    sum_dev, positions_out, leaf_ids_out, capacity);
-    INPC_LAUNCH("cull_finish", k_cull_finish, dim3(1), dim3(64), stream, sum_dev, rng_dev, (const CullState*)workspace,
-                capacity, total_candidates);
+    INPC_LAUNCH("cull_finish", k_cull_finish, dim3(std::max(std::min(div_up(capacity, kBlock), 1024u), 1u)), dim3(kBlock),
+                stream, sum_dev, rng_dev, (const CullState*)workspace, positions_out, leaf_ids_out, capacity,
+                total_candidates);
     return INPC_OK;
 }
 

@@ -138,7 +138,6 @@ class ProbabilityFieldSampler(torch.nn.Module):
         first = min(int(n_samples / max(self._acceptance, 1e-3) * self.OVERSAMPLE) + 4096, (1 << 30) - 1)
         cull_bytes = int(lib.inpc_cull_workspace_bytes(first))
         cull_ws = torch.empty(cull_bytes, dtype=torch.uint8, device=device)
-        _lib.check(lib.inpc_cull_begin(_lib.ptr(cull_ws), cull_bytes, stream), "inpc_cull_begin")
         k0, accepted, consumed = 0, C.c_uint32(0), C.c_uint32(0)
         n_round = first
         while True:

@@ -101,10 +101,10 @@ class CullDraw:
         self.pos = torch.full((capacity, 3), float("nan"), dtype=torch.float32, device=device)
         self.ids = torch.full((capacity,), -7, dtype=torch.int32, device=device)
         self.ws_bytes = int(self.lib.inpc_cull_workspace_bytes(max_round))
-        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=device)
+        # poisoned: the round that starts at candidate 0 clears the state of the draw itself
+        self.ws = torch.randint(0, 256, (self.ws_bytes,), dtype=torch.uint8, device=device)
         self.cam = cam_struct(hv.camera)
         self.k0 = 0
-        _lib.check(self.lib.inpc_cull_begin(_lib.ptr(self.ws), self.ws_bytes, stream()), "inpc_cull_begin")
 
     def round(self, n_candidates):
         _lib.check(self.lib.inpc_sample_cull_compact(
