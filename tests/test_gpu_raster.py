@@ -223,6 +223,36 @@ def test_edge_cases(gpu, oracle, tile):
     compare(np.stack([wx, wy, np.full_like(wx, z)], 1), "pixel / tile boundaries")
 
 
+@pytest.mark.parametrize("tile", [8, 16])
+@pytest.mark.parametrize("levels", [40000, 2500, 400, 30], ids=lambda v: f"{v}depths")
+def test_runs_of_equal_depth_keys(gpu, oracle, tile, levels):
+    # Depths from a set of `levels` values: in a tile of some thousand instances that gives hardly any ties, many runs
+    # of two or three equal keys, runs around the length up to which the tile sort puts ties right in place (16), or
+    # runs of hundreds (sorted again over the point indices). The instance order inside a run is by point index.
+    n, channels = 60000, 4
+    hv = synthetic.camera_on_z(64, 48, 50.0, 3.0)
+    rng = np.random.default_rng(levels)
+    depth = 3.0 + rng.integers(0, levels, n) / levels          # camera space, 3 .. 4
+    u, v = rng.uniform(0, 64, n), rng.uniform(0, 48, n)
+    pos = np.stack([(u - 32.0) / 50.0 * depth, (v - 24.0) / 50.0 * depth, depth - 3.0], 1).astype(np.float32)
+    feats, opac = synthetic.point_attributes(n, channels, "uniform", 5)
+    opac *= 0.01
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32).forward()
+    ref = oracle.raster_forward(oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32), pos, feats, opac,
+                                hv.w2c, debug=True)
+    dbg = run.debug()
+    check_structure(dbg, ref)
+    keys, ranges = dbg["instance_depth_keys"], dbg["tile_ranges"].astype(np.int64)
+    same = keys[1:] == keys[:-1]
+    same[ranges[1:, 0][ranges[1:, 0] < len(keys)] - 1] = False     # a run ends with its tile
+    if levels == 40000:
+        assert 0 < same.mean() < 0.2
+    elif levels == 30:
+        assert same.mean() > 0.9
+    out = run.outputs()
+    H.assert_close(out["image"], ref["image"], RTOL, 1e-5, "image")
+
+
 def test_too_many_tiles_is_rejected(gpu):
     # 65,536 tiles are the reference's limit (16-bit tile key, kernels.cu:204,214); one more is refused
     hv = synthetic.camera_on_z(8 * 257, 8 * 256, 500.0, 3.0)
