@@ -1404,15 +1404,19 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
                 lane = nullptr;
             }
         }
+        // the sort of the large tiles goes first (the blocks of the longest tiles are the ones to start early), then
+        // the records beside it
+        const TileSortBuffers sort{at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), at<uint64_t>(ws, L.pairs),
+                                   at<uint64_t>(ws, L.pairs_scratch), at<uint32_t>(ws, L.pub.instance_points),
+                                   L.geo.n_tiles, L.key_bits};
+        const int rc_sort = launch_tile_sort<tilesort::kLargeThreads>("raster_tile_sort", sort, stream);
         rc = dispatch_records(L, positions, features, opacities, w2c, cam_position,
                               L.inference ? nullptr : blending_weights, ws, record_stream);
+        if (rc == INPC_OK) rc = rc_sort;
         // the two launches of the tile sort touch different tiles. Where most tiles are large (going by the mean number
         // of instances per tile) the sort of the small ones runs behind the records, beside the sort of the large ones;
         // where most are small, the few large ones would only start late that way
         const bool small_beside = (uint64_t)L.geo.n * 5u / 4u > (uint64_t)L.geo.n_tiles * (tilesort::kSmallTile / 2u);
-        const TileSortBuffers sort{at<uint2>(ws, L.pub.tile_ranges), at<uint32_t>(ws, L.tile_order), at<uint64_t>(ws, L.pairs),
-                                   at<uint64_t>(ws, L.pairs_scratch), at<uint32_t>(ws, L.pub.instance_points),
-                                   L.geo.n_tiles, L.key_bits};
         if (rc == INPC_OK && small_beside)
             rc = launch_tile_sort<tilesort::kSmallThreads>("raster_tile_sort", sort, record_stream);
         // the caller's stream takes the second stream's work in again behind the tile sort, or wherever this
@@ -1430,8 +1434,6 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
             return fail(INPC_E_HIP, "inpc_raster_forward: cannot record on the record stream: %s",
                         hipGetErrorString(hipGetLastError()));
         }
-        if (rc != INPC_OK) return rc;
-        rc = launch_tile_sort<tilesort::kLargeThreads>("raster_tile_sort", sort, stream);
         if (rc == INPC_OK && !small_beside) rc = launch_tile_sort<tilesort::kSmallThreads>("raster_tile_sort", sort, stream);
         if (rc != INPC_OK) return rc;
     }
