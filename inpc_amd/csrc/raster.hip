@@ -8,7 +8,7 @@
 //                    and the schedule of the per-tile blocks: tiles with the longest instance lists first
 //   k_bin_fill       project, cull, tile bounds, depth key: a (depth key, point) pair per instance into the bin of
 //                    its tile (kernels.cu:11-84,198-220)
-//   k_records        (on a second stream, beside k_bin_fill and the tile sort) the blend record of a drawn point:
+//   k_records        (on a second stream, beside the tile sort) the blend record of a drawn point:
 //                    footprint weights, opacity, view features, at the point's place in the record array
 //                    (kernels.cu:11-84,106-184)
 //   tilesort.hpp     one block per tile sorts its bin by (depth key, point index) inside LDS: the order the
