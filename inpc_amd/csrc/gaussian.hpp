@@ -195,45 +195,60 @@ __global__ void __launch_bounds__(kBlock)
 constexpr uint32_t kOwnTiles = 64;
 constexpr int kQueue = 512;   // queued points per block; further ones are walked by their owner after all
 
-// Calls point(i, touched, bounds) once for every drawn point of the block's points [begin, end) and then visit(i, tile)
-// for the tiles of its rectangle in the rows that the window [tile_first, tile_first + tile_count) of tile ids reaches
-// into (the first and the last of these rows may lie partly outside the window: visit checks).
+// Calls point(i, touched, bounds) once for every drawn point of the block's points [begin, end) and then
+// visit(i, key, tile) for the tiles of its rectangle in the rows that the window [tile_first, tile_first + tile_count)
+// of tile ids reaches into (the first and the last of these rows may lie partly outside the window: visit checks).
+// `keys` may be null (key 0). A thread takes kUnroll points per round, their loads issued together.
 template <int THREADS, typename Point, typename Visit>
 __device__ __forceinline__ void for_each_instance(const uint32_t* __restrict__ touched, const uint2* __restrict__ bounds,
-                                                  uint32_t begin, uint32_t end, uint32_t gw, uint32_t tile_first,
-                                                  uint32_t tile_count, uint32_t* s_queue, uint32_t* s_queued,
-                                                  Point point, Visit visit) {
+                                                  const uint32_t* __restrict__ keys, uint32_t begin, uint32_t end,
+                                                  uint32_t gw, uint32_t tile_first, uint32_t tile_count,
+                                                  uint32_t* s_queue, uint32_t* s_queued, Point point, Visit visit) {
     constexpr uint32_t kThreads = THREADS;
+    constexpr int kUnroll = 8;
     const uint32_t band_y0 = tile_first / gw, band_y1 = (tile_first + tile_count + gw - 1u) / gw;
     if (threadIdx.x == 0) *s_queued = 0u;
     __syncthreads();
-    for (uint32_t base = begin; base < end; base += kThreads) {
-        const uint32_t i = base + threadIdx.x;
-        const uint32_t count = i < end ? touched[i] : 0u;
-        if (count == 0u) continue;
-        const uint2 b = bounds[i];
-        point(i, count, b);
-        const uint32_t x0 = b.x & 0xFFFFu, x1 = b.x >> 16;
-        const uint32_t y0 = max(b.y & 0xFFFFu, band_y0), y1 = min(b.y >> 16, band_y1);
-        if (y0 >= y1) continue;
-        if ((x1 - x0) * (y1 - y0) > kOwnTiles) {
-            const uint32_t slot = atomicAdd(s_queued, 1u);
-            if (slot < (uint32_t)kQueue) {
-                s_queue[slot] = i;
-                continue;
-            }
+    for (uint32_t base = begin; base < end; base += kUnroll * kThreads) {
+        uint32_t count[kUnroll], key[kUnroll];
+        uint2 b[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            // a thread behind the end reads the chunk's first point and drops it
+            const uint32_t at = base + u * kThreads + threadIdx.x;
+            const uint32_t i = at < end ? at : begin;
+            count[u] = touched[i];
+            b[u] = bounds[i];
+            key[u] = keys ? keys[i] : 0u;
         }
-        for (uint32_t ty = y0; ty < y1; ++ty)
-            for (uint32_t tx = x0; tx < x1; ++tx) visit(i, ty * gw + tx);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t i = base + u * kThreads + threadIdx.x;
+            if (i >= end || count[u] == 0u) continue;
+            point(i, count[u], b[u]);
+            const uint32_t x0 = b[u].x & 0xFFFFu, x1 = b[u].x >> 16;
+            const uint32_t y0 = max(b[u].y & 0xFFFFu, band_y0), y1 = min(b[u].y >> 16, band_y1);
+            if (y0 >= y1) continue;
+            if ((x1 - x0) * (y1 - y0) > kOwnTiles) {
+                const uint32_t slot = atomicAdd(s_queued, 1u);
+                if (slot < (uint32_t)kQueue) {
+                    s_queue[slot] = i;
+                    continue;
+                }
+            }
+            for (uint32_t ty = y0; ty < y1; ++ty)
+                for (uint32_t tx = x0; tx < x1; ++tx) visit(i, key[u], ty * gw + tx);
+        }
     }
     __syncthreads();
     const uint32_t queued = min(*s_queued, (uint32_t)kQueue);
     for (uint32_t q = 0; q < queued; ++q) {
         const uint32_t i = s_queue[q];
         const uint2 b = bounds[i];
+        const uint32_t key = keys ? keys[i] : 0u;
         const uint32_t x0 = b.x & 0xFFFFu, nx = (b.x >> 16) - x0;
         const uint32_t y0 = max(b.y & 0xFFFFu, band_y0), ny = min(b.y >> 16, band_y1) - y0;
-        for (uint32_t r = threadIdx.x; r < nx * ny; r += kThreads) visit(i, (y0 + r / nx) * gw + x0 + r % nx);
+        for (uint32_t r = threadIdx.x; r < nx * ny; r += kThreads) visit(i, key, (y0 + r / nx) * gw + x0 + r % nx);
     }
 }
 
@@ -253,14 +268,14 @@ __global__ void __launch_bounds__(THREADS)
     const uint32_t begin = min(blockIdx.x * chunk, n), end = min(begin + chunk, n);
     uint32_t my_split = 0u, my_rows = 0u;
     for_each_instance<THREADS>(
-        touched, bounds, begin, end, gw, tile_first, tile_count, s_queue, &s_queued,
+        touched, bounds, (const uint32_t*)nullptr, begin, end, gw, tile_first, tile_count, s_queue, &s_queued,
         [&](uint32_t, uint32_t count, uint2) {
             if (count > 1u) {
                 my_split += 1u;
                 my_rows += count;
             }
         },
-        [&](uint32_t, uint32_t tile) {
+        [&](uint32_t, uint32_t, uint32_t tile) {
             const uint32_t local = tile - tile_first;   // wraps around for a tile in front of the window
             if (local < tile_count) atomicAdd(&s_count[local], 1u);
         });
@@ -301,7 +316,7 @@ __global__ void __launch_bounds__(THREADS)
     const uint32_t chunk = bin_chunk_size(n, n_chunks);
     const uint32_t begin = min(blockIdx.x * chunk, n), end = min(begin + chunk, n);
     for_each_instance<THREADS>(
-        touched, bounds, begin, end, gw, tile_first, tile_count, s_queue, &s_queued,
+        touched, bounds, keys, begin, end, gw, tile_first, tile_count, s_queue, &s_queued,
         [&](uint32_t i, uint32_t count, uint2 b) {
             if (lists && count > 1u) {
                 const uint32_t first_row = atomicAdd(&s_rows, count);
@@ -310,9 +325,9 @@ __global__ void __launch_bounds__(THREADS)
                 multi_list[atomicAdd(&s_split, 1u)] = make_uint4(first_row, count, i, 0u);
             }
         },
-        [&](uint32_t i, uint32_t tile) {
+        [&](uint32_t i, uint32_t key, uint32_t tile) {
             const uint32_t local = tile - tile_first;
-            if (local < tile_count) pairs[atomicAdd(&s_cursor[local], 1u)] = ((uint64_t)keys[i] << 32) | (uint64_t)i;
+            if (local < tile_count) pairs[atomicAdd(&s_cursor[local], 1u)] = ((uint64_t)key << 32) | (uint64_t)i;
         });
 }
 
