@@ -791,7 +791,11 @@ int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* 
                              uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam, const uint64_t* rng_dev,
                              void* workspace, size_t workspace_bytes, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
-    if (n_candidates == 0) return INPC_OK;
+    if (n_candidates == 0) {   // nothing to draw; a new draw still starts from a cleared state
+        if (k0 == 0u && workspace && workspace_bytes >= sizeof(CullState))
+            return fill_u32(workspace, 0u, kCullHeaderWords, stream);
+        return INPC_OK;
+    }
     if (!cam || n_leaves == 0 || !boxes || !cdf || !sum_dev || !w2c || !positions_out || !leaf_ids_out || !rng_dev ||
         !workspace)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample_cull_compact: null pointer or no leaves");
