@@ -96,20 +96,26 @@ int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* 
 /* Bytes of scratch the CDF / counting passes need for n_leaves leaves. */
 size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
 
-/* Floats in the head of a CDF: the total and the top 14 levels of the search tree. */
+/* Floats in the head of a CDF: the total and the top levels of the search tree (the binary search
+ * of B/sampling/include/sampling_utils.h:49-69): 14 levels, which the sampling kernels keep in LDS,
+ * and for an octree of more than 278,527 leaves as many more as leave a search with at most sixteen
+ * elements (they are read from memory in place of the CDF itself). inpc_cdf_head_floats gives the
+ * size of the head for n_leaves leaves: INPC_CDF_HEAD_FLOATS = 2^14 up to 278,527 leaves, the next
+ * powers of two beyond (2^17 for 2,097,152 leaves). */
 #define INPC_CDF_HEAD_FLOATS 16384
+size_t inpc_cdf_head_floats(uint32_t n_leaves);
 
 /* Normalise the leaf weights and turn them into an inclusive CDF, in place.
  * Replaces compute_cdf (B/sampling/src/sampling.cu:150-186): cub::DeviceReduce::Sum, the
  * reciprocal-multiply normalisation (B/sampling/src/sampling_kernels.cu:66-75) and
  * cub::DeviceScan::InclusiveSum. The float association order is fixed: left-to-right inside
  * chunks of 64, chunk totals combined the same way one level up, recursively.
- * `sum_out` (dev, INPC_CDF_HEAD_FLOATS floats, 16-byte aligned) is the head of the CDF: [0]
+ * `sum_out` (dev, inpc_cdf_head_floats(n_leaves) floats, 16-byte aligned) is the head of the CDF: [0]
  * receives the un-normalised total; when it is <= 0 the weights are left un-normalised and later
  * sampling kernels take the failure path themselves. [1 .. INPC_CDF_HEAD_FLOATS - 1] receive
  * the CDF elements that the first 14 probes of the binary search of B/sampling/src/
- * sampling_kernels.cu:101-126 can read, in heap order; the sampling kernels keep them in LDS.
- * Every later call that takes `sum_dev` takes this buffer. No host synchronisation. */
+ * sampling_kernels.cu:101-126 can read, in heap order, and behind them those of the further
+ * levels. Every later call that takes `sum_dev` takes this buffer. No host synchronisation. */
 int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t workspace_bytes,
                    uint32_t n_leaves, void* stream);
 

@@ -149,6 +149,7 @@ SIGNATURES = {
     "inpc_field_prune": (C.c_int, [_P, _P, _P, _P, _U32, C.c_float, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "inpc_field_subdivide": (C.c_int, [_P, _P, _P, _P, _U32, C.c_float, C.c_int, C.POINTER(C.c_float), _P, _P, _P, _P,
                                        _P, _P, C.c_size_t, _P]),
+    "inpc_cdf_head_floats": (C.c_size_t, [_U32]),
     "inpc_extract_global_workspace_bytes": (C.c_size_t, [_U32]),
     "inpc_extract_global": (C.c_int, [_P, _P, _P, _U32, C.POINTER(C.c_float), _P, _U32, _P, C.c_size_t, _P]),
     "inpc_extract_global_check": (C.c_int, [_P, _U32, _P]),

@@ -174,7 +174,6 @@ __global__ void __launch_bounds__(kBlock) k_chunk_add_prefix(float* data, uint32
 // whose 64 lanes touch 64 different lines and costs the kernel as much as all its arithmetic (13 levels for 256
 // threads: cull kernel 0.32 instead of 0.27 ms).
 constexpr uint32_t kFetch = 16;   // elements of a search that four lanes fetch together
-constexpr uint32_t kFetchLeaves = 1u << 20;   // up to this many leaves
 constexpr int kTreeDepth = 14;
 constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNodes - 1; index 0 of the head: the total
 static_assert(kTreeNodes == INPC_CDF_HEAD_FLOATS, "the CDF head holds the total and the search tree");
@@ -182,9 +181,9 @@ static_assert(kSampleItems * (kDrawBlock / kWave) <= kWave, "one wave scans the 
 
 // head[node] for every node of the tree (one thread per node).
 __global__ void __launch_bounds__(kBlock) k_build_search_tree(const float* __restrict__ cdf, float* __restrict__ head,
-                                                              uint32_t n) {
+                                                              uint32_t n, uint32_t n_nodes) {
     const uint32_t node = blockIdx.x * kBlock + threadIdx.x;
-    if (node == 0u || node >= kTreeNodes) return;
+    if (node == 0u || node >= n_nodes) return;
     // replay the decisions that lead to this node
     const int depth = 31 - __clz(node);
     uint32_t first = 0, count = n;
@@ -198,6 +197,17 @@ __global__ void __launch_bounds__(kBlock) k_build_search_tree(const float* __res
         }
     }
     head[node] = count > 0 ? cdf[first + (count >> 1)] : 0.0f;
+}
+
+// Levels of the tree for n leaves: at least kTreeDepth (the part a block keeps in LDS), and as many as leave a search
+// with at most kFetch elements (every level halves what is left). The levels below kTreeDepth are read from the head
+// in memory: for 2,097,152 leaves three levels, 448 KB that stay in the second-level cache, where probes of the CDF
+// itself fetch a 128-byte line from memory for every 4-byte element (12.9 GB for 33,554,432 samples).
+constexpr int kMaxTreeDepth = 24;
+__host__ __device__ __forceinline__ int tree_levels(uint32_t n_leaves) {
+    int levels = kTreeDepth;
+    while (levels < kMaxTreeDepth && (n_leaves >> levels) > kFetch) ++levels;
+    return levels;
 }
 
 // Every thread of the block must call it; ends with a barrier. s_tree[0] (the total) is not used.
@@ -249,7 +259,8 @@ __device__ __forceinline__ TileJumps make_tile_jumps(uint64_t inc) {
 // `state0`: the generator at the first draw of the thread's first candidate; live[j]: candidate j exists.
 __device__ __forceinline__ void draw_candidates(uint64_t state0, const TileJumps& jumps, const bool (&live)[kSampleItems],
                                                 const float4* __restrict__ boxes, const float* __restrict__ cdf,
-                                                const float* s_tree, uint32_t n_leaves, Candidate (&c)[kSampleItems]) {
+                                                const float* __restrict__ head, const float* s_tree,
+                                                uint32_t n_leaves, Candidate (&c)[kSampleItems]) {
     float u[kSampleItems], ox[kSampleItems], oy[kSampleItems], oz[kSampleItems];
 #pragma unroll
     for (int j = 0; j < kSampleItems; ++j) {
@@ -279,14 +290,31 @@ __device__ __forceinline__ void draw_candidates(uint64_t state0, const TileJumps
             node[j] = active ? 2u * node[j] + (right ? 1u : 0u) : node[j];
         }
     }
-    // The probes below it read the CDF itself, one search after the other: a probe is a load whose 64 lanes read 64
-    // different lines, and what it costs goes with the lines it looks up. So a search only probes until kFetch elements
-    // are left; these are fetched by four neighbouring lanes, 16 bytes each (one or two lines per search instead of
-    // one per probe and lane), and the rest of the search is the number of fetched elements below the sample: the CDF
-    // is non-decreasing, so that is where the reference's probe sequence ends as well. (Measured with 8,388,608 samples:
-    // -6 % for 131,072 leaves, -13 % for 262,144 and 524,288, -7 % for 1,048,576; with 2,097,152 leaves, where three
-    // probes come first and have brought the lines in, +7 %: there every search probes to its end.)
-    const bool wide = n_leaves >= kFetch && n_leaves <= kFetchLeaves;
+    // the levels of the tree below that are read from the head in memory, all eight searches level by level again
+    const int levels = tree_levels(n_leaves);
+#pragma unroll 1
+    for (int level = kTreeDepth; level < levels; ++level) {
+        float key[kSampleItems];
+#pragma unroll
+        for (int j = 0; j < kSampleItems; ++j) key[j] = head[node[j]];
+#pragma unroll
+        for (int j = 0; j < kSampleItems; ++j) {
+            const bool active = count[j] > 0u;
+            const uint32_t step = count[j] >> 1;
+            const bool right = key[j] < u[j];
+            first[j] = active && right ? first[j] + step + 1u : first[j];
+            count[j] = !active ? 0u : right ? count[j] - (step + 1u) : step;
+            node[j] = active ? 2u * node[j] + (right ? 1u : 0u) : node[j];
+        }
+    }
+    // What is left of a search (at most kFetch elements, see tree_levels) reads the CDF itself. A probe is a load whose
+    // 64 lanes read 64 different lines, and what it costs goes with the lines it looks up: so four neighbouring lanes
+    // fetch the kFetch elements from the search's first one on, 16 bytes each (one or two lines per search instead of
+    // one per probe and lane), compare them with the sample, and the search's own lane makes the remaining probes of
+    // the reference's sequence on these sixteen outcomes. (The CDF is not monotone everywhere: where a chunk of the
+    // blocked scan ends an element can be an ulp above the next one, so the probe sequence itself is kept.)
+    // (Measured with 8,388,608 samples: -6 % for 131,072 leaves, -13 % for 262,144.)
+    const bool wide = n_leaves >= kFetch;
 #pragma unroll
     for (int j = 0; j < kSampleItems; ++j) {
         while (count[j] > (wide ? kFetch : 0u)) {
@@ -304,30 +332,34 @@ __device__ __forceinline__ void draw_candidates(uint64_t state0, const TileJumps
         const uint32_t lane = lane_id(), group = lane >> 2, part = lane & 3u;
 #pragma unroll
         for (int j = 0; j < kSampleItems; ++j) {
-            uint32_t below = 0u;
+            uint32_t below = 0u;   // bit i: element base + i is below the sample
 #pragma unroll
             for (uint32_t r = 0; r < 4u; ++r) {
                 // this sub-round serves the searches of lanes 16 r .. 16 r + 15; the lane helps with that of `owner`
                 const uint32_t owner = r * 16u + group;
                 const uint32_t f = (uint32_t)__shfl((int)first[j], (int)owner, 64);
-                const uint32_t n_left = (uint32_t)__shfl((int)count[j], (int)owner, 64);
                 const float sample = __shfl(u[j], (int)owner, 64);
                 const uint32_t base = min(f, n_leaves - kFetch);   // the fetch stays inside the array
-                const uint32_t at = base + 4u * part, lo = f - base;
                 float e[4];
-                __builtin_memcpy(e, cdf + at, 16);   // 4-byte aligned
+                __builtin_memcpy(e, cdf + base + 4u * part, 16);   // 4-byte aligned
                 uint32_t mine = 0u;
 #pragma unroll
-                for (uint32_t k = 0; k < 4u; ++k) {
-                    const uint32_t idx = 4u * part + k;   // inside [lo, lo + n_left): an element of the search
-                    mine += (idx - lo < n_left && e[k] < sample) ? 1u : 0u;
-                }
-                mine += (uint32_t)__shfl_xor((int)mine, 1, 64);
-                mine += (uint32_t)__shfl_xor((int)mine, 2, 64);
+                for (uint32_t k = 0; k < 4u; ++k) mine |= (e[k] < sample ? 1u : 0u) << (4u * part + k);
+                mine |= (uint32_t)__shfl_xor((int)mine, 1, 64);
+                mine |= (uint32_t)__shfl_xor((int)mine, 2, 64);
                 const uint32_t got = (uint32_t)__shfl((int)mine, (int)((lane & 15u) * 4u), 64);
                 if ((lane >> 4) == r) below = got;
             }
-            first[j] += below;
+            const uint32_t base = min(first[j], n_leaves - kFetch);
+#pragma unroll
+            for (int probe = 0; probe < 5; ++probe) {   // 16 elements: at most five probes
+                const bool active = count[j] > 0u;
+                const uint32_t step = count[j] >> 1;
+                const uint32_t it = first[j] + step;
+                const bool right = ((below >> ((it - base) & 31u)) & 1u) != 0u;
+                first[j] = active && right ? it + 1u : first[j];
+                count[j] = !active ? 0u : right ? count[j] - (step + 1u) : step;
+            }
         }
     }
     float4 box[kSampleItems];
@@ -366,7 +398,7 @@ __global__ void __launch_bounds__(kDrawBlock) k_sample(const float4* __restrict_
 #pragma unroll
     for (int j = 0; j < kSampleItems; ++j) live[j] = tile_first + (uint64_t)j * kDrawBlock + threadIdx.x < n_samples;
     Candidate c[kSampleItems];
-    draw_candidates(r.state, jumps, live, boxes, cdf, s_tree, n_leaves, c);
+    draw_candidates(r.state, jumps, live, boxes, cdf, sum_dev, s_tree, n_leaves, c);
 #pragma unroll
     for (int j = 0; j < kSampleItems; ++j) {
         const uint64_t k = tile_first + (uint64_t)j * kDrawBlock + threadIdx.x;
@@ -455,7 +487,7 @@ __global__ void __launch_bounds__(kDrawBlock)
         bool keep[kSampleItems];
 #pragma unroll
         for (int j = 0; j < kSampleItems; ++j) keep[j] = tile_first + (uint64_t)j * kDrawBlock + tid < n_candidates;
-        draw_candidates(state0, jumps, keep, boxes, cdf, s_tree, n_leaves, cand);
+        draw_candidates(state0, jumps, keep, boxes, cdf, sum_dev, s_tree, n_leaves, cand);
 #pragma unroll
         for (int j = 0; j < kSampleItems; ++j) {
             keep[j] = keep[j] && sample_accepted(m, cand[j].x, cand[j].y, cand[j].z, cam);
@@ -714,8 +746,9 @@ int launch_build_cdf(float* w, float* sum_out, float* totals, uint32_t n_leaves,
         INPC_LAUNCH("chunk_add_prefix", k_chunk_add_prefix, dim3(div_up(dn, kBlock)), dim3(kBlock), stream, dst, dn,
                     (const float*)(totals + plan.offset[d]), (const float*)sum_out);
     }
-    INPC_LAUNCH("search_tree", k_build_search_tree, dim3(kTreeNodes / kBlock), dim3(kBlock), stream, (const float*)w,
-                sum_out, n_leaves);
+    const uint32_t n_nodes = 1u << tree_levels(n_leaves);
+    INPC_LAUNCH("search_tree", k_build_search_tree, dim3(n_nodes / kBlock), dim3(kBlock), stream, (const float*)w, sum_out,
+                n_leaves, n_nodes);
     return INPC_OK;
 }
 
@@ -774,6 +807,8 @@ int inpc_leaf_weights(const float* centers, const int32_t* levels, const float* 
 }
 
 size_t inpc_sampler_workspace_bytes(uint32_t n_leaves) { return sampler_workspace_bytes(n_leaves); }
+
+size_t inpc_cdf_head_floats(uint32_t n_leaves) { return (size_t)1 << tree_levels(n_leaves); }
 
 int inpc_build_cdf(float* w, float* sum_out, void* workspace, size_t workspace_bytes, uint32_t n_leaves,
                    void* stream_) {

@@ -102,7 +102,8 @@ class ProbabilityFieldSampler(torch.nn.Module):
                    "inpc_leaf_weights")
         ws_bytes = int(lib.inpc_sampler_workspace_bytes(max(n, 1)))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=centers.device)
-        total = torch.zeros(_lib.CDF_HEAD_FLOATS, dtype=torch.float32, device=centers.device)  # CDF head; [0] = total
+        head_floats = int(lib.inpc_cdf_head_floats(max(n, 1)))
+        total = torch.zeros(head_floats, dtype=torch.float32, device=centers.device)  # CDF head; [0] = total
         return vw, boxes, ws, ws_bytes, total, cam, stream
 
     def _cdf(self, centers, levels, weights, w2c, view, initial_size):

@@ -72,7 +72,7 @@ def build_cdf(w_dev):
     cdf = w_dev.clone()
     ws_bytes = int(lib.inpc_sampler_workspace_bytes(n))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_dev.device)
-    total = torch.zeros(_lib.CDF_HEAD_FLOATS, dtype=torch.float32, device=w_dev.device)  # CDF head; [0] = total
+    total = torch.zeros(int(lib.inpc_cdf_head_floats(n)), dtype=torch.float32, device=w_dev.device)  # [0] = total
     _lib.check(lib.inpc_build_cdf(_lib.ptr(cdf), _lib.ptr(total), _lib.ptr(ws), ws_bytes, n, stream()),
                "inpc_build_cdf")
     return cdf, total

@@ -77,6 +77,36 @@ def test_sample_bit_exact_and_stream_continues(gpu, oracle, n_samples):
         assert H.rng_values(rng_dev) == (int(rng_ref.state[0]), int(rng_ref.state[1]))
 
 
+@pytest.mark.parametrize("n_leaves,level", [(15, 3), (16, 3), (17, 3), (262144, 9), (278527, 9), (278528, 9),
+                                            (300001, 9), (1048576, 10), (1500003, 11)])
+def test_sample_bit_exact_across_octree_sizes(gpu, oracle, n_leaves, level):
+    # The searches end in three ways: probes to the last element (fewer than 16 leaves), the last 16 elements fetched
+    # by four lanes (up to 278,527 leaves), and further tree levels read from memory in front of that (more leaves;
+    # sizes that are not powers of two leave the tree with ranges that do not start at multiples of 16). Many equal CDF
+    # elements (leaves outside the frustum weigh nothing), elements an ulp above their successor (where a chunk of the
+    # blocked scan ends) and samples at both ends of the CDF come with the scene.
+    oct, hv = small_scene(n_leaves, level, seed=5, mixed_levels=False, distance=1.5)
+    w = H.leaf_weights(oct, hv)
+    cdf, total = H.build_cdf(w)
+    cdf_host = cdf.cpu().numpy()
+    assert n_leaves < 1000 or (np.diff(cdf_host) == 0).mean() > 0.05
+    assert n_leaves < 200000 or (np.diff(cdf_host) < 0).any()
+    rng_dev, rng_ref = H.make_rng(77), oracle.Pcg32(77)
+    n_samples = 150000
+    pos, ids = H.sample(oct, cdf, total, n_samples, rng_dev)
+    pos_ref, ids_ref = oracle.sample(oct.centers, oct.levels, cdf_host, n_samples, oct.initial_size, rng_ref)
+    np.testing.assert_array_equal(ids, ids_ref)
+    np.testing.assert_array_equal(pos.view(np.uint32), pos_ref.view(np.uint32))
+    # the training draw takes the same path through the cull kernel
+    draw = H.CullDraw(oct, hv, cdf, total, rng_dev, 100000, 100000)
+    acc, cons = draw.round(100000)
+    pos_ref, ids_ref, acc_ref, cons_ref = oracle.sample_cull_compact(
+        oct.centers, oct.levels, cdf_host, hv.w2c, oracle_cam(oracle, hv), oct.initial_size, rng_ref, 100000, 0, 100000)
+    assert (acc, cons) == (acc_ref, cons_ref) and 0 < acc
+    np.testing.assert_array_equal(draw.ids.cpu().numpy()[:acc], ids_ref[:acc])
+    np.testing.assert_array_equal(draw.pos.cpu().numpy()[:acc].view(np.uint32), pos_ref[:acc].view(np.uint32))
+
+
 def test_sample_failure_path_writes_nothing(gpu):
     oct, hv = small_scene(500, 4)
     w = torch.zeros(500, dtype=torch.float32, device=gpu)

@@ -17,7 +17,7 @@ def _static_cdf(w_dev):
     lib = _lib.lib()
     n = w_dev.numel()
     cdf = w_dev.clone()
-    head = torch.zeros(_lib.CDF_HEAD_FLOATS, dtype=torch.float32, device=w_dev.device)
+    head = torch.zeros(int(lib.inpc_cdf_head_floats(n)), dtype=torch.float32, device=w_dev.device)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
     _lib.check(lib.inpc_build_cdf_static(_lib.ptr(cdf), _lib.ptr(head), n, H.stream()), "inpc_build_cdf_static")
