@@ -278,16 +278,34 @@ __device__ __forceinline__ void draw_candidates(uint64_t state0, const TileJumps
         node[j] = 1u;
     }
     // the probes whose element lies in the tree (a finished search keeps its node and reads it again)
-#pragma unroll 1
-    for (int level = 0; level < kTreeDepth; ++level) {
+    if (n_leaves >= (4u << kTreeDepth)) {
+        // no search ends inside the tree (every level leaves at least half of the elements minus one); a candidate
+        // that does not exist goes left all the way with nothing to search
 #pragma unroll
-        for (int j = 0; j < kSampleItems; ++j) {
-            const bool active = count[j] > 0u;
-            const uint32_t step = count[j] >> 1;
-            const bool right = s_tree[node[j]] < u[j];
-            first[j] = active && right ? first[j] + step + 1u : first[j];
-            count[j] = !active ? 0u : right ? count[j] - (step + 1u) : step;
-            node[j] = active ? 2u * node[j] + (right ? 1u : 0u) : node[j];
+        for (int j = 0; j < kSampleItems; ++j) u[j] = live[j] ? u[j] : -1.0f;
+#pragma unroll 1
+        for (int level = 0; level < kTreeDepth; ++level) {
+#pragma unroll
+            for (int j = 0; j < kSampleItems; ++j) {
+                const uint32_t step = count[j] >> 1;
+                const bool right = s_tree[node[j]] < u[j];
+                first[j] += right ? step + 1u : 0u;
+                count[j] = right ? count[j] - (step + 1u) : step;
+                node[j] = 2u * node[j] + (right ? 1u : 0u);
+            }
+        }
+    } else {
+#pragma unroll 1
+        for (int level = 0; level < kTreeDepth; ++level) {
+#pragma unroll
+            for (int j = 0; j < kSampleItems; ++j) {
+                const bool active = count[j] > 0u;
+                const uint32_t step = count[j] >> 1;
+                const bool right = s_tree[node[j]] < u[j];
+                first[j] = active && right ? first[j] + step + 1u : first[j];
+                count[j] = !active ? 0u : right ? count[j] - (step + 1u) : step;
+                node[j] = active ? 2u * node[j] + (right ? 1u : 0u) : node[j];
+            }
         }
     }
     // the levels of the tree below that are read from the head in memory, all eight searches level by level again
