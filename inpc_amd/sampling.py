@@ -103,7 +103,8 @@ class ProbabilityFieldSampler(torch.nn.Module):
         ws_bytes = int(lib.inpc_sampler_workspace_bytes(max(n, 1)))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=centers.device)
         head_floats = int(lib.inpc_cdf_head_floats(max(n, 1)))
-        total = torch.zeros(head_floats, dtype=torch.float32, device=centers.device)  # CDF head; [0] = total
+        # CDF head; [0] = total, written by inpc_build_cdf / inpc_expected_counts whenever there are leaves
+        total = (torch.empty if n > 0 else torch.zeros)(head_floats, dtype=torch.float32, device=centers.device)
         return vw, boxes, ws, ws_bytes, total, cam, stream
 
     def _cdf(self, centers, levels, weights, w2c, view, initial_size):
