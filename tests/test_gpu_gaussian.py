@@ -288,7 +288,7 @@ def test_reference_tile_size_on_large_images(gpu, oracle, width, height, focal):
     # 8x8 tiles on images of more than 16,384 tiles (32,400 and 63,860): the bins are counted and filled in windows
     # of 32,768 tiles by blocks of 1024 threads; footprints that straddle the windows come from the near points
     n, channels = 200000, 4
-    hv, pos, feats, opac = scene(n, channels, seed=81, width=width, height=height, focal=focal, near=300)
+    hv, pos, feats, opac = scene(n, channels, seed=81, width=width, height=height, focal=focal, near=300)   # the first 300
     run = H.GaussianRun(hv, pos, feats, opac, 8, channels, _lib.FEAT_DIRECT_F32).forward()
     assert run.layout.n_tiles > 16384
     g, ref = oracle_run(oracle, hv, pos, feats, opac, 8, channels)
@@ -305,8 +305,13 @@ def test_reference_tile_size_on_large_images(gpu, oracle, width, height, focal):
     gf, go = run.backward(gi, ga)
     gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
                                                gaussian=g)
-    H.assert_close(gf, gf_ref, RTOL, grad_atol(gf_ref), "feature gradients")
-    H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
+    # the near points cover up to thousands of pixels in dozens of tiles at this focal length: their gradients are
+    # sums of that many terms of both signs, added with float atomics in an order that changes from run to run
+    near = 300
+    H.assert_close(gf[near:], gf_ref[near:], RTOL, grad_atol(gf_ref), "feature gradients")
+    H.assert_close(go[near:], go_ref[near:], RTOL, grad_atol(go_ref), "opacity gradients")
+    H.assert_close(gf[:near], gf_ref[:near], 1e-3, 2e-6, "feature gradients of the near points")
+    H.assert_close(go[:near], go_ref[:near], 1e-3, 2e-5, "opacity gradients of the near points")
 
 
 def test_instances_beyond_the_capacity_are_reported(gpu, oracle):
