@@ -174,7 +174,11 @@ int inpc_cull_read_counts(const void* workspace, uint32_t* accepted_host, uint32
 /* End of a draw: advance the device generator by 4*consumed draws (4*total_candidates when
  * fewer than `capacity` samples were accepted), mirroring the host-side rng.advance of
  * B/sampling/src/sampling.cu:208. When *sum_dev <= 0 the outputs are filled with the
- * failure pattern of B/sampling/src/sampling.cu:107-111 (positions 0, ids -1). */
+ * failure pattern of B/sampling/src/sampling.cu:107-111 (positions 0, ids -1).
+ * total_candidates = INPC_CULL_IF_COMPLETE: the generator only moves if `capacity` samples were
+ * accepted; a caller can enqueue this behind a round before it has read the counts back, and
+ * makes the call again with the real number only if the draw needed more rounds. */
+#define INPC_CULL_IF_COMPLETE 0xFFFFFFFFu
 int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_ids_out,
                      uint32_t capacity, uint32_t total_candidates, uint64_t* rng_dev,
                      void* workspace, size_t workspace_bytes, void* stream);

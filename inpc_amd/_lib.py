@@ -19,6 +19,7 @@ FEAT_DIRECT_F16 = 2
 FEAT_RAW37_F16 = 3
 RASTER_INFERENCE = 1
 RASTER_KEEP_GEOMETRY = 2
+CULL_IF_COMPLETE = 0xFFFFFFFF  # INPC_CULL_IF_COMPLETE
 CDF_HEAD_FLOATS = 16384  # INPC_CDF_HEAD_FLOATS: total + the top of the CDF search tree
 
 

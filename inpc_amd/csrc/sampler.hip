@@ -568,7 +568,9 @@ __global__ void __launch_bounds__(kBlock) k_cull_finish(const float* __restrict_
     if (*sum_dev > 0.0f) {
         if (blockIdx.x == 0 && threadIdx.x == 0) {
             const uint32_t consumed = st->consumed != 0u ? st->consumed : total_candidates;
-            rng_dev[0] = pcg_apply(pcg_jump(rng_dev[1], 4ull * consumed), rng_dev[0]);
+            // INPC_CULL_IF_COMPLETE: a draw that has not reached its capacity is left as it is
+            if (consumed != INPC_CULL_IF_COMPLETE)
+                rng_dev[0] = pcg_apply(pcg_jump(rng_dev[1], 4ull * consumed), rng_dev[0]);
         }
         return;
     }

@@ -142,14 +142,27 @@ class ProbabilityFieldSampler(torch.nn.Module):
         cull_ws = torch.empty(cull_bytes, dtype=torch.uint8, device=device)
         k0, accepted, consumed = 0, C.c_uint32(0), C.c_uint32(0)
         n_round = first
+        finished = False
+
+        def finish(total_candidates):
+            _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples,
+                                            total_candidates, _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream),
+                       "inpc_cull_finish")
+            _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
+
         while True:
             _lib.check(lib.inpc_sample_cull_compact(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(w2c),
                                                     _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0, n_round,
                                                     n_leaves, C.byref(cam), _lib.ptr(rng), _lib.ptr(cull_ws),
                                                     cull_bytes, stream), "inpc_sample_cull_compact")
             k0 += n_round
+            if k0 == n_round:
+                # the first round nearly always completes the draw: its end is enqueued before the counts are read
+                # back, so the device does not wait for the host's round trip (it changes nothing if more rounds follow)
+                finish(_lib.CULL_IF_COMPLETE)
             _lib.check(lib.inpc_cull_read_counts(_lib.ptr(cull_ws), C.byref(accepted), C.byref(consumed), stream),
                        "inpc_cull_read_counts")
+            finished = k0 == n_round and consumed.value != 0
             if consumed.value != 0 or accepted.value >= n_samples:
                 break
             if accepted.value == 0 and k0 >= first:
@@ -163,8 +176,9 @@ class ProbabilityFieldSampler(torch.nn.Module):
         if consumed.value:
             self._acceptance = n_samples / consumed.value
         self.last_consumed = int(consumed.value) if consumed.value else k0
-        _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0,
-                                        _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream), "inpc_cull_finish")
+        if not finished:
+            _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0,
+                                            _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream), "inpc_cull_finish")
         if consumed.value == 0 and accepted.value < n_samples and float(total[0].item()) > 0.0:
             # the draw gave up (the frustum is hardly ever hit, or the candidate limit was reached): the slots behind
             # the accepted samples get the failure pattern of B/sampling/src/sampling.cu:107-111, positions 0 and
@@ -173,7 +187,8 @@ class ProbabilityFieldSampler(torch.nn.Module):
                          accepted.value, n_samples)
             positions[accepted.value:].zero_()
             ids32[accepted.value:].fill_(-1)
-        _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
+        if not finished:
+            _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
         return positions, ids64
 
     def generate_samples(self, centers, levels, weights, view, n_samples: int, initial_size: float) -> torch.Tensor:

@@ -170,6 +170,29 @@ def test_training_api_matches_oracle_draw(gpu, oracle):
         assert sampler.rng_state() == (int(rng_ref.state[0]), int(rng_ref.state[1]))
 
 
+def test_training_api_draw_of_several_rounds(gpu, oracle):
+    # A camera inside the octree: most candidates are rejected, the first round (sized for full acceptance) does not
+    # complete the draw, and the end of the draw that was enqueued behind it must have changed nothing.
+    from inpc_amd import ProbabilityFieldSampler
+
+    oct, hv = small_scene(distance=0.6)
+    view = hv.to_view(gpu)
+    centers, levels, weights = H.dev(oct.centers), H.dev(oct.levels), H.dev(oct.weights)
+    sampler = ProbabilityFieldSampler(seed=21)
+    rng_ref = oracle.Pcg32(21)
+    n = 30000
+    first_round = int(n * sampler.OVERSAMPLE) + 4096
+    for _ in range(2):   # the second call starts from the acceptance the first one saw
+        pos, ids = sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)
+        pos_ref, ids_ref, consumed = oracle.training_samples(oct.centers, oct.levels, oct.weights, hv.w2c,
+                                                             oracle_cam(oracle, hv), oct.initial_size, rng_ref, n)
+        np.testing.assert_array_equal(ids.cpu().numpy(), ids_ref.astype(np.int64))
+        np.testing.assert_array_equal(pos.cpu().numpy().view(np.uint32), pos_ref.view(np.uint32))
+        assert sampler.last_consumed == consumed
+        assert sampler.rng_state() == (int(rng_ref.state[0]), int(rng_ref.state[1]))
+    assert consumed > first_round, "the scene must need more than one round at full-acceptance sizing"
+
+
 def test_training_api_failure_pattern(gpu):
     from inpc_amd import ProbabilityFieldSampler
 
