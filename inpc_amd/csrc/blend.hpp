@@ -240,8 +240,10 @@ __device__ __forceinline__ void stage_instance(Stage<T, C, WITH_DEPTH>& st, bool
         st.alpha[t] = make_float4(h.opacity * weight[0], h.opacity * weight[1], h.opacity * weight[2], h.opacity * weight[3]);
         st.pixel[t] = pixel[0] | (pixel[1] << 8) | (pixel[2] << 16) | (pixel[3] << 24);
     }
-    const uint2 nothing_placed = make_uint2(0u, 0u);
-    __builtin_memcpy(st.frag[t], &nothing_placed, 8);
+    if (!WITH_DEPTH) {   // the write phase that reads the fields only exists in training configurations
+        const uint2 nothing_placed = make_uint2(0u, 0u);
+        __builtin_memcpy(st.frag[t], &nothing_placed, 8);
+    }
 }
 
 // The instances of one lane: entry k is staged instance k * 64 + lane; its (at most NF) fragments in this
@@ -325,7 +327,7 @@ __device__ __forceinline__ void build_fragment_lists(QuadScratch<T>& qs, Stage<T
 #pragma unroll
                 for (int kk = 0; kk < k; ++kk) pos += (uint32_t)__popcll(qs.hits[pix][kk]);
                 qs.fragment[pos] = make_float2(e.alpha[k][q], payload(k, q));
-                st.frag[e.j[k]][T == 16 ? quad : q] = (uint16_t)((pos << 8) | pix | kPlaced);
+                if (!WITH_DEPTH) st.frag[e.j[k]][T == 16 ? quad : q] = (uint16_t)((pos << 8) | pix | kPlaced);
             }
         }
     wave_sync();
@@ -524,7 +526,7 @@ __global__ void __launch_bounds__(T* T)
                     const float a = done ? 0.0f : e.x;
                     const uint32_t jj = __float_as_uint(e.y);
                     const float bw = Tr * a;
-                    qs.fragment[pos].x = bw;
+                    if (!INFERENCE) qs.fragment[pos].x = bw;
 #pragma unroll
                     for (int q4 = 0; q4 < C / 4; ++q4) {
                         const float4 v = st.feat[jj * (C / 4) + q4];
@@ -559,7 +561,7 @@ __global__ void __launch_bounds__(T* T)
                     const float t_before = wave_previous(t_after, p_T);
                     const bool reached = here && !(t_before < kTransmittanceThreshold);
                     const float bw = reached ? t_before * a : 0.0f;
-                    if (here) qs.fragment[pos].x = bw;
+                    if (!INFERENCE && here) qs.fragment[pos].x = bw;
                     if (reached) {
                         const uint32_t jj = __float_as_uint(e.y);
 #pragma unroll
@@ -577,7 +579,7 @@ __global__ void __launch_bounds__(T* T)
                     const int last = 63 - __builtin_clzll(reached_lanes | 1ull);
                     p_T = __shfl(t_after, last, 64);
                     // a walk that ended inside this round leaves the rest of the list untouched: weights 0
-                    if (p_T < kTransmittanceThreshold)
+                    if (!INFERENCE && p_T < kTransmittanceThreshold)
                         for (uint32_t rest = base + 64u + lane; rest < p_count; rest += 64u) qs.fragment[p_start + rest].x = 0.0f;
                 }
 #pragma unroll
