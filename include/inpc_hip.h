@@ -388,9 +388,9 @@ int inpc_gaussian_forward(const inpc_gaussian_config* cfg, const float* position
  * (B/rasterization/src/gaussian/backward.cu:9-68), blend_backward_cu and preprocess_backward_cu
  * (B/rasterization/src/gaussian/kernels.cu:326-344,476-579). Arguments as for
  * inpc_raster_backward. The gradient of a point that touches several tiles is the sum of
- * per-instance rows in the workspace, taken in a fixed order; only instances whose footprint
- * covers more than nine pixels of a tile (points close to the camera) add with float atomics,
- * so the last bits of those points' gradients depend on scheduling, as in the reference.
+ * per-instance rows in the workspace, taken in a fixed order, and an instance's row is a sum
+ * in a fixed order as well (also for footprints of many pixels): no float atomics, the same
+ * bits on every run (the reference adds with atomics, kernels.cu:548-571).
  * The workspace must be the one the forward pass of the same inputs has filled. Like the
  * forward pass it only enqueues kernels, so forward + backward can be captured in a graph
  * and replayed with new inputs written in place. */

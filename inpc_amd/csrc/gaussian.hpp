@@ -338,7 +338,11 @@ __global__ void __launch_bounds__(THREADS)
 // that has blended the instance replaces the value (positive) by minus its contribution (forward: G * blending
 // weight; backward: the blending weight, next to the opacity gradient in a second array); after the batch the
 // instance's thread adds up the negative slots, in slot order: no atomics.
-// Larger boxes (points close to the camera) are evaluated by the pixels and add to global memory directly.
+// Larger boxes (points close to the camera) have no slots. A training configuration takes such an instance through the
+// whole block at once, at its place in the depth order: every pixel of its box evaluates the footprint and blends it,
+// the waves add their pixels' contributions up (DPP sums, a fixed order), a block barrier, and the instance's own
+// thread adds the waves' sums in wave order: no atomics either, and the same bits on every run. The inference blend
+// has nothing to hand back to the instance and lets every pixel walk over such instances on its own.
 constexpr int kSlots = 9;
 constexpr int kSlotStride = kSlots;   // odd: rows of neighbouring instances spread over the LDS banks
 
@@ -521,6 +525,10 @@ __global__ void __launch_bounds__(T * T)
     for (int c = 0; c < C; ++c) acc[c] = 0.0f;
     float depth_acc = 0.0f, tr = 1.0f;
     bool done = !px.inside;
+    // per wave: what its pixels add to the blending weight of the instance without slots that the block is at; two
+    // sets, so that the next such instance does not overwrite what the thread of this one is still reading
+    __shared__ float s_big[2][TT / 64];
+    uint32_t big_parity = 0u;
     const uint2 range = ranges[tile];
     Ahead<C> ahead;
     ahead.start(inst_points, records, stride, range, TT);
@@ -537,23 +545,23 @@ __global__ void __launch_bounds__(T * T)
             if (tid < count) stage_instance<T, C>(st, tid, h0, h1, feat, tile_x0, tile_y0, reach2, threshold);
         }
         __syncthreads();
-        if (__ballot(!done) != 0ull) {
+        {
+            const bool wave_live = __ballot(!done) != 0ull;
             for (uint32_t first = 0; first < count; first += 64u) {
                 const uint32_t at = first + lane;
                 const uint32_t my_box = at < count ? st.box[at] : 0u;
+                // the instances without slots of these 64, the same mask in every wave of the block
+                const uint64_t big = INFERENCE ? 0ull : __ballot(!has_slots(my_box));
+                if (!wave_live && big == 0ull) continue;
                 const uint64_t reach = __ballot(box_reaches(my_box, px));
                 const bool all_slots = __ballot(box_reaches(my_box, px) && !has_slots(my_box)) == 0ull;
                 uint64_t over = reach != 0ull ? instances_over_pixel(my_box, px) : 0ull;
                 if (done) over = 0ull;
-                // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
-                auto blend = [&](uint32_t j, int slot, float G, auto has_slot) {
+                uint64_t now = 0ull;   // the part of `over` a walk is going through
+                // blend instance j, whose footprint value at this pixel is G; returns G * blending weight
+                auto blend = [&](uint32_t j, float G) {
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
-                    if (!INFERENCE) {
-                        const float part = bw > 0.0f ? G * bw : 0.0f;
-                        if (decltype(has_slot)::value || slot >= 0) st.value[j][slot] = -part;
-                        else if (part != 0.0f) atomicAdd(&blending_weights[__float_as_uint(st.head1[j].w) & kPointMask], part);
-                    }
 #pragma unroll
                     for (int q = 0; q < C / 4; ++q) {
                         const float4 f = st.feat[j * (C / 4) + q];
@@ -567,23 +575,34 @@ __global__ void __launch_bounds__(T * T)
                     if (tr < kTransmittanceThreshold) {
                         done = true;
                         over = 0ull;
+                        now = 0ull;
                     }
+                    return bw > 0.0f ? G * bw : 0.0f;
                 };
-                if (all_slots) {   // the usual case, without the branches of the other one
-                    while (__ballot(over != 0ull) != 0ull) {
-                        if (over != 0ull) {
-                            const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
-                            over &= over - 1ull;
+                // every lane its own instances of `now`, all of which have slots
+                auto walk_slots = [&]() {
+                    while (__ballot(now != 0ull) != 0ull) {
+                        if (now != 0ull) {
+                            const uint32_t j = first + (uint32_t)__builtin_ctzll(now);
+                            now &= now - 1ull;
                             const int slot = slot_in(st.box[j], px.lx, px.ly);
                             const float G = st.value[j][slot];
-                            if (G != 0.0f) blend(j, slot, G, std::true_type{});
+                            if (G != 0.0f) {
+                                const float part = blend(j, G);
+                                if (!INFERENCE) st.value[j][slot] = -part;
+                            }
                         }
                     }
-                } else {
-                    while (__ballot(over != 0ull) != 0ull) {
-                        if (over == 0ull) continue;
-                        const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
-                        over &= over - 1ull;
+                };
+                if (all_slots && big == 0ull) {   // the usual case
+                    now = over;
+                    walk_slots();
+                } else if (INFERENCE) {   // nothing goes back to the instances: every lane on its own
+                    now = over;
+                    while (__ballot(now != 0ull) != 0ull) {
+                        if (now == 0ull) continue;
+                        const uint32_t j = first + (uint32_t)__builtin_ctzll(now);
+                        now &= now - 1ull;
                         const int slot = slot_of(st.box[j], px.lx, px.ly);
                         float G;
                         if (slot >= 0) {
@@ -592,7 +611,35 @@ __global__ void __launch_bounds__(T * T)
                         } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
                             continue;
                         }
-                        blend(j, slot, G, std::false_type{});
+                        (void)blend(j, G);
+                    }
+                } else {
+                    // in depth order: the instances with slots up to the next one without, lane by lane, then that
+                    // one by the whole block
+                    uint64_t big_left = big;
+                    for (;;) {
+                        const uint32_t kb = big_left != 0ull ? (uint32_t)__builtin_ctzll(big_left) : 64u;
+                        now = kb == 64u ? over : over & ((1ull << kb) - 1ull);
+                        over &= ~now;
+                        walk_slots();
+                        if (kb == 64u) break;
+                        big_left &= big_left - 1ull;
+                        const uint32_t j = first + kb;
+                        float part = 0.0f, G;
+                        if (((over >> kb) & 1ull) != 0ull &&
+                            footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G))
+                            part = blend(j, G);
+                        over &= ~(1ull << kb);
+                        const float wave_part = blend::wave_sum(part);
+                        if (lane == 0u) s_big[big_parity][tid >> 6] = wave_part;
+                        __syncthreads();
+                        if (tid == j) {   // the instance's thread: its blending weight in this tile
+                            float w = 0.0f;
+#pragma unroll
+                            for (int q = 0; q < TT / 64; ++q) w += s_big[big_parity][q];
+                            st.value[j][0] = w;
+                        }
+                        big_parity ^= 1u;
                     }
                 }
             }
@@ -609,6 +656,8 @@ __global__ void __launch_bounds__(T * T)
                         const float v = st.value[tid][k];
                         if (k < used && v < 0.0f) w -= v;   // slots no pixel has blended still hold the footprint value
                     }
+                } else {
+                    w = st.value[tid][0];   // an instance without slots: added up when the block went through it
                 }
                 if (w != 0.0f) {
                     const uint32_t word = __float_as_uint(st.head1[tid].w);
@@ -654,7 +703,6 @@ __global__ void __launch_bounds__(kBlock)
     static_assert(kWords == (uint32_t)C / 4u + 1u && kWords <= kGroup, "row layout");
     if (counters[kCntKept] == 0u) return;
     const uint32_t n_multi = counters[kCntMulti];
-    const bool add = counters[kCntDirect] != 0u;
     const uint2 stamp = *rows.stamp;
     const uint32_t gtid = blockIdx.x * kBlock + threadIdx.x, lane = threadIdx.x & 63u;
     const uint32_t word = gtid % kGroup, tail_lane = (lane & ~(kGroup - 1u)) + kWords - 1u;
@@ -684,14 +732,8 @@ __global__ void __launch_bounds__(kBlock)
                 sum.w += v[k].w;
             }
         }
-        // stored, or added to what is there when instances without slots have put their share into the arrays directly
-        if (word < kWords - 1u) {
-            float4* gf = (float4*)(grad_features + (size_t)point * C) + word;
-            const float4 old = add ? *gf : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            *gf = make_float4(old.x + sum.x, old.y + sum.y, old.z + sum.z, old.w + sum.w);
-        } else if (word == kWords - 1u) {
-            grad_opacities[point] = (add ? grad_opacities[point] : 0.0f) + sum.x;
-        }
+        if (word < kWords - 1u) ((float4*)(grad_features + (size_t)point * C))[word] = sum;
+        else if (word == kWords - 1u) grad_opacities[point] = sum.x;
     }
 }
 
@@ -705,8 +747,7 @@ __global__ void __launch_bounds__(T * T)
                      const uint32_t* __restrict__ inst_points, const char* __restrict__ records, uint32_t stride,
                      const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
                      const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_features,
-                     float* grad_opacities, GradRows grad_rows, uint32_t* counters, int W, int H, uint32_t gw, float threshold,
-                     float reach2) {
+                     float* grad_opacities, GradRows grad_rows, int W, int H, uint32_t gw, float threshold, float reach2) {
     constexpr int TT = T * T;
     __shared__ Stage<T, C> st;
     __shared__ float s_d_opacity[TT][kSlotStride];   // per staged instance and box pixel: d loss / d opacity
@@ -735,7 +776,12 @@ __global__ void __launch_bounds__(T * T)
     }
     float running = 0.0f;
     const uint2 stamp = *grad_rows.stamp;
-    bool used_direct = false;   // this thread has added a gradient to the arrays directly (an instance without slots)
+    // per wave: what its pixels add to the gradient of the instance without slots that the block is at (C feature
+    // gradients and the opacity gradient); two sets, so that the next such instance does not overwrite what the thread
+    // of this one is still reading
+    static_assert(C + 1 <= 2 * kSlots, "the sums of an instance without slots are kept in its two slot rows");
+    __shared__ float s_big[2][TT / 64][C + 1];
+    uint32_t big_parity = 0u;
 #pragma unroll
     for (int c = 0; c < C; ++c) s_grad_px[px.ly * T + px.lx][c] = g[c];
     float tr = 1.0f;
@@ -770,16 +816,20 @@ __global__ void __launch_bounds__(T * T)
             }
         }
         __syncthreads();
-        if (__ballot(!done) != 0ull) {
+        {
+            const bool wave_live = __ballot(!done) != 0ull;
             for (uint32_t first = 0; first < count; first += 64u) {
                 const uint32_t at = first + lane;
                 const uint32_t my_box = at < count ? st.box[at] : 0u;
+                // the instances without slots of these 64, the same mask in every wave of the block
+                const uint64_t big = __ballot(!has_slots(my_box));
+                if (!wave_live && big == 0ull) continue;
                 const uint64_t reach = __ballot(box_reaches(my_box, px));
-                const bool all_slots = __ballot(box_reaches(my_box, px) && !has_slots(my_box)) == 0ull;
                 uint64_t over = reach != 0ull ? instances_over_pixel(my_box, px) : 0ull;
                 if (done) over = 0ull;
-                // blend instance j, whose footprint value at this pixel is G; slot < 0: the instance has no slots
-                auto blend = [&](uint32_t j, int slot, float G, auto has_slot) {
+                uint64_t now = 0ull;   // the part of `over` a walk is going through
+                // blend instance j, whose footprint value at this pixel is G: blending weight and d loss / d opacity
+                auto blend = [&](uint32_t j, float G, float& weight, float& d_opacity) {
                     const float a = st.head0[j].z * G;
                     const float bw = tr * a;
                     const float one_minus_a = 1.0f - a;
@@ -796,51 +846,65 @@ __global__ void __launch_bounds__(T * T)
                     }
                     running = fmaf(bw, sd, running);
                     const float d_alpha = fmaf(tr, sd, (running + offset) * rcp);
-                    const float d_opacity = d_alpha * G;
-                    const float weight = bw > 0.0f ? bw : 0.0f;
-                    if (decltype(has_slot)::value || slot >= 0) {
-                        st.value[j][slot] = -weight;
-                        s_d_opacity[j][slot] = d_opacity;
-                    } else {
-                        const uint32_t point = __float_as_uint(st.head1[j].w) & kPointMask;
-                        if (weight > 0.0f) {
-#pragma unroll
-                            for (int c = 0; c < C; ++c) atomicAdd(&grad_features[(size_t)point * C + c], weight * g[c]);
-                        }
-                        if (d_opacity != 0.0f) atomicAdd(&grad_opacities[point], d_opacity);
-                        used_direct = true;
-                    }
+                    d_opacity = d_alpha * G;
+                    weight = bw > 0.0f ? bw : 0.0f;
                     tr *= one_minus_a;
                     if (tr < kTransmittanceThreshold) {
                         done = true;
                         over = 0ull;
+                        now = 0ull;
                     }
                 };
-                if (all_slots) {   // the usual case, without the branches of the other one
-                    while (__ballot(over != 0ull) != 0ull) {
-                        if (over != 0ull) {
-                            const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
-                            over &= over - 1ull;
+                // in depth order: the instances with slots up to the next one without, lane by lane, then that one by
+                // the whole block (the usual case has none of those and is a single walk)
+                uint64_t big_left = big;
+                for (;;) {
+                    const uint32_t kb = big_left != 0ull ? (uint32_t)__builtin_ctzll(big_left) : 64u;
+                    now = kb == 64u ? over : over & ((1ull << kb) - 1ull);
+                    over &= ~now;
+                    while (__ballot(now != 0ull) != 0ull) {
+                        if (now != 0ull) {
+                            const uint32_t j = first + (uint32_t)__builtin_ctzll(now);
+                            now &= now - 1ull;
                             const int slot = slot_in(st.box[j], px.lx, px.ly);
                             const float G = st.value[j][slot];
-                            if (G != 0.0f) blend(j, slot, G, std::true_type{});
+                            if (G != 0.0f) {
+                                float weight, d_opacity;
+                                blend(j, G, weight, d_opacity);
+                                st.value[j][slot] = -weight;
+                                s_d_opacity[j][slot] = d_opacity;
+                            }
                         }
                     }
-                } else {
-                    while (__ballot(over != 0ull) != 0ull) {
-                        if (over == 0ull) continue;
-                        const uint32_t j = first + (uint32_t)__builtin_ctzll(over);
-                        over &= over - 1ull;
-                        const int slot = slot_of(st.box[j], px.lx, px.ly);
-                        float G;
-                        if (slot >= 0) {
-                            G = st.value[j][slot];
-                            if (G == 0.0f) continue;
-                        } else if (!footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G)) {
-                            continue;
-                        }
-                        blend(j, slot, G, std::false_type{});
+                    if (kb == 64u) break;
+                    big_left &= big_left - 1ull;
+                    const uint32_t j = first + kb;
+                    float weight = 0.0f, d_opacity = 0.0f, G;
+                    if (((over >> kb) & 1ull) != 0ull && footprint_value(st.head0[j], st.head1[j], cx, cy, threshold, G))
+                        blend(j, G, weight, d_opacity);
+                    over &= ~(1ull << kb);
+                    // what this wave's pixels add to the instance's gradient
+#pragma unroll
+                    for (int c = 0; c < C; ++c) {
+                        const float wave_part = blend::wave_sum(weight * g[c]);
+                        if (lane == 0u) s_big[big_parity][tid >> 6][c] = wave_part;
                     }
+                    {
+                        const float wave_part = blend::wave_sum(d_opacity);
+                        if (lane == 0u) s_big[big_parity][tid >> 6][C] = wave_part;
+                    }
+                    __syncthreads();
+                    if (tid == j) {   // the instance's thread: the waves' sums in wave order, kept in its unused slot rows
+#pragma unroll
+                        for (int c = 0; c <= C; ++c) {
+                            float sum = 0.0f;
+#pragma unroll
+                            for (int q = 0; q < TT / 64; ++q) sum += s_big[big_parity][q][c];
+                            if (c < kSlots) st.value[j][c] = sum;
+                            else s_d_opacity[j][c - kSlots] = sum;
+                        }
+                    }
+                    big_parity ^= 1u;
                 }
             }
         }
@@ -849,21 +913,26 @@ __global__ void __launch_bounds__(T * T)
             const uint32_t box = st.box[tid];
             const uint32_t cols = box & 0xFFFFu, rows = box >> 16;
             const int w = __popc(cols), h = __popc(rows), x_lo = __ffs(cols) - 1, y_lo = __ffs(rows) - 1;
-            if (w * h <= kSlots && w * h > 0) {
+            if (w * h > 0) {
                 float sum[C + 1];
 #pragma unroll
                 for (int c = 0; c <= C; ++c) sum[c] = 0.0f;
-                int slot = 0;
-                for (int yy = 0; yy < h; ++yy) {
-                    for (int xx = 0; xx < w; ++xx, ++slot) {
-                        const float v = st.value[tid][slot];
-                        if (!(__float_as_uint(v) >> 31)) continue;   // no pixel has blended it: still the footprint value
-                        const float weight = -v;
-                        const float* gp = s_grad_px[(y_lo + yy) * T + x_lo + xx];
+                if (w * h <= kSlots) {
+                    int slot = 0;
+                    for (int yy = 0; yy < h; ++yy) {
+                        for (int xx = 0; xx < w; ++xx, ++slot) {
+                            const float v = st.value[tid][slot];
+                            if (!(__float_as_uint(v) >> 31)) continue;   // no pixel has blended it: still the footprint value
+                            const float weight = -v;
+                            const float* gp = s_grad_px[(y_lo + yy) * T + x_lo + xx];
 #pragma unroll
-                        for (int c = 0; c < C; ++c) sum[c] = fmaf(weight, gp[c], sum[c]);
-                        sum[C] += s_d_opacity[tid][slot];
+                            for (int c = 0; c < C; ++c) sum[c] = fmaf(weight, gp[c], sum[c]);
+                            sum[C] += s_d_opacity[tid][slot];
+                        }
                     }
+                } else {   // an instance without slots: added up when the block went through it
+#pragma unroll
+                    for (int c = 0; c <= C; ++c) sum[c] = c < kSlots ? st.value[tid][c] : s_d_opacity[tid][c - kSlots];
                 }
                 const uint32_t word = __float_as_uint(st.head1[tid].w);
                 const uint32_t point = word & kPointMask;
@@ -883,8 +952,6 @@ __global__ void __launch_bounds__(T * T)
             }
         }
     }
-    // the pass that adds the rows up has to add to the arrays instead of storing into them
-    if (__ballot(used_direct) != 0ull && lane == 0u) atomicOr(&counters[kCntDirect], 1u);
 }
 
 }  // namespace gaussian

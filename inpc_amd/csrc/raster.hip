@@ -48,7 +48,6 @@ enum Counter : int {
     kCntOverflow = 5,      // the instances (or the gradient rows) do not fit the buffers: nothing is drawn
     kCntInstances64 = 6,   // Gaussian footprint: u64 at words 6, 7: exact instance count
     kCntMulti = 8,         // Gaussian footprint: drawn points that touch more than one tile
-    kCntDirect = 9,        // Gaussian footprint: set by a backward blend that added gradients to the arrays directly
     kCntRows = 10,         // instances of the points that touch more than one tile
     kCntWords = 16
 };
@@ -1278,8 +1277,8 @@ int launch_gaussian_blend_backward(const GaussianLayout& L, const float* grad_im
     INPC_LAUNCH("gaussian_blend_backward", (gaussian::k_blend_backward<T, C>), dim3(L.geo.n_tiles), dim3(T * T), stream,
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 (const uint32_t*)at<uint32_t>(ws, L.pub.instance_points), (const char*)at<char>(ws, L.pub.point_record),
-                L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, rows,
-                at<uint32_t>(ws, L.pub.counters), L.geo.W, L.geo.H, L.geo.gw, L.prm.threshold, L.prm.reach2);
+                L.geo.stride, grad_image, grad_alpha, image, alpha, grad_view, grad_opacities, rows, L.geo.W, L.geo.H,
+                L.geo.gw, L.prm.threshold, L.prm.reach2);
     INPC_LAUNCH("gaussian_grad_reduce", gaussian::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, kBlock), 4096u)),
                 dim3(kBlock), stream, (const uint4*)at<uint4>(ws, L.multi_list),
                 (const uint32_t*)at<uint32_t>(ws, L.pub.counters), rows, grad_view, grad_opacities);

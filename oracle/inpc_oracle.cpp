@@ -998,26 +998,52 @@ static int raster_forward_with_state(const RasterState& st, const inpc_raster_co
     return INPC_OK;
 }
 
+// What a test may ask of the backward pass besides the fp32 gradients, to judge a gradient by the conditioning of
+// the sum it is: every gradient is a sum of one term per (instance, pixel), of both signs for most points, so an
+// fp32 evaluation in whatever order is only good to a few rounding units of the sum of the terms' magnitudes.
+//   view64 (N,C), opacity64 (N)   the same sums with every term evaluated and accumulated in double precision
+//                                 (the transmittance and alpha stay the fp32 values that decide where a pixel ends)
+//   view_abs (N,C)                sum of |term|
+//   opacity_abs (N)               sum of the magnitudes a term of the opacity gradient is made of: the term is a
+//                                 difference of running and final pixel sums, which are rounded sums themselves
+// Any pointer may be null.
+struct oracle_grad_audit {
+    double* view64;
+    double* opacity64;
+    double* view_abs;
+    double* opacity_abs;
+};
+
 // Backward (B/rasterization/src/bilinear/backward.cu:9-67, kernels.cu:86-104,315-420).
 // grad_features: (N,36) fp16 [SH36], (N,C) f32 [DIRECT_F32], (N,C) fp16 [DIRECT_F16];
 // grad_view_out (N,C) f32 optional copy of the per-point view-space feature gradient.
 static int raster_backward_with_state(const RasterState& st, const inpc_raster_config* cfg, const float* grad_image,
                                       const float* grad_alpha, const float* image, const float* alpha,
                                       const float* positions, const float* cam_position, void* grad_features,
-                                      float* grad_opacities, float* grad_view_out) {
+                                      float* grad_opacities, float* grad_view_out,
+                                      const oracle_grad_audit* audit = nullptr) {
     const int W = cfg->cam.width, H = cfg->cam.height, T = st.T, C = st.C;
     const size_t n_pixels = (size_t)W * H;
     std::vector<float> gview((size_t)st.n * C, 0.0f);
     std::fill(grad_opacities, grad_opacities + st.n, 0.0f);
+    if (audit) {
+        if (audit->view64) std::fill(audit->view64, audit->view64 + (size_t)st.n * C, 0.0);
+        if (audit->view_abs) std::fill(audit->view_abs, audit->view_abs + (size_t)st.n * C, 0.0);
+        if (audit->opacity64) std::fill(audit->opacity64, audit->opacity64 + st.n, 0.0);
+        if (audit->opacity_abs) std::fill(audit->opacity_abs, audit->opacity_abs + st.n, 0.0);
+    }
 
 #pragma omp parallel
     {
         std::vector<float> Fnew((size_t)T * T * C), Tr((size_t)T * T);
+        std::vector<double> Fnew64(audit ? (size_t)T * T * C : 0), Fabs64(audit ? (size_t)T * T * C : 0);
         std::vector<uint8_t> done((size_t)T * T);
 #pragma omp for schedule(dynamic, 4)
         for (int64_t tile = 0; tile < (int64_t)st.n_tiles; ++tile) {
             const int tx = (int)(tile % st.gw), ty = (int)(tile / st.gw);
             std::fill(Fnew.begin(), Fnew.end(), 0.0f);
+            std::fill(Fnew64.begin(), Fnew64.end(), 0.0);
+            std::fill(Fabs64.begin(), Fabs64.end(), 0.0);
             std::fill(Tr.begin(), Tr.end(), 1.0f);
             std::fill(done.begin(), done.end(), 0);
             const uint32_t begin = st.ranges[2 * tile], end = st.ranges[2 * tile + 1];
@@ -1048,6 +1074,41 @@ static int raster_backward_with_state(const RasterState& st, const inpc_raster_c
                         const float a = op * wgt;
                         const float tr = Tr[lp];
                         const float bw = tr * a;
+                        if (audit) {
+                            // the same terms in double precision, from the fp32 transmittance and alpha
+                            const double bw64 = (double)tr * (double)a;
+                            const double rcp64 = 1.0 / std::fmax(1.0 - (double)a, (double)kOneMinusAlphaEps);
+                            double dot64 = 0.0, dot_abs = 0.0;
+                            for (int c = 0; c < C; ++c) {
+                                const double g = (double)grad_image[c * n_pixels + pix];
+                                double& fn = Fnew64[(size_t)lp * C + c];
+                                double& fa = Fabs64[(size_t)lp * C + c];
+                                fn += bw64 * (double)f[c];
+                                fa += std::fabs(bw64 * (double)f[c]);
+                                dot64 += ((double)tr * (double)f[c] + (fn - (double)image[c * n_pixels + pix]) * rcp64) * g;
+                                dot_abs += (std::fabs((double)tr * (double)f[c]) +
+                                            (fa + std::fabs((double)image[c * n_pixels + pix])) * rcp64) * std::fabs(g);
+                                if (bw > 0.0f) {
+                                    if (audit->view64) {
+#pragma omp atomic
+                                        audit->view64[(size_t)p * C + c] += bw64 * g;
+                                    }
+                                    if (audit->view_abs) {
+#pragma omp atomic
+                                        audit->view_abs[(size_t)p * C + c] += std::fabs(bw64 * g);
+                                    }
+                                }
+                            }
+                            const double common64 = (double)grad_alpha[pix] * (1.0 - (double)alpha[pix]);
+                            if (audit->opacity64) {
+#pragma omp atomic
+                                audit->opacity64[p] += (dot64 + common64 * rcp64) * (double)wgt;
+                            }
+                            if (audit->opacity_abs) {
+#pragma omp atomic
+                                audit->opacity_abs[p] += (dot_abs + std::fabs(common64) * rcp64) * (double)wgt;
+                            }
+                        }
                         if (bw > 0.0f) {
                             for (int c = 0; c < C; ++c) {
                                 const float g = bw * grad_image[c * n_pixels + pix];
@@ -1173,6 +1234,32 @@ int oracle_gaussian_backward(const inpc_gaussian_config* cfg, const float* grad_
     if (rc != INPC_OK) return rc;
     return raster_backward_with_state(st, &cfg->base, grad_image, grad_alpha, image, alpha, positions, cam_position,
                                       grad_features, grad_opacities, grad_view_out);
+}
+
+// The backward passes above with the audit outputs (see oracle_grad_audit) besides the fp32 gradients.
+int oracle_raster_backward_audit(const inpc_raster_config* cfg, const float* grad_image, const float* grad_alpha,
+                                 const float* image, const float* alpha, const float* positions, const void* features,
+                                 const float* opacities, const float* w2c, const float* cam_position,
+                                 void* grad_features, float* grad_opacities, float* grad_view_out,
+                                 const oracle_grad_audit* audit) {
+    RasterState st;
+    const int rc = raster_prepare(st, cfg, positions, features, opacities, w2c, cam_position);
+    if (rc != INPC_OK) return rc;
+    return raster_backward_with_state(st, cfg, grad_image, grad_alpha, image, alpha, positions, cam_position,
+                                      grad_features, grad_opacities, grad_view_out, audit);
+}
+
+int oracle_gaussian_backward_audit(const inpc_gaussian_config* cfg, const float* grad_image, const float* grad_alpha,
+                                   const float* image, const float* alpha, const float* positions, const void* features,
+                                   const float* opacities, const float* w2c, const float* cam_position,
+                                   void* grad_features, float* grad_opacities, float* grad_view_out,
+                                   const oracle_grad_audit* audit) {
+    RasterState st;
+    const FootprintParams fp = footprint_params(cfg, nullptr);
+    const int rc = raster_prepare(st, &cfg->base, positions, features, opacities, w2c, cam_position, &fp);
+    if (rc != INPC_OK) return rc;
+    return raster_backward_with_state(st, &cfg->base, grad_image, grad_alpha, image, alpha, positions, cam_position,
+                                      grad_features, grad_opacities, grad_view_out, audit);
 }
 
 float oracle_footprint_exp(float x) { return footprint_exp(x); }

@@ -377,9 +377,15 @@ def footprint_exp(x):
     return out
 
 
+class _GradAudit(C.Structure):
+    _fields_ = [("view64", C.c_void_p), ("opacity64", C.c_void_p), ("view_abs", C.c_void_p), ("opacity_abs", C.c_void_p)]
+
+
 def raster_backward(cfg: RasterConfig, grad_image, grad_alpha, image, alpha, positions, features, opacities, w2c,
-                    cam_position=None, gaussian: "GaussianConfig | None" = None):
-    """Returns (grad_features, grad_opacities (N,), grad_view (N,C))."""
+                    cam_position=None, gaussian: "GaussianConfig | None" = None, audit: bool = False):
+    """Returns (grad_features, grad_opacities (N,), grad_view (N,C)); with `audit` a fourth value, a dict of float64
+    arrays: view64 (N,C) / opacity64 (N) = the gradients with every term evaluated and added in double precision,
+    view_abs / opacity_abs = the sums of the magnitudes of what the terms are made of (the conditioning of each sum)."""
     n = cfg.n_points
     sh = cfg.feature_mode in (FEAT_SH36_F16, FEAT_RAW37_F16)
     Cn = 4 if sh else cfg.channels
@@ -396,6 +402,17 @@ def raster_backward(cfg: RasterConfig, grad_image, grad_alpha, image, alpha, pos
         gf = np.zeros((n, Cn), dtype=np.float32)
     go = np.zeros(n, dtype=np.float32)
     gv = np.zeros((n, Cn), dtype=np.float32)
+    if audit:
+        extra = {"view64": np.zeros((n, Cn)), "opacity64": np.zeros(n), "view_abs": np.zeros((n, Cn)),
+                 "opacity_abs": np.zeros(n)}
+        record = _GradAudit(*(_p(extra[k]) for k in ("view64", "opacity64", "view_abs", "opacity_abs")))
+        fn = lib().oracle_raster_backward_audit if gaussian is None else lib().oracle_gaussian_backward_audit
+        rc = fn(C.byref(cfg if gaussian is None else gaussian), _p(grad_image), _p(grad_alpha), _p(image), _p(alpha),
+                _p(positions), _p(features), _p(opacities), _p(w2c), _p(cam_position), _p(gf), _p(go), _p(gv),
+                C.byref(record))
+        if rc != 0:
+            raise RuntimeError(f"oracle_raster_backward_audit failed with {rc}")
+        return gf, go, gv, extra
     fn = lib().oracle_raster_backward if gaussian is None else lib().oracle_gaussian_backward
     rc = fn(C.byref(cfg if gaussian is None else gaussian), _p(grad_image), _p(grad_alpha), _p(image), _p(alpha),
             _p(positions), _p(features), _p(opacities), _p(w2c), _p(cam_position), _p(gf), _p(go), _p(gv))

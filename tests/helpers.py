@@ -417,6 +417,38 @@ class GaussianRun:
         return gf.cpu().numpy(), go.cpu().numpy()
 
 
+# A gradient of the rasterizer is a sum of one term per (instance, pixel), of both signs for most points: evaluated in
+# fp32, in whatever order, it is good to a few rounding units (2^-24) of the sum of the magnitudes its terms are made
+# of, however small the sum itself comes out. kGradUnits is how many of those units a result may be away from the same
+# sum taken in double precision, on top of the 1e-4 relative tolerance of the comparison. Sixteen: a term of the
+# opacity gradient goes through a dot product over the channels and two running sums before it is added; over 2,500
+# random scenes the CPU oracle's own fp32 sums needed up to 9.6 units and the HIP kernels' up to 11.5 (feature
+# gradients: 1.7 and 1.9).
+kGradUnits = 16.0
+
+
+def assert_gradient_close(actual, audit, name, what="", rtol=1e-4, units=kGradUnits):
+    """|actual - f64| <= rtol * |f64| + units * 2^-24 * (sum of magnitudes), element by element; `audit` is the fourth
+    value of oracle.raster_backward(..., audit=True) and `name` is "view" or "opacity". Returns the largest number of
+    rounding units any element needed beyond the relative tolerance."""
+    actual = np.asarray(actual, np.float64)
+    exact, magnitude = audit[name + "64"], audit[name + "_abs"]
+    assert actual.shape == exact.shape, f"{what}: shape {actual.shape} vs {exact.shape}"
+    assert np.isfinite(actual).all(), f"{what}: {int((~np.isfinite(actual)).sum())} non-finite elements"
+    err = np.abs(actual - exact)
+    unit = 2.0 ** -24 * magnitude
+    beyond = np.maximum(err - rtol * np.abs(exact), 0.0)
+    bad = beyond > units * unit
+    if bad.any():
+        idx = np.unravel_index(np.argmax(beyond - units * unit), err.shape)
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.size} elements differ; worst at {idx}: "
+                             f"{actual[idx]!r} vs {exact[idx]!r} (|err|={err[idx]:.3e}, sum of magnitudes "
+                             f"{magnitude[idx]:.3e}: {beyond[idx] / max(unit[idx], 1e-300):.1f} rounding units)")
+    with np.errstate(divide="ignore", invalid="ignore"):
+        used = np.where(unit > 0, beyond / unit, 0.0)
+    return float(used.max(initial=0.0))
+
+
 def assert_close(actual, expected, rtol=1e-4, atol=1e-6, what=""):
     """allclose with a report of the worst element."""
     actual, expected = np.asarray(actual, np.float64), np.asarray(expected, np.float64)

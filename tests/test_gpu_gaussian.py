@@ -303,15 +303,48 @@ def test_reference_tile_size_on_large_images(gpu, oracle, width, height, focal):
     gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
     ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
     gf, go = run.backward(gi, ga)
-    gf_ref, go_ref, _ = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
-                                               gaussian=g)
-    # the near points cover up to thousands of pixels in dozens of tiles at this focal length: their gradients are
-    # sums of that many terms of both signs, added with float atomics in an order that changes from run to run
+    gf_ref, go_ref, _, audit = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac,
+                                                      hv.w2c, gaussian=g, audit=True)
+    # The near points cover up to thousands of pixels in dozens of tiles at this focal length: their gradients are sums
+    # of that many terms of both signs, some of them orders of magnitude smaller than their terms. One bound for every
+    # point: 1e-4 of the sum taken in double precision plus kGradUnits rounding units of the sum of the magnitudes
+    # (tests/helpers.py); the oracle's own fp32 sums are held to the same bound.
+    H.assert_gradient_close(gf, audit, "view", "feature gradients")
+    H.assert_gradient_close(go, audit, "opacity", "opacity gradients")
+    H.assert_gradient_close(gf_ref, audit, "view", "the oracle's fp32 feature gradients")
+    H.assert_gradient_close(go_ref, audit, "opacity", "the oracle's fp32 opacity gradients")
+    # and the points with small footprints also against the fp32 oracle directly
     near = 300
     H.assert_close(gf[near:], gf_ref[near:], RTOL, grad_atol(gf_ref), "feature gradients")
     H.assert_close(go[near:], go_ref[near:], RTOL, grad_atol(go_ref), "opacity gradients")
-    H.assert_close(gf[:near], gf_ref[:near], 1e-3, 2e-6, "feature gradients of the near points")
-    H.assert_close(go[:near], go_ref[:near], 1e-3, 2e-5, "opacity gradients of the near points")
+
+
+@pytest.mark.parametrize("tile,channels", [(8, 4), (16, 8), (16, 16)])
+def test_gradients_are_the_same_bits_on_every_run(gpu, oracle, tile, channels):
+    # Footprints of many pixels and many tiles, added up without float atomics: per instance the pixels' shares in a
+    # fixed order (lanes, then waves), per point the instances' rows in row order. Three forward + backward passes,
+    # each in a workspace of its own with other stale bytes, must agree bit for bit.
+    n = 30000
+    hv, pos, feats, opac = scene(n, channels, seed=90 + tile + channels, near=2000)
+    rng = np.random.default_rng(91)
+    results = []
+    for _ in range(3):
+        run = H.GaussianRun(hv, pos, feats, opac, tile, channels).forward()
+        out = run.outputs()
+        if not results:
+            gi = rng.normal(0, 1e-2, out["image"].shape).astype(np.float32)
+            ga = rng.normal(0, 1e-2, out["alpha"].shape).astype(np.float32)
+        gf, go = run.backward(gi, ga)
+        results.append((gf.copy(), go.copy()))
+    assert np.abs(results[0][0]).max() > 0
+    for gf, go in results[1:]:
+        np.testing.assert_array_equal(gf.view(np.uint32), results[0][0].view(np.uint32))
+        np.testing.assert_array_equal(go.view(np.uint32), results[0][1].view(np.uint32))
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, channels)
+    _, _, _, audit = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                            gaussian=g, audit=True)
+    H.assert_gradient_close(results[0][0], audit, "view", "feature gradients")
+    H.assert_gradient_close(results[0][1], audit, "opacity", "opacity gradients")
 
 
 def test_instances_beyond_the_capacity_are_reported(gpu, oracle):

@@ -290,6 +290,22 @@ def test_backward_against_central_differences(oracle):
     # points that are not drawn get exact zeros
     hidden = ref["n_touched"] == 0
     assert np.all(gf[hidden] == 0) and np.all(go[hidden] == 0)
+    # the audit outputs the GPU tests judge gradients by (pinned against autograd for the bilinear footprint, whose
+    # code they share): the same derivatives, sums of magnitudes that bound the sums, zeros for hidden points, and the
+    # fp32 sums within the bound the GPU results are held to
+    from tests import helpers as H
+    gf2, go2, _, audit = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                                gaussian=g, audit=True)
+    # (two runs of the oracle differ in the last bits where a point lies in several tiles: its threads add in turn)
+    np.testing.assert_allclose(gf2, gf, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(go2, go, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(audit["view64"], gf, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(audit["opacity64"], go, rtol=1e-4, atol=1e-4)
+    assert (audit["view_abs"] >= np.abs(audit["view64"]) * (1 - 1e-12)).all()
+    assert (audit["opacity_abs"] >= np.abs(audit["opacity64"]) * (1 - 1e-12)).all()
+    assert np.all(audit["view_abs"][hidden] == 0) and np.all(audit["opacity_abs"][hidden] == 0)
+    H.assert_gradient_close(gf, audit, "view", "fp32 feature gradients")
+    H.assert_gradient_close(go, audit, "opacity", "fp32 opacity gradients")
 
 
 def test_backward_on_saturating_pixels(oracle):

@@ -292,6 +292,34 @@ def test_backward_against_autograd_and_finite_differences(oracle, tile, channels
     loss.backward()
     np.testing.assert_allclose(gf, f_t.grad.numpy(), rtol=2e-4, atol=2e-5)
     np.testing.assert_allclose(go, o_t.grad.numpy(), rtol=2e-4, atol=2e-5)
+    # The audit outputs that the GPU tests judge gradients by. The double-precision sums are autograd's gradients up
+    # to what the fp32 values they start from (screen position, transmittance, alpha, saved image) are off by: 1e-5 of
+    # the sums of magnitudes, where the fp32 gradients above are only held to 2e-4.
+    gf2, go2, _, audit = oracle.raster_backward(cfg, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                                audit=True)
+    # (two runs of the oracle differ in the last bits where a point lies in several tiles: its threads add in turn)
+    np.testing.assert_allclose(gf2, gf, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(go2, go, rtol=1e-5, atol=1e-6)
+    unit = 2.0 ** -24
+    print("audit vs autograd, in rounding units of the sums of magnitudes:",
+          (np.abs(audit["view64"] - f_t.grad.numpy()) / (unit * audit["view_abs"] + 1e-30)).max(),
+          (np.abs(audit["opacity64"] - o_t.grad.numpy()) / (unit * audit["opacity_abs"] + 1e-30)).max())
+    assert (np.abs(audit["view64"] - f_t.grad.numpy()) <= 1e-5 * audit["view_abs"] + 1e-12).all()
+    assert (np.abs(audit["opacity64"] - o_t.grad.numpy()) <= 1e-5 * audit["opacity_abs"] + 1e-12).all()
+    # a sum of magnitudes bounds its sum, and is not much larger than it has to be: the feature gradient is linear in
+    # the image gradient with non-negative coefficients (the blending weights), so its sum of magnitudes is the
+    # gradient for |grad_image|
+    assert (audit["view_abs"] >= np.abs(audit["view64"]) * (1 - 1e-12)).all()
+    assert (audit["opacity_abs"] >= np.abs(audit["opacity64"]) * (1 - 1e-12)).all()
+    gf_abs, _, _ = oracle.raster_backward(cfg, np.abs(gi), np.zeros_like(ga), ref["image"], ref["alpha"], pos, feats,
+                                          opac, hv.w2c)
+    np.testing.assert_allclose(audit["view_abs"], gf_abs, rtol=1e-5, atol=1e-9)
+    drawn = audit["opacity_abs"] > 0
+    assert np.median(audit["opacity_abs"][drawn] / np.maximum(np.abs(audit["opacity64"][drawn]), 1e-30)) < 50
+    # and the oracle's fp32 sums satisfy the bound the GPU results are held to
+    from tests import helpers as H
+    assert H.assert_gradient_close(gf, audit, "view", "fp32 feature gradients") <= H.kGradUnits
+    assert H.assert_gradient_close(go, audit, "opacity", "fp32 opacity gradients") <= H.kGradUnits
     # central finite differences on a few opacities, through the oracle's own forward
     for i in np.flatnonzero(ref["n_touched"])[:5]:
         eps = 1e-2
