@@ -231,8 +231,8 @@ def main() -> int:
         if args.no_extras:
             raise RuntimeError("skipped (--no-extras)")
         side = torch.cuda.Stream()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
+
+        def step_on_current_stream():
             s = _lib.current_stream()
             _lib.check(lib.inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
                                                _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image), _lib.ptr(alpha),
@@ -242,6 +242,16 @@ def main() -> int:
                                                 _lib.ptr(alpha), _lib.ptr(positions), _lib.ptr(cam_position),
                                                 _lib.ptr(grad_features), _lib.ptr(grad_opacities), None,
                                                 _lib.ptr(workspace), layout.total_bytes, s), "inpc_raster_backward")
+
+        # one eager step on the stream first: the library gives a stream its second stream (for the blend records)
+        # the first time it sees the stream outside a capture
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            step_on_current_stream()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step_on_current_stream()
         graph.replay()
         graph_ms = time_calls(graph.replay, args.steps)
     except Exception as exc:  # the figure is optional

@@ -100,9 +100,11 @@ size_t inpc_sampler_workspace_bytes(uint32_t n_leaves);
  * of B/sampling/include/sampling_utils.h:49-69): 14 levels, which the sampling kernels keep in LDS,
  * and for an octree of more than 278,527 leaves as many more as leave a search with at most sixteen
  * elements (they are read from memory in place of the CDF itself). inpc_cdf_head_floats gives the
- * size of the head for n_leaves leaves: INPC_CDF_HEAD_FLOATS = 2^14 up to 278,527 leaves, the next
- * powers of two beyond (2^17 for 2,097,152 leaves). */
-#define INPC_CDF_HEAD_FLOATS 16384
+ * size of the head for n_leaves leaves: INPC_CDF_HEAD_MIN_FLOATS = 2^14 up to 278,527 leaves, the
+ * next powers of two beyond (2^17 for 2,097,152 leaves). Every call that takes the head also takes
+ * the number of floats the caller's buffer holds (`head_floats`) and returns INPC_E_WORKSPACE, before
+ * anything is launched, when that is less than inpc_cdf_head_floats(n_leaves). */
+#define INPC_CDF_HEAD_MIN_FLOATS 16384
 size_t inpc_cdf_head_floats(uint32_t n_leaves);
 
 /* Normalise the leaf weights and turn them into an inclusive CDF, in place.
@@ -110,14 +112,15 @@ size_t inpc_cdf_head_floats(uint32_t n_leaves);
  * reciprocal-multiply normalisation (B/sampling/src/sampling_kernels.cu:66-75) and
  * cub::DeviceScan::InclusiveSum. The float association order is fixed: left-to-right inside
  * chunks of 64, chunk totals combined the same way one level up, recursively.
- * `sum_out` (dev, inpc_cdf_head_floats(n_leaves) floats, 16-byte aligned) is the head of the CDF: [0]
+ * `sum_out` (dev, head_floats >= inpc_cdf_head_floats(n_leaves) floats, 16-byte aligned) is the head of
+ * the CDF: [0]
  * receives the un-normalised total; when it is <= 0 the weights are left un-normalised and later
- * sampling kernels take the failure path themselves. [1 .. INPC_CDF_HEAD_FLOATS - 1] receive
+ * sampling kernels take the failure path themselves. [1 .. INPC_CDF_HEAD_MIN_FLOATS - 1] receive
  * the CDF elements that the first 14 probes of the binary search of B/sampling/src/
  * sampling_kernels.cu:101-126 can read, in heap order, and behind them those of the further
  * levels. Every later call that takes `sum_dev` takes this buffer. No host synchronisation. */
-int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t workspace_bytes,
-                   uint32_t n_leaves, void* stream);
+int inpc_build_cdf(float* weights_inout, float* sum_out, size_t head_floats, void* workspace,
+                   size_t workspace_bytes, uint32_t n_leaves, void* stream);
 
 /* The same as inpc_build_cdf without a workspace argument: the chunk totals live in a scratch array
  * built into the library (about 261 KB of device memory per GPU the library runs on, held until the
@@ -126,9 +129,12 @@ int inpc_build_cdf(float* weights_inout, float* sum_out, void* workspace, size_t
  * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid allocation).
  * At most INPC_BUILD_CDF_STATIC_MAX_LEAVES leaves (INPC_E_UNSUPPORTED beyond). All calls on one GPU
  * share the one scratch array: calls that overlap on one GPU (different streams or threads) race;
- * calls ordered on one stream do not. Nothing in the scratch has to be cleared between calls. */
+ * calls ordered on one stream do not. Nothing in the scratch has to be cleared between calls.
+ * The first call of a process on a device looks the array's device address up (the runtime may load
+ * the library's code object then): make one call outside any graph capture before capturing one. */
 #define INPC_BUILD_CDF_STATIC_MAX_LEAVES 4194304u
-int inpc_build_cdf_static(float* weights_inout, float* sum_out, uint32_t n_leaves, void* stream);
+int inpc_build_cdf_static(float* weights_inout, float* sum_out, size_t head_floats, uint32_t n_leaves,
+                          void* stream);
 
 /* Multinomial leaf pick + uniform in-leaf jitter, no culling.
  * Replaces create_samples (B/sampling/src/sampling.cu:188-209) and create_samples_cu
@@ -136,9 +142,9 @@ int inpc_build_cdf_static(float* weights_inout, float* sum_out, uint32_t n_leave
  * advanced by 4*i draws; afterwards the device generator is advanced by 4*n_samples.
  * boxes (L,4) f32 as written by inpc_leaf_weights; positions_out (n,3) f32; leaf_ids_out (n,) i32
  * or NULL. If *sum_dev <= 0 nothing is written and the generator is left untouched. */
-int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, float* positions_out,
-                int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves, uint64_t* rng_dev,
-                void* stream);
+int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, size_t head_floats,
+                float* positions_out, int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves,
+                uint64_t* rng_dev, void* stream);
 
 /* Bytes of scratch for inpc_sample_cull_compact over up to n_candidates per round. */
 size_t inpc_cull_workspace_bytes(uint32_t n_candidates);
@@ -158,12 +164,15 @@ int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream);
  * scheduling-dependent atomic slot order is replaced by ascending candidate order.
  * The workspace records, once `capacity` entries exist, how many candidates were consumed
  * (index of the last accepted candidate + 1). The generator is NOT advanced here; see
- * inpc_cull_finish. k0 = 0 starts a new draw: the state in the workspace is cleared first. */
+ * inpc_cull_finish. k0 = 0 starts a new draw: the state in the workspace is cleared first.
+ * leaf_ids_out holds `capacity` int32 values, or int64 values when ids_int64 is not 0 (the dtype of
+ * the tensor the reference returns, B/sampling/src/sampling_api.cu:71: written directly). */
 int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* sum_dev,
-                             const float* w2c, float* positions_out, int32_t* leaf_ids_out,
-                             uint32_t capacity, uint32_t k0, uint32_t n_candidates,
-                             uint32_t n_leaves, const inpc_camera* cam, const uint64_t* rng_dev,
-                             void* workspace, size_t workspace_bytes, void* stream);
+                             size_t head_floats, const float* w2c, float* positions_out,
+                             void* leaf_ids_out, int ids_int64, uint32_t capacity, uint32_t k0,
+                             uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam,
+                             const uint64_t* rng_dev, void* workspace, size_t workspace_bytes,
+                             void* stream);
 
 /* Copy {accepted, consumed} of the current draw to host memory. Synchronises `stream`.
  * The one host read-back of a training draw; it stands where the reference reads the weight
@@ -179,12 +188,12 @@ int inpc_cull_read_counts(const void* workspace, uint32_t* accepted_host, uint32
  * accepted; a caller can enqueue this behind a round before it has read the counts back, and
  * makes the call again with the real number only if the draw needed more rounds. */
 #define INPC_CULL_IF_COMPLETE 0xFFFFFFFFu
-int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_ids_out,
+int inpc_cull_finish(const float* sum_dev, float* positions_out, void* leaf_ids_out, int ids_int64,
                      uint32_t capacity, uint32_t total_candidates, uint64_t* rng_dev,
                      void* workspace, size_t workspace_bytes, void* stream);
 
-/* Widen int32 leaf ids to the int64 the Python API returns
- * (B/sampling/src/sampling_api.cu:71). */
+/* Widen int32 leaf ids to the int64 the Python API returns (B/sampling/src/sampling_api.cu:71),
+ * for callers that drew int32 ids; inpc_sample_cull_compact writes int64 ids itself on request. */
 int inpc_widen_ids(const int32_t* ids, int64_t* out, uint32_t n, void* stream);
 
 /* Expected-count sampler, step 1: count[l] = w>0 ? max(1, rint(w*(1/sum)*n_samples)) : 0 and
@@ -276,13 +285,25 @@ int inpc_raster_layout_query(const inpc_raster_config* cfg, inpc_raster_layout* 
  *   image (C,H,W) f32; alpha (1,H,W) f32;
  *   blending_weights (N,) f32 (training) or NULL; depth_image (1,H,W) f32 (inference) or NULL.
  * The workspace is the saved state the backward pass needs. No host synchronisation. Everything is enqueued on
- * `stream` except the kernel that writes the blend records, which runs beside the tile sort on a second stream of
- * the device (created by the library on first use, default priority); `stream` waits for it before the blend, so
- * to the caller the call is ordered on `stream` like any other. */
+ * `stream` except the kernel that writes the blend records, which runs beside the tile sort on a second stream that
+ * belongs to `stream` alone (created by the library the first time `stream` is used outside a graph capture, default
+ * priority, kept until the process ends); `stream` waits for it before the blend, so to the caller the call is
+ * ordered on `stream` like any other, and calls on different streams share nothing. A capture of `stream` takes its
+ * second stream into the graph; a stream that is first seen while it is being captured gets none and runs
+ * everything on itself (inpc_side_stream_policy). */
 int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, const void* features,
                         const float* opacities, const float* w2c, const float* cam_position,
                         float* image, float* alpha, float* blending_weights, float* depth_image,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* The rule by which inpc_raster_forward decides about the second stream of a caller's stream, as a pure function
+ * of what it finds (no GPU call): existing = a second stream for this (device, stream) exists; stream_is_capturing =
+ * the caller's stream is being captured; second_is_capturing = the second stream is; n_kept = second streams the
+ * process keeps. Returns 0: use the existing one, 1: create one, 2: none, everything runs on the caller's stream
+ * (first seen during a capture; 256 kept already; or the second stream is still inside a capture its owner has
+ * left, which happens when a capture was abandoned half-way). Library plumbing without a counterpart in the
+ * reference, which has a single stream. */
+int inpc_side_stream_policy(int existing, int stream_is_capturing, int second_is_capturing, int n_kept);
 
 /* Backward pass: replays the blend front to back with the saved final image.
  * Replaces backward_wrapper (B/rasterization/src/rasterization_api.cu:109-190),

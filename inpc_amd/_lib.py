@@ -20,7 +20,7 @@ FEAT_RAW37_F16 = 3
 RASTER_INFERENCE = 1
 RASTER_KEEP_GEOMETRY = 2
 CULL_IF_COMPLETE = 0xFFFFFFFF  # INPC_CULL_IF_COMPLETE
-CDF_HEAD_FLOATS = 16384  # INPC_CDF_HEAD_FLOATS: total + the top of the CDF search tree
+CDF_HEAD_MIN_FLOATS = 16384  # INPC_CDF_HEAD_MIN_FLOATS: the smallest CDF head; inpc_cdf_head_floats(n_leaves) sizes one
 
 
 class Camera(C.Structure):
@@ -120,19 +120,21 @@ SIGNATURES = {
     "inpc_pcg32_advance": (None, [_P, C.c_int64]),
     "inpc_leaf_weights": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _CAM, _F, _P]),
     "inpc_sampler_workspace_bytes": (_SZ, [_U32]),
-    "inpc_build_cdf": (C.c_int, [_P, _P, _P, _SZ, _U32, _P]),
-    "inpc_build_cdf_static": (C.c_int, [_P, _P, _U32, _P]),
-    "inpc_sample": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _P, _P]),
+    "inpc_build_cdf": (C.c_int, [_P, _P, _SZ, _P, _SZ, _U32, _P]),
+    "inpc_build_cdf_static": (C.c_int, [_P, _P, _SZ, _U32, _P]),
+    "inpc_sample": (C.c_int, [_P, _P, _P, _SZ, _P, _P, _U32, _U32, _P, _P]),
     "inpc_cull_workspace_bytes": (_SZ, [_U32]),
     "inpc_cull_begin": (C.c_int, [_P, _SZ, _P]),
-    "inpc_sample_cull_compact": (C.c_int, [_P, _P, _P, _P, _P, _P, _U32, _U32, _U32, _U32, _CAM, _P, _P, _SZ, _P]),
+    "inpc_sample_cull_compact": (C.c_int, [_P, _P, _P, _SZ, _P, _P, _P, C.c_int, _U32, _U32, _U32, _U32, _CAM, _P, _P,
+                                           _SZ, _P]),
     "inpc_cull_read_counts": (C.c_int, [_P, C.POINTER(_U32), C.POINTER(_U32), _P]),
-    "inpc_cull_finish": (C.c_int, [_P, _P, _P, _U32, _U32, _P, _P, _SZ, _P]),
+    "inpc_cull_finish": (C.c_int, [_P, _P, _P, C.c_int, _U32, _U32, _P, _P, _SZ, _P]),
     "inpc_widen_ids": (C.c_int, [_P, _P, _U32, _P]),
     "inpc_expected_counts": (C.c_int, [_P, _P, _P, _U32, _P, _SZ, _U32, _P]),
     "inpc_expected_samples": (C.c_int, [_P, _P, _P, _P, _P, _U32, _U32, _U32, _F, _P, _P]),
     "inpc_raster_layout_query": (C.c_int, [_CFG, C.POINTER(RasterLayout)]),
     "inpc_raster_forward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "inpc_side_stream_policy": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "inpc_raster_backward": (C.c_int, [_CFG, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "inpc_raster_read_counters": (C.c_int, [_CFG, _P, C.POINTER(_U32 * 3), _P]),
     "inpc_gaussian_layout_query": (C.c_int, [_GCFG, C.POINTER(GaussianLayout)]),

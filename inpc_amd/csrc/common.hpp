@@ -23,18 +23,22 @@ void timing_begin(const char* name, hipStream_t stream);
 void timing_end(hipStream_t stream);
 bool timing_enabled();   // for the calling thread
 
-// A second stream of the current device for work that does not depend on what the caller's stream is doing at the
-// moment, with the two events that tie it to the caller's stream: `fork` is recorded on the caller's stream and
-// awaited by `stream`, `join` the other way round. Created on first use (non-blocking, default priority) and kept
-// until the process ends; nullptr when it does not exist and `may_create` is false or it cannot be created (the caller
-// then keeps the work on its own stream). Record `fork` and make `stream` wait for it under side_lane_mutex(): the
-// lane is shared by all calls on the device.
+// A second stream for work that does not depend on what the caller's stream is doing at the moment, with the two
+// events that tie it to that stream: `fork` is recorded on the caller's stream and awaited by `stream`, `join` the
+// other way round. Every (device, caller's stream) pair has a lane of its own, so callers on different streams
+// never meet on one, and a capture of the caller's stream takes along a stream nobody else uses. Created on
+// first use (non-blocking, default priority) and kept until the process ends; nullptr when there is none and
+// `may_create` is false (a stream that is being captured gets no new lane), when it cannot be created, when the
+// process already keeps kMaxSideLanes of them, or when the lane's stream is in a capture that the caller's stream is
+// not part of (left over from a capture that was abandoned): the caller then keeps the work on its own stream.
+// Two host threads that enqueue on one stream share its lane: fork under `mutex`.
 struct SideLane {
     hipStream_t stream;
     hipEvent_t fork, join;
+    std::mutex mutex;
 };
-SideLane* side_lane(bool may_create);
-std::mutex& side_lane_mutex();
+constexpr int kMaxSideLanes = 256;
+SideLane* side_lane(hipStream_t owner, bool owner_is_capturing);
 
 #define INPC_HIP_CHECK(expr)                                                                        \
     do {                                                                                            \

@@ -868,12 +868,11 @@ int make_layout(const inpc_raster_config* cfg, Layout& L) {
     }
     capacity = std::max<uint64_t>(std::min(capacity, most), 1);
     g.capacity = (uint32_t)capacity;
-    // gradient rows: the instances of the points that touch several tiles, at most twice the instances beyond one per point
+    // gradient rows: the instances of the points that touch several tiles. With every point drawn they are at most twice
+    // the instances beyond one per point, but when part of the points is culled the rest may all touch several tiles:
+    // as many rows as instances, so that a call whose instances fit never fails for its rows
     g.row_capacity = 0xFFFFFFFFu;
-    if (training) {
-        const uint64_t beyond = capacity > g.n ? capacity - g.n : 0;
-        g.row_capacity = (uint32_t)std::min<uint64_t>(capacity, 2 * beyond + (capacity < most ? 262144ull : 0ull));
-    }
+    if (training) g.row_capacity = (uint32_t)capacity;
 
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -1385,16 +1384,16 @@ int inpc_raster_forward(const inpc_raster_config* cfg, const float* positions, c
         // k_bin_fill, which is bound by memory itself). With the
         // per-launch timing on, everything stays on the caller's stream, so that each duration is that of a kernel
         // that has the device to itself.
-        // (a stream that is being captured into a graph takes the second stream along, but the second stream is not
-        // created during a capture)
+        // A stream that is being captured into a graph takes its lane along (fork and join become edges of the graph);
+        // a lane is never created during a capture, and a stream whose capture state cannot be told gets none.
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         const bool capture_known = hipStreamIsCapturing(stream, &capture) == hipSuccess;
         if (!capture_known) (void)hipGetLastError();
         SideLane* lane = nullptr;
-        if (!timing_enabled() && capture_known) lane = side_lane(capture == hipStreamCaptureStatusNone);
+        if (!timing_enabled() && capture_known) lane = side_lane(stream, capture != hipStreamCaptureStatusNone);
         hipStream_t record_stream = stream;
         if (lane) {
-            std::lock_guard<std::mutex> lock(side_lane_mutex());
+            std::lock_guard<std::mutex> lock(lane->mutex);
             if (hipEventRecord(lane->fork, stream) == hipSuccess &&
                 hipStreamWaitEvent(lane->stream, lane->fork, 0) == hipSuccess) {
                 record_stream = lane->stream;

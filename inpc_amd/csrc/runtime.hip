@@ -1,5 +1,6 @@
 // runtime.hip — error reporting, per-launch timing hooks, fill kernel, PCG32 host helpers.
 #include <algorithm>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -50,21 +51,64 @@ int fail(int code, const char* fmt, ...) {
 bool timing_enabled() { return g_timing_on; }
 
 namespace {
-constexpr int kMaxDevices = 64;
+struct LaneEntry {
+    int device;
+    hipStream_t owner;
+    SideLane lane;
+};
 std::mutex g_lane_mutex;
-SideLane g_lanes[kMaxDevices] = {};
-bool g_lane_ready[kMaxDevices] = {};
+std::vector<std::unique_ptr<LaneEntry>> g_lanes;   // entries never move or go away: callers keep pointers to them
 }  // namespace
 
-std::mutex& side_lane_mutex() { return g_lane_mutex; }
+// Which lane, if any, a forward pass on `owner` may use: the decision of side_lane() without the HIP calls.
+//   existing:           a lane for (device, owner) exists
+//   owner_is_capturing: the caller's stream is being captured into a graph
+//   lane_is_capturing:  the lane's stream is (only asked when a lane exists)
+//   n_lanes:            lanes the process keeps
+enum class LaneChoice : int { kUse = 0, kCreate = 1, kNone = 2 };
+LaneChoice choose_lane(bool existing, bool owner_is_capturing, bool lane_is_capturing, int n_lanes) {
+    if (existing) {
+        // between two calls the lane's stream is idle and outside any capture: each call joins it back into the
+        // caller's stream before it returns. A lane that still captures although its owner does not belongs to a
+        // capture that was abandoned half-way; it is left alone.
+        if (lane_is_capturing && !owner_is_capturing) return LaneChoice::kNone;
+        return LaneChoice::kUse;
+    }
+    if (owner_is_capturing) return LaneChoice::kNone;   // creating a stream is no operation for a capture
+    if (n_lanes >= kMaxSideLanes) return LaneChoice::kNone;
+    return LaneChoice::kCreate;
+}
 
-SideLane* side_lane(bool may_create) {
+SideLane* side_lane(hipStream_t owner, bool owner_is_capturing) {
     int device = -1;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+    if (hipGetDevice(&device) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
     std::lock_guard<std::mutex> lock(g_lane_mutex);
-    if (g_lane_ready[device]) return &g_lanes[device];
-    if (!may_create) return nullptr;
-    SideLane lane{nullptr, nullptr, nullptr};
+    LaneEntry* found = nullptr;
+    for (auto& e : g_lanes)
+        if (e->device == device && e->owner == owner) found = e.get();
+    bool lane_is_capturing = false;
+    if (found) {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(found->lane.stream, &status) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        lane_is_capturing = status != hipStreamCaptureStatusNone;
+    }
+    switch (choose_lane(found != nullptr, owner_is_capturing, lane_is_capturing, (int)g_lanes.size())) {
+        case LaneChoice::kUse: return &found->lane;
+        case LaneChoice::kNone: return nullptr;
+        case LaneChoice::kCreate: break;
+    }
+    auto entry = std::make_unique<LaneEntry>();
+    entry->device = device;
+    entry->owner = owner;
+    SideLane& lane = entry->lane;
+    lane.stream = nullptr;
+    lane.fork = lane.join = nullptr;
     // no timing data in the events: they only order the two streams
     if (hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking) != hipSuccess ||
         hipEventCreateWithFlags(&lane.fork, hipEventDisableTiming) != hipSuccess ||
@@ -74,9 +118,8 @@ SideLane* side_lane(bool may_create) {
         if (lane.stream) (void)hipStreamDestroy(lane.stream);
         return nullptr;
     }
-    g_lanes[device] = lane;
-    g_lane_ready[device] = true;
-    return &g_lanes[device];
+    g_lanes.push_back(std::move(entry));
+    return &g_lanes.back()->lane;
 }
 
 void timing_begin(const char* name, hipStream_t stream) {
@@ -161,7 +204,11 @@ int inpc_calibration_copy(const void* src, void* dst, size_t bytes, void* stream
 
 const char* inpc_last_error(void) { return inpc::g_error; }
 
-int inpc_abi_version(void) { return 3; }
+int inpc_abi_version(void) { return 4; }
+
+int inpc_side_stream_policy(int existing, int stream_is_capturing, int second_is_capturing, int n_kept) {
+    return (int)inpc::choose_lane(existing != 0, stream_is_capturing != 0, second_is_capturing != 0, n_kept);
+}
 
 void inpc_timing_enable(int on) {
     inpc::g_timing_on = on != 0;

@@ -176,7 +176,7 @@ __global__ void __launch_bounds__(kBlock) k_chunk_add_prefix(float* data, uint32
 constexpr uint32_t kFetch = 16;   // elements of a search that four lanes fetch together
 constexpr int kTreeDepth = 14;
 constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNodes - 1; index 0 of the head: the total
-static_assert(kTreeNodes == INPC_CDF_HEAD_FLOATS, "the CDF head holds the total and the search tree");
+static_assert(kTreeNodes == INPC_CDF_HEAD_MIN_FLOATS, "the CDF head holds the total and the search tree");
 static_assert(kSampleItems * (kDrawBlock / kWave) <= kWave, "one wave scans the (round, wave) counts of a tile");
 
 // head[node] for every node of the tree (one thread per node).
@@ -447,9 +447,12 @@ struct CullState {
 constexpr size_t kCullHeaderWords = sizeof(CullState) / 4;
 constexpr int kTileJumpBits = 20;   // a round has fewer than 2^20 tiles (candidate indices stay below 2^30)
 
+// Id: the type the caller wants the leaf indices in (int32_t, or the int64_t of the Python API's tensors,
+// B/sampling/src/sampling_api.cu:71: written here directly instead of widened by a pass of its own).
+template <typename Id>
 __global__ void __launch_bounds__(kDrawBlock)
     k_sample_cull(const float4* __restrict__ boxes, const float* __restrict__ cdf, const float* __restrict__ sum_dev,
-                  const float* __restrict__ w2c, float* __restrict__ positions, int32_t* __restrict__ leaf_ids,
+                  const float* __restrict__ w2c, float* __restrict__ positions, Id* __restrict__ leaf_ids,
                   uint32_t capacity, uint32_t k0, uint32_t n_candidates, uint32_t n_blocks, uint32_t n_leaves, Camera cam,
                   const uint64_t* __restrict__ rng_dev, CullState* st, uint32_t* status) {
     __shared__ uint32_t s_accepted0, s_exclusive, s_done, s_bid;
@@ -541,7 +544,7 @@ __global__ void __launch_bounds__(kDrawBlock)
             positions[3 * slot] = cand[j].x;
             positions[3 * slot + 1] = cand[j].y;
             positions[3 * slot + 2] = cand[j].z;
-            leaf_ids[slot] = (int32_t)cand[j].leaf;
+            leaf_ids[slot] = (Id)cand[j].leaf;
             if (slot + 1 == capacity) {
                 const uint64_t rel = tile_first + (uint64_t)j * kDrawBlock + tid;
                 __hip_atomic_store(&st->consumed, (uint32_t)(k0 + rel + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -562,8 +565,9 @@ __global__ void k_cull_round_reset(uint32_t* status, uint32_t n_blocks, CullStat
 // End of a draw. A positive weight sum: the generator moves on by four draws per consumed candidate. Otherwise: the
 // failure pattern of B/sampling/src/sampling.cu:107-111 in the outputs (a small grid, so that the usual case costs
 // next to nothing) and the generator stays where it is.
+template <typename Id>
 __global__ void __launch_bounds__(kBlock) k_cull_finish(const float* __restrict__ sum_dev, uint64_t* rng_dev,
-                                                        const CullState* st, float* positions, int32_t* leaf_ids,
+                                                        const CullState* st, float* positions, Id* leaf_ids,
                                                         uint32_t capacity, uint32_t total_candidates) {
     if (*sum_dev > 0.0f) {
         if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -580,7 +584,7 @@ __global__ void __launch_bounds__(kBlock) k_cull_finish(const float* __restrict_
         positions[3 * (size_t)i] = 0.0f;
         positions[3 * (size_t)i + 1] = 0.0f;
         positions[3 * (size_t)i + 2] = 0.0f;
-        leaf_ids[i] = -1;
+        leaf_ids[i] = (Id)-1;
     }
 }
 
@@ -830,17 +834,27 @@ size_t inpc_sampler_workspace_bytes(uint32_t n_leaves) { return sampler_workspac
 
 size_t inpc_cdf_head_floats(uint32_t n_leaves) { return (size_t)1 << tree_levels(n_leaves); }
 
-int inpc_build_cdf(float* w, float* sum_out, void* workspace, size_t workspace_bytes, uint32_t n_leaves,
-                   void* stream_) {
+// The head of a CDF for n_leaves leaves holds inpc_cdf_head_floats(n_leaves) floats: the kernels write and read that many.
+static int check_head(const char* who, size_t head_floats, uint32_t n_leaves) {
+    const size_t need = (size_t)1 << tree_levels(n_leaves);
+    if (head_floats < need)
+        return fail(INPC_E_WORKSPACE, "%s: the CDF head has %zu floats, %u leaves need %zu (inpc_cdf_head_floats)", who,
+                    head_floats, n_leaves, need);
+    return INPC_OK;
+}
+
+int inpc_build_cdf(float* w, float* sum_out, size_t head_floats, void* workspace, size_t workspace_bytes,
+                   uint32_t n_leaves, void* stream_) {
     if (n_leaves == 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: no leaves");
     if (!w || !sum_out || !workspace) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: null pointer");
+    if (const int rc = check_head("inpc_build_cdf", head_floats, n_leaves); rc != INPC_OK) return rc;
     if (workspace_bytes < sampler_workspace_bytes(n_leaves))
         return fail(INPC_E_WORKSPACE, "inpc_build_cdf: workspace has %zu bytes, needs %zu", workspace_bytes,
                     sampler_workspace_bytes(n_leaves));
     return launch_build_cdf(w, sum_out, (float*)workspace, n_leaves, (hipStream_t)stream_);
 }
 
-int inpc_build_cdf_static(float* w, float* sum_out, uint32_t n_leaves, void* stream_) {
+int inpc_build_cdf_static(float* w, float* sum_out, size_t head_floats, uint32_t n_leaves, void* stream_) {
     if (n_leaves == 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf_static: no leaves");
     if (!w || !sum_out) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf_static: null pointer");
     if (n_leaves > INPC_BUILD_CDF_STATIC_MAX_LEAVES)
@@ -848,13 +862,14 @@ int inpc_build_cdf_static(float* w, float* sum_out, uint32_t n_leaves, void* str
                     n_leaves, (unsigned)INPC_BUILD_CDF_STATIC_MAX_LEAVES);
     if (plan_levels(n_leaves).total_floats > kStaticTotalsFloats)
         return fail(INPC_E_UNSUPPORTED, "inpc_build_cdf_static: the built-in scratch is too small for %u leaves", n_leaves);
+    if (const int rc = check_head("inpc_build_cdf_static", head_floats, n_leaves); rc != INPC_OK) return rc;
     float* totals = nullptr;
     const int rc = static_totals(totals);
     if (rc != INPC_OK) return rc;
     return launch_build_cdf(w, sum_out, totals, n_leaves, (hipStream_t)stream_);
 }
 
-int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, float* positions_out,
+int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, size_t head_floats, float* positions_out,
                 int32_t* leaf_ids_out, uint32_t n_samples, uint32_t n_leaves, uint64_t* rng_dev, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (n_samples == 0) return INPC_OK;
@@ -862,6 +877,7 @@ int inpc_sample(const float* boxes, const float* cdf, const float* sum_dev, floa
     if (n_leaves == 0 || !boxes || !cdf || !sum_dev || !positions_out || !rng_dev)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: null pointer or no leaves");
     if (((uintptr_t)boxes & 15u) != 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample: boxes must be 16-byte aligned");
+    if (const int rc = check_head("inpc_sample", head_floats, n_leaves); rc != INPC_OK) return rc;
     INPC_LAUNCH("sample", k_sample, dim3(div_up(n_samples, kDrawTile)), dim3(kDrawBlock), stream, (const float4*)boxes, cdf,
                 sum_dev, positions_out, leaf_ids_out, n_samples, n_leaves, (const uint64_t*)rng_dev);
     INPC_LAUNCH("rng_advance", k_rng_advance, dim3(1), dim3(64), stream, rng_dev, sum_dev, 4ull * n_samples);
@@ -878,10 +894,10 @@ int inpc_cull_begin(void* workspace, size_t workspace_bytes, void* stream) {
     return fill_u32(workspace, 0u, kCullHeaderWords, (hipStream_t)stream);
 }
 
-int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* sum_dev, const float* w2c,
-                             float* positions_out, int32_t* leaf_ids_out, uint32_t capacity, uint32_t k0,
-                             uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam, const uint64_t* rng_dev,
-                             void* workspace, size_t workspace_bytes, void* stream_) {
+int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* sum_dev, size_t head_floats,
+                             const float* w2c, float* positions_out, void* leaf_ids_out, int ids_int64, uint32_t capacity,
+                             uint32_t k0, uint32_t n_candidates, uint32_t n_leaves, const inpc_camera* cam,
+                             const uint64_t* rng_dev, void* workspace, size_t workspace_bytes, void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (n_candidates == 0) {   // nothing to draw; a new draw still starts from a cleared state
         if (k0 == 0u && workspace && workspace_bytes >= sizeof(CullState))
@@ -895,6 +911,7 @@ int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* 
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_sample_cull_compact: boxes must be 16-byte aligned");
     if ((uint64_t)k0 + n_candidates >= (1ull << 30))
         return fail(INPC_E_UNSUPPORTED, "inpc_sample_cull_compact: candidate index must stay below 2^30");
+    if (const int rc = check_head("inpc_sample_cull_compact", head_floats, n_leaves); rc != INPC_OK) return rc;
     if (workspace_bytes < inpc_cull_workspace_bytes(n_candidates))
         return fail(INPC_E_WORKSPACE, "inpc_sample_cull_compact: workspace has %zu bytes, needs %zu", workspace_bytes,
                     inpc_cull_workspace_bytes(n_candidates));
@@ -905,11 +922,18 @@ int inpc_sample_cull_compact(const float* boxes, const float* cdf, const float* 
                 dim3(kBlock), stream, status, n_blocks, st, k0 == 0u);
     // as many blocks as the GPU holds at once; each takes tiles until none is left
     uint32_t resident = 0;
-    const int rc = resident_blocks((const void*)k_sample_cull, kDrawBlock, resident);
+    const int rc = resident_blocks(ids_int64 ? (const void*)k_sample_cull<int64_t> : (const void*)k_sample_cull<int32_t>,
+                                   kDrawBlock, resident);
     if (rc != INPC_OK) return rc;
-    INPC_LAUNCH("sample_cull_compact", k_sample_cull, dim3(std::min(n_blocks, resident)), dim3(kDrawBlock), stream,
-                (const float4*)boxes, cdf, sum_dev, w2c, positions_out, leaf_ids_out, capacity, k0, n_candidates, n_blocks,
-                n_leaves, to_device_camera(*cam), rng_dev, st, status);
+    if (ids_int64) {
+        INPC_LAUNCH("sample_cull_compact", k_sample_cull<int64_t>, dim3(std::min(n_blocks, resident)), dim3(kDrawBlock),
+                    stream, (const float4*)boxes, cdf, sum_dev, w2c, positions_out, (int64_t*)leaf_ids_out, capacity, k0,
+                    n_candidates, n_blocks, n_leaves, to_device_camera(*cam), rng_dev, st, status);
+    } else {
+        INPC_LAUNCH("sample_cull_compact", k_sample_cull<int32_t>, dim3(std::min(n_blocks, resident)), dim3(kDrawBlock),
+                    stream, (const float4*)boxes, cdf, sum_dev, w2c, positions_out, (int32_t*)leaf_ids_out, capacity, k0,
+                    n_candidates, n_blocks, n_leaves, to_device_camera(*cam), rng_dev, st, status);
+    }
     return INPC_OK;
 }
 
@@ -924,15 +948,20 @@ int inpc_cull_read_counts(const void* workspace, uint32_t* accepted_host, uint32
     return INPC_OK;
 }
 
-int inpc_cull_finish(const float* sum_dev, float* positions_out, int32_t* leaf_ids_out, uint32_t capacity,
+int inpc_cull_finish(const float* sum_dev, float* positions_out, void* leaf_ids_out, int ids_int64, uint32_t capacity,
                      uint32_t total_candidates, uint64_t* rng_dev, void* workspace, size_t workspace_bytes,
                      void* stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     if (!sum_dev || !rng_dev || !workspace || workspace_bytes < sizeof(CullState))
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_cull_finish: null pointer");
-    INPC_LAUNCH("cull_finish", k_cull_finish, dim3(std::max(std::min(div_up(capacity, kBlock), 1024u), 1u)), dim3(kBlock),
-                stream, sum_dev, rng_dev, (const CullState*)workspace, positions_out, leaf_ids_out, capacity,
-                total_candidates);
+    const dim3 grid(std::max(std::min(div_up(capacity, kBlock), 1024u), 1u));
+    if (ids_int64) {
+        INPC_LAUNCH("cull_finish", k_cull_finish<int64_t>, grid, dim3(kBlock), stream, sum_dev, rng_dev,
+                    (const CullState*)workspace, positions_out, (int64_t*)leaf_ids_out, capacity, total_candidates);
+    } else {
+        INPC_LAUNCH("cull_finish", k_cull_finish<int32_t>, grid, dim3(kBlock), stream, sum_dev, rng_dev,
+                    (const CullState*)workspace, positions_out, (int32_t*)leaf_ids_out, capacity, total_candidates);
+    }
     return INPC_OK;
 }
 

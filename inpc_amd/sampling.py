@@ -111,8 +111,8 @@ class ProbabilityFieldSampler(torch.nn.Module):
         vw, boxes, ws, ws_bytes, total, cam, stream = self._weights(centers, levels, weights, w2c, view, initial_size)
         n = centers.shape[0]
         if n > 0:
-            _lib.check(_lib.lib().inpc_build_cdf(_lib.ptr(vw), _lib.ptr(total), _lib.ptr(ws), ws_bytes, n, stream),
-                       "inpc_build_cdf")
+            _lib.check(_lib.lib().inpc_build_cdf(_lib.ptr(vw), _lib.ptr(total), total.numel(), _lib.ptr(ws), ws_bytes, n,
+                                                 stream), "inpc_build_cdf")
         return vw, boxes, total, cam, stream
 
     # -- API ---------------------------------------------------------------------------------------------
@@ -127,8 +127,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
         n_leaves = centers.shape[0]
         n_samples = int(n_samples)
         positions = torch.empty((n_samples, 3), dtype=torch.float32, device=device)
-        ids32 = torch.empty(n_samples, dtype=torch.int32, device=device)
-        ids64 = torch.empty(n_samples, dtype=torch.int64, device=device)
+        ids64 = torch.empty(n_samples, dtype=torch.int64, device=device)   # written by the kernels as int64
         if n_samples == 0:
             return positions, ids64
         if n_leaves == 0:
@@ -145,16 +144,15 @@ class ProbabilityFieldSampler(torch.nn.Module):
         finished = False
 
         def finish(total_candidates):
-            _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples,
+            _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids64), 1, n_samples,
                                             total_candidates, _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream),
                        "inpc_cull_finish")
-            _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
 
         while True:
-            _lib.check(lib.inpc_sample_cull_compact(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(w2c),
-                                                    _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0, n_round,
-                                                    n_leaves, C.byref(cam), _lib.ptr(rng), _lib.ptr(cull_ws),
-                                                    cull_bytes, stream), "inpc_sample_cull_compact")
+            _lib.check(lib.inpc_sample_cull_compact(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), total.numel(),
+                                                    _lib.ptr(w2c), _lib.ptr(positions), _lib.ptr(ids64), 1, n_samples,
+                                                    k0, n_round, n_leaves, C.byref(cam), _lib.ptr(rng),
+                                                    _lib.ptr(cull_ws), cull_bytes, stream), "inpc_sample_cull_compact")
             k0 += n_round
             if k0 == n_round:
                 # the first round nearly always completes the draw: its end is enqueued before the counts are read
@@ -177,8 +175,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
             self._acceptance = n_samples / consumed.value
         self.last_consumed = int(consumed.value) if consumed.value else k0
         if not finished:
-            _lib.check(lib.inpc_cull_finish(_lib.ptr(total), _lib.ptr(positions), _lib.ptr(ids32), n_samples, k0,
-                                            _lib.ptr(rng), _lib.ptr(cull_ws), cull_bytes, stream), "inpc_cull_finish")
+            finish(k0)
         if consumed.value == 0 and accepted.value < n_samples and float(total[0].item()) > 0.0:
             # the draw gave up (the frustum is hardly ever hit, or the candidate limit was reached): the slots behind
             # the accepted samples get the failure pattern of B/sampling/src/sampling.cu:107-111, positions 0 and
@@ -186,9 +183,7 @@ class ProbabilityFieldSampler(torch.nn.Module):
             _log.warning("sampler accepted only %d of %d samples; the rest is filled with position 0 / index -1",
                          accepted.value, n_samples)
             positions[accepted.value:].zero_()
-            ids32[accepted.value:].fill_(-1)
-        if not finished:
-            _lib.check(lib.inpc_widen_ids(_lib.ptr(ids32), _lib.ptr(ids64), n_samples, stream), "inpc_widen_ids")
+            ids64[accepted.value:].fill_(-1)
         return positions, ids64
 
     def generate_samples(self, centers, levels, weights, view, n_samples: int, initial_size: float) -> torch.Tensor:
@@ -205,8 +200,9 @@ class ProbabilityFieldSampler(torch.nn.Module):
             return torch.empty((0, 3), dtype=torch.float32, device=device)
         n_samples = int(n_samples)
         positions = torch.empty((n_samples, 3), dtype=torch.float32, device=device)
-        _lib.check(_lib.lib().inpc_sample(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(positions), None,
-                                          n_samples, n_leaves, _lib.ptr(self._rng_dev(device)), stream), "inpc_sample")
+        _lib.check(_lib.lib().inpc_sample(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), total.numel(),
+                                          _lib.ptr(positions), None, n_samples, n_leaves,
+                                          _lib.ptr(self._rng_dev(device)), stream), "inpc_sample")
         return positions
 
     def generate_expected_samples(self, centers, levels, weights, view, n_samples: int, n_multi: int,

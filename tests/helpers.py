@@ -73,7 +73,7 @@ def build_cdf(w_dev):
     ws_bytes = int(lib.inpc_sampler_workspace_bytes(n))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=w_dev.device)
     total = torch.zeros(int(lib.inpc_cdf_head_floats(n)), dtype=torch.float32, device=w_dev.device)  # [0] = total
-    _lib.check(lib.inpc_build_cdf(_lib.ptr(cdf), _lib.ptr(total), _lib.ptr(ws), ws_bytes, n, stream()),
+    _lib.check(lib.inpc_build_cdf(_lib.ptr(cdf), _lib.ptr(total), total.numel(), _lib.ptr(ws), ws_bytes, n, stream()),
                "inpc_build_cdf")
     return cdf, total
 
@@ -84,22 +84,23 @@ def sample(oct, cdf, total, n_samples, rng_dev):
     pos = torch.full((n_samples, 3), float("nan"), dtype=torch.float32, device=device)
     ids = torch.full((n_samples,), -7, dtype=torch.int32, device=device)
     boxes = leaf_boxes(oct)
-    _lib.check(lib.inpc_sample(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), _lib.ptr(pos), _lib.ptr(ids), n_samples,
-                               len(oct.levels), _lib.ptr(rng_dev), stream()), "inpc_sample")
+    _lib.check(lib.inpc_sample(_lib.ptr(boxes), _lib.ptr(cdf), _lib.ptr(total), total.numel(), _lib.ptr(pos),
+                               _lib.ptr(ids), n_samples, len(oct.levels), _lib.ptr(rng_dev), stream()), "inpc_sample")
     return pos.cpu().numpy(), ids.cpu().numpy()
 
 
 class CullDraw:
     """One training draw made of explicit rounds."""
 
-    def __init__(self, oct, hv, cdf, total, rng_dev, capacity, max_round):
+    def __init__(self, oct, hv, cdf, total, rng_dev, capacity, max_round, ids_int64=False):
         self.lib = _lib.lib()
+        self.ids_int64 = int(ids_int64)
         self.oct, self.hv, self.cdf, self.total, self.rng = oct, hv, cdf, total, rng_dev
         self.capacity = capacity
         device = cdf.device
         self.boxes, self.w2c = leaf_boxes(oct, hv), dev(hv.w2c)
         self.pos = torch.full((capacity, 3), float("nan"), dtype=torch.float32, device=device)
-        self.ids = torch.full((capacity,), -7, dtype=torch.int32, device=device)
+        self.ids = torch.full((capacity,), -7, dtype=torch.int64 if ids_int64 else torch.int32, device=device)
         self.ws_bytes = int(self.lib.inpc_cull_workspace_bytes(max_round))
         # poisoned: the round that starts at candidate 0 clears the state of the draw itself
         self.ws = torch.randint(0, 256, (self.ws_bytes,), dtype=torch.uint8, device=device)
@@ -108,9 +109,9 @@ class CullDraw:
 
     def round(self, n_candidates):
         _lib.check(self.lib.inpc_sample_cull_compact(
-            _lib.ptr(self.boxes), _lib.ptr(self.cdf), _lib.ptr(self.total), _lib.ptr(self.w2c), _lib.ptr(self.pos),
-            _lib.ptr(self.ids), self.capacity, self.k0, n_candidates, len(self.oct.levels), C.byref(self.cam),
-            _lib.ptr(self.rng), _lib.ptr(self.ws), self.ws_bytes, stream()),
+            _lib.ptr(self.boxes), _lib.ptr(self.cdf), _lib.ptr(self.total), self.total.numel(), _lib.ptr(self.w2c),
+            _lib.ptr(self.pos), _lib.ptr(self.ids), self.ids_int64, self.capacity, self.k0, n_candidates,
+            len(self.oct.levels), C.byref(self.cam), _lib.ptr(self.rng), _lib.ptr(self.ws), self.ws_bytes, stream()),
             "inpc_sample_cull_compact")
         self.k0 += n_candidates
         return self.counts()
@@ -122,7 +123,7 @@ class CullDraw:
         return int(a.value), int(c.value)
 
     def finish(self):
-        _lib.check(self.lib.inpc_cull_finish(_lib.ptr(self.total), _lib.ptr(self.pos), _lib.ptr(self.ids),
+        _lib.check(self.lib.inpc_cull_finish(_lib.ptr(self.total), _lib.ptr(self.pos), _lib.ptr(self.ids), self.ids_int64,
                                              self.capacity, self.k0, _lib.ptr(self.rng), _lib.ptr(self.ws),
                                              self.ws_bytes, stream()), "inpc_cull_finish")
 

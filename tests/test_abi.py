@@ -33,7 +33,8 @@ def test_header_functions_are_exported_and_bound():
 def test_header_constants_match_the_binder():
     # the CDF head the callers allocate: the header's size is the one the Python layer uses
     text = HEADER.read_text()
-    assert int(re.search(r"#define\s+INPC_CDF_HEAD_FLOATS\s+(\d+)", text).group(1)) == _lib.CDF_HEAD_FLOATS
+    assert int(re.search(r"#define\s+INPC_CDF_HEAD_MIN_FLOATS\s+(\d+)", text).group(1)) == _lib.CDF_HEAD_MIN_FLOATS
+    assert _lib.lib().inpc_cdf_head_floats(1) == _lib.CDF_HEAD_MIN_FLOATS
     for name in ("DIRECT_F32", "DIRECT_F16", "SH36_F16", "RAW37_F16"):
         assert int(re.search(rf"#define\s+INPC_FEAT_{name}\s+(\d+)", text).group(1)) == getattr(_lib, f"FEAT_{name}")
 
@@ -45,7 +46,7 @@ def test_every_entry_point_cites_the_interface_it_replaces():
         if name in ("inpc_last_error", "inpc_abi_version", "inpc_timing_enable", "inpc_timing_collect",
                     "inpc_raster_layout_query", "inpc_raster_read_counters", "inpc_sampler_workspace_bytes",
                     "inpc_cull_workspace_bytes", "inpc_calibration_copy", "inpc_field_update_workspace_bytes",
-                    "inpc_field_update_check", "inpc_build_cdf_static"):
+                    "inpc_field_update_check", "inpc_build_cdf_static", "inpc_side_stream_policy"):
             continue  # library plumbing without a counterpart
         at = text.index(name + "(")
         before = text[:at]
@@ -93,7 +94,7 @@ def make_cfg(n, w, h, tile=16, channels=8, mode=_lib.FEAT_DIRECT_F32, flags=0, m
 
 def test_layout_query_on_the_host():
     lib = _lib.lib()
-    assert lib.inpc_abi_version() >= 3
+    assert lib.inpc_abi_version() >= 4
     n = 8_388_608
     layout = _lib.RasterLayout()
     cfg = make_cfg(n, 1237, 822)
@@ -108,7 +109,7 @@ def test_layout_query_on_the_host():
     assert 1.129 * n < layout.max_instances < 1.25 * n
     # one record per point, per instance a sort pair, a list entry and (training) an ordered record
     assert layout.total_bytes >= n * 64 + layout.max_instances * (8 + 4 + 64)
-    assert layout.total_bytes < 1.5e9
+    assert layout.total_bytes < 1.75e9   # the gradient rows are sized like the instances: culling never makes a call fail for its rows
     assert layout.end_bit == (layout.n_tiles - 1).bit_length() == 12
     # the caller may ask for room for every possible instance, and never gets more
     for asked, got in ((4 * n, 4 * n), (0xFFFFFFFF, 4 * n), (n, n)):
@@ -185,11 +186,44 @@ def test_argument_checks_come_before_any_launch():
     assert lib.inpc_raster_forward(C.byref(cfg), None, None, None, None, None, None, None, None, None, None, 0,
                                    None) in (-1, -2)
     assert lib.inpc_raster_layout_query(None, None) == -1
-    assert lib.inpc_build_cdf(None, None, None, 0, 10, None) in (-1, -2)
+    assert lib.inpc_build_cdf(None, None, 0, None, 0, 10, None) in (-1, -2)
     assert lib.inpc_cull_begin(None, 0, None) in (-1, -2)
     assert lib.inpc_sampler_workspace_bytes(1) > 0
     assert lib.inpc_sampler_workspace_bytes(1 << 27) >= lib.inpc_sampler_workspace_bytes(1 << 20)
     assert lib.inpc_cull_workspace_bytes(1 << 20) >= 256  # status words only: accepted samples go straight to the output
+
+
+def test_a_cdf_head_that_is_too_small_is_refused_before_any_launch():
+    # The head of a CDF grows with the octree (16,384 floats up to 278,527 leaves, 131,072 for 2,097,152): every call
+    # that writes or reads it is told how many floats the caller's buffer holds and refuses a short one on the host.
+    lib = _lib.lib()
+    assert lib.inpc_cdf_head_floats(278_527) == 16384 and lib.inpc_cdf_head_floats(278_528) == 32768
+    assert lib.inpc_cdf_head_floats(2_097_152) == 131072
+    fake = (C.c_char * 256)()   # never dereferenced: the calls below return before they launch anything
+    p = C.c_void_p((C.addressof(fake) + 15) & ~15)
+    cam = _lib.Camera(64, 64, 50.0, 50.0, 32.0, 32.0, 0.01, 100.0)
+    n_leaves, short = 2_097_152, 16384
+    assert lib.inpc_build_cdf(p, p, short, p, 1 << 30, n_leaves, None) == -2
+    assert b"131072" in lib.inpc_last_error()
+    assert lib.inpc_build_cdf_static(p, p, short, n_leaves, None) == -2
+    assert lib.inpc_sample(p, p, p, short, p, None, 1000, n_leaves, p, None) == -2
+    assert lib.inpc_sample_cull_compact(p, p, p, short, p, p, p, 0, 1000, 0, 1000, n_leaves, C.byref(cam), p, p, 1 << 20,
+                                        None) == -2
+    assert b"inpc_cdf_head_floats" in lib.inpc_last_error()
+
+
+def test_second_stream_policy():
+    # inpc_raster_forward writes its blend records on a second stream that belongs to the caller's stream alone.
+    use, create, none = 0, 1, 2
+    policy = _lib.lib().inpc_side_stream_policy
+    assert policy(0, 0, 0, 0) == create                 # first call on a stream, outside a capture
+    assert policy(0, 1, 0, 0) == none                   # first seen while it is captured: nothing is created then
+    assert policy(1, 0, 0, 5) == use
+    assert policy(1, 1, 0, 5) == use                    # the capture takes the second stream along ...
+    assert policy(1, 1, 1, 5) == use                    # ... also for the later calls of the same capture
+    assert policy(1, 0, 1, 5) == none                   # left inside a capture its owner has abandoned: not touched
+    assert policy(0, 0, 0, 256) == none                 # the process keeps 256 already
+    assert policy(1, 0, 0, 256) == use
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):

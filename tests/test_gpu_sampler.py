@@ -118,8 +118,9 @@ def test_sample_failure_path_writes_nothing(gpu):
     assert H.rng_values(rng_dev) == before
 
 
+@pytest.mark.parametrize("ids_int64", [False, True], ids=["int32_ids", "int64_ids"])
 @pytest.mark.parametrize("rounds", [[50000], [2048, 2047, 1, 30000], [10000, 10000, 10000]])
-def test_cull_compact_rounds_bit_exact(gpu, oracle, rounds):
+def test_cull_compact_rounds_bit_exact(gpu, oracle, rounds, ids_int64):
     oct, hv = small_scene(distance=2.2)  # close camera: a good share of candidates is rejected
     cam = oracle_cam(oracle, hv)
     w = H.leaf_weights(oct, hv)
@@ -128,7 +129,7 @@ def test_cull_compact_rounds_bit_exact(gpu, oracle, rounds):
     capacity = 20000
     rng_dev = H.make_rng(77)
     rng_ref = oracle.Pcg32(77)
-    draw = H.CullDraw(oct, hv, cdf, total, rng_dev, capacity, max(rounds))
+    draw = H.CullDraw(oct, hv, cdf, total, rng_dev, capacity, max(rounds), ids_int64=ids_int64)
     pos_ref, ids_ref, acc_ref, cons_ref, k0 = None, None, 0, 0, 0
     for m in rounds:
         acc_gpu, cons_gpu = draw.round(m)
@@ -144,6 +145,7 @@ def test_cull_compact_rounds_bit_exact(gpu, oracle, rounds):
             assert acc_gpu >= capacity
     filled = min(acc_ref, capacity)
     assert 0 < filled
+    assert draw.ids.dtype == (torch.int64 if ids_int64 else torch.int32)
     np.testing.assert_array_equal(draw.ids.cpu().numpy()[:filled], ids_ref[:filled])
     np.testing.assert_array_equal(draw.pos.cpu().numpy()[:filled].view(np.uint32), pos_ref[:filled].view(np.uint32))
     draw.finish()
