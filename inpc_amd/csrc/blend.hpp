@@ -128,7 +128,8 @@ struct Stage {
 // on the way out; forward: x = staged instance; backward: x = features . grad, y = d loss / d alpha.
 template <int T>
 struct QuadScratch {
-    uint64_t hits[64][Shape<T>::K];  // per pixel and entry round: lanes whose entry hits the pixel
+    uint64_t hits[Shape<T>::K][64];  // per entry round and pixel: lanes whose entry hits the pixel (round-major:
+                                     // the lanes of an access are a round's, their pixels spread over the banks)
     float2 fragment[256];            // per fragment, pixel by pixel, in depth order
 };
 
@@ -300,36 +301,41 @@ __device__ __forceinline__ void build_fragment_lists(QuadScratch<T>& qs, Stage<T
     constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
     const uint32_t lane = __lane_id();
 #pragma unroll
-    for (int k = 0; k < K; ++k) qs.hits[lane][k] = 0ull;
+    for (int k = 0; k < K; ++k) qs.hits[k][lane] = 0ull;
     wave_sync();
     const unsigned long long bit = 1ull << lane;
 #pragma unroll
     for (int k = 0; k < K; ++k)
 #pragma unroll
         for (int q = 0; q < NF; ++q)
-            if (e.pixel[k][q] != kNoPixel) atomicOr((unsigned long long*)&qs.hits[e.pixel[k][q]][k], bit);
+            if (e.pixel[k][q] != kNoPixel) atomicOr((unsigned long long*)&qs.hits[k][e.pixel[k][q]], bit);
     wave_sync();
+    // where the fragments of entry round k start in this lane's pixel's list: behind those of the rounds before
+    uint32_t round_start[K];
     my_count = 0u;
 #pragma unroll
-    for (int k = 0; k < K; ++k) my_count += (uint32_t)__popcll(qs.hits[lane][k]);
+    for (int k = 0; k < K; ++k) {
+        round_start[k] = my_count;
+        my_count += (uint32_t)__popcll(qs.hits[k][lane]);
+    }
     my_start = wave_exclusive_sum(my_count, n_fragments);
     if (n_fragments == 0u) return;
     const uint64_t below = lanes_below();
 #pragma unroll
-    for (int k = 0; k < K; ++k)
+    for (int k = 0; k < K; ++k) {
+        round_start[k] += my_start;
 #pragma unroll
         for (int q = 0; q < NF; ++q) {
             const bool hit = e.pixel[k][q] != kNoPixel;
             const uint32_t pix = hit ? e.pixel[k][q] : 0u;
-            const uint32_t start = __shfl(my_start, pix, 64);  // every lane takes part in the exchange
+            const uint32_t start = __shfl(round_start[k], pix, 64);  // every lane takes part in the exchange
             if (hit) {
-                uint32_t pos = start + (uint32_t)__popcll(qs.hits[pix][k] & below);
-#pragma unroll
-                for (int kk = 0; kk < k; ++kk) pos += (uint32_t)__popcll(qs.hits[pix][kk]);
+                const uint32_t pos = start + (uint32_t)__popcll(qs.hits[k][pix] & below);
                 qs.fragment[pos] = make_float2(e.alpha[k][q], payload(k, q));
                 if (!WITH_DEPTH) st.frag[e.j[k]][T == 16 ? quad : q] = (uint16_t)((pos << 8) | pix | kPlaced);
             }
         }
+    }
     wave_sync();
 }
 
@@ -370,6 +376,7 @@ __device__ __forceinline__ void start_gather(Gather<C>& g, const uint32_t* __res
     if (at < range.y) slot0 = inst_points[at];
     if (at + TT < range.y) slot1 = inst_points[at + TT];
     if (at + 2u * TT < range.y) g.next_slot = inst_points[at + 2u * TT];
+
     if (at < range.y) {
         const char* record = records + (size_t)slot0 * stride;
         g.h = read_header(record);
@@ -407,11 +414,35 @@ __device__ __forceinline__ void advance_gather(Gather<C>& g, const uint32_t* __r
 }
 
 // ---- ordered records: what the forward blend leaves for the backward blend ------------------------------------------
-// The record of every staged instance once more (header, C fp32 features: 2 + C / 4 words of 16 bytes), where the
-// instance stands in its tile's list. Within a batch the words are stored one after the other, word w of all the
-// batch's instances in a row, so that a wave writes and reads 1 KB runs (a thread that writes its own 64-byte record
-// costs the forward blend 0.11 ms, more than the backward blend gains). The batch that starts at instance `begin`
-// and holds `count` instances occupies words [begin * kWords, (begin + count) * kWords).
+// One record per staged instance (2 + C / 4 words of 16 bytes), where the instance stands in its tile's list, with a
+// header that is the instance's, not the point's: what the forward blend has worked out of the point's record for
+// this tile, so that the backward blend stages an instance with a handful of instructions.
+//   float weight[4]   interpolation weights of the four fragment slots
+//   float opacity
+//   u32   tag         as in the point's record (point index | kRecordMulti | span bits)
+//   u32   pixels      per slot one byte: pixel in the owning wave's grid, kNoPixel: no fragment
+//   u32   row         gradient row of this instance (points that touch several tiles)
+// Within a batch the words are stored one after the other, word w of all the batch's instances in a row, so that a wave
+// writes and reads 1 KB runs (a thread that writes its own 64-byte record costs the forward blend 0.11 ms, more than
+// the backward blend gains). The batch that starts at instance `begin` and holds `count` instances occupies words
+// [begin * kWords, (begin + count) * kWords).
+struct InstanceHeader {
+    float weight[4];
+    float opacity;
+    uint32_t tag, pixels, row;
+    __device__ __forceinline__ bool multi() const { return (tag & kRecordMulti) != 0u; }
+    __device__ __forceinline__ uint32_t point() const { return tag & kRecordIdMask; }
+};
+
+__device__ __forceinline__ void arrive(InstanceHeader& h) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) arrive(h.weight[c]);
+    arrive(h.opacity);
+    arrive(h.tag);
+    arrive(h.pixels);
+    arrive(h.row);
+}
+
 template <int C>
 struct Ordered {
     static constexpr uint32_t kWords = 2u + (uint32_t)C / 4u;
@@ -419,21 +450,30 @@ struct Ordered {
         return (size_t)begin * kWords + (size_t)w * count + threadIdx.x;
     }
     __device__ static __forceinline__ void store(float4* __restrict__ ordered, uint32_t begin, uint32_t count,
-                                                 const Header& h, const float (&f)[C]) {
-        ordered[word(begin, count, 0)] = make_float4(h.wx0, h.wx1, h.wy0, h.wy1);
-        ordered[word(begin, count, 1)] = make_float4(h.opacity, __uint_as_float(h.tag), __uint_as_float(h.cell),
-                                                     __uint_as_float(h.extra));
+                                                 const float (&weight)[4], float opacity, uint32_t tag, uint32_t pixels,
+                                                 uint32_t row, const float (&f)[C]) {
+        ordered[word(begin, count, 0)] = make_float4(weight[0], weight[1], weight[2], weight[3]);
+        ordered[word(begin, count, 1)] = make_float4(opacity, __uint_as_float(tag), __uint_as_float(pixels),
+                                                     __uint_as_float(row));
 #pragma unroll
         for (int q = 0; q < C / 4; ++q)
             ordered[word(begin, count, 2 + q)] = make_float4(f[4 * q], f[4 * q + 1], f[4 * q + 2], f[4 * q + 3]);
     }
     // this thread's instance of the batch that starts at `begin`, if the batch has one for it
     __device__ static __forceinline__ void load(const float4* __restrict__ ordered, uint32_t begin, uint32_t end,
-                                                Header& h, float (&f)[C]) {
+                                                InstanceHeader& h, float (&f)[C]) {
         if (begin >= end) return;
         const uint32_t count = min((uint32_t)blockDim.x, end - begin);
         if (threadIdx.x >= count) return;
-        h = make_header(ordered[word(begin, count, 0)], ordered[word(begin, count, 1)]);
+        const float4 h0 = ordered[word(begin, count, 0)], h1 = ordered[word(begin, count, 1)];
+        h.weight[0] = h0.x;
+        h.weight[1] = h0.y;
+        h.weight[2] = h0.z;
+        h.weight[3] = h0.w;
+        h.opacity = h1.x;
+        h.tag = __float_as_uint(h1.y);
+        h.pixels = __float_as_uint(h1.z);
+        h.row = __float_as_uint(h1.w);
 #pragma unroll
         for (int q = 0; q < C / 4; ++q) {
             const float4 v = ordered[word(begin, count, 2 + q)];
@@ -445,20 +485,27 @@ struct Ordered {
     }
 };
 
+// The ordered record of the batch being staged and the one of the batch after it (requested a batch earlier).
+template <int C>
+struct OrderedAhead {
+    InstanceHeader h, h_next;
+    float f[C], f_next[C];
+};
+
 template <int T, int C>
-__device__ __forceinline__ void start_ordered(Gather<C>& g, const float4* __restrict__ ordered, uint2 range) {
-    g.h = Header{};
-    g.h_next = Header{};
+__device__ __forceinline__ void start_ordered(OrderedAhead<C>& g, const float4* __restrict__ ordered, uint2 range) {
+    g.h = InstanceHeader{};
+    g.h_next = InstanceHeader{};
+    g.h.pixels = g.h_next.pixels = 0xFFFFFFFFu;   // no fragment in any slot
 #pragma unroll
     for (int c = 0; c < C; ++c) g.f[c] = g.f_next[c] = 0.0f;
-    g.next_slot = 0u;
     Ordered<C>::load(ordered, range.x, range.y, g.h, g.f);
     Ordered<C>::load(ordered, range.x + T * T, range.y, g.h_next, g.f_next);
 }
 
 // At the end of the batch that starts at `begin`: takes the next batch's record, requests the one after it.
 template <int T, int C>
-__device__ __forceinline__ void advance_ordered(Gather<C>& g, const float4* __restrict__ ordered, uint32_t begin,
+__device__ __forceinline__ void advance_ordered(OrderedAhead<C>& g, const float4* __restrict__ ordered, uint32_t begin,
                                                 uint32_t end) {
     arrive(g.h_next);
 #pragma unroll
@@ -467,6 +514,27 @@ __device__ __forceinline__ void advance_ordered(Gather<C>& g, const float4* __re
 #pragma unroll
     for (int c = 0; c < C; ++c) g.f[c] = g.f_next[c];
     Ordered<C>::load(ordered, begin + 2u * T * T, end, g.h_next, g.f_next);
+}
+
+// Stage instance `t` (thread t) of the backward blend from its ordered record; see stage_instance.
+template <int T, int C>
+__device__ __forceinline__ void stage_ordered(Stage<T, C, false>& st, bool valid, const InstanceHeader& h,
+                                              const float (&f)[C], float (&weight)[4], uint32_t (&pixel)[4]) {
+    const uint32_t t = threadIdx.x;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        weight[c] = h.weight[c];
+        pixel[c] = (h.pixels >> (8 * c)) & 0xFFu;
+    }
+    if (!valid) return;
+#pragma unroll
+    for (int q4 = 0; q4 < C / 4; ++q4) st.feat[t * (C / 4) + q4] = make_float4(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
+    if (T == 16) {
+        st.alpha[t] = make_float4(h.opacity * weight[0], h.opacity * weight[1], h.opacity * weight[2], h.opacity * weight[3]);
+        st.pixel[t] = h.pixels;
+    }
+    const uint2 nothing_placed = make_uint2(0u, 0u);
+    __builtin_memcpy(st.frag[t], &nothing_placed, 8);
 }
 
 // ---- forward ------------------------------------------------------------------------------------------------------
@@ -602,7 +670,18 @@ __global__ void __launch_bounds__(T* T)
         const Header mine = g.h;
         // the backward pass reads the records of this batch in runs (a gather pulls a 128-byte line per
         // 64-byte record and was 0.13 ms of the backward blend)
-        if (!INFERENCE && ordered_records && valid) Ordered<C>::store(ordered_records, begin, count, g.h, g.f);
+        if (!INFERENCE && ordered_records && valid) {
+            // the gradient row of this instance: the point's first row + the place of this tile among the point's
+            // tiles, row-major (the left / top candidate pixel lies in the tile in front when the point spans two)
+            uint32_t row = 0u;
+            if (g.h.multi()) {
+                const int lx = local_left(g.h.cell & 0xFFFFu, tile_x0), ly = local_left(g.h.cell >> 16, tile_y0);
+                row = g.h.extra + (lx < 0 && tile_x0 > 0 ? 1u : 0u) +
+                      (ly < 0 && tile_y0 > 0 ? ((g.h.tag & kRecordSpanX) ? 2u : 1u) : 0u);
+            }
+            const uint32_t pixels = slot_pixel[0] | (slot_pixel[1] << 8) | (slot_pixel[2] << 16) | (slot_pixel[3] << 24);
+            Ordered<C>::store(ordered_records, begin, count, weight, g.h.opacity, g.h.tag, pixels, row, g.f);
+        }
         advance_gather<T, C, HALF>(g, inst_points, records, stride, begin, range.y);
         // ---- write: thread t owns staged instance t (kernels.cu:291-295): its blending weight is the sum over
         // the fragments the waves placed
@@ -646,13 +725,6 @@ struct SplitRows {
     const uint2* list;
     const uint32_t* count;    // number of list entries
 };
-
-// Which of the (at most 2 x 2) tiles of a point the tile at (tile_x, tile_y) is, counted row-major.
-__device__ __forceinline__ uint32_t tile_rank(const Header& h, uint32_t tile_x, uint32_t tile_y, uint32_t tile_shift) {
-    const int left = (int)(h.cell & 0xFFFFu) - 1, top = (int)(h.cell >> 16) - 1;
-    const uint32_t x0 = (uint32_t)max(left, 0) >> tile_shift, y0 = (uint32_t)max(top, 0) >> tile_shift;
-    return (tile_y - y0) * ((h.tag & kRecordSpanX) ? 2u : 1u) + (tile_x - x0);
-}
 
 // gradient of the point = sum of its rows that were written, in row order (the gradient buffers are zero before). A
 // group of kGroup neighbouring lanes takes one point, lane j the j-th 16-byte word of each feature row (the last lane
@@ -717,13 +789,13 @@ __global__ void __launch_bounds__(T* T)
                      const float4* __restrict__ ordered_records, const uint32_t* __restrict__ tile_end,
                      const float* __restrict__ grad_image, const float* __restrict__ grad_alpha,
                      const float* __restrict__ image, const float* __restrict__ alpha_image, float* grad_view,
-                     float* grad_opacities, SplitRows rows, int W, int H, uint32_t gw, uint32_t tile_shift) {
+                     float* grad_opacities, SplitRows rows, int W, int H, uint32_t gw) {
     constexpr int TT = T * T;
     constexpr int NQ = TT / 64;
     constexpr int K = Shape<T>::K, NF = Shape<T>::NF;
     __shared__ Stage<T, C, false> st;
     __shared__ QuadScratch<T> s_quad[NQ];
-    __shared__ float4 s_grad[NQ][64][C / 4];   // upstream gradient of every wave's pixels (0 outside the image)
+    __shared__ float4 s_grad[NQ][C / 4][64];   // upstream gradient of every wave's pixels (0 outside the image)
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tile = tile_order[blockIdx.x];
@@ -750,7 +822,7 @@ __global__ void __launch_bounds__(T* T)
             if (inside) final_dot = fmaf(v[c], g[c], final_dot);
         }
 #pragma unroll
-        for (int q4 = 0; q4 < C / 4; ++q4) s_grad[wave][lane][q4] = make_float4(g[4 * q4], g[4 * q4 + 1], g[4 * q4 + 2], g[4 * q4 + 3]);
+        for (int q4 = 0; q4 < C / 4; ++q4) s_grad[wave][q4][lane] = make_float4(g[4 * q4], g[4 * q4 + 1], g[4 * q4 + 2], g[4 * q4 + 3]);
         if (inside) common = ga * (1.0f - av);
     }
     const float offset = common - final_dot;
@@ -760,14 +832,14 @@ __global__ void __launch_bounds__(T* T)
     // the records as the forward pass staged them, in the order of the tile's list; only as far as it got
     uint2 range = ranges[tile];
     range.y = min(range.y, tile_end[tile]);
-    Gather<C> g;
+    OrderedAhead<C> g;
     start_ordered<T, C>(g, ordered_records, range);
     for (uint32_t begin = range.x; begin < range.y; begin += TT) {
         const uint32_t count = min((uint32_t)TT, range.y - begin);
         const bool valid = tid < count;
         float weight[4];   // of this thread's staged instance, per fragment slot
         uint32_t slot_pixel[4];
-        stage_instance<T, C, false>(st, valid, g.h, g.f, tile_x0, tile_y0, weight, slot_pixel);
+        stage_ordered<T, C>(st, valid, g.h, g.f, weight, slot_pixel);
         __syncthreads();
 
         // ---- consume: this wave's list
@@ -787,7 +859,7 @@ __global__ void __launch_bounds__(T* T)
                     float d = 0.0f;
 #pragma unroll
                     for (int q4 = 0; q4 < C / 4; ++q4) {
-                        const float4 gr = s_grad[wave][pix][q4];
+                        const float4 gr = s_grad[wave][q4][pix];
                         d = fmaf(feat[q4].x, gr.x, d);
                         d = fmaf(feat[q4].y, gr.y, d);
                         d = fmaf(feat[q4].z, gr.z, d);
@@ -858,7 +930,7 @@ __global__ void __launch_bounds__(T* T)
         }
         const bool all_done = barrier_all_done<T>(s_quad, done);
         // ---- the gather moves on in front of the stores of the write phase (see the forward kernel)
-        const Header mine = g.h;
+        const uint32_t mine_tag = g.h.tag, mine_row = g.h.row;
         advance_ordered<T, C>(g, ordered_records, begin, range.y);
         // ---- write: thread t owns staged instance t: gradient of the point from the fragments the waves placed
         if (valid) {
@@ -880,7 +952,7 @@ __global__ void __launch_bounds__(T* T)
                         const uint32_t pix = field[c] & kPixelMask;
 #pragma unroll
                         for (int q4 = 0; q4 < C / 4; ++q4) {
-                            const float4 gr = s_grad[q][pix][q4];
+                            const float4 gr = s_grad[q][q4][pix];
                             gf[4 * q4] = fmaf(e.x, gr.x, gf[4 * q4]);
                             gf[4 * q4 + 1] = fmaf(e.x, gr.y, gf[4 * q4 + 1]);
                             gf[4 * q4 + 2] = fmaf(e.x, gr.z, gf[4 * q4 + 2]);
@@ -891,13 +963,13 @@ __global__ void __launch_bounds__(T* T)
             if (any_weight || gop != 0.0f) {
                 // a point that straddles tiles gets its gradient from up to four blocks: each writes a row of
                 // its own (summed up by k_grad_reduce); no atomics, and the sum has a fixed order
-                float* dst = grad_view + (size_t)mine.point() * C;
-                float* dst_opacity = grad_opacities + mine.point();
-                if (mine.multi()) {
-                    const size_t row = (size_t)mine.extra + tile_rank(mine, tile % gw, tile / gw, tile_shift);
-                    dst = rows.features + row * C;
-                    dst_opacity = rows.opacities + row;
-                    rows.flags[row] = 1;
+                const uint32_t point = mine_tag & kRecordIdMask;
+                float* dst = grad_view + (size_t)point * C;
+                float* dst_opacity = grad_opacities + point;
+                if (mine_tag & kRecordMulti) {
+                    dst = rows.features + (size_t)mine_row * C;
+                    dst_opacity = rows.opacities + mine_row;
+                    rows.flags[mine_row] = 1;
                 }
 #pragma unroll
                 for (int q4 = 0; q4 < C / 4; ++q4)

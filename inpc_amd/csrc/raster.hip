@@ -1031,7 +1031,7 @@ int launch_blend_backward(const Layout& L, const float* grad_image, const float*
                 at<uint2>(ws, L.pub.tile_ranges), (const uint32_t*)at<uint32_t>(ws, L.tile_order),
                 (const float4*)at<float4>(ws, L.ordered_records), (const uint32_t*)at<uint32_t>(ws, L.tile_end), grad_image,
                 grad_alpha, image, alpha, grad_view,
-                grad_opacities, rows, L.geo.W, L.geo.H, L.geo.gw, L.geo.tile_shift);
+                grad_opacities, rows, L.geo.W, L.geo.H, L.geo.gw);
     INPC_LAUNCH("raster_grad_reduce", blend::k_grad_reduce<C>, dim3(std::min(div_up(L.geo.n, 256u), 4096u)), dim3(256),
                 stream, rows, grad_view, grad_opacities);
     return INPC_OK;
