@@ -376,6 +376,109 @@ def main() -> int:
     except Exception as exc:  # the figure is optional
         print(f"bench.py: reference-shaped step not measured: {exc}", file=sys.stderr)
 
+    # BASELINE configuration 0, the reference's CPU-runnable case: forward only, 65,536 uniform points in the unit
+    # cube, 4 fp32 channels ~U(0,1), opacity ~U(0.05,0.95), 256x256, f = 300, distance 3, 16x16 tiles, seed 0: the GPU
+    # forward through the C ABI and the CPU oracle's forward on the same arrays
+    config0 = None
+    try:
+        if args.no_extras:
+            raise RuntimeError("skipped (--no-extras)")
+        n0 = 65_536
+        hv0 = synthetic.camera_on_z(256, 256, 300.0, 3.0)
+        view0 = hv0.to_view(device)
+        pos0_h = synthetic.cube_points(n0, 1.0, 0)
+        feats0_h, opac0_h = synthetic.point_attributes(n0, 4, "uniform", 0)
+        pos0, feats0, opac0 = (torch.from_numpy(np.ascontiguousarray(a)).to(device) for a in (pos0_h, feats0_h, opac0_h))
+        cfg0 = _lib.RasterConfig(n0, 16, 4, _lib.FEAT_DIRECT_F32, 0, _lib.make_camera(hv0.camera), 4 * n0)
+        layout0 = _lib.RasterLayout()
+        _lib.check(lib.inpc_raster_layout_query(C.byref(cfg0), C.byref(layout0)), "layout")
+        ws0 = torch.empty(layout0.total_bytes, dtype=torch.uint8, device=device)
+        image0 = torch.empty((4, 256, 256), dtype=torch.float32, device=device)
+        alpha0 = torch.empty((1, 256, 256), dtype=torch.float32, device=device)
+        bw0 = torch.empty(n0, dtype=torch.float32, device=device)
+        w2c0, camp0 = view0.w2c.contiguous(), view0.position.contiguous()
+
+        def forward0():
+            _lib.check(lib.inpc_raster_forward(C.byref(cfg0), _lib.ptr(pos0), _lib.ptr(feats0), _lib.ptr(opac0),
+                                               _lib.ptr(w2c0), _lib.ptr(camp0), _lib.ptr(image0), _lib.ptr(alpha0),
+                                               _lib.ptr(bw0), None, _lib.ptr(ws0), layout0.total_bytes, stream),
+                       "inpc_raster_forward")
+
+        forward0()
+        gpu0_ms = time_calls(forward0, 10 * args.steps)
+        config0 = {"workload": "65,536 pts uniform in the unit cube, 4 fp32 channels, 256x256, f=300, distance 3, "
+                               "16x16 tiles, forward only",
+                   "gpu_forward_ms": round(gpu0_ms, 4), "gpu_Mpoints_per_s": round(n0 / (gpu0_ms * 1e-3) / 1e6, 1)}
+        if not args.no_cpu_baseline:
+            from oracle import oracle as O
+
+            c0 = hv0.camera
+            ocfg0 = O.make_config(n0, O.make_camera(c0.width, c0.height, c0.focal_x, c0.focal_y, c0.center_x, c0.center_y,
+                                                    c0.near_plane, c0.far_plane), 16, 4, O.FEAT_DIRECT_F32)
+            ref0 = O.raster_forward(ocfg0, pos0_h, feats0_h, opac0_h, hv0.w2c)   # warm-up, and the images to compare
+            config0["max_abs_image_difference_to_cpu"] = float(np.abs(image0.cpu().numpy() - ref0["image"]).max())
+            threads0 = O.num_threads()
+            for label, threads in (("cpu_forward_ms", threads0), ("cpu_single_thread_forward_ms", 1)):
+                O.set_num_threads(threads)
+                reps, spent = 0, 0.0
+                while spent < 1.5 and reps < 200:
+                    t = O.now()
+                    O.raster_forward(ocfg0, pos0_h, feats0_h, opac0_h, hv0.w2c)
+                    spent += O.now() - t
+                    reps += 1
+                config0[label] = round(spent * 1e3 / reps, 3)
+            O.set_num_threads(threads0)
+            config0["cpu_cores"] = threads0
+        del ws0, image0, alpha0, bw0
+    except Exception as exc:  # the figure is optional
+        print(f"bench.py: configuration 0 not measured: {exc}", file=sys.stderr)
+
+    # The reference's default inference frame: four times (expected-count samples for 8,388,352 requested points,
+    # one sample per count, then the inference rasterizer on raw (N,37) fp16 appearance output), images added up.
+    # The appearance network between the two is not part of this path: its output is random numbers made beforehand.
+    inference_frame = None
+    try:
+        if args.no_extras:
+            raise RuntimeError("skipped (--no-extras)")
+        from inpc_amd import INPCRasterizer
+
+        n_req, n_multi = 8_388_352, 4
+        frame_sampler = ProbabilityFieldSampler(seed=0)
+        probe = frame_sampler.generate_expected_samples(centers, levels, weights, view, n_req, 1, oct.initial_size)
+        n_created = int(probe.shape[0])
+        raw = (torch.randn((n_created, 37), generator=gen, device=device) * 0.5).half()
+        frame_rasterizer = INPCRasterizer()
+        del probe
+
+        def frame():
+            acc = None
+            for _ in range(n_multi):
+                p = frame_sampler.generate_expected_samples(centers, levels, weights, view, n_req, 1, oct.initial_size)
+                img, dep, alp = frame_rasterizer.render(view, 0, p, raw[: p.shape[0]], 1.0, 3.0)
+                if acc is None:
+                    acc = [img, dep, alp]
+                else:
+                    acc[0] += img
+                    acc[1] += dep
+                    acc[2] += alp
+            return acc
+
+        frame()
+        frame_ms = time_calls(frame, max(args.steps // 4, 2))
+        with _lib.KernelTimer() as frame_timer:
+            frame()
+        frame_kernels = {}
+        for name, ms in frame_timer.records:
+            frame_kernels[name] = frame_kernels.get(name, 0.0) + ms
+        inference_frame = {
+            "workload": f"{n_multi} x (generate_expected_samples({n_req}, 1) -> {n_created} points, render on raw (N,37) "
+                        f"fp16, bilinear footprint, 16x16 tiles) @{W}x{H}",
+            "ms_per_frame": round(frame_ms, 3), "Mpoints_per_s": round(n_multi * n_created / (frame_ms * 1e-3) / 1e6, 1),
+            "kernel_ms_per_frame": {k: round(v, 4) for k, v in sorted(frame_kernels.items(), key=lambda kv: -kv[1])}}
+        del raw
+    except Exception as exc:  # the figure is optional
+        print(f"bench.py: inference frame not measured: {exc}", file=sys.stderr)
+
     # ---- per-kernel durations: HIP events around every launch, on the launch stream, same steps ----------
     with _lib.KernelTimer() as timer:
         for _ in range(args.steps):
@@ -461,10 +564,10 @@ def main() -> int:
         opac4 = torch.sigmoid(torch.randn(n4, generator=gen, device=device, dtype=torch.float32))
         config4 = {"workload": "33,554,432 pts @2473x1643, 16 channels stored fp16, inference forward",
                    "training_draw_ms": round(draw4_ms, 3)}
+        from inpc_amd import rasterize_points
+
         for label, mode, tile4, kw in (("bilinear", 0, 16, {}),
                                        ("gaussian", 1, 8, dict(sigma_world=0.002, sigma_cutoff=3.0))):
-            from inpc_amd import rasterize_points
-
             def infer():
                 rasterize_points(view4, pos4, feats4, opac4, tile=tile4, inference=True, mode=mode, **kw)
 
@@ -472,6 +575,69 @@ def main() -> int:
             ms = time_calls(infer, 5)
             config4[f"{label}_forward_ms"] = round(ms, 3)
             config4[f"{label}_Mpoints_per_s"] = round(n4 / (ms * 1e-3) / 1e6, 1)
+        # the bilinear forward once more through the C ABI: its counts, per-kernel durations (HIP events on the launch
+        # stream) and the share of the HBM roofline of the frame and of its largest kernel. Algorithmic bytes as for
+        # the training step, with 2 bytes per stored feature.
+        try:
+            cfg4 = _lib.RasterConfig(n4, 16, 16, _lib.FEAT_DIRECT_F16, _lib.RASTER_INFERENCE, _lib.make_camera(hv4.camera), 0)
+            layout4 = _lib.RasterLayout()
+            _lib.check(lib.inpc_raster_layout_query(C.byref(cfg4), C.byref(layout4)), "layout")
+            ws4 = torch.empty(layout4.total_bytes, dtype=torch.uint8, device=device)
+            image4 = torch.empty((16, H4, W4), dtype=torch.float32, device=device)
+            alpha4 = torch.empty((1, H4, W4), dtype=torch.float32, device=device)
+            depth4 = torch.empty((1, H4, W4), dtype=torch.float32, device=device)
+            w2c4, camp4 = view4.w2c.contiguous(), view4.position.contiguous()
+
+            def forward4():
+                _lib.check(lib.inpc_raster_forward(C.byref(cfg4), _lib.ptr(pos4), _lib.ptr(feats4), _lib.ptr(opac4),
+                                                   _lib.ptr(w2c4), _lib.ptr(camp4), _lib.ptr(image4), _lib.ptr(alpha4), None,
+                                                   _lib.ptr(depth4), _lib.ptr(ws4), layout4.total_bytes, stream),
+                           "inpc_raster_forward")
+
+            forward4()
+            counters4 = (C.c_uint32 * 3)()
+            _lib.check(lib.inpc_raster_read_counters(C.byref(cfg4), _lib.ptr(ws4), C.byref(counters4), stream), "counters")
+            v4, i4 = int(counters4[0]), int(counters4[1])
+            abi_ms = time_calls(forward4, 5)
+            with _lib.KernelTimer() as timer4:
+                for _ in range(3):
+                    forward4()
+            k4 = {}
+            for name, ms in timer4.records:
+                tot, cnt = k4.get(name, (0.0, 0))
+                k4[name] = (tot + ms, cnt + 1)
+            F4, R4, px4 = 2 * 16, 8 + 4 + 2 * 16, H4 * W4
+            sort_bytes = 2 + 12 * ((layout4.end_bit + 7) // 8) + 2
+            frame_bytes = float(n4 * (16 + F4) + v4 * (R4 + 8 + 68 + 20 + 16) + i4 * (6 + sort_bytes + 4 + R4)
+                                + px4 * 4 * (16 + 2))
+            per_kernel_bytes = {
+                "raster_bin_count": v4 * 20.0, "raster_records": float(n4 * (16 + F4) + v4 * R4),
+                "raster_bin_fill": float(v4 * (8 + 16) + i4 * 6), "raster_tile_sort": float(v4 * 68 + i4 * sort_bytes),
+                "raster_blend_inference": float(i4 * (4 + R4) + px4 * 4 * (16 + 2)),
+            }
+            rows4 = []
+            for name, (tot, cnt) in sorted(k4.items(), key=lambda kv: -kv[1][0]):
+                launches = cnt / 3
+                avg = tot / cnt
+                alg = per_kernel_bytes.get(name, 0.0) / launches
+                rows4.append({"kernel": name, "launches_per_frame": launches, "avg_ms": round(avg, 4),
+                              "ms_per_frame": round(tot / 3, 4),
+                              "algorithmic_GBps": round(alg / (avg * 1e-3) / 1e9, 1) if alg > 0 and avg > 0 else None})
+            top = rows4[0]
+            top_alg = per_kernel_bytes.get(top["kernel"], 0.0) / top["launches_per_frame"]
+            top_gbps = top_alg / (top["avg_ms"] * 1e-3) / 1e9
+            config4["bilinear_abi"] = {
+                "forward_ms": round(abi_ms, 3), "n_visible": v4, "n_instances": i4, "n_tiles": int(layout4.n_tiles),
+                "frame_algorithmic_GB": round(frame_bytes / 1e9, 3),
+                "frame_hbm_frac": round(frame_bytes / (abi_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "roofline": {"bound": "hbm", "kernel": top["kernel"], "achieved": round(top_gbps, 1),
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(top_gbps / HBM_PEAK_GBS, 4),
+                             "algorithmic_bytes_per_launch": top_alg, "avg_launch_ms": top["avg_ms"],
+                             "traffic": measured_traffic(top["kernel"], "config4")},
+                "kernels": rows4}
+            del ws4, image4, alpha4, depth4
+        except Exception as exc:  # the figure is optional
+            print(f"bench.py: config-4 per-kernel figures not measured: {exc}", file=sys.stderr)
 
     # the sampler (training draw of the same n points): 32 B per leaf (20 in, 4 out, 8 scan) and 32 B per candidate
     # (16 B of leaf data gathered, 12 B position + 4 B index written); the CDF probes are cache traffic and not counted
@@ -514,6 +680,8 @@ def main() -> int:
             "other_tile_size": other_tile,
             "gaussian_footprint": gaussian,
             "sh36_autograd_step": reference_shape,
+            "config0": config0,
+            "inference_frame": inference_frame,
             "config4_inference": config4,
             "step_algorithmic_GB": round((fwd_bytes + bwd_bytes) / 1e9, 3),
             "step_algorithmic_GBps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBS, 4),

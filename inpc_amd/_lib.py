@@ -169,6 +169,23 @@ SIGNATURES = {
 _lib = None
 
 
+# how the library gets built: in the tree, or into an installed package (setup.py runs the same build)
+BUILD_COMMAND = ["python", "-m", "inpc_amd.build"]
+INSTALL_COMMAND = ["pip", "install", str(LIB_PATH.parent.parent), "--no-build-isolation"]
+
+
+class ExtensionError(ImportError):
+    """The native library is missing. Carries the package name and the command that builds it, like the
+    Framework.ExtensionError the reference raises for its extension module (INPCCudaBackend/__init__.py:7-23)."""
+
+    def __init__(self, name: str, install_command: list[str], detail: str = ""):
+        self.name = name
+        self.install_command = install_command
+        super().__init__(f"extension '{name}' is not built{detail}; build it with `{' '.join(BUILD_COMMAND)}` "
+                         f"(hipcc, gfx950) or install it with `{' '.join(install_command)}`. "
+                         "inpc_amd has no fallback path.")
+
+
 class BackendError(RuntimeError):
     """A call into libinpc_hip.so failed (the counterpart of the RuntimeError pybind11 raises for
     the reference's C++ exceptions)."""
@@ -178,9 +195,7 @@ def lib() -> C.CDLL:
     global _lib
     if _lib is None:
         if not LIB_PATH.exists():
-            raise ImportError(
-                f"{LIB_PATH} is missing: build it with `python -m inpc_amd.build` (hipcc, gfx950). "
-                "inpc_amd has no fallback path.")
+            raise ExtensionError("inpc_amd", INSTALL_COMMAND, f": {LIB_PATH} is missing")
         handle = C.CDLL(str(LIB_PATH))
         for name, (restype, argtypes) in SIGNATURES.items():
             fn = getattr(handle, name)  # AttributeError if the symbol is not exported

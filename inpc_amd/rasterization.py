@@ -73,11 +73,14 @@ def _config(settings: RasterizerSettings, n_points: int, tile: int, channels: in
                              _lib.RASTER_INFERENCE if inference else 0, settings.camera(), int(max_instances))
 
 
-# Up to this many points the bilinear workspace is sized for four instances per point, which no input can exceed;
-# beyond it the library's default capacity (what evenly spread points need, with a margin) is used and the
-# instance count is read back after the forward pass, as the reference reads it back to size its buffers
-# (B/rasterization/src/bilinear/forward.cu:86-89).
-_ALWAYS_FITS_POINTS = 1 << 20
+# The bilinear workspace is sized for four instances per point, which no input can exceed, so that no count has to
+# come back to the host after the forward pass (the reference reads its instance count back on every call to size
+# its buffers, B/rasterization/src/bilinear/forward.cu:86-89): up to this many points and this many bytes (4.5 GB for
+# 8,388,608 points with a backward pass: room is not what a 288 GB device lacks, and memory that holds no instance
+# is never touched). Beyond either limit the library's default capacity (what evenly spread points need, with a
+# margin) is used, the counters are read back, and the call is repeated with room for everything if they say so.
+_ALWAYS_FITS_POINTS = 1 << 26
+_ALWAYS_FITS_BYTES = 48 << 30
 
 
 def query_layout(cfg: _lib.RasterConfig) -> _lib.RasterLayout:
@@ -199,6 +202,9 @@ def _forward_native(settings: RasterizerSettings, positions, features, opacities
     lib = _lib.lib()
     everything = max(4 * n, 1)
     capacity = everything if n <= _ALWAYS_FITS_POINTS else 0
+    if capacity and query_layout(_config(settings, n, tile, out_channels, feature_mode, inference,
+                                         capacity)).total_bytes > _ALWAYS_FITS_BYTES:
+        capacity = 0
     for _ in range(2):
         cfg = _config(settings, n, tile, out_channels, feature_mode, inference, capacity)
         layout = query_layout(cfg)

@@ -229,8 +229,12 @@ def test_second_stream_policy():
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libinpc_hip.so")
-    with pytest.raises(ImportError, match="no fallback"):
+    with pytest.raises(ImportError, match="no fallback") as caught:
         _lib.lib()
+    # the error names the package and the commands that build it, like the reference's ExtensionError
+    assert isinstance(caught.value, _lib.ExtensionError) and caught.value.name == "inpc_amd"
+    assert caught.value.install_command[:2] == ["pip", "install"] and "--no-build-isolation" in caught.value.install_command
+    assert "python -m inpc_amd.build" in str(caught.value)
 
 
 def test_product_does_not_import_the_oracle():
