@@ -179,11 +179,10 @@ class ExtensionError(ImportError):
     Framework.ExtensionError the reference raises for its extension module (INPCCudaBackend/__init__.py:7-23)."""
 
     def __init__(self, name: str, install_command: list[str], detail: str = ""):
-        self.name = name
-        self.install_command = install_command
         super().__init__(f"extension '{name}' is not built{detail}; build it with `{' '.join(BUILD_COMMAND)}` "
                          f"(hipcc, gfx950) or install it with `{' '.join(install_command)}`. "
-                         "inpc_amd has no fallback path.")
+                         "inpc_amd has no fallback path.", name=name)
+        self.install_command = install_command
 
 
 class BackendError(RuntimeError):
