@@ -12,7 +12,7 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libinpc_hip.so"
 SOURCES = ["runtime.hip", "sampler.hip", "raster.hip", "field.hip", "misc.hip"]
-HEADERS = ["common.hpp", "blend.hpp", "tilesort.hpp", "gaussian.hpp"]
+HEADERS = ["common.hpp", "geometry.hpp", "blend.hpp", "tilesort.hpp", "gaussian.hpp"]
 
 # -ffp-contract=off: tile bounds, depth keys, leaf picks and cull decisions must be bit-identical to
 #   a CPU evaluation of the same expressions, so nothing may be fused behind the source's back.

@@ -107,11 +107,6 @@ struct Shape {
     static constexpr int K = T == 16 ? 4 : 1;
 };
 
-// Fragment field of a staged instance (16 bits per slot), 0 until the slot's wave places the fragment in its
-// list: bits 0-5 the pixel in the owning wave's grid (row * 8 + column), bit 7: placed, bits 8-15: where.
-constexpr uint32_t kPixelMask = 63u, kPlaced = 0x80u;
-constexpr uint32_t kNoPixel = 0xFFu;
-
 // Per-block staging area of one batch.
 template <int T, int C, bool WITH_DEPTH>
 struct Stage {
@@ -149,18 +144,6 @@ __device__ __forceinline__ bool barrier_all_done(QuadScratch<T>* s_quad, bool do
     return all;
 }
 
-// The record header as the kernels use it.
-struct Header {
-    float wx0, wx1, wy0, wy1;   // weights of the candidate columns Lx, Lx + 1 and rows Ly, Ly + 1
-    float opacity;
-    uint32_t tag;     // point index | kRecordMulti | span bits (kept as the raw word until the write phase: a
-                      // flag derived at the load would make the gather wait for its own first reply)
-    uint32_t cell;    // (Lx + 1) | (Ly + 1) << 16
-    uint32_t extra;   // first gradient row (training, points that touch several tiles) or depth bits (inference)
-    __device__ __forceinline__ bool multi() const { return (tag & kRecordMulti) != 0u; }
-    __device__ __forceinline__ uint32_t point() const { return tag & kRecordIdMask; }
-};
-
 // Makes the value available here: the wait for an outstanding load that produces it lands at this point and not
 // at a later first use.
 __device__ __forceinline__ void arrive(float& v) { asm volatile("" : "+v"(v)); }
@@ -177,51 +160,8 @@ __device__ __forceinline__ void arrive(Header& h) {
     arrive(h.extra);
 }
 
-__device__ __forceinline__ Header make_header(const float4 h0, const float4 h1) {
-    Header h;
-    h.wx0 = h0.x;
-    h.wx1 = h0.y;
-    h.wy0 = h0.z;
-    h.wy1 = h0.w;
-    h.opacity = h1.x;
-    h.tag = __float_as_uint(h1.y);
-    h.cell = __float_as_uint(h1.z);
-    h.extra = __float_as_uint(h1.w);
-    return h;
-}
-
 __device__ __forceinline__ Header read_header(const char* __restrict__ record) {
     return make_header(((const float4*)record)[0], ((const float4*)record)[1]);
-}
-
-// Tile-local index of the left / top candidate pixel of a record.
-__device__ __forceinline__ int local_left(uint32_t cell_half, int tile_origin) { return (int)cell_half - 1 - tile_origin; }
-
-// The candidate (0: L, 1: L + 1) of one axis whose tile-local index has the parity `odd` (tiles start at even pixels).
-__device__ __forceinline__ int candidate_of_parity(int left, uint32_t odd) { return (left ^ (int)odd) & 1; }
-
-// The four fragment slots of a point in a tile. 16x16 tiles: slot = parity class (x parity | y parity << 1) of the
-// candidate pixel, i.e. the wave that owns it; 8x8 tiles: slot = candidate (kx | ky << 1). Per slot: the
-// interpolation weight (whether the fragment exists or not) and the pixel in the owning wave's 8 x 8 grid, kNoPixel
-// when the candidate lies outside the tile or a pixel centre is 1 or more away (B/rasterization/src/bilinear/
-// kernels.cu:284-285: weight 0).
-template <int T>
-__device__ __forceinline__ void fragment_slots(const Header& h, int tile_x0, int tile_y0, float (&weight)[4],
-                                               uint32_t (&pixel)[4]) {
-    // plain scalars: a choice between two members of the record would otherwise be made through memory
-    const float wx0 = h.wx0, wx1 = h.wx1, wy0 = h.wy0, wy1 = h.wy1;
-    const int lx = local_left(h.cell & 0xFFFFu, tile_x0), ly = local_left(h.cell >> 16, tile_y0);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const int kx = T == 16 ? candidate_of_parity(lx, c & 1) : (c & 1);
-        const int ky = T == 16 ? candidate_of_parity(ly, c >> 1) : (c >> 1);
-        const int cx = lx + kx, cy = ly + ky;
-        const float wx = kx ? wx1 : wx0, wy = ky ? wy1 : wy0;
-        weight[c] = wx * wy;
-        const bool hit = (uint32_t)(cx | cy) < (uint32_t)T && weight[c] > 0.0f;
-        const uint32_t pix = T == 16 ? (uint32_t)((cy >> 1) * 8 + (cx >> 1)) : (uint32_t)(cy * 8 + cx);
-        pixel[c] = hit ? (pix & kPixelMask) : kNoPixel;
-    }
 }
 
 // Stage instance `t` (thread t): features, and per fragment slot the blend's alpha and the pixel, so that the waves
@@ -671,13 +611,10 @@ __global__ void __launch_bounds__(T* T)
         // the backward pass reads the records of this batch in runs (a gather pulls a 128-byte line per
         // 64-byte record and was 0.13 ms of the backward blend)
         if (!INFERENCE && ordered_records && valid) {
-            // the gradient row of this instance: the point's first row + the place of this tile among the point's
-            // tiles, row-major (the left / top candidate pixel lies in the tile in front when the point spans two)
             uint32_t row = 0u;
             if (g.h.multi()) {
                 const int lx = local_left(g.h.cell & 0xFFFFu, tile_x0), ly = local_left(g.h.cell >> 16, tile_y0);
-                row = g.h.extra + (lx < 0 && tile_x0 > 0 ? 1u : 0u) +
-                      (ly < 0 && tile_y0 > 0 ? ((g.h.tag & kRecordSpanX) ? 2u : 1u) : 0u);
+                row = instance_row(g.h.extra, g.h.tag, lx, ly, tile_x0, tile_y0);
             }
             const uint32_t pixels = slot_pixel[0] | (slot_pixel[1] << 8) | (slot_pixel[2] << 16) | (slot_pixel[3] << 24);
             Ordered<C>::store(ordered_records, begin, count, weight, g.h.opacity, g.h.tag, pixels, row, g.f);

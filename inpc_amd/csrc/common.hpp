@@ -84,6 +84,21 @@ int resident_blocks(const void* kernel, int threads, uint32_t& blocks);
 // ------------------------------------------------------------------------------------------------
 constexpr int kWave = 64;
 
+// Plain per-thread arithmetic that the tests also run on the host (geometry.hpp, the generators below).
+#define INPC_HD __host__ __device__ __forceinline__
+
+INPC_HD uint32_t float_bits_of(float f) { return __builtin_bit_cast(uint32_t, f); }
+INPC_HD float float_of_bits(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// Clamp to [0, 1] (the device's saturate; finite input on either side).
+INPC_HD float saturate01(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __saturatef(v);
+#else
+    return v < 0.0f ? 0.0f : (v > 1.0f ? 1.0f : v);
+#endif
+}
+
 // Orders the LDS traffic of one wave: everything issued before is visible to every lane after.
 __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -100,7 +115,7 @@ __device__ __forceinline__ uint32_t mask_rank(uint64_t mask) {
 
 // One row of the affine world-to-camera transform, evaluated left to right without fused
 // multiply-add (this translation unit is compiled with -ffp-contract=off).
-__device__ __forceinline__ float affine_row(const float4 r, float x, float y, float z) {
+INPC_HD float affine_row(const float4 r, float x, float y, float z) {
     return ((r.x * x + r.y * y) + r.z * z) + r.w;
 }
 

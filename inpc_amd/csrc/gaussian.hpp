@@ -32,24 +32,6 @@ constexpr uint32_t kNoKey = 0xFFFFFFFFu;            // depth key of a point that
 
 inline uint32_t record_stride(int channels) { return (uint32_t)align_up(32 + (size_t)channels * 4, 32); }
 
-// exp(x) for x <= 0 by one fixed sequence of fp32 operations (the reference calls expf / __expf, kernels.cu:451,
-// 548,634): n = rint(x log2 e), r = x - n ln 2 in two parts, a degree-7 polynomial (Cephes' expf coefficients),
-// scaling by 2^n. Within one ulp of exp on [-87, 0], 0 below; a CPU evaluates the same sequence to the same bits,
-// so the cut at the footprint's threshold falls on the same pixels.
-__device__ __forceinline__ float footprint_exp(float x) {
-    if (!(x >= -87.0f)) return 0.0f;
-    const float n = __builtin_rintf(x * 1.44269504088896341f);
-    const float r = (x - n * 0.693359375f) - n * -2.12194440e-4f;
-    float p = 1.9875691500e-4f;
-    p = p * r + 1.3981999507e-3f;
-    p = p * r + 8.3334519073e-3f;
-    p = p * r + 4.1665795894e-2f;
-    p = p * r + 1.6666665459e-1f;
-    p = p * r + 5.0000001201e-1f;
-    const float y = (p * (r * r) + r) + 1.0f;
-    return ldexpf(y, (int)n);
-}
-
 struct Params {
     float variance;    // world-space variance of a point without a scale of its own
     float cutoff;      // the tile bounds reach cutoff * sigma - 0.5 pixels
@@ -345,17 +327,6 @@ __global__ void __launch_bounds__(THREADS)
 // has nothing to hand back to the instance and lets every pixel walk over such instances on its own.
 constexpr int kSlots = 9;
 constexpr int kSlotStride = kSlots;   // odd: rows of neighbouring instances spread over the LDS banks
-
-// Footprint value of a staged instance at the pixel centre (kernels.cu:447-452); false when the pixel is skipped.
-// Without branches, so that the values of several instances are computed side by side.
-__device__ __forceinline__ bool footprint_value(const float4 h0, const float4 h1, float cx, float cy, float threshold,
-                                                float& G) {
-    const float dx = h0.x - cx, dy = h0.y - cy;
-    const float exponent = -0.5f * (h0.w * dx * dx + h1.y * dy * dy) - h1.x * dx * dy;
-    const bool positive = exponent > 0.0f;
-    G = footprint_exp(positive ? 0.0f : exponent);   // a NaN exponent stays NaN and gives 0: skipped, as in the reference
-    return !positive && !(G < threshold);
-}
 
 // A staged instance: header words, features, and the pixel box (tile-local, conservative) its footprint can reach.
 template <int T, int C>

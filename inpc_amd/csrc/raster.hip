@@ -52,40 +52,12 @@ enum Counter : int {
     kCntWords = 16
 };
 
-// tile info word of a projected point: first tile id, spans, valid
-constexpr uint32_t kInfoValid = 1u << 18;
-__device__ __forceinline__ uint32_t info_tile0(uint32_t info) { return info & 0xFFFFu; }
-__device__ __forceinline__ uint32_t info_nx(uint32_t info) { return ((info >> 16) & 1u) + 1u; }
-__device__ __forceinline__ uint32_t info_ny(uint32_t info) { return ((info >> 17) & 1u) + 1u; }
+#include "geometry.hpp"
 
-// Blend record of a drawn point, at the point's index in the record array: a 32-byte header followed by the view
-// features, padded to a multiple of 32 bytes (64 bytes for every configuration but 16 fp32 channels).
-//   header: float wx0, wx1, wy0, wy1   interpolation weights of the two candidate pixel columns Lx, Lx + 1 and rows
-//                                      Ly, Ly + 1 (L = floor(s - 0.5)); 0 where the pixel centre is 1 or more away
-//                                      (kernels.cu:284-287)
-//           float opacity
-//           u32   point index | kRecordMulti when the point touches several tiles | span bits
-//           u32   (Lx + 1) | (Ly + 1) << 16
-//           u32   training: first gradient row of a point that touches several tiles; inference: depth
-constexpr uint32_t kRecordHeader = 32;
-constexpr uint32_t kRecordIdMask = (1u << 28) - 1u;
-constexpr uint32_t kRecordMulti = 1u << 28, kRecordSpanX = 1u << 29;   // bit 30: two tiles in y
 inline uint32_t record_stride(int channels, bool half_features) {
     return (uint32_t)align_up(kRecordHeader + (size_t)channels * (half_features ? 2 : 4), 32);
 }
 
-struct Geometry {
-    uint32_t n;
-    int W, H;
-    uint32_t gw, gh, n_tiles;
-    Camera cam;
-    uint32_t key_bias;      // depth key = float bits - key_bias
-    uint32_t stride;        // record stride in bytes
-    uint32_t capacity;      // instances the buffers hold
-    uint32_t row_capacity;  // gradient rows (instances of points that touch several tiles)
-    uint32_t tile_shift;    // log2 of the tile size
-    uint32_t n_chunks;      // contiguous chunks the points are cut into for binning (one block each)
-};
 
 // ---- SH degree 2 (sh_utils.cuh:6-23) ---------------------------------------------------------------------
 struct ShBasis {
@@ -140,66 +112,6 @@ __device__ __forceinline__ float4 sh_to_view_aligned(const ShBasis& s, const __h
     return make_float4(acc[0], acc[1], acc[2], acc[3]);
 }
 
-// ---- projection (kernels.cu:40-64) ---------------------------------------------------------------------------
-struct Projected {
-    float sx, sy, depth;
-    uint32_t info;     // 0 when the point is not drawn
-    uint32_t touched;  // number of tiles
-};
-
-struct ViewRows {
-    float4 r1, r2, r3;
-};
-
-__device__ __forceinline__ ViewRows load_view_rows(const float* __restrict__ w2c) {
-    ViewRows m;
-    m.r1 = make_float4(w2c[0], w2c[1], w2c[2], w2c[3]);
-    m.r2 = make_float4(w2c[4], w2c[5], w2c[6], w2c[7]);
-    m.r3 = make_float4(w2c[8], w2c[9], w2c[10], w2c[11]);
-    return m;
-}
-
-template <int T>
-__device__ __forceinline__ Projected project_point(const ViewRows& m, const Geometry& g, float px, float py, float pz) {
-    Projected o;
-    o.sx = 0.0f;
-    o.sy = 0.0f;
-    o.info = 0u;
-    o.touched = 0u;
-    o.depth = affine_row(m.r3, px, py, pz);
-    if (o.depth < g.cam.near_plane || o.depth > g.cam.far_plane) return o;
-    const float fT = (float)T, fgw = (float)g.gw, fgh = (float)g.gh;
-    const float x = affine_row(m.r1, px, py, pz) / o.depth;
-    const float y = affine_row(m.r2, px, py, pz) / o.depth;
-    o.sx = x * g.cam.fx + g.cam.cx;
-    o.sy = y * g.cam.fy + g.cam.cy;
-    const uint32_t x0 = (uint32_t)fminf(fgw, fmaxf(0.0f, floorf((o.sx - 0.5f) / fT)));
-    const uint32_t x1 = (uint32_t)fminf(fgw, fmaxf(0.0f, ceilf((o.sx + 0.5f) / fT)));
-    const uint32_t y0 = (uint32_t)fminf(fgh, fmaxf(0.0f, floorf((o.sy - 0.5f) / fT)));
-    const uint32_t y1 = (uint32_t)fminf(fgh, fmaxf(0.0f, ceilf((o.sy + 0.5f) / fT)));
-    o.touched = (x1 - x0) * (y1 - y0);
-    if (o.touched != 0u) o.info = (y0 * g.gw + x0) | ((x1 - x0 - 1u) << 16) | ((y1 - y0 - 1u) << 17) | kInfoValid;
-    return o;
-}
-
-// The two pixels of one axis that can lie closer than 1 to screen coordinate s: L = floor(s - 0.5) and L + 1.
-// Their interpolation weights as the reference's blend computes them per pixel (kernels.cu:284-287):
-// d = |s - (pixel + 0.5)|, skipped when d >= 1 (weight 0 here), else saturate(1 - d).
-struct AxisWeights {
-    int left;         // L, clamped to [-1, 65534]
-    float w0, w1;
-};
-
-__device__ __forceinline__ AxisWeights axis_weights(float s) {
-    AxisWeights a;
-    a.left = (int)fminf(fmaxf(floorf(s - 0.5f), -1.0f), 65534.0f);
-    const float d0 = fabsf(s - ((float)a.left + 0.5f));
-    const float d1 = fabsf(s - ((float)(a.left + 1) + 0.5f));
-    a.w0 = !(d0 >= 1.0f) ? __saturatef(1.0f - d0) : 0.0f;
-    a.w1 = !(d1 >= 1.0f) ? __saturatef(1.0f - d1) : 0.0f;
-    return a;
-}
-
 // ---- instance bins ----------------------------------------------------------------------------------------------
 // The points are cut into kBinBlocks contiguous chunks, one per block, the same way in k_bin_count,
 // k_bin_fill and k_records. k_bin_count leaves, per (chunk, tile), the number of instances the chunk's points have in the
@@ -227,19 +139,6 @@ __host__ __device__ inline uint32_t bin_chunk_size(uint32_t n, uint32_t n_chunks
 __device__ __forceinline__ uint32_t packed_counter_next(uint32_t* counters, uint32_t tile) {
     const uint32_t shift = (tile & 1u) * 16u;
     return (atomicAdd(&counters[tile >> 1], 1u << shift) >> shift) & 0xFFFFu;
-}
-
-// For every touched tile of a projected point, in the row-major order of the reference's create_instances_cu
-// (kernels.cu:208-217).
-template <typename F>
-__device__ __forceinline__ void for_each_tile(uint32_t info, uint32_t gw, F f) {
-    const uint32_t tile0 = info_tile0(info);
-    f(tile0);
-    if (info & (1u << 16)) f(tile0 + 1u);
-    if (info & (1u << 17)) {
-        f(tile0 + gw);
-        if (info & (1u << 16)) f(tile0 + gw + 1u);
-    }
 }
 
 template <int T, bool WIDE>
@@ -564,7 +463,7 @@ __global__ void __launch_bounds__(kBinThreads)
             const Projected p = project_point<T>(m, g, px[u], py[u], pz[u]);
             if (p.info == 0u) continue;
             my_visible += 1u;
-            const uint64_t pair = ((uint64_t)(__float_as_uint(p.depth) - g.key_bias) << 32) | (uint64_t)i;
+            const uint64_t pair = ((uint64_t)depth_key(p.depth, g.key_bias) << 32) | (uint64_t)i;
             if (!overflow)
                 for_each_tile(p.info, g.gw, [&](uint32_t tile) {
                     const uint32_t local = tile - tile_first;   // wraps around for a tile in front of the window
