@@ -146,8 +146,13 @@ __device__ __forceinline__ bool barrier_all_done(QuadScratch<T>* s_quad, bool do
 
 // Makes the value available here: the wait for an outstanding load that produces it lands at this point and not
 // at a later first use.
+#if defined(__AMDGCN__)
 __device__ __forceinline__ void arrive(float& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void arrive(uint32_t& v) { asm volatile("" : "+v"(v)); }
+#else   // only the device has loads in flight to wait for
+__device__ __forceinline__ void arrive(float&) {}
+__device__ __forceinline__ void arrive(uint32_t&) {}
+#endif
 
 __device__ __forceinline__ void arrive(Header& h) {
     arrive(h.wx0);
@@ -705,8 +710,9 @@ __global__ void __launch_bounds__(256) k_grad_reduce(SplitRows rows, float* __re
             }
         ((float4*)(grad_view + (size_t)i * C))[word] = acc;
         if (word == kGroup - 1u) grad_opacities[i] = opacity;
-        // the flags go back to zero for the next pass; the other lanes of the group have read them: they run in
-        // lockstep with this one (same wave, same control flow)
+        // the flags go back to zero for the next pass, once the other lanes of the group have read them (same wave,
+        // same control flow: their loads are complete behind this point)
+        wave_sync();
         if (word == 0u) {
 #pragma unroll
             for (int p = 0; p < 4; ++p)

@@ -84,6 +84,11 @@ int resident_blocks(const void* kernel, int threads, uint32_t& blocks);
 // ------------------------------------------------------------------------------------------------
 constexpr int kWave = 64;
 
+// The dynamic LDS of a launch as an array `name` of `type` (16-byte aligned).
+#ifndef INPC_DYNAMIC_LDS
+#define INPC_DYNAMIC_LDS(type, name) extern __shared__ __align__(16) type name[]
+#endif
+
 // Plain per-thread arithmetic that the tests also run on the host (geometry.hpp, the generators below).
 #define INPC_HD __host__ __device__ __forceinline__
 

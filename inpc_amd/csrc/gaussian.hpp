@@ -241,7 +241,7 @@ __global__ void __launch_bounds__(THREADS)
     k_bin_count(const uint32_t* __restrict__ touched, const uint2* __restrict__ bounds, uint32_t* __restrict__ table,
                 uint2* __restrict__ split_count, uint32_t tile_first, uint32_t tile_count, uint32_t n, uint32_t n_chunks,
                 uint32_t n_tiles, uint32_t gw) {
-    extern __shared__ uint32_t s_count[];   // tile_count
+    INPC_DYNAMIC_LDS(uint32_t, s_count);   // tile_count
     __shared__ uint32_t s_queue[kQueue];
     __shared__ uint32_t s_queued, s_split, s_rows;
     for (uint32_t t = threadIdx.x; t < tile_count; t += THREADS) s_count[t] = 0u;
@@ -283,7 +283,7 @@ __global__ void __launch_bounds__(THREADS)
                const uint2* __restrict__ split_base, uint4* __restrict__ multi_list, char* __restrict__ records,
                uint32_t stride, const uint32_t* __restrict__ counters, uint32_t tile_first, uint32_t tile_count,
                uint32_t n, uint32_t n_chunks, uint32_t n_tiles, uint32_t gw) {
-    extern __shared__ uint32_t s_cursor[];   // tile_count
+    INPC_DYNAMIC_LDS(uint32_t, s_cursor);   // tile_count
     __shared__ uint32_t s_queue[kQueue];
     __shared__ uint32_t s_queued, s_split, s_rows;
     if (counters[kCntKept] == 0u) return;   // nothing is drawn (no instances, or more than the buffers hold)

@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(WIDE ? kBinThreadsWide : kBinThreads) k_bin_co
                                                            const float* __restrict__ w2c, uint32_t* __restrict__ table,
                                                            uint2* __restrict__ split_count, Geometry g) {
     constexpr int kThreads = WIDE ? kBinThreadsWide : kBinThreads;
-    extern __shared__ uint32_t s_count[];
+    INPC_DYNAMIC_LDS(uint32_t, s_count);
     __shared__ uint32_t s_split, s_rows;   // the chunk's points that touch several tiles, and their instances
     const uint32_t n_words = WIDE ? (g.n_tiles + 1u) / 2u : g.n_tiles;
     for (uint32_t t = threadIdx.x; t < n_words; t += kThreads) s_count[t] = 0u;
@@ -433,7 +433,7 @@ __global__ void __launch_bounds__(kBinThreads)
                const uint32_t* __restrict__ bin_start, uint64_t* __restrict__ pairs, uint32_t* counters,
                uint32_t tile_first, uint32_t tile_count, Geometry g) {
     constexpr int kThreads = kBinThreads;
-    extern __shared__ __align__(16) uint32_t s_cursor[];   // tile_count
+    INPC_DYNAMIC_LDS(uint32_t, s_cursor);   // tile_count
     __shared__ uint32_t s_visible;
     const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then no instance is stored
     const uint32_t* row = table + (size_t)blockIdx.x * g.n_tiles;   // instances of the chunks before, per tile
@@ -489,7 +489,7 @@ __global__ void __launch_bounds__(kRecordThreads)
               float* __restrict__ blending_weights, SplitOut split, float4* __restrict__ debug_geometry,
               const uint32_t* __restrict__ counters, Geometry g) {
     constexpr int kThreads = kRecordThreads;
-    extern __shared__ __align__(16) uint32_t s_dyn[];
+    INPC_DYNAMIC_LDS(uint32_t, s_dyn);
     float4* s_stage = (float4*)s_dyn;      // record staging, 64 rows per wave
     __shared__ uint32_t s_split, s_rows;   // next list entry / gradient row for a point of this chunk
     const bool overflow = counters[kCntOverflow] != 0u;   // written by k_bin_scan: then nothing is drawn

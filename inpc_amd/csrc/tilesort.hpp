@@ -257,7 +257,7 @@ template <int THREADS>
 __global__ void __launch_bounds__(THREADS, 4)   // four waves per SIMD: 128 registers
     k_tile_sort(const uint2* __restrict__ ranges, const uint32_t* __restrict__ tile_order, uint64_t* pairs,
                 uint64_t* scratch, uint32_t* __restrict__ points, int key_bits) {
-    extern __shared__ __align__(16) unsigned char s_raw[];
+    INPC_DYNAMIC_LDS(unsigned char, s_raw);
     Shared<THREADS>& sh = *reinterpret_cast<Shared<THREADS>*>(s_raw);
     constexpr uint32_t kThreads = THREADS, kCap = Shared<THREADS>::kCap;
     const uint32_t t = threadIdx.x;

@@ -114,6 +114,11 @@ def _checked_inputs(positions, features, opacities, feature_mode: int, channels:
     return positions, features, opacities
 
 
+def _new_workspace(n_bytes: int, device) -> torch.Tensor:
+    """Uninitialised device bytes for one forward pass (the device allocator aligns them to 256 bytes and more)."""
+    return torch.empty(n_bytes, dtype=torch.uint8, device=device)
+
+
 def _checked_camera_tensor(t: torch.Tensor, numel: int, name: str, device) -> torch.Tensor:
     """The camera tensors reach the kernels as raw float pointers: they must be fp32 on the points' device
     (the reference's data_ptr<float>() raises for another dtype, B/rasterization/src/rasterization_api.cu:61-65)."""
@@ -158,7 +163,7 @@ def _forward_gaussian(settings: RasterizerSettings, positions, features, opaciti
                                   float(sigma_world), float(sigma_cutoff), capacity, 0)
         layout = _lib.GaussianLayout()
         _lib.check(lib.inpc_gaussian_layout_query(C.byref(cfg), C.byref(layout)), "inpc_gaussian_layout_query")
-        workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+        workspace = _new_workspace(layout.total_bytes, device)
         stream = _lib.current_stream()
         _lib.check(lib.inpc_gaussian_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
                                              _lib.ptr(scales), _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image),
@@ -208,7 +213,7 @@ def _forward_native(settings: RasterizerSettings, positions, features, opacities
     for _ in range(2):
         cfg = _config(settings, n, tile, out_channels, feature_mode, inference, capacity)
         layout = query_layout(cfg)
-        workspace = torch.empty(layout.total_bytes, dtype=torch.uint8, device=device)
+        workspace = _new_workspace(layout.total_bytes, device)
         stream = _lib.current_stream()
         _lib.check(lib.inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
                                            _lib.ptr(w2c), _lib.ptr(cam_position), _lib.ptr(image), _lib.ptr(alpha),

@@ -1,0 +1,179 @@
+// sim.cpp — fibers and meeting points of the SIMT simulator (see sim.hpp). x86-64 only.
+#include "sim.hpp"
+
+#include <cstdio>
+
+namespace sim {
+
+namespace {
+thread_local Block* g_block = nullptr;
+thread_local Fiber* g_fiber = nullptr;
+constexpr size_t kStackBytes = 256 * 1024;
+
+// Saves the callee-saved registers on the current stack, stores the stack pointer in *from, switches to `to`.
+extern "C" void sim_switch(void** from, void* to);
+asm(R"(
+.text
+.globl sim_switch
+.type sim_switch,@function
+sim_switch:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    subq $8, %rsp
+    stmxcsr (%rsp)
+    fnstcw 4(%rsp)
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    ldmxcsr (%rsp)
+    fldcw 4(%rsp)
+    addq $8, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+.size sim_switch,.-sim_switch
+)");
+
+void fiber_main() {
+    Block& b = *g_block;
+    Fiber& f = *g_fiber;
+    b.body();
+    f.done = true;
+    b.progress = true;
+    // a fiber that ends no longer takes part in meetings: the others may be waiting for exactly that
+    b.block_meeting.alive -= 1;
+    b.waves[f.tid >> 6].alive -= 1;
+    sim_switch(&f.sp, b.scheduler_sp);
+    std::fprintf(stderr, "sim: a finished fiber was resumed\n");
+    std::abort();
+}
+
+void prepare(Fiber& f) {
+    if (!f.stack) f.stack = (char*)std::aligned_alloc(64, kStackBytes);
+    // initial frame for sim_switch: mxcsr / x87 control word, six callee-saved registers, return address
+    uintptr_t top = ((uintptr_t)f.stack + kStackBytes) & ~(uintptr_t)63;
+    uint64_t* sp = (uint64_t*)top;
+    *--sp = 0;                       // alignment: at fiber_main's entry rsp + 8 must be a multiple of 16
+    *--sp = (uint64_t)&fiber_main;   // return address of the first switch
+    for (int i = 0; i < 6; ++i) *--sp = 0;
+    uint32_t mxcsr, fpcw = 0;
+    asm volatile("stmxcsr %0" : "=m"(mxcsr));
+    asm volatile("fnstcw %0" : "=m"(*(uint16_t*)&fpcw));
+    *--sp = ((uint64_t)fpcw << 32) | mxcsr;
+    f.sp = sp;
+}
+
+const uint64_t* meet(Meeting& m, uint64_t& my_gen, uint32_t index, uint64_t value) {
+    Block& b = *g_block;
+    const uint64_t g = my_gen;
+    const int p = (int)(g & 1u);
+    if (m.arrived[p] == 0) std::memset(m.present[p], 0, sizeof(m.present[p]));
+    m.slot[p][index] = value;
+    m.present[p][index >> 6] |= 1ull << (index & 63u);
+    m.arrived[p] += 1;
+    b.progress = true;
+    while (m.completed < g + 1) {
+        if (m.arrived[p] >= m.alive) {
+            std::memcpy(m.mask[p], m.present[p], sizeof(m.present[p]));
+            m.completed = g + 1;
+            m.arrived[p] = 0;
+            b.progress = true;
+            break;
+        }
+        yield();
+    }
+    my_gen = g + 1;
+    return m.slot[p];
+}
+}  // namespace
+
+Block& block() { return *g_block; }
+Fiber& fiber() { return *g_fiber; }
+
+void yield() {
+    Fiber& f = *g_fiber;
+    sim_switch(&f.sp, g_block->scheduler_sp);
+}
+
+const uint64_t* meet_wave(uint64_t value, uint64_t* members) {
+    Fiber& f = *g_fiber;
+    Meeting& m = g_block->waves[f.tid >> 6];
+    const int p = (int)(f.wave_gen & 1u);
+    const uint64_t* slots = meet(m, f.wave_gen, f.tid & 63u, value);
+    if (members) *members = m.mask[p][0];
+    return slots;
+}
+
+const uint64_t* meet_block(uint64_t value, const uint64_t** members) {
+    Fiber& f = *g_fiber;
+    Meeting& m = g_block->block_meeting;
+    const int p = (int)(f.block_gen & 1u);
+    const uint64_t* slots = meet(m, f.block_gen, f.tid, value);
+    if (members) *members = m.mask[p];
+    return slots;
+}
+
+void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<void()> body) {
+    const uint32_t n_threads = block_dim.x * block_dim.y * block_dim.z;
+    if (n_threads == 0 || n_threads > (uint32_t)kMaxThreads) {
+        std::fprintf(stderr, "sim: %u threads per block\n", n_threads);
+        std::abort();
+    }
+    static thread_local Block b;   // the stacks are kept from launch to launch
+    Block* outer_block = g_block;
+    Fiber* outer_fiber = g_fiber;
+    g_block = &b;
+    b.block_dim = block_dim;
+    b.grid_dim = grid;
+    b.n_threads = n_threads;
+    if (b.fibers.size() < n_threads) b.fibers.resize(n_threads);
+    b.waves.resize((n_threads + 63) / 64);
+    b.dynamic_lds.assign(dynamic_lds_bytes + 64, 0);
+    b.body = std::move(body);
+    for (uint32_t bz = 0; bz < grid.z; ++bz)
+        for (uint32_t by = 0; by < grid.y; ++by)
+            for (uint32_t bx = 0; bx < grid.x; ++bx) {
+                b.block_idx = Dim3(bx, by, bz);
+                b.block_meeting = Meeting{};
+                b.block_meeting.alive = n_threads;
+                for (size_t w = 0; w < b.waves.size(); ++w) {
+                    b.waves[w] = Meeting{};
+                    b.waves[w].alive = std::min<uint32_t>(64u, n_threads - (uint32_t)w * 64u);
+                }
+                for (uint32_t t = 0; t < n_threads; ++t) {
+                    Fiber& f = b.fibers[t];
+                    f.done = false;
+                    f.tid = t;
+                    f.wave_gen = f.block_gen = 0;
+                    prepare(f);
+                }
+                uint32_t left = n_threads;
+                while (left) {
+                    b.progress = false;
+                    left = 0;
+                    for (uint32_t t = 0; t < n_threads; ++t) {
+                        Fiber& f = b.fibers[t];
+                        if (f.done) continue;
+                        g_fiber = &f;
+                        sim_switch(&b.scheduler_sp, f.sp);
+                        if (!f.done) ++left;
+                    }
+                    if (left && !b.progress) {
+                        std::fprintf(stderr, "sim: deadlock in block (%u,%u,%u): %u fibers wait at meeting points "
+                                             "that not all live fibers of their wave or block reach\n", bx, by, bz, left);
+                        std::abort();
+                    }
+                }
+            }
+    g_block = outer_block;
+    g_fiber = outer_fiber;
+}
+
+}  // namespace sim

@@ -9,9 +9,29 @@ import torch
 
 from inpc_amd import _lib
 
+# Where the wrappers below put their buffers when the caller names no device. The simulator tier (tests/cpu_sim)
+# sets it to "cpu" while the kernels compiled for the host are the loaded library.
+DEVICE = "cuda:0"
 
-def dev(a, device="cuda:0"):
-    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+def device_of(device=None):
+    return torch.device(DEVICE if device is None else device)
+
+
+def dev(a, device=None):
+    """A tensor on the device with a copy of `a` (a copy also where the device is the host: the kernels write into
+    their arguments, and the caller keeps comparing against `a`)."""
+    device = device_of(device)
+    host = torch.from_numpy(np.ascontiguousarray(a))
+    return host.clone() if device.type == "cpu" else host.to(device)
+
+
+def poisoned_bytes(n_bytes: int, device) -> torch.Tensor:
+    """n_bytes of random bytes on `device`, 256-byte aligned like every allocation of the GPU's allocator (a host
+    allocation is only 64-byte aligned: a slice that starts at the next multiple of 256 is taken)."""
+    raw = torch.randint(0, 256, (n_bytes + 256,), dtype=torch.uint8, device=device)
+    skip = (-raw.data_ptr()) % 256
+    return raw[skip:skip + n_bytes]
 
 
 def cam_struct(camera) -> _lib.Camera:
@@ -22,11 +42,11 @@ def stream():
     return _lib.current_stream()
 
 
-def make_rng(seed: int, device="cuda:0"):
+def make_rng(seed: int, device=None):
     host = (C.c_uint64 * 2)()
     _lib.lib().inpc_pcg32_seed(host, C.c_uint64(seed), C.c_uint64(1))
     signed = [int(v) - 2**64 if int(v) >= 2**63 else int(v) for v in host]
-    return torch.tensor(signed, dtype=torch.int64, device=device)
+    return torch.tensor(signed, dtype=torch.int64, device=device_of(device))
 
 
 def rng_values(rng_dev):
@@ -34,7 +54,8 @@ def rng_values(rng_dev):
     return s % 2**64, i % 2**64
 
 
-def leaf_weights(oct, hv, device="cuda:0"):
+def leaf_weights(oct, hv, device=None):
+    device = device_of(device)
     lib = _lib.lib()
     n = len(oct.levels)
     out = torch.empty(n, dtype=torch.float32, device=device)
@@ -47,13 +68,14 @@ def leaf_weights(oct, hv, device="cuda:0"):
     return out
 
 
-def leaf_boxes(oct, hv=None, device="cuda:0"):
+def leaf_boxes(oct, hv=None, device=None):
     """(L, 4) device tensor {centre, edge length} as inpc_leaf_weights writes it for the sampling calls
     (the camera does not enter it)."""
     from inpc_amd import synthetic
 
     if hv is None:
         hv = synthetic.camera_on_z(8, 8, 8.0, 1.0)
+    device = device_of(device)
     lib = _lib.lib()
     n = len(oct.levels)
     out = torch.empty(n, dtype=torch.float32, device=device)
@@ -103,7 +125,7 @@ class CullDraw:
         self.ids = torch.full((capacity,), -7, dtype=torch.int64 if ids_int64 else torch.int32, device=device)
         self.ws_bytes = int(self.lib.inpc_cull_workspace_bytes(max_round))
         # poisoned: the round that starts at candidate 0 clears the state of the draw itself
-        self.ws = torch.randint(0, 256, (self.ws_bytes,), dtype=torch.uint8, device=device)
+        self.ws = poisoned_bytes(self.ws_bytes, device)
         self.cam = cam_struct(hv.camera)
         self.k0 = 0
 
@@ -136,7 +158,7 @@ class RasterRun:
     """inpc_raster_forward (+ backward) through the C ABI on numpy inputs."""
 
     def __init__(self, hv, positions, features, opacities, tile=16, channels=4, feature_mode=_lib.FEAT_DIRECT_F32,
-                 inference=False, device="cuda:0", max_instances=None, keep_geometry=True):
+                 inference=False, device=None, max_instances=None, keep_geometry=True):
         self.lib = _lib.lib()
         self.hv = hv
         self.n = len(positions)
@@ -149,7 +171,7 @@ class RasterRun:
         self.layout = _lib.RasterLayout()
         _lib.check(self.lib.inpc_raster_layout_query(C.byref(self.cfg), C.byref(self.layout)), "layout")
         self.inference = inference
-        self.device = device
+        self.device = device = device_of(device)
         self.positions = dev(np.asarray(positions, np.float32).reshape(-1, 3), device)
         self.features = dev(np.asarray(features, FEATURE_DTYPES[feature_mode]), device)
         self.opacities = None if opacities is None else dev(np.asarray(opacities, np.float32).reshape(-1), device)
@@ -161,7 +183,7 @@ class RasterRun:
         self.bw = None if inference else torch.full((max(self.n, 1),), float("nan"), dtype=torch.float32, device=device)
         self.depth_image = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device) if inference else None
         # poisoned: nothing may depend on what the workspace held before the call
-        self.ws = torch.randint(0, 256, (self.layout.total_bytes,), dtype=torch.uint8, device=device)
+        self.ws = poisoned_bytes(self.layout.total_bytes, device)
 
     def forward(self):
         _lib.check(self.lib.inpc_raster_forward(
@@ -281,7 +303,7 @@ class GaussianRun:
     """inpc_gaussian_forward (+ backward) through the C ABI on numpy inputs."""
 
     def __init__(self, hv, positions, features, opacities, tile=8, channels=4, feature_mode=_lib.FEAT_DIRECT_F32,
-                 inference=False, scales=None, sigma_world=0.0, sigma_cutoff=3.0, max_instances=0, device="cuda:0"):
+                 inference=False, scales=None, sigma_world=0.0, sigma_cutoff=3.0, max_instances=0, device=None):
         self.lib = _lib.lib()
         self.n = len(positions)
         sh = feature_mode in (_lib.FEAT_SH36_F16, _lib.FEAT_RAW37_F16)
@@ -292,7 +314,7 @@ class GaussianRun:
         self.layout = _lib.GaussianLayout()
         _lib.check(self.lib.inpc_gaussian_layout_query(C.byref(self.cfg), C.byref(self.layout)), "layout")
         self.inference = inference
-        self.device = device
+        self.device = device = device_of(device)
         self.positions = dev(np.asarray(positions, np.float32).reshape(-1, 3), device)
         self.features = dev(np.asarray(features, FEATURE_DTYPES[feature_mode]), device)
         self.opacities = None if opacities is None else dev(np.asarray(opacities, np.float32).reshape(-1), device)
@@ -305,7 +327,7 @@ class GaussianRun:
         self.bw = None if inference else torch.full((max(self.n, 1),), float("nan"), dtype=torch.float32, device=device)
         self.depth_image = torch.full((1, H, W), float("nan"), dtype=torch.float32, device=device) if inference else None
         # poisoned: nothing may depend on what the workspace held before the call
-        self.ws = torch.randint(0, 256, (self.layout.total_bytes,), dtype=torch.uint8, device=device)
+        self.ws = poisoned_bytes(self.layout.total_bytes, device)
 
     def forward(self):
         _lib.check(self.lib.inpc_gaussian_forward(

@@ -13,18 +13,6 @@ GOLDEN = Path(__file__).resolve().parent / "golden"
 RTOL = 1e-4
 
 
-def _load_maker():
-    spec = importlib.util.spec_from_file_location("make_golden", GOLDEN / "make_golden.py")
-    module = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(module)
-    return module
-
-
-@pytest.fixture(scope="module")
-def maker():
-    return _load_maker()
-
-
 def _bits(a):
     a = np.ascontiguousarray(a)
     return a.view(np.uint32) if a.dtype == np.float32 else a
@@ -108,7 +96,7 @@ def test_hip_sampler_gives_fixture(gpu, maker):
     assert H.rng_values(rng) == tuple(int(v) for v in want["plain_state"])
     # the whole training draw through the operator layer
     sampler = ProbabilityFieldSampler(seed=p["rng_seed"])
-    view = hv.to_view(torch.device("cuda:0"))
+    view = hv.to_view(gpu)
     tpos, tids = sampler.generate_training_samples(H.dev(oct.centers), H.dev(oct.levels), H.dev(oct.weights), view,
                                                    p["n_training"], oct.initial_size)
     np.testing.assert_array_equal(tids.cpu().numpy(), want["training_ids"].astype(np.int64))

@@ -14,7 +14,7 @@ from inpc_amd import ProbabilityFieldSampler, _lib, synthetic
 from tests import helpers as H
 from tests.test_gpu_raster import check_structure, oracle_cfg
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.real_gpu]
 
 RTOL = 1e-4
 

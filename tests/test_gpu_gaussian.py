@@ -102,6 +102,7 @@ def test_forward_backward_dense_opaque_scene(gpu, oracle, tile):
     H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
 
 
+@pytest.mark.real_gpu
 def test_forward_backward_replay_from_a_graph_with_new_inputs(gpu, oracle):
     # A captured step keeps its kernel arguments, so whatever tells this pass's gradient rows from an earlier
     # pass's has to change on the device. The scene saturates (tiles end early and leave rows unwritten) and has
@@ -121,10 +122,10 @@ def test_forward_backward_replay_from_a_graph_with_new_inputs(gpu, oracle):
     run = H.GaussianRun(hv, pos, feats, opac, tile, channels)
     lib = _lib.lib()
     Hh, Ww = hv.camera.height, hv.camera.width
-    gf = torch.empty((n, channels), dtype=torch.float32, device="cuda:0")
-    go = torch.empty((n,), dtype=torch.float32, device="cuda:0")
-    gi = torch.zeros((channels, Hh, Ww), dtype=torch.float32, device="cuda:0")
-    ga = torch.zeros((1, Hh, Ww), dtype=torch.float32, device="cuda:0")
+    gf = torch.empty((n, channels), dtype=torch.float32, device=gpu)
+    go = torch.empty((n,), dtype=torch.float32, device=gpu)
+    gi = torch.zeros((channels, Hh, Ww), dtype=torch.float32, device=gpu)
+    ga = torch.zeros((1, Hh, Ww), dtype=torch.float32, device=gpu)
 
     def step():
         s = _lib.current_stream()

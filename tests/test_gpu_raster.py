@@ -461,6 +461,7 @@ def test_random_scenes_forward_backward(gpu, oracle, case):
     H.assert_close(go, go_ref, RTOL, 2e-6, "opacity gradients")
 
 
+@pytest.mark.real_gpu
 def test_forward_backward_replays_from_a_graph(gpu, oracle):
     # The library enqueues kernels only (no allocation, no memset nodes, no host read-back in forward / backward),
     # so a caller may capture a step into a graph. Replays with new inputs written in place must give what eager
@@ -469,11 +470,11 @@ def test_forward_backward_replays_from_a_graph(gpu, oracle):
     hv, pos, feats, opac = scene(n, channels, seed=77)
     run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32)
     lib = _lib.lib()
-    gf = torch.empty((n, channels), dtype=torch.float32, device="cuda:0")
-    go = torch.empty((n,), dtype=torch.float32, device="cuda:0")
+    gf = torch.empty((n, channels), dtype=torch.float32, device=gpu)
+    go = torch.empty((n,), dtype=torch.float32, device=gpu)
     Hh, Ww = hv.camera.height, hv.camera.width
-    gi = torch.zeros((channels, Hh, Ww), dtype=torch.float32, device="cuda:0")
-    ga = torch.zeros((1, Hh, Ww), dtype=torch.float32, device="cuda:0")
+    gi = torch.zeros((channels, Hh, Ww), dtype=torch.float32, device=gpu)
+    ga = torch.zeros((1, Hh, Ww), dtype=torch.float32, device=gpu)
 
     def step():
         s = _lib.current_stream()

@@ -10,7 +10,7 @@ from tests import helpers as H
 from tests.test_gpu_gaussian import check_structure as check_gaussian_structure, grad_atol, oracle_run
 from tests.test_gpu_raster import check_structure, oracle_cfg
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.real_gpu]
 
 RTOL = 1e-4
 
