@@ -40,6 +40,7 @@ struct Shared {
     alignas(16) uint16_t count[kDigits * THREADS];        // [digit][thread], scanned in this order
     uint32_t wave_sum[THREADS / kWave];
     uint32_t bits_or[2], bits_and[2];                     // over the tile's elements: [0] point index, [1] key
+    static_assert(kCap <= kDigits * THREADS && kCap <= 65536, "count[] also holds one 16-bit place per element");
 };
 
 __device__ __forceinline__ uint32_t hi32(uint64_t v) { return (uint32_t)(v >> 32); }
@@ -65,8 +66,8 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t v, int shift) {
 // of 64) own kPer consecutive elements each; every thread of the block calls it (the others only meet the
 // barriers). All elements are in registers before the first one is stored, so one buffer suffices.
 template <int THREADS, int kPer>
-__device__ __forceinline__ void digit_pass(Shared<THREADS>& sh, uint32_t active, int shift) {
-    const uint32_t t = threadIdx.x, lane = t & 63u, wave = t >> 6;
+__device__ __forceinline__ void digit_pass(Shared<THREADS>& sh, uint32_t t, uint32_t active, int shift) {
+    const uint32_t lane = t & 63u, wave = t >> 6;
     const bool on = t < active;
     uint64_t v[kPer];
     uint64_t fields = 0ull;   // sixteen 4-bit counters: kPer <= 15 elements per thread cannot overflow one
@@ -124,7 +125,11 @@ __device__ __forceinline__ void digit_pass(Shared<THREADS>& sh, uint32_t active,
 // kPer * active, hold kPad). All threads of the block call it.
 template <int THREADS, int kPer>
 __device__ void sort_run(Shared<THREADS>& sh, uint32_t n, uint32_t active, int key_bits) {
-    const uint32_t t = threadIdx.x, lane = t & 63u;
+    // the thread index as a value of this function's own: the compiler otherwise computes the element addresses of
+    // all four instantiations (kPer = 3, 7, 11, 15) at the top of the kernel and keeps them in registers throughout
+    uint32_t t = threadIdx.x;
+    blend::arrive(t);
+    const uint32_t lane = t & 63u;
     const bool on = t < active;
     // bits that differ between the elements
     {
@@ -162,7 +167,7 @@ __device__ void sort_run(Shared<THREADS>& sh, uint32_t n, uint32_t active, int k
     const uint32_t vary_lo = sh.bits_or[0] ^ sh.bits_and[0], vary_hi = sh.bits_or[1] ^ sh.bits_and[1];
     auto key_passes = [&]() {
         for (int shift = 0; shift < key_bits; shift += 4)
-            if ((vary_hi >> shift) & 15u) digit_pass<THREADS, kPer>(sh, active, 32 + shift);
+            if ((vary_hi >> shift) & 15u) digit_pass<THREADS, kPer>(sh, t, active, 32 + shift);
     };
     key_passes();
     // elements with equal keys stand in the order they were binned; the order wanted is by point index
@@ -180,19 +185,18 @@ __device__ void sort_run(Shared<THREADS>& sh, uint32_t n, uint32_t active, int k
     }
     if (__syncthreads_or(any) == 0) return;
     // Runs of equal keys are mostly short, however many there are: every tied element looks along its run, up to
-    // kShortRun elements to either side, and takes the place its point index gives it inside the run. All of them
-    // are read before the first one is stored. A longer run anywhere in the tile sends the tile to the sort over
-    // all 64 bits below (nothing has been stored by then).
+    // kShortRun elements to either side, and takes the place its point index gives it inside the run. The places go
+    // to sh.count (free between the passes; a place is below kCap <= 65536 / 8), so that no thread keeps a table
+    // of them in registers; then all tied elements are read before the first one is stored. A longer run anywhere
+    // in the tile sends the tile to the sort over all 64 bits below (nothing has been stored by then).
     {
-        uint32_t at[kPer];
-        uint64_t v[kPer];
         bool long_run = false;
 #pragma unroll
         for (int e = 0; e < kPer; ++e) {
             if (!tied[e]) continue;
             const uint32_t p = t * kPer + e;
-            v[e] = sh.buf[p];
-            const uint32_t key = hi32(v[e]), mine = lo32(v[e]);
+            const uint64_t own = sh.buf[p];
+            const uint32_t key = hi32(own), mine = lo32(own);
             uint32_t first = p, last = p + 1u, smaller = 0u;
             for (uint32_t step = 0; first > 0u; ++step) {
                 const uint64_t w = sh.buf[first - 1u];
@@ -214,19 +218,24 @@ __device__ void sort_run(Shared<THREADS>& sh, uint32_t n, uint32_t active, int k
                 ++last;
                 smaller += lo32(w) < mine ? 1u : 0u;
             }
-            at[e] = first + smaller;
+            sh.count[p] = (uint16_t)(first + smaller);
         }
         if (__syncthreads_or(long_run) == 0) {
+            uint64_t v[kPer];
 #pragma unroll
             for (int e = 0; e < kPer; ++e)
-                if (tied[e]) sh.buf[at[e]] = v[e];
+                if (tied[e]) v[e] = sh.buf[t * kPer + e];
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < kPer; ++e)
+                if (tied[e]) sh.buf[sh.count[t * kPer + e]] = v[e];
             __syncthreads();
             return;
         }
     }
     // many ties: sort over all 64 bits, least significant digit first
     for (int shift = 0; shift < 32; shift += 4)
-        if ((vary_lo >> shift) & 15u) digit_pass<THREADS, kPer>(sh, active, shift);
+        if ((vary_lo >> shift) & 15u) digit_pass<THREADS, kPer>(sh, t, active, shift);
     key_passes();
 }
 
