@@ -118,12 +118,13 @@ size_t inpc_cdf_head_floats(uint32_t n_leaves);
  * sampling kernels take the failure path themselves. [1 .. INPC_CDF_HEAD_MIN_FLOATS - 1] receive
  * the CDF elements that the first 14 probes of the binary search of B/sampling/src/
  * sampling_kernels.cu:101-126 can read, in heap order, and behind them those of the further
- * levels. Every later call that takes `sum_dev` takes this buffer. No host synchronisation. */
+ * levels. Every later call that takes `sum_dev` takes this buffer. No host synchronisation.
+ * Three launches whatever the size; at most 2^30 leaves (INPC_E_UNSUPPORTED beyond). */
 int inpc_build_cdf(float* weights_inout, float* sum_out, size_t head_floats, void* workspace,
                    size_t workspace_bytes, uint32_t n_leaves, void* stream);
 
 /* The same as inpc_build_cdf without a workspace argument: the chunk totals live in a scratch array
- * built into the library (about 261 KB of device memory per GPU the library runs on, held until the
+ * built into the library (264 KB of device memory per GPU the library runs on, held until the
  * process ends), so the call allocates nothing and takes nothing but inputs and outputs. It has no
  * counterpart in the reference; it is for callers that cannot allocate device memory or size a
  * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid allocation).

@@ -1,9 +1,10 @@
 // sampler.hip — view-dependent point sampling from the octree probability field (gfx950).
 //
 //   k_leaf_weights        per-leaf visibility + weight   (B/sampling/src/sampling_kernels.cu:9-64)
-//   k_chunk_pass / k_chunk_add_prefix
+//   k_tile_totals / k_cdf_scan_tiles / k_cdf_finish
 //                         normalise + float CDF with a fixed association order (chunks of 64,
-//                         left to right, recursively)      (B/sampling/src/sampling.cu:150-186)
+//                         left to right, recursively) and the top of the search tree, in three
+//                         launches                         (B/sampling/src/sampling.cu:150-186)
 //   k_sample              multinomial leaf pick + jitter  (B/sampling/src/sampling_kernels.cu:128-150)
 //   k_sample_cull         the same draw, frustum test, ordered stream compaction
 //                                                         (B/sampling/src/sampling_kernels.cu:77-126)
@@ -98,20 +99,16 @@ __global__ void __launch_bounds__(kBlock) k_leaf_weights(const float* __restrict
     out[l] = wgt;
 }
 
-// One wave per block; the block stages 64 chunks of 64 floats through LDS (coalesced), lane c adds
-// up chunk c left to right. SCAN = false: totals only. SCAN = true: in-place inclusive scan inside
-// each chunk, optionally after multiplying by 1/(*norm_sum).
-template <bool SCAN>
-__global__ void __launch_bounds__(kWave) k_chunk_pass(float* data, uint32_t n, float* __restrict__ totals,
-                                                      const float* __restrict__ guard_sum,
-                                                      const float* __restrict__ norm_sum) {
-    __shared__ float tile[kChunksPerBlock * (kChunk + 1)];
-    if (guard_sum && !(*guard_sum > 0.0f)) return;
-    const uint32_t lane = threadIdx.x;
-    const size_t base = (size_t)blockIdx.x * kChunkTile;
-    float norm = 1.0f;
-    const bool normalise = SCAN && norm_sum != nullptr;
-    if (normalise) norm = 1.0f / *norm_sum;
+// ---- sums and scans in the fixed association order ------------------------------------------------------------------
+// Left to right inside chunks of 64 values, the chunk totals combined the same way one level up, recursively; a scanned
+// element is its chunk's local scan plus the final scanned total of the chunks in front (B/sampling/src/sampling.cu:
+// 150-186 leaves the order to cub; this one is the library's own, so that a CPU restatement can follow it bit for
+// bit). A block of one wave takes a tile of 64 chunks, which is one chunk of the level above.
+
+// Stages the tile's 64 rows of 64 floats in LDS (row stride 65: lane c then walks row c without bank conflicts).
+// `scale` multiplies every element on the way in.
+__device__ __forceinline__ void stage_tile(float* tile, const float* data, size_t base, uint32_t n, float scale,
+                                           uint32_t lane) {
     // the loads of sixteen rows are issued together (one row at a time left the wave waiting on every load)
     for (int r0 = 0; r0 < kChunksPerBlock; r0 += 16) {
         float v[16];
@@ -121,39 +118,154 @@ __global__ void __launch_bounds__(kWave) k_chunk_pass(float* data, uint32_t n, f
             v[k] = i < n ? data[i] : 0.0f;
         }
 #pragma unroll
-        for (int k = 0; k < 16; ++k) tile[(r0 + k) * (kChunk + 1) + lane] = normalise ? v[k] * norm : v[k];
+        for (int k = 0; k < 16; ++k) tile[(r0 + k) * (kChunk + 1) + lane] = v[k] * scale;
     }
+}
+
+// values[0] + values[1] + ... + values[len - 1], left to right; 1 <= len <= 64. All 64 values are fetched before the
+// first addition (the storage behind `values` holds a whole chunk; what lies behind `len` is not used).
+__device__ __forceinline__ float chunk_sum(const float* values, uint32_t len) {
+    float v[kChunk];
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) v[i] = values[i];
+    float s = v[0];
+#pragma unroll
+    for (int i = 1; i < kChunk; ++i)
+        if ((uint32_t)i < len) s += v[i];
+    return s;
+}
+
+// The totals of `m` values one and two levels up, by one wave: s_a[k] = total of chunk k of `values` (k < ceil(m / 64)
+// <= 4096), s_b[k] = total of chunk k of s_a. Ends with the LDS of the wave in order.
+constexpr uint32_t kMaxUpperValues = 1u << 18;   // values of the level that tops a tile: 2^30 leaves
+constexpr uint32_t kMaxCdfLeaves = 1u << 30;
+__device__ __forceinline__ void upper_totals(const float* values, uint32_t m, float* s_a, float* s_b, uint32_t lane) {
+    const uint32_t m_a = (m + kChunk - 1) / kChunk, m_b = (m_a + kChunk - 1) / kChunk;
+    for (uint32_t k = lane; k < m_a; k += kWave) s_a[k] = chunk_sum(values + (size_t)k * kChunk, min((uint32_t)kChunk, m - k * kChunk));
+    wave_sync();
+    if (lane < m_b) s_b[lane] = chunk_sum(s_a + lane * kChunk, min((uint32_t)kChunk, m_a - lane * kChunk));
+    wave_sync();
+}
+
+// Total of the `m` values (m <= kMaxUpperValues) behind upper_totals; the same in every lane.
+__device__ __forceinline__ float blocked_total(uint32_t m, const float* s_b) {
+    const uint32_t m_a = (m + kChunk - 1) / kChunk, m_b = (m_a + kChunk - 1) / kChunk;
+    return chunk_sum(s_b, m_b);
+}
+
+// Element j of the inclusive scan of the `m` values, behind upper_totals.
+__device__ __forceinline__ float blocked_scan_at(const float* values, uint32_t j, const float* s_a, const float* s_b) {
+    const uint32_t c0 = j / kChunk;
+    const float local0 = chunk_sum(values + (size_t)c0 * kChunk, j - c0 * kChunk + 1u);
+    if (c0 == 0u) return local0;
+    const uint32_t ja = c0 - 1u, ca = ja / kChunk;
+    const float local_a = chunk_sum(s_a + ca * kChunk, ja - ca * kChunk + 1u);
+    if (ca == 0u) return local_a + local0;
+    const float final_b = chunk_sum(s_b, ca);   // scan of s_b at ca - 1: s_b is a single chunk
+    return (final_b + local_a) + local0;
+}
+
+// totals[c] = data[64 c] + ... + data[64 c + 63], left to right: one level of a sum (the expected-count sampler's).
+__global__ void __launch_bounds__(kWave) k_chunk_totals(const float* __restrict__ data, uint32_t n,
+                                                        float* __restrict__ totals) {
+    __shared__ float tile[kChunksPerBlock * (kChunk + 1)];
+    const uint32_t lane = threadIdx.x;
+    const size_t base = (size_t)blockIdx.x * kChunkTile;
+    stage_tile(tile, data, base, n, 1.0f, lane);
     __syncthreads();
     const size_t chunk_base = base + (size_t)lane * kChunk;
     if (chunk_base < n) {
         const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
-        float* row = tile + lane * (kChunk + 1);
+        const float* row = tile + lane * (kChunk + 1);
         float s = row[0];
-        for (int i = 1; i < len; ++i) {
-            s += row[i];
-            if (SCAN) row[i] = s;
-        }
+        for (int i = 1; i < len; ++i) s += row[i];
         totals[(size_t)blockIdx.x * kChunksPerBlock + lane] = s;
-    }
-    if (SCAN) {
-        __syncthreads();
-#pragma unroll 16
-        for (int r = 0; r < kChunksPerBlock; ++r) {
-            const size_t i = base + (size_t)r * kChunk + lane;
-            if (i < n) data[i] = tile[r * (kChunk + 1) + lane];
-        }
     }
 }
 
-__global__ void __launch_bounds__(kBlock) k_chunk_add_prefix(float* data, uint32_t n,
-                                                             const float* __restrict__ inclusive_totals,
-                                                             const float* __restrict__ guard_sum) {
-    if (guard_sum && !(*guard_sum > 0.0f)) return;
-    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    const uint32_t c = i >> 6;
-    if (c == 0) return;
-    data[i] = inclusive_totals[c - 1] + data[i];
+// Level 1 and 2 of a sum: tile_totals[b] = total of tile b's chunk totals. Totals only, `data` is not written.
+// `clear` (n_clear floats, or null) is set to zero, a slice per block.
+__global__ void __launch_bounds__(kWave) k_tile_totals(const float* __restrict__ data, uint32_t n,
+                                                       float* __restrict__ tile_totals, float* __restrict__ clear,
+                                                       uint32_t n_clear) {
+    __shared__ float tile[kChunksPerBlock * (kChunk + 1)];
+    __shared__ float s_chunk[kChunk];
+    const uint32_t lane = threadIdx.x;
+    const size_t base = (size_t)blockIdx.x * kChunkTile;
+    if (clear) {
+        const uint32_t per_block = (n_clear + gridDim.x - 1u) / gridDim.x, first = blockIdx.x * per_block;
+        for (uint32_t i = first + lane; i < min(first + per_block, n_clear); i += kWave) clear[i] = 0.0f;
+    }
+    stage_tile(tile, data, base, n, 1.0f, lane);
+    __syncthreads();
+    const size_t chunk_base = base + (size_t)lane * kChunk;
+    float s = 0.0f;
+    if (chunk_base < n) {
+        const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
+        const float* row = tile + lane * (kChunk + 1);
+        s = row[0];
+        for (int i = 1; i < len; ++i) s += row[i];
+    }
+    s_chunk[lane] = s;
+    wave_sync();
+    const uint32_t n_chunks = min((uint32_t)kChunksPerBlock, (uint32_t)(((size_t)n - base + kChunk - 1) / kChunk));
+    const float total = chunk_sum(s_chunk, n_chunks);
+    if (lane == 0u) tile_totals[blockIdx.x] = total;
+}
+
+// The total on top of k_tile_totals (every block computes it: at most 2^18 values, 64 for 262,144 leaves), then the
+// tile's elements times 1 / total, scanned inside their chunks in place; scanned_chunk_totals[c] = the scan of the
+// tile's chunk totals inside the tile (level 1, local), tile_totals_out[b] = its last element (level 2). head[0] = the
+// total; when that is not positive nothing else is written.
+__global__ void __launch_bounds__(kWave) k_cdf_scan_tiles(float* data, uint32_t n, const float* __restrict__ raw_tile_totals,
+                                                          float* __restrict__ scanned_chunk_totals,
+                                                          float* __restrict__ tile_totals_out, float* __restrict__ head) {
+    __shared__ float tile[kChunksPerBlock * (kChunk + 1)];   // first the totals one level above the tile totals
+    __shared__ float s_b[kChunk];
+    __shared__ float s_chunk[kChunk];
+    static_assert(kMaxUpperValues / kChunk <= kChunksPerBlock * (kChunk + 1), "the upper totals fit the tile's LDS");
+    const uint32_t lane = threadIdx.x;
+    const uint32_t n_tiles = gridDim.x;
+    upper_totals(raw_tile_totals, n_tiles, tile, s_b, lane);
+    const float sum = blocked_total(n_tiles, s_b);
+    if (blockIdx.x == 0u && lane == 0u) head[0] = sum;
+    if (!(sum > 0.0f)) return;
+    const float norm = 1.0f / sum;
+    const size_t base = (size_t)blockIdx.x * kChunkTile;
+    wave_sync();   // the upper totals have been read
+    stage_tile(tile, data, base, n, norm, lane);
+    __syncthreads();
+    const size_t chunk_base = base + (size_t)lane * kChunk;
+    float s = 0.0f;
+    if (chunk_base < n) {
+        const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
+        float* row = tile + lane * (kChunk + 1);
+        s = row[0];
+        for (int i = 1; i < len; ++i) {
+            s += row[i];
+            row[i] = s;
+        }
+    }
+    s_chunk[lane] = s;
+    __syncthreads();
+#pragma unroll 16
+    for (int r = 0; r < kChunksPerBlock; ++r) {
+        const size_t i = base + (size_t)r * kChunk + lane;
+        if (i < n) data[i] = tile[r * (kChunk + 1) + lane];
+    }
+    // the chunk totals scanned left to right; lane c keeps element c
+    const uint32_t n_chunks = min((uint32_t)kChunksPerBlock, (uint32_t)(((size_t)n - base + kChunk - 1) / kChunk));
+    float v[kChunk];
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) v[i] = s_chunk[i];
+    float run = v[0], mine = v[0];
+#pragma unroll
+    for (int i = 1; i < kChunk; ++i) {
+        if ((uint32_t)i < n_chunks) run += v[i];
+        if ((uint32_t)i == lane) mine = run;
+    }
+    if (lane < n_chunks) scanned_chunk_totals[(size_t)blockIdx.x * kChunksPerBlock + lane] = mine;
+    if (lane == 0u) tile_totals_out[blockIdx.x] = run;
 }
 
 // The leaf of a sample is std::lower_bound over the CDF with the probe sequence of
@@ -179,26 +291,6 @@ constexpr uint32_t kTreeNodes = 1u << kTreeDepth;  // heap indices 1 .. kTreeNod
 static_assert(kTreeNodes == INPC_CDF_HEAD_MIN_FLOATS, "the CDF head holds the total and the search tree");
 static_assert(kSampleItems * (kDrawBlock / kWave) <= kWave, "one wave scans the (round, wave) counts of a tile");
 
-// head[node] for every node of the tree (one thread per node).
-__global__ void __launch_bounds__(kBlock) k_build_search_tree(const float* __restrict__ cdf, float* __restrict__ head,
-                                                              uint32_t n, uint32_t n_nodes) {
-    const uint32_t node = blockIdx.x * kBlock + threadIdx.x;
-    if (node == 0u || node >= n_nodes) return;
-    // replay the decisions that lead to this node
-    const int depth = 31 - __clz(node);
-    uint32_t first = 0, count = n;
-    for (int l = depth - 1; l >= 0 && count > 0; --l) {
-        const uint32_t step = count >> 1;
-        if ((node >> l) & 1u) {
-            first += step + 1;
-            count -= step + 1;
-        } else {
-            count = step;
-        }
-    }
-    head[node] = count > 0 ? cdf[first + (count >> 1)] : 0.0f;
-}
-
 // Levels of the tree for n leaves: at least kTreeDepth (the part a block keeps in LDS), and as many as leave a search
 // with at most kFetch elements (every level halves what is left). The levels below kTreeDepth are read from the head
 // in memory: for 2,097,152 leaves three levels, 448 KB that stay in the second-level cache, where probes of the CDF
@@ -208,6 +300,71 @@ __host__ __device__ __forceinline__ int tree_levels(uint32_t n_leaves) {
     int levels = kTreeDepth;
     while (levels < kMaxTreeDepth && (n_leaves >> levels) > kFetch) ++levels;
     return levels;
+}
+
+// Last step of the CDF: the scanned totals of the chunks in front are added to every element, and the elements that
+// the first `levels` probes of the search can read go to the head. Which node of the decision tree probes element i
+// follows from i alone: the search for position i is replayed on the indices (no memory access) until it probes i
+// itself; every element is probed by exactly one node. Nodes that no search reaches (fewer leaves than the tree has
+// nodes) keep the zero they got from k_tile_totals.
+constexpr int kFinishItems = 8;
+constexpr int kFinishTile = kBlock * kFinishItems;   // elements per block: a whole number of chunks, a divisor of a tile
+static_assert(kFinishTile % kChunk == 0 && kChunkTile % kFinishTile == 0, "a block's elements lie in one tile");
+__global__ void __launch_bounds__(kBlock) k_cdf_finish(float* data, uint32_t n, const float* __restrict__ scanned_chunk_totals,
+                                                       const float* __restrict__ tile_totals, uint32_t n_tiles,
+                                                       float* __restrict__ head, int levels) {
+    __shared__ float s_a[kMaxUpperValues / kChunk];
+    __shared__ float s_b[kChunk];
+    __shared__ float s_front[2];                      // scan of the tile totals at tile - 1 and tile - 2
+    __shared__ float s_prefix[kFinishTile / kChunk];  // what is added to the block's chunks
+    if (!(head[0] > 0.0f)) return;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t first = blockIdx.x * (uint32_t)kFinishTile;
+    const uint32_t tile = first / (uint32_t)kChunkTile;
+    // final scanned total (level 1) of the chunk in front of chunk c is
+    //   scanned_chunk_totals[c - 1] + the scan of the tile totals (level 2) at tile(c - 1) - 1
+    if (tid < (uint32_t)kWave && tile > 0u) {
+        upper_totals(tile_totals, tile, s_a, s_b, tid);   // only the tiles in front matter
+        if (tid < 2u && tile > tid) s_front[tid] = blocked_scan_at(tile_totals, tile - 1u - tid, s_a, s_b);
+    }
+    __syncthreads();
+    if (tid < (uint32_t)(kFinishTile / kChunk)) {
+        const uint32_t c = first / (uint32_t)kChunk + tid;
+        float prefix = 0.0f;
+        if (c > 0u && (size_t)c * kChunk < n) {
+            const uint32_t before = c - 1u, its_tile = before / (uint32_t)kChunksPerBlock;
+            prefix = scanned_chunk_totals[before];
+            if (its_tile > 0u) prefix = s_front[tile - its_tile] + prefix;
+        }
+        s_prefix[tid] = prefix;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kFinishItems; ++k) {
+        const uint32_t offset = (uint32_t)k * kBlock + tid, i = first + offset;
+        if (i >= n) continue;
+        float v = data[i];
+        if (i >= (uint32_t)kChunk) {
+            v = s_prefix[offset / (uint32_t)kChunk] + v;
+            data[i] = v;
+        }
+        uint32_t lo = 0u, count = n, node = 1u;
+        for (int depth = 0; depth < levels; ++depth) {
+            const uint32_t step = count >> 1, it = lo + step;
+            if (it == i) {
+                head[node] = v;
+                break;
+            }
+            if (it < i) {
+                lo = it + 1u;
+                count -= step + 1u;
+                node = 2u * node + 1u;
+            } else {
+                count = step;
+                node = 2u * node;
+            }
+        }
+    }
 }
 
 // Every thread of the block must call it; ends with a barrier. s_tree[0] (the total) is not used.
@@ -735,52 +892,56 @@ int launch_blocked_total(const float* data, uint32_t n, float* totals, float* su
     uint32_t m = n;
     for (int lv = 0; lv < plan.n_levels; ++lv) {
         float* dst = (lv == plan.n_levels - 1) ? sum_out : totals + plan.offset[lv];
-        INPC_LAUNCH("chunk_reduce", k_chunk_pass<false>, dim3(div_up(m, kChunkTile)), dim3(kWave), stream,
-                    const_cast<float*>(cur), m, dst, (const float*)nullptr, (const float*)nullptr);
+        INPC_LAUNCH("chunk_reduce", k_chunk_totals, dim3(div_up(m, kChunkTile)), dim3(kWave), stream, cur, m, dst);
         cur = dst;
         m = plan.size[lv];
     }
     return INPC_OK;
 }
 
+// Scratch of the CDF passes for n leaves, in floats: the raw tile totals, the tile totals of the normalised weights
+// (each padded to whole chunks: the kernels fetch whole chunks) and the scanned chunk totals.
+struct CdfScratch {
+    uint32_t n_tiles;
+    size_t raw_tile_totals, tile_totals, scanned_chunk_totals;   // offsets in floats
+    size_t total_floats;
+};
+
+CdfScratch plan_cdf(uint32_t n) {
+    CdfScratch p{};
+    p.n_tiles = div_up(n, kChunkTile);
+    p.raw_tile_totals = 0;
+    p.tile_totals = align_up(p.n_tiles, kChunk);
+    p.scanned_chunk_totals = 2 * align_up(p.n_tiles, kChunk);
+    p.total_floats = p.scanned_chunk_totals + (size_t)p.n_tiles * kChunksPerBlock;
+    return p;
+}
+
 // Sum, normalisation and inclusive scan of the n leaf weights in place; the head of the CDF into sum_out.
-// `totals` is scratch of plan_levels(n).total_floats floats; every element that is read has been written
-// by an earlier launch of the same call, so it needs no clearing.
-int launch_build_cdf(float* w, float* sum_out, float* totals, uint32_t n_leaves, hipStream_t stream) {
-    const LevelPlan plan = plan_levels(n_leaves);
-    int rc = launch_blocked_total(w, n_leaves, totals, sum_out, plan, stream);
-    if (rc != INPC_OK) return rc;
-    // down: local scans, level 0 normalises; stops once a level has a single chunk
-    float* cur = w;
-    uint32_t m = n_leaves;
-    int depth = 0;
-    for (;;) {
-        float* tot = totals + plan.offset[depth];
-        INPC_LAUNCH("chunk_scan", k_chunk_pass<true>, dim3(div_up(m, kChunkTile)), dim3(kWave), stream, cur, m, tot,
-                    (const float*)sum_out, depth == 0 ? (const float*)sum_out : (const float*)nullptr);
-        if (plan.size[depth] == 1) break;
-        cur = tot;
-        m = plan.size[depth];
-        ++depth;
-    }
-    // up: add the scanned chunk totals of level d+1 to level d
-    for (int d = depth - 1; d >= 0; --d) {
-        float* dst = d == 0 ? w : totals + plan.offset[d - 1];
-        const uint32_t dn = d == 0 ? n_leaves : plan.size[d - 1];
-        INPC_LAUNCH("chunk_add_prefix", k_chunk_add_prefix, dim3(div_up(dn, kBlock)), dim3(kBlock), stream, dst, dn,
-                    (const float*)(totals + plan.offset[d]), (const float*)sum_out);
-    }
-    const uint32_t n_nodes = 1u << tree_levels(n_leaves);
-    INPC_LAUNCH("search_tree", k_build_search_tree, dim3(n_nodes / kBlock), dim3(kBlock), stream, (const float*)w, sum_out,
-                n_leaves, n_nodes);
+// `scratch` holds plan_cdf(n).total_floats floats; every element that is read has been written by an earlier launch
+// of the same call (or is not used), so it needs no clearing.
+int launch_build_cdf(float* w, float* sum_out, float* scratch, uint32_t n_leaves, hipStream_t stream) {
+    const CdfScratch plan = plan_cdf(n_leaves);
+    const int levels = tree_levels(n_leaves);
+    const uint32_t n_nodes = 1u << levels;
+    float* raw = scratch + plan.raw_tile_totals;
+    float* tile_totals = scratch + plan.tile_totals;
+    float* scanned = scratch + plan.scanned_chunk_totals;
+    INPC_LAUNCH("cdf_tile_totals", k_tile_totals, dim3(plan.n_tiles), dim3(kWave), stream, (const float*)w, n_leaves, raw,
+                sum_out + 1, n_nodes - 1u);
+    INPC_LAUNCH("cdf_scan_tiles", k_cdf_scan_tiles, dim3(plan.n_tiles), dim3(kWave), stream, w, n_leaves,
+                (const float*)raw, scanned, tile_totals, sum_out);
+    INPC_LAUNCH("cdf_finish", k_cdf_finish, dim3(div_up(n_leaves, kFinishTile)), dim3(kBlock), stream, w, n_leaves,
+                (const float*)scanned, (const float*)tile_totals, plan.n_tiles, sum_out, levels);
     return INPC_OK;
 }
 
 // ---- built-in scratch of inpc_build_cdf_static ------------------------------------------------------------------
-// Chunk totals for up to INPC_BUILD_CDF_STATIC_MAX_LEAVES leaves (levels of 65536, 1024, 64 and 64 floats). The
+// Scratch of the CDF passes for up to INPC_BUILD_CDF_STATIC_MAX_LEAVES leaves (1024 tiles: two arrays of 1024 tile
+// totals and 65536 scanned chunk totals). The
 // array's name is only a handle in host code: the address kernels can use comes from hipGetSymbolAddress,
 // once per device (every device holds its own copy).
-constexpr size_t kStaticTotalsFloats = 65536 + 1024 + 64 + 64;
+constexpr size_t kStaticTotalsFloats = 65536 + 1024 + 1024;
 __device__ __align__(256) float g_static_totals[kStaticTotalsFloats];
 
 constexpr int kMaxDevices = 64;
@@ -804,10 +965,16 @@ int static_totals(float*& out) {
 
 }  // namespace
 
+// Floats at the start of the workspace: the CDF passes and the expected-count sampler's sum share them.
+size_t sampler_scratch_floats(uint32_t n_leaves) {
+    const uint32_t n = std::max(n_leaves, 1u);
+    return std::max(plan_levels(n).total_floats, plan_cdf(n).total_floats);
+}
+
 size_t sampler_workspace_bytes(uint32_t n_leaves) {
-    const LevelPlan plan = plan_levels(std::max(n_leaves, 1u));
+    const size_t floats = sampler_scratch_floats(n_leaves);
     const uint32_t scan_blocks = div_up(std::max(n_leaves, 1u), kCountTile);
-    return align_up(plan.total_floats * 4, 256) + align_up((kScanHeaderWords + scan_blocks) * 4, 256) + 256;
+    return align_up(floats * 4, 256) + align_up((kScanHeaderWords + scan_blocks) * 4, 256) + 256;
 }
 
 }  // namespace inpc
@@ -847,6 +1014,9 @@ int inpc_build_cdf(float* w, float* sum_out, size_t head_floats, void* workspace
                    uint32_t n_leaves, void* stream_) {
     if (n_leaves == 0) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: no leaves");
     if (!w || !sum_out || !workspace) return fail(INPC_E_INVALID_ARGUMENT, "inpc_build_cdf: null pointer");
+    if (n_leaves > kMaxCdfLeaves)
+        return fail(INPC_E_UNSUPPORTED, "inpc_build_cdf: %u leaves exceed the %u the scan's levels hold", n_leaves,
+                    kMaxCdfLeaves);
     if (const int rc = check_head("inpc_build_cdf", head_floats, n_leaves); rc != INPC_OK) return rc;
     if (workspace_bytes < sampler_workspace_bytes(n_leaves))
         return fail(INPC_E_WORKSPACE, "inpc_build_cdf: workspace has %zu bytes, needs %zu", workspace_bytes,
@@ -860,7 +1030,7 @@ int inpc_build_cdf_static(float* w, float* sum_out, size_t head_floats, uint32_t
     if (n_leaves > INPC_BUILD_CDF_STATIC_MAX_LEAVES)
         return fail(INPC_E_UNSUPPORTED, "inpc_build_cdf_static: %u leaves exceed the %u the built-in scratch holds",
                     n_leaves, (unsigned)INPC_BUILD_CDF_STATIC_MAX_LEAVES);
-    if (plan_levels(n_leaves).total_floats > kStaticTotalsFloats)
+    if (plan_cdf(n_leaves).total_floats > kStaticTotalsFloats)
         return fail(INPC_E_UNSUPPORTED, "inpc_build_cdf_static: the built-in scratch is too small for %u leaves", n_leaves);
     if (const int rc = check_head("inpc_build_cdf_static", head_floats, n_leaves); rc != INPC_OK) return rc;
     float* totals = nullptr;
@@ -982,7 +1152,7 @@ int inpc_expected_counts(const float* weights, float* sum_out, int32_t* offsets_
     float* totals = (float*)workspace;
     int rc = launch_blocked_total(weights, n_leaves, totals, sum_out, plan, stream);
     if (rc != INPC_OK) return rc;
-    uint32_t* scan = (uint32_t*)((char*)workspace + align_up(plan.total_floats * 4, 256));
+    uint32_t* scan = (uint32_t*)((char*)workspace + align_up(sampler_scratch_floats(n_leaves) * 4, 256));
     const uint32_t n_blocks = div_up(n_leaves, kCountTile);
     rc = fill_u32(scan, 0u, kScanHeaderWords + n_blocks, stream);
     if (rc != INPC_OK) return rc;

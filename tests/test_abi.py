@@ -210,6 +210,9 @@ def test_a_cdf_head_that_is_too_small_is_refused_before_any_launch():
     assert lib.inpc_sample_cull_compact(p, p, p, short, p, p, p, 0, 1000, 0, 1000, n_leaves, C.byref(cam), p, p, 1 << 20,
                                         None) == -2
     assert b"inpc_cdf_head_floats" in lib.inpc_last_error()
+    # the scan keeps two levels of totals above a tile of 4096 leaves in LDS: 2^30 leaves at most
+    assert lib.inpc_build_cdf(p, p, 1 << 24, p, 1 << 34, (1 << 30) + 1, None) == -3
+    assert b"1073741824" in lib.inpc_last_error()
 
 
 def test_second_stream_policy():

@@ -54,6 +54,47 @@ def test_cdf_of_exact_integers_matches_cumsum(gpu):
     np.testing.assert_array_equal(cdf.cpu().numpy(), expect)
 
 
+def search_tree_of(cdf, n_nodes):
+    """The head of a CDF as the probe sequence of B/sampling/include/sampling_utils.h:49-69 defines it: node 1 is the
+    element the first probe reads, nodes 2k and 2k + 1 those of the probe after going left and right; 0 where a
+    search has ended before."""
+    n = len(cdf)
+    head = np.zeros(n_nodes, np.float32)
+    first, count = np.zeros(1, np.int64), np.full(1, n, np.int64)
+    depth = 0
+    while (1 << depth) < n_nodes:
+        nodes = (1 << depth) + np.arange(1 << depth)
+        live = count > 0
+        head[nodes[live]] = cdf[first[live] + count[live] // 2]
+        step = count // 2
+        left_first, left_count = first, np.where(live, step, 0)
+        right_first, right_count = first + step + 1, np.where(live, count - step - 1, 0)
+        first = np.stack([left_first, right_first], 1).reshape(-1)
+        count = np.stack([left_count, right_count], 1).reshape(-1)
+        depth += 1
+    return head
+
+
+@pytest.mark.parametrize("n_leaves", [1, 2, 100, 16383, 16384, 70001, 278528, 4194304 + 65, 16777216 + 4097],
+                         ids=lambda n: f"{n}leaves")
+def test_cdf_and_search_tree_against_their_definitions(gpu, oracle, n_leaves):
+    # the CDF against the oracle and the head against the probe sequence replayed on the indices, for octrees whose
+    # tile totals fill one chunk, several chunks (above 262,144 leaves) and more than 4096 (above 16,777,216 leaves:
+    # one more level of totals)
+    rng = np.random.default_rng(n_leaves)
+    w = np.exp(rng.normal(0.0, 1.0, size=n_leaves)).astype(np.float32)
+    w[rng.random(n_leaves) < 0.25] = 0.0
+    w[0] = 1.0
+    cdf, head = H.build_cdf(H.dev(w))
+    ok, cdf_ref, total_ref = oracle.build_cdf(w)
+    assert ok
+    cdf, head = cdf.cpu().numpy(), head.cpu().numpy()
+    np.testing.assert_array_equal(cdf.view(np.uint32), cdf_ref.view(np.uint32))
+    assert head[:1].view(np.uint32)[0] == np.float32(total_ref).view(np.uint32)
+    want = search_tree_of(cdf_ref, len(head))
+    np.testing.assert_array_equal(head[1:].view(np.uint32), want[1:].view(np.uint32))
+
+
 def test_sum_not_positive_leaves_weights_untouched(gpu):
     w = np.zeros(5000, dtype=np.float32)
     cdf, total = H.build_cdf(H.dev(w))

@@ -20,6 +20,10 @@ CASES = [
     ("test_gpu_sampler", "test_leaf_weights_and_cdf_bit_exact", dict(n_leaves=65, level=4)),
     ("test_gpu_sampler", "test_leaf_weights_and_cdf_bit_exact", dict(n_leaves=6000, level=6)),
     ("test_gpu_sampler", "test_leaf_weights_and_cdf_bit_exact", dict(n_leaves=300000, level=8)),
+    ("test_gpu_sampler", "test_cdf_and_search_tree_against_their_definitions", dict(n_leaves=2)),
+    ("test_gpu_sampler", "test_cdf_and_search_tree_against_their_definitions", dict(n_leaves=16384)),
+    ("test_gpu_sampler", "test_cdf_and_search_tree_against_their_definitions", dict(n_leaves=278528)),
+    ("test_gpu_sampler", "test_cdf_and_search_tree_against_their_definitions", dict(n_leaves=4194304 + 65)),
     ("test_gpu_sampler", "test_cdf_of_exact_integers_matches_cumsum", {}),
     ("test_gpu_sampler", "test_sum_not_positive_leaves_weights_untouched", {}),
     ("test_gpu_sampler", "test_sample_bit_exact_and_stream_continues", dict(n_samples=2049)),

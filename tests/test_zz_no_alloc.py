@@ -63,7 +63,7 @@ def test_static_scratch_matches_workspace_variant_on_two_calls_in_a_row(gpu):
 
 
 def test_static_scratch_at_its_largest_size(gpu):
-    # 4,194,304 leaves need 65536 + 1024 + 64 + 64 chunk totals: exactly what the scratch array holds
+    # 4,194,304 leaves are 1024 tiles: 2 x 1024 tile totals + 65536 scanned chunk totals, exactly what the scratch array holds
     _compare(MAX_LEAVES, 3)
 
 
