@@ -827,15 +827,22 @@ __global__ void __launch_bounds__(kBlock)
     }
 }
 
-// ids[offsets[l-1] .. offsets[l]) = l; one wave per 64 leaves, lanes stride over each leaf's run.
+// ids[offsets[l-1] .. offsets[l]) = l; one wave per 64 leaves, lanes stride over each leaf's run. The wave fetches its
+// 64 offsets with one load and hands them round (two dependent loads per leaf made the walk a chain of 128 round trips).
 __global__ void __launch_bounds__(kBlock) k_repeat_interleave(const int32_t* __restrict__ offsets,
                                                               int32_t* __restrict__ ids, uint32_t n_leaves) {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave_global = (blockIdx.x * kBlock + threadIdx.x) >> 6;
     const uint32_t l0 = wave_global * 64u;
-    for (uint32_t l = l0; l < min(l0 + 64u, n_leaves); ++l) {
-        const int32_t b = l == 0 ? 0 : offsets[l - 1], e = offsets[l];
-        for (int32_t i = b + (int32_t)lane; i < e; i += 64) ids[i] = (int32_t)l;
+    if (l0 >= n_leaves) return;   // the whole wave
+    const uint32_t n_here = min(64u, n_leaves - l0);
+    const int32_t mine = offsets[min(l0 + lane, n_leaves - 1u)];
+    const int32_t front = l0 == 0u ? 0 : offsets[l0 - 1u];
+    int32_t b = front;
+    for (uint32_t k = 0; k < n_here; ++k) {
+        const int32_t e = __shfl(mine, (int)k, 64);
+        for (int32_t i = b + (int32_t)lane; i < e; i += 64) ids[i] = (int32_t)(l0 + k);
+        b = e;
     }
 }
 
