@@ -38,6 +38,12 @@ WORKLOADS = {
                   describe="rasterizer fwd+bwd, 262,144 pts @640x400, C=8 fp32, 16x16 tiles (quick check)"),
 }
 
+# Sizes of the side measurements of `extra` (module-level so that tests/test_bench_dry_run.py can shrink them).
+DEVICE = "cuda:0"
+CONFIG0_POINTS = 65_536                     # BASELINE configuration 0: the reference's CPU-sized case
+FRAME_REQUESTED_SAMPLES = 8_388_352         # per sampling round of the reference's default inference frame
+CONFIG4 = dict(n=33_554_432, width=2473, height=1643, focal=2000.0, leaves=2_097_152, level=11)
+
 
 def algorithmic_bytes(kernel: str, n, v, i, pixels, channels, end_bit):
     """Algorithmic bytes that all launches of `kernel` in one step move together: every array of the reference's
@@ -124,7 +130,7 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     lib = _lib.lib()
-    device = torch.device("cuda:0")
+    device = torch.device(DEVICE)
     torch.cuda.set_device(device)
     wl = WORKLOADS[args.workload]
     n, channels, tile = wl["n"], wl["channels"], wl["tile"]
@@ -383,7 +389,7 @@ def main() -> int:
     try:
         if args.no_extras:
             raise RuntimeError("skipped (--no-extras)")
-        n0 = 65_536
+        n0 = CONFIG0_POINTS
         hv0 = synthetic.camera_on_z(256, 256, 300.0, 3.0)
         view0 = hv0.to_view(device)
         pos0_h = synthetic.cube_points(n0, 1.0, 0)
@@ -406,7 +412,7 @@ def main() -> int:
 
         forward0()
         gpu0_ms = time_calls(forward0, 10 * args.steps)
-        config0 = {"workload": "65,536 pts uniform in the unit cube, 4 fp32 channels, 256x256, f=300, distance 3, "
+        config0 = {"workload": f"{n0:,} pts uniform in the unit cube, 4 fp32 channels, 256x256, f=300, distance 3, "
                                "16x16 tiles, forward only",
                    "gpu_forward_ms": round(gpu0_ms, 4), "gpu_Mpoints_per_s": round(n0 / (gpu0_ms * 1e-3) / 1e6, 1)}
         if not args.no_cpu_baseline:
@@ -442,7 +448,7 @@ def main() -> int:
             raise RuntimeError("skipped (--no-extras)")
         from inpc_amd import INPCRasterizer
 
-        n_req, n_multi = 8_388_352, 4
+        n_req, n_multi = FRAME_REQUESTED_SAMPLES, 4
         frame_sampler = ProbabilityFieldSampler(seed=0)
         probe = frame_sampler.generate_expected_samples(centers, levels, weights, view, n_req, 1, oct.initial_size)
         n_created = int(probe.shape[0])
@@ -552,17 +558,17 @@ def main() -> int:
         # free the training workload first: this one needs about 12 GB
         del workspace, image, alpha, blending_weights, grad_features, grad_opacities, features, opacities
         torch.cuda.empty_cache()
-        n4, W4, H4 = 33_554_432, 2473, 1643
-        hv4 = synthetic.camera_on_z(W4, H4, 2000.0, 6.0)
+        n4, W4, H4 = CONFIG4["n"], CONFIG4["width"], CONFIG4["height"]
+        hv4 = synthetic.camera_on_z(W4, H4, CONFIG4["focal"], 6.0)
         view4 = hv4.to_view(device)
-        oct4 = synthetic.octree_leaves(2_097_152, 11, 4.0, seed=0)
+        oct4 = synthetic.octree_leaves(CONFIG4["leaves"], CONFIG4["level"], 4.0, seed=0)
         c4, l4, w4 = (torch.from_numpy(a).to(device) for a in (oct4.centers, oct4.levels, oct4.weights))
         sampler4 = ProbabilityFieldSampler(seed=0)
         pos4, _ = sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size)
         draw4_ms = time_calls(lambda: sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size), 5)
         feats4 = torch.randn((n4, 16), generator=gen, device=device, dtype=torch.float32).half()
         opac4 = torch.sigmoid(torch.randn(n4, generator=gen, device=device, dtype=torch.float32))
-        config4 = {"workload": "33,554,432 pts @2473x1643, 16 channels stored fp16, inference forward",
+        config4 = {"workload": f"{n4:,} pts @{W4}x{H4}, 16 channels stored fp16, inference forward",
                    "training_draw_ms": round(draw4_ms, 3)}
         from inpc_amd import rasterize_points
 

@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes as C
+import os
 
 
 def _aligned_bytes(n_bytes, device):
@@ -34,7 +35,7 @@ def simulated_device():
     from tests import helpers
     from tests.cpu_sim import build
 
-    path = build.build()
+    path = build.build(sanitize=os.environ.get("INPC_SIM_SANITIZE", "") not in ("", "0"))
     saved = (_lib._lib, _lib.LIB_PATH, _lib.current_stream, helpers.DEVICE, rasterization._new_workspace)
     _lib._lib, _lib.LIB_PATH = None, path
     _lib.current_stream = lambda: C.c_void_p(None)

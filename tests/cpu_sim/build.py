@@ -1,10 +1,22 @@
 """Builds the library's own sources (inpc_amd/csrc/*.hip) with g++ against the simulator's stand-in for the HIP
 runtime (tests/cpu_sim/hip/, tests/cpu_sim/sim.cpp) into tests/cpu_sim/libinpc_sim.so: the same C ABI, kernels run
 on the CPU one block after the other (see sim.hpp). TEST INFRASTRUCTURE ONLY: nothing of the product imports this,
-and the product itself still refuses to run without its HIP library."""
+and the product itself still refuses to run without its HIP library.
+
+`sanitize=True` (or `python tests/cpu_sim/build.py --sanitize`) builds libinpc_sim_asan.so with AddressSanitizer and
+UndefinedBehaviorSanitizer: every load and store of every kernel is then checked against the bounds of the buffer it
+lands in (the tensors of the tests are heap allocations) and against the alignment of its type (a float4 access needs
+16 bytes, as the 128-bit LDS and memory instructions do), every shift against the width of its operand, every signed
+operation against overflow; the first finding ends the process. The process has to start with the sanitizer's
+runtime preloaded:
+
+    LD_PRELOAD=$(gcc -print-file-name=libasan.so) ASAN_OPTIONS=detect_leaks=0 INPC_SIM_SANITIZE=1 \\
+        python -m pytest tests/test_sim_kernels.py -q
+"""
 from __future__ import annotations
 
 import subprocess
+import sys
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
@@ -12,42 +24,49 @@ HERE = Path(__file__).resolve().parent
 ROOT = HERE.parent.parent
 CSRC = ROOT / "inpc_amd" / "csrc"
 LIB = HERE / "libinpc_sim.so"
+LIB_SANITIZE = HERE / "libinpc_sim_asan.so"
 SOURCES = ["runtime.hip", "sampler.hip", "raster.hip", "field.hip", "misc.hip"]
-FLAGS = ["-x", "c++", "-std=c++17", "-O2", "-fPIC", "-ffp-contract=off", "-Wno-unknown-pragmas", f"-I{HERE}"]
+COMMON = ["-std=c++17", "-fPIC"]
+OPTIMIZE = ["-O2"]
+SANITIZE = ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"]
+KERNEL_FLAGS = ["-x", "c++", "-ffp-contract=off", "-Wno-unknown-pragmas", f"-I{HERE}"]
 
 
-def _stale() -> bool:
-    if not LIB.exists():
+def _stale(lib: Path) -> bool:
+    if not lib.exists():
         return True
-    built = LIB.stat().st_mtime
+    built = lib.stat().st_mtime
     deps = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.hpp")) + [ROOT / "include" / "inpc_hip.h", HERE / "sim.cpp",
                                                                   HERE / "sim.hpp", HERE / "hip" / "hip_runtime.h",
-                                                                  HERE / "hip" / "hip_fp16.h"]
+                                                                  HERE / "hip" / "hip_fp16.h", Path(__file__)]
     return any(d.stat().st_mtime > built for d in deps)
 
 
 def _compile(src: Path, obj: Path, flags: list[str]) -> None:
     done = subprocess.run(["g++", *flags, "-c", str(src), "-o", str(obj)], capture_output=True, text=True,
-                          stdin=subprocess.DEVNULL, timeout=1200)
+                          stdin=subprocess.DEVNULL, timeout=1800)
     if done.returncode != 0:
         raise RuntimeError(f"g++ failed on {src}:\n{done.stderr[-4000:]}")
 
 
-def build(force: bool = False) -> Path:
-    if not force and not _stale():
-        return LIB
-    objdir = HERE / "obj"
+def build(force: bool = False, sanitize: bool = False) -> Path:
+    lib = LIB_SANITIZE if sanitize else LIB
+    if not force and not _stale(lib):
+        return lib
+    mode = SANITIZE if sanitize else OPTIMIZE
+    objdir = HERE / ("obj_asan" if sanitize else "obj")
     objdir.mkdir(exist_ok=True)
-    jobs = [(CSRC / s, objdir / (Path(s).stem + ".o"), FLAGS) for s in SOURCES]
-    jobs.append((HERE / "sim.cpp", objdir / "sim.o", ["-std=c++17", "-O2", "-fPIC"]))
+    jobs = [(CSRC / s, objdir / (Path(s).stem + ".o"), [*COMMON, *mode, *KERNEL_FLAGS]) for s in SOURCES]
+    jobs.append((HERE / "sim.cpp", objdir / "sim.o", [*COMMON, *mode]))
     with ThreadPoolExecutor(max_workers=6) as pool:
         list(pool.map(lambda job: _compile(*job), jobs))
-    done = subprocess.run(["g++", "-shared", "-o", str(LIB), *[str(obj) for _, obj, _ in jobs]], capture_output=True,
-                          text=True, stdin=subprocess.DEVNULL, timeout=600)
+    link = ["g++", "-shared", *(["-fsanitize=address,undefined"] if sanitize else []), "-o", str(lib)]
+    done = subprocess.run([*link, *[str(obj) for _, obj, _ in jobs]], capture_output=True, text=True,
+                          stdin=subprocess.DEVNULL, timeout=600)
     if done.returncode != 0:
-        raise RuntimeError(f"linking {LIB} failed:\n{done.stderr[-4000:]}")
-    return LIB
+        raise RuntimeError(f"linking {lib} failed:\n{done.stderr[-4000:]}")
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(force=True))
+    print(build(force=True, sanitize="--sanitize" in sys.argv[1:]))
