@@ -8,7 +8,6 @@ import contextlib
 import importlib.util
 import json
 import sys
-import types
 from pathlib import Path
 
 import pytest
@@ -33,10 +32,10 @@ def bench_on_the_simulator(sim, monkeypatch):
     bench = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(bench)
     monkeypatch.setattr(bench, "DEVICE", "cpu")
-    monkeypatch.setattr(bench, "CONFIG0_POINTS", 6_000)
-    monkeypatch.setattr(bench, "FRAME_REQUESTED_SAMPLES", 20_000)
-    monkeypatch.setattr(bench, "CONFIG4", dict(n=40_000, width=247, height=164, focal=200.0, leaves=300_000, level=9))
-    monkeypatch.setitem(bench.WORKLOADS, "config3", dict(n=30_000, width=320, height=200, focal=250.0, channels=8,
+    monkeypatch.setattr(bench, "CONFIG0_POINTS", 3_000)
+    monkeypatch.setattr(bench, "FRAME_REQUESTED_SAMPLES", 8_000)
+    monkeypatch.setattr(bench, "CONFIG4", dict(n=12_000, width=123, height=82, focal=100.0, leaves=70_000, level=8))
+    monkeypatch.setitem(bench.WORKLOADS, "config3", dict(n=10_000, width=160, height=100, focal=125.0, channels=8,
                                                          tile=16, leaves=5000, level=6, describe="dry run"))
     for name, value in dict(is_available=lambda: True, set_device=lambda d: None, synchronize=lambda *a: None,
                             empty_cache=lambda: None, Stream=_Stream, stream=lambda s: contextlib.nullcontext(),
@@ -57,7 +56,7 @@ def bench_on_the_simulator(sim, monkeypatch):
 
 
 def test_every_leg_of_the_benchmark_runs(bench_on_the_simulator, monkeypatch, capsys):
-    monkeypatch.setattr(sys, "argv", ["bench.py", "--steps", "2", "--warmup", "1", "--cpu-seconds", "0.4"])
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--steps", "1", "--warmup", "1", "--cpu-seconds", "0.2"])
     assert bench_on_the_simulator.main() == 0
     out = capsys.readouterr()
     lines = [line for line in out.out.splitlines() if line.startswith("{")]
@@ -66,7 +65,7 @@ def test_every_leg_of_the_benchmark_runs(bench_on_the_simulator, monkeypatch, ca
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in record, key
-    assert record["n_gpus"] == 1 and record["steps"] == 2 and record["warmup"] == 1
+    assert record["n_gpus"] == 1 and record["steps"] == 1 and record["warmup"] == 1
     assert record["vs_baseline"] is None and record["dtype"] == "f32" and record["data"] == "synthetic"
     assert set(record["roofline"]) >= {"bound", "achieved", "peak", "unit", "frac", "traffic"}
     assert record["roofline"]["bound"] == "hbm" and record["roofline"]["peak"] == 8000.0
