@@ -240,7 +240,7 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     assert "python -m inpc_amd.build" in str(caught.value)
 
 
-def test_product_does_not_import_the_oracle():
+def test_product_does_not_import_the_oracle_or_the_simulator():
     code = ("import sys, inpc_amd, inpc_amd.sampling, inpc_amd.rasterization, inpc_amd.synthetic\n"
             "bad = [m for m in sys.modules if m == 'oracle' or m.startswith('oracle.')]\n"
             "sys.exit(1 if bad else 0)")
@@ -249,3 +249,8 @@ def test_product_does_not_import_the_oracle():
         if path.suffix in (".py", ".hip", ".hpp", ".h"):
             text = path.read_text()
             assert "oracle" not in text.lower() or path.name == "build.py", f"{path} mentions the oracle"
+            # nor of the CPU build of the kernels that the tests keep under tests/cpu_sim (test infrastructure too)
+            assert "cpu_sim" not in text and "libinpc_sim" not in text, f"{path} mentions the simulator"
+    for path in (ROOT / "bench.py", ROOT / "__graft_entry__.py", ROOT / "setup.py"):
+        text = path.read_text()
+        assert "cpu_sim" not in text and "libinpc_sim" not in text, f"{path} mentions the simulator"
