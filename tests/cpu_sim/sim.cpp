@@ -1,6 +1,10 @@
 // sim.cpp — fibers and meeting points of the SIMT simulator (see sim.hpp). x86-64 only.
 #include "sim.hpp"
 
+#include <cstdlib>
+#include <cstring>
+#include <utility>
+
 #include <cstdio>
 
 namespace sim {
@@ -120,6 +124,38 @@ const uint64_t* meet_block(uint64_t value, const uint64_t** members) {
     return slots;
 }
 
+// The order in which the scheduler resumes the fibers of a block between meeting points. Nothing a kernel computes may
+// depend on it: lanes that hand data to each other through memory have a meeting point (a barrier) in between. The
+// environment variable INPC_SIM_ORDER picks it: "forward" (thread 0 first, the default), "reverse", or "shuffle" (a new
+// pseudo-random order for every sweep); a kernel that relies on its lanes running in step or in thread order gives
+// different results under different orders.
+namespace {
+enum class Order { kForward, kReverse, kShuffle };
+Order thread_order() {
+    static const Order order = [] {
+        const char* v = std::getenv("INPC_SIM_ORDER");
+        if (v && std::strcmp(v, "reverse") == 0) return Order::kReverse;
+        if (v && std::strcmp(v, "shuffle") == 0) return Order::kShuffle;
+        return Order::kForward;
+    }();
+    return order;
+}
+
+void next_order(std::vector<uint32_t>& order, uint32_t n) {
+    static thread_local uint64_t state = 0x9E3779B97F4A7C15ull;
+    const Order mode = thread_order();
+    if (order.size() != n || mode == Order::kShuffle) {
+        order.resize(n);
+        for (uint32_t i = 0; i < n; ++i) order[i] = mode == Order::kReverse ? n - 1u - i : i;
+    }
+    if (mode == Order::kShuffle)
+        for (uint32_t i = n; i > 1; --i) {
+            state = state * 6364136223846793005ull + 1442695040888963407ull;
+            std::swap(order[i - 1], order[(uint32_t)((state >> 33) % i)]);
+        }
+}
+}  // namespace
+
 void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<void()> body) {
     const uint32_t n_threads = block_dim.x * block_dim.y * block_dim.z;
     if (n_threads == 0 || n_threads > (uint32_t)kMaxThreads) {
@@ -137,9 +173,14 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
     b.waves.resize((n_threads + 63) / 64);
     b.dynamic_lds.assign(dynamic_lds_bytes + 64, 0);
     b.body = std::move(body);
-    for (uint32_t bz = 0; bz < grid.z; ++bz)
-        for (uint32_t by = 0; by < grid.y; ++by)
-            for (uint32_t bx = 0; bx < grid.x; ++bx) {
+    static thread_local std::vector<uint32_t> order;
+    const bool blocks_reversed = thread_order() != Order::kForward;
+    for (uint32_t iz = 0; iz < grid.z; ++iz)
+        for (uint32_t iy = 0; iy < grid.y; ++iy)
+            for (uint32_t ix = 0; ix < grid.x; ++ix) {
+                // the blocks of a grid may run in any order: with the threads' order the blocks' is turned round too
+                const uint32_t bx = blocks_reversed ? grid.x - 1u - ix : ix, by = blocks_reversed ? grid.y - 1u - iy : iy,
+                               bz = blocks_reversed ? grid.z - 1u - iz : iz;
                 b.block_idx = Dim3(bx, by, bz);
                 b.block_meeting = Meeting{};
                 b.block_meeting.alive = n_threads;
@@ -158,7 +199,9 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
                 while (left) {
                     b.progress = false;
                     left = 0;
-                    for (uint32_t t = 0; t < n_threads; ++t) {
+                    next_order(order, n_threads);
+                    for (uint32_t k = 0; k < n_threads; ++k) {
+                        const uint32_t t = order[k];
                         Fiber& f = b.fibers[t];
                         if (f.done) continue;
                         g_fiber = &f;

@@ -3,7 +3,9 @@
 // Wave-level operations (ballot, shuffles, DPP, wave barriers) and block barriers are meeting points: a fiber that
 // reaches one waits there until all live fibers of its wave (block) have reached it, then all of them take their
 // results. Between meeting points the fibers of a wave run one after the other, not in lockstep: code that hands data
-// from lane to lane through memory has to have a wave barrier in between, as the kernels do.
+// from lane to lane through memory has to have a wave barrier in between, as the kernels do. The order in which the
+// fibers of a block (and the blocks of a grid) are resumed is the environment variable INPC_SIM_ORDER's: forward, reverse
+// or shuffle; the tests must pass under all three.
 // TEST INFRASTRUCTURE ONLY: it exists so that the kernels' logic can be run against the oracle where there is no GPU.
 #pragma once
 

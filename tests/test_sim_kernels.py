@@ -7,6 +7,10 @@ library's place and host memory as the device: the same C-ABI calls, the same or
 are chosen to finish in about two minutes together and to reach every kernel; `pytest tests -m gpu --sim` runs all
 of the GPU tests this way (about ten minutes).
 
+INPC_SIM_ORDER=reverse or =shuffle in the environment makes the simulator resume the threads of a block (and the
+blocks of a grid) in another order: a kernel whose lanes hand data to each other without a barrier, or that relies on
+the order of its blocks, then gives other results; all cases pass under all three orders.
+
 This shows the kernels' indexing, arithmetic and synchronisation right or wrong. It says nothing about speed and
 nothing about what only the hardware does (scheduling of blocks against each other, memory ordering between blocks,
 register and LDS limits): the `gpu` tests stay the parity tests proper."""
