@@ -8,7 +8,7 @@
 //   k_sample              multinomial leaf pick + jitter  (B/sampling/src/sampling_kernels.cu:128-150)
 //   k_sample_cull         the same draw, frustum test, ordered stream compaction
 //                                                         (B/sampling/src/sampling_kernels.cu:77-126)
-//   k_expected_counts / k_repeat_interleave / k_expected_samples
+//   k_tile_totals + k_expected_counts / k_repeat_interleave / k_expected_samples
 //                                                         (B/sampling/src/sampling_kernels.cu:152-205)
 //
 // Candidate k always uses the sampler's generator advanced by 4*k draws. A thread walks candidates
@@ -163,24 +163,6 @@ __device__ __forceinline__ float blocked_scan_at(const float* values, uint32_t j
     if (ca == 0u) return local_a + local0;
     const float final_b = chunk_sum(s_b, ca);   // scan of s_b at ca - 1: s_b is a single chunk
     return (final_b + local_a) + local0;
-}
-
-// totals[c] = data[64 c] + ... + data[64 c + 63], left to right: one level of a sum (the expected-count sampler's).
-__global__ void __launch_bounds__(kWave) k_chunk_totals(const float* __restrict__ data, uint32_t n,
-                                                        float* __restrict__ totals) {
-    __shared__ float tile[kChunksPerBlock * (kChunk + 1)];
-    const uint32_t lane = threadIdx.x;
-    const size_t base = (size_t)blockIdx.x * kChunkTile;
-    stage_tile(tile, data, base, n, 1.0f, lane);
-    __syncthreads();
-    const size_t chunk_base = base + (size_t)lane * kChunk;
-    if (chunk_base < n) {
-        const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
-        const float* row = tile + lane * (kChunk + 1);
-        float s = row[0];
-        for (int i = 1; i < len; ++i) s += row[i];
-        totals[(size_t)blockIdx.x * kChunksPerBlock + lane] = s;
-    }
 }
 
 // Level 1 and 2 of a sum: tile_totals[b] = total of tile b's chunk totals. Totals only, `data` is not written.
@@ -785,15 +767,33 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
     return wave_base + incl - v;
 }
 
-// counts + inclusive integer scan in one pass (thread owns 4 consecutive leaves).
+// counts + inclusive integer scan in one pass (thread owns 4 consecutive leaves). The sum of the weights is what
+// k_tile_totals left, added up by every block itself (64 values for 262,144 leaves: less than a launch costs);
+// *sum_out receives it. A sum that is not positive leaves all offsets at zero.
 __global__ void __launch_bounds__(kBlock)
-    k_expected_counts(const float* __restrict__ weights, const float* __restrict__ sum_dev,
-                      int32_t* __restrict__ offsets, uint32_t n_samples, uint32_t n_leaves, ScanState* st,
-                      uint32_t* status) {
+    k_expected_counts(const float* __restrict__ weights, const float* __restrict__ raw_tile_totals, uint32_t n_tiles,
+                      float* __restrict__ sum_out, int32_t* __restrict__ offsets, uint32_t n_samples, uint32_t n_leaves,
+                      ScanState* st, uint32_t* status) {
+    __shared__ float s_a[kMaxUpperValues / kChunk];
+    __shared__ float s_b[kChunk];
+    __shared__ float s_sum;
     __shared__ uint32_t s_bid, s_exclusive;
     __shared__ uint32_t s_wave[kBlock / kWave];
-    const float sum = *sum_dev;
-    if (!(sum > 0.0f)) return;
+    if (threadIdx.x < (uint32_t)kWave) {
+        upper_totals(raw_tile_totals, n_tiles, s_a, s_b, threadIdx.x);
+        const float total = blocked_total(n_tiles, s_b);
+        if (threadIdx.x == 0) s_sum = total;
+    }
+    __syncthreads();
+    const float sum = s_sum;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *sum_out = sum;
+    if (!(sum > 0.0f)) {
+        for (int j = 0; j < kCountItems; ++j) {
+            const size_t l = (size_t)blockIdx.x * kCountTile + (size_t)j * kBlock + threadIdx.x;
+            if (l < n_leaves) offsets[l] = 0;
+        }
+        return;
+    }
     if (threadIdx.x == 0) s_bid = atomicAdd(&st->ticket, 1u);
     __syncthreads();
     const uint32_t bid = s_bid;
@@ -869,43 +869,6 @@ __global__ void __launch_bounds__(kBlock)
     }
 }
 
-// Chunk-total levels for n leaves: sizes n1 = ceil(n/64), n2 = ceil(n1/64), ... down to 1.
-struct LevelPlan {
-    int n_levels;
-    uint32_t size[8];
-    size_t offset[8];  // in floats, from the start of the totals area
-    size_t total_floats;
-};
-
-LevelPlan plan_levels(uint32_t n) {
-    LevelPlan p{};
-    uint32_t m = n;
-    size_t off = 0;
-    do {
-        m = div_up(m, kChunk);
-        p.size[p.n_levels] = m;
-        p.offset[p.n_levels] = off;
-        off += align_up(m, 64);
-        ++p.n_levels;
-    } while (m > 1 && p.n_levels < 8);
-    p.total_floats = off;
-    return p;
-}
-
-// Canonical total of `data` (n floats) into *sum_out; `totals` is scratch of plan.total_floats.
-int launch_blocked_total(const float* data, uint32_t n, float* totals, float* sum_out, const LevelPlan& plan,
-                         hipStream_t stream) {
-    const float* cur = data;
-    uint32_t m = n;
-    for (int lv = 0; lv < plan.n_levels; ++lv) {
-        float* dst = (lv == plan.n_levels - 1) ? sum_out : totals + plan.offset[lv];
-        INPC_LAUNCH("chunk_reduce", k_chunk_totals, dim3(div_up(m, kChunkTile)), dim3(kWave), stream, cur, m, dst);
-        cur = dst;
-        m = plan.size[lv];
-    }
-    return INPC_OK;
-}
-
 // Scratch of the CDF passes for n leaves, in floats: the raw tile totals, the tile totals of the normalised weights
 // (each padded to whole chunks: the kernels fetch whole chunks) and the scanned chunk totals.
 struct CdfScratch {
@@ -973,10 +936,7 @@ int static_totals(float*& out) {
 }  // namespace
 
 // Floats at the start of the workspace: the CDF passes and the expected-count sampler's sum share them.
-size_t sampler_scratch_floats(uint32_t n_leaves) {
-    const uint32_t n = std::max(n_leaves, 1u);
-    return std::max(plan_levels(n).total_floats, plan_cdf(n).total_floats);
-}
+size_t sampler_scratch_floats(uint32_t n_leaves) { return plan_cdf(std::max(n_leaves, 1u)).total_floats; }
 
 size_t sampler_workspace_bytes(uint32_t n_leaves) {
     const size_t floats = sampler_scratch_floats(n_leaves);
@@ -1153,20 +1113,20 @@ int inpc_expected_counts(const float* weights, float* sum_out, int32_t* offsets_
     hipStream_t stream = (hipStream_t)stream_;
     if (n_leaves == 0 || !weights || !sum_out || !offsets_out || !workspace)
         return fail(INPC_E_INVALID_ARGUMENT, "inpc_expected_counts: null pointer or no leaves");
+    if (n_leaves > kMaxCdfLeaves)
+        return fail(INPC_E_UNSUPPORTED, "inpc_expected_counts: %u leaves exceed the %u the sum's levels hold", n_leaves,
+                    kMaxCdfLeaves);
     if (workspace_bytes < sampler_workspace_bytes(n_leaves))
         return fail(INPC_E_WORKSPACE, "inpc_expected_counts: workspace too small");
-    const LevelPlan plan = plan_levels(n_leaves);
-    float* totals = (float*)workspace;
-    int rc = launch_blocked_total(weights, n_leaves, totals, sum_out, plan, stream);
-    if (rc != INPC_OK) return rc;
-    uint32_t* scan = (uint32_t*)((char*)workspace + align_up(sampler_scratch_floats(n_leaves) * 4, 256));
+    const CdfScratch plan = plan_cdf(n_leaves);
+    float* raw = (float*)workspace + plan.raw_tile_totals;
+    uint32_t* scan = (uint32_t*)((char*)workspace + align_up(plan.total_floats * 4, 256));
     const uint32_t n_blocks = div_up(n_leaves, kCountTile);
-    rc = fill_u32(scan, 0u, kScanHeaderWords + n_blocks, stream);
-    if (rc != INPC_OK) return rc;
-    rc = fill_u32(offsets_out, 0u, n_leaves, stream);  // sum <= 0 leaves all offsets at zero
-    if (rc != INPC_OK) return rc;
-    INPC_LAUNCH("expected_counts", k_expected_counts, dim3(n_blocks), dim3(kBlock), stream, weights,
-                (const float*)sum_out, offsets_out, n_samples, n_leaves, (ScanState*)scan, scan + kScanHeaderWords);
+    // the tile totals of the weights, and the state of the scan cleared on the way
+    INPC_LAUNCH("tile_totals", k_tile_totals, dim3(plan.n_tiles), dim3(kWave), stream, weights, n_leaves, raw,
+                (float*)scan, (uint32_t)kScanHeaderWords + n_blocks);
+    INPC_LAUNCH("expected_counts", k_expected_counts, dim3(n_blocks), dim3(kBlock), stream, weights, (const float*)raw,
+                plan.n_tiles, sum_out, offsets_out, n_samples, n_leaves, (ScanState*)scan, scan + kScanHeaderWords);
     return INPC_OK;
 }
 

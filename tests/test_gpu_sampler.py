@@ -281,6 +281,32 @@ def test_generate_samples_and_expected_samples_api(gpu, oracle):
     assert sampler.rng_state() == (int(rng_ref.state[0]), int(rng_ref.state[1]))
 
 
+def test_expected_counts_without_a_positive_sum_are_all_zero(gpu):
+    # no weight is positive (B/sampling/src/sampling_api.cu:196-199 returns no samples then): every offset is written
+    # as zero whatever the buffers held before, the sum is reported, and the next call with weights works as usual
+    lib = _lib.lib()
+    n = 70001
+    ws_bytes = lib.inpc_sampler_workspace_bytes(n)
+    ws = H.poisoned_bytes(ws_bytes, gpu)
+    offsets = torch.full((n,), 12345, dtype=torch.int32, device=gpu)
+    total = torch.full((1,), 7.0, dtype=torch.float32, device=gpu)
+    zeros = torch.zeros(n, dtype=torch.float32, device=gpu)
+    _lib.check(lib.inpc_expected_counts(_lib.ptr(zeros), _lib.ptr(total), _lib.ptr(offsets), 1000, _lib.ptr(ws), ws_bytes,
+                                        n, H.stream()), "inpc_expected_counts")
+    assert float(total.item()) == 0.0
+    assert int(offsets.abs().max().item()) == 0
+    w = np.zeros(n, np.float32)
+    w[[5, 4096, 70000]] = [1.0, 2.0, 1.0]
+    w_dev = H.dev(w)   # kept alive over the call
+    _lib.check(lib.inpc_expected_counts(_lib.ptr(w_dev), _lib.ptr(total), _lib.ptr(offsets), 1000, _lib.ptr(ws),
+                                        ws_bytes, n, H.stream()), "inpc_expected_counts")
+    assert float(total.item()) == 4.0
+    got = offsets.cpu().numpy()
+    want = np.zeros(n, np.int64)
+    want[5:], want[4096:], want[70000:] = 250, 750, 1000
+    np.testing.assert_array_equal(got, want)
+
+
 def test_non_perspective_and_distorted_cameras_are_rejected(gpu):
     from inpc_amd import ProbabilityFieldSampler, compute_viewpoint_weights
     from inpc_amd.views import View

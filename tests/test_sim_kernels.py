@@ -41,6 +41,7 @@ CASES = [
     ("test_gpu_sampler", "test_training_api_draw_of_several_rounds", {}),
     ("test_gpu_sampler", "test_training_api_failure_pattern", {}),
     ("test_gpu_sampler", "test_generate_samples_and_expected_samples_api", {}),
+    ("test_gpu_sampler", "test_expected_counts_without_a_positive_sum_are_all_zero", {}),
     ("test_gpu_sampler", "test_training_draw_that_never_hits_the_frustum_is_filled_with_the_failure_pattern", {}),
     # ---- bilinear rasterizer
     ("test_gpu_raster", "test_forward_direct_f32", dict(tile=8, channels=4)),
