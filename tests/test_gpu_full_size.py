@@ -14,7 +14,7 @@ from inpc_amd import ProbabilityFieldSampler, _lib, synthetic
 from tests import helpers as H
 from tests.test_gpu_raster import check_structure, oracle_cfg
 
-pytestmark = [pytest.mark.gpu, pytest.mark.real_gpu]
+pytestmark = pytest.mark.gpu
 
 RTOL = 1e-4
 
@@ -172,6 +172,7 @@ def test_config3_points_gaussian_footprint_full_size(config1, oracle):
     np.testing.assert_array_equal(go2.view(np.uint32), go.view(np.uint32))
 
 
+@pytest.mark.real_gpu   # 33,554,432 points: hours in the simulator
 def test_config4_large_frame_inference(gpu, oracle):
     """2,097,152 leaves of the level-11 grid, 33,554,432 samples, 16 channels stored as fp16, 2473x1643, f = 2000,
     16x16 tiles: sampling + inference forward end to end."""
