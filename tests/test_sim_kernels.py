@@ -5,7 +5,7 @@ threads of a block are fibers and a wave's ballots, shuffles, DPP moves and barr
 below is a test function of one of the GPU test modules, called with the simulator's library loaded in the HIP
 library's place and host memory as the device: the same C-ABI calls, the same oracle, the same tolerances. The cases
 are chosen to finish in about two minutes together and to reach every kernel; `pytest tests -m gpu --sim` runs all
-of the GPU tests this way (about ten minutes).
+of the GPU tests this way (about forty minutes, most of it the full-size configurations of test_gpu_full_size.py).
 
 INPC_SIM_ORDER=reverse or =shuffle in the environment makes the simulator resume the threads of a block (and the
 blocks of a grid) in another order: a kernel whose lanes hand data to each other without a barrier, or that relies on
