@@ -1,6 +1,7 @@
 // hip/hip_runtime.h of the tests' SIMT simulator: what the library's sources use of HIP, for a plain C++ compiler.
-// Kernels run on the CPU through sim::launch (sim.hpp); "device" pointers are host pointers; streams and events do
-// nothing (every launch has run when the call returns). TEST INFRASTRUCTURE ONLY, never part of the product's build.
+// Kernels run on the CPU through sim::launch (sim.hpp); "device" pointers are host pointers; streams do nothing
+// (every launch has run when the call returns) and an event is the host's clock when it is recorded.
+// TEST INFRASTRUCTURE ONLY, never part of the product's build.
 #pragma once
 
 #include <algorithm>
