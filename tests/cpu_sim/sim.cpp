@@ -171,7 +171,7 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
     b.n_threads = n_threads;
     if (b.fibers.size() < n_threads) b.fibers.resize(n_threads);
     b.waves.resize((n_threads + 63) / 64);
-    b.dynamic_lds.assign(dynamic_lds_bytes + 64, 0);
+    b.dynamic_lds.resize(dynamic_lds_bytes + 64);
     b.body = std::move(body);
     static thread_local std::vector<uint32_t> order;
     const bool blocks_reversed = thread_order() != Order::kForward;
@@ -182,6 +182,8 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
                 const uint32_t bx = blocks_reversed ? grid.x - 1u - ix : ix, by = blocks_reversed ? grid.y - 1u - iy : iy,
                                bz = blocks_reversed ? grid.z - 1u - iz : iz;
                 b.block_idx = Dim3(bx, by, bz);
+                // LDS holds what the block before left there, or anything: a kernel that counts on zeros shows up
+                std::memset(b.dynamic_lds.data(), 0xCD, b.dynamic_lds.size());
                 b.block_meeting = Meeting{};
                 b.block_meeting.alive = n_threads;
                 for (size_t w = 0; w < b.waves.size(); ++w) {
