@@ -7,7 +7,8 @@ and the product itself still refuses to run without its HIP library.
 UndefinedBehaviorSanitizer: every load and store of every kernel is then checked against the bounds of the buffer it
 lands in (the tensors of the tests are heap allocations) and against the alignment of its type (a float4 access needs
 16 bytes, as the 128-bit LDS and memory instructions do), every shift against the width of its operand, every signed
-operation against overflow; the first finding ends the process. The process has to start with the sanitizer's
+operation against overflow, every conversion of a float to an integer against the integer's range (where x86 and the
+GPU give different results); the first finding ends the process. The process has to start with the sanitizer's
 runtime preloaded:
 
     LD_PRELOAD=$(gcc -print-file-name=libasan.so) ASAN_OPTIONS=detect_leaks=0 INPC_SIM_SANITIZE=1 \\
@@ -28,7 +29,7 @@ LIB_SANITIZE = HERE / "libinpc_sim_asan.so"
 SOURCES = ["runtime.hip", "sampler.hip", "raster.hip", "field.hip", "misc.hip"]
 COMMON = ["-std=c++17", "-fPIC"]
 OPTIMIZE = ["-O2"]
-SANITIZE = ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"]
+SANITIZE = ["-O1", "-g", "-fsanitize=address,undefined,float-cast-overflow", "-fno-sanitize-recover=undefined,float-cast-overflow", "-fno-omit-frame-pointer"]
 KERNEL_FLAGS = ["-x", "c++", "-ffp-contract=off", "-Wno-unknown-pragmas", f"-I{HERE}"]
 
 

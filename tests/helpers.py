@@ -237,7 +237,8 @@ class RasterRun:
         top = (head_u[:, 6] >> 16).astype(np.int64) - 1
         for axis, first, w0, w1 in ((0, left, head[:, 0], head[:, 1]), (1, top, head[:, 2], head[:, 3])):
             s_ = geo[:, axis]
-            expect_first = np.floor((s_ - np.float32(0.5)).astype(np.float32)).astype(np.int64)
+            with np.errstate(invalid="ignore"):   # points that are not drawn may have any screen position
+                expect_first = np.floor((s_ - np.float32(0.5)).astype(np.float32)).astype(np.int64)
             assert (first[drawn] == expect_first[drawn]).all(), "left / top candidate pixel of a record is wrong"
             for k, w in ((0, w0), (1, w1)):
                 d = np.abs(s_ - ((first + k).astype(np.float32) + np.float32(0.5))).astype(np.float32)
@@ -484,3 +485,23 @@ def assert_close(actual, expected, rtol=1e-4, atol=1e-6, what=""):
         raise AssertionError(f"{what}: {int(bad.sum())} of {bad.size} elements differ; worst at {idx}: "
                              f"{actual[idx]!r} vs {expected[idx]!r} (|err|={err[idx]:.3e}); "
                              f"non-finite: {int((~np.isfinite(actual)).sum())}")
+
+
+def extreme_positions(hv, n, seed):
+    """Points of a cube around the origin of which four tenths are extreme: a coordinate that is NaN, infinite, huge
+    (1e30, 3e38) or denormal-small, and depths on, just inside and just outside zero and the two clipping planes."""
+    from inpc_amd import synthetic
+
+    rng = np.random.default_rng(seed)
+    pos = synthetic.cube_points(n, 2.0, seed)
+    k = max(1, n // 10)
+    order = rng.permutation(n)
+    specials = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 3e38, 1e-30, -1e-30, 0.0], np.float32)
+    for j in range(3):
+        chosen = order[j * k:(j + 1) * k]
+        pos[chosen, rng.integers(0, 3, len(chosen))] = specials[rng.integers(0, len(specials), len(chosen))]
+    chosen = order[3 * k:4 * k]
+    depths = np.array([0.0, 1e-9, -1e-9, 0.01, 0.0099999, 0.0100001, 100.0, 99.9999, 100.0001], np.float32)
+    # synthetic.camera_on_z looks along +z from (0, 0, -distance): camera-space depth = z - position.z
+    pos[chosen, 2] = (rng.choice(depths, len(chosen)) + np.float32(hv.position[2])).astype(np.float32)
+    return pos

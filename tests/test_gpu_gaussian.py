@@ -222,6 +222,33 @@ def test_backward_direct(gpu, oracle, mode):
     H.assert_close(go, go_ref, RTOL, grad_atol(go_ref), "opacity gradients")
 
 
+@pytest.mark.parametrize("seed,n,width,height,tile", [(71001, 20000, 233, 151, 8), (71002, 2000, 37, 211, 16)])
+def test_non_finite_and_extreme_positions(gpu, oracle, seed, n, width, height, tile):
+    # as for the bilinear footprint: NaN, infinite, huge and denormal coordinates, depths on and next to zero and the
+    # clipping planes (a depth next to zero makes a footprint of the whole image: kernels.cu:62-70 clamps the bounds)
+    channels = 4
+    hv = synthetic.camera_on_z(width, height, 120.0, 2.2)
+    pos = H.extreme_positions(hv, n, seed)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", seed + 1)
+    g, ref = oracle_run(oracle, hv, pos, feats, opac, tile, channels)
+    run = H.GaussianRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32,
+                        max_instances=max(int(ref["n_instances"]) + 1024, 4 * n)).forward()
+    check_structure(run.debug(), ref)
+    assert 0 < ref["n_visible"] < n
+    out = run.outputs()
+    assert np.isfinite(out["image"]).all()
+    H.assert_close(out["image"], ref["image"], RTOL, 2e-5, "image")
+    rng = np.random.default_rng(seed)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _, audit = oracle.raster_backward(g.base, gi, ga, ref["image"], ref["alpha"], pos, feats, opac, hv.w2c,
+                                                      gaussian=g, audit=True)
+    assert np.isfinite(gf).all() and np.isfinite(go).all()
+    H.assert_gradient_close(gf, audit, "view", "feature gradients")
+    H.assert_gradient_close(go, audit, "opacity", "opacity gradients")
+
+
 @pytest.mark.parametrize("with_scales", [False, True])
 @pytest.mark.parametrize("tile", [8, 16])
 def test_inference_preextracted(gpu, oracle, tile, with_scales):

@@ -223,6 +223,34 @@ def test_edge_cases(gpu, oracle, tile):
     compare(np.stack([wx, wy, np.full_like(wx, z)], 1), "pixel / tile boundaries")
 
 
+@pytest.mark.parametrize("seed,n,width,height,tile,channels", [(70001, 20000, 233, 151, 8, 8), (70002, 2000, 37, 211, 16, 4),
+                                                              (70003, 50, 15, 19, 16, 8)])
+def test_non_finite_and_extreme_positions(gpu, oracle, seed, n, width, height, tile, channels):
+    # NaN, infinite, huge and denormal coordinates, depths on and next to zero and the clipping planes: such points are
+    # culled or drawn exactly as the oracle does it (the comparisons of kernels.cu:52-60 with NaN false), nothing
+    # overflows a conversion to an integer, and the gradients of the points that are drawn are unaffected
+    hv = synthetic.camera_on_z(width, height, 120.0, 2.2)
+    pos = H.extreme_positions(hv, n, seed)
+    feats, opac = synthetic.point_attributes(n, channels, "normal", seed + 1)
+    run = H.RasterRun(hv, pos, feats, opac, tile, channels, _lib.FEAT_DIRECT_F32).forward()
+    cfg = oracle_cfg(oracle, hv, n, tile, channels, oracle.FEAT_DIRECT_F32)
+    ref = oracle.raster_forward(cfg, pos, feats, opac, hv.w2c, debug=True)
+    check_structure(run.debug(), ref)
+    assert 0 < ref["n_visible"] < n
+    out = run.outputs()
+    assert np.isfinite(out["image"]).all()
+    H.assert_close(out["image"], ref["image"], RTOL, 2e-5, "image")
+    H.assert_close(out["alpha"], ref["alpha"], RTOL, 1e-6, "alpha")
+    rng = np.random.default_rng(seed)
+    gi = rng.normal(0, 1e-2, ref["image"].shape).astype(np.float32)
+    ga = rng.normal(0, 1e-2, ref["alpha"].shape).astype(np.float32)
+    gf, go = run.backward(gi, ga)
+    gf_ref, go_ref, _ = oracle.raster_backward(cfg, gi, ga, out["image"], out["alpha"], pos, feats, opac, hv.w2c)
+    assert np.isfinite(gf).all() and np.isfinite(go).all()
+    H.assert_close(gf, gf_ref, RTOL, 2e-7, "feature gradients")
+    H.assert_close(go, go_ref, RTOL, 2e-6, "opacity gradients")
+
+
 @pytest.mark.parametrize("tile", [8, 16])
 @pytest.mark.parametrize("levels", [40000, 2500, 400, 30], ids=lambda v: f"{v}depths")
 def test_runs_of_equal_depth_keys(gpu, oracle, tile, levels):

@@ -58,6 +58,8 @@ CASES = [
     ("test_gpu_raster", "test_inference_direct_f16_16_channels", {}),
     ("test_gpu_raster", "test_edge_cases", dict(tile=8)),
     ("test_gpu_raster", "test_edge_cases", dict(tile=16)),
+    ("test_gpu_raster", "test_non_finite_and_extreme_positions",
+     dict(seed=70002, n=2000, width=37, height=211, tile=16, channels=4)),
     ("test_gpu_raster", "test_runs_of_equal_depth_keys", dict(tile=16, levels=400)),
     ("test_gpu_raster", "test_runs_of_equal_depth_keys", dict(tile=8, levels=30)),
     ("test_gpu_raster", "test_instances_beyond_the_capacity_are_reported_and_nothing_is_drawn", {}),
@@ -77,6 +79,7 @@ CASES = [
     ("test_gpu_gaussian", "test_inference_preextracted", dict(tile=16, with_scales=True)),
     ("test_gpu_gaussian", "test_inference_raw37", {}),
     ("test_gpu_gaussian", "test_edge_cases", {}),
+    ("test_gpu_gaussian", "test_non_finite_and_extreme_positions", dict(seed=71002, n=2000, width=37, height=211, tile=16)),
     ("test_gpu_gaussian", "test_instances_beyond_the_capacity_are_reported", {}),
     ("test_gpu_gaussian", "test_random_scenes_forward_backward", dict(case=201)),
     ("test_gpu_gaussian", "test_random_scenes_forward_backward", dict(case=205)),   # footprints of hundreds of pixels
