@@ -1,4 +1,4 @@
-"""bench.py from end to end without a GPU: every leg of it (the timed step, the roofline and CPU-baseline objects, the
+"""bench.py and __graft_entry__.smoke() from end to end without a GPU: every leg of it (the timed step, the roofline and CPU-baseline objects, the
 sampler draw, the other tile size, the Gaussian footprint, the reference-shaped autograd step, configuration 0, the
 inference frame, configuration 4) runs once on shrunken sizes through the kernels compiled for the CPU simulator of
 tests/cpu_sim, with a stand-in for the few torch.cuda calls the script makes. The figures mean nothing here (the
@@ -80,6 +80,17 @@ def test_every_leg_of_the_benchmark_runs(bench_on_the_simulator, monkeypatch, ca
     assert extra["other_tile_size"]["max_abs_image_difference"] < 1e-5
     assert extra["config4_inference"]["bilinear_abi"]["roofline"]["kernel"]
     assert {"sample_cull_compact", "cdf_tile_totals", "cdf_scan_tiles", "cdf_finish"} <= set(extra["sampler"]["kernel_ms"])
+
+
+def test_smoke_runs(sim, monkeypatch, capsys):
+    """__graft_entry__.smoke(), the check that runs on the GPU box before the benchmark, through the simulator."""
+    spec = importlib.util.spec_from_file_location("graft_entry_dry_run", ROOT / "__graft_entry__.py")
+    entry = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(entry)
+    monkeypatch.setattr(entry, "SMOKE_DEVICE", "cpu")
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    entry.smoke()
+    assert "smoke ok" in capsys.readouterr().out
 
 
 def test_more_than_one_gpu_is_refused(monkeypatch, capsys):
