@@ -1,5 +1,5 @@
-"""bench.py and __graft_entry__.smoke() from end to end without a GPU: every leg of it (the timed step, the roofline and CPU-baseline objects, the
-sampler draw, the other tile size, the Gaussian footprint, the reference-shaped autograd step, configuration 0, the
+"""bench.py and __graft_entry__.smoke() from end to end without a GPU. Every leg of the benchmark (the timed step, the
+roofline and CPU-baseline objects, the sampler draw, the other tile size, the Gaussian footprint, the reference-shaped autograd step, configuration 0, the
 inference frame, configuration 4) runs once on shrunken sizes through the kernels compiled for the CPU simulator of
 tests/cpu_sim, with a stand-in for the few torch.cuda calls the script makes. The figures mean nothing here (the
 simulator is thousands of times slower than the device); what is checked is that the script runs, prints its one JSON
