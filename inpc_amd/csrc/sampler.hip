@@ -135,6 +135,23 @@ __device__ __forceinline__ float chunk_sum(const float* values, uint32_t len) {
     return s;
 }
 
+// The same additions with every partial sum written back: values[i] = values[0] + ... + values[i] for i < len; returns
+// the last one. One round of loads, the additions in registers, one round of stores (a load and a store per step kept
+// the chain waiting on LDS 64 times).
+__device__ __forceinline__ float chunk_scan(float* values, uint32_t len) {
+    float v[kChunk];
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) v[i] = values[i];
+    float s = v[0];
+#pragma unroll
+    for (int i = 1; i < kChunk; ++i)
+        if ((uint32_t)i < len) {
+            s += v[i];
+            values[i] = s;
+        }
+    return s;
+}
+
 // The totals of `m` values one and two levels up, by one wave: s_a[k] = total of chunk k of `values` (k < ceil(m / 64)
 // <= 4096), s_b[k] = total of chunk k of s_a. Ends with the LDS of the wave in order.
 constexpr uint32_t kMaxUpperValues = 1u << 18;   // values of the level that tops a tile: 2^30 leaves
@@ -184,9 +201,7 @@ __global__ void __launch_bounds__(kWave) k_tile_totals(const float* __restrict__
     float s = 0.0f;
     if (chunk_base < n) {
         const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
-        const float* row = tile + lane * (kChunk + 1);
-        s = row[0];
-        for (int i = 1; i < len; ++i) s += row[i];
+        s = chunk_sum(tile + lane * (kChunk + 1), (uint32_t)len);
     }
     s_chunk[lane] = s;
     wave_sync();
@@ -221,12 +236,7 @@ __global__ void __launch_bounds__(kWave) k_cdf_scan_tiles(float* data, uint32_t 
     float s = 0.0f;
     if (chunk_base < n) {
         const int len = (int)min((size_t)kChunk, (size_t)n - chunk_base);
-        float* row = tile + lane * (kChunk + 1);
-        s = row[0];
-        for (int i = 1; i < len; ++i) {
-            s += row[i];
-            row[i] = s;
-        }
+        s = chunk_scan(tile + lane * (kChunk + 1), (uint32_t)len);
     }
     s_chunk[lane] = s;
     __syncthreads();
