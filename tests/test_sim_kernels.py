@@ -16,6 +16,10 @@ nothing about what only the hardware does (scheduling of blocks against each oth
 register and LDS limits): the `gpu` tests stay the parity tests proper."""
 import importlib
 import inspect
+import os
+import subprocess
+import sys
+from pathlib import Path
 
 import pytest
 
@@ -151,3 +155,22 @@ def test_every_case_names_a_gpu_test():
         assert set(kwargs) <= taken, (module_name, name, kwargs)
         marks = [m.name for m in getattr(function, "pytestmark", [])]
         assert "real_gpu" not in marks, (module_name, name)
+
+
+@pytest.mark.parametrize("order", ["reverse", "shuffle"])
+def test_results_do_not_depend_on_the_order_of_threads_and_blocks(order):
+    """A handful of the cases above in a process of their own whose simulator resumes threads and blocks in another
+    order (the order is fixed when the library is loaded): gradient rows of straddling points, ties in the tile sort,
+    large Gaussian footprints, the CDF, the ordered compaction of the training draw."""
+    chosen = ("gpu_raster.backward_direct[16-8-f32]", "gpu_raster.runs_of_equal_depth_keys[8-30]",
+              "gpu_gaussian.random_scenes_forward_backward[205]",
+              "gpu_sampler.cdf_and_search_tree_against_their_definitions[278528]",
+              "gpu_sampler.cull_compact_rounds_bit_exact[[10000,10000,10000]-True]",
+              "gpu_field.closes_the_loop_with_sampler_and_rasterizer")
+    nodes = [f"{Path(__file__)}::test_on_the_simulator[{case}]" for case in chosen]
+    env = dict(os.environ, INPC_SIM_ORDER=order)
+    done = subprocess.run([sys.executable, "-m", "pytest", *nodes, "-q", "-x", "-p", "no:cacheprovider"], env=env,
+                          capture_output=True, text=True, stdin=subprocess.DEVNULL, timeout=900,
+                          cwd=Path(__file__).resolve().parent.parent)
+    assert done.returncode == 0, done.stdout[-3000:] + done.stderr[-2000:]
+    assert f"{len(chosen)} passed" in done.stdout, done.stdout[-2000:]
