@@ -69,5 +69,21 @@ def build(force: bool = False, sanitize: bool = False) -> Path:
     return lib
 
 
+SELFTEST_LIB = HERE / "libsim_selftest.so"
+
+
+def build_selftest() -> Path:
+    """selftest.cpp (kernels that check the simulator itself) with the simulator core, as a library of its own."""
+    deps = [HERE / "selftest.cpp", HERE / "sim.cpp", HERE / "sim.hpp", HERE / "hip" / "hip_runtime.h"]
+    if SELFTEST_LIB.exists() and all(SELFTEST_LIB.stat().st_mtime >= d.stat().st_mtime for d in deps):
+        return SELFTEST_LIB
+    done = subprocess.run(["g++", *COMMON, *OPTIMIZE, "-ffp-contract=off", f"-I{HERE}", "-shared", "-o", str(SELFTEST_LIB),
+                           str(HERE / "selftest.cpp"), str(HERE / "sim.cpp")], capture_output=True, text=True,
+                          stdin=subprocess.DEVNULL, timeout=600)
+    if done.returncode != 0:
+        raise RuntimeError(f"building {SELFTEST_LIB} failed:\n{done.stderr[-4000:]}")
+    return SELFTEST_LIB
+
+
 if __name__ == "__main__":
     print(build(force=True, sanitize="--sanitize" in sys.argv[1:]))
