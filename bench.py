@@ -651,7 +651,7 @@ def main() -> int:
     draw_bytes = 32.0 * wl["leaves"] + 32.0 * draw_candidates
     sampler_extra = {
         "workload": f"training draw of {n} samples from {wl['leaves']} leaves (level {wl['level']}), same camera",
-        "call_ms": round(sampler_ms, 3), "kernels_ms": round(draw_kernel_ms, 4),
+        "call_ms": round(sampler_ms, 3), "kernels_ms": round(draw_kernel_ms, 4), "launches": len(draw_timer.records),
         "candidates": draw_candidates,
         "Msamples_per_s": round(n / (sampler_ms * 1e-3) / 1e6, 1),
         "Msamples_per_s_kernels_only": round(n / (draw_kernel_ms * 1e-3) / 1e6, 1) if draw_kernel_ms > 0 else None,

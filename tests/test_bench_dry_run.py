@@ -80,6 +80,8 @@ def test_every_leg_of_the_benchmark_runs(bench_on_the_simulator, monkeypatch, ca
     assert extra["other_tile_size"]["max_abs_image_difference"] < 1e-5
     assert extra["config4_inference"]["bilinear_abi"]["roofline"]["kernel"]
     assert {"sample_cull_compact", "cdf_tile_totals", "cdf_scan_tiles", "cdf_finish"} <= set(extra["sampler"]["kernel_ms"])
+    # a training draw that needs one round: leaf weights, three for the CDF, the round's reset, the draw, its end
+    assert extra["sampler"]["launches"] == 7
 
 
 def test_smoke_runs(sim, monkeypatch, capsys):
