@@ -174,3 +174,33 @@ def test_results_do_not_depend_on_the_order_of_threads_and_blocks(order):
                           cwd=Path(__file__).resolve().parent.parent)
     assert done.returncode == 0, done.stdout[-3000:] + done.stderr[-2000:]
     assert f"{len(chosen)} passed" in done.stdout, done.stdout[-2000:]
+
+
+def test_images_and_gradients_are_the_same_bits_under_any_order(tmp_path):
+    """One scene through both footprints under three orders of threads and blocks: images, alphas and both gradients
+    come out bit for bit the same (their sums have a fixed order: no float atomics), which no run on the hardware can
+    show; only the blending weights of points that straddle tiles are added up by float atomics, as in the reference
+    (B/rasterization/src/bilinear/kernels.cu:294; the reference adds its gradients that way too, :399-402), and may differ in
+    the last bit."""
+    import numpy as np
+
+    probe = Path(__file__).resolve().parent / "cpu_sim" / "order_probe.py"
+    runs = {}
+    for order in ("forward", "reverse", "shuffle"):
+        out = tmp_path / f"{order}.npz"
+        runs[order] = (out, subprocess.Popen([sys.executable, str(probe), str(out)], env=dict(os.environ, INPC_SIM_ORDER=order),
+                                            stdin=subprocess.DEVNULL, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    results = {}
+    for order, (out, process) in runs.items():
+        log, _ = process.communicate(timeout=900)
+        assert process.returncode == 0, log[-3000:]
+        results[order] = np.load(out)
+    base = results["forward"]
+    assert len(base.files) == 20
+    for order in ("reverse", "shuffle"):
+        for name in base.files:
+            a, b = base[name], results[order][name]
+            if name.endswith("blending_weights"):
+                np.testing.assert_allclose(a, b, rtol=0, atol=2e-7, err_msg=f"{name} under {order}")
+            else:
+                np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32), err_msg=f"{name} under {order}")
