@@ -115,6 +115,8 @@ def main() -> int:
     ap.add_argument("--no-config4", action="store_true",
                     help="skip the large-frame inference configuration (33,554,432 points @2473x1643, 16 fp16 "
                          "channels: training draw + inference forward, reported in extra.config4_inference)")
+    ap.add_argument("--only-config4", action="store_true",
+                    help="only the large-frame inference configuration, as the one JSON line (for profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus N with N > 1 is not supported "
@@ -134,6 +136,122 @@ def main() -> int:
     torch.cuda.set_device(device)
     wl = WORKLOADS[args.workload]
     n, channels, tile = wl["n"], wl["channels"], wl["tile"]
+    stream = _lib.current_stream()
+    gen = torch.Generator(device=device).manual_seed(1)
+
+    def time_calls(fn, reps):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e3 / reps
+
+    def config4_leg():
+        """BASELINE configuration 4: the large frame's training draw and its inference forward pass (both footprints
+        through the operator layer, the bilinear one once more through the C ABI with per-kernel figures)."""
+        n4, W4, H4 = CONFIG4["n"], CONFIG4["width"], CONFIG4["height"]
+        hv4 = synthetic.camera_on_z(W4, H4, CONFIG4["focal"], 6.0)
+        view4 = hv4.to_view(device)
+        oct4 = synthetic.octree_leaves(CONFIG4["leaves"], CONFIG4["level"], 4.0, seed=0)
+        c4, l4, w4 = (torch.from_numpy(a).to(device) for a in (oct4.centers, oct4.levels, oct4.weights))
+        sampler4 = ProbabilityFieldSampler(seed=0)
+        pos4, _ = sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size)
+        draw4_ms = time_calls(lambda: sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size), 5)
+        feats4 = torch.randn((n4, 16), generator=gen, device=device, dtype=torch.float32).half()
+        opac4 = torch.sigmoid(torch.randn(n4, generator=gen, device=device, dtype=torch.float32))
+        config4 = {"workload": f"{n4:,} pts @{W4}x{H4}, 16 channels stored fp16, inference forward",
+                   "training_draw_ms": round(draw4_ms, 3)}
+        from inpc_amd import rasterize_points
+
+        for label, mode, tile4, kw in (("bilinear", 0, 16, {}),
+                                       ("gaussian", 1, 8, dict(sigma_world=0.002, sigma_cutoff=3.0))):
+            def infer():
+                rasterize_points(view4, pos4, feats4, opac4, tile=tile4, inference=True, mode=mode, **kw)
+
+            infer()
+            ms = time_calls(infer, 5)
+            config4[f"{label}_forward_ms"] = round(ms, 3)
+            config4[f"{label}_Mpoints_per_s"] = round(n4 / (ms * 1e-3) / 1e6, 1)
+        # the bilinear forward once more through the C ABI: its counts, per-kernel durations (HIP events on the launch
+        # stream) and the share of the HBM roofline of the frame and of its largest kernel. Algorithmic bytes as for
+        # the training step, with 2 bytes per stored feature.
+        try:
+            cfg4 = _lib.RasterConfig(n4, 16, 16, _lib.FEAT_DIRECT_F16, _lib.RASTER_INFERENCE, _lib.make_camera(hv4.camera), 0)
+            layout4 = _lib.RasterLayout()
+            _lib.check(lib.inpc_raster_layout_query(C.byref(cfg4), C.byref(layout4)), "layout")
+            ws4 = torch.empty(layout4.total_bytes, dtype=torch.uint8, device=device)
+            image4 = torch.empty((16, H4, W4), dtype=torch.float32, device=device)
+            alpha4 = torch.empty((1, H4, W4), dtype=torch.float32, device=device)
+            depth4 = torch.empty((1, H4, W4), dtype=torch.float32, device=device)
+            w2c4, camp4 = view4.w2c.contiguous(), view4.position.contiguous()
+
+            def forward4():
+                _lib.check(lib.inpc_raster_forward(C.byref(cfg4), _lib.ptr(pos4), _lib.ptr(feats4), _lib.ptr(opac4),
+                                                   _lib.ptr(w2c4), _lib.ptr(camp4), _lib.ptr(image4), _lib.ptr(alpha4), None,
+                                                   _lib.ptr(depth4), _lib.ptr(ws4), layout4.total_bytes, stream),
+                           "inpc_raster_forward")
+
+            forward4()
+            counters4 = (C.c_uint32 * 3)()
+            _lib.check(lib.inpc_raster_read_counters(C.byref(cfg4), _lib.ptr(ws4), C.byref(counters4), stream), "counters")
+            v4, i4 = int(counters4[0]), int(counters4[1])
+            abi_ms = time_calls(forward4, 5)
+            with _lib.KernelTimer() as timer4:
+                for _ in range(3):
+                    forward4()
+            k4 = {}
+            for name, ms in timer4.records:
+                tot, cnt = k4.get(name, (0.0, 0))
+                k4[name] = (tot + ms, cnt + 1)
+            F4, R4, px4 = 2 * 16, 8 + 4 + 2 * 16, H4 * W4
+            sort_bytes = 2 + 12 * ((layout4.end_bit + 7) // 8) + 2
+            frame_bytes = float(n4 * (16 + F4) + v4 * (R4 + 8 + 68 + 20 + 16) + i4 * (6 + sort_bytes + 4 + R4)
+                                + px4 * 4 * (16 + 2))
+            per_kernel_bytes = {
+                "raster_bin_count": v4 * 20.0, "raster_records": float(n4 * (16 + F4) + v4 * R4),
+                "raster_bin_fill": float(v4 * (8 + 16) + i4 * 6), "raster_tile_sort": float(v4 * 68 + i4 * sort_bytes),
+                "raster_blend_inference": float(i4 * (4 + R4) + px4 * 4 * (16 + 2)),
+            }
+            rows4 = []
+            for name, (tot, cnt) in sorted(k4.items(), key=lambda kv: -kv[1][0]):
+                launches = cnt / 3
+                avg = tot / cnt
+                alg = per_kernel_bytes.get(name, 0.0) / launches
+                rows4.append({"kernel": name, "launches_per_frame": launches, "avg_ms": round(avg, 4),
+                              "ms_per_frame": round(tot / 3, 4),
+                              "algorithmic_GBps": round(alg / (avg * 1e-3) / 1e9, 1) if alg > 0 and avg > 0 else None})
+            top = rows4[0]
+            top_alg = per_kernel_bytes.get(top["kernel"], 0.0) / top["launches_per_frame"]
+            top_gbps = top_alg / (top["avg_ms"] * 1e-3) / 1e9
+            config4["bilinear_abi"] = {
+                "forward_ms": round(abi_ms, 3), "n_visible": v4, "n_instances": i4, "n_tiles": int(layout4.n_tiles),
+                "frame_algorithmic_GB": round(frame_bytes / 1e9, 3),
+                "frame_hbm_frac": round(frame_bytes / (abi_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "roofline": {"bound": "hbm", "kernel": top["kernel"], "achieved": round(top_gbps, 1),
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(top_gbps / HBM_PEAK_GBS, 4),
+                             "algorithmic_bytes_per_launch": top_alg, "avg_launch_ms": top["avg_ms"],
+                             "traffic": measured_traffic(top["kernel"], "config4")},
+                "kernels": rows4}
+            del ws4, image4, alpha4, depth4
+        except Exception as exc:  # the figure is optional
+            print(f"bench.py: config-4 per-kernel figures not measured: {exc}", file=sys.stderr)
+
+        return config4
+
+    if args.only_config4:
+        # the large frame alone (for profiler runs that must not mix its kernels with the training step's)
+        config4 = config4_leg()
+        abi = config4.get("bilinear_abi") or {}
+        ms = abi.get("forward_ms", config4["bilinear_forward_ms"])
+        print(json.dumps({
+            "metric": "Mpoints/s, inference forward of the large frame (ms/frame in ms_per_step)",
+            "value": round(CONFIG4["n"] / (ms * 1e-3) / 1e6, 1), "unit": "Mpoints/s", "n_gpus": 1, "steps": 5, "warmup": 1,
+            "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic", "config": {"workload": config4["workload"]}, "roofline": abi.get("roofline"),
+            "cpu_baseline": None, "extra": {"config4_inference": config4}}))
+        return 0
+
 
     # ---- inputs ---------------------------------------------------------------------------------------
     hv = synthetic.camera_on_z(wl["width"], wl["height"], wl["focal"], 6.0)
@@ -161,7 +279,6 @@ def main() -> int:
     positions, leaf_ids = sampler.generate_training_samples(centers, levels, weights, view, n, oct.initial_size)
     torch.cuda.synchronize()
 
-    gen = torch.Generator(device=device).manual_seed(1)
     features = torch.randn((n, channels), generator=gen, device=device, dtype=torch.float32)
     opacities = torch.sigmoid(torch.randn(n, generator=gen, device=device, dtype=torch.float32))
     H, W = wl["height"], wl["width"]
@@ -178,7 +295,6 @@ def main() -> int:
     grad_features = torch.empty((n, channels), dtype=torch.float32, device=device)
     grad_opacities = torch.empty(n, dtype=torch.float32, device=device)
     w2c, cam_position = view.w2c.contiguous(), view.position.contiguous()
-    stream = _lib.current_stream()
 
     def forward():
         _lib.check(lib.inpc_raster_forward(C.byref(cfg), _lib.ptr(positions), _lib.ptr(features), _lib.ptr(opacities),
@@ -219,14 +335,6 @@ def main() -> int:
     n_visible, n_instances = int(counters[0]), int(counters[1])
 
     # forward alone / backward alone
-    def time_calls(fn, reps):
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(reps):
-            fn()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t) * 1e3 / reps
-
     fwd_ms = time_calls(forward, args.steps)
     bwd_ms = time_calls(backward, args.steps)
 
@@ -558,92 +666,7 @@ def main() -> int:
         # free the training workload first: this one needs about 12 GB
         del workspace, image, alpha, blending_weights, grad_features, grad_opacities, features, opacities
         torch.cuda.empty_cache()
-        n4, W4, H4 = CONFIG4["n"], CONFIG4["width"], CONFIG4["height"]
-        hv4 = synthetic.camera_on_z(W4, H4, CONFIG4["focal"], 6.0)
-        view4 = hv4.to_view(device)
-        oct4 = synthetic.octree_leaves(CONFIG4["leaves"], CONFIG4["level"], 4.0, seed=0)
-        c4, l4, w4 = (torch.from_numpy(a).to(device) for a in (oct4.centers, oct4.levels, oct4.weights))
-        sampler4 = ProbabilityFieldSampler(seed=0)
-        pos4, _ = sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size)
-        draw4_ms = time_calls(lambda: sampler4.generate_training_samples(c4, l4, w4, view4, n4, oct4.initial_size), 5)
-        feats4 = torch.randn((n4, 16), generator=gen, device=device, dtype=torch.float32).half()
-        opac4 = torch.sigmoid(torch.randn(n4, generator=gen, device=device, dtype=torch.float32))
-        config4 = {"workload": f"{n4:,} pts @{W4}x{H4}, 16 channels stored fp16, inference forward",
-                   "training_draw_ms": round(draw4_ms, 3)}
-        from inpc_amd import rasterize_points
-
-        for label, mode, tile4, kw in (("bilinear", 0, 16, {}),
-                                       ("gaussian", 1, 8, dict(sigma_world=0.002, sigma_cutoff=3.0))):
-            def infer():
-                rasterize_points(view4, pos4, feats4, opac4, tile=tile4, inference=True, mode=mode, **kw)
-
-            infer()
-            ms = time_calls(infer, 5)
-            config4[f"{label}_forward_ms"] = round(ms, 3)
-            config4[f"{label}_Mpoints_per_s"] = round(n4 / (ms * 1e-3) / 1e6, 1)
-        # the bilinear forward once more through the C ABI: its counts, per-kernel durations (HIP events on the launch
-        # stream) and the share of the HBM roofline of the frame and of its largest kernel. Algorithmic bytes as for
-        # the training step, with 2 bytes per stored feature.
-        try:
-            cfg4 = _lib.RasterConfig(n4, 16, 16, _lib.FEAT_DIRECT_F16, _lib.RASTER_INFERENCE, _lib.make_camera(hv4.camera), 0)
-            layout4 = _lib.RasterLayout()
-            _lib.check(lib.inpc_raster_layout_query(C.byref(cfg4), C.byref(layout4)), "layout")
-            ws4 = torch.empty(layout4.total_bytes, dtype=torch.uint8, device=device)
-            image4 = torch.empty((16, H4, W4), dtype=torch.float32, device=device)
-            alpha4 = torch.empty((1, H4, W4), dtype=torch.float32, device=device)
-            depth4 = torch.empty((1, H4, W4), dtype=torch.float32, device=device)
-            w2c4, camp4 = view4.w2c.contiguous(), view4.position.contiguous()
-
-            def forward4():
-                _lib.check(lib.inpc_raster_forward(C.byref(cfg4), _lib.ptr(pos4), _lib.ptr(feats4), _lib.ptr(opac4),
-                                                   _lib.ptr(w2c4), _lib.ptr(camp4), _lib.ptr(image4), _lib.ptr(alpha4), None,
-                                                   _lib.ptr(depth4), _lib.ptr(ws4), layout4.total_bytes, stream),
-                           "inpc_raster_forward")
-
-            forward4()
-            counters4 = (C.c_uint32 * 3)()
-            _lib.check(lib.inpc_raster_read_counters(C.byref(cfg4), _lib.ptr(ws4), C.byref(counters4), stream), "counters")
-            v4, i4 = int(counters4[0]), int(counters4[1])
-            abi_ms = time_calls(forward4, 5)
-            with _lib.KernelTimer() as timer4:
-                for _ in range(3):
-                    forward4()
-            k4 = {}
-            for name, ms in timer4.records:
-                tot, cnt = k4.get(name, (0.0, 0))
-                k4[name] = (tot + ms, cnt + 1)
-            F4, R4, px4 = 2 * 16, 8 + 4 + 2 * 16, H4 * W4
-            sort_bytes = 2 + 12 * ((layout4.end_bit + 7) // 8) + 2
-            frame_bytes = float(n4 * (16 + F4) + v4 * (R4 + 8 + 68 + 20 + 16) + i4 * (6 + sort_bytes + 4 + R4)
-                                + px4 * 4 * (16 + 2))
-            per_kernel_bytes = {
-                "raster_bin_count": v4 * 20.0, "raster_records": float(n4 * (16 + F4) + v4 * R4),
-                "raster_bin_fill": float(v4 * (8 + 16) + i4 * 6), "raster_tile_sort": float(v4 * 68 + i4 * sort_bytes),
-                "raster_blend_inference": float(i4 * (4 + R4) + px4 * 4 * (16 + 2)),
-            }
-            rows4 = []
-            for name, (tot, cnt) in sorted(k4.items(), key=lambda kv: -kv[1][0]):
-                launches = cnt / 3
-                avg = tot / cnt
-                alg = per_kernel_bytes.get(name, 0.0) / launches
-                rows4.append({"kernel": name, "launches_per_frame": launches, "avg_ms": round(avg, 4),
-                              "ms_per_frame": round(tot / 3, 4),
-                              "algorithmic_GBps": round(alg / (avg * 1e-3) / 1e9, 1) if alg > 0 and avg > 0 else None})
-            top = rows4[0]
-            top_alg = per_kernel_bytes.get(top["kernel"], 0.0) / top["launches_per_frame"]
-            top_gbps = top_alg / (top["avg_ms"] * 1e-3) / 1e9
-            config4["bilinear_abi"] = {
-                "forward_ms": round(abi_ms, 3), "n_visible": v4, "n_instances": i4, "n_tiles": int(layout4.n_tiles),
-                "frame_algorithmic_GB": round(frame_bytes / 1e9, 3),
-                "frame_hbm_frac": round(frame_bytes / (abi_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                "roofline": {"bound": "hbm", "kernel": top["kernel"], "achieved": round(top_gbps, 1),
-                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(top_gbps / HBM_PEAK_GBS, 4),
-                             "algorithmic_bytes_per_launch": top_alg, "avg_launch_ms": top["avg_ms"],
-                             "traffic": measured_traffic(top["kernel"], "config4")},
-                "kernels": rows4}
-            del ws4, image4, alpha4, depth4
-        except Exception as exc:  # the figure is optional
-            print(f"bench.py: config-4 per-kernel figures not measured: {exc}", file=sys.stderr)
+        config4 = config4_leg()
 
     # the sampler (training draw of the same n points): 32 B per leaf (20 in, 4 out, 8 scan) and 32 B per candidate
     # (16 B of leaf data gathered, 12 B position + 4 B index written); the CDF probes are cache traffic and not counted

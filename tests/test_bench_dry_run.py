@@ -84,6 +84,18 @@ def test_every_leg_of_the_benchmark_runs(bench_on_the_simulator, monkeypatch, ca
     assert extra["sampler"]["launches"] == 7
 
 
+def test_the_large_frame_alone(bench_on_the_simulator, monkeypatch, capsys):
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--only-config4"])
+    assert bench_on_the_simulator.main() == 0
+    out = capsys.readouterr()
+    lines = [line for line in out.out.splitlines() if line.startswith("{")]
+    assert len(lines) == 1, out.out
+    record = json.loads(lines[0])
+    assert record["roofline"]["kernel"].startswith("raster_") and record["cpu_baseline"] is None
+    assert record["extra"]["config4_inference"]["bilinear_abi"]["n_visible"] > 0
+    assert record["config"]["workload"].startswith("12,000 pts")
+
+
 def test_smoke_runs(sim, monkeypatch, capsys):
     """__graft_entry__.smoke(), the check that runs on the GPU box before the benchmark, through the simulator."""
     spec = importlib.util.spec_from_file_location("graft_entry_dry_run", ROOT / "__graft_entry__.py")
