@@ -10,8 +10,10 @@ before the timed region.
 Prints ONE JSON line. `value` is Mpoints/s of forward+backward; `roofline` describes the kernel with the
 largest share of the step (algorithmic bytes per launch / HIP-event duration on the launch stream);
 `cpu_baseline` is the CPU oracle running the same step on a bounded sample, with all host threads and with one.
-`extra` carries the sampler's figures, the Gaussian footprint, the reference-shaped autograd step and the
-large-frame inference configuration (33,554,432 points @2473x1643).
+`extra` carries the sampler's figures, the Gaussian footprint, the reference-shaped autograd step, BASELINE
+configuration 0, the reference's default inference frame and the large-frame inference configuration (33,554,432
+points @2473x1643). `--only-config4` runs that last configuration alone and prints it as the one line, so that a
+profiler run of it holds no kernel of the training step.
 """
 from __future__ import annotations
 
