@@ -69,10 +69,7 @@ inline T pick(const uint64_t* slots, uint64_t members, int source, T fallback) {
 }
 }  // namespace detail
 
-inline void* dynamic_lds() {
-    char* p = block().dynamic_lds.data();
-    return (void*)(((uintptr_t)p + 63) & ~(uintptr_t)63);
-}
+inline void* dynamic_lds() { return block().dynamic_lds; }
 }  // namespace sim
 
 // extern __shared__ arrays: the launch's dynamic LDS

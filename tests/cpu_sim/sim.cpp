@@ -171,7 +171,13 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
     b.n_threads = n_threads;
     if (b.fibers.size() < n_threads) b.fibers.resize(n_threads);
     b.waves.resize((n_threads + 63) / 64);
-    b.dynamic_lds.resize(dynamic_lds_bytes + 64);
+    if (b.dynamic_lds_bytes != dynamic_lds_bytes || !b.dynamic_lds) {
+        std::free(b.dynamic_lds);
+        void* p = nullptr;
+        if (posix_memalign(&p, 64, dynamic_lds_bytes ? dynamic_lds_bytes : 1) != 0) std::abort();
+        b.dynamic_lds = (char*)p;
+        b.dynamic_lds_bytes = dynamic_lds_bytes;
+    }
     b.body = std::move(body);
     static thread_local std::vector<uint32_t> order;
     const bool blocks_reversed = thread_order() != Order::kForward;
@@ -183,7 +189,7 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
                                bz = blocks_reversed ? grid.z - 1u - iz : iz;
                 b.block_idx = Dim3(bx, by, bz);
                 // LDS holds what the block before left there, or anything: a kernel that counts on zeros shows up
-                std::memset(b.dynamic_lds.data(), 0xCD, b.dynamic_lds.size());
+                std::memset(b.dynamic_lds, 0xCD, b.dynamic_lds_bytes);
                 b.block_meeting = Meeting{};
                 b.block_meeting.alive = n_threads;
                 for (size_t w = 0; w < b.waves.size(); ++w) {

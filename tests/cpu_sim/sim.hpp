@@ -50,7 +50,8 @@ struct Block {
     std::vector<Fiber> fibers;
     Meeting block_meeting;
     std::vector<Meeting> waves;
-    std::vector<char> dynamic_lds;
+    char* dynamic_lds = nullptr;        // 64-byte aligned, exactly as many bytes as the launch asked for (so that a
+    size_t dynamic_lds_bytes = 0;       // sanitizer sees an access behind them)
     void* scheduler_sp = nullptr;
     std::function<void()> body;
     bool progress = false;
