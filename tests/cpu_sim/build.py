@@ -16,6 +16,8 @@ runtime preloaded:
 """
 from __future__ import annotations
 
+import os
+import shutil
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -31,6 +33,20 @@ COMMON = ["-std=c++17", "-fPIC"]
 OPTIMIZE = ["-O2"]
 SANITIZE = ["-O1", "-g", "-fsanitize=address,undefined,float-cast-overflow", "-fno-sanitize-recover=undefined,float-cast-overflow", "-fno-omit-frame-pointer"]
 KERNEL_FLAGS = ["-x", "c++", "-ffp-contract=off", "-Wno-unknown-pragmas", f"-I{HERE}"]
+# The host compiler: INPC_SIM_CXX if set; else ROCm's clang++ for the plain build (it is there wherever hipcc is) and
+# g++ for the sanitizer build (whose runtime the command above preloads), g++ for both where there is no clang++.
+# Unlike g++, clang++ also puts the __shared__ variables of function templates into the section that the simulator
+# fills with a byte pattern before every block (hip/hip_runtime.h), so with it no kernel can count on what an earlier
+# block left in any of its LDS.
+def _compiler(sanitize: bool) -> str:
+    chosen = os.environ.get("INPC_SIM_CXX")
+    if chosen:
+        return chosen
+    if not sanitize:
+        for candidate in (shutil.which("clang++"), "/opt/rocm/lib/llvm/bin/clang++"):
+            if candidate and Path(candidate).exists():
+                return candidate
+    return "g++"
 
 
 def _stale(lib: Path) -> bool:
@@ -43,11 +59,11 @@ def _stale(lib: Path) -> bool:
     return any(d.stat().st_mtime > built for d in deps)
 
 
-def _compile(src: Path, obj: Path, flags: list[str]) -> None:
-    done = subprocess.run(["g++", *flags, "-c", str(src), "-o", str(obj)], capture_output=True, text=True,
+def _compile(cxx: str, src: Path, obj: Path, flags: list[str]) -> None:
+    done = subprocess.run([cxx, *flags, "-c", str(src), "-o", str(obj)], capture_output=True, text=True,
                           stdin=subprocess.DEVNULL, timeout=1800)
     if done.returncode != 0:
-        raise RuntimeError(f"g++ failed on {src}:\n{done.stderr[-4000:]}")
+        raise RuntimeError(f"{cxx} failed on {src}:\n{done.stderr[-4000:]}")
 
 
 def build(force: bool = False, sanitize: bool = False) -> Path:
@@ -55,13 +71,14 @@ def build(force: bool = False, sanitize: bool = False) -> Path:
     if not force and not _stale(lib):
         return lib
     mode = SANITIZE if sanitize else OPTIMIZE
+    cxx = _compiler(sanitize)
     objdir = HERE / ("obj_asan" if sanitize else "obj")
     objdir.mkdir(exist_ok=True)
     jobs = [(CSRC / s, objdir / (Path(s).stem + ".o"), [*COMMON, *mode, *KERNEL_FLAGS]) for s in SOURCES]
     jobs.append((HERE / "sim.cpp", objdir / "sim.o", [*COMMON, *mode]))
     with ThreadPoolExecutor(max_workers=6) as pool:
-        list(pool.map(lambda job: _compile(*job), jobs))
-    link = ["g++", "-shared", *(["-fsanitize=address,undefined"] if sanitize else []), "-o", str(lib)]
+        list(pool.map(lambda job: _compile(cxx, *job), jobs))
+    link = [cxx, "-shared", *(["-fsanitize=address,undefined"] if sanitize else []), "-o", str(lib)]
     done = subprocess.run([*link, *[str(obj) for _, obj, _ in jobs]], capture_output=True, text=True,
                           stdin=subprocess.DEVNULL, timeout=600)
     if done.returncode != 0:
@@ -77,7 +94,7 @@ def build_selftest() -> Path:
     deps = [HERE / "selftest.cpp", HERE / "sim.cpp", HERE / "sim.hpp", HERE / "hip" / "hip_runtime.h"]
     if SELFTEST_LIB.exists() and all(SELFTEST_LIB.stat().st_mtime >= d.stat().st_mtime for d in deps):
         return SELFTEST_LIB
-    done = subprocess.run(["g++", *COMMON, *OPTIMIZE, "-ffp-contract=off", f"-I{HERE}", "-shared", "-o", str(SELFTEST_LIB),
+    done = subprocess.run([_compiler(False), *COMMON, *OPTIMIZE, "-ffp-contract=off", f"-I{HERE}", "-shared", "-o", str(SELFTEST_LIB),
                            str(HERE / "selftest.cpp"), str(HERE / "sim.cpp")], capture_output=True, text=True,
                           stdin=subprocess.DEVNULL, timeout=600)
     if done.returncode != 0:

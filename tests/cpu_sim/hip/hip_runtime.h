@@ -21,7 +21,10 @@
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
-#define __shared__ static thread_local
+// __shared__ variables are statics gathered in one section of the library, which sim::launch fills with a byte
+// pattern before every block: LDS holds nothing a block can count on. (One launch at a time per process.)
+#define __shared__ static __attribute__((section("sim_lds")))
+extern "C" char __start_sim_lds[], __stop_sim_lds[];
 #define __align__(n) __attribute__((aligned(n)))
 
 // ---- vector types ------------------------------------------------------------------------------------------------

@@ -7,6 +7,11 @@
 
 #include <cstdio>
 
+// The section that holds every __shared__ variable of the library this file is linked into (hip/hip_runtime.h); the
+// linker provides its bounds. Weak: a library without __shared__ variables has no such section.
+extern "C" char __start_sim_lds[] __attribute__((weak));
+extern "C" char __stop_sim_lds[] __attribute__((weak));
+
 namespace sim {
 
 namespace {
@@ -190,6 +195,8 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
                 b.block_idx = Dim3(bx, by, bz);
                 // LDS holds what the block before left there, or anything: a kernel that counts on zeros shows up
                 std::memset(b.dynamic_lds, 0xCD, b.dynamic_lds_bytes);
+                if (__start_sim_lds && __stop_sim_lds > __start_sim_lds)
+                    std::memset(__start_sim_lds, 0xCD, (size_t)(__stop_sim_lds - __start_sim_lds));
                 b.block_meeting = Meeting{};
                 b.block_meeting.alive = n_threads;
                 for (size_t w = 0; w < b.waves.size(); ++w) {
