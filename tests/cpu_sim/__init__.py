@@ -1,11 +1,11 @@
 """A SIMT simulator for the library's own kernels, for tests that have no GPU (TEST INFRASTRUCTURE ONLY).
 
-tests/cpu_sim/build.py compiles inpc_amd/csrc/*.hip, unchanged, with g++ against a stand-in for the HIP runtime
-(tests/cpu_sim/hip/hip_runtime.h): every thread of a block is a fiber, a wave's cross-lane operations and a block's
-barriers are meeting points where the fibers exchange values, blocks run one after the other (each starting with its
-LDS filled with a byte pattern), and device memory is host memory. The result, libinpc_sim.so, exports the same C ABI as the product's library. `simulated_device()` makes
-it the library that inpc_amd._lib hands out and "cpu" the device the test helpers allocate on, for as long as the
-context lasts.
+tests/cpu_sim/build.py compiles inpc_amd/csrc/*.hip, unchanged, with a host compiler (clang++ or g++) against a
+stand-in for the HIP runtime (tests/cpu_sim/hip/hip_runtime.h): every thread of a block is a fiber, a wave's
+cross-lane operations and a block's barriers are meeting points where the fibers exchange values, blocks run one after
+the other (each starting with its LDS filled with a byte pattern), and device memory is host memory. The result,
+libinpc_sim.so, exports the same C ABI as the product's library. `simulated_device()` makes it the library that
+inpc_amd._lib hands out and "cpu" the device the test helpers allocate on, for as long as the context lasts.
 
 What the simulator shows: the kernels' indexing, their arithmetic (up to the host compiler's and libm's rounding of
 exp/log/rsqrt, which the tolerances of the tests cover) and their use of barriers, ballots, shuffles, DPP moves and

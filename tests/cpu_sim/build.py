@@ -1,4 +1,4 @@
-"""Builds the library's own sources (inpc_amd/csrc/*.hip) with g++ against the simulator's stand-in for the HIP
+"""Builds the library's own sources (inpc_amd/csrc/*.hip) with a host compiler against the simulator's stand-in for the HIP
 runtime (tests/cpu_sim/hip/, tests/cpu_sim/sim.cpp) into tests/cpu_sim/libinpc_sim.so: the same C ABI, kernels run
 on the CPU one block after the other (see sim.hpp). TEST INFRASTRUCTURE ONLY: nothing of the product imports this,
 and the product itself still refuses to run without its HIP library.
