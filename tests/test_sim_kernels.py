@@ -1,6 +1,6 @@
 """The library's kernels on the CPU: a selection of the GPU parity tests, run without a GPU.
 
-tests/cpu_sim compiles inpc_amd/csrc/*.hip unchanged with g++ against a stand-in for the HIP runtime in which the
+tests/cpu_sim compiles inpc_amd/csrc/*.hip unchanged for the host against a stand-in for the HIP runtime in which the
 threads of a block are fibers and a wave's ballots, shuffles, DPP moves and barriers are meeting points. Each case
 below is a test function of one of the GPU test modules, called with the simulator's library loaded in the HIP
 library's place and host memory as the device: the same C-ABI calls, the same oracle, the same tolerances. The cases
