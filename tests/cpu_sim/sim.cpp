@@ -146,6 +146,15 @@ Order thread_order() {
     return order;
 }
 
+// The byte that fills LDS before every block: 0xCD, or INPC_SIM_LDS_BYTE (a number) to see that no result depends on it.
+int lds_pattern() {
+    static const int pattern = [] {
+        const char* v = std::getenv("INPC_SIM_LDS_BYTE");
+        return v ? (int)(std::strtol(v, nullptr, 0) & 0xFF) : 0xCD;
+    }();
+    return pattern;
+}
+
 void next_order(std::vector<uint32_t>& order, uint32_t n) {
     static thread_local uint64_t state = 0x9E3779B97F4A7C15ull;
     const Order mode = thread_order();
@@ -194,9 +203,9 @@ void launch(Dim3 grid, Dim3 block_dim, size_t dynamic_lds_bytes, std::function<v
                                bz = blocks_reversed ? grid.z - 1u - iz : iz;
                 b.block_idx = Dim3(bx, by, bz);
                 // LDS holds what the block before left there, or anything: a kernel that counts on zeros shows up
-                std::memset(b.dynamic_lds, 0xCD, b.dynamic_lds_bytes);
+                std::memset(b.dynamic_lds, lds_pattern(), b.dynamic_lds_bytes);
                 if (__start_sim_lds && __stop_sim_lds > __start_sim_lds)
-                    std::memset(__start_sim_lds, 0xCD, (size_t)(__stop_sim_lds - __start_sim_lds));
+                    std::memset(__start_sim_lds, lds_pattern(), (size_t)(__stop_sim_lds - __start_sim_lds));
                 b.block_meeting = Meeting{};
                 b.block_meeting.alive = n_threads;
                 for (size_t w = 0; w < b.waves.size(); ++w) {

@@ -177,8 +177,8 @@ def test_results_do_not_depend_on_the_order_of_threads_and_blocks(order):
 
 
 def test_images_and_gradients_are_the_same_bits_under_any_order(tmp_path):
-    """One scene through both footprints under three orders of threads and blocks: images, alphas and both gradients
-    come out bit for bit the same (their sums have a fixed order: no float atomics), which no run on the hardware can
+    """One scene through both footprints under three orders of threads and blocks (and three byte patterns in the LDS
+    that a block finds): images, alphas and both gradients come out bit for bit the same (their sums have a fixed order: no float atomics), which no run on the hardware can
     show; only the blending weights of points that straddle tiles are added up by float atomics, as in the reference
     (B/rasterization/src/bilinear/kernels.cu:294; the reference adds its gradients that way too, :399-402), and may differ in
     the last bit."""
@@ -186,9 +186,10 @@ def test_images_and_gradients_are_the_same_bits_under_any_order(tmp_path):
 
     probe = Path(__file__).resolve().parent / "cpu_sim" / "order_probe.py"
     runs = {}
-    for order in ("forward", "reverse", "shuffle"):
+    for order, lds_byte in (("forward", "0xCD"), ("reverse", "0x00"), ("shuffle", "0xFF")):   # and what LDS holds at first
         out = tmp_path / f"{order}.npz"
-        runs[order] = (out, subprocess.Popen([sys.executable, str(probe), str(out)], env=dict(os.environ, INPC_SIM_ORDER=order),
+        runs[order] = (out, subprocess.Popen([sys.executable, str(probe), str(out)],
+                                            env=dict(os.environ, INPC_SIM_ORDER=order, INPC_SIM_LDS_BYTE=lds_byte),
                                             stdin=subprocess.DEVNULL, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
     results = {}
     for order, (out, process) in runs.items():
