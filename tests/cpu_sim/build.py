@@ -102,5 +102,42 @@ def build_selftest() -> Path:
     return SELFTEST_LIB
 
 
+MSAN_DRIVER = HERE / "msan_driver"
+MSAN_FLAGS = ["-O1", "-g", "-fsanitize=memory", "-fsanitize-memory-track-origins=2", "-fno-omit-frame-pointer"]
+
+
+def clang() -> str | None:
+    """A clang++ (MemorySanitizer is clang's): INPC_SIM_CXX if it is one, one on the PATH, or ROCm's."""
+    for candidate in (os.environ.get("INPC_SIM_CXX"), shutil.which("clang++"), "/opt/rocm/lib/llvm/bin/clang++"):
+        if candidate and "clang" in Path(candidate).name and Path(candidate).exists():
+            return candidate
+    return None
+
+
+def build_msan_driver() -> Path:
+    """msan_driver.cpp, the library's sources and the simulator as one executable under MemorySanitizer."""
+    cxx = clang()
+    if cxx is None:
+        raise RuntimeError("MemorySanitizer needs clang++")
+    deps = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.hpp")) + [ROOT / "include" / "inpc_hip.h", HERE / "sim.cpp",
+                                                                  HERE / "sim.hpp", HERE / "hip" / "hip_runtime.h",
+                                                                  HERE / "hip" / "hip_fp16.h", HERE / "msan_driver.cpp",
+                                                                  Path(__file__)]
+    if MSAN_DRIVER.exists() and all(MSAN_DRIVER.stat().st_mtime >= d.stat().st_mtime for d in deps):
+        return MSAN_DRIVER
+    objdir = HERE / "obj_msan"
+    objdir.mkdir(exist_ok=True)
+    jobs = [(CSRC / s, objdir / (Path(s).stem + ".o"), [*COMMON, *MSAN_FLAGS, *KERNEL_FLAGS]) for s in SOURCES]
+    jobs.append((HERE / "sim.cpp", objdir / "sim.o", [*COMMON, *MSAN_FLAGS]))
+    jobs.append((HERE / "msan_driver.cpp", objdir / "msan_driver.o", [*COMMON, *MSAN_FLAGS, f"-I{HERE}"]))
+    with ThreadPoolExecutor(max_workers=7) as pool:
+        list(pool.map(lambda job: _compile(cxx, *job), jobs))
+    done = subprocess.run([cxx, "-fsanitize=memory", "-o", str(MSAN_DRIVER), *[str(obj) for _, obj, _ in jobs]],
+                          capture_output=True, text=True, stdin=subprocess.DEVNULL, timeout=600)
+    if done.returncode != 0:
+        raise RuntimeError(f"linking {MSAN_DRIVER} failed:\n{done.stderr[-4000:]}")
+    return MSAN_DRIVER
+
+
 if __name__ == "__main__":
     print(build(force=True, sanitize="--sanitize" in sys.argv[1:]))
