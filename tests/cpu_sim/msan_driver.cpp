@@ -228,6 +228,87 @@ int rasterizer(int tile, int channels, bool gaussian) {
     return 0;
 }
 
+// fp16 bits of a float of ordinary size (no rounding needed for the tests: truncation)
+uint16_t half_bits(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const int32_t exponent = (int32_t)((u >> 23) & 0xFF) - 127 + 15;
+    if (exponent <= 0) return (uint16_t)sign;
+    if (exponent >= 31) return (uint16_t)(sign | 0x7BFFu);
+    return (uint16_t)(sign | ((uint32_t)exponent << 10) | ((u >> 13) & 0x3FFu));
+}
+
+// The spherical-harmonics modes: training on (N,36) fp16 coefficients (the gradient comes back as fp16 through a
+// scratch array) and inference on the raw (N,37) fp16 output of the appearance field.
+int rasterizer_sh(bool gaussian) {
+    const uint32_t n = 20000;
+    const int width = 157, height = 101, tile = 16;
+    const Scene s = make_scene(n, 4);
+    const inpc_camera cam{width, height, 140.f, 140.f, width / 2.f, height / 2.f, 0.01f, 100.f};
+    const size_t pixels = (size_t)width * height;
+    uint16_t* sh = (uint16_t*)fresh((size_t)n * 36 * 2);
+    uint16_t* raw = (uint16_t*)fresh((size_t)n * 37 * 2);
+    for (size_t i = 0; i < (size_t)n * 36; ++i) sh[i] = half_bits(uniform(-0.5f, 0.5f));
+    for (size_t i = 0; i < (size_t)n * 37; ++i) raw[i] = half_bits(uniform(-0.5f, 0.5f));
+    float* image = (float*)fresh(pixels * 4 * 4);
+    float* alpha = (float*)fresh(pixels * 4);
+    float* depth = (float*)fresh(pixels * 4);
+    float* blending_weights = (float*)fresh(n * 4);
+    float* grad_image = (float*)fresh(pixels * 4 * 4);
+    float* grad_alpha = (float*)fresh(pixels * 4);
+    for (size_t i = 0; i < pixels * 4; ++i) grad_image[i] = uniform(-0.01f, 0.01f);
+    for (size_t i = 0; i < pixels; ++i) grad_alpha[i] = uniform(-0.01f, 0.01f);
+    uint16_t* grad_sh = (uint16_t*)fresh((size_t)n * 36 * 2);
+    float* grad_opacities = (float*)fresh(n * 4);
+    float* scratch = (float*)fresh((size_t)n * 4 * 4);
+    inpc_raster_config cfg{n, tile, 4, INPC_FEAT_SH36_F16, 0u, cam, 0u};
+    inpc_raster_config raw_cfg{n, tile, 4, INPC_FEAT_RAW37_F16, INPC_RASTER_INFERENCE, cam, 0u};
+    if (gaussian) {
+        inpc_gaussian_config g{cfg, 0.0f, 3.0f, 40u * n, 0u};
+        inpc_gaussian_layout layout;
+        CHECK(inpc_gaussian_layout_query(&g, &layout));
+        void* ws = filled(layout.total_bytes);
+        CHECK(inpc_gaussian_forward(&g, s.positions, sh, s.opacities, nullptr, s.w2c, s.cam_position, image, alpha,
+                                    blending_weights, nullptr, ws, layout.total_bytes, nullptr));
+        CHECK(inpc_gaussian_backward(&g, grad_image, grad_alpha, image, alpha, s.positions, s.cam_position, grad_sh,
+                                     grad_opacities, scratch, ws, layout.total_bytes, nullptr));
+    } else {
+        inpc_raster_layout layout;
+        CHECK(inpc_raster_layout_query(&cfg, &layout));
+        void* ws = fresh(layout.total_bytes);
+        CHECK(inpc_raster_forward(&cfg, s.positions, sh, s.opacities, s.w2c, s.cam_position, image, alpha, blending_weights,
+                                  nullptr, ws, layout.total_bytes, nullptr));
+        CHECK(inpc_raster_backward(&cfg, grad_image, grad_alpha, image, alpha, s.positions, s.cam_position, grad_sh,
+                                   grad_opacities, scratch, ws, layout.total_bytes, nullptr));
+    }
+    __msan_check_mem_is_initialized(image, pixels * 4 * 4);
+    __msan_check_mem_is_initialized(alpha, pixels * 4);
+    __msan_check_mem_is_initialized(blending_weights, n * 4);
+    __msan_check_mem_is_initialized(grad_sh, (size_t)n * 36 * 2);
+    __msan_check_mem_is_initialized(grad_opacities, n * 4);
+    if (gaussian) {
+        inpc_gaussian_config g{raw_cfg, 0.004f, 2.5f, 40u * n, 0u};
+        inpc_gaussian_layout layout;
+        CHECK(inpc_gaussian_layout_query(&g, &layout));
+        void* ws = filled(layout.total_bytes);
+        CHECK(inpc_gaussian_forward(&g, s.positions, raw, nullptr, nullptr, s.w2c, s.cam_position, image, alpha, nullptr, depth,
+                                    ws, layout.total_bytes, nullptr));
+    } else {
+        inpc_raster_layout layout;
+        CHECK(inpc_raster_layout_query(&raw_cfg, &layout));
+        void* ws = fresh(layout.total_bytes);
+        CHECK(inpc_raster_forward(&raw_cfg, s.positions, raw, nullptr, s.w2c, s.cam_position, image, alpha, nullptr, depth, ws,
+                                  layout.total_bytes, nullptr));
+    }
+    __msan_check_mem_is_initialized(image, pixels * 4 * 4);
+    __msan_check_mem_is_initialized(alpha, pixels * 4);
+    __msan_check_mem_is_initialized(depth, pixels * 4);
+    std::printf("%s footprint, spherical harmonics: training on (N,36) fp16, inference on raw (N,37) fp16\n",
+                gaussian ? "Gaussian" : "bilinear");
+    return 0;
+}
+
 }  // namespace
 
 int main() {
@@ -235,6 +316,8 @@ int main() {
     for (const bool gaussian : {false, true})
         for (const int tile : {16, 8})
             if (rasterizer(tile, tile == 16 ? 8 : 4, gaussian) != 0) return 1;
+    for (const bool gaussian : {false, true})
+        if (rasterizer_sh(gaussian) != 0) return 1;
     std::printf("no use of uninitialised memory\n");
     return 0;
 }
