@@ -228,6 +228,78 @@ int rasterizer(int tile, int channels, bool gaussian) {
     return 0;
 }
 
+// The bookkeeping of the probability field (selections, extraction of a global cloud, Morton codes) and the
+// element-wise operators.
+int field_and_misc() {
+    const uint32_t n = 33333;
+    float* centers = (float*)fresh(n * 12);
+    int32_t* levels = (int32_t*)fresh(n * 4);
+    float* weights = (float*)fresh(n * 4);
+    float* scores = (float*)fresh(n * 4);
+    int64_t* counts = (int64_t*)fresh(n * 8);
+    uint32_t n_samples = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        for (int k = 0; k < 3; ++k) centers[3 * i + k] = uniform(-2.f, 2.f);
+        levels[i] = 3 + (int)(i % 5);
+        weights[i] = uniform(0.f, 1.f);
+        scores[i] = uniform(0.f, 1.f);
+        counts[i] = (int64_t)(i % 4);
+        n_samples += (uint32_t)counts[i];
+    }
+    const float initial_size[3] = {4.f, 4.f, 4.f};
+    const size_t select_bytes = inpc_field_select_workspace_bytes(n);
+    void* select_ws = fresh(select_bytes);
+    uint32_t* count = (uint32_t*)fresh(4);
+    CHECK(inpc_field_select_count(scores, levels, n, 0.5f, 7, count, select_ws, select_bytes, nullptr));
+    __msan_check_mem_is_initialized(count, 4);
+    const uint32_t split = *count, n_out = n + 7u * split;
+    float* centers_out = (float*)fresh((size_t)n_out * 12);
+    int32_t* levels_out = (int32_t*)fresh((size_t)n_out * 4);
+    float* weights_out = (float*)fresh((size_t)n_out * 4);
+    float* scores_out = (float*)fresh((size_t)n_out * 4);
+    CHECK(inpc_field_subdivide(centers, levels, weights, scores, n, 0.5f, 7, initial_size, centers_out, levels_out, weights_out,
+                               scores_out, count, select_ws, select_bytes, nullptr));
+    __msan_check_mem_is_initialized(centers_out, (size_t)n_out * 12);
+    __msan_check_mem_is_initialized(levels_out, (size_t)n_out * 4);
+    __msan_check_mem_is_initialized(weights_out, (size_t)n_out * 4);
+    __msan_check_mem_is_initialized(scores_out, (size_t)n_out * 4);
+    CHECK(inpc_field_prune(centers, levels, weights, scores, n, 0.3f, centers_out, levels_out, weights_out, scores_out, count,
+                           select_ws, select_bytes, nullptr));
+    __msan_check_mem_is_initialized(count, 4);
+    __msan_check_mem_is_initialized(centers_out, (size_t)*count * 12);
+    __msan_check_mem_is_initialized(scores_out, (size_t)*count * 4);
+    const size_t extract_bytes = inpc_extract_global_workspace_bytes(n);
+    void* extract_ws = fresh(extract_bytes);
+    float* cloud = (float*)fresh((size_t)n_samples * 12);
+    CHECK(inpc_extract_global(centers, levels, counts, n, initial_size, cloud, n_samples, extract_ws, extract_bytes, nullptr));
+    CHECK(inpc_extract_global_check(extract_ws, n_samples, nullptr));
+    __msan_check_mem_is_initialized(cloud, (size_t)n_samples * 12);
+    int64_t* codes = (int64_t*)fresh((size_t)n_samples * 8);
+    void* morton_ws = fresh(inpc_morton_workspace_bytes());
+    CHECK(inpc_morton_encode(cloud, n_samples, codes, morton_ws, inpc_morton_workspace_bytes(), nullptr));
+    __msan_check_mem_is_initialized(codes, (size_t)n_samples * 8);
+    float* contracted = (float*)fresh((size_t)n_samples * 12);
+    CHECK(inpc_spherical_contraction(cloud, contracted, n_samples, nullptr));
+    __msan_check_mem_is_initialized(contracted, (size_t)n_samples * 12);
+    float* out_a = (float*)fresh(n * 4);
+    float* out_b = (float*)fresh(n * 4);
+    CHECK(inpc_opacity_forward(scores, out_a, n, nullptr));
+    CHECK(inpc_opacity_backward(weights, scores, out_b, n, nullptr));
+    __msan_check_mem_is_initialized(out_a, n * 4);
+    __msan_check_mem_is_initialized(out_b, n * 4);
+    CHECK(inpc_weight_decay_grads(weights, out_a, n, 0, nullptr));
+    CHECK(inpc_weight_decay_grads(weights, out_a, n, 1, nullptr));
+    CHECK(inpc_cauchy_loss(weights, scores, out_b, n, nullptr));
+    __msan_check_mem_is_initialized(out_a, n * 4);
+    __msan_check_mem_is_initialized(out_b, n * 4);
+    float* upstream = (float*)fresh(4);
+    *upstream = 1.5f;
+    CHECK(inpc_cauchy_loss_backward(upstream, weights, scores, out_a, n, nullptr));
+    __msan_check_mem_is_initialized(out_a, n * 4);
+    std::printf("field bookkeeping and element-wise operators: %u leaves split, %u samples extracted\n", split, n_samples);
+    return 0;
+}
+
 // fp16 bits of a float of ordinary size (no rounding needed for the tests: truncation)
 uint16_t half_bits(float f) {
     uint32_t u;
@@ -313,6 +385,7 @@ int rasterizer_sh(bool gaussian) {
 
 int main() {
     if (sampler() != 0) return 1;
+    if (field_and_misc() != 0) return 1;
     for (const bool gaussian : {false, true})
         for (const int tile : {16, 8})
             if (rasterizer(tile, tile == 16 ? 8 : 4, gaussian) != 0) return 1;
