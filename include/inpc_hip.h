@@ -385,7 +385,12 @@ typedef struct inpc_gaussian_layout {
 } inpc_gaussian_layout;
 
 /* Workspace size and layout. Replaces the growable blobs of
- * B/rasterization/include/gaussian/buffer_utils.h:24-117 with one caller-owned buffer. */
+ * B/rasterization/include/gaussian/buffer_utils.h:24-117 with one caller-owned buffer.
+ * The workspace needs no clearing, whatever it held before. (Its backward pass tells the gradient
+ * rows of the current pass from older ones by a 64-bit number that every forward pass takes from
+ * the workspace and steps by one; in a workspace never used before, that number and the rows are
+ * whatever the memory held, and an unwritten row passes for a written one only if 64 arbitrary
+ * bits equal it.) */
 int inpc_gaussian_layout_query(const inpc_gaussian_config* cfg, inpc_gaussian_layout* out);
 
 /* Forward pass with the Gaussian footprint. Replaces the gaussian branches of forward_wrapper /
